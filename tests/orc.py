@@ -1,0 +1,290 @@
+"""ctypes view of the parity oracle (oracle/liboracle.so) and, when it was built, of the compiled reference
+(oracle/_ref/libstrix_ref.so). Test infrastructure only: the GPU library never imports this module."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+
+Q8_0, Q4_K = 8, 12
+Q8_0_BLOCK, Q4_K_BLOCK = 34, 144
+EXP_GFX1151, EXP_DECLARED = 0, 1
+LOGITS_FMA, LOGITS_LANE32 = 0, 1
+COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
+
+u8p, i8p, f32p, i32p, u32p = (C.POINTER(t) for t in (C.c_uint8, C.c_int8, C.c_float, C.c_int32, C.c_uint32))
+
+
+def _ptr(a, t):
+    if a is None:
+        return C.cast(None, t)
+    assert a.flags["C_CONTIGUOUS"], "oracle arguments must be contiguous"
+    return a.ctypes.data_as(t)
+
+
+def build_oracle():
+    """Compile the oracle (and the reference shim when /root/reference exists). Idempotent."""
+    subprocess.run(["make", "-C", ORACLE_DIR, "-j8"], check=True, stdout=subprocess.DEVNULL)
+
+
+def _load(path):
+    return C.CDLL(path) if os.path.exists(path) else None
+
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        path = os.path.join(ORACLE_DIR, "liboracle.so")
+        if not os.path.exists(path):
+            build_oracle()
+        _lib = C.CDLL(path)
+        _declare(_lib)
+    return _lib
+
+
+def ref():
+    """The compiled reference, or None when oracle/_ref was not built (no reference tree at build time)."""
+    global _ref
+    if _ref is None:
+        _ref = _load(os.path.join(ORACLE_DIR, "_ref", "libstrix_ref.so")) or False
+        if _ref:
+            _ref.ref_half_to_float.restype = C.c_float
+            _ref.ref_contract_half_to_float.restype = C.c_float
+            _ref.ref_ggml_fp16.restype = C.c_float
+            _ref.ref_declared_exp.restype = C.c_float
+            _ref.ref_declared_exp.argtypes = [C.c_float]
+            _ref.ref_gfx1151_expf_empty_tables.restype = C.c_float
+            _ref.ref_gfx1151_expf_empty_tables.argtypes = [C.c_float]
+            _ref.ref_last_error.restype = C.c_char_p
+            _ref.ref_executor_create.restype = C.c_void_p
+            _ref.ref_executor_isa.restype = C.c_char_p
+            _ref.ref_executor_isa.argtypes = [C.c_void_p]
+            _ref.ref_executor_destroy.argtypes = [C.c_void_p]
+    return _ref or None
+
+
+class Q8a8View(C.Structure):
+    _fields_ = [("weight", C.c_void_p), ("codes", C.c_void_p), ("deltas", C.c_void_p), ("out", C.c_void_p),
+                ("row_bytes", C.c_uint32), ("in_", C.c_uint32), ("count", C.c_uint32), ("rows", C.c_uint32),
+                ("x_stride", C.c_uint32), ("out_stride", C.c_uint32), ("accumulate", C.c_uint32)]
+
+
+class RoutePolicy(C.Structure):
+    _fields_ = [("experts", C.c_uint32), ("top_k", C.c_uint32), ("logits_order", C.c_int), ("exp_kind", C.c_int),
+                ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_int)]
+
+
+class ExpertWeights(C.Structure):
+    _fields_ = [("hidden", C.c_uint32), ("ffn", C.c_uint32), ("experts", C.c_uint32), ("top_k", C.c_uint32),
+                ("gate_type", C.c_uint32), ("down_type", C.c_uint32),
+                ("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p),
+                ("gate_expert_stride", C.c_uint64), ("gate_row_stride", C.c_uint64),
+                ("down_expert_stride", C.c_uint64), ("down_row_stride", C.c_uint64), ("exp_kind", C.c_int)]
+
+
+class ExpertJob(C.Structure):
+    _fields_ = [("codes", C.c_void_p), ("deltas", C.c_void_p), ("sums", C.c_void_p), ("ids", C.c_void_p),
+                ("rows", C.c_uint32),
+                ("gate_out", C.c_void_p), ("up_out", C.c_void_p), ("h_out", C.c_void_p), ("h_codes", C.c_void_p),
+                ("h_deltas", C.c_void_p), ("h_sums", C.c_void_p), ("rawdots", C.c_void_p), ("status", C.c_void_p)]
+
+
+def _declare(L):
+    L.orc_half_to_float.restype = C.c_float
+    L.orc_half_to_float.argtypes = [C.c_uint16]
+    L.orc_float_to_half.restype = C.c_uint16
+    L.orc_float_to_half.argtypes = [C.c_float]
+    L.orc_q4k_factor_words.restype = C.c_uint
+    L.orc_q4k_row_a8.restype = C.c_float
+    L.orc_q4k_row_a8_contract_form.restype = C.c_float
+    L.orc_q8_0_down_row_a8.restype = C.c_float
+    L.orc_expf_gfx1151.restype = C.c_float
+    L.orc_expf_gfx1151.argtypes = [C.c_float]
+    L.orc_declared_exp.restype = C.c_float
+    L.orc_declared_exp.argtypes = [C.c_float]
+    L.orc_lane_dot.restype = C.c_float
+    L.orc_lane_dot.argtypes = [f32p, f32p, C.c_size_t]
+
+
+# ---------------------------------------------------------------- numpy-level helpers
+def row_bytes(qtype, elements):
+    return elements // 32 * Q8_0_BLOCK if qtype == Q8_0 else elements // 256 * Q4_K_BLOCK
+
+
+def half_to_float(bits):
+    return lib().orc_half_to_float(int(bits))
+
+
+def float_to_half(value):
+    return lib().orc_float_to_half(float(np.float32(value)))
+
+
+def dequant_rows(qtype, packed, elements):
+    """packed: uint8 [rows][row_bytes] -> float32 [rows][elements]."""
+    packed = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1, row_bytes(qtype, elements))
+    out = np.empty((packed.shape[0], elements), np.float32)
+    fn = lib().orc_dequant_q8_0_row if qtype == Q8_0 else lib().orc_dequant_q4_k_row
+    for r in range(packed.shape[0]):
+        fn(_ptr(packed[r], u8p), C.c_size_t(elements), _ptr(out[r], f32p))
+    return out
+
+
+def quantize_rows(qtype, x):
+    """x: float32 [rows][elements] -> uint8 [rows][row_bytes] with the oracle's writer."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    x2 = x.reshape(-1, x.shape[-1])
+    out = np.empty((x2.shape[0], row_bytes(qtype, x2.shape[1])), np.uint8)
+    fn = lib().orc_quantize_q8_0_row if qtype == Q8_0 else lib().orc_quantize_q4_k_row
+    for r in range(x2.shape[0]):
+        fn(_ptr(x2[r], f32p), C.c_size_t(x2.shape[1]), _ptr(out[r], u8p))
+    return out.reshape(x.shape[:-1] + (out.shape[1],))
+
+
+def quantize_a8(x, tiny_rule=True):
+    """x float32 [rows][width] -> (codes int8, deltas f32, sums i32, rc list)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    x2 = x.reshape(-1, x.shape[-1])
+    rows, width = x2.shape
+    codes = np.zeros((rows, width), np.int8)
+    deltas = np.zeros((rows, width // 32), np.float32)
+    sums = np.zeros((rows, width // 32), np.int32)
+    rcs = [lib().orc_quantize_a8(_ptr(x2[r], f32p), C.c_size_t(width), _ptr(codes[r], i8p), _ptr(deltas[r], f32p),
+                                 _ptr(sums[r], i32p), int(tiny_rule)) for r in range(rows)]
+    return codes, deltas, sums, rcs
+
+
+def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False, threads=1):
+    weight = np.ascontiguousarray(weight, np.uint8)
+    rows = codes.shape[0]
+    if out is None:
+        out = np.zeros((rows, count), np.float32)
+    v = Q8a8View(weight.ctypes.data, codes.ctypes.data, deltas.ctypes.data, out.ctypes.data,
+                 n_in // 32 * Q8_0_BLOCK, n_in, count, rows, codes.shape[1], out.shape[1], int(accumulate))
+    rc = lib().orc_gemv_q8_0_a8(C.byref(v), threads)
+    return out, rc
+
+
+def q4k_row_a8(wrow, codes, deltas, sums, contract_form=False):
+    wrow = np.ascontiguousarray(wrow, np.uint8)
+    fn = lib().orc_q4k_row_a8_contract_form if contract_form else lib().orc_q4k_row_a8
+    return np.float32(fn(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q4_K_BLOCK), _ptr(codes, i8p), _ptr(deltas, f32p),
+                         _ptr(sums, i32p)))
+
+
+def q8_0_down_row_a8(wrow, codes, deltas):
+    wrow = np.ascontiguousarray(wrow, np.uint8)
+    return np.float32(lib().orc_q8_0_down_row_a8(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q8_0_BLOCK), _ptr(codes, i8p),
+                                                 _ptr(deltas, f32p)))
+
+
+def swiglu_quantize(g, u, exp_kind=EXP_GFX1151):
+    g = np.ascontiguousarray(g, np.float32)
+    u = np.ascontiguousarray(u, np.float32)
+    codes = np.zeros(32, np.int8)
+    delta = C.c_float(0)
+    s = C.c_int32(0)
+    h = np.zeros(32, np.float32)
+    ok = lib().orc_swiglu_quantize(exp_kind, _ptr(g, f32p), _ptr(u, f32p), _ptr(codes, i8p), C.byref(delta), C.byref(s),
+                                   _ptr(h, f32p))
+    return ok, codes, np.float32(delta.value), s.value, h
+
+
+def route(x, w, top_k, bias=None, logits_order=LOGITS_FMA, exp_kind=EXP_DECLARED, renorm_eps=0.0, scale=1.0,
+          renormalize=True, threads=0):
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    rows, hidden = x.shape
+    experts = w.shape[0]
+    p = RoutePolicy(experts, top_k, logits_order, exp_kind, renorm_eps, scale, int(renormalize))
+    ids = np.zeros((rows, top_k), np.uint32)
+    weights = np.zeros((rows, top_k), np.float32)
+    scores = np.zeros((rows, experts), np.float32)
+    logits = np.zeros((rows, experts), np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    lib().orc_route(C.byref(p), _ptr(x, f32p), rows, hidden, _ptr(w, f32p), _ptr(b, f32p), _ptr(ids, u32p),
+                    _ptr(weights, f32p), _ptr(scores, f32p), _ptr(logits, f32p), threads or lib().orc_max_threads())
+    return ids, weights, scores, logits
+
+
+def route_select(scores, top_k, renorm_eps=0.0, scale=1.0, renormalize=True):
+    scores = np.ascontiguousarray(scores, np.float32)
+    p = RoutePolicy(scores.size, top_k, 0, 0, renorm_eps, scale, int(renormalize))
+    ids = np.zeros(top_k, np.uint32)
+    weights = np.zeros(top_k, np.float32)
+    lib().orc_route_select(C.byref(p), _ptr(scores, f32p), _ptr(ids, u32p), _ptr(weights, f32p))
+    return ids, weights
+
+
+def combine(form, w, ids, raw, base=None):
+    rows, top_k, width = raw.shape
+    raw = np.ascontiguousarray(raw, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    ids = np.ascontiguousarray(ids, np.uint32)
+    y = np.zeros((rows, width), np.float32)
+    b = None if base is None else np.ascontiguousarray(base, np.float32)
+    lib().orc_combine(form, rows, top_k, width, _ptr(w, f32p), _ptr(ids, u32p), _ptr(raw, f32p), _ptr(b, f32p), _ptr(y, f32p))
+    return y
+
+
+class ExpertResult:
+    pass
+
+
+def routed_experts(hidden, ffn, top_k, gate, up, down, down_type, codes, deltas, sums, ids, exp_kind=EXP_GFX1151,
+                   gate_expert_stride=None, gate_row_stride=None, down_expert_stride=None, down_row_stride=None,
+                   threads=0, want_intermediates=True, down_only_from=None):
+    """gate/up/down: uint8 arrays holding every expert (GGUF order unless strides are given).
+    down_only_from: (h_codes, h_deltas, h_sums) -> run the down phase alone on that image."""
+    gate = np.ascontiguousarray(gate, np.uint8)
+    up = np.ascontiguousarray(up, np.uint8)
+    down = np.ascontiguousarray(down, np.uint8)
+    rows = codes.shape[0]
+    grb = gate_row_stride or hidden // 256 * Q4_K_BLOCK
+    geb = gate_expert_stride or grb * ffn
+    drb = down_row_stride or row_bytes(down_type, ffn)
+    deb = down_expert_stride or drb * hidden
+    w = ExpertWeights(hidden, ffn, 0, top_k, Q4_K, down_type, gate.ctypes.data, up.ctypes.data, down.ctypes.data,
+                      geb, grb, deb, drb, exp_kind)
+    ids = np.ascontiguousarray(ids, np.uint32)
+    n = rows * top_k
+    r = ExpertResult()
+    r.rawdots = np.zeros((rows, top_k, hidden), np.float32)
+    r.status = np.zeros(rows, np.uint32)
+    if down_only_from is not None:
+        r.h_codes, r.h_deltas, r.h_sums = (np.ascontiguousarray(a) for a in down_only_from)
+        r.gate = r.up = r.h = None
+    else:
+        r.h_codes = np.zeros((n, ffn), np.int8)
+        r.h_deltas = np.zeros((n, ffn // 32), np.float32)
+        r.h_sums = np.zeros((n, ffn // 32), np.int32)
+        r.gate = np.zeros((n, ffn), np.float32) if want_intermediates else None
+        r.up = np.zeros((n, ffn), np.float32) if want_intermediates else None
+        r.h = np.zeros((n, ffn), np.float32) if want_intermediates else None
+    job = ExpertJob(codes.ctypes.data, deltas.ctypes.data, sums.ctypes.data, ids.ctypes.data, rows,
+                    r.gate.ctypes.data if r.gate is not None else None, r.up.ctypes.data if r.up is not None else None,
+                    r.h.ctypes.data if r.h is not None else None, r.h_codes.ctypes.data, r.h_deltas.ctypes.data,
+                    r.h_sums.ctypes.data, r.rawdots.ctypes.data, r.status.ctypes.data)
+    t = threads or lib().orc_max_threads()
+    if down_only_from is not None:
+        lib().orc_routed_down(C.byref(w), C.byref(job), t)
+        r.bad = 0
+    else:
+        r.bad = lib().orc_routed_experts(C.byref(w), C.byref(job), t)
+    return r
+
+
+def base_linear(qtype, weight, row_stride, outputs, n_in, x, threads=0):
+    weight = np.ascontiguousarray(weight, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    rows = x.shape[0]
+    y = np.zeros((rows, outputs), np.float32)
+    lib().orc_base_linear(qtype, _ptr(weight, u8p), C.c_uint64(row_stride), outputs, n_in, _ptr(x, f32p), rows,
+                          x.shape[1], _ptr(y, f32p), outputs, threads or lib().orc_max_threads())
+    return y

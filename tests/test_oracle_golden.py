@@ -1,0 +1,777 @@
+"""Pins the CPU oracle (oracle/strix_oracle.c) WITHOUT the GPU:
+  * the literal vectors the reference's own host tests hold for this path (tests/golden/reference_literals.json),
+  * closed forms / brute force / invariants chosen so that a plausible mistake fails,
+  * mutation checks (a wrong order, a fused multiply-add, a swapped nibble must change the bits),
+  * bitwise equality with the compiled reference (oracle/_ref) where that library was built,
+  * the committed reference-generated vectors (tests/golden/ref_vectors.npz)."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+import orc
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIT = json.load(open(os.path.join(HERE, "golden", "reference_literals.json")))
+
+
+def f32_from_bits(b):
+    return np.array([int(b, 16) if isinstance(b, str) else b], np.uint32).view(np.float32)[0]
+
+
+def bits(x):
+    return np.asarray(x, np.float32).view(np.uint32)
+
+
+# ---------------------------------------------------------------- fp16
+def test_half_to_float_all_65536_values():
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([orc.half_to_float(int(v)) for v in h], np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(bits(got)[~nan], bits(want)[~nan])
+
+
+def test_float_to_half_round_trip_and_ties():
+    h = np.arange(65536, dtype=np.uint16)
+    f = h.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(f)
+    back = np.array([orc.float_to_half(v) for v in f[ok]], np.uint16)
+    assert np.array_equal(back, h[ok])
+    rng = np.random.default_rng(5)
+    sample = np.concatenate([rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 20000).astype(np.float32),
+                             # exact midpoints between neighbouring halves: ties must go to even
+                             ((f[ok][:-1].astype(np.float64) + f[ok][1:].astype(np.float64)) / 2).astype(np.float32)[::7]])
+    sample = sample[np.isfinite(sample)]
+    with np.errstate(over="ignore"):
+        want = sample.astype(np.float16).view(np.uint16)
+    got = np.array([orc.float_to_half(v) for v in sample], np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- Q8_0 decode / writer
+def test_q8_0_dequant_closed_form():
+    rng = np.random.default_rng(1)
+    raw = rng.integers(0, 256, (5, 4 * 34), dtype=np.uint8)
+    raw[:, 1::34] &= 0x7B  # finite scales
+    got = orc.dequant_rows(orc.Q8_0, raw, 128)
+    blocks = raw.reshape(5, 4, 34)
+    d = blocks[:, :, :2].copy().view(np.float16).astype(np.float32)
+    want = (blocks[:, :, 2:].view(np.int8).astype(np.float32) * d).reshape(5, 128)
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_q8_0_writer_reference_literals():
+    for case in LIT["q8_0_writer"]["cases"]:
+        v = np.zeros(32, np.float32)
+        if case.get("ramp"):
+            v = (np.arange(32) - 16).astype(np.float32)
+        for k, x in case.get("values", {}).items():
+            v[int(k)] = x
+        packed = orc.quantize_rows(orc.Q8_0, v[None, :])[0]
+        d = np.float32(case["d"]) if "d" in case else np.float32(case["d_num"]) / np.float32(case["d_den"])
+        assert packed[:2].view(np.uint16)[0] == orc.float_to_half(d), case["name"]
+        codes = packed[2:].view(np.int8)
+        for k, c in case["codes"].items():
+            assert codes[int(k)] == c, (case["name"], k)
+
+
+# ---------------------------------------------------------------- Q4_K decode
+def _independent_q4k_value(block, k):
+    """Element k of one 144-byte block from the published layout, written element-wise (no loops shared with the oracle)."""
+    g, l = k // 32, k % 32
+    s = block[4:16].astype(np.uint32)
+    if g < 4:
+        sc, m = s[g] & 63, s[g + 4] & 63
+    else:
+        sc = (s[g + 4] & 15) | ((s[g - 4] >> 6) << 4)
+        m = (s[g + 4] >> 4) | ((s[g] >> 6) << 4)
+    d = block[0:2].copy().view(np.float16)[0].astype(np.float32)
+    dm = block[2:4].copy().view(np.float16)[0].astype(np.float32)
+    q = (int(block[16 + 32 * (g // 2) + l]) >> (4 * (g % 2))) & 15
+    return np.float32(np.float32(d * np.float32(sc)) * np.float32(q)) - np.float32(dm * np.float32(m))
+
+
+def test_q4k_dequant_every_position_brute_force():
+    rng = np.random.default_rng(2)
+    raw = rng.integers(0, 256, (3, 2 * 144), dtype=np.uint8)
+    for r in range(3):
+        for b in range(2):
+            raw[r, b * 144 + 1] &= 0x7B
+            raw[r, b * 144 + 3] &= 0x7B
+    got = orc.dequant_rows(orc.Q4_K, raw, 512)
+    for r in range(3):
+        for k in range(512):
+            want = _independent_q4k_value(raw[r, (k // 256) * 144:(k // 256 + 1) * 144], k % 256)
+            assert bits(got[r, k]) == bits(want), (r, k)
+
+
+def test_q4k_factor_unpack_all_scale_min_group_triples():
+    """Both statements of the 6-bit unpack (byte form and 32-bit-word form) against every (scale, min, group)
+    (the reference sweeps the same 64 x 64 x 8 triples: tests/moe_q4k_a8_contract_tests.cpp:103-118)."""
+    import ctypes as C
+    L = orc.lib()
+    rng = np.random.default_rng(3)
+    block = np.zeros(144, np.uint8)
+    sc_out, m_out = C.c_uint8(0), C.c_uint8(0)
+    for group in range(8):
+        lo = group & 3
+        for s in range(64):
+            for m in range(64):
+                p = rng.integers(0, 256, 12, dtype=np.uint8)
+                if group < 4:
+                    p[lo] = (p[lo] & 192) | s
+                    p[lo + 4] = (p[lo + 4] & 192) | m
+                else:
+                    p[lo] = (p[lo] & 63) | ((s >> 4) << 6)
+                    p[lo + 4] = (p[lo + 4] & 63) | ((m >> 4) << 6)
+                    p[lo + 8] = (s & 15) | ((m & 15) << 4)
+                block[4:16] = p
+                L.orc_q4k_scale_min(block[4:].ctypes.data_as(orc.u8p), group, C.byref(sc_out), C.byref(m_out))
+                assert (sc_out.value, m_out.value) == (s, m)
+                assert L.orc_q4k_factor_words(block.ctypes.data_as(orc.u8p), group, 0) == s
+                assert L.orc_q4k_factor_words(block.ctypes.data_as(orc.u8p), group, 1) == m
+
+
+def test_q4k_writer_round_trip_error_bound():
+    """The writer has no reference counterpart (parity unpinned); it must still produce valid blocks whose decode is
+    within one quantisation step of the input."""
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((4, 1024)) * 0.02).astype(np.float32)
+    x[1, :32] = 0.0
+    x[2, 256:512] = np.abs(x[2, 256:512])
+    packed = orc.quantize_rows(orc.Q4_K, x)
+    y = orc.dequant_rows(orc.Q4_K, packed, 1024)
+    span = (x.reshape(4, -1, 32).max(-1) - np.minimum(x.reshape(4, -1, 32).min(-1), 0)).repeat(32, -1).reshape(4, 1024)
+    assert np.all(np.abs(x - y) <= span / 15 * 0.75 + 1e-6)
+
+
+# ---------------------------------------------------------------- A8 quantiser
+def test_a8_reference_literals():
+    for case in LIT["a8_quantiser"]["cases"]:
+        w = case["width"]
+        v = np.full(w, f32_from_bits(case["fill_bits"]) if "fill_bits" in case else case["fill"], np.float32)
+        for k, x in case.get("set", {}).items():
+            v[int(k)] = x
+        for k, b in case.get("set_bits", {}).items():
+            v[int(k)] = f32_from_bits(b)
+        codes, deltas, sums, rc = orc.quantize_a8(v[None, :], tiny_rule=case.get("tiny_rule", False))
+        src = case["source"]
+        if "all_codes" in case:
+            assert np.all(codes == case["all_codes"]), src
+        for k, c in case.get("codes", {}).items():
+            assert codes[0, int(k)] == c, (src, k)
+        if "delta" in case:
+            assert np.all(deltas == np.float32(case["delta"])), src
+        if "delta_not" in case:
+            assert deltas[0, 0] != np.float32(case["delta_not"]), src
+        if "delta_bits" in case:
+            assert bits(deltas[0, 0]) == int(case["delta_bits"], 16), src
+        if "sum" in case:
+            assert np.all(sums == case["sum"]), src
+
+
+def _rne_ratio(n, d):
+    q, r = divmod(n, d)
+    if r * 2 > d or (r * 2 == d and (q & 1)):
+        q += 1
+    return q
+
+
+def _soft_divide(a, b):
+    """Correctly rounded binary32 quotient from integer significands (independent of the native divide);
+    the reference carries the same construction in tests/q4k_a8_oracle.hpp:20-45."""
+    sign = (a ^ b) & 0x80000000
+    a &= 0x7FFFFFFF
+    b &= 0x7FFFFFFF
+    if a == 0:
+        return sign
+
+    def unpack(x):
+        e = x >> 23
+        m = (x & 0x7FFFFF) | (0x800000 if e else 0)
+        ex = e - 150 if e else -149
+        sh = 24 - m.bit_length()
+        return m << sh, ex - sh
+    ma, ea = unpack(a)
+    mb, eb = unpack(b)
+    diff = ea - eb
+    exponent = diff + (-1 if ma < mb else 0)
+    if exponent < -126:
+        shift = diff + 149
+        if shift < -1:
+            return sign
+        return sign | _rne_ratio(ma << max(shift, 0), mb << max(-shift, 0))
+    if exponent > 127:
+        return sign | 0x7F800000
+    m = _rne_ratio(ma << (diff - exponent + 23), mb)
+    if m == 0x1000000:
+        m >>= 1
+        exponent += 1
+    if exponent > 127:
+        return sign | 0x7F800000
+    return sign | ((exponent + 127) << 23) | (m - 0x800000)
+
+
+def test_a8_against_software_division_at_rounding_boundaries():
+    rng = np.random.default_rng(6)
+    for _ in range(300):
+        amax_bits = int(rng.integers(0x20000000, 0x7F000000))
+        dbits = _soft_divide(amax_bits, 0x42FE0000)
+        delta = f32_from_bits(dbits)
+        amax = f32_from_bits(amax_bits)
+        v = np.zeros(32, np.float32)
+        v[0] = amax
+        for lane in range(1, 32):
+            boundary = np.float32(delta * np.float32(lane + 0.5))
+            x = np.nextafter(boundary, np.float32(0.0) if lane & 1 else amax)
+            v[lane] = -min(amax, x) if lane & 2 else min(amax, x)
+        codes, deltas, sums, _ = orc.quantize_a8(v[None, :], tiny_rule=False)
+        assert bits(deltas[0, 0]) == dbits
+        for lane in range(32):
+            qb = _soft_divide(int(bits(v[lane])), dbits)
+            mag = abs(float(f32_from_bits(qb)))
+            c = math.floor(mag)
+            frac = mag - c
+            if frac > 0.5 or (frac == 0.5 and (c & 1)):
+                c += 1
+            c = min(c, 127)
+            assert codes[0, lane] == (-c if qb & 0x80000000 else c)
+        assert sums[0, 0] == int(codes.astype(np.int32).sum())
+
+
+def test_a8_rejects_partial_group_before_any_write():
+    x = np.ones(64, np.float32)
+    import ctypes as C
+    codes = np.full(64, 17, np.int8)
+    deltas = np.full(2, 19, np.float32)
+    sums = np.full(2, 23, np.int32)
+    for width in (31, 33):
+        rc = orc.lib().orc_quantize_a8(x.ctypes.data_as(orc.f32p), C.c_size_t(width), codes.ctypes.data_as(orc.i8p),
+                                       deltas.ctypes.data_as(orc.f32p), sums.ctypes.data_as(orc.i32p), 1)
+        assert rc == -1 and np.all(codes == 17) and np.all(deltas == 19) and np.all(sums == 23)
+
+
+# ---------------------------------------------------------------- Q8_0 x A8 product order
+def test_q8_0_gemv_order_fixture_distinguishes_lane_and_tree_order():
+    f = LIT["q8_0_gemv"]["product_order"]
+    g = f["groups"]
+    w = np.zeros(g * 34, np.uint8)
+    w[0::34] = int(f["scale_bits"], 16) & 255
+    w[1::34] = int(f["scale_bits"], 16) >> 8
+    w[2::34] = f["first_weight_code"]
+    codes = np.full((1, g * 32), f["codes_fill"], np.int8)
+    deltas = np.zeros((1, g), np.float32)
+    for k, v in f["deltas"].items():
+        deltas[0, int(k)] = v
+    y = np.full((1, 1), f["y_initial"], np.float32)
+    orc.gemv_q8_0_a8(w, codes, deltas, g * 32, 1, out=y)
+    assert y[0, 0] == f["expect_overwrite"]
+    y[:] = f["y_initial"]
+    orc.gemv_q8_0_a8(w, codes, deltas, g * 32, 1, out=y, accumulate=True)
+    assert y[0, 0] == f["expect_accumulate"]
+    # the plain ascending sum gives a different answer, so the fixture really pins the order
+    seq = np.float32(0)
+    for gi in range(g):
+        seq = np.float32(seq + np.float32(32.0) * deltas[0, gi])
+    assert seq != np.float32(f["expect_overwrite"])
+
+
+def test_q8_0_gemv_subnormal_scales_and_padding():
+    import ctypes as C
+    f = LIT["q8_0_gemv"]["subnormal_scales"]
+    w = np.zeros(70, np.uint8)
+    w[0] = 1
+    w[35], w[36] = 0xFF, 0x83
+    w[2:34] = 1
+    w[37:69] = 1
+    codes = np.full((2, 64), 17, np.int8)
+    deltas = np.full((2, 2), 19, np.float32)
+    sums = np.full((2, 2), 23, np.int32)
+    for r, fb in enumerate(f["x_fill_bits"]):
+        x = np.full(32, f32_from_bits(fb), np.float32)
+        orc.lib().orc_quantize_a8(x.ctypes.data_as(orc.f32p), C.c_size_t(32), codes[r].ctypes.data_as(orc.i8p),
+                                  deltas[r].ctypes.data_as(orc.f32p), sums[r].ctypes.data_as(orc.i32p), 1)
+    assert np.all(codes[:, 32:] == 17) and np.all(deltas[:, 1] == 19) and np.all(sums[:, 1] == 23)
+    y = np.full((2, 3), 29, np.float32)
+    v = orc.Q8a8View(w.ctypes.data, codes.ctypes.data, deltas.ctypes.data, y.ctypes.data, 35, 32, 2, 2, 64, 3, 0)
+    assert orc.lib().orc_gemv_q8_0_a8(C.byref(v), 1) == 0
+    e = f["expect"]
+    assert y[0, 0] == 0 and y[0, 1] == 0
+    assert y[1, 0] == np.float32(e["y10_num"]) * np.float32(e["scale"])
+    assert y[1, 1] == np.float32(e["y11_num"]) * np.float32(e["scale"])
+    assert y[0, 2] == 29 and y[1, 2] == 29
+
+
+def test_q8_0_gemv_rejects_partial_group_untouched():
+    import ctypes as C
+    y = np.full((1, 1), 29, np.float32)
+    w = np.zeros(68, np.uint8)
+    codes = np.zeros((1, 64), np.int8)
+    deltas = np.ones((1, 2), np.float32)
+    for width in (31, 33):
+        v = orc.Q8a8View(w.ctypes.data, codes.ctypes.data, deltas.ctypes.data, y.ctypes.data, 68, width, 1, 1, 64, 1, 0)
+        assert orc.lib().orc_gemv_q8_0_a8(C.byref(v), 1) == -1 and y[0, 0] == 29
+
+
+# ---------------------------------------------------------------- Q4_K x A8 row
+def _random_q4k_case(rng, width, headers=None):
+    x = np.ldexp((rng.integers(0, 255, width) - 127).astype(np.float32), rng.integers(-8, 7, width).astype(np.int32)).astype(np.float32)
+    codes, deltas, sums, _ = orc.quantize_a8(x[None, :], tiny_rule=False)
+    w = rng.integers(0, 256, width // 256 * 144, dtype=np.uint8)
+    hs = headers or [0, 0x8000, 1, 0x8001, 0x03FF, 0x83FF, 0x3C00, 0xBC00, 0x7BFF, 0xFBFF]
+    for b in range(width // 256):
+        d, dm = (hs[int(rng.integers(len(hs)))] for _ in range(2))
+        w[b * 144:b * 144 + 4] = [d & 255, d >> 8, dm & 255, dm >> 8]
+    return w, codes[0], deltas[0], sums[0]
+
+
+def _py_q4k_row(w, codes, deltas, sums, mutation=None):
+    """Independent element-wise evaluation in numpy float32 scalars, with the mutation list of the reference's own
+    oracle test (tests/q4k_a8_oracle.hpp:90-127): each mutant must change the bits somewhere."""
+    f = np.float32
+    acc = [f(-0.0) if mutation == "negative_zero_seed" else f(0.0)] * 4
+    nb = codes.size // 256
+    for it in range(nb):
+        b = nb - 1 - it if mutation == "reverse_blocks" else it
+        blk = w[b * 144:(b + 1) * 144]
+        d = blk[0:2].copy().view(np.float16)[0].astype(f)
+        dm = blk[2:4].copy().view(np.float16)[0].astype(f)
+        if mutation == "header_swap":
+            d, dm = dm, d
+        c = []
+        for j in range(8):
+            pair = j // 2
+            sel = (j ^ 1) if mutation == "nibble_swap" else j
+            q = (blk[16 + 32 * pair:16 + 32 * pair + 32].astype(np.int64) >> (4 * (sel & 1))) & 15
+            a = codes[b * 256 + j * 32:b * 256 + j * 32 + 32].astype(np.int64)
+            if mutation == "unsigned_a":
+                a = a & 255
+            dot = int((q * a).sum())
+            s = int(codes[b * 256 + j * 32:b * 256 + j * 32 + 32].astype(np.int64).sum())
+            sc, m = int(orc.lib().orc_q4k_factor_words(blk.ctypes.data_as(orc.u8p), j, 0)), int(orc.lib().orc_q4k_factor_words(blk.ctypes.data_as(orc.u8p), j, 1))
+            if mutation == "factor_swap":
+                sc, m = m, sc
+            i, k = f(sc * dot), f(m * s)
+            if mutation == "fused":
+                t = f(float(d) * float(i) - float(f(dm * k)))  # one rounding of d*i - RN(dm*k): double is exact enough for 24x24 bits
+            else:
+                t = f(f(d * i) - f(dm * k))
+            c.append(f(deltas[b * 8 + j] * t))
+        for p in range(4):
+            acc[p] = f(acc[p] + f(c[2 * p] + c[2 * p + 1]))
+    if mutation == "missing_xor4":
+        return f(acc[0] + acc[1])
+    if mutation == "wrong_tree":
+        return f(f(acc[0] + acc[2]) + f(acc[1] + acc[3]))
+    return f(f(acc[0] + acc[1]) + f(acc[2] + acc[3]))
+
+
+def test_q4k_row_three_formulations_agree_and_mutants_differ():
+    rng = np.random.default_rng(7)
+    mutants = ["fused", "reverse_blocks", "wrong_tree", "nibble_swap", "header_swap", "factor_swap", "unsigned_a", "missing_xor4"]
+    detected = dict.fromkeys(mutants, False)
+    with np.errstate(all="ignore"):
+        for width in (256, 512, 2560):
+            for _ in range(25):
+                w, codes, deltas, sums = _random_q4k_case(rng, width)
+                a = orc.q4k_row_a8(w, codes, deltas, sums)
+                b = orc.q4k_row_a8(w, codes, deltas, sums, contract_form=True)
+                c = _py_q4k_row(w, codes, deltas, sums)
+                if np.isnan(c):
+                    assert np.isnan(a) and np.isnan(b)
+                    continue
+                assert bits(a) == bits(b) == bits(c)
+                for m in mutants:
+                    detected[m] |= bool(bits(_py_q4k_row(w, codes, deltas, sums, m)) != bits(c))
+    assert all(detected.values()), detected
+
+
+def test_q4k_zero_row_is_plus_zero():
+    f = LIT["q4k_zero_row"]
+    w = np.full(144, f["fill_byte"], np.uint8)
+    w[:4] = f["header"]
+    codes, deltas, sums, _ = orc.quantize_a8(np.zeros((1, 256), np.float32), tiny_rule=False)
+    assert bits(orc.q4k_row_a8(w, codes[0], deltas[0], sums[0])) == int(f["expect_bits"], 16)
+    assert bits(_py_q4k_row(w, codes[0], deltas[0], sums[0], "negative_zero_seed")) == 0x80000000
+
+
+def test_q8_0_down_row_reference_literal_and_chain_order():
+    f = LIT["down_rows"]["q8_0"]
+    w = np.zeros(f["groups"] * 34, np.uint8)
+    w[0::34] = int(f["scale_bits"], 16) & 255
+    w[1::34] = int(f["scale_bits"], 16) >> 8
+    for g in range(f["groups"]):
+        w[g * 34 + 2:(g + 1) * 34] = f["weight_byte"]
+    codes = np.full(f["groups"] * 32, f["codes_fill"], np.int8)
+    deltas = np.full(f["groups"], f["delta"], np.float32)
+    assert orc.q8_0_down_row_a8(w, codes, deltas) == np.float32(f["expect"])
+    # cancellation witness for the 4-chain tree: terms 2^30, 1, -2^30, 1 -> (a0+a1)+(a2+a3) = 0, ascending sum = 1
+    w2 = np.zeros(4 * 34, np.uint8)
+    w2[0::34], w2[1::34] = 0x00, 0x3C
+    w2[2::34] = 1
+    c2 = np.zeros(128, np.int8)
+    c2[0::32] = 1
+    d2 = np.array([2.0 ** 30, 1.0, -2.0 ** 30, 1.0], np.float32)
+    assert orc.q8_0_down_row_a8(w2, c2, d2) == 0.0
+
+
+# ---------------------------------------------------------------- exp / SwiGLU
+def test_declared_exp_accuracy_and_limits():
+    xs = np.linspace(-100, 88, 4001).astype(np.float32)
+    got = np.array([orc.lib().orc_declared_exp(float(x)) for x in xs], np.float64)
+    want = np.exp(xs.astype(np.float64))
+    ok = want > 1e-37
+    assert np.max(np.abs(got[ok] / want[ok] - 1)) < 4e-7
+    assert orc.lib().orc_declared_exp(89.0) == math.inf and orc.lib().orc_declared_exp(-104.0) == 0.0
+    assert orc.lib().orc_declared_exp(0.0) == 1.0
+
+
+def test_gfx1151_exp_without_tables_is_correctly_rounded_in_range():
+    rng = np.random.default_rng(8)
+    xs = (rng.uniform(-80, 80, 20000)).astype(np.float32)
+    got = np.array([orc.lib().orc_expf_gfx1151(float(x)) for x in xs], np.float32)
+    want = np.exp(xs.astype(np.float64))
+    # exp2 of the reduced argument is correctly rounded; the reduction adds well under half an ulp
+    assert np.max(np.abs(got.astype(np.float64) / want - 1)) < 1.2e-7
+    assert orc.lib().orc_expf_gfx1151(-104.0) == 0.0 and orc.lib().orc_expf_gfx1151(89.0) == math.inf
+
+
+def test_swiglu_quantize_matches_elementwise_definition_and_fails_closed():
+    rng = np.random.default_rng(9)
+    g = rng.standard_normal(32).astype(np.float32) * 3
+    u = rng.standard_normal(32).astype(np.float32) * 3
+    ok, codes, delta, s, h = orc.swiglu_quantize(g, u)
+    f = np.float32
+    hv = np.array([f(f(g[i] / f(f(1.0) + f(orc.lib().orc_expf_gfx1151(float(-g[i]))))) * u[i]) for i in range(32)], np.float32)
+    assert ok == 1 and np.array_equal(bits(h), bits(hv))
+    c2, d2, s2, _ = orc.quantize_a8(hv[None, :], tiny_rule=True)
+    assert np.array_equal(codes, c2[0]) and bits(delta) == bits(d2[0, 0]) and s == s2[0, 0]
+    g[5] = np.inf
+    ok, codes, *_ = orc.swiglu_quantize(g, u)
+    assert ok == 0 and np.all(codes == 0)
+
+
+# ---------------------------------------------------------------- router
+def test_router_selection_equals_stable_sort_and_weight_bits():
+    rng = np.random.default_rng(10)
+    for experts, top_k in ((128, 8), (256, 8), (160, 8), (64, 1)):
+        for _ in range(20):
+            z = (rng.integers(-512, 513, experts) / 64.0).astype(np.float32)  # 1/64 grid: exact ties
+            m = z.max()
+            p = np.array([orc.lib().orc_declared_exp(float(np.float32(v - m))) for v in z], np.float32)
+            tot = np.float32(0)
+            for v in p:
+                tot = np.float32(tot + v)
+            s = (p / tot).astype(np.float32)
+            ids, w = orc.route_select(s, top_k, renorm_eps=1e-20, scale=2.5)
+            want = sorted(range(experts), key=lambda e: (-s[e], e))[:top_k]
+            assert list(ids) == want
+            acc = np.float32(0)
+            for e in ids:
+                acc = np.float32(acc + s[e])
+            den = np.float32(acc + np.float32(1e-20))
+            for k, e in enumerate(ids):
+                assert bits(w[k]) == bits(np.float32(np.float32(s[e] / den) * np.float32(2.5)))
+    s = np.full(16, 0.25, np.float32)
+    ids, _ = orc.route_select(s, 4)
+    assert list(ids) == [0, 1, 2, 3]
+
+
+def test_router_logit_chains_softmax_and_bias():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((3, 96)).astype(np.float32)
+    w = (rng.standard_normal((16, 96)) * 0.02).astype(np.float32)
+    bias = rng.standard_normal(16).astype(np.float32)
+    ids, wt, scores, logits = orc.route(x, w, 4, bias=bias)
+    for r in range(3):
+        for e in range(16):
+            acc = 0.0
+            for k in range(96):  # fma in double then one rounding == fmaf for 24-bit operands
+                acc = float(np.float32(float(x[r, k]) * float(w[e, k]) + acc))
+            assert bits(logits[r, e]) == bits(np.float32(np.float32(acc) + bias[e]))
+        assert abs(float(scores[r].sum()) - 1) < 1e-5
+        assert list(ids[r]) == sorted(range(16), key=lambda e: (-scores[r, e], e))[:4]
+    _, _, _, lg2 = orc.route(x, w, 4, logits_order=orc.LOGITS_LANE32)
+    for r in range(3):
+        for e in range(16):
+            assert bits(lg2[r, e]) == bits(np.float32(orc.lib().orc_lane_dot((w[e] * 1).ctypes.data_as(orc.f32p), x[r].ctypes.data_as(orc.f32p), 96)))
+    assert np.max(np.abs(lg2 - (logits - bias))) < 1e-5
+
+
+# ---------------------------------------------------------------- combine
+def test_combine_forms_and_commit_threshold():
+    rng = np.random.default_rng(12)
+    raw = rng.standard_normal((2, 4, 8)).astype(np.float32)
+    w = rng.random((2, 4)).astype(np.float32)
+    ids = np.array([[7, 2, 9, 0], [1, 5, 3, 4]], np.uint32)
+    base = rng.standard_normal((2, 8)).astype(np.float32)
+    y = orc.combine(orc.COMBINE_FMA_SLOT, w, ids, raw, base)
+    z = orc.combine(orc.COMBINE_MULADD_ASC, w, ids, raw)
+    for r in range(2):
+        for d in range(8):
+            acc = np.float32(0)
+            for k in range(4):
+                acc = np.float32(float(w[r, k]) * float(raw[r, k, d]) + float(acc))
+            assert bits(y[r, d]) == bits(np.float32(acc + base[r, d]))
+            s = np.float32(0)
+            for k in np.argsort(ids[r], kind="stable"):
+                s = np.float32(s + np.float32(w[r, k] * raw[r, k, d]))
+            assert bits(z[r, d]) == bits(s)
+    assert int(LIT["commit_threshold"]["bf16_bits"], 16) == 0x7F7F8000
+
+
+# ---------------------------------------------------------------- whole layer, brute force on tiny shapes
+def _tiny_layer(rng, H, I, E, T, K, down_type):
+    gate = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32))
+    up = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32))
+    down = orc.quantize_rows(down_type, (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32))
+    x = rng.standard_normal((T, H)).astype(np.float16).astype(np.float32)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.uint32)
+    return gate, up, down, x, ids
+
+
+@pytest.mark.parametrize("down_type", [orc.Q4_K, orc.Q8_0])
+def test_routed_experts_against_double_precision_dequant_reference(down_type):
+    """Brute force: A8-quantise explicitly, dequantise weights with the (separately pinned) block decoders, sum in
+    double. The declared fp32 chain must agree to fp32 accumulation accuracy; a dropped term or a wrong index is O(1)."""
+    rng = np.random.default_rng(13)
+    H, I, E, T, K = 512, 256, 6, 3, 2
+    gate, up, down, x, ids = _tiny_layer(rng, H, I, E, T, K, down_type)
+    codes, deltas, sums, _ = orc.quantize_a8(x)
+    r = orc.routed_experts(H, I, K, gate, up, down, down_type, codes, deltas, sums, ids)
+    assert r.bad == 0 and np.all(r.status == 0)
+    xa = (codes.astype(np.float64) * np.repeat(deltas.astype(np.float64), 32, axis=1))
+    for t in range(T):
+        for k in range(K):
+            e = ids[t, k]
+            a = t * K + k
+            G = orc.dequant_rows(orc.Q4_K, gate[e], H).astype(np.float64) @ xa[t]
+            U = orc.dequant_rows(orc.Q4_K, up[e], H).astype(np.float64) @ xa[t]
+            assert np.max(np.abs(r.gate[a] - G)) < 2e-5 * max(1, np.abs(G).max())
+            assert np.max(np.abs(r.up[a] - U)) < 2e-5 * max(1, np.abs(U).max())
+            ha = r.h_codes[a].astype(np.float64) * np.repeat(r.h_deltas[a].astype(np.float64), 32)
+            hd = r.gate[a].astype(np.float64) / (1 + np.exp(-r.gate[a].astype(np.float64))) * r.up[a].astype(np.float64)
+            assert np.max(np.abs(ha - hd)) <= np.abs(hd).reshape(-1, 32).max(-1).repeat(32).max() / 127 * 0.51 + 1e-9
+            D = orc.dequant_rows(down_type, down[e], I).astype(np.float64) @ ha
+            assert np.max(np.abs(r.rawdots[t, k] - D)) < 2e-5 * max(1, np.abs(D).max())
+    # the down phase alone, from the same h image, gives the same bits (stage-by-stage form used by the GPU tests)
+    r2 = orc.routed_experts(H, I, K, gate, up, down, down_type, codes, deltas, sums, ids, down_only_from=(r.h_codes, r.h_deltas, r.h_sums))
+    assert np.array_equal(bits(r2.rawdots), bits(r.rawdots))
+    # thread count never changes a bit
+    r1 = orc.routed_experts(H, I, K, gate, up, down, down_type, codes, deltas, sums, ids, threads=1)
+    assert np.array_equal(bits(r1.rawdots), bits(r.rawdots)) and np.array_equal(r1.h_codes, r.h_codes)
+
+
+def test_routed_experts_nonfinite_row_sets_status_and_skips_down():
+    rng = np.random.default_rng(14)
+    H, I, E, T, K = 256, 128, 3, 2, 2
+    gate, up, down, x, ids = _tiny_layer(rng, H, I, E, T, K, orc.Q8_0)
+    codes, deltas, sums, _ = orc.quantize_a8(x)
+    deltas[1, 3] = 3.0e38  # the host-forceable failure of tests/cpu/routed_expert_host_tests.cpp:393-406
+    r = orc.routed_experts(H, I, K, gate, up, down, orc.Q8_0, codes, deltas, sums, ids)
+    assert r.bad == 1 and r.status[0] == 0 and r.status[1] & 8
+    assert np.all(r.rawdots == 0)
+
+
+def test_tp_rank_partials_tile_the_unsplit_expert():
+    """Expert tensor-parallel split by the intermediate dimension: each rank's gate/up rows and h groups are exactly
+    the unsplit expert's (whole 32-groups move), and the two rank partials sum to the unsplit down product up to fp32
+    reassociation (the split is its own arithmetic identity: include/strix/ds41_expert_tp.hpp:3-19)."""
+    rng = np.random.default_rng(15)
+    H, I, E, T, K = 512, 512, 4, 2, 2
+    gate, up, down, x, ids = _tiny_layer(rng, H, I, E, T, K, orc.Q4_K)
+    codes, deltas, sums, _ = orc.quantize_a8(x)
+    full = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, codes, deltas, sums, ids)
+    half = I // 2
+    grb, drb = H // 256 * 144, I // 256 * 144
+    parts = []
+    for rank in range(2):
+        g = gate.reshape(-1)[rank * half * grb:]
+        u = up.reshape(-1)[rank * half * grb:]
+        d = down.reshape(-1)[rank * (half // 256) * 144:]
+        p = orc.routed_experts(H, half, K, g, u, d, orc.Q4_K, codes, deltas, sums, ids, gate_expert_stride=I * grb,
+                               gate_row_stride=grb, down_expert_stride=H * drb, down_row_stride=drb)
+        assert np.array_equal(p.h_codes, full.h_codes[:, rank * half:(rank + 1) * half])
+        assert np.array_equal(bits(p.h_deltas), bits(full.h_deltas[:, rank * half // 32:(rank + 1) * half // 32]))
+        assert np.array_equal(bits(p.gate), bits(full.gate[:, rank * half:(rank + 1) * half]))
+        parts.append(p.rawdots)
+    total = parts[0].astype(np.float64) + parts[1].astype(np.float64)
+    assert np.max(np.abs(total - full.rawdots)) < 1e-5 * np.abs(full.rawdots).max()
+    assert not np.array_equal(bits(parts[0]), bits(full.rawdots))
+
+
+def test_base_linear_matches_numpy_double():
+    rng = np.random.default_rng(16)
+    wq = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((8, 512)) * 0.02).astype(np.float32))
+    x = rng.standard_normal((3, 512)).astype(np.float16).astype(np.float32)
+    y = orc.base_linear(orc.Q4_K, wq, 2 * 144, 8, 512, x)
+    want = x.astype(np.float64) @ orc.dequant_rows(orc.Q4_K, wq, 512).astype(np.float64).T
+    assert np.array_equal(bits(y), bits(want.astype(np.float32)))
+
+
+# ---------------------------------------------------------------- bitwise against the compiled reference
+needs_ref = pytest.mark.skipif(orc.ref() is None, reason="oracle/_ref not built (no reference tree at build time)")
+
+
+@needs_ref
+def test_ref_half_and_dequant_bits():
+    import ctypes as C
+    R = orc.ref()
+    for h in range(0, 65536, 1):
+        a, b = orc.half_to_float(h), R.ref_half_to_float(C.c_uint16(h))
+        assert (math.isnan(a) and math.isnan(b)) or bits(a) == bits(b)
+    rng = np.random.default_rng(20)
+    for qtype, rb, n in ((orc.Q8_0, 34 * 8, 256), (orc.Q4_K, 144 * 2, 512)):
+        raw = rng.integers(0, 256, (16, rb), dtype=np.uint8)
+        mine = orc.dequant_rows(qtype, raw, n)
+        theirs = np.zeros_like(mine)
+        for r in range(16):
+            assert R.ref_dequantize_row(qtype, raw[r].ctypes.data_as(orc.u8p), C.c_size_t(rb), theirs[r].ctypes.data_as(orc.f32p), C.c_size_t(n)) == 0
+        assert np.array_equal(bits(mine), bits(theirs))
+
+
+@needs_ref
+def test_ref_a8_and_q8_0_gemv_bits():
+    import ctypes as C
+    R = orc.ref()
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((4, 1024)).astype(np.float32)
+    x[1, :32] = 0
+    x[2, 32:64] = 1e-37
+    codes, deltas, sums, _ = orc.quantize_a8(x, tiny_rule=True)
+    c2, d2, s2 = np.zeros_like(codes), np.zeros_like(deltas), np.zeros_like(sums)
+    for r in range(4):
+        assert R.ref_quantize_a8(x[r].ctypes.data_as(orc.f32p), C.c_size_t(1024), c2[r].ctypes.data_as(orc.i8p),
+                                 d2[r].ctypes.data_as(orc.f32p), s2[r].ctypes.data_as(orc.i32p)) == 0
+    assert np.array_equal(codes, c2) and np.array_equal(bits(deltas), bits(d2)) and np.array_equal(sums, s2)
+    w = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((96, 1024)) * 0.02).astype(np.float32))
+    y, rc = orc.gemv_q8_0_a8(w, codes, deltas, 1024, 96, threads=3)
+    y2 = np.zeros_like(y)
+    v = orc.Q8a8View(w.ctypes.data, codes.ctypes.data, deltas.ctypes.data, y2.ctypes.data, 1024 // 32 * 34, 1024, 96, 4, 1024, 96, 0)
+    assert R.ref_gemv_q8_0_a8(C.byref(v)) == 0
+    assert np.array_equal(bits(y), bits(y2))
+
+
+@needs_ref
+def test_ref_q4k_row_and_down_row_bits_at_config_widths():
+    import ctypes as C
+    R = orc.ref()
+    rng = np.random.default_rng(22)
+    out = C.c_float(0)
+    for width in (256, 2048, 768, 1280, 2560):   # contract oracle caps: hidden <= 2560
+        for _ in range(8):
+            x = (rng.standard_normal(width) * rng.choice([1e-3, 1.0, 30.0])).astype(np.float32)
+            codes, deltas, sums, _ = orc.quantize_a8(x[None, :], tiny_rule=False)
+            w = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((1, width)) * 0.02).astype(np.float32))[0]
+            mine = orc.q4k_row_a8(w, codes[0], deltas[0], sums[0])
+            assert R.ref_q4k_evaluate_row(w.ctypes.data_as(orc.u8p), C.c_size_t(w.size), codes[0].ctypes.data_as(orc.i8p),
+                                          deltas[0].ctypes.data_as(orc.f32p), sums[0].ctypes.data_as(orc.i32p), C.c_size_t(width), C.byref(out)) == 0, R.ref_last_error()
+            assert bits(mine) == bits(np.float32(out.value))
+    for width in (5120, 27648, 4096, 6144):       # the host executor's row kernel has no cap
+        x = rng.standard_normal(width).astype(np.float32)
+        codes, deltas, sums, _ = orc.quantize_a8(x[None, :])
+        w = rng.integers(0, 256, width // 256 * 144, dtype=np.uint8)
+        w[1::144] = (w[1::144] & 0x03) | 0x10
+        w[3::144] = (w[3::144] & 0x03) | 0x10
+        R.ref_gate_row_q4k(w.ctypes.data_as(orc.u8p), width // 256, codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
+                           sums[0].ctypes.data_as(orc.i32p), C.byref(out))
+        assert bits(orc.q4k_row_a8(w, codes[0], deltas[0], sums[0])) == bits(np.float32(out.value))
+        w8 = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((1, width)) * 0.02).astype(np.float32))[0]
+        R.ref_down_row_q8_0(w8.ctypes.data_as(orc.u8p), width // 32, codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
+                            sums[0].ctypes.data_as(orc.i32p), C.byref(out))
+        assert bits(orc.q8_0_down_row_a8(w8, codes[0], deltas[0])) == bits(np.float32(out.value))
+
+
+@needs_ref
+def test_ref_exp_functions_bits():
+    R = orc.ref()
+    rng = np.random.default_rng(23)
+    xs = np.concatenate([rng.uniform(-110, 95, 40000), rng.standard_normal(40000) * 4, [0.0, -0.0, 88.0, -103.0, 88.7, -104.0]]).astype(np.float32)
+    for x in xs:
+        assert bits(orc.lib().orc_declared_exp(float(x))) == bits(R.ref_declared_exp(float(x)))
+        assert bits(orc.lib().orc_expf_gfx1151(float(x))) == bits(R.ref_gfx1151_expf_empty_tables(float(x)))
+
+
+@needs_ref
+def test_ref_whole_routed_expert_job_bits():
+    """reference_run and the pooled executor (scalar and AVX2 tables) against the restated layer: Q4_K gate/up, Q8_0 down."""
+    import ctypes as C
+    R = orc.ref()
+    rng = np.random.default_rng(24)
+    H, I, E, T, K = 512, 256, 6, 5, 3
+    gate, up, down, x, ids = _tiny_layer(rng, H, I, E, T, K, orc.Q8_0)
+    codes, deltas, sums, _ = orc.quantize_a8(x)
+    mine = orc.routed_experts(H, I, K, gate, up, down, orc.Q8_0, codes, deltas, sums, ids)
+    asg = np.array([[t, k, ids[t, k]] for t in range(T) for k in range(K)], np.uint32)
+    for threads, simd in ((0, 0), (1, 0), (3, 1), (8, 1)):
+        raw = np.zeros((T, K, H), np.float32)
+        status = np.zeros(T, np.uint32)
+        rc = R.ref_routed_expert_run(H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down.ctypes.data_as(orc.u8p),
+                                     codes.ctypes.data_as(orc.i8p), deltas.ctypes.data_as(orc.f32p), sums.ctypes.data_as(orc.i32p), T,
+                                     asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
+                                     status.ctypes.data_as(orc.u32p), threads, simd)
+        assert rc == 0, R.ref_last_error()
+        assert np.array_equal(bits(raw), bits(mine.rawdots)) and np.all(status == 0)
+
+
+@needs_ref
+def test_ref_router_policy_and_combine_bits():
+    import ctypes as C
+    R = orc.ref()
+    rng = np.random.default_rng(25)
+    for experts, top_k in ((128, 8), (256, 8), (160, 8)):
+        z = (rng.standard_normal(experts) * 0.9).astype(np.float32)
+        z[5] = z[17]  # an exact tie
+        s_ref = np.zeros(experts, np.float32)
+        assert R.ref_route_scores_softmax(z.ctypes.data_as(orc.f32p), C.c_size_t(experts), s_ref.ctypes.data_as(orc.f32p), 0) == 0
+        x = np.zeros((1, 1), np.float32)
+        # drive the oracle's softmax with the same logits: hidden 1, x = 1, w = z  (fma(1, z, 0) = z)
+        ids, w, scores, logits = orc.route(np.ones((1, 1), np.float32), z[:, None].copy(), top_k, renorm_eps=0.0)
+        assert np.array_equal(bits(scores[0]), bits(s_ref))
+        ids_ref, w_ref = np.zeros(top_k, np.uint32), np.zeros(top_k, np.float32)
+        assert R.ref_route_select(experts, top_k, C.c_float(0.0), C.c_float(1.0), 1, s_ref.ctypes.data_as(orc.f32p),
+                                  ids_ref.ctypes.data_as(orc.u32p), w_ref.ctypes.data_as(orc.f32p)) == 0
+        assert np.array_equal(ids[0], ids_ref) and np.array_equal(bits(w[0]), bits(w_ref))
+    raw = rng.standard_normal((3, 8, 64)).astype(np.float32)
+    w = rng.random((3, 8)).astype(np.float32)
+    base = rng.standard_normal((3, 64)).astype(np.float32)
+    y_ref = np.zeros((3, 64), np.float32)
+    assert R.ref_combine_fma(3, 8, 64, w.ctypes.data_as(orc.f32p), raw.ctypes.data_as(orc.f32p), base.ctypes.data_as(orc.f32p),
+                             y_ref.ctypes.data_as(orc.f32p)) == 0
+    y = orc.combine(orc.COMBINE_FMA_SLOT, w, np.zeros((3, 8), np.uint32), raw, base)
+    assert np.array_equal(bits(y), bits(y_ref))
+
+
+# ---------------------------------------------------------------- committed reference-generated vectors
+def test_committed_reference_vectors():
+    """tests/golden/ref_vectors.npz holds outputs the compiled reference produced (tests/golden/make_ref_vectors.py);
+    the inputs are regenerated from their seeds here, so this runs where the reference tree is absent."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_ref_vectors", os.path.join(HERE, "golden", "make_ref_vectors.py"))
+    mk = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mk)
+    gold = np.load(os.path.join(HERE, "golden", "ref_vectors.npz"))
+    for seed, H, I, E, T, K in mk.LAYER_CASES:
+        gate, up, down, x, ids = mk.layer_case(seed, H, I, E, T, K)
+        codes, deltas, sums, _ = orc.quantize_a8(x)
+        r = orc.routed_experts(H, I, K, gate, up, down, orc.Q8_0, codes, deltas, sums, ids, want_intermediates=False)
+        assert np.array_equal(bits(r.rawdots), gold[f"layer_{seed}_rawdots_bits"]), seed
+    rng = np.random.default_rng(300)
+    vals = []
+    for width in mk.ROW_WIDTHS:
+        w = mk.random_q4k(rng, 1, width)[0]
+        x = rng.standard_normal(width).astype(np.float32)
+        codes, deltas, sums, _ = orc.quantize_a8(x[None, :])
+        vals.append(orc.q4k_row_a8(w, codes[0], deltas[0], sums[0]))
+    assert np.array_equal(bits(np.array(vals, np.float32)), gold["q4k_rows_bits"])
+    for seed, width, count, rows in mk.GEMV_CASES:
+        rng = np.random.default_rng(seed)
+        w = mk.random_q8_0(rng, count, width)
+        x = rng.standard_normal((rows, width)).astype(np.float32)
+        codes, deltas, sums, _ = orc.quantize_a8(x)
+        y, _ = orc.gemv_q8_0_a8(w, codes, deltas, width, count, threads=2)
+        assert np.array_equal(bits(y), gold[f"gemv_{seed}_bits"])
