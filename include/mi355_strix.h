@@ -1,0 +1,180 @@
+/*
+ * mi355_strix.h - C ABI of the MI355X (gfx950) implementation of the engine's quantized weight-product path:
+ * GGUF Q8_0 / Q4_K decode products on int8 ("A8") activations, the softmax MoE router, the expert-grouped
+ * SwiGLU gate/up/down products with the ordered combine, and one rank's partial sums of the expert
+ * tensor-parallel split. Plain pointers and sizes only; every pointer is DEVICE memory unless said otherwise.
+ *
+ * Conventions (those of the reference's enqueue_* entry points, include/strix/hip_moe_q4k_a8_probe.hpp:8-11):
+ *   - an entry point validates its arguments on the host, then only enqueues kernels on `stream`; it never
+ *     allocates, synchronises, resets or reads back. The caller owns every buffer until the stream is idle.
+ *   - return value: 0 on success; a negative MI355_E_* on an admission failure (nothing was enqueued and no
+ *     buffer was written; mi355_last_error() holds the reason for the calling thread). Nothing throws.
+ *   - numerical problems are reported on the device, in the caller's sticky per-row status words
+ *     (bits below = include/strix/hip_moe_q4k_a8_probe.hpp:7, include/strix/moe_a8_down_contract.hpp:53-54).
+ *   - arithmetic: the reference's A8 class. Every product is an exact int32 group dot followed by the
+ *     declared chain of single-rounding fp32 operations (no contraction), so gate/up/down values and the
+ *     combine are bitwise those of the reference CPU functions named at each entry point.
+ */
+#ifndef MI355_STRIX_H
+#define MI355_STRIX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mi355_stream;   /* hipStream_t */
+
+enum {
+    MI355_OK = 0,
+    MI355_E_INVALID_ARGUMENT = -1,   /* shape / alignment / null pointer: std::invalid_argument in the reference */
+    MI355_E_UNSUPPORTED = -2,        /* a weight type or form this library does not implement */
+    MI355_E_HIP = -3,                /* a HIP runtime call failed (hip_check in the reference) */
+    MI355_E_NO_DEVICE = -4
+};
+
+/* device status word bits */
+enum {
+    MI355_STATUS_INVALID_ROUTE = 1,          /* route id >= experts, or non-finite route weight */
+    MI355_STATUS_NONFINITE_ACTIVATION = 2,   /* non-finite input activation */
+    MI355_STATUS_INVALID_DELTA = 4,
+    MI355_STATUS_NONFINITE_PROJECTION = 8,   /* non-finite gate, up or h; the down phase of the job is skipped */
+    MI355_STATUS_AGGREGATE = 16              /* merged output failed the commit threshold */
+};
+
+enum { MI355_TYPE_Q8_0 = 8, MI355_TYPE_Q4_K = 12 };              /* ggml tensor type ids */
+enum { MI355_INPUT_F32 = 0, MI355_INPUT_F16 = 1, MI355_INPUT_BF16 = 2 };
+enum { MI355_LOGITS_FMA_ASCENDING = 0, MI355_LOGITS_LANE32_BUTTERFLY = 1 };
+enum { MI355_COMBINE_FMA_SLOT_ORDER = 0, MI355_COMBINE_MULADD_ASCENDING_EXPERT = 1 };
+enum { MI355_EXP_GFX1151 = 0, MI355_EXP_DECLARED = 1 };
+
+const char* mi355_last_error(void);
+const char* mi355_version(void);
+/* Numerical identity strings this library implements (the caller opts in by passing them back, as with
+ * Request::approved_numerical_identity, include/strix/moe_q4k_a8_contract.hpp:24-26,104-116). */
+const char* mi355_numerical_identity(uint32_t weight_type, int down);
+
+/* ------------------------------------------------------------------------------------------------------
+ * Block decode. Replaces strix::ggml_dequant::dequantize_row (include/strix/ggml_dequant.hpp:41,
+ * src/ggml_dequant.cpp:84-87,119-130). Row r is read at rows + r * row_stride_bytes and written at
+ * out + r * out_stride (floats). Bitwise the reference's values.
+ */
+int32_t mi355_dequantize_rows(uint32_t weight_type, const void* rows, uint64_t row_stride_bytes, uint32_t n_rows,
+                              uint32_t elements, float* out, uint64_t out_stride, mi355_stream stream);
+
+/* Writers used to build synthetic weights on the device. Q8_0 = strix::q8_0::quantize_group
+ * (include/strix/q8_0_rule.hpp:25-33) with the scale stored as fp16 (round to nearest even). The Q4_K writer has no
+ * counterpart in the reference (it only reads GGUF); it is the min/max writer documented in oracle/strix_oracle.c. */
+int32_t mi355_quantize_weight_rows(uint32_t weight_type, const float* x, uint32_t n_rows, uint32_t elements,
+                                   void* out, mi355_stream stream);
+
+/* ------------------------------------------------------------------------------------------------------
+ * A8 activation quantiser. Replaces strix::cpu::Kernels::quantize_a8 (src/cpu/core/backend.hpp:68-69,
+ * src/cpu/core/reference.cpp:35-55): groups of 32, delta = amax / 127 (1 for an all-zero group or amax < 2^-119),
+ * code = rint(x / delta) clamped to +-127, per-group code sums. width % 32 != 0 -> MI355_E_INVALID_ARGUMENT before any
+ * write. x row r at x + r * x_stride_bytes; codes row r at codes + r * width; deltas / sums row r at + r * width / 32.
+ * sums and status may be NULL. A non-finite input sets status[r] |= MI355_STATUS_NONFINITE_ACTIVATION.
+ */
+int32_t mi355_quantize_a8(const void* x, uint32_t input_kind, uint32_t rows, uint32_t width, uint64_t x_stride_bytes,
+                          int8_t* codes, float* deltas, int32_t* sums, uint32_t* status, mi355_stream stream);
+
+/* ------------------------------------------------------------------------------------------------------
+ * Dense Q8_0 x A8 product. Field for field strix::cpu::Q8a8View (src/cpu/core/backend.hpp:52-59); replaces
+ * strix::cpu::Kernels::gemv_q8_0_a8 (src/cpu/core/backend.hpp:70, src/cpu/core/reference.cpp:57-84):
+ * group g into lane g % 32 ascending, float(dot) * (scale_w * delta_x), tree32, optional out += product.
+ * in % 32 != 0 -> MI355_E_INVALID_ARGUMENT before any write.
+ */
+typedef struct mi355_q8a8_view {
+    const uint8_t* weight;   /* output o at weight + o * row_bytes (2-byte aligned) */
+    const int8_t* codes;     /* A8 codes, row r at codes + r * x_stride */
+    const float* deltas;     /* deltas[r * (x_stride / 32) + k / 32] */
+    float* out;              /* out[r * out_stride + o] */
+    uint32_t row_bytes, in, count, rows, x_stride, out_stride;
+    uint32_t accumulate;
+} mi355_q8a8_view;
+int32_t mi355_gemv_q8_0_a8(const mi355_q8a8_view* view, mi355_stream stream);
+
+/* ------------------------------------------------------------------------------------------------------
+ * Router. Replaces the Qwen route launcher (include/strix/hip_moe_route_launcher.hpp:16-30,
+ * src/hip_moe_route_launcher.hip:322-365) with the host policy's bits (include/strix/moe/route_policy.hpp:99-156):
+ * logits by the per-expert ascending fma chain (or the 32-lane strided sum + butterfly), optional per-expert logit
+ * bias, softmax (max, exp(z - max), ascending sum, divide) with Math::exp = the declared exp
+ * (include/strix/ds41_moe.hpp:38-54), k selection passes in ascending id (greater score wins, lower id on ties),
+ * weights (s / (sum_in_selection_order + renorm_eps)) * scale.
+ */
+typedef struct mi355_route_policy {
+    uint32_t experts, top_k;          /* experts <= 1024, top_k <= 16 */
+    uint32_t logits_order;            /* MI355_LOGITS_* */
+    float renorm_eps, scale;
+    uint32_t renormalize;
+} mi355_route_policy;
+/* x: [rows] activations (input_kind), row r at x + r * x_stride_bytes. router_weight: fp32 [experts][hidden].
+ * logit_bias: fp32 [experts] or NULL. ids / weights: [rows][top_k]. scores: [rows][experts] workspace AND output. */
+int32_t mi355_moe_route(const mi355_route_policy* policy, const void* x, uint32_t input_kind, uint32_t rows,
+                        uint32_t hidden, uint64_t x_stride_bytes, const float* router_weight, const float* logit_bias,
+                        uint32_t* ids, float* weights, float* scores, mi355_stream stream);
+
+/* ------------------------------------------------------------------------------------------------------
+ * Routed experts. The whole-layer form follows the reference's host API for one MoE layer
+ * (include/strix/cuda/qwen_moe.hpp:55-110: Rows / Weights, enqueue_prologue / csr / project / down / merge) and
+ * computes what strix::cpu::expert::reference_run computes (src/cpu/core/routed_expert.cpp:264-300) with Q4_K gate/up
+ * and Q4_K down (down rows by the gate/up row contract: src/moe_a8_down_contract.cpp:146). The single-row C1 forms of
+ * include/strix/hip_moe_q4k_a8_probe.hpp:12 and include/strix/hip_moe_a8_down.hpp:11-30 are rows = 1.
+ */
+typedef struct mi355_moe_weights {
+    uint32_t hidden;      /* multiple of 256 */
+    uint32_t ffn;         /* intermediate rows computed by this call (a TP rank: its share), multiple of 256 */
+    uint32_t experts, top_k;
+    uint32_t gate_type, down_type;                    /* MI355_TYPE_Q4_K */
+    const uint8_t *gate, *up, *down;                  /* GGUF order [experts][ffn][hidden/256], [experts][hidden][ffn/256] */
+    uint64_t gate_expert_stride, gate_row_stride;     /* bytes; 0 = dense GGUF order. 16-byte multiples */
+    uint64_t down_expert_stride, down_row_stride;     /* a TP rank reads the first ffn/256 blocks of each down row */
+    uint32_t exp_kind;                                /* MI355_EXP_* used by SiLU */
+} mi355_moe_weights;
+
+typedef struct mi355_moe_rows {
+    const void* input; uint32_t input_kind; uint64_t input_stride;  /* [rows] activations, stride in bytes */
+    const uint32_t* routes;          /* [rows][top_k] expert ids */
+    const float* route_weights;      /* [rows][top_k] */
+    int8_t* codes; float* deltas; int32_t* sums;      /* A8 image of the input: [rows][hidden], [rows][hidden/32] x2 */
+    uint32_t* status;                /* [rows] sticky status words (cleared by the prologue) */
+    float* gate_out; float* up_out; float* h_out;     /* optional [rows][top_k][ffn] fp32 intermediates, may be NULL */
+    int8_t* down_codes; float* down_deltas; int32_t* down_sums;   /* A8 image of h: [rows][top_k][ffn], [..][ffn/32] x2 */
+    float* rawdots;                  /* [rows][top_k][hidden] unweighted down outputs */
+    const float* base;               /* optional [rows][hidden] added by the merge (shared expert output) */
+    float* output; uint64_t output_stride;            /* [rows][hidden] fp32, stride in floats */
+    uint32_t* plan;                  /* mi355_moe_plan_words(experts, rows, top_k) words, 16-byte aligned */
+    uint32_t* job_status;            /* 1 word: OR of every row's status (decides whether the down phase runs) */
+} mi355_moe_rows;
+
+size_t mi355_moe_plan_words(uint32_t experts, uint32_t rows, uint32_t top_k);
+
+/* prologue: clear status, validate routes and route weights, A8-quantise the input rows. */
+int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, mi355_stream);
+/* csr: the expert grouping plan - assignments (row, slot) of each expert, stable rows-then-slots order
+ * (src/hip_moe_q4k_a8_probe.hip:91-147). */
+int32_t mi355_moe_enqueue_csr(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, mi355_stream);
+/* project: gate and up rows of every touched expert, SwiGLU, A8 re-quantisation of h per 32 outputs. */
+int32_t mi355_moe_enqueue_project(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, mi355_stream);
+/* down: rawdots[row][slot][hidden]; skipped on the device when any row reported a non-finite projection. */
+int32_t mi355_moe_enqueue_down(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, mi355_stream);
+/* merge: ordered combine of the slots (+ base) into output; form = MI355_COMBINE_*. */
+int32_t mi355_moe_enqueue_merge(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, uint32_t form,
+                                mi355_stream);
+/* prologue + csr + project + down + merge. */
+int32_t mi355_moe_enqueue(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, uint32_t combine_form,
+                          mi355_stream);
+
+/* SwiGLU + A8 re-quantisation of h for a dense gate/up pair (the shared expert and the dense FFN):
+ * gate / up: fp32 [rows][ffn]; writes h codes / deltas / sums as above and optionally h values.
+ * Replaces enqueue_down_activation_quantize (include/strix/hip_moe_a8_down.hpp:18) for rows of gate|up. */
+int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows, uint32_t ffn, uint32_t exp_kind,
+                              int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
+                              mi355_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

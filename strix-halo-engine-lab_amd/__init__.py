@@ -1,0 +1,218 @@
+"""Python view of libmi355_strix.so (include/mi355_strix.h) for tests and the benchmark.
+
+torch is used for device memory and streams only; every computation goes through the C ABI. There is no CPU or
+eager fallback: a missing library or a missing GPU raises."""
+import ctypes as C
+import os
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmi355_strix.so")
+
+TYPE_Q8_0, TYPE_Q4_K = 8, 12
+INPUT_F32, INPUT_F16, INPUT_BF16 = 0, 1, 2
+LOGITS_FMA, LOGITS_LANE32 = 0, 1
+COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
+EXP_GFX1151, EXP_DECLARED = 0, 1
+STATUS_INVALID_ROUTE, STATUS_NONFINITE_ACTIVATION, STATUS_INVALID_DELTA, STATUS_NONFINITE_PROJECTION, STATUS_AGGREGATE = 1, 2, 4, 8, 16
+E_INVALID_ARGUMENT, E_UNSUPPORTED, E_HIP = -1, -2, -3
+Q8_0_BLOCK, Q4_K_BLOCK = 34, 144
+
+
+class StrixError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"mi355_strix error {code}: {message}")
+        self.code = code
+
+
+class Q8a8View(C.Structure):
+    _fields_ = [("weight", C.c_void_p), ("codes", C.c_void_p), ("deltas", C.c_void_p), ("out", C.c_void_p),
+                ("row_bytes", C.c_uint32), ("in_", C.c_uint32), ("count", C.c_uint32), ("rows", C.c_uint32),
+                ("x_stride", C.c_uint32), ("out_stride", C.c_uint32), ("accumulate", C.c_uint32)]
+
+
+class RoutePolicy(C.Structure):
+    _fields_ = [("experts", C.c_uint32), ("top_k", C.c_uint32), ("logits_order", C.c_uint32),
+                ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_uint32)]
+
+
+class MoeWeights(C.Structure):
+    _fields_ = [("hidden", C.c_uint32), ("ffn", C.c_uint32), ("experts", C.c_uint32), ("top_k", C.c_uint32),
+                ("gate_type", C.c_uint32), ("down_type", C.c_uint32),
+                ("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p),
+                ("gate_expert_stride", C.c_uint64), ("gate_row_stride", C.c_uint64),
+                ("down_expert_stride", C.c_uint64), ("down_row_stride", C.c_uint64), ("exp_kind", C.c_uint32)]
+
+
+class MoeRows(C.Structure):
+    _fields_ = [("input", C.c_void_p), ("input_kind", C.c_uint32), ("input_stride", C.c_uint64),
+                ("routes", C.c_void_p), ("route_weights", C.c_void_p),
+                ("codes", C.c_void_p), ("deltas", C.c_void_p), ("sums", C.c_void_p), ("status", C.c_void_p),
+                ("gate_out", C.c_void_p), ("up_out", C.c_void_p), ("h_out", C.c_void_p),
+                ("down_codes", C.c_void_p), ("down_deltas", C.c_void_p), ("down_sums", C.c_void_p),
+                ("rawdots", C.c_void_p), ("base", C.c_void_p), ("output", C.c_void_p), ("output_stride", C.c_uint64),
+                ("plan", C.c_void_p), ("job_status", C.c_void_p)]
+
+
+_lib = None
+
+
+def lib():
+    """The HIP library. Raises when it was not built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`")
+        L = C.CDLL(LIB_PATH)
+        L.mi355_last_error.restype = C.c_char_p
+        L.mi355_version.restype = C.c_char_p
+        L.mi355_numerical_identity.restype = C.c_char_p
+        L.mi355_numerical_identity.argtypes = [C.c_uint32, C.c_int]
+        L.mi355_moe_plan_words.restype = C.c_size_t
+        L.mi355_moe_plan_words.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32]
+        _lib = L
+    return _lib
+
+
+EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
+           "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
+           "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_swiglu_quantize"]
+
+
+def require_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU visible: the MI355X kernels cannot run (and nothing falls back to the CPU)")
+    lib()
+
+
+def check(rc):
+    if rc != 0:
+        raise StrixError(rc, lib().mi355_last_error().decode())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def input_kind(t):
+    return {torch.float32: INPUT_F32, torch.float16: INPUT_F16, torch.bfloat16: INPUT_BF16}[t.dtype]
+
+
+def row_bytes(qtype, elements):
+    return elements // 32 * Q8_0_BLOCK if qtype == TYPE_Q8_0 else elements // 256 * Q4_K_BLOCK
+
+
+# ---------------------------------------------------------------------------------------------- thin wrappers
+def dequantize_rows(qtype, packed, elements):
+    packed = packed.contiguous().view(torch.uint8).reshape(-1, row_bytes(qtype, elements))
+    out = torch.empty((packed.shape[0], elements), dtype=torch.float32, device=packed.device)
+    check(lib().mi355_dequantize_rows(qtype, _p(packed), C.c_uint64(packed.shape[1]), packed.shape[0], elements, _p(out),
+                                      C.c_uint64(elements), _stream()))
+    return out
+
+
+def quantize_weight_rows(qtype, x):
+    x = x.contiguous()
+    rows = x.numel() // x.shape[-1]
+    out = torch.empty(x.shape[:-1] + (row_bytes(qtype, x.shape[-1]),), dtype=torch.uint8, device=x.device)
+    check(lib().mi355_quantize_weight_rows(qtype, _p(x), rows, x.shape[-1], _p(out), _stream()))
+    return out
+
+
+def quantize_a8(x, want_sums=True):
+    assert x.dim() == 2 and x.stride(1) == 1
+    rows, width = x.shape
+    codes = torch.empty((rows, width), dtype=torch.int8, device=x.device)
+    deltas = torch.empty((rows, width // 32), dtype=torch.float32, device=x.device)
+    sums = torch.empty((rows, width // 32), dtype=torch.int32, device=x.device) if want_sums else None
+    status = torch.zeros(rows, dtype=torch.int32, device=x.device)
+    check(lib().mi355_quantize_a8(_p(x), input_kind(x), rows, width, C.c_uint64(x.stride(0) * x.element_size()), _p(codes),
+                                  _p(deltas), _p(sums), _p(status), _stream()))
+    return codes, deltas, sums, status
+
+
+def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False, row_bytes_=None, out_stride=None):
+    rows = codes.shape[0]
+    if out is None:
+        out = torch.zeros((rows, count), dtype=torch.float32, device=codes.device)
+    v = Q8a8View(weight.data_ptr(), codes.data_ptr(), deltas.data_ptr(), out.data_ptr(),
+                 row_bytes_ or n_in // 32 * Q8_0_BLOCK, n_in, count, rows, codes.shape[1], out_stride or out.shape[1], int(accumulate))
+    check(lib().mi355_gemv_q8_0_a8(C.byref(v), _stream()))
+    return out
+
+
+def route(x, router_weight, top_k, bias=None, logits_order=LOGITS_FMA, renorm_eps=0.0, scale=1.0, renormalize=True):
+    rows, hidden = x.shape
+    experts = router_weight.shape[0]
+    p = RoutePolicy(experts, top_k, logits_order, renorm_eps, scale, int(renormalize))
+    ids = torch.empty((rows, top_k), dtype=torch.int32, device=x.device)
+    weights = torch.empty((rows, top_k), dtype=torch.float32, device=x.device)
+    scores = torch.empty((rows, experts), dtype=torch.float32, device=x.device)
+    check(lib().mi355_moe_route(C.byref(p), _p(x), input_kind(x), rows, hidden, C.c_uint64(x.stride(0) * x.element_size()),
+                                _p(router_weight), _p(bias), _p(ids), _p(weights), _p(scores), _stream()))
+    return ids, weights, scores
+
+
+def swiglu_quantize(gate, up, exp_kind=EXP_GFX1151):
+    rows, ffn = gate.shape
+    codes = torch.zeros((rows, ffn), dtype=torch.int8, device=gate.device)
+    deltas = torch.zeros((rows, ffn // 32), dtype=torch.float32, device=gate.device)
+    sums = torch.zeros((rows, ffn // 32), dtype=torch.int32, device=gate.device)
+    h = torch.zeros((rows, ffn), dtype=torch.float32, device=gate.device)
+    status = torch.zeros(rows, dtype=torch.int32, device=gate.device)
+    check(lib().mi355_swiglu_quantize(_p(gate), _p(up), rows, ffn, exp_kind, _p(codes), _p(deltas), _p(sums), _p(h), _p(status), _stream()))
+    return codes, deltas, sums, h, status
+
+
+class MoeLayer:
+    """One MoE layer's expert tensors plus caller-owned work buffers for up to max_rows rows (the reference's
+    Rows / Weights bundle, include/strix/cuda/qwen_moe.hpp:55-93)."""
+
+    def __init__(self, hidden, ffn, experts, top_k, gate, up, down, max_rows, exp_kind=EXP_GFX1151, intermediates=False,
+                 gate_expert_stride=0, gate_row_stride=0, down_expert_stride=0, down_row_stride=0):
+        dev = gate.device
+        self.hidden, self.ffn, self.experts, self.top_k, self.max_rows = hidden, ffn, experts, top_k, max_rows
+        self.gate, self.up, self.down = gate, up, down
+        self.w = MoeWeights(hidden, ffn, experts, top_k, TYPE_Q4_K, TYPE_Q4_K, gate.data_ptr(), up.data_ptr(), down.data_ptr(),
+                            gate_expert_stride, gate_row_stride, down_expert_stride, down_row_stride, exp_kind)
+        n = max_rows * top_k
+        z = lambda shape, dt: torch.zeros(shape, dtype=dt, device=dev)
+        self.codes, self.deltas, self.sums = z((max_rows, hidden), torch.int8), z((max_rows, hidden // 32), torch.float32), z((max_rows, hidden // 32), torch.int32)
+        self.status, self.job_status = z(max_rows, torch.int32), z(4, torch.int32)
+        self.down_codes, self.down_deltas, self.down_sums = z((n, ffn), torch.int8), z((n, ffn // 32), torch.float32), z((n, ffn // 32), torch.int32)
+        self.rawdots = z((max_rows, top_k, hidden), torch.float32)
+        self.output = z((max_rows, hidden), torch.float32)
+        self.gate_out = z((n, ffn), torch.float32) if intermediates else None
+        self.up_out = z((n, ffn), torch.float32) if intermediates else None
+        self.h_out = z((n, ffn), torch.float32) if intermediates else None
+        self.plan = z(int(lib().mi355_moe_plan_words(experts, max_rows, top_k)), torch.int32)
+
+    def rows_view(self, x, ids, weights, base=None):
+        rows = x.shape[0]
+        assert rows <= self.max_rows and x.stride(1) == 1
+        self._keep = (x, ids, weights, base)
+        return rows, MoeRows(x.data_ptr(), input_kind(x), x.stride(0) * x.element_size(), ids.data_ptr(), weights.data_ptr(),
+                             self.codes.data_ptr(), self.deltas.data_ptr(), self.sums.data_ptr(), self.status.data_ptr(),
+                             _p(self.gate_out).value or 0, _p(self.up_out).value or 0, _p(self.h_out).value or 0,
+                             self.down_codes.data_ptr(), self.down_deltas.data_ptr(), self.down_sums.data_ptr(),
+                             self.rawdots.data_ptr(), 0 if base is None else base.data_ptr(), self.output.data_ptr(), self.hidden,
+                             self.plan.data_ptr(), self.job_status.data_ptr())
+
+    def run(self, x, ids, weights, base=None, combine=COMBINE_FMA_SLOT):
+        rows, rv = self.rows_view(x, ids, weights, base)
+        check(lib().mi355_moe_enqueue(C.byref(self.w), C.byref(rv), rows, combine, _stream()))
+        return self.output[:rows]
+
+    def stage(self, name, x, ids, weights, base=None, combine=COMBINE_FMA_SLOT):
+        rows, rv = self.rows_view(x, ids, weights, base)
+        fn = getattr(lib(), "mi355_moe_enqueue_" + name)
+        if name == "merge":
+            check(fn(C.byref(self.w), C.byref(rv), rows, combine, _stream()))
+        else:
+            check(fn(C.byref(self.w), C.byref(rv), rows, _stream()))

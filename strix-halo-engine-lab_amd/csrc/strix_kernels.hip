@@ -1,0 +1,812 @@
+// MI355X (gfx950, wave64) kernels and C ABI of the quantized weight-product path. See include/mi355_strix.h for the
+// contract of every entry point; reference file:line citations are relative to the reference tree.
+#include "mi355_strix.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "device_math.hpp"
+
+namespace strix950 {
+
+// ======================================================================================================== host side
+thread_local std::string g_error;
+
+int32_t fail(int32_t code, const char* what) {
+    g_error = what;
+    return code;
+}
+int32_t hip_fail(hipError_t e, const char* what) {
+    g_error = std::string(what) + ": " + hipGetErrorString(e);
+    return MI355_E_HIP;
+}
+#define STRIX_REQUIRE(cond, what) do { if (!(cond)) return fail(MI355_E_INVALID_ARGUMENT, what); } while (0)
+#define STRIX_LAUNCHED(what) do { const hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return hip_fail(e_, what); } while (0)
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+inline hipStream_t hs(mi355_stream s) { return static_cast<hipStream_t>(s); }
+
+constexpr uint32_t kQ4kBlock = 144, kQ80Block = 34;
+
+// ======================================================================================================== block decode
+// One thread per output element. Q4_K: y = (d * sc) * q - (dmin * m), two products and one subtraction
+// (src/ggml_dequant.cpp:119-130); Q8_0: y = int8 * d (src/ggml_dequant.cpp:84-87).
+__device__ __forceinline__ void q4k_scale_min(const uint8_t* q, uint32_t j, uint32_t& sc, uint32_t& m) {
+    if (j < 4) { sc = q[j] & 63U; m = q[j + 4] & 63U; }
+    else { sc = (q[j + 4] & 0xFU) | ((q[j - 4] >> 6) << 4); m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4); }
+}
+
+__global__ __launch_bounds__(256) void dequantize_rows_kernel(uint32_t type, const uint8_t* rows, uint64_t row_stride,
+                                                              uint32_t elements, float* out, uint64_t out_stride) {
+    const uint32_t r = blockIdx.y;
+    const uint8_t* row = rows + r * row_stride;
+    for (uint32_t i = blockIdx.x * 256U + threadIdx.x; i < elements; i += gridDim.x * 256U) {
+        float y;
+        if (type == MI355_TYPE_Q8_0) {
+            const uint8_t* b = row + (i / 32U) * kQ80Block;
+            const float d = half_bits_to_float(b[0] | (static_cast<uint32_t>(b[1]) << 8));
+            y = static_cast<float>(static_cast<int8_t>(b[2 + (i % 32U)])) * d;
+        } else {
+            const uint8_t* b = row + (i / 256U) * kQ4kBlock;
+            const uint32_t k = i % 256U, j = k / 32U, l = k % 32U;
+            uint32_t sc, m;
+            q4k_scale_min(b + 4, j, sc, m);
+            const float d = half_bits_to_float(b[0] | (static_cast<uint32_t>(b[1]) << 8));
+            const float mn = half_bits_to_float(b[2] | (static_cast<uint32_t>(b[3]) << 8));
+            const float d1 = d * static_cast<float>(sc), m1 = mn * static_cast<float>(m);
+            const uint32_t byte = b[16 + 32 * (j / 2) + l];
+            const float q = static_cast<float>((j & 1U) ? (byte >> 4) : (byte & 15U));
+            y = d1 * q - m1;
+        }
+        out[r * out_stride + i] = y;
+    }
+}
+
+// ======================================================================================================== weight writers
+// Q8_0: include/strix/q8_0_rule.hpp:25-33 (d = amax / 127, id = 1 / d, q = roundf(v * id), d stored as fp16).
+__global__ __launch_bounds__(256) void quantize_q8_0_rows_kernel(const float* x, uint64_t blocks, uint8_t* out) {
+    for (uint64_t b = blockIdx.x * 256ULL + threadIdx.x; b < blocks; b += 256ULL * gridDim.x) {
+        const float* v = x + b * 32;
+        float amax = 0.0F;
+        for (int j = 0; j < 32; ++j) amax = __builtin_fmaxf(amax, __builtin_fabsf(v[j]));
+        const float d = amax / 127.0F;
+        const float id = d != 0.0F ? 1.0F / d : 0.0F;
+        uint8_t* o = out + b * kQ80Block;
+        const uint32_t h = float_to_half_bits(d);
+        o[0] = static_cast<uint8_t>(h); o[1] = static_cast<uint8_t>(h >> 8);
+        for (int j = 0; j < 32; ++j) o[2 + j] = static_cast<uint8_t>(static_cast<int8_t>(static_cast<int>(__builtin_roundf(v[j] * id))));
+    }
+}
+
+// Q4_K min/max writer (no reference counterpart): the steps of oracle/strix_oracle.c orc_quantize_q4_k_row.
+__global__ __launch_bounds__(64) void quantize_q4_k_rows_kernel(const float* x, uint64_t blocks, uint8_t* out) {
+    for (uint64_t b = blockIdx.x * 64ULL + threadIdx.x; b < blocks; b += 64ULL * gridDim.x) {
+        const float* v = x + b * 256;
+        uint8_t* o = out + b * kQ4kBlock;
+        float scale[8], offset[8], smax = 0.0F, omax = 0.0F;
+        for (int j = 0; j < 8; ++j) {
+            float lo = 0.0F, hi = v[32 * j];
+            for (int l = 0; l < 32; ++l) { lo = __builtin_fminf(lo, v[32 * j + l]); hi = __builtin_fmaxf(hi, v[32 * j + l]); }
+            hi = __builtin_fmaxf(hi, lo);
+            scale[j] = (hi - lo) / 15.0F; offset[j] = -lo;
+            smax = __builtin_fmaxf(smax, scale[j]); omax = __builtin_fmaxf(omax, offset[j]);
+        }
+        const uint32_t dh = float_to_half_bits(smax / 63.0F), mh = float_to_half_bits(omax / 63.0F);
+        const float d = half_bits_to_float(dh), dm = half_bits_to_float(mh);
+        uint32_t sc[8], mn[8];
+        for (int j = 0; j < 8; ++j) {
+            sc[j] = d > 0.0F ? static_cast<uint32_t>(__builtin_fminf(63.0F, __builtin_rintf(scale[j] / d))) : 0U;
+            mn[j] = dm > 0.0F ? static_cast<uint32_t>(__builtin_fminf(63.0F, __builtin_rintf(offset[j] / dm))) : 0U;
+        }
+        o[0] = static_cast<uint8_t>(dh); o[1] = static_cast<uint8_t>(dh >> 8);
+        o[2] = static_cast<uint8_t>(mh); o[3] = static_cast<uint8_t>(mh >> 8);
+        for (int j = 0; j < 4; ++j) {
+            o[4 + j] = static_cast<uint8_t>((sc[j] & 63U) | ((sc[j + 4] >> 4) << 6));
+            o[8 + j] = static_cast<uint8_t>((mn[j] & 63U) | ((mn[j + 4] >> 4) << 6));
+            o[12 + j] = static_cast<uint8_t>((sc[j + 4] & 15U) | ((mn[j + 4] & 15U) << 4));
+        }
+        for (int p = 0; p < 4; ++p) {
+            const float ed0 = d * static_cast<float>(sc[2 * p]), em0 = dm * static_cast<float>(mn[2 * p]);
+            const float ed1 = d * static_cast<float>(sc[2 * p + 1]), em1 = dm * static_cast<float>(mn[2 * p + 1]);
+            for (int l = 0; l < 32; ++l) {
+                float r0 = 0.0F, r1 = 0.0F;
+                if (ed0 > 0.0F) r0 = __builtin_fminf(15.0F, __builtin_fmaxf(0.0F, __builtin_rintf((v[64 * p + l] + em0) / ed0)));
+                if (ed1 > 0.0F) r1 = __builtin_fminf(15.0F, __builtin_fmaxf(0.0F, __builtin_rintf((v[64 * p + 32 + l] + em1) / ed1)));
+                o[16 + 32 * p + l] = static_cast<uint8_t>(static_cast<uint32_t>(r0) | (static_cast<uint32_t>(r1) << 4));
+            }
+        }
+    }
+}
+
+// ======================================================================================================== A8 quantiser
+// One aligned group of 32 lanes per 32-value group; 8 groups per 256-thread block.
+// Reference: src/cpu/core/reference.cpp:35-55.
+template <int KIND>
+__global__ __launch_bounds__(256) void quantize_a8_kernel(const uint8_t* x, uint64_t x_stride, uint32_t width, int8_t* codes,
+                                                          float* deltas, int32_t* sums, uint32_t* status) {
+    const uint32_t r = blockIdx.y, groups = width / 32U;
+    const uint32_t g = blockIdx.x * 8U + (threadIdx.x >> 5), j = threadIdx.x & 31U;
+    if (g >= groups) return;
+    const float v = load_activation<KIND>(x + r * x_stride, g * 32U + j);
+    const float amax = max32(__builtin_fabsf(v));
+    const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+    const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+    const int code = a8_code(v, delta, tiny);
+    const int sum = sum32_i(code);
+    const int bad = or32_i(finite_f(v) ? 0 : 1);
+    codes[static_cast<size_t>(r) * width + g * 32U + j] = static_cast<int8_t>(code);
+    if (j == 0) {
+        deltas[static_cast<size_t>(r) * groups + g] = delta;
+        if (sums) sums[static_cast<size_t>(r) * groups + g] = sum;
+        if (bad && status) atomicOr(&status[r], static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
+    }
+}
+
+// ======================================================================================================== Q8_0 x A8 GEMV
+// One aligned group of 32 lanes per output row: lane l owns the reference's accumulator lane l (groups g = l, l + 32,
+// ... ascending), then the tree32 butterfly. Up to RB activation rows share one sweep of the weight row.
+// Reference: src/cpu/core/reference.cpp:57-84, src/core/integer_math.hpp:11-13,43-47.
+template <int RB>
+__global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v, uint32_t row0) {
+    const uint32_t o = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U;
+    if (o >= v.count) return;
+    const uint32_t groups = v.in / 32U;
+    const uint32_t nr = v.rows - row0 < static_cast<uint32_t>(RB) ? v.rows - row0 : static_cast<uint32_t>(RB);
+    const uint8_t* wrow = v.weight + static_cast<size_t>(o) * v.row_bytes;
+    float lane[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) lane[r] = 0.0F;
+    for (uint32_t g = l; g < groups; g += 32U) {
+        const unsigned short* b = reinterpret_cast<const unsigned short*>(wrow + static_cast<size_t>(g) * kQ80Block);
+        const float scale = half_bits_to_float(b[0]);
+        int w[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w[i] = static_cast<int>(static_cast<uint32_t>(b[1 + 2 * i]) | (static_cast<uint32_t>(b[2 + 2 * i]) << 16));
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            if (static_cast<uint32_t>(r) < nr) {
+                const int4* xc = reinterpret_cast<const int4*>(v.codes + static_cast<size_t>(row0 + r) * v.x_stride + g * 32U);
+                const int4 a = xc[0], c = xc[1];
+                int dot = 0;
+                dot = __builtin_amdgcn_sdot4(w[0], a.x, dot, false); dot = __builtin_amdgcn_sdot4(w[1], a.y, dot, false);
+                dot = __builtin_amdgcn_sdot4(w[2], a.z, dot, false); dot = __builtin_amdgcn_sdot4(w[3], a.w, dot, false);
+                dot = __builtin_amdgcn_sdot4(w[4], c.x, dot, false); dot = __builtin_amdgcn_sdot4(w[5], c.y, dot, false);
+                dot = __builtin_amdgcn_sdot4(w[6], c.z, dot, false); dot = __builtin_amdgcn_sdot4(w[7], c.w, dot, false);
+                const float xd = v.deltas[static_cast<size_t>(row0 + r) * (v.x_stride / 32U) + g];
+                lane[r] = lane[r] + static_cast<float>(dot) * (scale * xd);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+        float p = lane[r];
+        p = p + xor16_f(p); p = p + xor8_f(p); p = p + xor4_f(p); p = p + xor2_f(p); p = p + xor1_f(p);
+        if (l == 0 && static_cast<uint32_t>(r) < nr) {
+            float* y = &v.out[static_cast<size_t>(row0 + r) * v.out_stride + o];
+            *y = v.accumulate ? *y + p : p;
+        }
+    }
+}
+
+// ======================================================================================================== router
+// One block per row. Logits: thread e runs expert e's chain over the row staged in LDS.
+// Reference: tests/hip_moe_route_launcher_tests.hip:281-330 (chain), include/strix/moe/route_policy.hpp:99-156.
+constexpr uint32_t kRouteMaxHidden = 8192, kRouteMaxExperts = 1024, kRouteMaxTopK = 16;
+
+__global__ __launch_bounds__(256) void route_kernel(mi355_route_policy p, const uint8_t* x, uint32_t kind, uint32_t hidden,
+                                                    uint64_t x_stride, const float* wr, const float* bias, uint32_t* ids,
+                                                    float* weights, float* scores) {
+    __shared__ float xs[kRouteMaxHidden];
+    __shared__ float sc[kRouteMaxExperts];
+    __shared__ float red_v[4];
+    __shared__ uint32_t red_i[4];
+    __shared__ float total;
+    __shared__ uint32_t picked[kRouteMaxTopK];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    for (uint32_t i = tid; i < hidden; i += 256U) xs[i] = load_activation_kind(x + row * x_stride, i, kind);
+    __syncthreads();
+    for (uint32_t e = tid; e < p.experts; e += 256U) {
+        const float* we = wr + static_cast<size_t>(e) * hidden;
+        float acc;
+        if (p.logits_order == MI355_LOGITS_LANE32_BUTTERFLY) {
+            float lanes[32];
+#pragma unroll
+            for (int l = 0; l < 32; ++l) lanes[l] = 0.0F;
+            for (uint32_t i = 0; i < hidden; i += 32U) {
+#pragma unroll
+                for (int l = 0; l < 32; ++l)
+                    if (i + l < hidden) lanes[l] = lanes[l] + we[i + l] * xs[i + l];
+            }
+#pragma unroll
+            for (int s = 16; s; s /= 2)
+#pragma unroll
+                for (int i = 0; i < s; ++i) lanes[i] = lanes[i] + lanes[i + s];
+            acc = lanes[0];
+        } else {
+            acc = 0.0F;
+            uint32_t i = 0;
+            for (; i + 4 <= hidden; i += 4) {
+                const float4 w4 = *reinterpret_cast<const float4*>(we + i);
+                acc = __builtin_fmaf(xs[i], w4.x, acc); acc = __builtin_fmaf(xs[i + 1], w4.y, acc);
+                acc = __builtin_fmaf(xs[i + 2], w4.z, acc); acc = __builtin_fmaf(xs[i + 3], w4.w, acc);
+            }
+            for (; i < hidden; ++i) acc = __builtin_fmaf(xs[i], we[i], acc);
+        }
+        sc[e] = bias ? acc + bias[e] : acc;
+    }
+    __syncthreads();
+    // softmax: m = max, p = exp(z - m), sum ascending from 0, s = p / sum
+    float m = -INFINITY;
+    for (uint32_t e = tid; e < p.experts; e += 256U) m = sc[e] > m ? sc[e] : m;
+    for (int d = 32; d; d >>= 1) { const float o = __shfl_xor(m, d); m = o > m ? o : m; }
+    if ((tid & 63U) == 0) red_v[tid >> 6] = m;
+    __syncthreads();
+    m = red_v[0];
+    for (int w = 1; w < 4; ++w) m = red_v[w] > m ? red_v[w] : m;
+    __syncthreads();
+    for (uint32_t e = tid; e < p.experts; e += 256U) sc[e] = declared_exp(sc[e] - m);
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.0F;
+        for (uint32_t e = 0; e < p.experts; ++e) sum = sum + sc[e];
+        total = sum;
+    }
+    __syncthreads();
+    const float sum = total;
+    for (uint32_t e = tid; e < p.experts; e += 256U) {
+        const float s = sc[e] / sum;
+        sc[e] = s;
+        scores[static_cast<size_t>(row) * p.experts + e] = s;
+    }
+    __syncthreads();
+    // k passes; a pass takes the greatest remaining score, the lower id on ties (ascending serial scan semantics)
+    for (uint32_t k = 0; k < p.top_k; ++k) {
+        float bv = -1.0F;
+        uint32_t bi = 0xffffffffU;
+        for (uint32_t e = tid; e < p.experts; e += 256U) {
+            bool taken = false;
+            for (uint32_t q = 0; q < k; ++q) taken |= picked[q] == e;
+            if (taken) continue;
+            const float c = sc[e];
+            if (bi == 0xffffffffU || c > bv) { bv = c; bi = e; }
+        }
+        for (int d = 32; d; d >>= 1) {
+            const float ov = __shfl_xor(bv, d);
+            const uint32_t oi = __shfl_xor(bi, d);
+            if (oi != 0xffffffffU && (bi == 0xffffffffU || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+        }
+        if ((tid & 63U) == 0) { red_v[tid >> 6] = bv; red_i[tid >> 6] = bi; }
+        __syncthreads();
+        if (tid == 0) {
+            float v = red_v[0];
+            uint32_t i = red_i[0];
+            for (int w = 1; w < 4; ++w)
+                if (red_i[w] != 0xffffffffU && (i == 0xffffffffU || red_v[w] > v || (red_v[w] == v && red_i[w] < i))) { v = red_v[w]; i = red_i[w]; }
+            picked[k] = i;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        float s = 0.0F;
+        for (uint32_t k = 0; k < p.top_k; ++k) s = s + sc[picked[k]];
+        const float den = s + p.renorm_eps;
+        for (uint32_t k = 0; k < p.top_k; ++k) {
+            const float v = sc[picked[k]];
+            ids[static_cast<size_t>(row) * p.top_k + k] = picked[k];
+            weights[static_cast<size_t>(row) * p.top_k + k] = (p.renormalize ? v / den : v) * p.scale;
+        }
+    }
+}
+
+// ======================================================================================================== expert plan
+// Plan words: [0] assignments A = rows * top_k, [1] touched experts, [2] largest group, [16 ..] offsets[experts + 1],
+// then order[A]: assignment indices (row * top_k + slot) grouped by expert, ascending row then slot inside an expert.
+// Reference: src/hip_moe_q4k_a8_probe.hip:91-147 (stable CSR of (row, slot) by expert).
+__host__ __device__ inline uint32_t plan_order_at(uint32_t experts) { return 16U + ((experts + 1U + 3U) & ~3U); }
+
+__global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
+    __shared__ uint32_t count[kRouteMaxExperts + 1];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t e = tid; e <= experts; e += 1024U) count[e] = 0;
+    __syncthreads();
+    for (uint32_t a = tid; a < assignments; a += 1024U) {
+        const uint32_t e = routes[a];
+        if (e < experts) atomicAdd(&count[e], 1U);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t run = 0, touched = 0, largest = 0;
+        for (uint32_t e = 0; e < experts; ++e) {
+            const uint32_t c = count[e];
+            count[e] = run;
+            run += c;
+            touched += c != 0;
+            largest = c > largest ? c : largest;
+        }
+        count[experts] = run;
+        plan[0] = assignments; plan[1] = touched; plan[2] = largest;
+    }
+    __syncthreads();
+    uint32_t* offsets = plan + 16;
+    uint32_t* order = plan + plan_order_at(experts);
+    for (uint32_t e = tid; e <= experts; e += 1024U) offsets[e] = count[e];
+    for (uint32_t e = tid; e < experts; e += 1024U) {
+        const uint32_t end = e + 1 <= experts ? count[e + 1] : 0;
+        uint32_t at = count[e];
+        if (at == end) continue;
+        for (uint32_t a = 0; a < assignments && at < end; ++a)
+            if (routes[a] == e) order[at++] = a;
+    }
+}
+
+__global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* routes, const float* route_weights, uint32_t experts,
+                                                            uint32_t top_k, uint32_t* status, uint32_t* job_status) {
+    const uint32_t row = blockIdx.x;
+    uint32_t bad = 0;
+    for (uint32_t k = threadIdx.x; k < top_k; k += 64U) {
+        if (routes[row * top_k + k] >= experts) bad = MI355_STATUS_INVALID_ROUTE;
+        if (route_weights && !finite_f(route_weights[row * top_k + k])) bad = MI355_STATUS_INVALID_ROUTE;
+    }
+    for (int d = 32; d; d >>= 1) bad |= __shfl_xor(bad, d);
+    if (threadIdx.x == 0) {
+        status[row] = bad;
+        if (row == 0) *job_status = 0;
+    }
+}
+
+// ======================================================================================================== Q4_K x A8 rows
+// 32 weight rows per 256-thread block, 8 lanes per row: lane s of a row owns 16-byte quant chunk s of every 144-byte
+// super-block (pair p = s / 2, half h = s & 1) and evaluates the group term of sub-block j = s:
+//   x_j = E_g * ((D_j * float(dot_j)) - (DM_j * float(S_g))),  D_j = d * sc_j, DM_j = dmin * m_j, g = 8 b + j
+//   acc_p += (x_2p + x_2p+1) over super-blocks b ascending;  value = (acc0 + acc1) + (acc2 + acc3)
+// dot_j is exact: each lane's two 16-element int8 dot products (v_dot4_i32_i8) are exchanged with lane ^ 1 by DPP.
+// Up to NB activation rows (assignments) share one sweep of the weights; their A8 images are staged in LDS.
+// Reference: src/cpu/core/routed_expert.cpp:73-108, src/moe_q4k_a8_contract.cpp:126-140, lane roles of
+// src/hip_moe_q4k_a8_probe.hip:202-249.
+constexpr int kNB = 8;              // assignments per sweep
+constexpr uint32_t kChunk = 2048;   // activation elements staged per LDS pass
+
+struct ActImage {                   // A8 image of assignment a: codes [K], deltas [K/32], sums [K/32]
+    const int8_t* codes;
+    const float* deltas;
+    const int32_t* sums;
+    uint32_t width;                 // K
+};
+
+struct RowsLds {
+    int8_t codes[kNB][kChunk];
+    float delta[kNB][kChunk / 32];
+    float sumf[kNB][kChunk / 32];
+};
+
+// src_index(a) gives the row of the A8 image read by assignment a of this sweep.
+template <class Index>
+__device__ __forceinline__ void stage_chunk(RowsLds& lds, const ActImage& img, Index src_index, uint32_t na, uint32_t k0, uint32_t kc) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t vec = kc / 16U;
+    for (uint32_t i = tid; i < na * vec; i += 256U) {
+        const uint32_t a = i / vec, c = i % vec;
+        const int4 v = *reinterpret_cast<const int4*>(img.codes + static_cast<size_t>(src_index(a)) * img.width + k0 + c * 16U);
+        *reinterpret_cast<int4*>(&lds.codes[a][c * 16U]) = v;
+    }
+    const uint32_t gc = kc / 32U, groups = img.width / 32U;
+    for (uint32_t i = tid; i < na * gc; i += 256U) {
+        const uint32_t a = i / gc, g = i % gc;
+        const size_t at = static_cast<size_t>(src_index(a)) * groups + k0 / 32U + g;
+        lds.delta[a][g] = img.deltas[at];
+        lds.sumf[a][g] = static_cast<float>(img.sums[at]);
+    }
+}
+
+// Sweeps `blocks` super-blocks of one weight row share (this lane: row of the block, chunk s) against na staged rows.
+// acc[a] accumulates pair p = s / 2 of assignment a.
+template <class Index>
+__device__ __forceinline__ void q4k_rows_sweep(RowsLds& lds, const uint8_t* wrow, uint32_t blocks, const ActImage& img,
+                                               Index src_index, uint32_t na, float (&acc)[kNB]) {
+    const uint32_t s = threadIdx.x & 7U, h = s & 1U, p = s >> 1;
+#pragma unroll
+    for (int a = 0; a < kNB; ++a) acc[a] = 0.0F;
+    for (uint32_t k0 = 0; k0 < blocks * 256U; k0 += kChunk) {
+        const uint32_t kc = blocks * 256U - k0 < kChunk ? blocks * 256U - k0 : kChunk;
+        __syncthreads();
+        stage_chunk(lds, img, src_index, na, k0, kc);
+        __syncthreads();
+        for (uint32_t b = 0; b < kc / 256U; ++b) {
+            const uint8_t* blk = wrow + static_cast<size_t>(k0 / 256U + b) * kQ4kBlock;
+            const uint4 hd = *reinterpret_cast<const uint4*>(blk);
+            const uint4 q = *reinterpret_cast<const uint4*>(blk + 16U + 16U * s);
+            // 6-bit factors of sub-block j = s from the three scale words (src/cpu/core/routed_expert.cpp:65-71)
+            const uint32_t shift = 8U * (s & 3U);
+            const uint32_t fa = (hd.y >> shift) & 255U, fb = (hd.z >> shift) & 255U, fc = (hd.w >> shift) & 255U;
+            const uint32_t scj = s < 4U ? (fa & 63U) : ((fc & 15U) | ((fa >> 6) << 4));
+            const uint32_t mnj = s < 4U ? (fb & 63U) : ((fc >> 4) | ((fb >> 6) << 4));
+            const float d = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
+            const float D = d * static_cast<float>(scj), DM = dm * static_cast<float>(mnj);
+            const int lo0 = static_cast<int>(q.x & 0x0f0f0f0fU), lo1 = static_cast<int>(q.y & 0x0f0f0f0fU);
+            const int lo2 = static_cast<int>(q.z & 0x0f0f0f0fU), lo3 = static_cast<int>(q.w & 0x0f0f0f0fU);
+            const int hi0 = static_cast<int>((q.x >> 4) & 0x0f0f0f0fU), hi1 = static_cast<int>((q.y >> 4) & 0x0f0f0f0fU);
+            const int hi2 = static_cast<int>((q.z >> 4) & 0x0f0f0f0fU), hi3 = static_cast<int>((q.w >> 4) & 0x0f0f0f0fU);
+            const uint32_t at = b * 256U + p * 64U + h * 16U;   // elements of sub-block 2p held by this lane; 2p+1 is +32
+            const uint32_t g = b * 8U + s;
+#pragma unroll
+            for (int a = 0; a < kNB; ++a) {
+                if (static_cast<uint32_t>(a) < na) {
+                    const int4 cl = *reinterpret_cast<const int4*>(&lds.codes[a][at]);
+                    const int4 ch = *reinterpret_cast<const int4*>(&lds.codes[a][at + 32U]);
+                    int dl = 0, dh = 0;
+                    dl = __builtin_amdgcn_sdot4(lo0, cl.x, dl, false); dl = __builtin_amdgcn_sdot4(lo1, cl.y, dl, false);
+                    dl = __builtin_amdgcn_sdot4(lo2, cl.z, dl, false); dl = __builtin_amdgcn_sdot4(lo3, cl.w, dl, false);
+                    dh = __builtin_amdgcn_sdot4(hi0, ch.x, dh, false); dh = __builtin_amdgcn_sdot4(hi1, ch.y, dh, false);
+                    dh = __builtin_amdgcn_sdot4(hi2, ch.z, dh, false); dh = __builtin_amdgcn_sdot4(hi3, ch.w, dh, false);
+                    const int recv = xor1_i(h ? dl : dh);
+                    const int dot = (h ? dh : dl) + recv;
+                    const float u = D * static_cast<float>(dot);
+                    const float v = DM * lds.sumf[a][g];
+                    const float t = u - v;
+                    const float x = lds.delta[a][g] * t;
+                    const float pair = x + xor1_f(x);
+                    acc[a] = acc[a] + pair;
+                }
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ float q4k_row_tree(float v) {   // (acc0 + acc1) + (acc2 + acc3) over the row's 8 lanes
+    v = v + xor2_f(v);
+    v = v + xor4_f(v);
+    return v;
+}
+
+// gate + up + SwiGLU + A8 re-quantisation of one (expert, 32-output group).
+// Reference: src/cpu/core/routed_expert.cpp:403-427 (gate item), :147-170 (swiglu_quantize).
+__global__ __launch_bounds__(256) void project_kernel(mi355_moe_weights w, mi355_moe_rows r) {
+    __shared__ RowsLds lds;
+    __shared__ float val[2][kNB][32];
+    const uint32_t grp = blockIdx.x, e = blockIdx.y, tid = threadIdx.x;
+    const uint32_t* offsets = r.plan + 16;
+    const uint32_t* order = r.plan + plan_order_at(w.experts);
+    const uint32_t begin = offsets[e], end = offsets[e + 1];
+    if (begin == end) return;
+    const uint32_t rrow = tid >> 3, blocks = w.hidden / 256U, groups = w.ffn / 32U;
+    const ActImage img{r.codes, r.deltas, r.sums, w.hidden};
+    const size_t row_off = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U + rrow) * w.gate_row_stride;
+    for (uint32_t c0 = begin; c0 < end; c0 += kNB) {
+        const uint32_t na = end - c0 < static_cast<uint32_t>(kNB) ? end - c0 : static_cast<uint32_t>(kNB);
+        const auto src = [&](uint32_t a) { return order[c0 + a] / w.top_k; };   // input row of the assignment
+        for (int which = 0; which < 2; ++which) {
+            float acc[kNB];
+            q4k_rows_sweep(lds, (which ? w.up : w.gate) + row_off, blocks, img, src, na, acc);
+#pragma unroll
+            for (int a = 0; a < kNB; ++a) {
+                const float v = q4k_row_tree(acc[a]);
+                if ((tid & 7U) == 0 && static_cast<uint32_t>(a) < na) val[which][a][rrow] = v;
+            }
+        }
+        __syncthreads();
+        const uint32_t a = tid >> 5, l = tid & 31U;
+        if (a < na) {
+            const uint32_t sidx = order[c0 + a];
+            const float g = val[0][a][l], u = val[1][a][l];
+            const float ex = exp_of(w.exp_kind, -g);
+            const float hv = (g / (1.0F + ex)) * u;
+            const size_t at = static_cast<size_t>(sidx) * w.ffn + grp * 32U + l;
+            if (r.gate_out) r.gate_out[at] = g;
+            if (r.up_out) r.up_out[at] = u;
+            if (r.h_out) r.h_out[at] = hv;
+            const int bad = or32_i((finite_f(g) && finite_f(u) && finite_f(hv)) ? 0 : 1);
+            if (bad) {
+                if (l == 0) {
+                    atomicOr(&r.status[sidx / w.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                    atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                }
+            } else {
+                const float amax = max32(__builtin_fabsf(hv));
+                const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+                const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+                const int code = a8_code(hv, dl, tiny);
+                const int sum = sum32_i(code);
+                r.down_codes[at] = static_cast<int8_t>(code);
+                if (l == 0) {
+                    r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
+                    r.down_sums[static_cast<size_t>(sidx) * groups + grp] = sum;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// down rows of one (expert, 32 hidden outputs): rawdots[assignment][o].
+// Reference: src/cpu/core/routed_expert.cpp:429-447 (down item), src/moe_a8_down_contract.cpp:146 (Q4_K down row).
+__global__ __launch_bounds__(256) void down_kernel(mi355_moe_weights w, mi355_moe_rows r) {
+    __shared__ RowsLds lds;
+    const uint32_t og = blockIdx.x, e = blockIdx.y, tid = threadIdx.x;
+    if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
+    const uint32_t* offsets = r.plan + 16;
+    const uint32_t* order = r.plan + plan_order_at(w.experts);
+    const uint32_t begin = offsets[e], end = offsets[e + 1];
+    if (begin == end) return;
+    const uint32_t rrow = tid >> 3, o = og * 32U + rrow;
+    const ActImage img{r.down_codes, r.down_deltas, r.down_sums, w.ffn};
+    const uint8_t* wrow = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o) * w.down_row_stride;
+    for (uint32_t c0 = begin; c0 < end; c0 += kNB) {
+        const uint32_t na = end - c0 < static_cast<uint32_t>(kNB) ? end - c0 : static_cast<uint32_t>(kNB);
+        const auto src = [&](uint32_t a) { return order[c0 + a]; };
+        float acc[kNB];
+        q4k_rows_sweep(lds, wrow, w.ffn / 256U, img, src, na, acc);
+#pragma unroll
+        for (int a = 0; a < kNB; ++a) {
+            const float v = q4k_row_tree(acc[a]);
+            if ((tid & 7U) == 0 && static_cast<uint32_t>(a) < na) r.rawdots[static_cast<size_t>(order[c0 + a]) * w.hidden + o] = v;
+        }
+    }
+}
+
+// Ordered combine of the slots of one row. Reference: include/strix/moe/combine.hpp:36-59 (fma form),
+// src/ds41_expert_tp.cpp:189-199 (product then add, slots in ascending expert id).
+__global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t form) {
+    __shared__ uint32_t slot_order[16];
+    __shared__ float slot_weight[16];
+    __shared__ uint32_t row_failed;
+    const uint32_t row = blockIdx.y, o = blockIdx.x * 256U + threadIdx.x;
+    if (threadIdx.x == 0) {
+        // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is this kernel's own)
+        row_failed = r.status[row] & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE);
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
+        if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
+            for (uint32_t i = 1; i < w.top_k; ++i)
+                for (uint32_t j = i; j > 0 && r.routes[row * w.top_k + slot_order[j]] < r.routes[row * w.top_k + slot_order[j - 1]]; --j) {
+                    const uint32_t t = slot_order[j]; slot_order[j] = slot_order[j - 1]; slot_order[j - 1] = t;
+                }
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights[row * w.top_k + slot_order[k]];
+    }
+    __syncthreads();
+    if (o >= w.hidden || row_failed) return;
+    float acc = 0.0F;
+    for (uint32_t k = 0; k < w.top_k; ++k) {
+        const float e = r.rawdots[(static_cast<size_t>(row) * w.top_k + slot_order[k]) * w.hidden + o];
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], e, acc);
+        else acc = acc + slot_weight[k] * e;
+    }
+    const float y = r.base ? acc + r.base[static_cast<size_t>(row) * w.hidden + o] : acc;
+    if (!finite_f(y)) atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
+}
+
+// SwiGLU + A8 re-quantisation of dense gate/up rows. Reference: src/cpu/core/routed_expert.cpp:147-170.
+__global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate, const float* up, uint32_t ffn, uint32_t exp_kind,
+                                                              int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status) {
+    const uint32_t row = blockIdx.y, groups = ffn / 32U, grp = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U;
+    if (grp >= groups) return;
+    const size_t at = static_cast<size_t>(row) * ffn + grp * 32U + l;
+    const float g = gate[at], u = up[at];
+    const float ex = exp_of(exp_kind, -g);
+    const float hv = (g / (1.0F + ex)) * u;
+    if (h_out) h_out[at] = hv;
+    const int bad = or32_i((finite_f(g) && finite_f(u) && finite_f(hv)) ? 0 : 1);
+    if (bad) {
+        if (l == 0 && status) atomicOr(&status[row], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+        return;
+    }
+    const float amax = max32(__builtin_fabsf(hv));
+    const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+    const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+    const int code = a8_code(hv, dl, tiny);
+    const int sum = sum32_i(code);
+    codes[at] = static_cast<int8_t>(code);
+    if (l == 0) {
+        deltas[static_cast<size_t>(row) * groups + grp] = dl;
+        sums[static_cast<size_t>(row) * groups + grp] = sum;
+    }
+}
+
+// ======================================================================================================== admission
+int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv) {
+    STRIX_REQUIRE(w && r, "moe: null weights or rows");
+    STRIX_REQUIRE(rows > 0, "moe: rows must be positive");
+    STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K, "moe: gate/up weights must be Q4_K (type 12)");
+    if (w->down_type != MI355_TYPE_Q4_K) return fail(MI355_E_UNSUPPORTED, "moe: down weights must be Q4_K (type 12)");
+    STRIX_REQUIRE(w->hidden >= 256 && w->hidden % 256U == 0, "moe: hidden must be a positive multiple of 256");
+    STRIX_REQUIRE(w->ffn >= 256 && w->ffn % 256U == 0, "moe: ffn must be a positive multiple of 256");
+    STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
+    STRIX_REQUIRE(w->top_k > 0 && w->top_k <= kRouteMaxTopK && w->top_k <= w->experts, "moe: top_k must be within 1..16 and <= experts");
+    STRIX_REQUIRE(static_cast<uint64_t>(rows) * w->top_k < (1ULL << 31), "moe: too many assignments");
+    wv = *w;
+    if (wv.gate_row_stride == 0) wv.gate_row_stride = static_cast<uint64_t>(w->hidden / 256U) * kQ4kBlock;
+    if (wv.gate_expert_stride == 0) wv.gate_expert_stride = wv.gate_row_stride * w->ffn;
+    if (wv.down_row_stride == 0) wv.down_row_stride = static_cast<uint64_t>(w->ffn / 256U) * kQ4kBlock;
+    if (wv.down_expert_stride == 0) wv.down_expert_stride = wv.down_row_stride * w->hidden;
+    STRIX_REQUIRE(wv.gate_row_stride % 16U == 0 && wv.gate_expert_stride % 16U == 0 && wv.down_row_stride % 16U == 0 &&
+                  wv.down_expert_stride % 16U == 0, "moe: weight strides must be multiples of 16 bytes");
+    STRIX_REQUIRE(wv.gate_row_stride >= static_cast<uint64_t>(w->hidden / 256U) * kQ4kBlock &&
+                  wv.down_row_stride >= static_cast<uint64_t>(w->ffn / 256U) * kQ4kBlock, "moe: weight row stride shorter than the row");
+    STRIX_REQUIRE(w->gate && w->up && w->down && aligned(w->gate, 16) && aligned(w->up, 16) && aligned(w->down, 16),
+                  "moe: weight pointers must be non-null and 16-byte aligned");
+    STRIX_REQUIRE(w->exp_kind <= MI355_EXP_DECLARED, "moe: unknown exp kind");
+    STRIX_REQUIRE(r->routes && r->route_weights && r->codes && r->deltas && r->sums && r->status && r->down_codes && r->down_deltas &&
+                  r->down_sums && r->rawdots && r->output && r->plan && r->job_status, "moe: a required row view is null");
+    STRIX_REQUIRE(aligned(r->codes, 16) && aligned(r->down_codes, 16) && aligned(r->plan, 16) && aligned(r->rawdots, 16) &&
+                  aligned(r->deltas, 4) && aligned(r->down_deltas, 4), "moe: row views must be 16-byte aligned");
+    STRIX_REQUIRE(r->output_stride >= w->hidden, "moe: output stride shorter than hidden");
+    return MI355_OK;
+}
+
+}  // namespace strix950
+
+// ============================================================================================================ C ABI
+using namespace strix950;
+
+extern "C" {
+
+const char* mi355_last_error(void) { return g_error.c_str(); }
+const char* mi355_version(void) { return "mi355-strix 0.1 (gfx950)"; }
+
+const char* mi355_numerical_identity(uint32_t weight_type, int down) {
+    // The reference's identity strings name wave32; the arithmetic clauses are the ones implemented here.
+    if (weight_type == MI355_TYPE_Q4_K && !down)
+        return "strix-moe-q4k-a8g32-probe-v2:f32-div-rne:g32-sym127-zero1-finite-noflush:"
+               "dot-s8xu8-i32:combine-separate-f32:pair-ascending-sb-tree4:writer-c0:wave64-gfx950";
+    if (weight_type == MI355_TYPE_Q4_K)
+        return "q4k-a8g32-down-v1:s8xu4-i32:delta*((d*(sc*I))-(dmin*(m*S))):pair-ascending-sb-tree4:"
+               "silu-div-expf-times-up:g32-sym127-f32delta-rne:tiny-lt2^-119-zero1:raw-slot-major:finite-failclosed";
+    if (weight_type == MI355_TYPE_Q8_0) return "cpu-q8a8-tree32@1";
+    return "";
+}
+
+int32_t mi355_dequantize_rows(uint32_t type, const void* rows, uint64_t row_stride, uint32_t n_rows, uint32_t elements,
+                              float* out, uint64_t out_stride, mi355_stream stream) {
+    if (type != MI355_TYPE_Q8_0 && type != MI355_TYPE_Q4_K) return fail(MI355_E_UNSUPPORTED, "dequantize: type must be Q8_0 (8) or Q4_K (12)");
+    const uint32_t be = type == MI355_TYPE_Q8_0 ? 32U : 256U, bb = type == MI355_TYPE_Q8_0 ? kQ80Block : kQ4kBlock;
+    STRIX_REQUIRE(rows && out, "dequantize: null pointer");
+    STRIX_REQUIRE(elements % be == 0, "dequantize: row length is not a multiple of the block");
+    STRIX_REQUIRE(row_stride >= static_cast<uint64_t>(elements / be) * bb && out_stride >= elements, "dequantize: stride shorter than the row");
+    if (n_rows == 0 || elements == 0) return MI355_OK;
+    const uint32_t gx = (elements + 255U) / 256U;
+    for (uint32_t r0 = 0; r0 < n_rows; r0 += 65535U) {
+        const uint32_t nr = n_rows - r0 < 65535U ? n_rows - r0 : 65535U;
+        dequantize_rows_kernel<<<dim3(gx < 64U ? gx : 64U, nr), 256, 0, hs(stream)>>>(
+            type, static_cast<const uint8_t*>(rows) + r0 * row_stride, row_stride, elements, out + r0 * out_stride, out_stride);
+    }
+    STRIX_LAUNCHED("dequantize_rows");
+    return MI355_OK;
+}
+
+int32_t mi355_quantize_weight_rows(uint32_t type, const float* x, uint32_t n_rows, uint32_t elements, void* out, mi355_stream stream) {
+    if (type != MI355_TYPE_Q8_0 && type != MI355_TYPE_Q4_K) return fail(MI355_E_UNSUPPORTED, "quantize_weight: type must be Q8_0 (8) or Q4_K (12)");
+    const uint32_t be = type == MI355_TYPE_Q8_0 ? 32U : 256U;
+    STRIX_REQUIRE(x && out, "quantize_weight: null pointer");
+    STRIX_REQUIRE(elements % be == 0, "quantize_weight: row length is not a multiple of the block");
+    const uint64_t blocks = static_cast<uint64_t>(n_rows) * (elements / be);
+    if (blocks == 0) return MI355_OK;
+    if (type == MI355_TYPE_Q8_0) {
+        const uint64_t g = (blocks + 255U) / 256U;
+        quantize_q8_0_rows_kernel<<<static_cast<uint32_t>(g < 65535U ? g : 65535U), 256, 0, hs(stream)>>>(x, blocks, static_cast<uint8_t*>(out));
+    } else {
+        const uint64_t g = (blocks + 63U) / 64U;
+        quantize_q4_k_rows_kernel<<<static_cast<uint32_t>(g < 262144U ? g : 262144U), 64, 0, hs(stream)>>>(x, blocks, static_cast<uint8_t*>(out));
+    }
+    STRIX_LAUNCHED("quantize_weight_rows");
+    return MI355_OK;
+}
+
+int32_t mi355_quantize_a8(const void* x, uint32_t kind, uint32_t rows, uint32_t width, uint64_t x_stride, int8_t* codes, float* deltas,
+                          int32_t* sums, uint32_t* status, mi355_stream stream) {
+    STRIX_REQUIRE(width % 32U == 0, "A8 activation width must be a multiple of 32");
+    STRIX_REQUIRE(kind <= MI355_INPUT_BF16, "A8: unknown input kind");
+    if (rows == 0 || width == 0) return MI355_OK;
+    STRIX_REQUIRE(x && codes && deltas, "A8: null pointer");
+    STRIX_REQUIRE(rows <= 65535U, "A8: at most 65535 rows per call");
+    const dim3 grid((width / 32U + 7U) / 8U, rows);
+    const uint8_t* xb = static_cast<const uint8_t*>(x);
+    if (kind == MI355_INPUT_F32) quantize_a8_kernel<0><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, sums, status);
+    else if (kind == MI355_INPUT_F16) quantize_a8_kernel<1><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, sums, status);
+    else quantize_a8_kernel<2><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, sums, status);
+    STRIX_LAUNCHED("quantize_a8");
+    return MI355_OK;
+}
+
+int32_t mi355_gemv_q8_0_a8(const mi355_q8a8_view* v, mi355_stream stream) {
+    STRIX_REQUIRE(v, "Q8_0 product: null view");
+    STRIX_REQUIRE(v->in % 32U == 0, "Q8_0 product width must be a multiple of 32");
+    if (v->rows == 0 || v->count == 0) return MI355_OK;
+    STRIX_REQUIRE(v->weight && v->codes && v->deltas && v->out, "Q8_0 product: null pointer");
+    STRIX_REQUIRE(aligned(v->weight, 2) && v->row_bytes % 2U == 0, "Q8_0 product: weight rows must be 2-byte aligned");
+    STRIX_REQUIRE(aligned(v->codes, 16) && v->x_stride % 32U == 0 && v->x_stride >= v->in, "Q8_0 product: codes must be 16-byte aligned with x_stride a multiple of 32");
+    STRIX_REQUIRE(v->row_bytes >= v->in / 32U * kQ80Block && v->out_stride >= v->count, "Q8_0 product: stride shorter than the row");
+    const uint32_t grid = (v->count + 7U) / 8U;
+    for (uint32_t r0 = 0; r0 < v->rows; r0 += 8U) gemv_q8_0_a8_kernel<8><<<grid, 256, 0, hs(stream)>>>(*v, r0);
+    STRIX_LAUNCHED("gemv_q8_0_a8");
+    return MI355_OK;
+}
+
+int32_t mi355_moe_route(const mi355_route_policy* p, const void* x, uint32_t kind, uint32_t rows, uint32_t hidden, uint64_t x_stride,
+                        const float* wr, const float* bias, uint32_t* ids, float* weights, float* scores, mi355_stream stream) {
+    STRIX_REQUIRE(p && x && wr && ids && weights && scores, "route: null pointer");
+    STRIX_REQUIRE(p->experts > 0 && p->experts <= kRouteMaxExperts && p->top_k > 0 && p->top_k <= kRouteMaxTopK && p->top_k <= p->experts,
+                  "route policy: need 0 < top_k <= experts, experts <= 1024, top_k <= 16");
+    STRIX_REQUIRE(hidden > 0 && hidden <= kRouteMaxHidden && hidden % 4U == 0, "route: hidden must be a multiple of 4 within 8192");
+    STRIX_REQUIRE(kind <= MI355_INPUT_BF16 && p->logits_order <= MI355_LOGITS_LANE32_BUTTERFLY, "route: unknown input kind or logits order");
+    STRIX_REQUIRE(aligned(wr, 16), "route: router weight must be 16-byte aligned");
+    if (rows == 0) return MI355_OK;
+    route_kernel<<<rows, 256, 0, hs(stream)>>>(*p, static_cast<const uint8_t*>(x), kind, hidden, x_stride, wr, bias, ids, weights, scores);
+    STRIX_LAUNCHED("moe_route");
+    return MI355_OK;
+}
+
+size_t mi355_moe_plan_words(uint32_t experts, uint32_t rows, uint32_t top_k) {
+    return plan_order_at(experts) + ((static_cast<size_t>(rows) * top_k + 3U) & ~static_cast<size_t>(3));
+}
+
+int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    STRIX_REQUIRE(r->input && r->input_kind <= MI355_INPUT_BF16, "moe prologue: input view invalid");
+    clear_validate_kernel<<<rows, 64, 0, hs(stream)>>>(r->routes, r->route_weights, wv.experts, wv.top_k, r->status, r->job_status);
+    STRIX_LAUNCHED("moe clear/validate");
+    return mi355_quantize_a8(r->input, r->input_kind, rows, wv.hidden, r->input_stride, r->codes, r->deltas, r->sums, r->status, stream);
+}
+
+int32_t mi355_moe_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    plan_kernel<<<1, 1024, 0, hs(stream)>>>(r->routes, wv.experts, rows * wv.top_k, r->plan);
+    STRIX_LAUNCHED("moe plan");
+    return MI355_OK;
+}
+
+int32_t mi355_moe_enqueue_project(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    project_kernel<<<dim3(wv.ffn / 32U, wv.experts), 256, 0, hs(stream)>>>(wv, *r);
+    STRIX_LAUNCHED("moe project");
+    return MI355_OK;
+}
+
+int32_t mi355_moe_enqueue_down(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    down_kernel<<<dim3(wv.hidden / 32U, wv.experts), 256, 0, hs(stream)>>>(wv, *r);
+    STRIX_LAUNCHED("moe down");
+    return MI355_OK;
+}
+
+int32_t mi355_moe_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe merge: unknown combine form");
+    STRIX_REQUIRE(rows <= 65535U, "moe merge: at most 65535 rows per call");
+    merge_kernel<<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(wv, *r, form);
+    STRIX_LAUNCHED("moe merge");
+    return MI355_OK;
+}
+
+int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;   // the whole bundle is validated before the first enqueue
+    STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
+    STRIX_REQUIRE(r->input && r->input_kind <= MI355_INPUT_BF16, "moe: input view invalid");
+    if (const int32_t rc = mi355_moe_enqueue_prologue(w, r, rows, stream)) return rc;
+    if (const int32_t rc = mi355_moe_enqueue_csr(w, r, rows, stream)) return rc;
+    if (const int32_t rc = mi355_moe_enqueue_project(w, r, rows, stream)) return rc;
+    if (const int32_t rc = mi355_moe_enqueue_down(w, r, rows, stream)) return rc;
+    return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+}
+
+int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows, uint32_t ffn, uint32_t exp_kind, int8_t* codes,
+                              float* deltas, int32_t* sums, float* h_out, uint32_t* status, mi355_stream stream) {
+    STRIX_REQUIRE(ffn % 32U == 0, "swiglu: ffn must be a multiple of 32");
+    STRIX_REQUIRE(exp_kind <= MI355_EXP_DECLARED, "swiglu: unknown exp kind");
+    if (rows == 0 || ffn == 0) return MI355_OK;
+    STRIX_REQUIRE(gate && up && codes && deltas && sums, "swiglu: null pointer");
+    STRIX_REQUIRE(rows <= 65535U, "swiglu: at most 65535 rows per call");
+    swiglu_quantize_kernel<<<dim3((ffn / 32U + 7U) / 8U, rows), 256, 0, hs(stream)>>>(gate, up, ffn, exp_kind, codes, deltas, sums, h_out, status);
+    STRIX_LAUNCHED("swiglu_quantize");
+    return MI355_OK;
+}
+
+}  // extern "C"

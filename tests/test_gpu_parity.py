@@ -1,0 +1,376 @@
+"""GPU parity tests: every value comes through the C ABI (libmi355_strix.so) and is compared with the CPU oracle on the
+same seeded inputs. Integer / byte / index results and the declared fp32 chains must be bit-exact; whole-layer outputs
+are additionally held to the stated tolerances (fp32-accumulated outputs: max relative error 1e-3; fp16 activations
+2e-3), with "relative" = |gpu - ref| / rms(ref) and the elementwise form restricted to |ref| > 1e-2 rms(ref)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import orc
+
+pytestmark = pytest.mark.gpu
+TOL_F32, TOL_F16 = 1e-3, 2e-3
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def rel_err(got, want):
+    want64 = want.astype(np.float64)
+    rms = np.sqrt(np.mean(want64 ** 2)) + 1e-30
+    abs_over_rms = np.max(np.abs(got - want64)) / rms
+    big = np.abs(want64) > 1e-2 * rms
+    elementwise = np.max(np.abs(got[big] - want64[big]) / np.abs(want64[big])) if big.any() else 0.0
+    return abs_over_rms, elementwise
+
+
+def random_q4k(rng, shape_rows, width):
+    w = rng.integers(0, 256, shape_rows + (width // 256 * 144,), dtype=np.uint8)
+    w[..., 1::144] = (w[..., 1::144] & 0x03) | 0x0C | (rng.integers(0, 2, w[..., 1::144].shape, dtype=np.uint8) << 4)
+    w[..., 3::144] = (w[..., 3::144] & 0x03) | 0x0C
+    return w
+
+
+# ------------------------------------------------------------------------------------------- block decode / writers
+@pytest.mark.parametrize("qtype,width", [(orc.Q8_0, 4096), (orc.Q4_K, 2048), (orc.Q4_K, 5120)])
+def test_dequantised_weights_bit_exact(strix, qtype, width):
+    rng = np.random.default_rng(100 + width)
+    rb = orc.row_bytes(qtype, width)
+    raw = rng.integers(0, 256, (37, rb), dtype=np.uint8)
+    if qtype == orc.Q8_0:   # every fp16 scale pattern incl. subnormals, infinities excluded from the bit compare below
+        raw[:, 1::34] &= 0xFB
+    else:
+        raw[:, 1::144] &= 0xFB
+        raw[:, 3::144] &= 0xFB
+    got = strix.dequantize_rows(qtype, dev(raw), width).cpu().numpy()
+    want = orc.dequant_rows(qtype, raw, width)
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_fp16_scale_decode_all_65536_values(strix):
+    blocks = np.zeros((65536, 34), np.uint8)
+    h = np.arange(65536, dtype=np.uint16)
+    blocks[:, 0], blocks[:, 1], blocks[:, 2] = h & 255, h >> 8, 1
+    got = strix.dequantize_rows(orc.Q8_0, dev(blocks.reshape(64, -1)), 1024 * 32).cpu().numpy().reshape(65536, 32)[:, 0]
+    want = h.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(bits(got)[~nan], bits(want)[~nan])
+
+
+@pytest.mark.parametrize("qtype", [orc.Q8_0, orc.Q4_K])
+def test_weight_writers_match_oracle_bytes(strix, qtype):
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal((64, 2048)) * 0.02).astype(np.float32)
+    x[3, :64] = 0
+    x[5, 256:512] = np.abs(x[5, 256:512])
+    got = strix.quantize_weight_rows(qtype, dev(x)).cpu().numpy()
+    assert np.array_equal(got, orc.quantize_rows(qtype, x))
+
+
+# ------------------------------------------------------------------------------------------- A8 quantiser
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_quantize_a8_bit_exact(strix, dtype):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((9, 5120)).astype(dtype)
+    x[1, :32] = 0
+    x[2, 32:64] = dtype(6e-8) if dtype == np.float16 else 1e-37
+    x[3, 64:96] *= dtype(100)
+    if dtype == np.float32:
+        x[4, :32] = np.float32(2.0 ** -120)     # tiny rule: codes 0, delta 1
+        x[4, 32:64] = np.float32(2.0 ** -119)   # not tiny
+        x[5, 0], x[5, 1] = np.array([0x3A8BE27E, 0x37B03B95], np.uint32).view(np.float32)  # division-then-round hard case
+        x[5, 2:32] = 0
+    codes, deltas, sums, status = strix.quantize_a8(dev(x))
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32), tiny_rule=True)
+    assert np.array_equal(codes.cpu().numpy(), c)
+    assert np.array_equal(bits(deltas.cpu().numpy()), bits(d))
+    assert np.array_equal(sums.cpu().numpy(), s)
+    assert np.all(status.cpu().numpy() == 0)
+
+
+def test_quantize_a8_rejects_partial_group_before_any_write(strix):
+    x = torch.ones((1, 64), device="cuda")
+    codes = torch.full((1, 64), 17, dtype=torch.int8, device="cuda")
+    deltas = torch.full((1, 2), 19.0, device="cuda")
+    for width in (31, 33):
+        rc = strix.lib().mi355_quantize_a8(C.c_void_p(x.data_ptr()), 0, 1, width, C.c_uint64(256), C.c_void_p(codes.data_ptr()),
+                                           C.c_void_p(deltas.data_ptr()), None, None, None)
+        assert rc == strix.E_INVALID_ARGUMENT and b"multiple of 32" in strix.lib().mi355_last_error()
+    torch.cuda.synchronize()
+    assert bool((codes == 17).all()) and bool((deltas == 19).all())
+
+
+def test_nonfinite_activation_sets_status(strix):
+    x = torch.randn((3, 256), device="cuda")
+    x[1, 7] = float("inf")
+    *_, status = strix.quantize_a8(x)
+    assert status.cpu().tolist() == [0, strix.STATUS_NONFINITE_ACTIVATION, 0]
+
+
+# ------------------------------------------------------------------------------------------- config 1: dense Q8_0 GEMV
+def test_config1_dense_q8_0_gemv_bit_exact(strix):
+    """BASELINE config 1: x[4096] ~ N(0,1) fp32, W 4096x4096 ~ N(0,0.02) -> Q8_0 by the ggml rule, y = W x."""
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((1, 4096)).astype(np.float32)
+    w = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((4096, 4096)) * 0.02).astype(np.float32))
+    codes, deltas, _, _ = strix.quantize_a8(dev(x))
+    y = strix.gemv_q8_0_a8(dev(w), codes, deltas, 4096, 4096).cpu().numpy()
+    c, d, s, _ = orc.quantize_a8(x)
+    want, _ = orc.gemv_q8_0_a8(w, c, d, 4096, 4096, threads=8)
+    assert np.array_equal(bits(y), bits(want))
+    exact = x.astype(np.float64) @ orc.dequant_rows(orc.Q8_0, w, 4096).astype(np.float64).T
+    assert rel_err(y, exact.astype(np.float32))[0] < 2e-2    # informational: distance of the A8 class from exact weights
+
+
+def test_q8_0_gemv_order_fixture_rows_accumulate_and_padding(strix):
+    g = 33
+    w = np.zeros(g * 34, np.uint8)
+    w[1::34], w[2::34] = 0x3C, 1
+    codes = np.ones((1, g * 32), np.int8)
+    deltas = np.zeros((1, g), np.float32)
+    deltas[0, 0], deltas[0, 16], deltas[0, 1], deltas[0, 32] = 2.0 ** 24, -2.0 ** 24, 1, 1
+    y = torch.full((1, 1), -1.0, device="cuda")
+    strix.gemv_q8_0_a8(dev(w), dev(codes), dev(deltas), g * 32, 1, out=y)
+    assert y.item() == 1.0
+    y.fill_(-1.0)
+    strix.gemv_q8_0_a8(dev(w), dev(codes), dev(deltas), g * 32, 1, out=y, accumulate=True)
+    assert y.item() == 0.0
+    # 11 rows x 19 outputs with padded strides, against the oracle
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((11, 1024)).astype(np.float32)
+    wq = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((19, 1024)) * 0.02).astype(np.float32))
+    c, d, s, _ = orc.quantize_a8(x)
+    out = torch.full((11, 24), 29.0, device="cuda")
+    strix.gemv_q8_0_a8(dev(wq), dev(c), dev(d), 1024, 19, out=out)
+    want, _ = orc.gemv_q8_0_a8(wq, c, d, 1024, 19)
+    got = out.cpu().numpy()
+    assert np.array_equal(bits(got[:, :19]), bits(want)) and np.all(got[:, 19:] == 29.0)
+    v = strix.Q8a8View(1, 1, 1, 1, 68, 33, 1, 1, 64, 1, 0)
+    assert strix.lib().mi355_gemv_q8_0_a8(C.byref(v), None) == strix.E_INVALID_ARGUMENT
+
+
+# ------------------------------------------------------------------------------------------- router
+@pytest.mark.parametrize("experts,hidden,rows,bias", [(128, 2048, 8, False), (256, 4096, 32, True), (160, 6144, 16, False)])
+def test_router_topk_ids_bit_exact(strix, experts, hidden, rows, bias):
+    rng = np.random.default_rng(experts)
+    x = rng.standard_normal((rows, hidden)).astype(np.float16)
+    wr = (rng.standard_normal((experts, hidden)) * 0.02).astype(np.float32)
+    b = (rng.standard_normal(experts) * 1.5).astype(np.float32) if bias else None
+    ids, wts, scores = strix.route(dev(x), dev(wr), 8, bias=None if b is None else dev(b))
+    ids_ref, w_ref, s_ref, _ = orc.route(x.astype(np.float32), wr, 8, bias=b)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref)
+    assert np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    assert np.array_equal(bits(scores.cpu().numpy()), bits(s_ref))
+
+
+def test_router_exact_ties_lane32_order_and_policy_constants(strix):
+    rng = np.random.default_rng(5)
+    x = np.zeros((4, 256), np.float16)
+    x[:, 0] = 1
+    wr = np.zeros((64, 256), np.float32)
+    wr[:, 0] = (rng.integers(-8, 9, 64) / 4.0)           # many exact ties: the lower id must win
+    ids, wts, _ = strix.route(dev(x), dev(wr), 6, renorm_eps=1e-20, scale=2.5)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, 6, renorm_eps=1e-20, scale=2.5)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    x = rng.standard_normal((3, 512)).astype(np.float32)
+    wr = (rng.standard_normal((32, 512)) * 0.05).astype(np.float32)
+    ids, wts, sc = strix.route(dev(x), dev(wr), 4, logits_order=strix.LOGITS_LANE32)
+    ids_ref, w_ref, s_ref, _ = orc.route(x, wr, 4, logits_order=orc.LOGITS_LANE32)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(sc.cpu().numpy()), bits(s_ref))
+
+
+# ------------------------------------------------------------------------------------------- routed experts, stage by stage
+def make_layer(rng, H, I, E, full_entropy=False):
+    if full_entropy:
+        return random_q4k(rng, (E, I), H), random_q4k(rng, (E, I), H), random_q4k(rng, (E, H), I)
+    q = lambda shape: orc.quantize_rows(orc.Q4_K, (rng.standard_normal(shape) * 0.02).astype(np.float32))
+    return q((E, I, H)), q((E, I, H)), q((E, H, I))
+
+
+def run_layer_both(strix, H, I, E, K, T, seed, full_entropy=False, combine=0, exp_kind=0, tp=None):
+    rng = np.random.default_rng(seed)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    kw, okw, ffn = {}, {}, I
+    g_np, u_np, d_np = gate, up, down
+    if tp is not None:   # this rank's share of every expert, read in place from the unsplit tensors through strides
+        rank, ranks = tp
+        ffn = I // ranks
+        grb, drb = H // 256 * 144, I // 256 * 144
+        kw = dict(gate_expert_stride=I * grb, gate_row_stride=grb, down_expert_stride=H * drb, down_row_stride=drb)
+        okw = kw
+        g_np, u_np, d_np = gate.reshape(-1)[rank * ffn * grb:], up.reshape(-1)[rank * ffn * grb:], down.reshape(-1)[rank * (ffn // 256) * 144:]
+    gd, ud, dd = dev(gate.reshape(-1)), dev(up.reshape(-1)), dev(down.reshape(-1))
+    if tp is not None:
+        off_g, off_d = tp[0] * ffn * (H // 256 * 144), tp[0] * (ffn // 256) * 144
+        gd_v, ud_v, dd_v = gd[off_g:], ud[off_g:], dd[off_d:]
+    else:
+        gd_v, ud_v, dd_v = gd, ud, dd
+    layer = strix.MoeLayer(H, ffn, E, K, gd_v, ud_v, dd_v, T, exp_kind=exp_kind, intermediates=True, **kw)
+    y = layer.run(dev(x), dev(ids_ref.astype(np.int32)), dev(w_ref), combine=combine).cpu().numpy()
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    ref = orc.routed_experts(H, ffn, K, g_np, u_np, d_np, orc.Q4_K, c, d, s, ids_ref, exp_kind=exp_kind, **okw)
+    want = orc.combine(combine, w_ref, ids_ref, ref.rawdots)
+    return layer, y, ref, want, (c, d, s), ids_ref, w_ref, (g_np, u_np, d_np, ffn, okw)
+
+
+def check_layer_stages(strix, layer, y, ref, want, a8, ids_ref, w_ref, tensors, H, K, T, combine, exp_kind, tol):
+    g_np, u_np, d_np, ffn, okw = tensors
+    c, d, s = a8
+    n = T * K
+    # (1) device A8 image of the input == oracle
+    assert np.array_equal(layer.codes[:T].cpu().numpy(), c) and np.array_equal(bits(layer.deltas[:T].cpu().numpy()), bits(d))
+    assert np.array_equal(layer.sums[:T].cpu().numpy(), s)
+    # (2) device gate / up bits == oracle (the declared fp32 chain, any lane schedule)
+    assert np.array_equal(bits(layer.gate_out[:n].cpu().numpy()), bits(ref.gate))
+    assert np.array_equal(bits(layer.up_out[:n].cpu().numpy()), bits(ref.up))
+    # (3) the device's own h, re-quantised on the CPU, == the device's down image (so exp never enters a bit compare) ...
+    h_dev = layer.h_out[:n].cpu().numpy()
+    hc, hd, hs, _ = orc.quantize_a8(h_dev, tiny_rule=True)
+    dc, dd_, ds = layer.down_codes[:n].cpu().numpy(), layer.down_deltas[:n].cpu().numpy(), layer.down_sums[:n].cpu().numpy()
+    assert np.array_equal(dc, hc) and np.array_equal(bits(dd_), bits(hd)) and np.array_equal(ds, hs)
+    # ... and h itself is within an ulp or two of the oracle's h (the device exp2 in double vs the host's)
+    assert np.max(np.abs(h_dev - ref.h)) <= 4e-7 * np.max(np.abs(ref.h))
+    h_codes_equal = np.array_equal(dc, ref.h_codes)
+    # (4) device rawdot bits == oracle down rows evaluated on the DEVICE's down image
+    ref_down = orc.routed_experts(H, ffn, K, g_np, u_np, d_np, orc.Q4_K, c, d, s, ids_ref, exp_kind=exp_kind,
+                                  down_only_from=(dc, dd_, ds), **okw)
+    raw_dev = layer.rawdots[:T].cpu().numpy()
+    assert np.array_equal(bits(raw_dev), bits(ref_down.rawdots))
+    # (5) combine bits from the device rawdots
+    assert np.array_equal(bits(y), bits(orc.combine(combine, w_ref, ids_ref, raw_dev)))
+    # (6) whole layer vs the oracle end to end: tolerance, and bit-exact whenever the h codes agree
+    a, e = rel_err(y, want)
+    assert a < tol and e < tol, (a, e)
+    if h_codes_equal:
+        assert np.array_equal(bits(y), bits(want))
+    assert np.all(layer.status[:T].cpu().numpy() == 0)
+    return h_codes_equal
+
+
+@pytest.mark.parametrize("H,I,E,K,T,full", [(512, 256, 6, 2, 3, False), (2048, 768, 16, 8, 8, False), (768, 512, 5, 3, 11, True),
+                                            (2560, 256, 4, 2, 1, True)])
+def test_moe_layer_stage_by_stage_bit_exact(strix, H, I, E, K, T, full):
+    out = run_layer_both(strix, H, I, E, K, T, seed=H + T, full_entropy=full)
+    check_layer_stages(strix, *out[:7], out[7], H, K, T, 0, 0, TOL_F16)
+
+
+def test_moe_layer_declared_exp_is_bit_exact_end_to_end(strix):
+    """With the declared exp (basic IEEE operations only) host and device share every bit of the layer."""
+    H, I, E, K, T = 1024, 512, 8, 4, 5
+    layer, y, ref, want, *_ = run_layer_both(strix, H, I, E, K, T, seed=77, exp_kind=1)
+    assert np.array_equal(layer.down_codes[:T * K].cpu().numpy(), ref.h_codes)
+    assert np.array_equal(bits(layer.h_out[:T * K].cpu().numpy()), bits(ref.h))
+    assert np.array_equal(bits(y), bits(want))
+
+
+def test_config3_moe_decode_layer_shape(strix):
+    """BASELINE config 3 geometry (hidden 2048, 128 experts, top-8, intermediate 768) at 1 / 4 / 8 tokens, router included."""
+    H, I, E, K = 2048, 768, 128, 8
+    rng = np.random.default_rng(3)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    gd, ud, dd, wrd = dev(gate), dev(up), dev(down), dev(wr)
+    layer = strix.MoeLayer(H, I, E, K, gd, ud, dd, 8, intermediates=True)
+    for T in (1, 4, 8):
+        x = rng.standard_normal((T, H)).astype(np.float16)
+        xd = dev(x)
+        ids, wts, _ = strix.route(xd, wrd, K)
+        y = layer.run(xd, ids, wts).cpu().numpy()
+        ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+        assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref)          # top-k ids bit-exact
+        assert np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+        c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+        ref = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref)
+        want = orc.combine(0, w_ref, ids_ref, ref.rawdots)
+        check_layer_stages(strix, layer, y, ref, want, (c, d, s), ids_ref, w_ref, (gate, up, down, I, {}), H, K, T, 0, 0, TOL_F16)
+
+
+def test_config5_tp_rank_partial_sums(strix):
+    """BASELINE config 5 structure at reduced size: rank 0 of TP = 2 holds the first half of every expert's intermediate
+    rows and the matching K blocks of every down row, read in place through strides; the kernel emits the rank's partial
+    sums (product-then-add fold in ascending expert id), with no cross-rank reduction."""
+    H, I, E, K, T = 1536, 1024, 10, 4, 16
+    for rank in (0, 1):
+        out = run_layer_both(strix, H, I, E, K, T, seed=55, combine=1, tp=(rank, 2))
+        check_layer_stages(strix, *out[:7], out[7], H, K, T, 1, 0, TOL_F16)
+
+
+def test_dense_q4k_ffn_is_the_single_expert_case(strix):
+    """BASELINE config 2 structure at reduced size: a dense Q4_K FFN is the one-expert, top-1, weight-1 layer."""
+    H, I = 1280, 1792
+    for T in (1, 4, 8):
+        rng = np.random.default_rng(20 + T)
+        gate, up, down = make_layer(rng, H, I, 1)
+        x = rng.standard_normal((T, H)).astype(np.float16)
+        ids = np.zeros((T, 1), np.int32)
+        w = np.ones((T, 1), np.float32)
+        layer = strix.MoeLayer(H, I, 1, 1, dev(gate), dev(up), dev(down), T, intermediates=True)
+        y = layer.run(dev(x), dev(ids), dev(w)).cpu().numpy()
+        c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+        ref = orc.routed_experts(H, I, 1, gate, up, down, orc.Q4_K, c, d, s, ids.astype(np.uint32))
+        want = orc.combine(0, w, ids.astype(np.uint32), ref.rawdots)
+        check_layer_stages(strix, layer, y, ref, want, (c, d, s), ids.astype(np.uint32), w, (gate, up, down, I, {}), H, 1, T, 0, 0, TOL_F16)
+        # informational: the A8 class sits ~0.5 % from the exact-weight product, which is why classes are never mixed
+        g_exact = orc.base_linear(orc.Q4_K, gate[0], H // 256 * 144, I, H, x.astype(np.float32))
+        assert 1e-4 < rel_err(layer.gate_out[:T].cpu().numpy(), g_exact)[0] < 5e-2
+
+
+# ------------------------------------------------------------------------------------------- failure handling
+def test_invalid_route_and_nonfinite_projection_fail_closed(strix):
+    H, I, E, K, T = 512, 256, 4, 2, 3
+    rng = np.random.default_rng(9)
+    gate, up, down = make_layer(rng, H, I, E)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    ids = np.array([[0, 1], [2, 9], [3, 1]], np.int32)     # row 1 names expert 9 >= E
+    w = np.full((T, K), 0.5, np.float32)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T)
+    layer.output.fill_(-7.0)
+    y = layer.run(dev(x), dev(ids), dev(w)).cpu().numpy()
+    st = layer.status[:T].cpu().numpy()
+    assert st[1] & strix.STATUS_INVALID_ROUTE and st[0] == 0 and st[2] == 0
+    assert np.all(y[1] == -7.0) and np.all(y[0] != -7.0)    # the flagged row publishes nothing
+    # a non-finite projection (huge activation delta, forced from the host) stops the job before the down phase
+    ids[1, 1] = 0
+    layer.stage("prologue", dev(x), dev(ids), dev(w))
+    layer.stage("csr", dev(x), dev(ids), dev(w))
+    layer.deltas[1, 3] = 3.0e38
+    layer.rawdots.fill_(-3.0)
+    layer.stage("project", dev(x), dev(ids), dev(w))
+    layer.stage("down", dev(x), dev(ids), dev(w))
+    st = layer.status[:T].cpu().numpy()
+    assert st[1] & strix.STATUS_NONFINITE_PROJECTION and st[0] == 0
+    assert bool((layer.rawdots == -3.0).all())
+
+
+def test_admission_failures_return_before_any_enqueue(strix):
+    H, I, E, K, T = 512, 256, 4, 2, 2
+    rng = np.random.default_rng(10)
+    gate, up, down = make_layer(rng, H, I, E)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T)
+    x = dev(rng.standard_normal((T, H)).astype(np.float16))
+    ids, w = dev(np.zeros((T, K), np.int32)), dev(np.ones((T, K), np.float32))
+    layer.output.fill_(5.0)
+    for field, value in (("hidden", 500), ("ffn", 100), ("top_k", 17), ("gate_type", 13), ("gate", 8)):
+        saved = getattr(layer.w, field)
+        setattr(layer.w, field, value)
+        with pytest.raises(strix.StrixError) as err:
+            layer.run(x, ids, w)
+        assert err.value.code == strix.E_INVALID_ARGUMENT
+        setattr(layer.w, field, saved)
+    layer.w.down_type = 7
+    with pytest.raises(strix.StrixError) as err:
+        layer.run(x, ids, w)
+    assert err.value.code == strix.E_UNSUPPORTED
+    layer.w.down_type = 12
+    torch.cuda.synchronize()
+    assert bool((layer.output == 5.0).all())
