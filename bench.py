@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized weight-product path on one MI355X.
+
+A step is one pass of the headline workload, BASELINE config 3: one MoE decode layer (hidden 2048, 128 experts, softmax
+router top-8, expert intermediate 768, Q4_K gate/up/down, 8 fp16 tokens) = router + A8 prologue + expert plan + gate/up/
+SwiGLU/re-quantise + down + ordered combine. Inputs are resident in HBM before the timed region. To keep the experts out
+of the 256 MB last-level cache between steps, the steps rotate over several independent layers (distinct weights and
+tokens), as consecutive layers of a model do.
+
+Prints ONE JSON line. `value` = microseconds per layer (lower is better). `roofline` prices the dominant kernel (gate/up
+projection) by its algorithmic bytes against the 8 TB/s HBM peak, from HIP events recorded around that kernel on its own
+stream inside this run. `cpu_baseline` times the CPU oracle (a port of the reference's CPU path) on the same layer."""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBPS = 8000.0     # MI355X published HBM3E peak
+Q4K_ROW = lambda k: k // 256 * 144
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--tokens", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=6, help="independent layers rotated through (cold-cache working set)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--extra", action="store_true", help="also time BASELINE configs 1, 2 and 5 (reported under 'extra')")
+    return ap.parse_args()
+
+
+class Config3:
+    H, I, E, K = 2048, 768, 128, 8
+
+    def __init__(self, strix, torch, layers, tokens, seed=3):
+        self.strix, self.torch, self.T = strix, torch, tokens
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        H, I, E, K = self.H, self.I, self.E, self.K
+        self.layers = []
+        for _ in range(layers):
+            q = lambda shape: strix.quantize_weight_rows(strix.TYPE_Q4_K, torch.randn(shape, generator=g, device="cuda") * 0.02)
+            gate, up, down = q((E, I, H)), q((E, I, H)), q((E, H, I))
+            wr = torch.randn((E, H), generator=g, device="cuda") * 0.02
+            x = torch.randn((tokens, H), generator=g, device="cuda").to(torch.float16)
+            layer = strix.MoeLayer(H, I, E, K, gate, up, down, tokens)
+            self.layers.append((layer, wr, x))
+        torch.cuda.synchronize()
+
+    def step(self, i):
+        layer, wr, x = self.layers[i % len(self.layers)]
+        ids, wts, _ = self.strix.route(x, wr, self.K)
+        layer.run(x, ids, wts)
+
+    def staged_step(self, i, events):
+        """Same work, one entry point per stage, with an event pair around each stage on the launch stream."""
+        torch, strix = self.torch, self.strix
+        layer, wr, x = self.layers[i % len(self.layers)]
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(7)]
+        marks[0].record()
+        ids, wts, _ = strix.route(x, wr, self.K)
+        marks[1].record()
+        for n, name in enumerate(("prologue", "csr", "project", "down", "merge")):
+            layer.stage(name, x, ids, wts)
+            marks[2 + n].record()
+        events.append(marks)
+        return ids
+
+    def distinct_experts(self):
+        out = []
+        for layer, wr, x in self.layers:
+            ids, _, _ = self.strix.route(x, wr, self.K)
+            out.append(int(self.torch.unique(ids).numel()))
+        return out
+
+    def layer_bytes(self, u):
+        return u * 3 * self.I * Q4K_ROW(self.H) + self.E * self.H * 4 + self.T * (self.H * 2 + self.H * 4)
+
+    def project_bytes(self, u):
+        # gate + up rows of the touched experts, the A8 image read and the h image written
+        return u * 2 * self.I * Q4K_ROW(self.H) + self.T * self.H * 1.25 + self.T * self.K * self.I * 1.25
+
+
+def time_steps(torch, fn, steps, warmup):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(warmup + i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def cpu_baseline_config3(cfg, budget_s=12.0):
+    """The CPU oracle (port of the reference's CPU path) on layer 0 of the same workload, all host threads."""
+    import orc
+    layer, wr, x = cfg.layers[0]
+    H, I, E, K, T = cfg.H, cfg.I, cfg.E, cfg.K, cfg.T
+    gate, up, down = (t.cpu().numpy() for t in (layer.gate, layer.up, layer.down))
+    xn, wrn = x.cpu().numpy().astype(np.float32), wr.cpu().numpy()
+    threads = orc.lib().orc_max_threads()
+
+    def run():
+        ids, wts, _, _ = orc.route(xn, wrn, K, threads=threads)
+        c, d, s, _ = orc.quantize_a8(xn)
+        r = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids, threads=threads, want_intermediates=False)
+        return orc.combine(orc.COMBINE_FMA_SLOT, wts, ids, r.rawdots)
+
+    run()
+    times, t_end = [], time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {"value": med * 1e6, "unit": "us/layer", "cores": threads, "kind": "port",
+            "sample": f"layer 0 of the same config-3 workload (T={T}), median of {len(times)} passes after one warm-up; "
+                      "scalar C restatement of the reference CPU path, OpenMP over (assignment, 32-output group) and (assignment, output)"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from __graft_entry__ import load_package
+    strix = load_package()
+    strix.require_gpu()
+    torch.cuda.set_device(0)
+
+    cfg = Config3(strix, torch, args.layers, args.tokens)
+    u_list = cfg.distinct_experts()
+    u_mean = sum(u_list) / len(u_list)
+
+    sec = time_steps(torch, cfg.step, args.steps, args.warmup)
+
+    # per-kernel durations: HIP events on the launch stream (torch's current stream), same rotation, same inputs
+    events = []
+    for i in range(args.warmup):
+        cfg.staged_step(i, [])
+    torch.cuda.synchronize()
+    for i in range(args.steps):
+        cfg.staged_step(args.warmup + i, events)
+    torch.cuda.synchronize()
+    names = ("route", "prologue", "csr", "project", "down", "merge")
+    kernel_us = {n: statistics.mean(m[k].elapsed_time(m[k + 1]) for m in events) * 1e3 for k, n in enumerate(names)}
+    proj_s = kernel_us["project"] * 1e-6
+    achieved = cfg.project_bytes(u_mean) / proj_s / 1e9
+    layer_gbps = cfg.layer_bytes(u_mean) / sec / 1e9
+
+    out = {
+        "metric": "moe_decode_us_per_layer", "value": sec * 1e6, "unit": "us/layer", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8", "data": "synthetic",
+        "config": {"workload": f"BASELINE config 3: MoE decode layer, Q4_K experts, hidden 2048, 128 experts, softmax router top-8, "
+                               f"intermediate 768, {args.tokens} fp16 tokens, router + experts + combine, {args.layers} rotating layers (cold cache)",
+                   "tokens": args.tokens, "distinct_experts_mean": u_mean},
+        "hbm_GBps_layer": layer_gbps, "hbm_frac_layer": layer_gbps / HBM_PEAK_GBPS,
+        "layer_algorithmic_bytes": cfg.layer_bytes(u_mean), "kernel_us": kernel_us,
+        "roofline": {"bound": "hbm", "kernel": "project_kernel (gate/up + SwiGLU + A8 re-quantise)", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes_per_launch": cfg.project_bytes(u_mean), "avg_launch_us": kernel_us["project"]},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_config3(cfg)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

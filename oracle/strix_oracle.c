@@ -120,7 +120,7 @@ void orc_quantize_q8_0_row(const float* x, size_t n, uint8_t* out) {
 }
 
 /* A plain min/max Q4_K writer (no reference counterpart; the GPU writer restates the same steps):
- * per 32: lo = min(min x, 0), hi = max(max x, lo); scale = (hi - lo) / 15, offset = -lo;
+ * per 32: lo = min(min x, 0), hi = max(max x, lo); scale = (hi - lo) / 15, offset = 0 - lo (never -0);
  * per 256: d = fp16(max scale / 63), dmin = fp16(max offset / 63); sc = min(63, rint(scale / d)),
  * m = min(63, rint(offset / dmin)); q = clamp(rint((x + dmin * m) / (d * sc)), 0, 15). */
 void orc_quantize_q4_k_row(const float* x, size_t n, uint8_t* out) {
@@ -132,7 +132,7 @@ void orc_quantize_q4_k_row(const float* x, size_t n, uint8_t* out) {
             float lo = 0.0F, hi = v[32 * j];
             for (int l = 0; l < 32; ++l) { lo = fminf(lo, v[32 * j + l]); hi = fmaxf(hi, v[32 * j + l]); }
             hi = fmaxf(hi, lo);
-            scale[j] = (hi - lo) / 15.0F; offset[j] = -lo;
+            scale[j] = (hi - lo) / 15.0F; offset[j] = 0.0F - lo;
             smax = fmaxf(smax, scale[j]); omax = fmaxf(omax, offset[j]);
         }
         const uint16_t dh = orc_float_to_half(smax / 63.0F), mh = orc_float_to_half(omax / 63.0F);

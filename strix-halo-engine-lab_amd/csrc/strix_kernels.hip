@@ -92,7 +92,7 @@ __global__ __launch_bounds__(64) void quantize_q4_k_rows_kernel(const float* x, 
             float lo = 0.0F, hi = v[32 * j];
             for (int l = 0; l < 32; ++l) { lo = __builtin_fminf(lo, v[32 * j + l]); hi = __builtin_fmaxf(hi, v[32 * j + l]); }
             hi = __builtin_fmaxf(hi, lo);
-            scale[j] = (hi - lo) / 15.0F; offset[j] = -lo;
+            scale[j] = (hi - lo) / 15.0F; offset[j] = 0.0F - lo;
             smax = __builtin_fmaxf(smax, scale[j]); omax = __builtin_fmaxf(omax, offset[j]);
         }
         const uint32_t dh = float_to_half_bits(smax / 63.0F), mh = float_to_half_bits(omax / 63.0F);
