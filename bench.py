@@ -58,8 +58,7 @@ class Config3:
 
     def step(self, i):
         layer, wr, x = self.layers[i % len(self.layers)]
-        ids, wts, _ = self.strix.route(x, wr, self.K)
-        layer.run(x, ids, wts)
+        layer.run_layer(x, wr)
 
     def staged_step(self, i, events):
         """Same work, one entry point per stage, with an event pair around each stage on the launch stream."""

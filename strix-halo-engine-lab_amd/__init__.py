@@ -78,7 +78,8 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_swiglu_quantize"]
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer",
+           "mi355_swiglu_quantize"]
 
 
 def require_gpu():
@@ -208,6 +209,20 @@ class MoeLayer:
         rows, rv = self.rows_view(x, ids, weights, base)
         check(lib().mi355_moe_enqueue(C.byref(self.w), C.byref(rv), rows, combine, _stream()))
         return self.output[:rows]
+
+    def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,
+                  scale=1.0, renormalize=True):
+        """Router + experts + combine through mi355_moe_enqueue_layer. Returns (output, ids, weights, scores)."""
+        rows = x.shape[0]
+        if not hasattr(self, "ids") or self.ids.shape[0] < rows:
+            self.ids = torch.zeros((self.max_rows, self.top_k), dtype=torch.int32, device=x.device)
+            self.route_w = torch.zeros((self.max_rows, self.top_k), dtype=torch.float32, device=x.device)
+            self.scores = torch.zeros((self.max_rows, self.experts), dtype=torch.float32, device=x.device)
+        _, rv = self.rows_view(x, self.ids, self.route_w, base)
+        p = RoutePolicy(self.experts, self.top_k, logits_order, renorm_eps, scale, int(renormalize))
+        check(lib().mi355_moe_enqueue_layer(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), C.byref(self.w), C.byref(rv), rows,
+                                            combine, _stream()))
+        return self.output[:rows], self.ids[:rows], self.route_w[:rows], self.scores[:rows]
 
     def stage(self, name, x, ids, weights, base=None, combine=COMBINE_FMA_SLOT):
         rows, rv = self.rows_view(x, ids, weights, base)

@@ -8,6 +8,11 @@
 
 namespace strix950 {
 
+// Plain 128-bit register values. (HIP's uint4 / float4 are structs whose whole-value copies lower to memcpy, which can
+// pin an array of them in scratch memory; these vector types always live in VGPRs.)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ float f_of(uint32_t b) { return __builtin_bit_cast(float, b); }
 __device__ __forceinline__ uint32_t b_of(float f) { return __builtin_bit_cast(uint32_t, f); }
 __device__ __forceinline__ bool finite_f(float x) { return (b_of(x) & 0x7f800000U) != 0x7f800000U; }
@@ -91,7 +96,8 @@ __device__ __forceinline__ float exp_of(uint32_t kind, float x) { return kind ==
 // lane ^ 1 and lane ^ 2 are DPP quad permutes (no LDS traffic); wider distances go through the swizzle crossbar.
 __device__ __forceinline__ int xor1_i(int v) { return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true); }
 __device__ __forceinline__ int xor2_i(int v) { return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true); }
-__device__ __forceinline__ int xor4_i(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x101F); }
+// lane ^ 4 inside a group of 8: mirror the 8 lanes (row_half_mirror), then reverse each quad - two DPP moves.
+__device__ __forceinline__ int xor4_i(int v) { return __builtin_amdgcn_mov_dpp(__builtin_amdgcn_mov_dpp(v, 0x141, 0xF, 0xF, true), 0x1B, 0xF, 0xF, true); }
 __device__ __forceinline__ int xor8_i(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x201F); }
 __device__ __forceinline__ int xor16_i(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401F); }
 __device__ __forceinline__ float xor1_f(float v) { return __builtin_bit_cast(float, xor1_i(__builtin_bit_cast(int, v))); }

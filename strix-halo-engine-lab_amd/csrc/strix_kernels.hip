@@ -6,10 +6,13 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 
 #include "device_math.hpp"
+#include "q4k_wave.hpp"
+#include "route_wave.hpp"
 
 namespace strix950 {
 
@@ -193,120 +196,131 @@ __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v, ui
 }
 
 // ======================================================================================================== router
-// One block per row. Logits: thread e runs expert e's chain over the row staged in LDS.
-// Reference: tests/hip_moe_route_launcher_tests.hip:281-330 (chain), include/strix/moe/route_policy.hpp:99-156.
-constexpr uint32_t kRouteMaxHidden = 8192, kRouteMaxExperts = 1024, kRouteMaxTopK = 16;
+// Plan words (uint32): [0] assignments A = rows * top_k, [1] touched experts U, [2] largest group, [3] launch ticket,
+// [16 ..] offsets[experts + 1]; touched[experts] (ids of the experts with work, ascending); order[A]: assignment indices
+// (row * top_k + slot) grouped by expert, ascending row then slot inside an expert; items[min(experts, A)] x 4 words
+// {expert, begin, end, 0} (one record per touched expert, zero records after the last); 256 ticket / scratch words.
+// Reference: src/hip_moe_q4k_a8_probe.hip:91-147 (stable CSR of (row, slot) by expert).
+__host__ __device__ inline uint32_t pad4(uint32_t v) { return (v + 3U) & ~3U; }
+__host__ __device__ inline uint32_t plan_touched_at(uint32_t experts) { return 16U + pad4(experts + 1U); }
+__host__ __device__ inline uint32_t plan_order_at(uint32_t experts) { return plan_touched_at(experts) + pad4(experts); }
+__host__ __device__ inline uint32_t plan_item_bound(uint32_t experts, uint32_t assignments) { return assignments < experts ? assignments : experts; }
+__host__ __device__ inline uint32_t plan_items_at(uint32_t experts, uint32_t assignments) { return plan_order_at(experts) + pad4(assignments); }
+__host__ __device__ inline uint32_t plan_tickets_at(uint32_t experts, uint32_t assignments) {
+    return plan_items_at(experts, assignments) + 4U * plan_item_bound(experts, assignments);
+}
+constexpr uint32_t kPlanTicketWords = 256;     // [0, 128): merge tickets, [128, 256): per-row A8 flags of the fused prologue
 
-__global__ __launch_bounds__(256) void route_kernel(mi355_route_policy p, const uint8_t* x, uint32_t kind, uint32_t hidden,
-                                                    uint64_t x_stride, const float* wr, const float* bias, uint32_t* ids,
-                                                    float* weights, float* scores) {
-    __shared__ float xs[kRouteMaxHidden];
-    __shared__ float sc[kRouteMaxExperts];
-    __shared__ float red_v[4];
-    __shared__ uint32_t red_i[4];
-    __shared__ float total;
-    __shared__ uint32_t picked[kRouteMaxTopK];
-    const uint32_t row = blockIdx.x, tid = threadIdx.x;
-    for (uint32_t i = tid; i < hidden; i += 256U) xs[i] = load_activation_kind(x + row * x_stride, i, kind);
+// Expert plan by one wave from the ids of a decode batch held in LDS (A <= 256 assignments).
+__device__ __forceinline__ void build_plan_wave(uint32_t* count, const uint32_t* ids, uint32_t experts, uint32_t assignments, uint32_t* plan) {
+    const uint32_t lane = threadIdx.x;
+    for (uint32_t e = lane; e <= experts; e += 64U) count[e] = 0;
     __syncthreads();
-    for (uint32_t e = tid; e < p.experts; e += 256U) {
-        const float* we = wr + static_cast<size_t>(e) * hidden;
-        float acc;
-        if (p.logits_order == MI355_LOGITS_LANE32_BUTTERFLY) {
-            float lanes[32];
-#pragma unroll
-            for (int l = 0; l < 32; ++l) lanes[l] = 0.0F;
-            for (uint32_t i = 0; i < hidden; i += 32U) {
-#pragma unroll
-                for (int l = 0; l < 32; ++l)
-                    if (i + l < hidden) lanes[l] = lanes[l] + we[i + l] * xs[i + l];
-            }
-#pragma unroll
-            for (int s = 16; s; s /= 2)
-#pragma unroll
-                for (int i = 0; i < s; ++i) lanes[i] = lanes[i] + lanes[i + s];
-            acc = lanes[0];
-        } else {
-            acc = 0.0F;
-            uint32_t i = 0;
-            for (; i + 4 <= hidden; i += 4) {
-                const float4 w4 = *reinterpret_cast<const float4*>(we + i);
-                acc = __builtin_fmaf(xs[i], w4.x, acc); acc = __builtin_fmaf(xs[i + 1], w4.y, acc);
-                acc = __builtin_fmaf(xs[i + 2], w4.z, acc); acc = __builtin_fmaf(xs[i + 3], w4.w, acc);
-            }
-            for (; i < hidden; ++i) acc = __builtin_fmaf(xs[i], we[i], acc);
-        }
-        sc[e] = bias ? acc + bias[e] : acc;
+    for (uint32_t a = lane; a < assignments; a += 64U) atomicAdd(&count[ids[a]], 1U);
+    __syncthreads();
+    const uint32_t chunk = (experts + 63U) / 64U, first = lane * chunk, last = first + chunk < experts ? first + chunk : experts;
+    uint32_t local = 0, local_touched = 0, largest = 0;
+    for (uint32_t e = first; e < last; ++e) {
+        const uint32_t c = count[e];
+        local += c; local_touched += c != 0; largest = c > largest ? c : largest;
     }
-    __syncthreads();
-    // softmax: m = max, p = exp(z - m), sum ascending from 0, s = p / sum
-    float m = -INFINITY;
-    for (uint32_t e = tid; e < p.experts; e += 256U) m = sc[e] > m ? sc[e] : m;
-    for (int d = 32; d; d >>= 1) { const float o = __shfl_xor(m, d); m = o > m ? o : m; }
-    if ((tid & 63U) == 0) red_v[tid >> 6] = m;
-    __syncthreads();
-    m = red_v[0];
-    for (int w = 1; w < 4; ++w) m = red_v[w] > m ? red_v[w] : m;
-    __syncthreads();
-    for (uint32_t e = tid; e < p.experts; e += 256U) sc[e] = declared_exp(sc[e] - m);
-    __syncthreads();
-    if (tid == 0) {
-        float sum = 0.0F;
-        for (uint32_t e = 0; e < p.experts; ++e) sum = sum + sc[e];
-        total = sum;
+    uint32_t run = local, trun = local_touched;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_up(run, d), t = __shfl_up(trun, d);
+        if (lane >= static_cast<uint32_t>(d)) { run += o; trun += t; }
     }
+    for (int d = 32; d; d >>= 1) { const uint32_t o = __shfl_xor(largest, d); largest = o > largest ? o : largest; }
+    const uint32_t touched_total = __shfl(trun, 63);
+    run -= local; trun -= local_touched;                    // exclusive prefixes
+    uint32_t* offsets = plan + 16;
+    uint32_t* touched = plan + plan_touched_at(experts);
+    uint32_t* order = plan + plan_order_at(experts);
+    uint32_t* items = plan + plan_items_at(experts, assignments);
     __syncthreads();
-    const float sum = total;
-    for (uint32_t e = tid; e < p.experts; e += 256U) {
-        const float s = sc[e] / sum;
-        sc[e] = s;
-        scores[static_cast<size_t>(row) * p.experts + e] = s;
+    for (uint32_t e = first; e < last; ++e) {
+        const uint32_t c = count[e];
+        offsets[e] = run;
+        count[e] = run;                                     // LDS now holds the exclusive offsets
+        if (c) {
+            touched[trun] = e;
+            items[4U * trun] = e; items[4U * trun + 1U] = run; items[4U * trun + 2U] = run + c; items[4U * trun + 3U] = 0;
+            ++trun;
+        }
+        run += c;
     }
+    const uint32_t bound = plan_item_bound(experts, assignments);
+    for (uint32_t u = touched_total + lane; u < bound; u += 64U) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
+    if (lane == 0) { offsets[experts] = assignments; plan[0] = assignments; plan[1] = touched_total; plan[2] = largest; }
     __syncthreads();
-    // k passes; a pass takes the greatest remaining score, the lower id on ties (ascending serial scan semantics)
-    for (uint32_t k = 0; k < p.top_k; ++k) {
-        float bv = -1.0F;
-        uint32_t bi = 0xffffffffU;
-        for (uint32_t e = tid; e < p.experts; e += 256U) {
-            bool taken = false;
-            for (uint32_t q = 0; q < k; ++q) taken |= picked[q] == e;
-            if (taken) continue;
-            const float c = sc[e];
-            if (bi == 0xffffffffU || c > bv) { bv = c; bi = e; }
-        }
-        for (int d = 32; d; d >>= 1) {
-            const float ov = __shfl_xor(bv, d);
-            const uint32_t oi = __shfl_xor(bi, d);
-            if (oi != 0xffffffffU && (bi == 0xffffffffU || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
-        }
-        if ((tid & 63U) == 0) { red_v[tid >> 6] = bv; red_i[tid >> 6] = bi; }
-        __syncthreads();
-        if (tid == 0) {
-            float v = red_v[0];
-            uint32_t i = red_i[0];
-            for (int w = 1; w < 4; ++w)
-                if (red_i[w] != 0xffffffffU && (i == 0xffffffffU || red_v[w] > v || (red_v[w] == v && red_i[w] < i))) { v = red_v[w]; i = red_i[w]; }
-            picked[k] = i;
-        }
-        __syncthreads();
-    }
-    if (tid == 0) {
-        float s = 0.0F;
-        for (uint32_t k = 0; k < p.top_k; ++k) s = s + sc[picked[k]];
-        const float den = s + p.renorm_eps;
-        for (uint32_t k = 0; k < p.top_k; ++k) {
-            const float v = sc[picked[k]];
-            ids[static_cast<size_t>(row) * p.top_k + k] = picked[k];
-            weights[static_cast<size_t>(row) * p.top_k + k] = (p.renormalize ? v / den : v) * p.scale;
-        }
+    // stable order: the rank of an assignment inside its expert = earlier assignments of the same expert
+    for (uint32_t a = lane; a < assignments; a += 64U) {
+        const uint32_t e = ids[a];
+        uint32_t rank = 0;
+        for (uint32_t b = 0; b < a; ++b) rank += ids[b] == e;
+        order[count[e] + rank] = a;
     }
 }
 
+// Router launch. Blocks [0, route_blocks) run the logit chains of 8 experts x 8 rows; in the fused decode form, blocks
+// [route_blocks, route_blocks + quant_blocks) quantise the input rows to A8 (8 groups of 32 per block), and the block
+// that takes the last launch ticket runs softmax / top-k / weights for every row, publishes the row status words and
+// builds the expert plan. In the plain form (a.plan == nullptr) the kernel stops after the logits.
+template <int KIND>
+__global__ __launch_bounds__(64) void route_logits_kernel(RouteArgs a) {
+    __shared__ RouteLds lds;
+    const uint32_t bid = blockIdx.x, lane = threadIdx.x;
+    if (bid < a.route_blocks) {
+        const uint32_t neb = (a.p.experts + 7U) / 8U;
+        route_logits_block<KIND>(lds, a, (bid % neb) * 8U, (bid / neb) * 8U);
+    } else {
+        // A8 prologue (src/cpu/core/reference.cpp:35-55): two groups of 32 at a time, 8 groups per block
+        const uint32_t groups = a.hidden / 32U, total = a.rows * groups, g0 = (bid - a.route_blocks) * 8U;
+        uint32_t* flags = a.plan + plan_tickets_at(a.p.experts, a.rows * a.p.top_k) + 128U;
+        for (uint32_t i = 0; i < 8U; i += 2U) {
+            const uint32_t g = g0 + i + (lane >> 5), j = lane & 31U;
+            if (g < total) {
+                const uint32_t r = g / groups, gi = g % groups;
+                const float v = load_activation<KIND>(a.x + r * a.x_stride, gi * 32U + j);
+                const float amax = max32(__builtin_fabsf(v));
+                const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+                const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+                const int code = a8_code(v, delta, tiny);
+                const int sum = sum32_i(code);
+                const int bad = or32_i(finite_f(v) ? 0 : 1);
+                a.codes[static_cast<size_t>(r) * a.hidden + gi * 32U + j] = static_cast<int8_t>(code);
+                if (j == 0) {
+                    a.deltas[static_cast<size_t>(r) * groups + gi] = delta;
+                    a.sums[static_cast<size_t>(r) * groups + gi] = sum;
+                    if (bad) atomicOr(&flags[r], static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
+                }
+            }
+        }
+    }
+    if (!a.plan) return;
+    __threadfence();
+    __syncthreads();
+    if (lane == 0) lds.is_last = atomicAdd(&a.plan[3], 1U) == gridDim.x - 1U;
+    __syncthreads();
+    if (!lds.is_last) return;
+    __threadfence();
+    for (uint32_t r0 = 0; r0 < a.rows; r0 += 8U)
+        route_select_rows(lds.sel.p, lds.picked, a, r0, a.rows - r0 < 8U ? a.rows - r0 : 8U, lds.ids + r0 * a.p.top_k);
+    uint32_t* flags = a.plan + plan_tickets_at(a.p.experts, a.rows * a.p.top_k) + 128U;
+    if (lane < a.rows) { a.status[lane] = flags[lane]; flags[lane] = 0; }
+    if (lane == 0) { *a.job_status = 0; a.plan[3] = 0; }
+    build_plan_wave(lds.plan.count, lds.ids, a.p.experts, a.rows * a.p.top_k, a.plan);
+}
+
+// softmax / top-k / weights for 8 rows per one-wave block (the plain router and batches above the fused bound).
+__global__ __launch_bounds__(64) void route_select_kernel(RouteArgs a) {
+    __shared__ RouteSelLds lds;
+    const uint32_t r0 = blockIdx.x * 8U;
+    route_select_rows(lds.p, lds.picked, a, r0, a.rows - r0 < 8U ? a.rows - r0 : 8U, nullptr);
+}
+
 // ======================================================================================================== expert plan
-// Plan words: [0] assignments A = rows * top_k, [1] touched experts, [2] largest group, [16 ..] offsets[experts + 1],
-// then order[A]: assignment indices (row * top_k + slot) grouped by expert, ascending row then slot inside an expert.
-// Reference: src/hip_moe_q4k_a8_probe.hip:91-147 (stable CSR of (row, slot) by expert).
-__host__ __device__ inline uint32_t plan_order_at(uint32_t experts) { return 16U + ((experts + 1U + 3U) & ~3U); }
+// (layout of the plan words: see the router section above)
 
 __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
     __shared__ uint32_t count[kRouteMaxExperts + 1];
@@ -320,13 +334,19 @@ __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint
     __syncthreads();
     if (tid == 0) {
         uint32_t run = 0, touched = 0, largest = 0;
+        uint32_t* touched_ids = plan + plan_touched_at(experts);
+        uint32_t* items = plan + plan_items_at(experts, assignments);
         for (uint32_t e = 0; e < experts; ++e) {
             const uint32_t c = count[e];
             count[e] = run;
+            if (c != 0) {
+                items[4U * touched] = e; items[4U * touched + 1U] = run; items[4U * touched + 2U] = run + c; items[4U * touched + 3U] = 0;
+                touched_ids[touched++] = e;
+            }
             run += c;
-            touched += c != 0;
             largest = c > largest ? c : largest;
         }
+        for (uint32_t u = touched; u < plan_item_bound(experts, assignments); ++u) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
         count[experts] = run;
         plan[0] = assignments; plan[1] = touched; plan[2] = largest;
     }
@@ -359,161 +379,66 @@ __global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* rout
 }
 
 // ======================================================================================================== Q4_K x A8 rows
-// 32 weight rows per 256-thread block, 8 lanes per row: lane s of a row owns 16-byte quant chunk s of every 144-byte
-// super-block (pair p = s / 2, half h = s & 1) and evaluates the group term of sub-block j = s:
-//   x_j = E_g * ((D_j * float(dot_j)) - (DM_j * float(S_g))),  D_j = d * sc_j, DM_j = dmin * m_j, g = 8 b + j
-//   acc_p += (x_2p + x_2p+1) over super-blocks b ascending;  value = (acc0 + acc1) + (acc2 + acc3)
-// dot_j is exact: each lane's two 16-element int8 dot products (v_dot4_i32_i8) are exchanged with lane ^ 1 by DPP.
-// Up to NB activation rows (assignments) share one sweep of the weights; their A8 images are staged in LDS.
-// Reference: src/cpu/core/routed_expert.cpp:73-108, src/moe_q4k_a8_contract.cpp:126-140, lane roles of
-// src/hip_moe_q4k_a8_probe.hip:202-249.
-constexpr int kNB = 8;              // assignments per sweep
-constexpr uint32_t kChunk = 2048;   // activation elements staged per LDS pass
-
-struct ActImage {                   // A8 image of assignment a: codes [K], deltas [K/32], sums [K/32]
-    const int8_t* codes;
-    const float* deltas;
-    const int32_t* sums;
-    uint32_t width;                 // K
-};
-
-struct RowsLds {
-    int8_t codes[kNB][kChunk];
-    float delta[kNB][kChunk / 32];
-    float sumf[kNB][kChunk / 32];
-};
-
-// src_index(a) gives the row of the A8 image read by assignment a of this sweep.
-template <class Index>
-__device__ __forceinline__ void stage_chunk(RowsLds& lds, const ActImage& img, Index src_index, uint32_t na, uint32_t k0, uint32_t kc) {
-    const uint32_t tid = threadIdx.x;
-    const uint32_t vec = kc / 16U;
-    for (uint32_t i = tid; i < na * vec; i += 256U) {
-        const uint32_t a = i / vec, c = i % vec;
-        const int4 v = *reinterpret_cast<const int4*>(img.codes + static_cast<size_t>(src_index(a)) * img.width + k0 + c * 16U);
-        *reinterpret_cast<int4*>(&lds.codes[a][c * 16U]) = v;
-    }
-    const uint32_t gc = kc / 32U, groups = img.width / 32U;
-    for (uint32_t i = tid; i < na * gc; i += 256U) {
-        const uint32_t a = i / gc, g = i % gc;
-        const size_t at = static_cast<size_t>(src_index(a)) * groups + k0 / 32U + g;
-        lds.delta[a][g] = img.deltas[at];
-        lds.sumf[a][g] = static_cast<float>(img.sums[at]);
-    }
-}
-
-// Sweeps `blocks` super-blocks of one weight row share (this lane: row of the block, chunk s) against na staged rows.
-// acc[a] accumulates pair p = s / 2 of assignment a.
-template <class Index>
-__device__ __forceinline__ void q4k_rows_sweep(RowsLds& lds, const uint8_t* wrow, uint32_t blocks, const ActImage& img,
-                                               Index src_index, uint32_t na, float (&acc)[kNB]) {
-    const uint32_t s = threadIdx.x & 7U, h = s & 1U, p = s >> 1;
-#pragma unroll
-    for (int a = 0; a < kNB; ++a) acc[a] = 0.0F;
-    for (uint32_t k0 = 0; k0 < blocks * 256U; k0 += kChunk) {
-        const uint32_t kc = blocks * 256U - k0 < kChunk ? blocks * 256U - k0 : kChunk;
-        __syncthreads();
-        stage_chunk(lds, img, src_index, na, k0, kc);
-        __syncthreads();
-        for (uint32_t b = 0; b < kc / 256U; ++b) {
-            const uint8_t* blk = wrow + static_cast<size_t>(k0 / 256U + b) * kQ4kBlock;
-            const uint4 hd = *reinterpret_cast<const uint4*>(blk);
-            const uint4 q = *reinterpret_cast<const uint4*>(blk + 16U + 16U * s);
-            // 6-bit factors of sub-block j = s from the three scale words (src/cpu/core/routed_expert.cpp:65-71)
-            const uint32_t shift = 8U * (s & 3U);
-            const uint32_t fa = (hd.y >> shift) & 255U, fb = (hd.z >> shift) & 255U, fc = (hd.w >> shift) & 255U;
-            const uint32_t scj = s < 4U ? (fa & 63U) : ((fc & 15U) | ((fa >> 6) << 4));
-            const uint32_t mnj = s < 4U ? (fb & 63U) : ((fc >> 4) | ((fb >> 6) << 4));
-            const float d = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
-            const float D = d * static_cast<float>(scj), DM = dm * static_cast<float>(mnj);
-            const int lo0 = static_cast<int>(q.x & 0x0f0f0f0fU), lo1 = static_cast<int>(q.y & 0x0f0f0f0fU);
-            const int lo2 = static_cast<int>(q.z & 0x0f0f0f0fU), lo3 = static_cast<int>(q.w & 0x0f0f0f0fU);
-            const int hi0 = static_cast<int>((q.x >> 4) & 0x0f0f0f0fU), hi1 = static_cast<int>((q.y >> 4) & 0x0f0f0f0fU);
-            const int hi2 = static_cast<int>((q.z >> 4) & 0x0f0f0f0fU), hi3 = static_cast<int>((q.w >> 4) & 0x0f0f0f0fU);
-            const uint32_t at = b * 256U + p * 64U + h * 16U;   // elements of sub-block 2p held by this lane; 2p+1 is +32
-            const uint32_t g = b * 8U + s;
-#pragma unroll
-            for (int a = 0; a < kNB; ++a) {
-                if (static_cast<uint32_t>(a) < na) {
-                    const int4 cl = *reinterpret_cast<const int4*>(&lds.codes[a][at]);
-                    const int4 ch = *reinterpret_cast<const int4*>(&lds.codes[a][at + 32U]);
-                    int dl = 0, dh = 0;
-                    dl = __builtin_amdgcn_sdot4(lo0, cl.x, dl, false); dl = __builtin_amdgcn_sdot4(lo1, cl.y, dl, false);
-                    dl = __builtin_amdgcn_sdot4(lo2, cl.z, dl, false); dl = __builtin_amdgcn_sdot4(lo3, cl.w, dl, false);
-                    dh = __builtin_amdgcn_sdot4(hi0, ch.x, dh, false); dh = __builtin_amdgcn_sdot4(hi1, ch.y, dh, false);
-                    dh = __builtin_amdgcn_sdot4(hi2, ch.z, dh, false); dh = __builtin_amdgcn_sdot4(hi3, ch.w, dh, false);
-                    const int recv = xor1_i(h ? dl : dh);
-                    const int dot = (h ? dh : dl) + recv;
-                    const float u = D * static_cast<float>(dot);
-                    const float v = DM * lds.sumf[a][g];
-                    const float t = u - v;
-                    const float x = lds.delta[a][g] * t;
-                    const float pair = x + xor1_f(x);
-                    acc[a] = acc[a] + pair;
-                }
-            }
-        }
-    }
-}
-
-__device__ __forceinline__ float q4k_row_tree(float v) {   // (acc0 + acc1) + (acc2 + acc3) over the row's 8 lanes
-    v = v + xor2_f(v);
-    v = v + xor4_f(v);
-    return v;
-}
-
-// gate + up + SwiGLU + A8 re-quantisation of one (expert, 32-output group).
+// gate + up + SwiGLU + A8 re-quantisation: one wavefront per (touched expert, 32-output group). The lane's four rows
+// are gate rows {rs, rs + 16} and up rows {rs, rs + 16} of the group, so silu(g) * u needs no exchange, and the
+// 32-value h group is reduced over the wave's 16 row slots.
 // Reference: src/cpu/core/routed_expert.cpp:403-427 (gate item), :147-170 (swiglu_quantize).
-__global__ __launch_bounds__(256) void project_kernel(mi355_moe_weights w, mi355_moe_rows r) {
-    __shared__ RowsLds lds;
-    __shared__ float val[2][kNB][32];
-    const uint32_t grp = blockIdx.x, e = blockIdx.y, tid = threadIdx.x;
-    const uint32_t* offsets = r.plan + 16;
-    const uint32_t* order = r.plan + plan_order_at(w.experts);
-    const uint32_t begin = offsets[e], end = offsets[e + 1];
+template <int NB>
+__global__ __launch_bounds__(64, 2) void project_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    __shared__ __attribute__((aligned(16))) uint8_t w0[kStageBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t w1[kStageBytes];
+    __shared__ ActLds<NB> lds;
+    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
+    const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
     if (begin == end) return;
-    const uint32_t rrow = tid >> 3, blocks = w.hidden / 256U, groups = w.ffn / 32U;
-    const ActImage img{r.codes, r.deltas, r.sums, w.hidden};
-    const size_t row_off = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U + rrow) * w.gate_row_stride;
-    for (uint32_t c0 = begin; c0 < end; c0 += kNB) {
-        const uint32_t na = end - c0 < static_cast<uint32_t>(kNB) ? end - c0 : static_cast<uint32_t>(kNB);
-        const auto src = [&](uint32_t a) { return order[c0 + a] / w.top_k; };   // input row of the assignment
-        for (int which = 0; which < 2; ++which) {
-            float acc[kNB];
-            q4k_rows_sweep(lds, (which ? w.up : w.gate) + row_off, blocks, img, src, na, acc);
+    const uint32_t* order = r.plan + plan_order_at(w.experts);
+    const uint32_t lane = threadIdx.x & 63U, rs = lane >> 2, p = lane & 3U;
+    const uint32_t groups = w.ffn / 32U, grp = blockIdx.x;
+    const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U) * w.gate_row_stride;
+    // stages: gate rows 0..15 and 16..31 of the group, then the same up rows
+    const uint8_t* const stage_base[4] = {w.gate + base, w.gate + base + 16U * w.gate_row_stride, w.up + base, w.up + base + 16U * w.gate_row_stride};
+    const A8Image img{r.codes, r.deltas, r.sums, w.hidden};
+    for (uint32_t c0 = begin; c0 < end; c0 += NB) {
+        const uint32_t na = end - c0 < static_cast<uint32_t>(NB) ? end - c0 : static_cast<uint32_t>(NB);
+        const auto src = [&](uint32_t a) { return order[c0 + a] / w.top_k; };
+        float acc[4][NB];
+        sweep_rows<NB>(w0, w1, lds, stage_base, static_cast<uint32_t>(w.gate_row_stride), w.hidden / 256U, img, src, na, acc);
+        {
 #pragma unroll
-            for (int a = 0; a < kNB; ++a) {
-                const float v = q4k_row_tree(acc[a]);
-                if ((tid & 7U) == 0 && static_cast<uint32_t>(a) < na) val[which][a][rrow] = v;
-            }
-        }
-        __syncthreads();
-        const uint32_t a = tid >> 5, l = tid & 31U;
-        if (a < na) {
-            const uint32_t sidx = order[c0 + a];
-            const float g = val[0][a][l], u = val[1][a][l];
-            const float ex = exp_of(w.exp_kind, -g);
-            const float hv = (g / (1.0F + ex)) * u;
-            const size_t at = static_cast<size_t>(sidx) * w.ffn + grp * 32U + l;
-            if (r.gate_out) r.gate_out[at] = g;
-            if (r.up_out) r.up_out[at] = u;
-            if (r.h_out) r.h_out[at] = hv;
-            const int bad = or32_i((finite_f(g) && finite_f(u) && finite_f(hv)) ? 0 : 1);
-            if (bad) {
-                if (l == 0) {
-                    atomicOr(&r.status[sidx / w.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
-                    atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
-                }
-            } else {
-                const float amax = max32(__builtin_fabsf(hv));
-                const bool tiny = amax > 0.0F && amax < 0x1p-119F;
-                const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
-                const int code = a8_code(hv, dl, tiny);
-                const int sum = sum32_i(code);
-                r.down_codes[at] = static_cast<int8_t>(code);
-                if (l == 0) {
-                    r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
-                    r.down_sums[static_cast<size_t>(sidx) * groups + grp] = sum;
+            for (int a = 0; a < NB; ++a) {
+                if (static_cast<uint32_t>(a) < na) {
+                    const uint32_t sidx = order[c0 + a];
+                    const float g0 = row_tree4(acc[0][a]), g1 = row_tree4(acc[1][a]);
+                    const float u0 = row_tree4(acc[2][a]), u1 = row_tree4(acc[3][a]);
+                    const float h0 = (g0 / (1.0F + exp_of(w.exp_kind, -g0))) * u0;
+                    const float h1 = (g1 / (1.0F + exp_of(w.exp_kind, -g1))) * u1;
+                    const size_t at = static_cast<size_t>(sidx) * w.ffn + grp * 32U + rs;
+                    if (p == 0) {
+                        if (r.gate_out) { r.gate_out[at] = g0; r.gate_out[at + 16] = g1; }
+                        if (r.up_out) { r.up_out[at] = u0; r.up_out[at + 16] = u1; }
+                        if (r.h_out) { r.h_out[at] = h0; r.h_out[at + 16] = h1; }
+                    }
+                    const bool ok = finite_f(g0) && finite_f(g1) && finite_f(u0) && finite_f(u1) && finite_f(h0) && finite_f(h1);
+                    if (or_over_slots(ok ? 0 : 1)) {
+                        if (lane == 0) {
+                            atomicOr(&r.status[sidx / w.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                            atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                        }
+                    } else {
+                        const float amax = max_over_slots(__builtin_fmaxf(__builtin_fabsf(h0), __builtin_fabsf(h1)));
+                        const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+                        const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+                        const int k0 = a8_code(h0, dl, tiny), k1 = a8_code(h1, dl, tiny);
+                        const int sum = sum_over_slots(k0 + k1);
+                        if (p == 0) {
+                            r.down_codes[at] = static_cast<int8_t>(k0);
+                            r.down_codes[at + 16] = static_cast<int8_t>(k1);
+                        }
+                        if (lane == 0) {
+                            r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
+                            r.down_sums[static_cast<size_t>(sidx) * groups + grp] = sum;
+                        }
+                    }
                 }
             }
         }
@@ -521,29 +446,42 @@ __global__ __launch_bounds__(256) void project_kernel(mi355_moe_weights w, mi355
     }
 }
 
-// down rows of one (expert, 32 hidden outputs): rawdots[assignment][o].
+// down rows: one wavefront per (touched expert, 64 hidden outputs); the lane's rows are o = 64 tile + rs + 16 i.
 // Reference: src/cpu/core/routed_expert.cpp:429-447 (down item), src/moe_a8_down_contract.cpp:146 (Q4_K down row).
-__global__ __launch_bounds__(256) void down_kernel(mi355_moe_weights w, mi355_moe_rows r) {
-    __shared__ RowsLds lds;
-    const uint32_t og = blockIdx.x, e = blockIdx.y, tid = threadIdx.x;
-    if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
-    const uint32_t* offsets = r.plan + 16;
-    const uint32_t* order = r.plan + plan_order_at(w.experts);
-    const uint32_t begin = offsets[e], end = offsets[e + 1];
+template <int NB>
+__global__ __launch_bounds__(64, 2) void down_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    __shared__ __attribute__((aligned(16))) uint8_t w0[kStageBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t w1[kStageBytes];
+    __shared__ ActLds<NB> lds;
+    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
+    const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
     if (begin == end) return;
-    const uint32_t rrow = tid >> 3, o = og * 32U + rrow;
-    const ActImage img{r.down_codes, r.down_deltas, r.down_sums, w.ffn};
-    const uint8_t* wrow = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o) * w.down_row_stride;
-    for (uint32_t c0 = begin; c0 < end; c0 += kNB) {
-        const uint32_t na = end - c0 < static_cast<uint32_t>(kNB) ? end - c0 : static_cast<uint32_t>(kNB);
+    if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
+    const uint32_t* order = r.plan + plan_order_at(w.experts);
+    const uint32_t lane = threadIdx.x & 63U, rs = lane >> 2, p = lane & 3U;
+    const uint32_t o = blockIdx.x * 64U + rs;
+    const uint8_t* r0 = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
+    const uint8_t* const stage_base[4] = {r0, r0 + 16U * w.down_row_stride, r0 + 32U * w.down_row_stride, r0 + 48U * w.down_row_stride};
+    const A8Image img{r.down_codes, r.down_deltas, r.down_sums, w.ffn};
+    for (uint32_t c0 = begin; c0 < end; c0 += NB) {
+        const uint32_t na = end - c0 < static_cast<uint32_t>(NB) ? end - c0 : static_cast<uint32_t>(NB);
         const auto src = [&](uint32_t a) { return order[c0 + a]; };
-        float acc[kNB];
-        q4k_rows_sweep(lds, wrow, w.ffn / 256U, img, src, na, acc);
+        float acc[4][NB];
+        sweep_rows<NB>(w0, w1, lds, stage_base, static_cast<uint32_t>(w.down_row_stride), w.ffn / 256U, img, src, na, acc);
+        {
 #pragma unroll
-        for (int a = 0; a < kNB; ++a) {
-            const float v = q4k_row_tree(acc[a]);
-            if ((tid & 7U) == 0 && static_cast<uint32_t>(a) < na) r.rawdots[static_cast<size_t>(order[c0 + a]) * w.hidden + o] = v;
+            for (int a = 0; a < NB; ++a) {
+                if (static_cast<uint32_t>(a) < na) {
+                    float* out = r.rawdots + static_cast<size_t>(order[c0 + a]) * w.hidden + o;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float v = row_tree4(acc[i][a]);
+                        if (p == 0) out[16 * i] = v;
+                    }
+                }
+            }
         }
+        __syncthreads();
     }
 }
 
@@ -605,6 +543,45 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate,
     }
 }
 
+// ======================================================================================================== dispatch
+// NB = activation rows sharing one sweep of an expert's weights (an expert with more assignments is swept again for the
+// rest). STRIX950_NB overrides the heuristic (tuning aid).
+inline int env_int(const char* name) {
+    const char* v = std::getenv(name);
+    return v && *v ? std::atoi(v) : 0;
+}
+inline int sweep_nb(const mi355_moe_weights& w, uint32_t rows) {
+    static const int env_nb = env_int("STRIX950_NB");
+    if (env_nb == 2 || env_nb == 4 || env_nb == 8) return env_nb;
+    if (w.experts == 1U) return rows > 4U ? 8 : rows > 2U ? 4 : 2;
+    return rows > 8U ? 4 : 2;
+}
+inline void debug_init() {
+    static bool done = false;
+    if (!done) { done = true; const uint32_t v = static_cast<uint32_t>(env_int("STRIX950_DEBUG")); if (v) (void)hipMemcpyToSymbol(HIP_SYMBOL(g_debug), &v, 4); }
+}
+inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+    debug_init();
+    const dim3 grid(w.ffn / 32U, umax);
+    switch (sweep_nb(w, rows)) {
+    case 2: project_wave_kernel<2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    case 4: project_wave_kernel<4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    default: project_wave_kernel<8><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    }
+}
+inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+    const dim3 grid(w.hidden / 64U, umax);
+    switch (sweep_nb(w, rows)) {
+    case 2: down_wave_kernel<2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    case 4: down_wave_kernel<4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    default: down_wave_kernel<8><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    }
+}
+inline uint32_t touched_bound(const mi355_moe_weights& w, uint32_t rows) {
+    const uint64_t a = static_cast<uint64_t>(rows) * w.top_k;
+    return static_cast<uint32_t>(a < w.experts ? a : w.experts);
+}
+
 // ======================================================================================================== admission
 int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv) {
     STRIX_REQUIRE(w && r, "moe: null weights or rows");
@@ -623,6 +600,7 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
     if (wv.down_expert_stride == 0) wv.down_expert_stride = wv.down_row_stride * w->hidden;
     STRIX_REQUIRE(wv.gate_row_stride % 16U == 0 && wv.gate_expert_stride % 16U == 0 && wv.down_row_stride % 16U == 0 &&
                   wv.down_expert_stride % 16U == 0, "moe: weight strides must be multiples of 16 bytes");
+    STRIX_REQUIRE(wv.gate_row_stride < (1ULL << 27) && wv.down_row_stride < (1ULL << 27), "moe: weight row stride must be below 128 MiB");
     STRIX_REQUIRE(wv.gate_row_stride >= static_cast<uint64_t>(w->hidden / 256U) * kQ4kBlock &&
                   wv.down_row_stride >= static_cast<uint64_t>(w->ffn / 256U) * kQ4kBlock, "moe: weight row stride shorter than the row");
     STRIX_REQUIRE(w->gate && w->up && w->down && aligned(w->gate, 16) && aligned(w->up, 16) && aligned(w->down, 16),
@@ -724,22 +702,40 @@ int32_t mi355_gemv_q8_0_a8(const mi355_q8a8_view* v, mi355_stream stream) {
     return MI355_OK;
 }
 
-int32_t mi355_moe_route(const mi355_route_policy* p, const void* x, uint32_t kind, uint32_t rows, uint32_t hidden, uint64_t x_stride,
-                        const float* wr, const float* bias, uint32_t* ids, float* weights, float* scores, mi355_stream stream) {
+namespace {
+int32_t check_route(const mi355_route_policy* p, const void* x, uint32_t kind, uint32_t hidden, uint64_t x_stride, const float* wr,
+                    const uint32_t* ids, const float* weights, const float* scores) {
     STRIX_REQUIRE(p && x && wr && ids && weights && scores, "route: null pointer");
     STRIX_REQUIRE(p->experts > 0 && p->experts <= kRouteMaxExperts && p->top_k > 0 && p->top_k <= kRouteMaxTopK && p->top_k <= p->experts,
                   "route policy: need 0 < top_k <= experts, experts <= 1024, top_k <= 16");
-    STRIX_REQUIRE(hidden > 0 && hidden <= kRouteMaxHidden && hidden % 4U == 0, "route: hidden must be a multiple of 4 within 8192");
+    STRIX_REQUIRE(hidden > 0 && hidden <= kRouteMaxHidden && hidden % 32U == 0, "route: hidden must be a multiple of 32 within 16384");
     STRIX_REQUIRE(kind <= MI355_INPUT_BF16 && p->logits_order <= MI355_LOGITS_LANE32_BUTTERFLY, "route: unknown input kind or logits order");
-    STRIX_REQUIRE(aligned(wr, 16), "route: router weight must be 16-byte aligned");
+    STRIX_REQUIRE(aligned(wr, 16) && aligned(x, 16) && x_stride % 16U == 0, "route: router weight, activations and their row stride must be 16-byte aligned");
+    return MI355_OK;
+}
+void launch_route_logits(const RouteArgs& a, uint32_t blocks, hipStream_t st) {
+    if (a.kind == MI355_INPUT_F32) route_logits_kernel<0><<<blocks, 64, 0, st>>>(a);
+    else if (a.kind == MI355_INPUT_F16) route_logits_kernel<1><<<blocks, 64, 0, st>>>(a);
+    else route_logits_kernel<2><<<blocks, 64, 0, st>>>(a);
+}
+}  // namespace
+
+int32_t mi355_moe_route(const mi355_route_policy* p, const void* x, uint32_t kind, uint32_t rows, uint32_t hidden, uint64_t x_stride,
+                        const float* wr, const float* bias, uint32_t* ids, float* weights, float* scores, mi355_stream stream) {
+    if (const int32_t rc = check_route(p, x, kind, hidden, x_stride, wr, ids, weights, scores)) return rc;
     if (rows == 0) return MI355_OK;
-    route_kernel<<<rows, 256, 0, hs(stream)>>>(*p, static_cast<const uint8_t*>(x), kind, hidden, x_stride, wr, bias, ids, weights, scores);
+    RouteArgs a{};
+    a.p = *p; a.x = static_cast<const uint8_t*>(x); a.kind = kind; a.x_stride = x_stride; a.rows = rows; a.hidden = hidden;
+    a.wr = wr; a.bias = bias; a.ids = ids; a.weights = weights; a.scores = scores;
+    a.route_blocks = ((p->experts + 7U) / 8U) * ((rows + 7U) / 8U);
+    launch_route_logits(a, a.route_blocks, hs(stream));
+    route_select_kernel<<<(rows + 7U) / 8U, 64, 0, hs(stream)>>>(a);
     STRIX_LAUNCHED("moe_route");
     return MI355_OK;
 }
 
 size_t mi355_moe_plan_words(uint32_t experts, uint32_t rows, uint32_t top_k) {
-    return plan_order_at(experts) + ((static_cast<size_t>(rows) * top_k + 3U) & ~static_cast<size_t>(3));
+    return plan_tickets_at(experts, rows * top_k) + kPlanTicketWords;
 }
 
 int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
@@ -762,7 +758,7 @@ int32_t mi355_moe_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows* 
 int32_t mi355_moe_enqueue_project(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    project_kernel<<<dim3(wv.ffn / 32U, wv.experts), 256, 0, hs(stream)>>>(wv, *r);
+    launch_project(wv, *r, rows, touched_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe project");
     return MI355_OK;
 }
@@ -770,7 +766,7 @@ int32_t mi355_moe_enqueue_project(const mi355_moe_weights* w, const mi355_moe_ro
 int32_t mi355_moe_enqueue_down(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    down_kernel<<<dim3(wv.hidden / 32U, wv.experts), 256, 0, hs(stream)>>>(wv, *r);
+    launch_down(wv, *r, rows, touched_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe down");
     return MI355_OK;
 }
@@ -794,6 +790,34 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, u
     if (const int32_t rc = mi355_moe_enqueue_csr(w, r, rows, stream)) return rc;
     if (const int32_t rc = mi355_moe_enqueue_project(w, r, rows, stream)) return rc;
     if (const int32_t rc = mi355_moe_enqueue_down(w, r, rows, stream)) return rc;
+    return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+}
+
+int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
+                                const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
+    STRIX_REQUIRE(r->input && r->input_kind <= MI355_INPUT_BF16, "moe: input view invalid");
+    uint32_t* ids = const_cast<uint32_t*>(r->routes);
+    float* weights = const_cast<float*>(r->route_weights);
+    if (const int32_t rc = check_route(p, r->input, r->input_kind, wv.hidden, r->input_stride, router_weight, ids, weights, scores)) return rc;
+    STRIX_REQUIRE(p->experts == wv.experts && p->top_k == wv.top_k, "moe layer: router policy and expert tensors disagree on experts / top_k");
+    if (rows > kFusedMaxRows) {      // large batches: router, then the staged prologue / plan
+        if (const int32_t rc = mi355_moe_route(p, r->input, r->input_kind, rows, wv.hidden, r->input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
+        return mi355_moe_enqueue(w, r, rows, form, stream);
+    }
+    RouteArgs a{};
+    a.p = *p; a.x = static_cast<const uint8_t*>(r->input); a.kind = r->input_kind; a.x_stride = r->input_stride; a.rows = rows; a.hidden = wv.hidden;
+    a.wr = router_weight; a.bias = logit_bias; a.ids = ids; a.weights = weights; a.scores = scores;
+    a.codes = r->codes; a.deltas = r->deltas; a.sums = r->sums; a.status = r->status; a.job_status = r->job_status; a.plan = r->plan;
+    a.route_blocks = ((p->experts + 7U) / 8U) * ((rows + 7U) / 8U);
+    a.quant_blocks = (rows * (wv.hidden / 32U) + 7U) / 8U;
+    launch_route_logits(a, a.route_blocks + a.quant_blocks, hs(stream));
+    STRIX_LAUNCHED("moe layer router");
+    launch_project(wv, *r, rows, touched_bound(wv, rows), hs(stream));
+    launch_down(wv, *r, rows, touched_bound(wv, rows), hs(stream));
+    STRIX_LAUNCHED("moe layer experts");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
 

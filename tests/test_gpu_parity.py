@@ -295,6 +295,35 @@ def test_config3_moe_decode_layer_shape(strix):
         check_layer_stages(strix, layer, y, ref, want, (c, d, s), ids_ref, w_ref, (gate, up, down, I, {}), H, K, T, 0, 0, TOL_F16)
 
 
+@pytest.mark.parametrize("E,H,I,K,T,order", [(128, 2048, 768, 8, 8, 0), (128, 2048, 768, 8, 1, 0), (160, 1536, 512, 8, 16, 0), (20, 512, 256, 3, 5, 1),
+                                             (64, 1024, 256, 16, 16, 0)])
+def test_whole_layer_entry_router_prologue_plan_in_one_launch(strix, E, H, I, K, T, order):
+    """mi355_moe_enqueue_layer: ids / weights / scores, the A8 image, the plan-driven experts and the combine must equal
+    the staged entry points bit for bit, twice in a row on the same workspace (the launch tickets return to zero)."""
+    rng = np.random.default_rng(E + T)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), 16)
+    staged = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, 16)
+    wrd = dev(wr)
+    for trial in range(2):
+        x = rng.standard_normal((T, H)).astype(np.float16)
+        xd = dev(x)
+        y, ids, wts, scores = layer.run_layer(xd, wrd, logits_order=order)
+        ids_ref, w_ref, s_ref, _ = orc.route(x.astype(np.float32), wr, K, logits_order=order)
+        assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref)
+        assert np.array_equal(bits(wts.cpu().numpy()), bits(w_ref)) and np.array_equal(bits(scores.cpu().numpy()), bits(s_ref))
+        c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+        assert np.array_equal(layer.codes[:T].cpu().numpy(), c) and np.array_equal(bits(layer.deltas[:T].cpu().numpy()), bits(d))
+        ids2, wts2, _ = strix.route(xd, wrd, K, logits_order=order)
+        assert torch.equal(ids2, ids) and torch.equal(wts2, wts)
+        y2 = staged.run(xd, ids2, wts2)
+        assert torch.equal(y, y2) and torch.equal(layer.rawdots[:T], staged.rawdots[:T])
+        assert np.all(layer.status[:T].cpu().numpy() == 0)
+        n_plan = int(strix.lib().mi355_moe_plan_words(E, 16, K))
+        assert int(layer.plan[3]) == 0 and bool((layer.plan[n_plan - 256:] == 0).all())
+
+
 def test_config5_tp_rank_partial_sums(strix):
     """BASELINE config 5 structure at reduced size: rank 0 of TP = 2 holds the first half of every expert's intermediate
     rows and the matching K blocks of every down row, read in place through strides; the kernel emits the rank's partial
