@@ -11,7 +11,7 @@
 #include <string>
 
 #include "device_math.hpp"
-#include "q4k_wave.hpp"
+#include "q4k_rows.hpp"
 #include "route_wave.hpp"
 
 namespace strix950 {
@@ -379,109 +379,149 @@ __global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* rout
 }
 
 // ======================================================================================================== Q4_K x A8 rows
-// gate + up + SwiGLU + A8 re-quantisation: one wavefront per (touched expert, 32-output group). The lane's four rows
-// are gate rows {rs, rs + 16} and up rows {rs, rs + 16} of the group, so silu(g) * u needs no exchange, and the
-// 32-value h group is reduced over the wave's 16 row slots.
+// gate + up + SwiGLU + A8 re-quantisation: one wavefront per (touched expert, 32-output group). Lanes 0..31 hold the
+// gate rows of the group, lanes 32..63 the up rows; one cross-half exchange pairs them, then both halves evaluate the
+// same 32-value h group.
 // Reference: src/cpu/core/routed_expert.cpp:403-427 (gate item), :147-170 (swiglu_quantize).
-template <int NB>
-__global__ __launch_bounds__(64, 2) void project_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
-    __shared__ __attribute__((aligned(16))) uint8_t w0[kStageBytes];
-    __shared__ __attribute__((aligned(16))) uint8_t w1[kStageBytes];
-    __shared__ ActLds<NB> lds;
+template <int NA, int DEPTH>
+__device__ __forceinline__ void project_chunk(uint8_t* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
+                                              const mi355_moe_rows& r, uint32_t grp, const uint32_t* order, uint32_t c0) {
+    const uint32_t lane = threadIdx.x & 63U, o = lane & 31U, groups = w.ffn / 32U;
+    uint32_t sidx[NA], src[NA];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+        sidx[a] = __builtin_amdgcn_readfirstlane(order[c0 + a]);
+        src[a] = sidx[a] / w.top_k;
+    }
+    const ActRows<NA> act(A8Image{r.codes, r.deltas, r.sums, w.hidden}, src);
+    float value[NA];
+    sweep_rows<NA, DEPTH>(slots, source, w.hidden / 256U, act, value);
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+        const float other = __shfl_xor(value[a], 32);
+        const float g = lane < 32U ? value[a] : other, u = lane < 32U ? other : value[a];
+        const float h = (g / (1.0F + exp_of(w.exp_kind, -g))) * u;
+        const size_t at = static_cast<size_t>(sidx[a]) * w.ffn + grp * 32U + o;
+        if (lane < 32U) {
+            if (r.gate_out) r.gate_out[at] = g;
+            if (r.up_out) r.up_out[at] = u;
+            if (r.h_out) r.h_out[at] = h;
+        }
+        if (or32_i((finite_f(g) && finite_f(u) && finite_f(h)) ? 0 : 1)) {
+            if (lane == 0) {
+                atomicOr(&r.status[sidx[a] / w.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            }
+        } else {
+            const float amax = max32(__builtin_fabsf(h));
+            const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+            const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+            const int code = a8_code(h, dl, tiny);
+            const int sum = sum32_i(code);
+            if (lane < 32U) r.down_codes[at] = static_cast<int8_t>(code);
+            if (lane == 0) {
+                r.down_deltas[static_cast<size_t>(sidx[a]) * groups + grp] = dl;
+                r.down_sums[static_cast<size_t>(sidx[a]) * groups + grp] = sum;
+            }
+        }
+    }
+}
+
+#define STRIX_RING_SLOTS(DEPTH)                                                                  \
+    __shared__ __attribute__((aligned(16))) uint8_t ring0[kStageBytes];                          \
+    __shared__ __attribute__((aligned(16))) uint8_t ring1[kStageBytes];                          \
+    __shared__ __attribute__((aligned(16))) uint8_t ring2[DEPTH > 2 ? kStageBytes : 16];         \
+    __shared__ __attribute__((aligned(16))) uint8_t ring3[DEPTH > 2 ? kStageBytes : 16];         \
+    uint8_t* const ring[4] = {ring0, ring1, ring2, ring3};                                       \
+    uint8_t* slots[DEPTH];                                                                       \
+    _Pragma("unroll") for (int i = 0; i < DEPTH; ++i) slots[i] = ring[i];
+
+// NBMAX = most activation rows sharing one sweep of the weights (4 for routed experts, 8 for a dense matrix).
+template <int NBMAX, int DEPTH>
+__global__ __launch_bounds__(64, DEPTH > 2 ? 1 : 2) void project_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    STRIX_RING_SLOTS(DEPTH)
     const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
     const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
     if (begin == end) return;
     const uint32_t* order = r.plan + plan_order_at(w.experts);
-    const uint32_t lane = threadIdx.x & 63U, rs = lane >> 2, p = lane & 3U;
-    const uint32_t groups = w.ffn / 32U, grp = blockIdx.x;
+    const uint32_t grp = blockIdx.x;
     const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U) * w.gate_row_stride;
-    // stages: gate rows 0..15 and 16..31 of the group, then the same up rows
-    const uint8_t* const stage_base[4] = {w.gate + base, w.gate + base + 16U * w.gate_row_stride, w.up + base, w.up + base + 16U * w.gate_row_stride};
-    const A8Image img{r.codes, r.deltas, r.sums, w.hidden};
-    for (uint32_t c0 = begin; c0 < end; c0 += NB) {
-        const uint32_t na = end - c0 < static_cast<uint32_t>(NB) ? end - c0 : static_cast<uint32_t>(NB);
-        const auto src = [&](uint32_t a) { return order[c0 + a] / w.top_k; };
-        float acc[4][NB];
-        sweep_rows<NB>(w0, w1, lds, stage_base, static_cast<uint32_t>(w.gate_row_stride), w.hidden / 256U, img, src, na, acc);
-        {
-#pragma unroll
-            for (int a = 0; a < NB; ++a) {
-                if (static_cast<uint32_t>(a) < na) {
-                    const uint32_t sidx = order[c0 + a];
-                    const float g0 = row_tree4(acc[0][a]), g1 = row_tree4(acc[1][a]);
-                    const float u0 = row_tree4(acc[2][a]), u1 = row_tree4(acc[3][a]);
-                    const float h0 = (g0 / (1.0F + exp_of(w.exp_kind, -g0))) * u0;
-                    const float h1 = (g1 / (1.0F + exp_of(w.exp_kind, -g1))) * u1;
-                    const size_t at = static_cast<size_t>(sidx) * w.ffn + grp * 32U + rs;
-                    if (p == 0) {
-                        if (r.gate_out) { r.gate_out[at] = g0; r.gate_out[at + 16] = g1; }
-                        if (r.up_out) { r.up_out[at] = u0; r.up_out[at + 16] = u1; }
-                        if (r.h_out) { r.h_out[at] = h0; r.h_out[at + 16] = h1; }
-                    }
-                    const bool ok = finite_f(g0) && finite_f(g1) && finite_f(u0) && finite_f(u1) && finite_f(h0) && finite_f(h1);
-                    if (or_over_slots(ok ? 0 : 1)) {
-                        if (lane == 0) {
-                            atomicOr(&r.status[sidx / w.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
-                            atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
-                        }
-                    } else {
-                        const float amax = max_over_slots(__builtin_fmaxf(__builtin_fabsf(h0), __builtin_fabsf(h1)));
-                        const bool tiny = amax > 0.0F && amax < 0x1p-119F;
-                        const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
-                        const int k0 = a8_code(h0, dl, tiny), k1 = a8_code(h1, dl, tiny);
-                        const int sum = sum_over_slots(k0 + k1);
-                        if (p == 0) {
-                            r.down_codes[at] = static_cast<int8_t>(k0);
-                            r.down_codes[at + 16] = static_cast<int8_t>(k1);
-                        }
-                        if (lane == 0) {
-                            r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
-                            r.down_sums[static_cast<size_t>(sidx) * groups + grp] = sum;
-                        }
-                    }
+    const uint8_t* gate = w.gate + base;
+    const uint8_t* up = w.up + base;
+    const uint32_t stride = static_cast<uint32_t>(w.gate_row_stride);
+    StageSource source;
+    source.init([&](uint32_t row) { return row < 32U ? gate + row * stride : up + (row - 32U) * stride; });
+    uint8_t* const (&sl)[DEPTH] = slots;
+    for (uint32_t c0 = begin; c0 < end;) {
+        const uint32_t left = end - c0, na = left < static_cast<uint32_t>(NBMAX) ? left : static_cast<uint32_t>(NBMAX);
+        switch (na) {
+        case 1: project_chunk<1, DEPTH>(sl, source, w, r, grp, order, c0); break;
+        case 2: project_chunk<2, DEPTH>(sl, source, w, r, grp, order, c0); break;
+        case 3: project_chunk<3, DEPTH>(sl, source, w, r, grp, order, c0); break;
+        case 4: project_chunk<4, DEPTH>(sl, source, w, r, grp, order, c0); break;
+        default:
+            if constexpr (NBMAX == 8) {
+                switch (na) {
+                case 5: project_chunk<5, DEPTH>(sl, source, w, r, grp, order, c0); break;
+                case 6: project_chunk<6, DEPTH>(sl, source, w, r, grp, order, c0); break;
+                case 7: project_chunk<7, DEPTH>(sl, source, w, r, grp, order, c0); break;
+                default: project_chunk<8, DEPTH>(sl, source, w, r, grp, order, c0); break;
                 }
             }
+            break;
         }
-        __syncthreads();
+        c0 += na;
     }
 }
 
-// down rows: one wavefront per (touched expert, 64 hidden outputs); the lane's rows are o = 64 tile + rs + 16 i.
+// down rows: one wavefront per (touched expert, 64 hidden outputs), lane = output row.
 // Reference: src/cpu/core/routed_expert.cpp:429-447 (down item), src/moe_a8_down_contract.cpp:146 (Q4_K down row).
-template <int NB>
-__global__ __launch_bounds__(64, 2) void down_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
-    __shared__ __attribute__((aligned(16))) uint8_t w0[kStageBytes];
-    __shared__ __attribute__((aligned(16))) uint8_t w1[kStageBytes];
-    __shared__ ActLds<NB> lds;
+template <int NA, int DEPTH>
+__device__ __forceinline__ void down_chunk(uint8_t* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
+                                           const mi355_moe_rows& r, const uint32_t* order, uint32_t c0) {
+    uint32_t src[NA];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) src[a] = __builtin_amdgcn_readfirstlane(order[c0 + a]);
+    const ActRows<NA> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src);
+    float value[NA];
+    sweep_rows<NA, DEPTH>(slots, source, w.ffn / 256U, act, value);
+    const uint32_t o = blockIdx.x * 64U + (threadIdx.x & 63U);
+#pragma unroll
+    for (int a = 0; a < NA; ++a) r.rawdots[static_cast<size_t>(src[a]) * w.hidden + o] = value[a];
+}
+
+template <int NBMAX, int DEPTH>
+__global__ __launch_bounds__(64, DEPTH > 2 ? 1 : 2) void down_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    STRIX_RING_SLOTS(DEPTH)
     const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
     const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
     if (begin == end) return;
     if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
     const uint32_t* order = r.plan + plan_order_at(w.experts);
-    const uint32_t lane = threadIdx.x & 63U, rs = lane >> 2, p = lane & 3U;
-    const uint32_t o = blockIdx.x * 64U + rs;
-    const uint8_t* r0 = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
-    const uint8_t* const stage_base[4] = {r0, r0 + 16U * w.down_row_stride, r0 + 32U * w.down_row_stride, r0 + 48U * w.down_row_stride};
-    const A8Image img{r.down_codes, r.down_deltas, r.down_sums, w.ffn};
-    for (uint32_t c0 = begin; c0 < end; c0 += NB) {
-        const uint32_t na = end - c0 < static_cast<uint32_t>(NB) ? end - c0 : static_cast<uint32_t>(NB);
-        const auto src = [&](uint32_t a) { return order[c0 + a]; };
-        float acc[4][NB];
-        sweep_rows<NB>(w0, w1, lds, stage_base, static_cast<uint32_t>(w.down_row_stride), w.ffn / 256U, img, src, na, acc);
-        {
-#pragma unroll
-            for (int a = 0; a < NB; ++a) {
-                if (static_cast<uint32_t>(a) < na) {
-                    float* out = r.rawdots + static_cast<size_t>(order[c0 + a]) * w.hidden + o;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float v = row_tree4(acc[i][a]);
-                        if (p == 0) out[16 * i] = v;
-                    }
+    const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
+    const uint32_t stride = static_cast<uint32_t>(w.down_row_stride);
+    StageSource source;
+    source.init([&](uint32_t row) { return rows + row * stride; });
+    uint8_t* const (&sl)[DEPTH] = slots;
+    for (uint32_t c0 = begin; c0 < end;) {
+        const uint32_t left = end - c0, na = left < static_cast<uint32_t>(NBMAX) ? left : static_cast<uint32_t>(NBMAX);
+        switch (na) {
+        case 1: down_chunk<1, DEPTH>(sl, source, w, r, order, c0); break;
+        case 2: down_chunk<2, DEPTH>(sl, source, w, r, order, c0); break;
+        case 3: down_chunk<3, DEPTH>(sl, source, w, r, order, c0); break;
+        case 4: down_chunk<4, DEPTH>(sl, source, w, r, order, c0); break;
+        default:
+            if constexpr (NBMAX == 8) {
+                switch (na) {
+                case 5: down_chunk<5, DEPTH>(sl, source, w, r, order, c0); break;
+                case 6: down_chunk<6, DEPTH>(sl, source, w, r, order, c0); break;
+                case 7: down_chunk<7, DEPTH>(sl, source, w, r, order, c0); break;
+                default: down_chunk<8, DEPTH>(sl, source, w, r, order, c0); break;
                 }
             }
+            break;
         }
-        __syncthreads();
+        c0 += na;
     }
 }
 
@@ -544,37 +584,38 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate,
 }
 
 // ======================================================================================================== dispatch
-// NB = activation rows sharing one sweep of an expert's weights (an expert with more assignments is swept again for the
-// rest). STRIX950_NB overrides the heuristic (tuning aid).
+// Up to 4 (routed experts) or 8 (dense matrix) activation rows share one sweep of an expert's weights; an expert with
+// more assignments is swept again for the rest. The copy ring is 4 stages deep when the launch has too few wavefronts
+// to cover the HBM latency with 2 (few touched experts, or a dense matrix), else 2 to leave LDS for more wavefronts.
 inline int env_int(const char* name) {
     const char* v = std::getenv(name);
     return v && *v ? std::atoi(v) : 0;
 }
-inline int sweep_nb(const mi355_moe_weights& w, uint32_t rows) {
-    static const int env_nb = env_int("STRIX950_NB");
-    if (env_nb == 2 || env_nb == 4 || env_nb == 8) return env_nb;
-    if (w.experts == 1U) return rows > 4U ? 8 : rows > 2U ? 4 : 2;
-    return rows > 8U ? 4 : 2;
-}
-inline void debug_init() {
-    static bool done = false;
-    if (!done) { done = true; const uint32_t v = static_cast<uint32_t>(env_int("STRIX950_DEBUG")); if (v) (void)hipMemcpyToSymbol(HIP_SYMBOL(g_debug), &v, 4); }
+inline bool deep_ring(uint64_t waves) {
+    static const int env_depth = env_int("STRIX950_DEPTH");   // tuning aid: 2 or 4 overrides the heuristic
+    if (env_depth == 2 || env_depth == 4) return env_depth == 4;
+    return waves < 256U * 5U;
 }
 inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
-    debug_init();
     const dim3 grid(w.ffn / 32U, umax);
-    switch (sweep_nb(w, rows)) {
-    case 2: project_wave_kernel<2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
-    case 4: project_wave_kernel<4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
-    default: project_wave_kernel<8><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    const bool deep = deep_ring(static_cast<uint64_t>(grid.x) * grid.y);
+    if (w.experts == 1U && rows > 4U) {
+        if (deep) project_wave_kernel<8, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
+        else project_wave_kernel<8, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
+    } else {
+        if (deep) project_wave_kernel<4, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
+        else project_wave_kernel<4, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
     }
 }
 inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     const dim3 grid(w.hidden / 64U, umax);
-    switch (sweep_nb(w, rows)) {
-    case 2: down_wave_kernel<2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
-    case 4: down_wave_kernel<4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
-    default: down_wave_kernel<8><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    const bool deep = deep_ring(static_cast<uint64_t>(grid.x) * grid.y);
+    if (w.experts == 1U && rows > 4U) {
+        if (deep) down_wave_kernel<8, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
+        else down_wave_kernel<8, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
+    } else {
+        if (deep) down_wave_kernel<4, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
+        else down_wave_kernel<4, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
     }
 }
 inline uint32_t touched_bound(const mi355_moe_weights& w, uint32_t rows) {
