@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0     # MI355X published HBM3E peak
+# HBM bytes per launch of the gate/up kernel on the default workload, from two rocprofv3 --pmc passes (FETCH_SIZE scaled
+# x2.000, WRITE_SIZE x1.000 by a 256 MiB device copy in the same runs): profiles/project_wave_kernel_config3_moe_decode_T8.txt
+PROJECT_TRAFFIC_BYTES_DEFAULT = 98_739_405 + 147_968
 Q4K_ROW = lambda k: k // 256 * 144
 
 
@@ -35,7 +38,8 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8)
     ap.add_argument("--layers", type=int, default=6, help="independent layers rotated through (cold-cache working set)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--extra", action="store_true", help="also time BASELINE configs 1, 2 and 5 (reported under 'extra')")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy 4 times (a kernel of known HBM traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -142,6 +146,13 @@ def main():
     u_list = cfg.distinct_experts()
     u_mean = sum(u_list) / len(u_list)
 
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
     sec = time_steps(torch, cfg.step, args.steps, args.warmup)
 
     # per-kernel durations: HIP events on the launch stream (torch's current stream), same rotation, same inputs
@@ -167,8 +178,9 @@ def main():
                    "tokens": args.tokens, "distinct_experts_mean": u_mean},
         "hbm_GBps_layer": layer_gbps, "hbm_frac_layer": layer_gbps / HBM_PEAK_GBPS,
         "layer_algorithmic_bytes": cfg.layer_bytes(u_mean), "kernel_us": kernel_us,
-        "roofline": {"bound": "hbm", "kernel": "project_kernel (gate/up + SwiGLU + A8 re-quantise)", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "project_wave_kernel (gate/up + SwiGLU + A8 re-quantise)", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": PROJECT_TRAFFIC_BYTES_DEFAULT if (args.tokens, args.layers) == (8, 6) else None,
                      "algorithmic_bytes_per_launch": cfg.project_bytes(u_mean), "avg_launch_us": kernel_us["project"]},
     }
     if not args.no_cpu:

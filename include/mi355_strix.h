@@ -66,7 +66,9 @@ int32_t mi355_dequantize_rows(uint32_t weight_type, const void* rows, uint64_t r
 
 /* Writers used to build synthetic weights on the device. Q8_0 = strix::q8_0::quantize_group
  * (include/strix/q8_0_rule.hpp:25-33) with the scale stored as fp16 (round to nearest even). The Q4_K writer has no
- * counterpart in the reference (it only reads GGUF); it is the min/max writer documented in oracle/strix_oracle.c. */
+ * counterpart in the reference (it only reads GGUF): per 32-value sub-block scale = (max - min) / 15 and offset = -min
+ * (min clamped to <= 0), super-block d = max scale / 63 and dmin = max offset / 63 stored as fp16, 6-bit sub-block factors
+ * and 4-bit codes by round-to-nearest against the fp16-rounded d / dmin. */
 int32_t mi355_quantize_weight_rows(uint32_t weight_type, const float* x, uint32_t n_rows, uint32_t elements,
                                    void* out, mi355_stream stream);
 

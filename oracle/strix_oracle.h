@@ -20,9 +20,10 @@
  *   exp is UNPINNED.
  *   orc_quantize_q4_k_row (fp32 -> Q4_K writer): the reference has no such writer -> parity unpinned
  *   (any valid writer serves: parity is defined from the packed bytes onward).
- *   orc_tp_partial (Q4_K form of the expert tensor-parallel split): the reference declares the split
- *   for IQ2_XXS/Q2_K only; the Q4_K form here keeps its structure (rank-local SwiGLU groups, rank-local
- *   K blocks, mul-then-add fold in ascending expert id) -> pinned by invariants only.
+ *   Expert tensor-parallel rank partial on Q4_K blocks (orc_routed_experts with the rank's ffn share and the
+ *   full-matrix strides, then orc_combine in the mul-then-add ascending-expert form): the reference declares the
+ *   split for its own TP pack only; the Q4_K form here keeps its structure (rank-local SwiGLU groups, rank-local
+ *   K blocks, fold in ascending expert id) -> pinned by invariants only, parity unpinned.
  */
 #ifndef STRIX_ORACLE_H
 #define STRIX_ORACLE_H

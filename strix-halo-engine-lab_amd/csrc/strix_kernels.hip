@@ -85,7 +85,9 @@ __global__ __launch_bounds__(256) void quantize_q8_0_rows_kernel(const float* x,
     }
 }
 
-// Q4_K min/max writer (no reference counterpart): the steps of oracle/strix_oracle.c orc_quantize_q4_k_row.
+// Q4_K min/max writer (no reference counterpart; the reference only reads GGUF). Per 32-value sub-block: scale =
+// (max - min) / 15 and offset = 0 - min with min clamped to <= 0; super-block d = max scale / 63, dmin = max offset / 63,
+// both stored as fp16; 6-bit factors and 4-bit codes by round-to-nearest against the fp16-rounded d / dmin.
 __global__ __launch_bounds__(64) void quantize_q4_k_rows_kernel(const float* x, uint64_t blocks, uint8_t* out) {
     for (uint64_t b = blockIdx.x * 64ULL + threadIdx.x; b < blocks; b += 64ULL * gridDim.x) {
         const float* v = x + b * 256;
