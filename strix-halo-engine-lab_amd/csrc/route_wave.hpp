@@ -18,14 +18,7 @@ constexpr uint32_t kFusedMaxRows = 16;        // decode batches: router + prolog
 
 constexpr uint32_t kRouteRowPitch = kRoutePass + 4;   // floats; +16 bytes keeps the 8 rows of a slab on different banks
 struct RouteLds {
-    union {
-        struct { float w[8][kRouteRowPitch]; float x[8][kRouteRowPitch]; } slab;   // 131,328 bytes: one pass of 8 expert rows + 8 activation rows
-        struct { float p[8][kRouteMaxExperts + 1]; } sel;             // 32,800 bytes
-        struct { uint32_t count[kRouteMaxExperts + 64]; } plan;
-    };
-    uint32_t ids[kFusedMaxRows * kRouteMaxTopK];    // selected experts of a decode batch, [row][top_k]
-    float picked[8 * kRouteMaxTopK];                // selected scores of the 8 rows in flight, [row][k]
-    uint32_t is_last;
+    struct { float w[8][kRouteRowPitch]; float x[8][kRouteRowPitch]; } slab;   // 131,328 bytes: one pass of 8 expert rows + 8 activation rows
 };
 
 struct RouteArgs {
@@ -144,109 +137,283 @@ __device__ __forceinline__ void route_logits_block(RouteLds& lds, const RouteArg
     __syncthreads();
 }
 
-// ---------------------------------------------------------------------------------------------------- softmax + top-k
-// One wave, up to 8 rows [r0, r0 + n): logits are read from scores[row][expert]; scores, ids and weights are written.
-// Selection: k passes; a pass takes the greatest remaining score, the lower id on ties - the result of the reference's
-// ascending serial scan with "c > best" (include/strix/moe/route_policy.hpp:107-121). sel_ids (optional, LDS) receives the
-// ids as [row - r0][top_k].
-struct RouteSelLds { float p[8][kRouteMaxExperts + 1]; float picked[8 * kRouteMaxTopK]; };
-__device__ __forceinline__ void route_select_rows(float (*sel_p)[kRouteMaxExperts + 1], float* picked_lds, const RouteArgs& a, uint32_t r0, uint32_t n, uint32_t* sel_ids) {
-    const uint32_t lane = threadIdx.x, E = a.p.experts, K = a.p.top_k;
-    // softmax numerators, 8 lanes per row (all rows at once): m = max over the row, p = exp(z - m)
+// ---------------------------------------------------------------------------------------------------- decode chains
+// Decode batches (rows <= 16): one wavefront per (row, 8 experts). The chain of `hidden` dependent fmas is the whole
+// cost (about 6 cycles per step), so everything else is taken off its path: the 8 router-weight rows and the activation
+// row stream global -> LDS by global_load_lds_dwordx4 in chunks of 512 features through a ring of 4 slots (three chunks
+// in flight during a chunk's chain, waits counted with s_waitcnt vmcnt); fp16 / bf16 activations are widened to fp32 in
+// LDS once per chunk (a widening fma, v_fma_mix_f32, more than doubles the latency of a chain step); a lane reads its
+// operands 32 features ahead of the chain with 128-bit LDS loads (the activation read is a broadcast).
+// Lanes 8..63 repeat lanes 0..7 (a chain gains nothing from idle lanes).
+constexpr uint32_t kChainChunk = 512;                 // features per ring slot
+constexpr uint32_t kChainPitch = kChainChunk + 4;     // floats; +16 bytes keeps the 8 weight rows on different banks
+constexpr uint32_t kChainExperts = 8;
+struct __attribute__((aligned(16))) ChainSlot {
+    float w[kChainExperts][kChainPitch];
+    float x[kChainChunk];                             // the row's features as fp32
+    uint32_t raw[kChainChunk / 2];                    // fp16 / bf16 input as copied (unused for fp32 input)
+};
+template <int KIND> constexpr uint32_t chain_copies() { return 2U * kChainExperts + (KIND == 0 ? 2U : 1U); }
+
+// Start the copy of features [k0, k0 + 512) of 8 router-weight rows and of the activation row. Every chunk issues the
+// same number of copy instructions (the waits count them): lanes past the end of the row re-fetch its last piece into
+// slot positions that are never read.
+template <int KIND>
+__device__ __forceinline__ void chain_start(ChainSlot& slot, const RouteArgs& a, uint32_t row, uint32_t e0, uint32_t k0) {
+    const uint32_t lane = threadIdx.x & 63U;
+#pragma unroll
+    for (uint32_t i = 0; i < kChainExperts; ++i) {
+        const uint32_t e = e0 + i < a.p.experts ? e0 + i : a.p.experts - 1U;
+        const float* src = a.wr + static_cast<size_t>(e) * a.hidden;
+#pragma unroll
+        for (uint32_t j = 0; j < 2U; ++j) {
+            const uint32_t k = k0 + 256U * j + 4U * lane, kk = k + 4U <= a.hidden ? k : a.hidden - 4U;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + kk),
+                                             (__attribute__((address_space(3))) void*)(&slot.w[i][256U * j]), 16, 0, 0);
+        }
+    }
+    const uint8_t* xrow = a.x + row * a.x_stride;
+    if constexpr (KIND == 0) {
+#pragma unroll
+        for (uint32_t j = 0; j < 2U; ++j) {
+            const uint32_t k = k0 + 256U * j + 4U * lane, kk = k + 4U <= a.hidden ? k : a.hidden - 4U;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xrow + 4U * kk),
+                                             (__attribute__((address_space(3))) void*)(&slot.x[256U * j]), 16, 0, 0);
+        }
+    } else {
+        const uint32_t k = k0 + 8U * lane, kk = k + 8U <= a.hidden ? k : a.hidden - 8U;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xrow + 2U * kk),
+                                         (__attribute__((address_space(3))) void*)(&slot.raw[0]), 16, 0, 0);
+    }
+}
+// fp16 / bf16: widen the landed chunk to fp32 (8 features per lane).
+template <int KIND>
+__device__ __forceinline__ void chain_widen(ChainSlot& slot) {
+    if constexpr (KIND != 0) {
+        const uint32_t lane = threadIdx.x & 63U;
+        const u32x4 r = *reinterpret_cast<const u32x4*>(&slot.raw[4U * lane]);
+        const uint32_t h[4] = {r.x, r.y, r.z, r.w};
+        float f[8];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if constexpr (KIND == 1) { f[2 * q] = half_bits_to_float(h[q] & 0xffffU); f[2 * q + 1] = half_bits_to_float(h[q] >> 16); }
+            else { f[2 * q] = f_of(h[q] << 16); f[2 * q + 1] = f_of(h[q] & 0xffff0000U); }
+        }
+        *reinterpret_cast<f32x4*>(&slot.x[8U * lane]) = f32x4{f[0], f[1], f[2], f[3]};
+        *reinterpret_cast<f32x4*>(&slot.x[8U * lane + 4U]) = f32x4{f[4], f[5], f[6], f[7]};
+        __syncthreads();
+    }
+}
+
+// Operands of 16 features: eight 128-bit LDS reads (the activation reads are broadcasts). Measured on MI355X a wave
+// pays ~5 cycles per dependent fma and ~9 per ds_read_b128, with no overlap between them, so a chain step costs about
+// 10 cycles; the operands of the next 16 features are requested before the current 16 are chained (8 reads in flight,
+// within the 15 the LDS counter can express).
+struct ChainStep { f32x4 w[4]; f32x4 x[4]; };
+__device__ __forceinline__ void chain_load(ChainStep& s, const ChainSlot& slot, uint32_t el, uint32_t k) {
+    const float* wrow = slot.w[el] + k;
+#pragma unroll
+    for (uint32_t i = 0; i < 4U; ++i) s.w[i] = *reinterpret_cast<const f32x4*>(wrow + 4U * i);
+#pragma unroll
+    for (uint32_t i = 0; i < 4U; ++i) s.x[i] = *reinterpret_cast<const f32x4*>(slot.x + k + 4U * i);
+}
+__device__ __forceinline__ float chain_run(const ChainStep& s, float acc) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        acc = __builtin_fmaf(s.x[i].x, s.w[i].x, acc); acc = __builtin_fmaf(s.x[i].y, s.w[i].y, acc);
+        acc = __builtin_fmaf(s.x[i].z, s.w[i].z, acc); acc = __builtin_fmaf(s.x[i].w, s.w[i].w, acc);
+    }
+    return acc;
+}
+
+template <int N>
+__device__ __forceinline__ void chain_wait() { __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8)); }
+
+// Logits of experts [e0, e0 + 8) for one row -> scores[row][expert] (+ bias), stored for readers in other workgroups of
+// the same launch. hidden % 32 == 0. slots: 4 separate LDS objects.
+template <int KIND>
+__device__ __forceinline__ void route_chain_block(ChainSlot* const (&slots)[4], const RouteArgs& a, uint32_t row, uint32_t e0) {
+    constexpr uint32_t NI = chain_copies<KIND>();
+    const uint32_t lane = threadIdx.x & 63U, chunks = (a.hidden + kChainChunk - 1U) / kChainChunk;
+    const bool butterfly = a.p.logits_order == MI355_LOGITS_LANE32_BUTTERFLY;
+    const uint32_t el = lane & 7U;                      // chain form: the lane's expert
+    const uint32_t bh = lane >> 5, bl = lane & 31U;     // butterfly form: experts bh, bh + 2, bh + 4, bh + 6; partial sum bl
+    float acc = 0.0F, part[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+#pragma unroll
+    for (uint32_t s = 0; s < 3U; ++s)
+        if (s < chunks) chain_start<KIND>(*slots[s], a, row, e0, s * kChainChunk);
+    for (uint32_t c0 = 0; c0 < chunks; c0 += 4U) {
+#pragma unroll
+        for (uint32_t s = 0; s < 4U; ++s) {
+            const uint32_t c = c0 + s;
+            if (c < chunks) {
+                const uint32_t last = c + 3U < chunks ? c + 3U : chunks;       // chunks started so far: 0 .. last - 1
+                const uint32_t ahead = last - 1U - c;
+                if (ahead == 0) chain_wait<0>();
+                else if (ahead == 1) chain_wait<NI>();
+                else chain_wait<2 * NI>();
+                if (c + 3U < chunks) chain_start<KIND>(*slots[(s + 3U) % 4U], a, row, e0, (c + 3U) * kChainChunk);
+                ChainSlot& slot = *slots[s];
+                chain_widen<KIND>(slot);
+                const uint32_t kc = a.hidden - c * kChainChunk < kChainChunk ? a.hidden - c * kChainChunk : kChainChunk;
+                if (!butterfly) {
+                    if (kc == kChainChunk) {      // full chunk: straight-line code, operands fetched 16 features ahead
+                        ChainStep A, B;
+                        chain_load(A, slot, el, 0);
+#pragma unroll
+                        for (uint32_t k = 0; k < kChainChunk; k += 32U) {     // the barriers pin "fetch next, then chain"
+                            chain_load(B, slot, el, k + 16U);
+                            __builtin_amdgcn_sched_barrier(0);
+                            acc = chain_run(A, acc);
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (k + 32U < kChainChunk) chain_load(A, slot, el, k + 32U);
+                            __builtin_amdgcn_sched_barrier(0);
+                            acc = chain_run(B, acc);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    } else {                      // the last, partial chunk of the row
+                        for (uint32_t k = 0; k < kc; k += 16U) {
+                            ChainStep S;
+                            chain_load(S, slot, el, k);
+                            acc = chain_run(S, acc);
+                        }
+                    }
+                } else {      // 32 strided partial sums per expert (product, then add); src/ds41_moe.cpp:74-83
+                    for (uint32_t k = 0; k < kc; k += 32U) {
+                        const float xv = slot.x[k + bl];
+#pragma unroll
+                        for (uint32_t j = 0; j < 4U; ++j) part[j] = part[j] + slot.w[bh + 2U * j][k + bl] * xv;
+                    }
+                }
+            }
+        }
+    }
+    float* out = a.scores + static_cast<size_t>(row) * a.p.experts;
+    if (!butterfly) {
+        const uint32_t e = e0 + el;
+        if (lane < kChainExperts && e < a.p.experts)
+            __hip_atomic_store(out + e, a.bias ? acc + a.bias[e] : acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+#pragma unroll
+        for (uint32_t j = 0; j < 4U; ++j) {
+            float v = part[j];
+            v = v + xor16_f(v); v = v + xor8_f(v); v = v + xor4_f(v); v = v + xor2_f(v); v = v + xor1_f(v);
+            const uint32_t e = e0 + bh + 2U * j;
+            if (bl == 0 && e < a.p.experts)
+                __hip_atomic_store(out + e, a.bias ? v + a.bias[e] : v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------- softmax + top-k (one row)
+// One wave, one row: logits are read from scores[row][expert]; scores, ids and weights are written. Lane l owns experts
+// l, l + 64, ... in registers (PER of them). Selection: k passes; a pass takes the greatest remaining score, the lower id
+// on ties - the result of the reference's ascending serial scan with "c > best"
+// (include/strix/moe/route_policy.hpp:107-121). A pass is one wave-wide maximum of 64-bit keys
+// (score bits + 1) << 32 | ~id (scores are >= 0, so their bit patterns order like the values; 0 = taken or absent), reduced
+// with DPP row shifts and row broadcasts into lane 63 and read back as a scalar. p_lds: kRouteMaxExperts floats.
+__device__ __forceinline__ float max64(float v) {
+    v = __builtin_fmaxf(v, xor1_f(v)); v = __builtin_fmaxf(v, xor2_f(v)); v = __builtin_fmaxf(v, xor4_f(v));
+    v = __builtin_fmaxf(v, xor8_f(v)); v = __builtin_fmaxf(v, xor16_f(v)); v = __builtin_fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t key_max_step(uint64_t key) {
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(static_cast<uint32_t>(key)), CTRL, ROW_MASK, 0xF, false));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(static_cast<uint32_t>(key >> 32)), CTRL, ROW_MASK, 0xF, false));
+    const uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
+    return other > key ? other : key;
+}
+__device__ __forceinline__ uint64_t key_max_wave(uint64_t key) {        // the wave's maximum, as a wave-uniform value
+    key = key_max_step<0x111, 0xF>(key);      // row_shr:1
+    key = key_max_step<0x112, 0xF>(key);      // row_shr:2
+    key = key_max_step<0x114, 0xF>(key);      // row_shr:4
+    key = key_max_step<0x118, 0xF>(key);      // row_shr:8   -> lane 15 of every row holds its row's maximum
+    key = key_max_step<0x142, 0xA>(key);      // row_bcast:15 into rows 1 and 3
+    key = key_max_step<0x143, 0xC>(key);      // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave's maximum
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(key)), 63));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(key >> 32)), 63));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+template <uint32_t PER>
+__device__ __forceinline__ void route_select_row_per(float* p_lds, const RouteArgs& a, uint32_t row) {
+    const uint32_t lane = threadIdx.x & 63U, E = a.p.experts, K = a.p.top_k;
+    float* z = a.scores + static_cast<size_t>(row) * E;
+    float v[PER];
+    float m = -INFINITY;
+#pragma unroll
+    for (uint32_t i = 0; i < PER; ++i) {
+        const uint32_t e = lane + 64U * i;
+        v[i] = e < E ? __hip_atomic_load(z + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;   // written by other workgroups of this launch
+        m = v[i] > m ? v[i] : m;
+    }
+    m = max64(m);
+#pragma unroll
+    for (uint32_t i = 0; i < PER; ++i) {
+        const uint32_t e = lane + 64U * i;
+        if (e < E) p_lds[e] = declared_exp(v[i] - m);
+    }
+    __syncthreads();
+    // denominator: ascending expert order from 0, computed by every lane (LDS broadcast reads, 16 values fetched ahead)
+    float total = 0.0F;
     {
-        const uint32_t r = lane >> 3, sub = lane & 7U, rr = r < n ? r : n - 1U;
-        const float* z = a.scores + static_cast<size_t>(r0 + rr) * E;
-        float m = -INFINITY;
-        for (uint32_t e = sub; e < E; e += 8U) { const float v = z[e]; m = v > m ? v : m; }
-        { float o = xor1_f(m); m = o > m ? o : m; o = xor2_f(m); m = o > m ? o : m; o = xor4_f(m); m = o > m ? o : m; }
-        if (r < n)
-            for (uint32_t e = sub; e < E; e += 8U) sel_p[r][e] = declared_exp(z[e] - m);
-    }
-    __syncthreads();
-    // denominators: one lane per row adds its row in ascending expert order from 0
-    float total = 1.0F;
-    if (lane < n) {
-        float s = 0.0F;
-        uint32_t e = 0;
-        for (; e + 16U <= E; e += 16U) {         // 16 values per trip keep the LDS reads ahead of the dependent adds
-            float v[16];
+        const uint32_t full = E & ~15U;
+        f32x4 t[4], n[4];
+        if (full) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) v[i] = sel_p[lane][e + i];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s = s + v[i];
+            for (int i = 0; i < 4; ++i) t[i] = *reinterpret_cast<const f32x4*>(p_lds + 4 * i);
         }
-        for (; e < E; ++e) s = s + sel_p[lane][e];
-        total = s;
+        for (uint32_t e = 0; e < full; e += 16U) {
+            const uint32_t en = e + 16U < full ? e + 16U : e;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) n[i] = *reinterpret_cast<const f32x4*>(p_lds + en + 4 * i);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { total = total + t[i].x; total = total + t[i].y; total = total + t[i].z; total = total + t[i].w; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t[i] = n[i];
+        }
+        for (uint32_t e = full; e < E; ++e) total = total + p_lds[e];
     }
-    for (uint32_t r = 0; r < n; ++r) {
-        const float sum = __shfl(total, static_cast<int>(r));
-        for (uint32_t e = lane; e < E; e += 64U) {
-            const float s = sel_p[r][e] / sum;
-            sel_p[r][e] = s;
-            a.scores[static_cast<size_t>(r0 + r) * E + e] = s;
+    uint64_t key[PER];
+#pragma unroll
+    for (uint32_t i = 0; i < PER; ++i) {
+        const uint32_t e = lane + 64U * i;
+        key[i] = 0;
+        if (e < E) {
+            const float s = p_lds[e] / total;
+            z[e] = s;
+            key[i] = (static_cast<uint64_t>(b_of(s) + 1U) << 32) | (~e);
         }
     }
-    __syncthreads();
-    // top-k: 8 lanes per row; lane `sub` owns experts sub, sub + 8, ... (ascending). A taken score is replaced by -1
-    // (scores are >= 0), so one pass is a plain arg-max with the lower id winning ties. The pass loop is not unrolled.
-    const uint32_t r = lane >> 3, sub = lane & 7U;
-    const bool live = r < n;
-    float* p = sel_p[live ? r : 0U];
-    constexpr uint32_t kInReg = 32;                    // scores per lane kept in registers (experts <= 256)
-    const bool in_reg = E <= 8U * kInReg;
-    float mine[kInReg];
-    if (in_reg) {
-#pragma unroll
-        for (uint32_t i = 0; i < kInReg; ++i) mine[i] = sub + 8U * i < E ? p[sub + 8U * i] : -2.0F;
-    }
-    __syncthreads();
-    float* picked = picked_lds;
-    float sum = 0.0F;
+    float sum = 0.0F, my_v = 0.0F;
+    uint32_t my_id = 0;
 #pragma unroll 1
     for (uint32_t k = 0; k < K; ++k) {
-        float bv = -3.0F;
-        uint32_t bi = 0xffffffffU;
-        if (in_reg) {
+        uint64_t best = key[0];
 #pragma unroll
-            for (uint32_t i = 0; i < kInReg; ++i)
-                if (mine[i] > bv) { bv = mine[i]; bi = sub + 8U * i; }
-        } else {
-            for (uint32_t e = sub; e < E; e += 8U) {
-                const float c = p[e];
-                if (c > bv) { bv = c; bi = e; }
-            }
-        }
-        {   // arg-max over the row's 8 lanes by DPP (lane ^ 1, ^ 2, ^ 4)
-            float ov = xor1_f(bv); uint32_t oi = static_cast<uint32_t>(xor1_i(static_cast<int>(bi)));
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-            ov = xor2_f(bv); oi = static_cast<uint32_t>(xor2_i(static_cast<int>(bi)));
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-            ov = xor4_f(bv); oi = static_cast<uint32_t>(xor4_i(static_cast<int>(bi)));
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-        }
-        if ((bi & 7U) == sub) {                        // the owner retires the pick
-            if (in_reg) {
+        for (uint32_t i = 1; i < PER; ++i) best = key[i] > best ? key[i] : best;
+        best = key_max_wave(best);
+        const uint32_t bi = ~static_cast<uint32_t>(best);
+        const float bv = f_of(static_cast<uint32_t>(best >> 32) - 1U);
 #pragma unroll
-                for (uint32_t i = 0; i < kInReg; ++i)
-                    if (i == (bi >> 3)) mine[i] = -1.0F;
-            } else if (live) {
-                p[bi] = -1.0F;
-            }
-        }
+        for (uint32_t i = 0; i < PER; ++i)
+            if (lane + 64U * i == bi) key[i] = 0;       // the owner retires the pick
         sum = sum + bv;                                // ((0 + s_0) + s_1) + ... in selection order
-        if (live && sub == 0) {
-            a.ids[static_cast<size_t>(r0 + r) * K + k] = bi;
-            if (sel_ids) sel_ids[r * K + k] = bi;
-            picked[r * kRouteMaxTopK + k] = bv;
-        }
+        if (lane == k) { my_v = bv; my_id = bi; }
     }
     const float den = sum + a.p.renorm_eps;
-    if (live && sub == 0)
-        for (uint32_t k = 0; k < K; ++k) {
-            const float v = picked[r * kRouteMaxTopK + k];
-            a.weights[static_cast<size_t>(r0 + r) * K + k] = (a.p.renormalize ? v / den : v) * a.p.scale;
-        }
+    if (lane < K) {
+        __hip_atomic_store(a.ids + static_cast<size_t>(row) * K + lane, my_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // read by the plan builder
+        a.weights[static_cast<size_t>(row) * K + lane] = (a.p.renormalize ? my_v / den : my_v) * a.p.scale;
+    }
     __syncthreads();
+}
+__device__ __forceinline__ void route_select_row(float* p_lds, const RouteArgs& a, uint32_t row) {
+    const uint32_t E = a.p.experts;
+    if (E <= 128U) route_select_row_per<2>(p_lds, a, row);
+    else if (E <= 256U) route_select_row_per<4>(p_lds, a, row);
+    else if (E <= 512U) route_select_row_per<8>(p_lds, a, row);
+    else route_select_row_per<16>(p_lds, a, row);
 }
 
 }  // namespace strix950

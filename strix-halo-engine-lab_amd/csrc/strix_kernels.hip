@@ -264,21 +264,50 @@ __device__ __forceinline__ void build_plan_wave(uint32_t* count, const uint32_t*
     }
 }
 
-// Router launch. Blocks [0, route_blocks) run the logit chains of 8 experts x 8 rows; in the fused decode form, blocks
-// [route_blocks, route_blocks + quant_blocks) quantise the input rows to A8 (8 groups of 32 per block), and the block
-// that takes the last launch ticket runs softmax / top-k / weights for every row, publishes the row status words and
-// builds the expert plan. In the plain form (a.plan == nullptr) the kernel stops after the logits.
+// Router logits for batches above the decode bound: blocks of 8 experts x 8 rows.
 template <int KIND>
 __global__ __launch_bounds__(64) void route_logits_kernel(RouteArgs a) {
     __shared__ RouteLds lds;
-    const uint32_t bid = blockIdx.x, lane = threadIdx.x;
+    const uint32_t neb = (a.p.experts + 7U) / 8U;
+    route_logits_block<KIND>(lds, a, (blockIdx.x % neb) * 8U, (blockIdx.x / neb) * 8U);
+}
+
+// Decode router launch (rows <= 16). Blocks [0, route_blocks) run the logit chains of (row, 8 experts). In the plain form
+// (a.plan == nullptr) the kernel stops there. In the fused form blocks [route_blocks, route_blocks + quant_blocks)
+// quantise the input rows to A8 (8 groups of 32 per block); the block that finishes a row's last 8 experts (row ticket)
+// runs that row's softmax / top-k / weights, and the block that takes the last launch ticket publishes the row status
+// words and builds the expert plan. Every ticket word is left zero.
+template <int KIND>
+__global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
+    __shared__ ChainSlot slot0;
+    __shared__ ChainSlot slot1;
+    __shared__ ChainSlot slot2;
+    __shared__ ChainSlot slot3;
+    __shared__ __attribute__((aligned(16))) float sel_p[kRouteMaxExperts];
+    __shared__ uint32_t count[kRouteMaxExperts + 64];
+    __shared__ uint32_t ids[kFusedMaxRows * kRouteMaxTopK];
+    __shared__ uint32_t flag;
+    ChainSlot* const slots[4] = {&slot0, &slot1, &slot2, &slot3};
+    const uint32_t bid = blockIdx.x, lane = threadIdx.x, neb = (a.p.experts + 7U) / 8U;
+    uint32_t* tickets = a.plan ? a.plan + plan_tickets_at(a.p.experts, a.rows * a.p.top_k) : nullptr;
     if (bid < a.route_blocks) {
-        const uint32_t neb = (a.p.experts + 7U) / 8U;
-        route_logits_block<KIND>(lds, a, (bid % neb) * 8U, (bid / neb) * 8U);
+        const uint32_t row = bid / neb;
+        route_chain_block<KIND>(slots, a, row, (bid % neb) * 8U);
+        if (!a.plan) return;
+        // hand-off between workgroups without cache-wide fences: the logits were stored write-through at device scope and
+        // are complete once the wave's store counter drains; the reader loads them at device scope
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (lane == 0) flag = __hip_atomic_fetch_add(&tickets[row], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == neb - 1U;
+        __syncthreads();
+        if (flag) {
+            if (lane == 0) tickets[row] = 0;
+            route_select_row(sel_p, a, row);
+        }
     } else {
         // A8 prologue (src/cpu/core/reference.cpp:35-55): two groups of 32 at a time, 8 groups per block
         const uint32_t groups = a.hidden / 32U, total = a.rows * groups, g0 = (bid - a.route_blocks) * 8U;
-        uint32_t* flags = a.plan + plan_tickets_at(a.p.experts, a.rows * a.p.top_k) + 128U;
+        uint32_t* flags = tickets + 128U;
         for (uint32_t i = 0; i < 8U; i += 2U) {
             const uint32_t g = g0 + i + (lane >> 5), j = lane & 31U;
             if (g < total) {
@@ -299,26 +328,24 @@ __global__ __launch_bounds__(64) void route_logits_kernel(RouteArgs a) {
             }
         }
     }
-    if (!a.plan) return;
-    __threadfence();
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (lane == 0) lds.is_last = atomicAdd(&a.plan[3], 1U) == gridDim.x - 1U;
+    if (lane == 0) flag = __hip_atomic_fetch_add(&a.plan[3], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1U;
     __syncthreads();
-    if (!lds.is_last) return;
-    __threadfence();
-    for (uint32_t r0 = 0; r0 < a.rows; r0 += 8U)
-        route_select_rows(lds.sel.p, lds.picked, a, r0, a.rows - r0 < 8U ? a.rows - r0 : 8U, lds.ids + r0 * a.p.top_k);
-    uint32_t* flags = a.plan + plan_tickets_at(a.p.experts, a.rows * a.p.top_k) + 128U;
-    if (lane < a.rows) { a.status[lane] = flags[lane]; flags[lane] = 0; }
+    if (!flag) return;
+    const uint32_t assignments = a.rows * a.p.top_k;
+    for (uint32_t i = lane; i < assignments; i += 64U) ids[i] = __hip_atomic_load(a.ids + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t* flags = tickets + 128U;
+    if (lane < a.rows) { a.status[lane] = __hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); flags[lane] = 0; }
     if (lane == 0) { *a.job_status = 0; a.plan[3] = 0; }
-    build_plan_wave(lds.plan.count, lds.ids, a.p.experts, a.rows * a.p.top_k, a.plan);
+    __syncthreads();
+    build_plan_wave(count, ids, a.p.experts, assignments, a.plan);
 }
 
-// softmax / top-k / weights for 8 rows per one-wave block (the plain router and batches above the fused bound).
+// softmax / top-k / weights, one row per one-wave block (the plain router).
 __global__ __launch_bounds__(64) void route_select_kernel(RouteArgs a) {
-    __shared__ RouteSelLds lds;
-    const uint32_t r0 = blockIdx.x * 8U;
-    route_select_rows(lds.p, lds.picked, a, r0, a.rows - r0 < 8U ? a.rows - r0 : 8U, nullptr);
+    __shared__ __attribute__((aligned(16))) float sel_p[kRouteMaxExperts];
+    route_select_row(sel_p, a, blockIdx.x);
 }
 
 // ======================================================================================================== expert plan
@@ -756,10 +783,22 @@ int32_t check_route(const mi355_route_policy* p, const void* x, uint32_t kind, u
     STRIX_REQUIRE(aligned(wr, 16) && aligned(x, 16) && x_stride % 16U == 0, "route: router weight, activations and their row stride must be 16-byte aligned");
     return MI355_OK;
 }
-void launch_route_logits(const RouteArgs& a, uint32_t blocks, hipStream_t st) {
-    if (a.kind == MI355_INPUT_F32) route_logits_kernel<0><<<blocks, 64, 0, st>>>(a);
-    else if (a.kind == MI355_INPUT_F16) route_logits_kernel<1><<<blocks, 64, 0, st>>>(a);
-    else route_logits_kernel<2><<<blocks, 64, 0, st>>>(a);
+// Logits of every (row, expert) into a.scores. Decode batches: one block per (row, 8 experts), plus a.quant_blocks blocks
+// in the fused form; larger batches: one block per (8 rows, 8 experts).
+void launch_route_logits(RouteArgs& a, hipStream_t st) {
+    const uint32_t neb = (a.p.experts + 7U) / 8U;
+    if (a.rows <= kFusedMaxRows) {
+        a.route_blocks = neb * a.rows;
+        const uint32_t blocks = a.route_blocks + a.quant_blocks;
+        if (a.kind == MI355_INPUT_F32) route_decode_kernel<0><<<blocks, 64, 0, st>>>(a);
+        else if (a.kind == MI355_INPUT_F16) route_decode_kernel<1><<<blocks, 64, 0, st>>>(a);
+        else route_decode_kernel<2><<<blocks, 64, 0, st>>>(a);
+    } else {
+        a.route_blocks = neb * ((a.rows + 7U) / 8U);
+        if (a.kind == MI355_INPUT_F32) route_logits_kernel<0><<<a.route_blocks, 64, 0, st>>>(a);
+        else if (a.kind == MI355_INPUT_F16) route_logits_kernel<1><<<a.route_blocks, 64, 0, st>>>(a);
+        else route_logits_kernel<2><<<a.route_blocks, 64, 0, st>>>(a);
+    }
 }
 }  // namespace
 
@@ -770,9 +809,8 @@ int32_t mi355_moe_route(const mi355_route_policy* p, const void* x, uint32_t kin
     RouteArgs a{};
     a.p = *p; a.x = static_cast<const uint8_t*>(x); a.kind = kind; a.x_stride = x_stride; a.rows = rows; a.hidden = hidden;
     a.wr = wr; a.bias = bias; a.ids = ids; a.weights = weights; a.scores = scores;
-    a.route_blocks = ((p->experts + 7U) / 8U) * ((rows + 7U) / 8U);
-    launch_route_logits(a, a.route_blocks, hs(stream));
-    route_select_kernel<<<(rows + 7U) / 8U, 64, 0, hs(stream)>>>(a);
+    launch_route_logits(a, hs(stream));
+    route_select_kernel<<<rows, 64, 0, hs(stream)>>>(a);
     STRIX_LAUNCHED("moe_route");
     return MI355_OK;
 }
@@ -854,9 +892,8 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     a.p = *p; a.x = static_cast<const uint8_t*>(r->input); a.kind = r->input_kind; a.x_stride = r->input_stride; a.rows = rows; a.hidden = wv.hidden;
     a.wr = router_weight; a.bias = logit_bias; a.ids = ids; a.weights = weights; a.scores = scores;
     a.codes = r->codes; a.deltas = r->deltas; a.sums = r->sums; a.status = r->status; a.job_status = r->job_status; a.plan = r->plan;
-    a.route_blocks = ((p->experts + 7U) / 8U) * ((rows + 7U) / 8U);
     a.quant_blocks = (rows * (wv.hidden / 32U) + 7U) / 8U;
-    launch_route_logits(a, a.route_blocks + a.quant_blocks, hs(stream));
+    launch_route_logits(a, hs(stream));
     STRIX_LAUNCHED("moe layer router");
     launch_project(wv, *r, rows, touched_bound(wv, rows), hs(stream));
     launch_down(wv, *r, rows, touched_bound(wv, rows), hs(stream));
