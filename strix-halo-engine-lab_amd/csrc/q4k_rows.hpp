@@ -11,9 +11,10 @@
 // LDS side: lane r reads its nine pieces with ds_read_b128 at r * 144 + 16 c; the 36-word row pitch makes every group
 // of eight lanes cover all banks, so the reads are conflict free without padding.
 //
-// Activation side: the A8 image (codes, deltas, sums) of an activation row is the same for every lane, so it is read
-// through the constant address space with wave-uniform addresses: the compiler emits scalar loads, and the codes feed
-// v_dot4_i32_i8 as scalar operands. No activation byte passes through LDS or a VGPR.
+// Activation side: the 256 int8 codes of the stage's super-block of each activation row ride in the same ring slot
+// (one more global_load_lds per 4 activation rows), a full stage ahead of their use; every lane reads them with broadcast
+// 128-bit LDS loads. (Scalar loads of the codes were measured slower: they return out of order, so each step exposed a
+// full L2 round trip.) The group deltas and sums sit one group per lane and are broadcast with v_readlane.
 //
 // Arithmetic per row, super-block b ascending, pair p = 0..3 (sub-blocks j = 2p: low nibbles, 2p + 1: high nibbles):
 //   x_j = E_g * ((D_j * float(dot_j)) - (DM_j * float(S_g))),  D_j = d * sc_j, DM_j = dmin * m_j, g = 8 b + j
@@ -29,10 +30,11 @@ namespace strix950 {
 constexpr uint32_t kWaveRows = 64;
 constexpr uint32_t kStageBytes = kWaveRows * 144U;   // 9,216
 constexpr uint32_t kStagePieces = 9;                 // global_load_lds instructions per stage (576 pieces / 64 lanes)
+// a ring slot: the stage's weights + its codes of up to nbmax (4 or 8) activation rows
+__host__ __device__ constexpr uint32_t slot_bytes(int nbmax) { return kStageBytes + 256U * static_cast<uint32_t>(nbmax); }
+typedef __attribute__((address_space(3))) uint8_t lds_u8;      // ring slots are addressed in the LDS address space
+template <int NA> constexpr uint32_t stage_copies() { return kStagePieces + (NA + 3) / 4; }   // copy instructions per stage
 
-typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-#define STRIX_CONSTANT __attribute__((address_space(4)))
 
 struct A8Image {                             // device A8 image: codes [rows][width], deltas / sums [rows][width / 32]
     const int8_t* codes;
@@ -44,6 +46,7 @@ struct A8Image {                             // device A8 image: codes [rows][wi
 // Per-lane source pointers of the nine pieces the lane copies in every stage. row_ptr(r) = first byte of row r (0..63).
 struct StageSource {
     const uint8_t* piece[kStagePieces];
+    const uint8_t* act_piece[2];              // the lane's 16 bytes of activation rows lane / 16 and 4 + lane / 16
     template <class RowPtr>
     __device__ __forceinline__ void init(RowPtr row_ptr) {
         const uint32_t lane = threadIdx.x & 63U;
@@ -53,27 +56,44 @@ struct StageSource {
             piece[i] = row_ptr(r) + 16U * c;
         }
     }
-    // start the copy of the next super-block of all 64 rows into one ring slot, then step to the block after it
-    __device__ __forceinline__ void start(uint8_t* slot) {
+    // lane_row[h] = index (into the A8 image) of activation row 4 h + lane / 16, any valid row where that is >= NA
+    template <int NA>
+    __device__ __forceinline__ void init_act(const int8_t* codes, uint32_t width, const uint32_t (&lane_row)[(NA + 3) / 4]) {
+        const uint32_t lane = threadIdx.x & 63U;
+#pragma unroll
+        for (int h = 0; h < (NA + 3) / 4; ++h)
+            act_piece[h] = reinterpret_cast<const uint8_t*>(codes) + static_cast<size_t>(lane_row[h]) * width + 16U * (lane & 15U);
+    }
+    // start the copy of the next super-block of all 64 rows (and of the activation rows' codes) into one ring slot,
+    // then step to the block after it
+    template <int NA>
+    __device__ __forceinline__ void start(lds_u8* slot) {
 #pragma unroll
         for (uint32_t i = 0; i < kStagePieces; ++i) {
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)piece[i],
                                              (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
             piece[i] += 144;
         }
+#pragma unroll
+        for (int h = 0; h < (NA + 3) / 4; ++h) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)act_piece[h],
+                                             (__attribute__((address_space(3))) void*)(slot + kStageBytes + 1024U * h), 16, 0, 0);
+            act_piece[h] += 256;
+        }
     }
 };
 
-// s_waitcnt vmcnt(N): at most N vector memory operations (here: stage copies, nine per stage) still outstanding.
+// s_waitcnt vmcnt(N): at most N vector memory operations (here: stage copies, PER per stage) still outstanding.
 template <int N>
 __device__ __forceinline__ void wait_copies() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
+template <int PER>
 __device__ __forceinline__ void wait_stages_ahead(uint32_t ahead) {   // ahead = stages started after the one needed
     if (ahead == 0) wait_copies<0>();
-    else if (ahead == 1) wait_copies<9>();
-    else if (ahead == 2) wait_copies<18>();
-    else wait_copies<27>();
+    else if (ahead == 1) wait_copies<PER>();
+    else if (ahead == 2) wait_copies<2 * PER>();
+    else wait_copies<3 * PER>();
 }
 
 // 6-bit scale / min of sub-block J (compile-time) from the three scale words of a block header
@@ -90,20 +110,23 @@ __device__ __forceinline__ void q4k_factors(const u32x4& hd, uint32_t& sc, uint3
     }
 }
 
-// Uniform view of the NA activation rows of one sweep. The codes are read with scalar loads of 64 bytes (one pair's
-// 64 codes); the group deltas and sums are held one group per lane (64 groups = 8 super-blocks per refill) and
-// broadcast with v_readlane.
+// Uniform view of the NA activation rows of one sweep (row bases, wave-uniform).
 template <int NA>
 struct ActRows {
-    const STRIX_CONSTANT u32x16* codes[NA];    // row base, wave-uniform
-    const float* deltas[NA];                   // row base
+    const int8_t* codes;                       // image base
+    uint32_t width;
+    uint32_t lane_row[(NA + 3) / 4];           // per lane: image row of activation row 4 h + lane / 16 (see StageSource::init_act)
+    const float* deltas[NA];
     const int32_t* sums[NA];
     uint32_t groups;                           // per activation row
-    __device__ __forceinline__ ActRows(const A8Image& img, const uint32_t (&row)[NA]) : groups(img.width / 32U) {
+    // row[a]: image row of activation row a (any lane's value is taken); lane_rows: the per-lane rows for the code copies
+    __device__ __forceinline__ ActRows(const A8Image& img, const uint32_t (&row)[NA], const uint32_t (&lane_rows)[(NA + 3) / 4])
+        : codes(img.codes), width(img.width), groups(img.width / 32U) {
+#pragma unroll
+        for (int h = 0; h < (NA + 3) / 4; ++h) lane_row[h] = lane_rows[h];
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             const uint32_t r = __builtin_amdgcn_readfirstlane(row[a]);
-            codes[a] = (const STRIX_CONSTANT u32x16*)(img.codes + static_cast<size_t>(r) * img.width);
             deltas[a] = img.deltas + static_cast<size_t>(r) * groups;
             sums[a] = img.sums + static_cast<size_t>(r) * groups;
         }
@@ -114,30 +137,18 @@ __device__ __forceinline__ float lane_value(float v, uint32_t lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), static_cast<int>(lane)));
 }
 
-// One super-block (index kb along K, `blocks` in the row) of the lane's row, from ring slot `slot`, against the NA
-// activation rows. The work is cut into 2 NA steps (activation row a, pair half); the codes of a step (two scalar
-// loads of 64 bytes: n0, n1) are requested one step ahead, so on entry n0 / n1 hold step (kb, 0, 0) and on exit step
-// (kb + 1, 0, 0). Scalar loads return out of order, so the only usable wait is "all of them": each step first waits for
-// its own codes, then requests the next step's, then computes.
+// One super-block (index kb along K) of the lane's row against the NA activation rows, both from ring slot `slot`.
+// vd / vf: the activation rows' group deltas / sums, group 8 (kb % 8) + j in lane 8 (kb % 8) + j.
 template <int NA>
-__device__ __forceinline__ void block_compute(const uint8_t* slot, const ActRows<NA>& act, uint32_t kb, uint32_t blocks,
-                                              const float (&vd)[NA], const float (&vf)[NA], u32x16& n0, u32x16& n1, float (&acc)[NA][4]) {
-    const u32x4* blk = reinterpret_cast<const u32x4*>(slot + (threadIdx.x & 63U) * 144U);
+__device__ __forceinline__ void block_compute(const lds_u8* slot, uint32_t kb, const float (&vd)[NA], const float (&vf)[NA],
+                                              float (&acc)[NA][4]) {
+    typedef const __attribute__((address_space(3))) u32x4 lds_u32x4;
+    lds_u32x4* blk = (lds_u32x4*)(slot + (threadIdx.x & 63U) * 144U);
     const u32x4 hd = blk[0];
     u32x4 q[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) q[i] = blk[1 + i];
     const float d = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
-    int lo[4][8], hi[4][8];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const uint32_t w[8] = {q[2 * p].x, q[2 * p].y, q[2 * p].z, q[2 * p].w, q[2 * p + 1].x, q[2 * p + 1].y, q[2 * p + 1].z, q[2 * p + 1].w};
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            lo[p][k] = static_cast<int>(w[k] & 0x0f0f0f0fU);
-            hi[p][k] = static_cast<int>((w[k] >> 4) & 0x0f0f0f0fU);
-        }
-    }
     uint32_t sc[8], mn[8];
     q4k_factors<0>(hd, sc[0], mn[0]); q4k_factors<1>(hd, sc[1], mn[1]); q4k_factors<2>(hd, sc[2], mn[2]); q4k_factors<3>(hd, sc[3], mn[3]);
     q4k_factors<4>(hd, sc[4], mn[4]); q4k_factors<5>(hd, sc[5], mn[5]); q4k_factors<6>(hd, sc[6], mn[6]); q4k_factors<7>(hd, sc[7], mn[7]);
@@ -147,50 +158,43 @@ __device__ __forceinline__ void block_compute(const uint8_t* slot, const ActRows
         D[j] = d * static_cast<float>(sc[j]);
         M[j] = dm * static_cast<float>(mn[j]);
     }
-    const uint32_t next_kb = kb + 1U < blocks ? kb + 1U : kb;      // the last block re-requests itself (unused)
     const uint32_t g0 = (kb & 7U) * 8U;
 #pragma unroll
-    for (int a = 0; a < NA; ++a) {
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t w[8] = {q[2 * p].x, q[2 * p].y, q[2 * p].z, q[2 * p].w, q[2 * p + 1].x, q[2 * p + 1].y, q[2 * p + 1].z, q[2 * p + 1].w};
+        int lo[8], hi[8];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            __builtin_amdgcn_s_waitcnt(0xC07F);                    // lgkmcnt(0): this step's codes have arrived
-            const u32x16 c0 = n0, c1 = n1;
-            __builtin_amdgcn_sched_barrier(0);
-            {
-                const int na = half ? (a + 1 < NA ? a + 1 : 0) : a;
-                const uint32_t nb = (half && a + 1 == NA) ? next_kb : kb;
-                const STRIX_CONSTANT u32x16* next = act.codes[na] + (nb * 4U + (half ? 0U : 2U));
-                n0 = next[0];
-                n1 = next[1];
+        for (int k = 0; k < 8; ++k) {
+            lo[k] = static_cast<int>(w[k] & 0x0f0f0f0fU);
+            hi[k] = static_cast<int>((w[k] >> 4) & 0x0f0f0f0fU);
+        }
+#pragma unroll
+        for (int a = 0; a < NA; ++a) {
+            lds_u32x4* codes = (lds_u32x4*)(slot + kStageBytes + 256U * a + 64U * p);
+            const u32x4 c0 = codes[0], c1 = codes[1], c2 = codes[2], c3 = codes[3];
+            const uint32_t c[16] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w, c2.x, c2.y, c2.z, c2.w, c3.x, c3.y, c3.z, c3.w};
+            int dot0 = 0, dot1 = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                dot0 = __builtin_amdgcn_sdot4(lo[k], static_cast<int>(c[k]), dot0, false);
+                dot1 = __builtin_amdgcn_sdot4(hi[k], static_cast<int>(c[8 + k]), dot1, false);
             }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int pp = 0; pp < 2; ++pp) {
-                const int p = 2 * half + pp;
-                const u32x16& c = pp ? c1 : c0;
-                int dot0 = 0, dot1 = 0;
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    dot0 = __builtin_amdgcn_sdot4(lo[p][k], static_cast<int>(c[k]), dot0, false);
-                    dot1 = __builtin_amdgcn_sdot4(hi[p][k], static_cast<int>(c[8 + k]), dot1, false);
-                }
-                const float e0 = lane_value(vd[a], g0 + 2U * p), e1 = lane_value(vd[a], g0 + 2U * p + 1U);
-                const float f0 = lane_value(vf[a], g0 + 2U * p), f1 = lane_value(vf[a], g0 + 2U * p + 1U);
-                const float u0 = D[2 * p] * static_cast<float>(dot0), v0 = M[2 * p] * f0;
-                const float u1 = D[2 * p + 1] * static_cast<float>(dot1), v1 = M[2 * p + 1] * f1;
-                const float t0 = u0 - v0, t1 = u1 - v1;
-                const float x0 = e0 * t0, x1 = e1 * t1;
-                acc[a][p] = acc[a][p] + (x0 + x1);
-            }
+            const float e0 = lane_value(vd[a], g0 + 2U * p), e1 = lane_value(vd[a], g0 + 2U * p + 1U);
+            const float f0 = lane_value(vf[a], g0 + 2U * p), f1 = lane_value(vf[a], g0 + 2U * p + 1U);
+            const float u0 = D[2 * p] * static_cast<float>(dot0), v0 = M[2 * p] * f0;
+            const float u1 = D[2 * p + 1] * static_cast<float>(dot1), v1 = M[2 * p + 1] * f1;
+            const float t0 = u0 - v0, t1 = u1 - v1;
+            const float x0 = e0 * t0, x1 = e1 * t1;
+            acc[a][p] = acc[a][p] + (x0 + x1);
         }
     }
 }
 
 // Whole sweep: K = blocks super-blocks of the 64 rows described by `source` against the NA rows of `act`.
-// value[a] = the lane's row against activation row a. `slots` are DEPTH separate LDS buffers of kStageBytes.
+// value[a] = the lane's row against activation row a. `slots` are DEPTH separate LDS buffers of slot_bytes().
 // On entry nothing is in flight; on exit every copy has landed and been consumed.
 template <int NA, int DEPTH>
-__device__ __forceinline__ void sweep_rows(uint8_t* const (&slots)[DEPTH], StageSource source, uint32_t blocks,
+__device__ __forceinline__ void sweep_rows(lds_u8* const (&slots)[DEPTH], StageSource source, uint32_t blocks,
                                            const ActRows<NA>& act, float (&value)[NA]) {
     const uint32_t lane = threadIdx.x & 63U;
     float acc[NA][4];
@@ -201,10 +205,10 @@ __device__ __forceinline__ void sweep_rows(uint8_t* const (&slots)[DEPTH], Stage
     float vd[NA], vf[NA];
 #pragma unroll
     for (int a = 0; a < NA; ++a) vd[a] = vf[a] = 0.0F;
+    source.init_act<NA>(act.codes, act.width, act.lane_row);
 #pragma unroll
     for (int s = 0; s < DEPTH - 1; ++s)
-        if (static_cast<uint32_t>(s) < blocks) source.start(slots[s]);
-    u32x16 n0 = act.codes[0][0], n1 = act.codes[0][1];
+        if (static_cast<uint32_t>(s) < blocks) source.start<NA>(slots[s]);
     for (uint32_t b0 = 0; b0 < blocks; b0 += DEPTH) {
 #pragma unroll
         for (int s = 0; s < DEPTH; ++s) {
@@ -220,9 +224,9 @@ __device__ __forceinline__ void sweep_rows(uint8_t* const (&slots)[DEPTH], Stage
                 }
                 // started so far: stages 0 .. min(blocks, b + DEPTH - 1) - 1; stage b must have landed
                 const uint32_t last = b + DEPTH - 1U < blocks ? b + DEPTH - 1U : blocks;
-                wait_stages_ahead(last - 1U - b);
-                if (b + DEPTH - 1U < blocks) source.start(slots[(s + DEPTH - 1) % DEPTH]);
-                block_compute<NA>(slots[s], act, b, blocks, vd, vf, n0, n1, acc);
+                wait_stages_ahead<stage_copies<NA>()>(last - 1U - b);
+                if (b + DEPTH - 1U < blocks) source.start<NA>(slots[(s + DEPTH - 1) % DEPTH]);
+                block_compute<NA>(slots[s], b, vd, vf, acc);
             }
         }
     }

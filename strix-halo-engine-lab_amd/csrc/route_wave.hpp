@@ -28,7 +28,7 @@ struct RouteArgs {
     uint32_t* ids; float* weights; float* scores;
     // fused decode extras (all null / zero for the plain router)
     int8_t* codes; float* deltas; int32_t* sums; uint32_t* status; uint32_t* job_status; uint32_t* plan;
-    uint32_t route_blocks, quant_blocks;
+    uint32_t route_blocks, quant_blocks, split, item_bound;
 };
 
 // ---------------------------------------------------------------------------------------------------- logit chains

@@ -199,32 +199,41 @@ __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v, ui
 
 // ======================================================================================================== router
 // Plan words (uint32): [0] assignments A = rows * top_k, [1] touched experts U, [2] largest group, [3] launch ticket,
-// [16 ..] offsets[experts + 1]; touched[experts] (ids of the experts with work, ascending); order[A]: assignment indices
-// (row * top_k + slot) grouped by expert, ascending row then slot inside an expert; items[min(experts, A)] x 4 words
-// {expert, begin, end, 0} (one record per touched expert, zero records after the last); 256 ticket / scratch words.
+// [4] work items; [16 ..] offsets[experts + 1]; touched[experts] (ids of the experts with work, ascending); order[A]:
+// assignment indices (row * top_k + slot) grouped by expert, ascending row then slot inside an expert; items[A] x 4 words
+// {expert, begin, end, 0}: the work items of the expert kernels, a touched expert's assignments cut into pieces of at
+// most `split` (zero records after the last item, up to the launch's item bound); 256 ticket / scratch words.
 // Reference: src/hip_moe_q4k_a8_probe.hip:91-147 (stable CSR of (row, slot) by expert).
 __host__ __device__ inline uint32_t pad4(uint32_t v) { return (v + 3U) & ~3U; }
 __host__ __device__ inline uint32_t plan_touched_at(uint32_t experts) { return 16U + pad4(experts + 1U); }
 __host__ __device__ inline uint32_t plan_order_at(uint32_t experts) { return plan_touched_at(experts) + pad4(experts); }
-__host__ __device__ inline uint32_t plan_item_bound(uint32_t experts, uint32_t assignments) { return assignments < experts ? assignments : experts; }
+// most work items a plan can hold (layout) and most a launch with pieces of `split` assignments can produce (grid size)
+__host__ __device__ inline uint32_t plan_item_capacity(uint32_t assignments) { return assignments; }
+__host__ __device__ inline uint32_t plan_item_bound(uint32_t experts, uint32_t assignments, uint32_t split) {
+    const uint32_t most = experts + assignments / split;
+    return assignments < most ? assignments : most;
+}
 __host__ __device__ inline uint32_t plan_items_at(uint32_t experts, uint32_t assignments) { return plan_order_at(experts) + pad4(assignments); }
 __host__ __device__ inline uint32_t plan_tickets_at(uint32_t experts, uint32_t assignments) {
-    return plan_items_at(experts, assignments) + 4U * plan_item_bound(experts, assignments);
+    return plan_items_at(experts, assignments) + 4U * plan_item_capacity(assignments);
 }
-constexpr uint32_t kPlanTicketWords = 256;     // [0, 128): merge tickets, [128, 256): per-row A8 flags of the fused prologue
+// ticket / scratch words at the end of a plan: [0, 16) row tickets of the fused router, [128, 144) per-row A8 flags of the
+// fused prologue
+constexpr uint32_t kPlanTicketWords = 256;
 
 // Expert plan by one wave from the ids of a decode batch held in LDS (A <= 256 assignments).
-__device__ __forceinline__ void build_plan_wave(uint32_t* count, const uint32_t* ids, uint32_t experts, uint32_t assignments, uint32_t* plan) {
+__device__ __forceinline__ void build_plan_wave(uint32_t* count, const uint32_t* ids, uint32_t experts, uint32_t assignments, uint32_t split,
+                                                uint32_t item_bound, uint32_t* plan) {
     const uint32_t lane = threadIdx.x;
     for (uint32_t e = lane; e <= experts; e += 64U) count[e] = 0;
     __syncthreads();
     for (uint32_t a = lane; a < assignments; a += 64U) atomicAdd(&count[ids[a]], 1U);
     __syncthreads();
     const uint32_t chunk = (experts + 63U) / 64U, first = lane * chunk, last = first + chunk < experts ? first + chunk : experts;
-    uint32_t local = 0, local_touched = 0, largest = 0;
+    uint32_t local = 0, local_touched = 0, largest = 0;     // local_touched: touched experts << 16 | work items (A <= 256)
     for (uint32_t e = first; e < last; ++e) {
         const uint32_t c = count[e];
-        local += c; local_touched += c != 0; largest = c > largest ? c : largest;
+        local += c; local_touched += ((c != 0) << 16) + (c + split - 1U) / split; largest = c > largest ? c : largest;
     }
     uint32_t run = local, trun = local_touched;
 #pragma unroll
@@ -233,8 +242,10 @@ __device__ __forceinline__ void build_plan_wave(uint32_t* count, const uint32_t*
         if (lane >= static_cast<uint32_t>(d)) { run += o; trun += t; }
     }
     for (int d = 32; d; d >>= 1) { const uint32_t o = __shfl_xor(largest, d); largest = o > largest ? o : largest; }
-    const uint32_t touched_total = __shfl(trun, 63);
+    const uint32_t totals = __shfl(trun, 63), touched_total = totals >> 16, items_total = totals & 0xffffU;
     run -= local; trun -= local_touched;                    // exclusive prefixes
+    uint32_t irun = trun & 0xffffU;
+    trun >>= 16;
     uint32_t* offsets = plan + 16;
     uint32_t* touched = plan + plan_touched_at(experts);
     uint32_t* order = plan + plan_order_at(experts);
@@ -245,15 +256,15 @@ __device__ __forceinline__ void build_plan_wave(uint32_t* count, const uint32_t*
         offsets[e] = run;
         count[e] = run;                                     // LDS now holds the exclusive offsets
         if (c) {
-            touched[trun] = e;
-            items[4U * trun] = e; items[4U * trun + 1U] = run; items[4U * trun + 2U] = run + c; items[4U * trun + 3U] = 0;
-            ++trun;
+            touched[trun++] = e;
+            for (uint32_t b = 0; b < c; b += split, ++irun) {
+                items[4U * irun] = e; items[4U * irun + 1U] = run + b; items[4U * irun + 2U] = run + (b + split < c ? b + split : c); items[4U * irun + 3U] = 0;
+            }
         }
         run += c;
     }
-    const uint32_t bound = plan_item_bound(experts, assignments);
-    for (uint32_t u = touched_total + lane; u < bound; u += 64U) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
-    if (lane == 0) { offsets[experts] = assignments; plan[0] = assignments; plan[1] = touched_total; plan[2] = largest; }
+    for (uint32_t u = items_total + lane; u < item_bound; u += 64U) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
+    if (lane == 0) { offsets[experts] = assignments; plan[0] = assignments; plan[1] = touched_total; plan[2] = largest; plan[4] = items_total; }
     __syncthreads();
     // stable order: the rank of an assignment inside its expert = earlier assignments of the same expert
     for (uint32_t a = lane; a < assignments; a += 64U) {
@@ -339,7 +350,7 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
     if (lane < a.rows) { a.status[lane] = __hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); flags[lane] = 0; }
     if (lane == 0) { *a.job_status = 0; a.plan[3] = 0; }
     __syncthreads();
-    build_plan_wave(count, ids, a.p.experts, assignments, a.plan);
+    build_plan_wave(count, ids, a.p.experts, assignments, a.split, a.item_bound, a.plan);
 }
 
 // softmax / top-k / weights, one row per one-wave block (the plain router).
@@ -351,7 +362,8 @@ __global__ __launch_bounds__(64) void route_select_kernel(RouteArgs a) {
 // ======================================================================================================== expert plan
 // (layout of the plan words: see the router section above)
 
-__global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
+__global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t split,
+                                                    uint32_t item_bound, uint32_t* plan) {
     __shared__ uint32_t count[kRouteMaxExperts + 1];
     const uint32_t tid = threadIdx.x;
     for (uint32_t e = tid; e <= experts; e += 1024U) count[e] = 0;
@@ -362,22 +374,24 @@ __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint
     }
     __syncthreads();
     if (tid == 0) {
-        uint32_t run = 0, touched = 0, largest = 0;
+        uint32_t run = 0, touched = 0, largest = 0, made = 0;
         uint32_t* touched_ids = plan + plan_touched_at(experts);
         uint32_t* items = plan + plan_items_at(experts, assignments);
         for (uint32_t e = 0; e < experts; ++e) {
             const uint32_t c = count[e];
             count[e] = run;
             if (c != 0) {
-                items[4U * touched] = e; items[4U * touched + 1U] = run; items[4U * touched + 2U] = run + c; items[4U * touched + 3U] = 0;
+                for (uint32_t b = 0; b < c; b += split, ++made) {
+                    items[4U * made] = e; items[4U * made + 1U] = run + b; items[4U * made + 2U] = run + (b + split < c ? b + split : c); items[4U * made + 3U] = 0;
+                }
                 touched_ids[touched++] = e;
             }
             run += c;
             largest = c > largest ? c : largest;
         }
-        for (uint32_t u = touched; u < plan_item_bound(experts, assignments); ++u) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
+        for (uint32_t u = made; u < item_bound; ++u) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
         count[experts] = run;
-        plan[0] = assignments; plan[1] = touched; plan[2] = largest;
+        plan[0] = assignments; plan[1] = touched; plan[2] = largest; plan[4] = made;
     }
     __syncthreads();
     uint32_t* offsets = plan + 16;
@@ -413,16 +427,21 @@ __global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* rout
 // same 32-value h group.
 // Reference: src/cpu/core/routed_expert.cpp:403-427 (gate item), :147-170 (swiglu_quantize).
 template <int NA, int DEPTH>
-__device__ __forceinline__ void project_chunk(uint8_t* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
+__device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
                                               const mi355_moe_rows& r, uint32_t grp, const uint32_t* order, uint32_t c0) {
     const uint32_t lane = threadIdx.x & 63U, o = lane & 31U, groups = w.ffn / 32U;
-    uint32_t sidx[NA], src[NA];
+    uint32_t sidx[NA], src[NA], lane_rows[(NA + 3) / 4];
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
         sidx[a] = __builtin_amdgcn_readfirstlane(order[c0 + a]);
         src[a] = sidx[a] / w.top_k;
     }
-    const ActRows<NA> act(A8Image{r.codes, r.deltas, r.sums, w.hidden}, src);
+#pragma unroll
+    for (int h = 0; h < (NA + 3) / 4; ++h) {
+        const uint32_t a = 4U * h + (lane >> 4);
+        lane_rows[h] = order[c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)] / w.top_k;
+    }
+    const ActRows<NA> act(A8Image{r.codes, r.deltas, r.sums, w.hidden}, src, lane_rows);
     float value[NA];
     sweep_rows<NA, DEPTH>(slots, source, w.hidden / 256U, act, value);
 #pragma unroll
@@ -456,22 +475,24 @@ __device__ __forceinline__ void project_chunk(uint8_t* const (&slots)[DEPTH], co
     }
 }
 
-#define STRIX_RING_SLOTS(DEPTH)                                                                  \
-    __shared__ __attribute__((aligned(16))) uint8_t ring0[kStageBytes];                          \
-    __shared__ __attribute__((aligned(16))) uint8_t ring1[kStageBytes];                          \
-    __shared__ __attribute__((aligned(16))) uint8_t ring2[DEPTH > 2 ? kStageBytes : 16];         \
-    __shared__ __attribute__((aligned(16))) uint8_t ring3[DEPTH > 2 ? kStageBytes : 16];         \
-    uint8_t* const ring[4] = {ring0, ring1, ring2, ring3};                                       \
-    uint8_t* slots[DEPTH];                                                                       \
+#define STRIX_RING_SLOTS(DEPTH, NBMAX)                                                           \
+    __shared__ __attribute__((aligned(16))) uint8_t ring0[slot_bytes(NBMAX)];                    \
+    __shared__ __attribute__((aligned(16))) uint8_t ring1[slot_bytes(NBMAX)];                    \
+    __shared__ __attribute__((aligned(16))) uint8_t ring2[DEPTH > 2 ? slot_bytes(NBMAX) : 16];   \
+    __shared__ __attribute__((aligned(16))) uint8_t ring3[DEPTH > 3 ? slot_bytes(NBMAX) : 16];   \
+    lds_u8* const ring[4] = {(lds_u8*)ring0, (lds_u8*)ring1, (lds_u8*)ring2, (lds_u8*)ring3};    \
+    lds_u8* slots[DEPTH];                                                                        \
     _Pragma("unroll") for (int i = 0; i < DEPTH; ++i) slots[i] = ring[i];
 
 // NBMAX = most activation rows sharing one sweep of the weights (4 for routed experts, 8 for a dense matrix).
 template <int NBMAX, int DEPTH>
-__global__ __launch_bounds__(64, DEPTH > 2 ? 1 : 2) void project_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
-    STRIX_RING_SLOTS(DEPTH)
+__global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void project_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    STRIX_RING_SLOTS(DEPTH, NBMAX)
     const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
     const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
     if (begin == end) return;
+    // a wave that serves several activation rows has the longest instruction stream of the launch: let it issue first
+    if (end - begin > 1U) __builtin_amdgcn_s_setprio(3);
     const uint32_t* order = r.plan + plan_order_at(w.experts);
     const uint32_t grp = blockIdx.x;
     const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U) * w.gate_row_stride;
@@ -480,7 +501,7 @@ __global__ __launch_bounds__(64, DEPTH > 2 ? 1 : 2) void project_wave_kernel(mi3
     const uint32_t stride = static_cast<uint32_t>(w.gate_row_stride);
     StageSource source;
     source.init([&](uint32_t row) { return row < 32U ? gate + row * stride : up + (row - 32U) * stride; });
-    uint8_t* const (&sl)[DEPTH] = slots;
+    lds_u8* const (&sl)[DEPTH] = slots;
     for (uint32_t c0 = begin; c0 < end;) {
         const uint32_t left = end - c0, na = left < static_cast<uint32_t>(NBMAX) ? left : static_cast<uint32_t>(NBMAX);
         switch (na) {
@@ -506,12 +527,17 @@ __global__ __launch_bounds__(64, DEPTH > 2 ? 1 : 2) void project_wave_kernel(mi3
 // down rows: one wavefront per (touched expert, 64 hidden outputs), lane = output row.
 // Reference: src/cpu/core/routed_expert.cpp:429-447 (down item), src/moe_a8_down_contract.cpp:146 (Q4_K down row).
 template <int NA, int DEPTH>
-__device__ __forceinline__ void down_chunk(uint8_t* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
+__device__ __forceinline__ void down_chunk(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
                                            const mi355_moe_rows& r, const uint32_t* order, uint32_t c0) {
-    uint32_t src[NA];
+    uint32_t src[NA], lane_rows[(NA + 3) / 4];
 #pragma unroll
     for (int a = 0; a < NA; ++a) src[a] = __builtin_amdgcn_readfirstlane(order[c0 + a]);
-    const ActRows<NA> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src);
+#pragma unroll
+    for (int h = 0; h < (NA + 3) / 4; ++h) {
+        const uint32_t a = 4U * h + ((threadIdx.x & 63U) >> 4);
+        lane_rows[h] = order[c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)];
+    }
+    const ActRows<NA> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src, lane_rows);
     float value[NA];
     sweep_rows<NA, DEPTH>(slots, source, w.ffn / 256U, act, value);
     const uint32_t o = blockIdx.x * 64U + (threadIdx.x & 63U);
@@ -520,18 +546,19 @@ __device__ __forceinline__ void down_chunk(uint8_t* const (&slots)[DEPTH], const
 }
 
 template <int NBMAX, int DEPTH>
-__global__ __launch_bounds__(64, DEPTH > 2 ? 1 : 2) void down_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
-    STRIX_RING_SLOTS(DEPTH)
+__global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    STRIX_RING_SLOTS(DEPTH, NBMAX)
     const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
     const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
     if (begin == end) return;
     if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
+    if (end - begin > 1U) __builtin_amdgcn_s_setprio(3);     // as in the projection: the longest instruction streams issue first
     const uint32_t* order = r.plan + plan_order_at(w.experts);
     const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
     const uint32_t stride = static_cast<uint32_t>(w.down_row_stride);
     StageSource source;
     source.init([&](uint32_t row) { return rows + row * stride; });
-    uint8_t* const (&sl)[DEPTH] = slots;
+    lds_u8* const (&sl)[DEPTH] = slots;
     for (uint32_t c0 = begin; c0 < end;) {
         const uint32_t left = end - c0, na = left < static_cast<uint32_t>(NBMAX) ? left : static_cast<uint32_t>(NBMAX);
         switch (na) {
@@ -614,42 +641,56 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate,
 
 // ======================================================================================================== dispatch
 // Up to 4 (routed experts) or 8 (dense matrix) activation rows share one sweep of an expert's weights; an expert with
-// more assignments is swept again for the rest. The copy ring is 4 stages deep when the launch has too few wavefronts
-// to cover the HBM latency with 2 (few touched experts, or a dense matrix), else 2 to leave LDS for more wavefronts.
+// more assignments is swept again for the rest.
 inline int env_int(const char* name) {
     const char* v = std::getenv(name);
     return v && *v ? std::atoi(v) : 0;
 }
-inline bool deep_ring(uint64_t waves) {
-    static const int env_depth = env_int("STRIX950_DEPTH");   // tuning aid: 2 or 4 overrides the heuristic
-    if (env_depth == 2 || env_depth == 4) return env_depth == 4;
-    return waves < 256U * 5U;
+// Ring depth: the deepest of 4, 3, 2 at which every workgroup of the launch is resident at once (LDS is what limits it).
+inline int ring_depth(uint64_t waves, int nbmax) {
+    static const int env_depth = env_int("STRIX950_DEPTH");   // tuning aid: 2, 3 or 4 overrides the heuristic
+    if (env_depth >= 2 && env_depth <= 4) return env_depth;
+    for (int d = 4; d > 2; --d)
+        if (waves <= 256ULL * (163840U / (static_cast<uint32_t>(d) * slot_bytes(nbmax)))) return d;
+    return 2;
+}
+template <int NBMAX>
+inline void launch_project_nb(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, dim3 grid, hipStream_t st) {
+    switch (ring_depth(static_cast<uint64_t>(grid.x) * grid.y, NBMAX)) {
+    case 4: project_wave_kernel<NBMAX, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    case 3: project_wave_kernel<NBMAX, 3><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    default: project_wave_kernel<NBMAX, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    }
+}
+template <int NBMAX>
+inline void launch_down_nb(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, dim3 grid, hipStream_t st) {
+    switch (ring_depth(static_cast<uint64_t>(grid.x) * grid.y, NBMAX)) {
+    case 4: down_wave_kernel<NBMAX, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    case 3: down_wave_kernel<NBMAX, 3><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    default: down_wave_kernel<NBMAX, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
+    }
 }
 inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     const dim3 grid(w.ffn / 32U, umax);
-    const bool deep = deep_ring(static_cast<uint64_t>(grid.x) * grid.y);
-    if (w.experts == 1U && rows > 4U) {
-        if (deep) project_wave_kernel<8, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-        else project_wave_kernel<8, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-    } else {
-        if (deep) project_wave_kernel<4, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-        else project_wave_kernel<4, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-    }
+    if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
+    else launch_project_nb<4>(w, r, rows, grid, st);
 }
 inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     const dim3 grid(w.hidden / 64U, umax);
-    const bool deep = deep_ring(static_cast<uint64_t>(grid.x) * grid.y);
-    if (w.experts == 1U && rows > 4U) {
-        if (deep) down_wave_kernel<8, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-        else down_wave_kernel<8, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-    } else {
-        if (deep) down_wave_kernel<4, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-        else down_wave_kernel<4, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k);
-    }
+    if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
+    else launch_down_nb<4>(w, r, rows, grid, st);
 }
-inline uint32_t touched_bound(const mi355_moe_weights& w, uint32_t rows) {
-    const uint64_t a = static_cast<uint64_t>(rows) * w.top_k;
-    return static_cast<uint32_t>(a < w.experts ? a : w.experts);
+// An expert's assignments are cut into work items of at most `split` rows: a wave's instruction stream grows with every
+// activation row it serves while its weight stream does not, so wide items finish last; the second read of a split
+// expert's weights comes from the last-level cache. A dense matrix: every row shares one sweep.
+inline uint32_t plan_split(const mi355_moe_weights& w, uint32_t rows) {
+    static const int env_split = env_int("STRIX950_SPLIT");   // tuning aid: 1..4 overrides the heuristic for routed experts
+    if (w.experts == 1U) return 8;
+    if (env_split >= 1 && env_split <= 4) return static_cast<uint32_t>(env_split);
+    return rows <= kFusedMaxRows ? 1U : 4U;
+}
+inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
+    return plan_item_bound(w.experts, rows * w.top_k, plan_split(w, rows));
 }
 
 // ======================================================================================================== admission
@@ -831,7 +872,7 @@ int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_r
 int32_t mi355_moe_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    plan_kernel<<<1, 1024, 0, hs(stream)>>>(r->routes, wv.experts, rows * wv.top_k, r->plan);
+    plan_kernel<<<1, 1024, 0, hs(stream)>>>(r->routes, wv.experts, rows * wv.top_k, plan_split(wv, rows), item_bound(wv, rows), r->plan);
     STRIX_LAUNCHED("moe plan");
     return MI355_OK;
 }
@@ -839,7 +880,7 @@ int32_t mi355_moe_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows* 
 int32_t mi355_moe_enqueue_project(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    launch_project(wv, *r, rows, touched_bound(wv, rows), hs(stream));
+    launch_project(wv, *r, rows, item_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe project");
     return MI355_OK;
 }
@@ -847,7 +888,7 @@ int32_t mi355_moe_enqueue_project(const mi355_moe_weights* w, const mi355_moe_ro
 int32_t mi355_moe_enqueue_down(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    launch_down(wv, *r, rows, touched_bound(wv, rows), hs(stream));
+    launch_down(wv, *r, rows, item_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe down");
     return MI355_OK;
 }
@@ -893,10 +934,11 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     a.wr = router_weight; a.bias = logit_bias; a.ids = ids; a.weights = weights; a.scores = scores;
     a.codes = r->codes; a.deltas = r->deltas; a.sums = r->sums; a.status = r->status; a.job_status = r->job_status; a.plan = r->plan;
     a.quant_blocks = (rows * (wv.hidden / 32U) + 7U) / 8U;
+    a.split = plan_split(wv, rows); a.item_bound = item_bound(wv, rows);
     launch_route_logits(a, hs(stream));
     STRIX_LAUNCHED("moe layer router");
-    launch_project(wv, *r, rows, touched_bound(wv, rows), hs(stream));
-    launch_down(wv, *r, rows, touched_bound(wv, rows), hs(stream));
+    launch_project(wv, *r, rows, item_bound(wv, rows), hs(stream));
+    launch_down(wv, *r, rows, item_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe layer experts");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
