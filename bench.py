@@ -38,6 +38,8 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8)
     ap.add_argument("--layers", type=int, default=6, help="independent layers rotated through (cold-cache working set)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--extra", action="store_true",
+                    help="also time BASELINE configs 1, 2, 4 and 5 (reported under 'extra'; the headline value stays config 3)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy 4 times (a kernel of known HBM traffic, for scaling rocprof FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -91,6 +93,72 @@ class Config3:
     def project_bytes(self, u):
         # gate + up rows of the touched experts, the A8 image read and the h image written
         return u * 2 * self.I * Q4K_ROW(self.H) + self.T * self.H * 1.25 + self.T * self.K * self.I * 1.25
+
+
+def device_q4k(torch, gen, rows_shape, width):
+    """Random Q4_K blocks with finite, moderate fp16 d / dmin (every other bit random) - no fp32 staging tensor needed."""
+    w = torch.randint(0, 256, rows_shape + (width // 256, 144), dtype=torch.uint8, device="cuda", generator=gen)
+    w[..., 1] = (w[..., 1] & 0x13) | 0x0C
+    w[..., 3] = (w[..., 3] & 0x03) | 0x0C
+    return w.reshape(rows_shape + (width // 256 * 144,))
+
+
+def extra_configs(strix, torch, steps, warmup):
+    """BASELINE configs 1, 2, 4, 5 on synthetic full-entropy blocks; HBM-bound ones rotate over enough weight sets to stay cold."""
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    out = {}
+    # config 1: Q8_0 4096 x 4096 GEMV, one fp32 row
+    n = 4096
+    sets = []
+    for _ in range(24):      # 24 x 17.8 MB = 428 MB
+        w = torch.randint(0, 256, (n, n // 32, 34), dtype=torch.uint8, device="cuda", generator=gen)
+        w[..., 1] = (w[..., 1] & 0x03) | 0x14
+        sets.append(w.reshape(n, -1))
+    x = torch.randn((1, n), device="cuda", generator=gen)
+    c, d, _, _ = strix.quantize_a8(x)
+    y = torch.zeros((1, n), device="cuda")
+    sec = time_steps(torch, lambda i: strix.gemv_q8_0_a8(sets[i % len(sets)], c, d, n, n, out=y), steps, warmup)
+    nbytes = n * (n // 32) * 34 + n * 1.125 + n * 4
+    out["config1_q8_0_gemv_4096x4096"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                          "algorithmic_bytes": nbytes}
+    del sets
+    # config 2: dense Q4_K FFN 27648 x 5120, B = 1, 4, 8 (3 rotating weight sets = 717 MB)
+    H, I = 5120, 27648
+    layers = [strix.MoeLayer(H, I, 1, 1, device_q4k(torch, gen, (1, I), H), device_q4k(torch, gen, (1, I), H), device_q4k(torch, gen, (1, H), I), 8, intermediates=True)
+              for _ in range(3)]
+    for B in (1, 4, 8):
+        xb = torch.randn((B, H), device="cuda", generator=gen).to(torch.float16)
+        ids = torch.zeros((B, 1), dtype=torch.int32, device="cuda")
+        w1 = torch.ones((B, 1), dtype=torch.float32, device="cuda")
+        sec = time_steps(torch, lambda i: layers[i % 3].run(xb, ids, w1), max(steps // 4, 10), max(warmup // 4, 3))
+        nbytes = 3 * I * (H // 256) * 144 + B * (H * 2 + H * 4)
+        out[f"config2_dense_q4k_ffn_B{B}"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                              "algorithmic_bytes": nbytes}
+    del layers
+    # config 5: expert-TP rank 0 of 2, 16 rows, hidden 6144, 160 experts top-8, intermediate 2560 / 2
+    H, I, E, K, T = 6144, 2560, 160, 8, 16
+    grb, drb = H // 256 * 144, I // 256 * 144
+    layer = strix.MoeLayer(H, I // 2, E, K, device_q4k(torch, gen, (E, I), H), device_q4k(torch, gen, (E, I), H), device_q4k(torch, gen, (E, H), I), T,
+                           gate_expert_stride=I * grb, gate_row_stride=grb, down_expert_stride=H * drb, down_row_stride=drb)
+    wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
+    xs = [torch.randn((T, H), device="cuda", generator=gen).to(torch.float16) for _ in range(4)]
+    sec = time_steps(torch, lambda i: layer.run_layer(xs[i % 4], wr, combine=strix.COMBINE_MULADD_ASC), max(steps // 4, 10), max(warmup // 4, 3))
+    u = statistics.mean(int(torch.unique(strix.route(xv, wr, K)[0]).numel()) for xv in xs)
+    nbytes = u * 3 * (I // 2) * grb + E * H * 4 + T * H * 6
+    out["config5_tp_rank_shard_T16"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                        "algorithmic_bytes": nbytes, "distinct_experts_mean": u}
+    del layer
+    # config 4: 4096-row prefill, hidden 4096, 256 experts top-8 (+ logit bias), intermediate 2048; routed experts + router
+    H, I, E, K, T = 4096, 2048, 256, 8, 4096
+    layer = strix.MoeLayer(H, I, E, K, device_q4k(torch, gen, (E, I), H), device_q4k(torch, gen, (E, I), H), device_q4k(torch, gen, (E, H), I), T)
+    wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
+    bias = torch.randn(E, device="cuda", generator=gen) * 1.5
+    xp = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)
+    sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 3, 1)
+    flops = 2.0 * T * K * 3 * I * H + 2.0 * T * E * H
+    out["config4_prefill_T4096"] = {"ms": sec * 1e3, "TFLOPs": flops / sec / 1e12, "frac_of_fp16_mfma_peak": flops / sec / 2.5e15,
+                                    "algorithmic_flops": flops, "note": "routed experts + router; A8 integer-dot class on the decode kernels (no MFMA path yet)"}
+    return out
 
 
 def time_steps(torch, fn, steps, warmup):
@@ -183,6 +251,9 @@ def main():
                      "traffic": PROJECT_TRAFFIC_BYTES_DEFAULT if (args.tokens, args.layers) == (8, 6) else None,
                      "algorithmic_bytes_per_launch": cfg.project_bytes(u_mean), "avg_launch_us": kernel_us["project"]},
     }
+    if args.extra:
+        del cfg.layers[1:]
+        out["extra"] = extra_configs(strix, torch, args.steps, args.warmup)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_config3(cfg)
     else:

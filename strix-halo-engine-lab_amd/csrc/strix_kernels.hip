@@ -12,6 +12,7 @@
 
 #include "device_math.hpp"
 #include "q4k_rows.hpp"
+#include "q4k_pairs.hpp"
 #include "route_wave.hpp"
 
 namespace strix950 {
@@ -614,7 +615,8 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, mi355_m
 
 // SwiGLU + A8 re-quantisation of dense gate/up rows. Reference: src/cpu/core/routed_expert.cpp:147-170.
 __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate, const float* up, uint32_t ffn, uint32_t exp_kind,
-                                                              int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status) {
+                                                              int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
+                                                              uint32_t* job_status) {
     const uint32_t row = blockIdx.y, groups = ffn / 32U, grp = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U;
     if (grp >= groups) return;
     const size_t at = static_cast<size_t>(row) * ffn + grp * 32U + l;
@@ -625,6 +627,7 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate,
     const int bad = or32_i((finite_f(g) && finite_f(u) && finite_f(hv)) ? 0 : 1);
     if (bad) {
         if (l == 0 && status) atomicOr(&status[row], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+        if (l == 0 && job_status) atomicOr(job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
         return;
     }
     const float amax = max32(__builtin_fabsf(hv));
@@ -670,12 +673,56 @@ inline void launch_down_nb(const mi355_moe_weights& w, const mi355_moe_rows& r, 
     default: down_wave_kernel<NBMAX, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
     }
 }
+// ---- dense matrix (one expert, every row uses it): the pair-per-lane sweep ------------------------------------------
+template <int NA, int AL>
+inline void launch_pairs_depth(const PairArgs& a, uint32_t matrices, hipStream_t st) {
+    const dim3 grid(a.rows / pair_rows<AL>(), matrices);
+    const uint64_t waves = static_cast<uint64_t>(grid.x) * grid.y;
+    // 4 slots when every wavefront of the launch is resident with them and the wait counter can express 3 stages ahead
+    const bool deep = 3U * pair_copies<NA, AL>() <= 63U && waves <= 256ULL * (163840U / (4U * pair_slot_bytes<NA, AL>()));
+    if (deep) q4k_pairs_kernel<NA, AL, 4><<<grid, 64, 0, st>>>(a);
+    else q4k_pairs_kernel<NA, AL, 2><<<grid, 64, 0, st>>>(a);
+}
+// nacts <= 8 activation rows. Matrices with few rows spread every row over two activation lanes when there are >= 4 rows
+// of activations, which doubles the wavefronts and halves each one's instruction stream.
+inline void launch_pairs(const PairArgs& a, uint32_t matrices, hipStream_t st) {
+    const bool narrow = static_cast<uint64_t>(a.rows) * matrices < 16384U;
+    if (a.nacts <= 1U) launch_pairs_depth<1, 1>(a, matrices, st);
+    else if (a.nacts <= 2U) launch_pairs_depth<2, 1>(a, matrices, st);
+    else if (a.nacts <= 4U) { if (narrow) launch_pairs_depth<2, 2>(a, matrices, st); else launch_pairs_depth<4, 1>(a, matrices, st); }
+    else { if (narrow) launch_pairs_depth<4, 2>(a, matrices, st); else launch_pairs_depth<8, 1>(a, matrices, st); }
+}
+// The dense form needs fp32 gate / up rows as workspace (the optional intermediates views) because a wavefront holds
+// 16 rows, not a whole 32-output SwiGLU group.
+inline bool dense_pairs_ok(const mi355_moe_weights& w, uint32_t rows) {
+    return w.experts == 1U && w.top_k == 1U && rows <= 8U && (w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0 &&
+           w.gate_row_stride < (1ULL << 24) && w.down_row_stride < (1ULL << 24);
+}
+inline void launch_project_dense(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, hipStream_t st) {
+    PairArgs a{};
+    a.m[0] = PairMatrix{w.gate, w.gate_row_stride, r.gate_out, w.ffn};
+    a.m[1] = PairMatrix{w.up, w.gate_row_stride, r.up_out, w.ffn};
+    a.rows = w.ffn; a.blocks = w.hidden / 256U; a.img = A8Image{r.codes, r.deltas, r.sums, w.hidden}; a.nacts = rows;
+    launch_pairs(a, 2, st);
+    swiglu_quantize_kernel<<<dim3((w.ffn / 32U + 7U) / 8U, rows), 256, 0, st>>>(r.gate_out, r.up_out, w.ffn, w.exp_kind, r.down_codes, r.down_deltas,
+                                                                                r.down_sums, r.h_out, r.status, r.job_status);
+}
+inline void launch_down_dense(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, hipStream_t st) {
+    PairArgs a{};
+    a.m[0] = PairMatrix{w.down, w.down_row_stride, r.rawdots, w.hidden};
+    a.rows = w.hidden; a.blocks = w.ffn / 256U; a.img = A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}; a.nacts = rows;
+    a.skip_flag = r.job_status; a.skip_mask = MI355_STATUS_NONFINITE_PROJECTION;
+    launch_pairs(a, 1, st);
+}
+
 inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+    if (dense_pairs_ok(w, rows) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
     const dim3 grid(w.ffn / 32U, umax);
     if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
     else launch_project_nb<4>(w, r, rows, grid, st);
 }
 inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+    if (dense_pairs_ok(w, rows)) return launch_down_dense(w, r, rows, st);
     const dim3 grid(w.hidden / 64U, umax);
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
     else launch_down_nb<4>(w, r, rows, grid, st);
@@ -909,7 +956,9 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, u
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
     STRIX_REQUIRE(r->input && r->input_kind <= MI355_INPUT_BF16, "moe: input view invalid");
     if (const int32_t rc = mi355_moe_enqueue_prologue(w, r, rows, stream)) return rc;
-    if (const int32_t rc = mi355_moe_enqueue_csr(w, r, rows, stream)) return rc;
+    // a dense matrix on the pair-per-lane sweep reads no expert plan
+    if (!(dense_pairs_ok(wv, rows) && r->gate_out && r->up_out))
+        if (const int32_t rc = mi355_moe_enqueue_csr(w, r, rows, stream)) return rc;
     if (const int32_t rc = mi355_moe_enqueue_project(w, r, rows, stream)) return rc;
     if (const int32_t rc = mi355_moe_enqueue_down(w, r, rows, stream)) return rc;
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
@@ -950,7 +999,7 @@ int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows,
     if (rows == 0 || ffn == 0) return MI355_OK;
     STRIX_REQUIRE(gate && up && codes && deltas && sums, "swiglu: null pointer");
     STRIX_REQUIRE(rows <= 65535U, "swiglu: at most 65535 rows per call");
-    swiglu_quantize_kernel<<<dim3((ffn / 32U + 7U) / 8U, rows), 256, 0, hs(stream)>>>(gate, up, ffn, exp_kind, codes, deltas, sums, h_out, status);
+    swiglu_quantize_kernel<<<dim3((ffn / 32U + 7U) / 8U, rows), 256, 0, hs(stream)>>>(gate, up, ffn, exp_kind, codes, deltas, sums, h_out, status, nullptr);
     STRIX_LAUNCHED("swiglu_quantize");
     return MI355_OK;
 }
