@@ -154,10 +154,21 @@ def extra_configs(strix, torch, steps, warmup):
     wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
     bias = torch.randn(E, device="cuda", generator=gen) * 1.5
     xp = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)
-    sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 3, 1)
-    flops = 2.0 * T * K * 3 * I * H + 2.0 * T * E * H
-    out["config4_prefill_T4096"] = {"ms": sec * 1e3, "TFLOPs": flops / sec / 1e12, "frac_of_fp16_mfma_peak": flops / sec / 2.5e15,
-                                    "algorithmic_flops": flops, "note": "routed experts + router; A8 integer-dot class on the decode kernels (no MFMA path yet)"}
+    layer = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, T, prefill_f16=True)
+    flops_experts, flops_router = 2.0 * T * K * 3 * I * H, 2.0 * T * E * H
+    ids, wts, _ = strix.route(xp, wr, K, bias=bias)
+    sec_route = time_steps(torch, lambda i: strix.route(xp, wr, K, bias=bias), 5, 2)
+    sec_f16 = time_steps(torch, lambda i: layer.run_prefill_f16(xp, ids, wts), 10, 3)
+    out["config4_prefill_T4096_f16_mfma"] = {
+        "ms": (sec_f16 + sec_route) * 1e3, "experts_ms": sec_f16 * 1e3, "router_ms": sec_route * 1e3,
+        "TFLOPs": (flops_experts + flops_router) / (sec_f16 + sec_route) / 1e12, "experts_TFLOPs": flops_experts / sec_f16 / 1e12,
+        "frac_of_fp16_mfma_peak": (flops_experts + flops_router) / (sec_f16 + sec_route) / 2.5e15,
+        "experts_frac_of_fp16_mfma_peak": flops_experts / sec_f16 / 2.5e15, "algorithmic_flops": flops_experts + flops_router,
+        "note": "routed experts on fp16 MFMA (weights as fp16 hi + lo, fp32 accumulation) + exact-order router; FAST class, tolerance 2e-3"}
+    sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 2, 1)
+    out["config4_prefill_T4096_integer_class"] = {
+        "ms": sec * 1e3, "TFLOPs": (flops_experts + flops_router) / sec / 1e12, "algorithmic_flops": flops_experts + flops_router,
+        "note": "same work in the bit-exact integer-dot class on the decode kernels (router included)"}
     return out
 
 

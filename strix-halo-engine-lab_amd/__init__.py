@@ -52,7 +52,7 @@ class MoeRows(C.Structure):
                 ("gate_out", C.c_void_p), ("up_out", C.c_void_p), ("h_out", C.c_void_p),
                 ("down_codes", C.c_void_p), ("down_deltas", C.c_void_p), ("down_sums", C.c_void_p),
                 ("rawdots", C.c_void_p), ("base", C.c_void_p), ("output", C.c_void_p), ("output_stride", C.c_uint64),
-                ("plan", C.c_void_p), ("job_status", C.c_void_p)]
+                ("plan", C.c_void_p), ("job_status", C.c_void_p), ("h_f16", C.c_void_p)]
 
 
 _lib = None
@@ -78,7 +78,7 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_prefill_f16",
            "mi355_swiglu_quantize"]
 
 
@@ -176,7 +176,7 @@ class MoeLayer:
     Rows / Weights bundle, include/strix/cuda/qwen_moe.hpp:55-93)."""
 
     def __init__(self, hidden, ffn, experts, top_k, gate, up, down, max_rows, exp_kind=EXP_GFX1151, intermediates=False,
-                 gate_expert_stride=0, gate_row_stride=0, down_expert_stride=0, down_row_stride=0):
+                 gate_expert_stride=0, gate_row_stride=0, down_expert_stride=0, down_row_stride=0, prefill_f16=False):
         dev = gate.device
         self.hidden, self.ffn, self.experts, self.top_k, self.max_rows = hidden, ffn, experts, top_k, max_rows
         self.gate, self.up, self.down = gate, up, down
@@ -193,6 +193,7 @@ class MoeLayer:
         self.up_out = z((n, ffn), torch.float32) if intermediates else None
         self.h_out = z((n, ffn), torch.float32) if intermediates else None
         self.plan = z(int(lib().mi355_moe_plan_words(experts, max_rows, top_k)), torch.int32)
+        self.h_f16 = z((n, ffn), torch.float16) if prefill_f16 else None      # workspace of the fp16 MFMA prefill form
 
     def rows_view(self, x, ids, weights, base=None):
         rows = x.shape[0]
@@ -203,11 +204,17 @@ class MoeLayer:
                              _p(self.gate_out).value or 0, _p(self.up_out).value or 0, _p(self.h_out).value or 0,
                              self.down_codes.data_ptr(), self.down_deltas.data_ptr(), self.down_sums.data_ptr(),
                              self.rawdots.data_ptr(), 0 if base is None else base.data_ptr(), self.output.data_ptr(), self.hidden,
-                             self.plan.data_ptr(), self.job_status.data_ptr())
+                             self.plan.data_ptr(), self.job_status.data_ptr(), _p(self.h_f16).value or 0)
 
     def run(self, x, ids, weights, base=None, combine=COMBINE_FMA_SLOT):
         rows, rv = self.rows_view(x, ids, weights, base)
         check(lib().mi355_moe_enqueue(C.byref(self.w), C.byref(rv), rows, combine, _stream()))
+        return self.output[:rows]
+
+    def run_prefill_f16(self, x, ids, weights, base=None, combine=COMBINE_FMA_SLOT):
+        """The routed experts on the matrix cores (fp16 weights x fp16 rows, fp32 accumulation): mi355_moe_enqueue_prefill_f16."""
+        rows, rv = self.rows_view(x, ids, weights, base)
+        check(lib().mi355_moe_enqueue_prefill_f16(C.byref(self.w), C.byref(rv), rows, combine, _stream()))
         return self.output[:rows]
 
     def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,

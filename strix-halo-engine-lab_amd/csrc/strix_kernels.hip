@@ -13,6 +13,7 @@
 #include "device_math.hpp"
 #include "q4k_rows.hpp"
 #include "q4k_pairs.hpp"
+#include "prefill_f16.hpp"
 #include "route_wave.hpp"
 
 namespace strix950 {
@@ -363,8 +364,24 @@ __global__ __launch_bounds__(64) void route_select_kernel(RouteArgs a) {
 // ======================================================================================================== expert plan
 // (layout of the plan words: see the router section above)
 
+// Stable order of a large batch: one wave per expert walks the assignments in order, 64 at a time, and places its own by
+// ballot + prefix count (the offsets are already in the plan).
+__global__ __launch_bounds__(64) void plan_order_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
+    const uint32_t e = blockIdx.x, lane = threadIdx.x;
+    uint32_t at = plan[16 + e];
+    const uint32_t end = plan[16 + e + 1];
+    uint32_t* order = plan + plan_order_at(experts);
+    for (uint32_t a0 = 0; a0 < assignments && at < end; a0 += 64U) {
+        const uint32_t a = a0 + lane;
+        const bool mine = a < assignments && routes[a] == e;
+        const uint64_t votes = __ballot(mine);
+        if (mine) order[at + __popcll(votes & ((1ULL << lane) - 1ULL))] = a;
+        at += static_cast<uint32_t>(__popcll(votes));
+    }
+}
+
 __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t split,
-                                                    uint32_t item_bound, uint32_t* plan) {
+                                                    uint32_t item_bound, uint32_t fill_order, uint32_t* plan) {
     __shared__ uint32_t count[kRouteMaxExperts + 1];
     const uint32_t tid = threadIdx.x;
     for (uint32_t e = tid; e <= experts; e += 1024U) count[e] = 0;
@@ -398,6 +415,7 @@ __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint
     uint32_t* offsets = plan + 16;
     uint32_t* order = plan + plan_order_at(experts);
     for (uint32_t e = tid; e <= experts; e += 1024U) offsets[e] = count[e];
+    if (!fill_order) return;                  // large batches: plan_order_kernel follows
     for (uint32_t e = tid; e < experts; e += 1024U) {
         const uint32_t end = e + 1 <= experts ? count[e + 1] : 0;
         uint32_t at = count[e];
@@ -715,6 +733,12 @@ inline void launch_down_dense(const mi355_moe_weights& w, const mi355_moe_rows& 
     launch_pairs(a, 1, st);
 }
 
+inline void launch_plan(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t split, uint32_t bound, uint32_t* plan,
+                        hipStream_t st) {
+    const bool large = assignments > 4096U;
+    plan_kernel<<<1, 1024, 0, st>>>(routes, experts, assignments, split, bound, large ? 0U : 1U, plan);
+    if (large) plan_order_kernel<<<experts, 64, 0, st>>>(routes, experts, assignments, plan);
+}
 inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     if (dense_pairs_ok(w, rows) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
     const dim3 grid(w.ffn / 32U, umax);
@@ -919,7 +943,7 @@ int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_r
 int32_t mi355_moe_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    plan_kernel<<<1, 1024, 0, hs(stream)>>>(r->routes, wv.experts, rows * wv.top_k, plan_split(wv, rows), item_bound(wv, rows), r->plan);
+    launch_plan(r->routes, wv.experts, rows * wv.top_k, plan_split(wv, rows), item_bound(wv, rows), r->plan, hs(stream));
     STRIX_LAUNCHED("moe plan");
     return MI355_OK;
 }
@@ -989,6 +1013,33 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     launch_project(wv, *r, rows, item_bound(wv, rows), hs(stream));
     launch_down(wv, *r, rows, item_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe layer experts");
+    return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+}
+
+int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe prefill: unknown combine form");
+    STRIX_REQUIRE(r->input && r->input_kind == MI355_INPUT_F16, "moe prefill: the fp16 form takes fp16 input rows");
+    STRIX_REQUIRE(r->input_stride % 16U == 0 && aligned(r->input, 16), "moe prefill: input rows must be 16-byte aligned");
+    STRIX_REQUIRE(r->h_f16 && aligned(r->h_f16, 16), "moe prefill: h_f16 workspace is null or misaligned");
+    STRIX_REQUIRE(rows <= 65535U, "moe prefill: at most 65535 rows per call");
+    const uint32_t assignments = rows * wv.top_k, bound = plan_item_bound(wv.experts, assignments, kPfTile);
+    STRIX_REQUIRE(bound <= 65535U, "moe prefill: too many work items for one launch");
+    hipStream_t st = hs(stream);
+    clear_validate_kernel<<<rows, 64, 0, st>>>(r->routes, r->route_weights, wv.experts, wv.top_k, r->status, r->job_status);
+    launch_plan(r->routes, wv.experts, assignments, kPfTile, bound, r->plan, st);
+    PrefillArgs a{};
+    a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.x = static_cast<const uint8_t*>(r->input); a.x_stride = r->input_stride;
+    a.h = static_cast<_Float16*>(r->h_f16); a.rawdots = r->rawdots; a.plan = r->plan; a.experts = wv.experts; a.assignments = assignments;
+    a.status = r->status; a.job_status = r->job_status;
+    const uint32_t items_at = plan_items_at(wv.experts, assignments), order_at = plan_order_at(wv.experts);
+    a.wa = wv.gate; a.wb = wv.up; a.expert_stride = wv.gate_expert_stride; a.row_stride = wv.gate_row_stride; a.k = wv.hidden; a.features = wv.ffn;
+    prefill_f16_kernel<0><<<dim3(wv.ffn / 64U, bound), 256, 0, st>>>(a, items_at, order_at);
+    a.wa = wv.down; a.wb = nullptr; a.expert_stride = wv.down_expert_stride; a.row_stride = wv.down_row_stride; a.k = wv.ffn; a.features = wv.hidden;
+    STRIX_REQUIRE(wv.hidden % 128U == 0, "moe prefill: hidden must be a multiple of 128");
+    prefill_f16_kernel<1><<<dim3(wv.hidden / 128U, bound), 256, 0, st>>>(a, items_at, order_at);
+    STRIX_LAUNCHED("moe prefill f16");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
 

@@ -405,3 +405,47 @@ def test_admission_failures_return_before_any_enqueue(strix):
     layer.w.down_type = 12
     torch.cuda.synchronize()
     assert bool((layer.output == 5.0).all())
+
+
+# ------------------------------------------------------------------------------------------- prefill on the matrix cores
+def exact_weight_layer(x, ids, wts, gate, up, down, H, I, K, base=None):
+    """Exact-weight (BASE class) evaluation of the routed experts in float64 from the decoder's fp32 weights."""
+    T = x.shape[0]
+    raw = np.zeros((T, K, H), np.float32)
+    x64 = x.astype(np.float64)
+    for e in np.unique(ids):
+        wg = orc.dequant_rows(orc.Q4_K, gate[e], H).astype(np.float64)
+        wu = orc.dequant_rows(orc.Q4_K, up[e], H).astype(np.float64)
+        wd = orc.dequant_rows(orc.Q4_K, down[e], I).astype(np.float64)
+        rows, slots = np.nonzero(ids == e)
+        g, u = x64[rows] @ wg.T, x64[rows] @ wu.T
+        h = (g / (1.0 + np.exp(-g))) * u
+        raw[rows, slots] = (h @ wd.T).astype(np.float32)
+    return orc.combine(0, wts, ids, raw, base=base), raw
+
+
+@pytest.mark.parametrize("H,I,E,K,T", [(512, 256, 6, 2, 300), (1024, 512, 12, 4, 77), (256, 256, 3, 1, 129)])
+def test_prefill_f16_mfma_matches_exact_weight_product(strix, H, I, E, K, T):
+    """The fp16 MFMA prefill form against the exact-weight product: tolerance 2e-3 (fp16 activations), both as max abs
+    error over the output rms and elementwise on the outputs of at least rms size; the gate / up / down tiles are checked
+    through the unweighted down outputs as well as the combined output. One dense projection is also tied to the oracle's BASE-class
+    routine (lane-strided fp32 sums) so that the float64 reference and the oracle agree on what "exact weight" means."""
+    rng = np.random.default_rng(H + T)
+    gate, up, down = make_layer(rng, H, I, E)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, prefill_f16=True)
+    y = layer.run_prefill_f16(dev(x), dev(ids_ref.astype(np.int32)), dev(w_ref)).cpu().numpy()
+    want, raw_ref = exact_weight_layer(x, ids_ref, w_ref, gate, up, down, H, I, K)
+    for got, ref in ((layer.rawdots[:T].cpu().numpy(), raw_ref), (y, want)):
+        ref64 = ref.astype(np.float64)
+        rms = np.sqrt(np.mean(ref64 ** 2))
+        assert np.max(np.abs(got - ref64)) / rms < TOL_F16                       # max abs error over the output rms
+        big = np.abs(ref64) >= rms                                               # elementwise relative error of the rms-sized outputs
+        assert np.max(np.abs(got[big] - ref64[big]) / np.abs(ref64[big])) < TOL_F16
+    assert np.all(layer.status[:T].cpu().numpy() == 0)
+    e0 = int(ids_ref[0, 0])
+    g_oracle = orc.base_linear(orc.Q4_K, gate[e0], H // 256 * 144, I, H, x[:4].astype(np.float32))
+    g64 = x[:4].astype(np.float64) @ orc.dequant_rows(orc.Q4_K, gate[e0], H).astype(np.float64).T
+    assert rel_err(g_oracle, g64.astype(np.float32))[0] < 1e-5
