@@ -137,6 +137,96 @@ __device__ __forceinline__ void route_logits_block(RouteLds& lds, const RouteArg
     __syncthreads();
 }
 
+// ---------------------------------------------------------------------------------------------------- batch chains
+// Logits of large batches (the ascending fma chain form): throughput, not latency. A 256-thread workgroup owns 64 rows x
+// 64 experts; a lane runs 4 x 4 independent chains (rows lr + 8 i, experts lc + 8 j of its wave's 32 x 32 quarter), so
+// sixteen fmas separate two steps of the same chain and every pair of 128-bit LDS reads feeds 16 fmas. The tiles of 64
+// features (activations widened to fp32 once) are register-staged one step ahead and double-buffered in LDS.
+constexpr uint32_t kBatchTile = 64, kBatchStep = 64, kBatchPitch = kBatchStep + 4;     // floats; +16 bytes spreads the rows over the banks
+struct BatchTiles { float w[2][kBatchTile][kBatchPitch]; float x[2][kBatchTile][kBatchPitch]; };     // 69,632 bytes
+
+template <int KIND>
+__device__ __forceinline__ void route_batch_block(BatchTiles& lds, const RouteArgs& a, uint32_t r0, uint32_t e0) {
+    const uint32_t t = threadIdx.x, lane = t & 63U, wave = t >> 6;
+    const uint32_t lrow = t >> 2, quarter = t & 3U;                    // loader role: tile row t / 4, 16 features
+    const uint32_t le = e0 + lrow < a.p.experts ? e0 + lrow : a.p.experts - 1U;
+    const uint32_t lr = r0 + lrow < a.rows ? r0 + lrow : a.rows - 1U;
+    const float* wsrc = a.wr + static_cast<size_t>(le) * a.hidden + 16U * quarter;
+    const uint8_t* xsrc = a.x + lr * a.x_stride + (KIND == 0 ? 64U : 32U) * quarter;
+    const uint32_t steps = (a.hidden + kBatchStep - 1U) / kBatchStep;
+    f32x4 wreg[4];
+    u32x4 xreg[KIND == 0 ? 4 : 2];
+    auto fetch = [&](uint32_t s) {
+        // the last step of a row whose length is 32 mod 64: quarters 2, 3 re-read valid features (never used)
+        const uint32_t k = s * kBatchStep, back = (k + 16U * quarter + 16U <= a.hidden) ? 0U : 32U;
+        const float* ws = wsrc + k - back;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wreg[i] = *reinterpret_cast<const f32x4*>(ws + 4 * i);
+        const uint8_t* xs = xsrc + static_cast<size_t>(k - back) * (KIND == 0 ? 4U : 2U);
+#pragma unroll
+        for (int i = 0; i < (KIND == 0 ? 4 : 2); ++i) xreg[i] = *reinterpret_cast<const u32x4*>(xs + 16 * i);
+    };
+    auto stage = [&](uint32_t buf) {
+        float* wd = &lds.w[buf][lrow][16U * quarter];
+        float* xd = &lds.x[buf][lrow][16U * quarter];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4*>(wd + 4 * i) = wreg[i];
+        if constexpr (KIND == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(xd + 4 * i) = xreg[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const uint32_t h[4] = {xreg[i].x, xreg[i].y, xreg[i].z, xreg[i].w};
+                float f[8];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (KIND == 1) { f[2 * q] = half_bits_to_float(h[q] & 0xffffU); f[2 * q + 1] = half_bits_to_float(h[q] >> 16); }
+                    else { f[2 * q] = f_of(h[q] << 16); f[2 * q + 1] = f_of(h[q] & 0xffff0000U); }
+                }
+                *reinterpret_cast<f32x4*>(xd + 8 * i) = f32x4{f[0], f[1], f[2], f[3]};
+                *reinterpret_cast<f32x4*>(xd + 8 * i + 4) = f32x4{f[4], f[5], f[6], f[7]};
+            }
+        }
+    };
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.0F;
+    const uint32_t qr = 32U * (wave >> 1) + (lane >> 3), qe = 32U * (wave & 1U) + (lane & 7U);     // the lane's first row / expert in the tile
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (uint32_t s = 0; s < steps; ++s) {
+        const uint32_t buf = s & 1U;
+        if (s + 1U < steps) fetch(s + 1U);
+        const uint32_t kc = a.hidden - s * kBatchStep < kBatchStep ? a.hidden - s * kBatchStep : kBatchStep;
+        for (uint32_t k = 0; k < kc; k += 4U) {
+            f32x4 xv[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xv[i] = *reinterpret_cast<const f32x4*>(&lds.x[buf][qr + 8 * i][k]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[j] = *reinterpret_cast<const f32x4*>(&lds.w[buf][qe + 8 * j][k]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(xv[i][c], wv[j][c], acc[i][j]);
+        }
+        if (s + 1U < steps) stage(buf ^ 1U);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t r = r0 + qr + 8U * i, e = e0 + qe + 8U * j;
+            if (r < a.rows && e < a.p.experts) a.scores[static_cast<size_t>(r) * a.p.experts + e] = a.bias ? acc[i][j] + a.bias[e] : acc[i][j];
+        }
+}
+
 // ---------------------------------------------------------------------------------------------------- decode chains
 // Decode batches (rows <= 16): one wavefront per (row, 8 experts). The chain of `hidden` dependent fmas is the whole
 // cost (about 6 cycles per step), so everything else is taken off its path: the 8 router-weight rows and the activation

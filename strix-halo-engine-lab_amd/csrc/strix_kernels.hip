@@ -285,6 +285,13 @@ __global__ __launch_bounds__(64) void route_logits_kernel(RouteArgs a) {
     route_logits_block<KIND>(lds, a, (blockIdx.x % neb) * 8U, (blockIdx.x / neb) * 8U);
 }
 
+// Router logits of large batches in the ascending fma chain order: 64 rows x 64 experts per 256-thread workgroup.
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void route_batch_kernel(RouteArgs a) {
+    __shared__ __attribute__((aligned(16))) BatchTiles lds;
+    route_batch_block<KIND>(lds, a, blockIdx.y * kBatchTile, blockIdx.x * kBatchTile);
+}
+
 // Decode router launch (rows <= 16). Blocks [0, route_blocks) run the logit chains of (row, 8 experts). In the plain form
 // (a.plan == nullptr) the kernel stops there. In the fused form blocks [route_blocks, route_blocks + quant_blocks)
 // quantise the input rows to A8 (8 groups of 32 per block); the block that finishes a row's last 8 experts (row ticket)
@@ -905,6 +912,11 @@ void launch_route_logits(RouteArgs& a, hipStream_t st) {
         if (a.kind == MI355_INPUT_F32) route_decode_kernel<0><<<blocks, 64, 0, st>>>(a);
         else if (a.kind == MI355_INPUT_F16) route_decode_kernel<1><<<blocks, 64, 0, st>>>(a);
         else route_decode_kernel<2><<<blocks, 64, 0, st>>>(a);
+    } else if (a.p.logits_order == MI355_LOGITS_FMA_ASCENDING && (a.rows + kBatchTile - 1U) / kBatchTile <= 65535U) {
+        const dim3 grid((a.p.experts + kBatchTile - 1U) / kBatchTile, (a.rows + kBatchTile - 1U) / kBatchTile);
+        if (a.kind == MI355_INPUT_F32) route_batch_kernel<0><<<grid, 256, 0, st>>>(a);
+        else if (a.kind == MI355_INPUT_F16) route_batch_kernel<1><<<grid, 256, 0, st>>>(a);
+        else route_batch_kernel<2><<<grid, 256, 0, st>>>(a);
     } else {
         a.route_blocks = neb * ((a.rows + 7U) / 8U);
         if (a.kind == MI355_INPUT_F32) route_logits_kernel<0><<<a.route_blocks, 64, 0, st>>>(a);
