@@ -12,8 +12,11 @@
 // weight rows x tokens, K walked in steps of 64 (one pair of Q4_K sub-blocks: the 32 quant bytes whose low / high nibbles
 // are sub-blocks 2p / 2p + 1). Per step every thread fetches 16 quant bytes + the block header of one weight row and 64
 // bytes of one token row into registers (one step ahead of the arithmetic), dequantises its 32 weights and stores the
-// tiles row-major [row][k] (pitch 144 bytes: conflict-free 128-bit reads) in LDS (weights hi, weights lo, tokens: 54 KB,
-// two workgroups per CU). Each of the 4 waves multiplies all 128 weight rows with its own 32 tokens: 32 MFMAs per step.
+// tiles row-major [row][k] (pitch 144 bytes: conflict-free 128-bit reads) in LDS (weights hi, weights lo, tokens).
+// The workgroup has 8 waves in two roles: waves 0-3 are the loaders just described, waves 4-7 each multiply a 64 x 64
+// quarter of the tile (2 x 2 MFMA tiles: every operand read from LDS feeds two MFMAs; 32 MFMAs per step). Tile rows are
+// ordered [gate 0-31, up 0-31, gate 32-63, up 32-63] so that a wave holds gate and up of the same features. The LDS tiles are double-buffered and there is one barrier per
+// step, so the loaders prepare step s + 1 (VALU) while the multipliers run step s (matrix cores) on the same SIMDs.
 //
 // Weights are read from HBM once per (item, feature tile); with ~128 rows per item the arithmetic intensity is ~450
 // flop per weight byte, above the machine balance, so the kernel is bound by the matrix cores and the dequantisation
@@ -55,24 +58,31 @@ __device__ __forceinline__ uint32_t pack_half2(float a, float b) {
 struct PfRaw { u32x4 hd, qs, x[4]; };
 
 template <int MODE>
-__global__ __launch_bounds__(256, 2) void prefill_f16_kernel(PrefillArgs a, uint32_t items_at, uint32_t order_at) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile_a[2][kPfTileBytes];     // [0]: w_hi, [1]: w_lo
-    __shared__ __attribute__((aligned(16))) uint8_t tile_b[kPfTileBytes];
+__global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_t items_at, uint32_t order_at) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile_a[2][2][kPfTileBytes];     // [buffer][0: w_hi, 1: w_lo]
+    __shared__ __attribute__((aligned(16))) uint8_t tile_b[2][kPfTileBytes];
     const uint4 item = *reinterpret_cast<const uint4*>(a.plan + items_at + 4U * blockIdx.y);
     const uint32_t e = item.x, begin = item.y, count = item.z - item.y;
     if (count == 0) return;
     if (MODE == 1 && (*a.job_status & MI355_STATUS_NONFINITE_PROJECTION)) return;
     const uint32_t* order = a.plan + order_at;
-    const uint32_t t = threadIdx.x, lane = t & 63U, wave = t >> 6;
+    const bool loader = threadIdx.x < 256U;
+    const uint32_t t = threadIdx.x & 255U, lane = t & 63U, wave = t >> 6;      // index within the role
     // loader role: thread t owns weight row t / 2 of the tile and token t / 2, half = which 16 quant bytes / 32 features
     const uint32_t lrow = t >> 1, half = t & 1U;
     const uint32_t m0 = blockIdx.x * (MODE == 0 ? 64U : 128U);
-    const uint8_t* wbase = (MODE == 0 && lrow >= 64U) ? a.wb : a.wa;
-    const uint8_t* wrow = wbase + static_cast<size_t>(e) * a.expert_stride + static_cast<size_t>(m0 + (MODE == 0 ? (lrow & 63U) : lrow)) * a.row_stride;
-    const uint32_t tok = lrow < count ? lrow : count - 1U;
-    const uint8_t* xrow;
-    if (MODE == 0) xrow = a.x + static_cast<size_t>(order[begin + tok] / a.top_k) * a.x_stride;
-    else xrow = reinterpret_cast<const uint8_t*>(a.h + static_cast<size_t>(begin + tok) * a.k);
+    const uint8_t* wbase = (MODE == 0 && (lrow & 32U)) ? a.wb : a.wa;
+    const uint32_t wfeature = MODE == 0 ? 32U * (lrow >> 6) + (lrow & 31U) : lrow;
+    const uint8_t* wrow = wbase + static_cast<size_t>(e) * a.expert_stride + static_cast<size_t>(m0 + wfeature) * a.row_stride;
+    // token loads: 8 consecutive lanes fetch the 128 bytes of one token row's step (whole cache lines); a thread serves
+    // tokens t / 8 + 32 i, i = 0..3
+    const uint8_t* xrow[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4U; ++i) {
+        const uint32_t token = (t >> 3) + 32U * i, tok = token < count ? token : count - 1U;
+        if (MODE == 0) xrow[i] = a.x + static_cast<size_t>(order[begin + tok] / a.top_k) * a.x_stride + 16U * (t & 7U);
+        else xrow[i] = reinterpret_cast<const uint8_t*>(a.h + static_cast<size_t>(begin + tok) * a.k) + 16U * (t & 7U);
+    }
     const uint32_t steps = a.k / kPfStep;
 
     auto fetch = [&](uint32_t s, PfRaw& r) {
@@ -80,11 +90,10 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(PrefillArgs a, uint
         const uint8_t* blk = wrow + static_cast<size_t>(kb) * 144U;
         r.hd = *reinterpret_cast<const u32x4*>(blk);
         r.qs = *reinterpret_cast<const u32x4*>(blk + 16U + 32U * p + 16U * half);
-        const uint8_t* xs = xrow + (static_cast<size_t>(s) * kPfStep + 32U * half) * 2U;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r.x[i] = *reinterpret_cast<const u32x4*>(xs + 16 * i);
+        for (int i = 0; i < 4; ++i) r.x[i] = *reinterpret_cast<const u32x4*>(xrow[i] + static_cast<size_t>(s) * kPfStep * 2U);
     };
-    auto stage = [&](uint32_t s, const PfRaw& r) {
+    auto stage = [&](uint32_t s, const PfRaw& r, uint32_t buf) {
         const uint32_t p = s & 3U, j0 = 2U * p, sh0 = 8U * (j0 & 3U), sh1 = sh0 + 8U;
         const uint32_t fa0 = (r.hd.y >> sh0) & 255U, fb0 = (r.hd.z >> sh0) & 255U, fc0 = (r.hd.w >> sh0) & 255U;
         const uint32_t fa1 = (r.hd.y >> sh1) & 255U, fb1 = (r.hd.z >> sh1) & 255U, fc1 = (r.hd.w >> sh1) & 255U;
@@ -112,8 +121,8 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(PrefillArgs a, uint
             split2(l0, l1, lo_hi[2 * i], lo_lo[2 * i]); split2(l2, l3, lo_hi[2 * i + 1], lo_lo[2 * i + 1]);
             split2(h0, h1, hi_hi[2 * i], hi_lo[2 * i]); split2(h2, h3, hi_hi[2 * i + 1], hi_lo[2 * i + 1]);
         }
-        uint8_t* ah = tile_a[0] + lrow * kPfPitch;
-        uint8_t* al = tile_a[1] + lrow * kPfPitch;
+        uint8_t* ah = tile_a[buf][0] + lrow * kPfPitch;
+        uint8_t* al = tile_a[buf][1] + lrow * kPfPitch;
         *reinterpret_cast<u32x4*>(ah + 32U * half) = u32x4{lo_hi[0], lo_hi[1], lo_hi[2], lo_hi[3]};
         *reinterpret_cast<u32x4*>(ah + 32U * half + 16U) = u32x4{lo_hi[4], lo_hi[5], lo_hi[6], lo_hi[7]};
         *reinterpret_cast<u32x4*>(ah + 64U + 32U * half) = u32x4{hi_hi[0], hi_hi[1], hi_hi[2], hi_hi[3]};
@@ -122,75 +131,98 @@ __global__ __launch_bounds__(256, 2) void prefill_f16_kernel(PrefillArgs a, uint
         *reinterpret_cast<u32x4*>(al + 32U * half + 16U) = u32x4{lo_lo[4], lo_lo[5], lo_lo[6], lo_lo[7]};
         *reinterpret_cast<u32x4*>(al + 64U + 32U * half) = u32x4{hi_lo[0], hi_lo[1], hi_lo[2], hi_lo[3]};
         *reinterpret_cast<u32x4*>(al + 64U + 32U * half + 16U) = u32x4{hi_lo[4], hi_lo[5], hi_lo[6], hi_lo[7]};
-        uint8_t* br = tile_b + lrow * kPfPitch + 64U * half;
+        uint8_t* br = tile_b[buf] + (t >> 3) * kPfPitch + 16U * (t & 7U);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(br + 16 * i) = r.x[i];
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(br + 32 * i * kPfPitch) = r.x[i];
     };
 
-    floatx16 acc[4];
+    floatx16 acc[2][2];                           // [row tile][token tile] of the wave's 64 x 64 quarter
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acc[i][j] = 0.0F;
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[i][n][j] = 0.0F;
+    const uint32_t wr = wave >> 1, wc = wave & 1U;
 
-    PfRaw raw;
-    fetch(0, raw);
     const uint32_t arow = lane & 31U, kq = (lane >> 5) * 16U;     // MFMA operand role: row / token lane & 31, 8 halves at k = 8 (lane / 32)
-    const uint8_t* ta = tile_a[0] + arow * kPfPitch + kq;
-    const uint8_t* tl = tile_a[1] + arow * kPfPitch + kq;
-    const uint8_t* tb = tile_b + (32U * wave + arow) * kPfPitch + kq;
+    PfRaw raw;
+    if (loader) {
+        fetch(0, raw);
+        stage(0, raw, 0);
+        if (steps > 1U) fetch(1, raw);
+    }
+    __syncthreads();
     for (uint32_t s = 0; s < steps; ++s) {
-        stage(s, raw);
-        __syncthreads();
-        if (s + 1U < steps) fetch(s + 1U, raw);          // in flight during the step's MFMAs
+        const uint32_t buf = s & 1U;
+        if (loader) {
+            if (s + 1U < steps) {
+                stage(s + 1U, raw, buf ^ 1U);                 // operands fetched during the previous step
+                if (s + 2U < steps) fetch(s + 2U, raw);       // in flight during the next step
+            }
+        } else {
+            const uint8_t* ta = tile_a[buf][0] + (64U * wr + arow) * kPfPitch + kq;
+            const uint8_t* tl = tile_a[buf][1] + (64U * wr + arow) * kPfPitch + kq;
+            const uint8_t* tb = tile_b[buf] + (64U * wc + arow) * kPfPitch + kq;
 #pragma unroll
-        for (uint32_t ks = 0; ks < 4U; ++ks) {
-            const half8 b = *reinterpret_cast<const half8*>(tb + 32U * ks);
+            for (uint32_t ks = 0; ks < 4U; ++ks) {
+                half8 b[2], wl[2], wh[2];
 #pragma unroll
-            for (uint32_t m = 0; m < 4U; ++m) {
-                const half8 wh = *reinterpret_cast<const half8*>(ta + m * 32U * kPfPitch + 32U * ks);
-                const half8 wl = *reinterpret_cast<const half8*>(tl + m * 32U * kPfPitch + 32U * ks);
-                acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wl, b, acc[m], 0, 0, 0);
-                acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh, b, acc[m], 0, 0, 0);
+                for (uint32_t i = 0; i < 2U; ++i) {
+                    b[i] = *reinterpret_cast<const half8*>(tb + i * 32U * kPfPitch + 32U * ks);
+                    wl[i] = *reinterpret_cast<const half8*>(tl + i * 32U * kPfPitch + 32U * ks);
+                    wh[i] = *reinterpret_cast<const half8*>(ta + i * 32U * kPfPitch + 32U * ks);
+                }
+                // low planes first: consecutive MFMAs never wait for each other's accumulator
+#pragma unroll
+                for (uint32_t i = 0; i < 2U; ++i)
+#pragma unroll
+                    for (uint32_t n = 0; n < 2U; ++n) acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wl[i], b[n], acc[i][n], 0, 0, 0);
+#pragma unroll
+                for (uint32_t i = 0; i < 2U; ++i)
+#pragma unroll
+                    for (uint32_t n = 0; n < 2U; ++n) acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[i], b[n], acc[i][n], 0, 0, 0);
             }
         }
         __syncthreads();
     }
+    if (loader) return;
 
     // C layout of a 32 x 32 tile: lane holds token (lane & 31); register i is weight row 8 (i / 4) + 4 (lane / 32) + i % 4
-    const uint32_t n = 32U * wave + (lane & 31U);
-    const bool live = n < count;
-    if (MODE == 0) {
-        bool bad = false;
 #pragma unroll
-        for (uint32_t m = 0; m < 2U; ++m)
+    for (uint32_t nt = 0; nt < 2U; ++nt) {
+        const uint32_t n = 64U * wc + 32U * nt + (lane & 31U);
+        const bool live = n < count;
+        if (MODE == 0) {
+            bool bad = false;
 #pragma unroll
             for (uint32_t i4 = 0; i4 < 4U; ++i4) {
                 float hv[4];
 #pragma unroll
                 for (uint32_t j = 0; j < 4U; ++j) {
-                    const float g = acc[m][4 * i4 + j], u = acc[m + 2][4 * i4 + j];
+                    const float g = acc[0][nt][4 * i4 + j], u = acc[1][nt][4 * i4 + j];
                     hv[j] = (g / (1.0F + declared_exp(-g))) * u;
                     bad = bad || !(finite_f(g) && finite_f(u) && finite_f(hv[j]));
                 }
                 if (live) {
-                    const uint32_t row = m0 + 32U * m + 8U * i4 + 4U * (lane >> 5);
+                    const uint32_t row = m0 + 32U * wr + 8U * i4 + 4U * (lane >> 5);
                     u32x2 packed = {pack_half2(hv[0], hv[1]), pack_half2(hv[2], hv[3])};
                     *reinterpret_cast<u32x2*>(a.h + static_cast<size_t>(begin + n) * a.features + row) = packed;
                 }
             }
-        if (live && bad) {
-            atomicOr(&a.status[order[begin + n] / a.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
-            atomicOr(a.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            if (live && bad) {
+                atomicOr(&a.status[order[begin + n] / a.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                atomicOr(a.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            }
+        } else if (live) {
+            float* out = a.rawdots + static_cast<size_t>(order[begin + n]) * a.features + m0 + 64U * wr;
+#pragma unroll
+            for (uint32_t m = 0; m < 2U; ++m)
+#pragma unroll
+                for (uint32_t i4 = 0; i4 < 4U; ++i4)
+                    *reinterpret_cast<f32x4*>(out + 32U * m + 8U * i4 + 4U * (lane >> 5)) =
+                        f32x4{acc[m][nt][4 * i4], acc[m][nt][4 * i4 + 1], acc[m][nt][4 * i4 + 2], acc[m][nt][4 * i4 + 3]};
         }
-    } else if (live) {
-        float* out = a.rawdots + static_cast<size_t>(order[begin + n]) * a.features + m0;
-#pragma unroll
-        for (uint32_t m = 0; m < 4U; ++m)
-#pragma unroll
-            for (uint32_t i4 = 0; i4 < 4U; ++i4)
-                *reinterpret_cast<f32x4*>(out + 32U * m + 8U * i4 + 4U * (lane >> 5)) =
-                    f32x4{acc[m][4 * i4], acc[m][4 * i4 + 1], acc[m][4 * i4 + 2], acc[m][4 * i4 + 3]};
     }
 }
 
