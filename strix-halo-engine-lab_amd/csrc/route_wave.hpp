@@ -28,7 +28,7 @@ struct RouteArgs {
     uint32_t* ids; float* weights; float* scores;
     // fused decode extras (all null / zero for the plain router)
     int8_t* codes; float* deltas; int32_t* sums; uint32_t* status; uint32_t* job_status; uint32_t* plan;
-    uint32_t route_blocks, quant_blocks, split, item_bound;
+    uint32_t route_blocks, quant_blocks;
 };
 
 // ---------------------------------------------------------------------------------------------------- logit chains
@@ -425,8 +425,9 @@ __device__ __forceinline__ uint64_t key_max_wave(uint64_t key) {        // the w
     const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(key >> 32)), 63));
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
+// Returns, in lane k < top_k, the k-th selected expert.
 template <uint32_t PER>
-__device__ __forceinline__ void route_select_row_per(float* p_lds, const RouteArgs& a, uint32_t row) {
+__device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const RouteArgs& a, uint32_t row) {
     const uint32_t lane = threadIdx.x & 63U, E = a.p.experts, K = a.p.top_k;
     float* z = a.scores + static_cast<size_t>(row) * E;
     float v[PER];
@@ -493,17 +494,18 @@ __device__ __forceinline__ void route_select_row_per(float* p_lds, const RouteAr
     }
     const float den = sum + a.p.renorm_eps;
     if (lane < K) {
-        __hip_atomic_store(a.ids + static_cast<size_t>(row) * K + lane, my_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // read by the plan builder
+        a.ids[static_cast<size_t>(row) * K + lane] = my_id;
         a.weights[static_cast<size_t>(row) * K + lane] = (a.p.renormalize ? my_v / den : my_v) * a.p.scale;
     }
     __syncthreads();
+    return my_id;
 }
-__device__ __forceinline__ void route_select_row(float* p_lds, const RouteArgs& a, uint32_t row) {
+__device__ __forceinline__ uint32_t route_select_row(float* p_lds, const RouteArgs& a, uint32_t row) {
     const uint32_t E = a.p.experts;
-    if (E <= 128U) route_select_row_per<2>(p_lds, a, row);
-    else if (E <= 256U) route_select_row_per<4>(p_lds, a, row);
-    else if (E <= 512U) route_select_row_per<8>(p_lds, a, row);
-    else route_select_row_per<16>(p_lds, a, row);
+    if (E <= 128U) return route_select_row_per<2>(p_lds, a, row);
+    if (E <= 256U) return route_select_row_per<4>(p_lds, a, row);
+    if (E <= 512U) return route_select_row_per<8>(p_lds, a, row);
+    return route_select_row_per<16>(p_lds, a, row);
 }
 
 }  // namespace strix950

@@ -223,60 +223,6 @@ __host__ __device__ inline uint32_t plan_tickets_at(uint32_t experts, uint32_t a
 // fused prologue
 constexpr uint32_t kPlanTicketWords = 256;
 
-// Expert plan by one wave from the ids of a decode batch held in LDS (A <= 256 assignments).
-__device__ __forceinline__ void build_plan_wave(uint32_t* count, const uint32_t* ids, uint32_t experts, uint32_t assignments, uint32_t split,
-                                                uint32_t item_bound, uint32_t* plan) {
-    const uint32_t lane = threadIdx.x;
-    for (uint32_t e = lane; e <= experts; e += 64U) count[e] = 0;
-    __syncthreads();
-    for (uint32_t a = lane; a < assignments; a += 64U) atomicAdd(&count[ids[a]], 1U);
-    __syncthreads();
-    const uint32_t chunk = (experts + 63U) / 64U, first = lane * chunk, last = first + chunk < experts ? first + chunk : experts;
-    uint32_t local = 0, local_touched = 0, largest = 0;     // local_touched: touched experts << 16 | work items (A <= 256)
-    for (uint32_t e = first; e < last; ++e) {
-        const uint32_t c = count[e];
-        local += c; local_touched += ((c != 0) << 16) + (c + split - 1U) / split; largest = c > largest ? c : largest;
-    }
-    uint32_t run = local, trun = local_touched;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t o = __shfl_up(run, d), t = __shfl_up(trun, d);
-        if (lane >= static_cast<uint32_t>(d)) { run += o; trun += t; }
-    }
-    for (int d = 32; d; d >>= 1) { const uint32_t o = __shfl_xor(largest, d); largest = o > largest ? o : largest; }
-    const uint32_t totals = __shfl(trun, 63), touched_total = totals >> 16, items_total = totals & 0xffffU;
-    run -= local; trun -= local_touched;                    // exclusive prefixes
-    uint32_t irun = trun & 0xffffU;
-    trun >>= 16;
-    uint32_t* offsets = plan + 16;
-    uint32_t* touched = plan + plan_touched_at(experts);
-    uint32_t* order = plan + plan_order_at(experts);
-    uint32_t* items = plan + plan_items_at(experts, assignments);
-    __syncthreads();
-    for (uint32_t e = first; e < last; ++e) {
-        const uint32_t c = count[e];
-        offsets[e] = run;
-        count[e] = run;                                     // LDS now holds the exclusive offsets
-        if (c) {
-            touched[trun++] = e;
-            for (uint32_t b = 0; b < c; b += split, ++irun) {
-                items[4U * irun] = e; items[4U * irun + 1U] = run + b; items[4U * irun + 2U] = run + (b + split < c ? b + split : c); items[4U * irun + 3U] = 0;
-            }
-        }
-        run += c;
-    }
-    for (uint32_t u = items_total + lane; u < item_bound; u += 64U) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
-    if (lane == 0) { offsets[experts] = assignments; plan[0] = assignments; plan[1] = touched_total; plan[2] = largest; plan[4] = items_total; }
-    __syncthreads();
-    // stable order: the rank of an assignment inside its expert = earlier assignments of the same expert
-    for (uint32_t a = lane; a < assignments; a += 64U) {
-        const uint32_t e = ids[a];
-        uint32_t rank = 0;
-        for (uint32_t b = 0; b < a; ++b) rank += ids[b] == e;
-        order[count[e] + rank] = a;
-    }
-}
-
 // Router logits for batches above the decode bound: blocks of 8 experts x 8 rows.
 template <int KIND>
 __global__ __launch_bounds__(64) void route_logits_kernel(RouteArgs a) {
@@ -294,9 +240,10 @@ __global__ __launch_bounds__(256, 2) void route_batch_kernel(RouteArgs a) {
 
 // Decode router launch (rows <= 16). Blocks [0, route_blocks) run the logit chains of (row, 8 experts). In the plain form
 // (a.plan == nullptr) the kernel stops there. In the fused form blocks [route_blocks, route_blocks + quant_blocks)
-// quantise the input rows to A8 (8 groups of 32 per block); the block that finishes a row's last 8 experts (row ticket)
-// runs that row's softmax / top-k / weights, and the block that takes the last launch ticket publishes the row status
-// words and builds the expert plan. Every ticket word is left zero.
+// quantise the input rows to A8 (8 groups of 32 per block; the last of a row's blocks publishes the row's status word),
+// and the block that finishes a row's last 8 experts (row ticket) runs that row's softmax / top-k / weights and writes the
+// row's work items: a decode batch is planned one item per assignment (item i = assignment i, order = identity; the CSR
+// fields of the plan are not written), so nothing waits for the other rows. Every ticket word is left zero.
 template <int KIND>
 __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
     __shared__ ChainSlot slot0;
@@ -304,8 +251,6 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
     __shared__ ChainSlot slot2;
     __shared__ ChainSlot slot3;
     __shared__ __attribute__((aligned(16))) float sel_p[kRouteMaxExperts];
-    __shared__ uint32_t count[kRouteMaxExperts + 64];
-    __shared__ uint32_t ids[kFusedMaxRows * kRouteMaxTopK];
     __shared__ uint32_t flag;
     ChainSlot* const slots[4] = {&slot0, &slot1, &slot2, &slot3};
     const uint32_t bid = blockIdx.x, lane = threadIdx.x, neb = (a.p.experts + 7U) / 8U;
@@ -322,7 +267,17 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
         __syncthreads();
         if (flag) {
             if (lane == 0) tickets[row] = 0;
-            route_select_row(sel_p, a, row);
+            const uint32_t expert = route_select_row(sel_p, a, row);
+            if (lane < a.p.top_k) {
+                const uint32_t assignments = a.rows * a.p.top_k, i = row * a.p.top_k + lane;
+                *reinterpret_cast<uint4*>(a.plan + plan_items_at(a.p.experts, assignments) + 4U * i) = make_uint4(expert, i, i + 1U, 0U);
+                a.plan[plan_order_at(a.p.experts) + i] = i;
+            }
+        }
+        if (bid == 0 && lane == 0) {
+            const uint32_t assignments = a.rows * a.p.top_k;
+            *a.job_status = 0;
+            a.plan[0] = assignments; a.plan[1] = 0; a.plan[2] = 1; a.plan[4] = assignments;
         }
     } else {
         // A8 prologue (src/cpu/core/reference.cpp:35-55): two groups of 32 at a time, 8 groups per block
@@ -347,19 +302,15 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
                 }
             }
         }
+        // the row's last quantiser block publishes the row's status word (a row's 32-groups fill whole blocks: hidden % 256 == 0)
+        const uint32_t r = g0 / groups;
+        __builtin_amdgcn_s_waitcnt(0);
+        if (lane == 0 && __hip_atomic_fetch_add(&tickets[16U + r], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups / 8U - 1U) {
+            a.status[r] = __hip_atomic_load(flags + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            flags[r] = 0;
+            tickets[16U + r] = 0;
+        }
     }
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (lane == 0) flag = __hip_atomic_fetch_add(&a.plan[3], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1U;
-    __syncthreads();
-    if (!flag) return;
-    const uint32_t assignments = a.rows * a.p.top_k;
-    for (uint32_t i = lane; i < assignments; i += 64U) ids[i] = __hip_atomic_load(a.ids + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    uint32_t* flags = tickets + 128U;
-    if (lane < a.rows) { a.status[lane] = __hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); flags[lane] = 0; }
-    if (lane == 0) { *a.job_status = 0; a.plan[3] = 0; }
-    __syncthreads();
-    build_plan_wave(count, ids, a.p.experts, assignments, a.split, a.item_bound, a.plan);
 }
 
 // softmax / top-k / weights, one row per one-wave block (the plain router).
@@ -1019,11 +970,10 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     a.wr = router_weight; a.bias = logit_bias; a.ids = ids; a.weights = weights; a.scores = scores;
     a.codes = r->codes; a.deltas = r->deltas; a.sums = r->sums; a.status = r->status; a.job_status = r->job_status; a.plan = r->plan;
     a.quant_blocks = (rows * (wv.hidden / 32U) + 7U) / 8U;
-    a.split = plan_split(wv, rows); a.item_bound = item_bound(wv, rows);
     launch_route_logits(a, hs(stream));
     STRIX_LAUNCHED("moe layer router");
-    launch_project(wv, *r, rows, item_bound(wv, rows), hs(stream));
-    launch_down(wv, *r, rows, item_bound(wv, rows), hs(stream));
+    launch_project(wv, *r, rows, rows * wv.top_k, hs(stream));       // the fused router planned one item per assignment
+    launch_down(wv, *r, rows, rows * wv.top_k, hs(stream));
     STRIX_LAUNCHED("moe layer experts");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
