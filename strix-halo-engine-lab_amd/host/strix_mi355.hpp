@@ -70,6 +70,12 @@ inline void enqueue(const Rows& r, std::uint32_t rows, const Weights& w, mi355_s
                     std::uint32_t form = MI355_COMBINE_FMA_SLOT_ORDER) {
     check(mi355_moe_enqueue(&w, &r, rows, form, s));
 }
+// the routed experts of a prefill batch on fp16 MFMA (FAST class: follows the exact-weight product to 2e-3, not the
+// integer-dot bits); needs r.h_f16 and fp16 input rows
+inline void enqueue_prefill_f16(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s,
+                                std::uint32_t form = MI355_COMBINE_FMA_SLOT_ORDER) {
+    check(mi355_moe_enqueue_prefill_f16(&w, &r, rows, form, s));
+}
 // router + the layer; r.routes / r.route_weights receive the selection
 inline void enqueue_layer(const moe_route::Policy& policy, const float* router_weight, const float* logit_bias, float* scores,
                           const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s,

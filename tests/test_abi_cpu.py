@@ -56,3 +56,14 @@ def test_product_path_never_references_the_oracle():
             if f.endswith((".py", ".hip", ".hpp", ".h", ".cpp")):
                 text = open(os.path.join(base, f), errors="ignore").read()
                 assert "liboracle" not in text and "import orc" not in text and "strix_oracle.h" not in text, f
+
+
+def test_cpp_host_mirror_compiles_against_the_header():
+    """The header-only C++ mirror of the reference interfaces must compile against include/mi355_strix.h with a host compiler."""
+    import subprocess, tempfile
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with tempfile.NamedTemporaryFile("w", suffix=".cpp", delete=False) as f:
+        f.write('#include "strix_mi355.hpp"\nint main() { return 0; }\n')
+    subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I" + os.path.join(root, "include"),
+                    "-I" + os.path.join(root, "strix-halo-engine-lab_amd", "host"), f.name], check=True)
+    os.unlink(f.name)
