@@ -149,10 +149,12 @@ typedef struct mi355_moe_rows {
     float* output; uint64_t output_stride;            /* [rows][hidden] fp32, stride in floats */
     uint32_t* plan;                  /* mi355_moe_plan_words(experts, rows, top_k) words, 16-byte aligned */
     uint32_t* job_status;            /* 1 word: OR of every row's status (decides whether the down phase runs) */
-    void* h_f16;                     /* optional [rows][top_k][ffn] fp16 workspace, used only by mi355_moe_enqueue_prefill_f16 */
+    void* h_f16;                     /* optional workspace of mi355_moe_prefill_f16_workspace_bytes() bytes, 16-byte aligned,
+                                        used only by mi355_moe_enqueue_prefill_f16 (h in fp16 and sub-block sums) */
 } mi355_moe_rows;
 
 size_t mi355_moe_plan_words(uint32_t experts, uint32_t rows, uint32_t top_k);
+size_t mi355_moe_prefill_f16_workspace_bytes(uint32_t hidden, uint32_t ffn, uint32_t rows, uint32_t top_k);
 
 /* prologue: clear status, validate routes and route weights, A8-quantise the input rows. */
 int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, mi355_stream);
@@ -182,12 +184,13 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* policy, const float* r
 
 /* The routed experts of a prefill batch on the matrix cores - the path's FAST arithmetic class (the reference's
  * bit-changing MMA forms: include/strix/cuda/qwen_moe.hpp:100-101 moe_mma, known_rows::enqueue_prefill
- * include/strix/hip_moe_q4k_a8_known_rows.hpp:109-111). Q4_K weights are decoded exactly as mi355_dequantize_rows does,
- * rounded once to fp16 and multiplied with the fp16 input rows by fp16 MFMA with fp32 accumulation; SiLU uses the declared
- * exp; h is kept in fp16 (rows->h_f16). Results follow the exact-weight product (include/strix/ds41_layer.hpp:96-121) to
+ * include/strix/hip_moe_q4k_a8_known_rows.hpp:109-111). The integers sc * q of the Q4_K blocks (exact in fp16) are multiplied
+ * with the fp16 rows by fp16 MFMA with fp32 accumulation, the block scale d applied in fp32 per super-block, the dmin * m
+ * terms added as a product over sub-block sums; SiLU uses the declared exp; h is kept in fp16 (rows->h_f16). Results follow the exact-weight product (include/strix/ds41_layer.hpp:96-121) to
  * the library's tolerance (2e-3 of the output rms), NOT the integer-dot class's bits: a caller opts in by calling this
  * entry point. Runs: status clear + route validation, expert plan, gate/up + SwiGLU, down, ordered combine.
- * Requires input_kind = MI355_INPUT_F16, rows->h_f16, hidden % 256 == 0, ffn % 256 == 0. */
+ * Requires input_kind = MI355_INPUT_F16, rows->h_f16 (see mi355_moe_prefill_f16_workspace_bytes), hidden % 256 == 0,
+ * ffn % 256 == 0. */
 int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, uint32_t combine_form,
                                       mi355_stream);
 

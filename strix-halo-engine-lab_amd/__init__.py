@@ -71,6 +71,8 @@ def lib():
         L.mi355_numerical_identity.argtypes = [C.c_uint32, C.c_int]
         L.mi355_moe_plan_words.restype = C.c_size_t
         L.mi355_moe_plan_words.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32]
+        L.mi355_moe_prefill_f16_workspace_bytes.restype = C.c_size_t
+        L.mi355_moe_prefill_f16_workspace_bytes.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32]
         _lib = L
     return _lib
 
@@ -78,7 +80,7 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_prefill_f16",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize"]
 
 
@@ -193,7 +195,8 @@ class MoeLayer:
         self.up_out = z((n, ffn), torch.float32) if intermediates else None
         self.h_out = z((n, ffn), torch.float32) if intermediates else None
         self.plan = z(int(lib().mi355_moe_plan_words(experts, max_rows, top_k)), torch.int32)
-        self.h_f16 = z((n, ffn), torch.float16) if prefill_f16 else None      # workspace of the fp16 MFMA prefill form
+        # workspace of the fp16 MFMA prefill form: h in fp16 and the sub-block sums of h and of the input rows
+        self.h_f16 = z((int(lib().mi355_moe_prefill_f16_workspace_bytes(hidden, ffn, max_rows, top_k)),), torch.uint8) if prefill_f16 else None
 
     def rows_view(self, x, ids, weights, base=None):
         rows = x.shape[0]

@@ -1,28 +1,41 @@
 // Prefill form of the routed experts for gfx950: an expert-grouped GEMM on the matrix cores. This is the path's second
-// arithmetic class (the reference's FAST forms, include/strix/cuda/qwen_moe.hpp:100-101 "bit-changing"): Q4_K weights are
-// dequantised exactly as the block decoder does (src/ggml_dequant.cpp:119-130: (d * sc) * q - (dmin * m), two fp32
-// roundings), split into two fp16 numbers (w_hi = fp16(w), w_lo = fp16(w - w_hi): together ~22 significant bits - a single
-// fp16 weight alone costs ~3e-3 of the output rms, above the tolerance), and multiplied with fp16 activations by
-// v_mfma_f32_32x32x16_f16 with fp32 accumulation (two MFMAs per operand pair).
-// Its parity target is the exact-weight product (include/strix/ds41_layer.hpp:96-121) within the stated tolerance, not
-// the integer-dot class's bits.
+// arithmetic class (the reference's FAST forms, include/strix/cuda/qwen_moe.hpp:100-101 "bit-changing"); its parity target
+// is the exact-weight product (include/strix/ds41_layer.hpp:96-121) within the stated tolerance, not the integer-dot
+// class's bits.
 //
-// Work decomposition: the expert plan cuts every expert's assignments into items of at most 128 rows. A 256-thread
-// workgroup owns (item, 64 output features of gate AND up) or (item, 128 output features of down): a 128 x 128 tile of
-// weight rows x tokens, K walked in steps of 64 (one pair of Q4_K sub-blocks: the 32 quant bytes whose low / high nibbles
-// are sub-blocks 2p / 2p + 1). Per step every thread fetches 16 quant bytes + the block header of one weight row and 64
-// bytes of one token row into registers (one step ahead of the arithmetic), dequantises its 32 weights and stores the
-// tiles row-major [row][k] (pitch 144 bytes: conflict-free 128-bit reads) in LDS (weights hi, weights lo, tokens).
-// The workgroup has 8 waves in two roles: waves 0-3 are the loaders just described, waves 4-7 each multiply a 64 x 64
-// quarter of the tile (2 x 2 MFMA tiles: every operand read from LDS feeds two MFMAs; 32 MFMAs per step). Tile rows are
-// ordered [gate 0-31, up 0-31, gate 32-63, up 32-63] so that a wave holds gate and up of the same features. The LDS tiles are double-buffered and there is one barrier per
-// step, so the loaders prepare step s + 1 (VALU) while the multipliers run step s (matrix cores) on the same SIMDs.
+// Arithmetic. A Q4_K weight is w = d_b (sc_j q) - dmin_b m_j (super-block b of 256, sub-block j of 32, q a nibble;
+// src/ggml_dequant.cpp:119-130). The kernel never rounds a weight to fp16. For output feature f and token t
+//   out[t][f] = sum_b d_b[f] * P_b[t][f]  +  sum_(b,j) S_bj[t] * M_bj[f],
+//   P_b = sum_(k in b) (sc_j q_k) x_k[t],   S_bj[t] = sum_(k in sub-block j of b) x_k[t],   M_bj[f] = -(dmin_b m_j).
+// sc_j q_k is an integer <= 945: exact in fp16, so P_b is an fp16 MFMA with fp32 accumulation whose only rounding is the
+// fp32 accumulation; d_b is applied in fp32 once per super-block. The second sum is a product over K / 32 sub-blocks:
+// S and M are each carried as two fp16 numbers (hi = fp16(v), lo = fp16(v - hi)) and multiplied by three MFMAs per 16
+// sub-blocks (hi*hi + lo*hi + hi*lo). S of the input rows comes from token_sums_kernel, S of h from the epilogue of
+// the gate / up launch.
 //
-// Weights are read from HBM once per (item, feature tile); with ~128 rows per item the arithmetic intensity is ~450
-// flop per weight byte, above the machine balance, so the kernel is bound by the matrix cores and the dequantisation
-// that feeds them.
+// Work decomposition. The expert plan cuts every expert's assignments into items of at most 128 rows. A 512-thread
+// workgroup owns (item, 64 output features of gate AND up) or (item, 128 output features of down): 128 weight rows x
+// 128 tokens, K walked in steps of 64 (one pair of Q4_K sub-blocks: 32 quant bytes whose low / high nibbles are
+// sub-blocks 2p / 2p + 1). Waves 0-3 are loaders, waves 4-7 multipliers (one of each per SIMD):
+//   * token rows go from global memory straight into a 4-stage LDS ring (global_load_lds by the multiplier waves, 3 steps ahead of their use);
+//   * a loader thread owns (weight row, 16 quant bytes): a super-block's raw bytes are fetched into registers five steps
+//     ahead, turned into
+//     32 fp16 integers sc q with v_perm / v_and_or / v_pk_fma_f16 (1024 + q is the fp16 bit pattern 0x6400 | q, and
+//     fma(1024 + q, sc, -1024 sc) = sc q exactly) and stored in a double-buffered LDS tile; d_b, and every two
+//     super-blocks the M tile, go to small LDS arrays; the S tile of the same 16 sub-blocks is copied by global_load_lds;
+//   * a multiplier wave holds a 64 x 64 quarter (2 x 2 MFMA tiles, A = tokens, B = weights: a lane of the result is
+//     one feature, so d_b is one register per tile row) in two sets of accumulators: P (cleared every super-block) and
+//     the running sum.
+// LDS tiles are [row][64 halves] with a 128-byte pitch and the 16-byte pieces of a row XOR-swizzled by row % 8: a 128-bit
+// LDS access is served eight lanes at a time, and eight consecutive rows then cover all 32 banks for the MFMA operand
+// reads and the loaders' stores, while a copy instruction still writes 1 KB of consecutive LDS. One barrier per step.
+//
+// Workgroups are numbered so that the feature tiles of one item run on one XCD (consecutive workgroup ids go round
+// the 8 XCDs): its token rows are then read from HBM once per XCD and served from that XCD's L2 afterwards.
 #pragma once
 #include "device_math.hpp"
+#include "q4k_rows.hpp"
+#include <type_traits>
 
 namespace strix950 {
 
@@ -31,11 +44,22 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float2v __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) uint8_t pf_lds;
 
 constexpr uint32_t kPfTile = 128;                 // weight rows and tokens per workgroup tile
 constexpr uint32_t kPfStep = 64;                  // K per step
-constexpr uint32_t kPfPitch = 144;                // bytes per tile row: 64 halves + 16 bytes of padding
-constexpr uint32_t kPfTileBytes = kPfTile * kPfPitch;   // 18,432
+constexpr uint32_t kPfTileBytes = kPfTile * 128U; // one step of a tile: 128 rows x 64 halves
+constexpr uint32_t kPfRing = 4;                   // token stages (separate LDS objects: stage = step % 4)
+constexpr uint32_t kPfTokenAhead = 3;             // steps between a token copy and its use
+
+// sub-block sums of a row: two fp16 planes (hi, lo) of `pf_sum_slots(k)` halves each, the slots past k / 32 zero
+__host__ __device__ constexpr uint32_t pf_sum_slots(uint32_t k) { return (k / 32U + 15U) & ~15U; }
+__host__ __device__ constexpr size_t pf_sum_row_bytes(uint32_t k) { return 4U * static_cast<size_t>(pf_sum_slots(k)); }
+// bytes of the fp16 workspace: h [assignments][ffn], sums of h [assignments], sums of the input rows [rows]
+__host__ __device__ constexpr size_t pf_h_bytes(uint32_t assignments, uint32_t ffn) { return 2U * static_cast<size_t>(assignments) * ffn; }
+__host__ __device__ constexpr size_t pf_workspace_bytes(uint32_t hidden, uint32_t ffn, uint32_t rows, uint32_t top_k) {
+    return pf_h_bytes(rows * top_k, ffn) + static_cast<size_t>(rows) * top_k * pf_sum_row_bytes(ffn) + static_cast<size_t>(rows) * pf_sum_row_bytes(hidden);
+}
 
 struct PrefillArgs {
     const uint8_t* wa; const uint8_t* wb;         // MODE 0: gate, up; MODE 1: down (wb unused)
@@ -45,183 +69,378 @@ struct PrefillArgs {
     uint32_t top_k, exp_kind;
     const uint8_t* x; uint64_t x_stride;          // MODE 0: fp16 token rows (bytes); MODE 1: unused
     _Float16* h;                                  // [assignments in plan order][ffn] fp16: written by MODE 0, read by MODE 1
+    uint8_t* h_sums;                              // [assignments in plan order] sub-block sums of h: written by MODE 0, read by MODE 1
+    const uint8_t* x_sums;                        // [rows] sub-block sums of the input rows (MODE 0)
     float* rawdots;                               // MODE 1: [assignment][hidden]
     const uint32_t* plan; uint32_t experts, assignments;
     uint32_t* status; uint32_t* job_status;
+    uint32_t tiles, items;                        // feature tiles per item, item bound of the launch
 };
 
 __device__ __forceinline__ uint32_t pack_half2(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, half2v));      // v_cvt_pk_f16_f32: round to nearest even
 }
+// v -> fp16 hi = fp16(v), lo = fp16(v - hi)
+__device__ __forceinline__ void split_half(float v, _Float16& hi, _Float16& lo) {
+    hi = static_cast<_Float16>(v);
+    lo = static_cast<_Float16>(v - static_cast<float>(hi));
+}
 
-// Raw operands of one K step held in registers between their global loads and their use.
-struct PfRaw { u32x4 hd, qs, x[4]; };
+// Sub-block sums of fp16 rows: one thread per (row, sub-block of 32), fp32 sum in index order.
+__global__ __launch_bounds__(256) void token_sums_kernel(const uint8_t* x, uint64_t x_stride, uint32_t k, uint8_t* sums) {
+    const uint32_t row = blockIdx.x, slots = pf_sum_slots(k);
+    _Float16* hi = reinterpret_cast<_Float16*>(sums + static_cast<size_t>(row) * pf_sum_row_bytes(k));
+    _Float16* lo = hi + slots;
+    for (uint32_t s = threadIdx.x; s < slots; s += 256U) {
+        float sum = 0.0F;
+        if (s < k / 32U) {
+            const half8* p = reinterpret_cast<const half8*>(x + static_cast<size_t>(row) * x_stride + 64U * s);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const half8 v = p[i];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sum += static_cast<float>(v[j]);
+            }
+        }
+        split_half(sum, hi[s], lo[s]);
+    }
+}
+
+// Padding slots of the sums of h (ffn / 32 not a multiple of 16) must read as zero.
+__global__ __launch_bounds__(64) void clear_sum_padding_kernel(uint8_t* sums, uint32_t k) {
+    const uint32_t slots = pf_sum_slots(k), used = k / 32U;
+    _Float16* hi = reinterpret_cast<_Float16*>(sums + static_cast<size_t>(blockIdx.x) * pf_sum_row_bytes(k));
+    for (uint32_t s = used + threadIdx.x; s < slots; s += 64U) { hi[s] = static_cast<_Float16>(0.0F); hi[slots + s] = static_cast<_Float16>(0.0F); }
+}
+
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every outstanding global memory operation
+// of the wave, which would drain the copies and fetches that are in flight for later steps at every barrier; their
+// arrival is awaited explicitly where it is needed.
+// (A fence on the LDS address space counts the copies' LDS writes and waits for them too, hence the plain instructions:
+// LDS stores of this wave complete, barrier; the compiler moves no memory access across the statement.)
+__device__ __forceinline__ void pf_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// One global -> LDS copy of 16 bytes per lane (lane l lands at lds_base + 16 l), issued as plain instructions: the
+// compiler is not told about it, so it adds no waits of its own around later LDS reads; the arrival of a copy is awaited
+// by a counted s_waitcnt before the barrier that publishes the stage.
+__device__ __forceinline__ void copy16_to_lds(const uint8_t* src, pf_lds* lds_base) {
+    const uint32_t at = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(at), "v"(src) : "memory", "m0");
+}
+
+// byte offset of 16-byte piece `piece` (0..7) of tile row `row`
+__device__ __forceinline__ uint32_t pf_at(uint32_t row, uint32_t piece) { return row * 128U + ((piece ^ (row & 7U)) << 4); }
+
+// the loader's per-step global operands
+struct PfRaw { u32x4 hd, qs[4]; };           // one super-block of a weight row: header and the thread's 16 quant bytes of its four steps
 
 template <int MODE>
 __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_t items_at, uint32_t order_at) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile_a[2][2][kPfTileBytes];     // [buffer][0: w_hi, 1: w_lo]
-    __shared__ __attribute__((aligned(16))) uint8_t tile_b[2][kPfTileBytes];
-    const uint4 item = *reinterpret_cast<const uint4*>(a.plan + items_at + 4U * blockIdx.y);
+    __shared__ __attribute__((aligned(16))) uint8_t tok0[kPfTileBytes];                     // token steps: stage s % 4
+    __shared__ __attribute__((aligned(16))) uint8_t tok1[kPfTileBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t tok2[kPfTileBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t tok3[kPfTileBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t w_tile[2][kPfTileBytes];                // sc q of one step
+    __shared__ __attribute__((aligned(16))) uint8_t s_tile_mem[2][kPfTile * 64U];           // [token][hi 16 | lo 16] sums of 16 sub-blocks
+    __shared__ __attribute__((aligned(16))) uint8_t m_tile[2][kPfTile * 64U];               // [feature][hi 16 | lo 16] -(dmin m)
+    __shared__ float d_scale[2][kPfTile];                                                   // d of one super-block
+    pf_lds* const tok_stage[4] = {(pf_lds*)tok0, (pf_lds*)tok1, (pf_lds*)tok2, (pf_lds*)tok3};
+    pf_lds* const s_tile = (pf_lds*)s_tile_mem;
+
+    // workgroup -> (item, feature tile): ids i, i + 8, i + 16, ... share an XCD; they walk the tiles of one item first
+    const uint32_t xcd = blockIdx.x & 7U, q = blockIdx.x >> 3;
+    const uint32_t item_index = (q / a.tiles) * 8U + xcd, tile = q % a.tiles;
+    if (item_index >= a.items) return;
+    const uint4 item = *reinterpret_cast<const uint4*>(a.plan + items_at + 4U * item_index);
     const uint32_t e = item.x, begin = item.y, count = item.z - item.y;
     if (count == 0) return;
     if (MODE == 1 && (*a.job_status & MI355_STATUS_NONFINITE_PROJECTION)) return;
     const uint32_t* order = a.plan + order_at;
     const bool loader = threadIdx.x < 256U;
     const uint32_t t = threadIdx.x & 255U, lane = t & 63U, wave = t >> 6;      // index within the role
-    // loader role: thread t owns weight row t / 2 of the tile and token t / 2, half = which 16 quant bytes / 32 features
-    const uint32_t lrow = t >> 1, half = t & 1U;
-    const uint32_t m0 = blockIdx.x * (MODE == 0 ? 64U : 128U);
-    const uint8_t* wbase = (MODE == 0 && (lrow & 32U)) ? a.wb : a.wa;
-    const uint32_t wfeature = MODE == 0 ? 32U * (lrow >> 6) + (lrow & 31U) : lrow;
-    const uint8_t* wrow = wbase + static_cast<size_t>(e) * a.expert_stride + static_cast<size_t>(m0 + wfeature) * a.row_stride;
-    // token loads: 8 consecutive lanes fetch the 128 bytes of one token row's step (whole cache lines); a thread serves
-    // tokens t / 8 + 32 i, i = 0..3
-    const uint8_t* xrow[4];
-#pragma unroll
-    for (uint32_t i = 0; i < 4U; ++i) {
-        const uint32_t token = (t >> 3) + 32U * i, tok = token < count ? token : count - 1U;
-        if (MODE == 0) xrow[i] = a.x + static_cast<size_t>(order[begin + tok] / a.top_k) * a.x_stride + 16U * (t & 7U);
-        else xrow[i] = reinterpret_cast<const uint8_t*>(a.h + static_cast<size_t>(begin + tok) * a.k) + 16U * (t & 7U);
-    }
-    const uint32_t steps = a.k / kPfStep;
+    const uint32_t m0 = tile * (MODE == 0 ? 64U : 128U);
+    const uint32_t steps = a.k / kPfStep, blocks = a.k / 256U, steps8 = (steps + 7U) & ~7U;
+    const size_t sum_row = pf_sum_row_bytes(a.k);
 
-    auto fetch = [&](uint32_t s, PfRaw& r) {
-        const uint32_t kb = s >> 2, p = s & 3U;
-        const uint8_t* blk = wrow + static_cast<size_t>(kb) * 144U;
-        r.hd = *reinterpret_cast<const u32x4*>(blk);
-        r.qs = *reinterpret_cast<const u32x4*>(blk + 16U + 32U * p + 16U * half);
+    if (loader) {
+        // ---- weight side: row lrow of the tile, quant bytes [16 half, 16 half + 16) of every step
+        const uint32_t lrow = 32U * wave + (lane & 31U), half = lane >> 5;
+        const uint8_t* wbase = (MODE == 0 && (lrow & 32U)) ? a.wb : a.wa;
+        const uint32_t wfeature = MODE == 0 ? 32U * (lrow >> 6) + (lrow & 31U) : lrow;
+        const uint8_t* wrow = wbase + static_cast<size_t>(e) * a.expert_stride + static_cast<size_t>(m0 + wfeature) * a.row_stride;
+        // ---- token side: copy i of a step moves tile rows 8 (4 i + wave) .. + 8; lane = (row % 8, slot)
+        const uint8_t* tsrc[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r.x[i] = *reinterpret_cast<const u32x4*>(xrow[i] + static_cast<size_t>(s) * kPfStep * 2U);
-    };
-    auto stage = [&](uint32_t s, const PfRaw& r, uint32_t buf) {
-        const uint32_t p = s & 3U, j0 = 2U * p, sh0 = 8U * (j0 & 3U), sh1 = sh0 + 8U;
-        const uint32_t fa0 = (r.hd.y >> sh0) & 255U, fb0 = (r.hd.z >> sh0) & 255U, fc0 = (r.hd.w >> sh0) & 255U;
-        const uint32_t fa1 = (r.hd.y >> sh1) & 255U, fb1 = (r.hd.z >> sh1) & 255U, fc1 = (r.hd.w >> sh1) & 255U;
-        const bool low = p < 2U;                  // uniform: p is the same for the whole workgroup
-        const uint32_t s0 = low ? (fa0 & 63U) : ((fc0 & 15U) | ((fa0 >> 6) << 4)), n0 = low ? (fb0 & 63U) : ((fc0 >> 4) | ((fb0 >> 6) << 4));
-        const uint32_t s1 = low ? (fa1 & 63U) : ((fc1 & 15U) | ((fa1 >> 6) << 4)), n1 = low ? (fb1 & 63U) : ((fc1 >> 4) | ((fb1 >> 6) << 4));
-        const float d = half_bits_to_float(r.hd.x & 0xffffU), dm = half_bits_to_float(r.hd.x >> 16);
-        const float D0 = d * static_cast<float>(s0), M0 = dm * static_cast<float>(n0);
-        const float D1 = d * static_cast<float>(s1), M1 = dm * static_cast<float>(n1);
-        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
-        // value -> (fp16 hi, fp16 lo) packed pairs; lo = fp16(value - hi) is exact to ~2^-22 of the value
-        uint32_t lo_hi[8], lo_lo[8], hi_hi[8], hi_lo[8];
-        const auto split2 = [](float v0, float v1, uint32_t& hi2, uint32_t& lo2) {
-            const half2v h = __builtin_convertvector(float2v{v0, v1}, half2v);
-            hi2 = __builtin_bit_cast(uint32_t, h);
-            lo2 = pack_half2(v0 - static_cast<float>(h.x), v1 - static_cast<float>(h.y));
-        };
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t w = q[i];
-            const float l0 = D0 * static_cast<float>(w & 15U) - M0, l1 = D0 * static_cast<float>((w >> 8) & 15U) - M0;
-            const float l2 = D0 * static_cast<float>((w >> 16) & 15U) - M0, l3 = D0 * static_cast<float>((w >> 24) & 15U) - M0;
-            const float h0 = D1 * static_cast<float>((w >> 4) & 15U) - M1, h1 = D1 * static_cast<float>((w >> 12) & 15U) - M1;
-            const float h2 = D1 * static_cast<float>((w >> 20) & 15U) - M1, h3 = D1 * static_cast<float>(w >> 28) - M1;
-            split2(l0, l1, lo_hi[2 * i], lo_lo[2 * i]); split2(l2, l3, lo_hi[2 * i + 1], lo_lo[2 * i + 1]);
-            split2(h0, h1, hi_hi[2 * i], hi_lo[2 * i]); split2(h2, h3, hi_hi[2 * i + 1], hi_lo[2 * i + 1]);
+        for (uint32_t i = 0; i < 4U; ++i) {
+            const uint32_t row = 8U * (4U * i + wave) + (lane >> 3), tok = row < count ? row : count - 1U;
+            const uint32_t piece = (lane & 7U) ^ (row & 7U);
+            if (MODE == 0) tsrc[i] = a.x + static_cast<size_t>(order[begin + tok] / a.top_k) * a.x_stride + 16U * piece;
+            else tsrc[i] = reinterpret_cast<const uint8_t*>(a.h + static_cast<size_t>(begin + tok) * a.k) + 16U * piece;
         }
-        uint8_t* ah = tile_a[buf][0] + lrow * kPfPitch;
-        uint8_t* al = tile_a[buf][1] + lrow * kPfPitch;
-        *reinterpret_cast<u32x4*>(ah + 32U * half) = u32x4{lo_hi[0], lo_hi[1], lo_hi[2], lo_hi[3]};
-        *reinterpret_cast<u32x4*>(ah + 32U * half + 16U) = u32x4{lo_hi[4], lo_hi[5], lo_hi[6], lo_hi[7]};
-        *reinterpret_cast<u32x4*>(ah + 64U + 32U * half) = u32x4{hi_hi[0], hi_hi[1], hi_hi[2], hi_hi[3]};
-        *reinterpret_cast<u32x4*>(ah + 64U + 32U * half + 16U) = u32x4{hi_hi[4], hi_hi[5], hi_hi[6], hi_hi[7]};
-        *reinterpret_cast<u32x4*>(al + 32U * half) = u32x4{lo_lo[0], lo_lo[1], lo_lo[2], lo_lo[3]};
-        *reinterpret_cast<u32x4*>(al + 32U * half + 16U) = u32x4{lo_lo[4], lo_lo[5], lo_lo[6], lo_lo[7]};
-        *reinterpret_cast<u32x4*>(al + 64U + 32U * half) = u32x4{hi_lo[0], hi_lo[1], hi_lo[2], hi_lo[3]};
-        *reinterpret_cast<u32x4*>(al + 64U + 32U * half + 16U) = u32x4{hi_lo[4], hi_lo[5], hi_lo[6], hi_lo[7]};
-        uint8_t* br = tile_b[buf] + (t >> 3) * kPfPitch + 16U * (t & 7U);
+        // ---- sums side: copy c of a group moves pieces 256 c + t; piece = (token, part): part 0, 1 = hi, part 2, 3 = lo
+        const uint8_t* ssrc[2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(br + 32 * i * kPfPitch) = r.x[i];
-    };
+        for (uint32_t c = 0; c < 2U; ++c) {
+            const uint32_t piece = 256U * c + t, row = piece >> 2, part = piece & 3U, tok = row < count ? row : count - 1U;
+            const uint8_t* base = MODE == 0 ? a.x_sums + static_cast<size_t>(order[begin + tok] / a.top_k) * sum_row
+                                            : a.h_sums + static_cast<size_t>(begin + tok) * sum_row;
+            ssrc[c] = base + 16U * (part & 1U) + (part >> 1) * (sum_row / 2U);
+        }
+        const uint32_t last = steps - 1U, last_block = blocks - 1U, last_group = (blocks + 1U) / 2U - 1U;
+        // Every memory operation below is issued unconditionally (indices past the end are clamped: such copies land in
+        // stages nobody reads any more), so the number of operations between an issue and the point that needs its data
+        // is a compile-time constant and the waits are plain s_waitcnt vmcnt(n) of this code's own: the compiler is not
+        // told about these operations, whose bookkeeping across loop iterations it resolves by waiting for all of them.
+        const auto copy_tokens = [&](uint32_t s, pf_lds* stage) {          // 4 operations: step s -> its stage
+            const uint32_t sc = s < last ? s : last;
+#pragma unroll
+            for (uint32_t i = 0; i < 4U; ++i) copy16_to_lds(tsrc[i] + static_cast<size_t>(sc) * 128U, stage + 1024U * (4U * i + wave));
+        };
+        const auto copy_sums = [&](uint32_t g) {                           // 2 operations: 16 sub-blocks of group g -> s_tile[g % 2]
+            const uint32_t gc = g < last_group ? g : last_group;
+#pragma unroll
+            for (uint32_t c = 0; c < 2U; ++c)
+                copy16_to_lds(ssrc[c] + static_cast<size_t>(gc) * 32U, s_tile + (g & 1U) * (kPfTile * 64U) + 4096U * c + 1024U * wave);
+        };
+        // 5 operations: a super-block's header and the thread's 16 quant bytes of each of its four steps, issued together
+        // (they touch the same two or three cache lines)
+        const auto fetch = [&](uint32_t b, PfRaw& r) {
+            const uint8_t* blk = wrow + static_cast<size_t>(b < last_block ? b : last_block) * 144U;
+            const uint8_t* quants = blk + 16U + 16U * half;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.hd) : "v"(blk) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.qs[0]) : "v"(quants) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=v"(r.qs[1]) : "v"(quants) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off offset:64" : "=v"(r.qs[2]) : "v"(quants) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off offset:96" : "=v"(r.qs[3]) : "v"(quants) : "memory");
+        };
+        // (p = step % 4 and the step's parity are compile-time constants at every call)
+        const auto stage_weights = [&](uint32_t b, uint32_t p, const u32x4& hd, const u32x4& quants) {
+            const uint32_t sh0 = 16U * (p & 1U), sh1 = sh0 + 8U;
+            const uint32_t fa0 = (hd.y >> sh0) & 255U, fc0 = (hd.w >> sh0) & 255U;
+            const uint32_t fa1 = (hd.y >> sh1) & 255U, fc1 = (hd.w >> sh1) & 255U;
+            const bool low = p < 2U;                          // uniform: p is the same for the whole workgroup
+            const uint32_t s0 = low ? (fa0 & 63U) : ((fc0 & 15U) | ((fa0 >> 6) << 4));
+            const uint32_t s1 = low ? (fa1 & 63U) : ((fc1 & 15U) | ((fa1 >> 6) << 4));
+            const _Float16 c0 = static_cast<_Float16>(static_cast<float>(s0)), c1 = static_cast<_Float16>(static_cast<float>(s1));
+            const _Float16 n0 = static_cast<_Float16>(-1024.0F * static_cast<float>(s0)), n1 = static_cast<_Float16>(-1024.0F * static_cast<float>(s1));
+            const half2v mul0 = {c0, c0}, add0 = {n0, n0}, mul1 = {c1, c1}, add1 = {n1, n1};
+            const uint32_t qs[4] = {quants.x, quants.y, quants.z, quants.w};
+            uint32_t lo[8], hi[8];
+            const auto scaled = [](uint32_t bytes, uint32_t sel, half2v mul, half2v add) {
+                // two nibbles -> (1024 + q) as fp16 bit patterns -> sc q
+                const uint32_t two = (__builtin_amdgcn_perm(0U, bytes, sel) & 0x000f000fU) | 0x64006400U;
+                return __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(half2v, two), mul, add));
+            };
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t w = qs[i], w4 = w >> 4;
+                lo[2 * i] = scaled(w, 0x0c010c00U, mul0, add0); lo[2 * i + 1] = scaled(w, 0x0c030c02U, mul0, add0);
+                hi[2 * i] = scaled(w4, 0x0c010c00U, mul1, add1); hi[2 * i + 1] = scaled(w4, 0x0c030c02U, mul1, add1);
+            }
+            uint8_t* tile_w = w_tile[p & 1U];
+            *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 2U * half)) = u32x4{lo[0], lo[1], lo[2], lo[3]};
+            *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 2U * half + 1U)) = u32x4{lo[4], lo[5], lo[6], lo[7]};
+            *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 4U + 2U * half)) = u32x4{hi[0], hi[1], hi[2], hi[3]};
+            *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 5U + 2U * half)) = u32x4{hi[4], hi[5], hi[6], hi[7]};
+            if (p == 0) {
+                if (half == 0) d_scale[b & 1U][lrow] = half_bits_to_float(hd.x & 0xffffU);
+                // -(dmin m_j) of this super-block's eight sub-blocks: sub-blocks 8 (b % 2) .. + 8 of the group
+                uint8_t* mrow = m_tile[(b >> 1) & 1U] + lrow * 64U;
+                if ((b & 1U) == half) {
+                    const float dm = -half_bits_to_float(hd.x >> 16);
+                    uint32_t mh[4], ml[4];
+#pragma unroll
+                    for (int j = 0; j < 8; j += 2) {
+                        float v[2];
+#pragma unroll
+                        for (int jj = 0; jj < 2; ++jj) {
+                            const uint32_t sh = 8U * ((j + jj) & 3U);
+                            const uint32_t mn = (j + jj) < 4 ? ((hd.z >> sh) & 63U) : (((hd.w >> (sh + 4U)) & 15U) | (((hd.z >> (sh + 6U)) & 3U) << 4));
+                            v[jj] = dm * static_cast<float>(mn);
+                        }
+                        const half2v h = __builtin_convertvector(float2v{v[0], v[1]}, half2v);
+                        mh[j / 2] = __builtin_bit_cast(uint32_t, h);
+                        ml[j / 2] = pack_half2(v[0] - static_cast<float>(h.x), v[1] - static_cast<float>(h.y));
+                    }
+                    *reinterpret_cast<u32x4*>(mrow + 16U * half) = u32x4{mh[0], mh[1], mh[2], mh[3]};
+                    *reinterpret_cast<u32x4*>(mrow + 32U + 16U * half) = u32x4{ml[0], ml[1], ml[2], ml[3]};
+                } else if ((b & 1U) == 0 && b + 1U == blocks) {   // odd count: the last group's second super-block does not exist
+                    *reinterpret_cast<u32x4*>(mrow + 16U * half) = u32x4{0U, 0U, 0U, 0U};
+                    *reinterpret_cast<u32x4*>(mrow + 32U + 16U * half) = u32x4{0U, 0U, 0U, 0U};
+                }
+            }
+        };
 
-    floatx16 acc[2][2];                           // [row tile][token tile] of the wave's 64 x 64 quarter
+        // Schedule of one step (u = step % 8, super-block slot = (step / 4) % 2):
+        //   [u == 0: sums copy of the next group] [token copy of step + 3] [u == 3, 7: wait for the slot staged next]
+        //   stage step + 1   [u == 2, 6: fetch of the super-block two ahead into the slot just used up]
+        //   wait for the token copy of step + 1, barrier.
+        // Operations per step: 4 (+ 2 at u == 0, + 5 at u == 2, 6). The prologue issues the same sequence as steps
+        // u = 5, 6, 7 of an iteration before the first, so the counts below hold from the first step on.
+        PfRaw raw[2];
+        copy_sums(0);
+        fetch(0, raw[0]);
+        copy_tokens(0, tok_stage[0]);
+        copy_tokens(1, tok_stage[1]);
+        fetch(1, raw[1]);
+        copy_tokens(2, tok_stage[2]);
+        // younger than the first token copy: 4 + 5 + 4; the first fetch is older still
+        asm volatile("s_waitcnt vmcnt(13)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]) : : "memory");
+        stage_weights(0, 0, raw[0].hd, raw[0].qs[0]);
+        pf_barrier();
+        for (uint32_t s0 = 0; s0 < steps8; s0 += 8U) {
+            const uint32_t b0 = s0 >> 2;
+#pragma unroll
+            for (uint32_t u = 0; u < 8U; ++u) {
+                const uint32_t s = s0 + u;
+                if (u == 0) copy_sums((s >> 3) + 1U);
+                copy_tokens(s + kPfTokenAhead, tok_stage[(u + kPfTokenAhead) & 3U]);
+                // the slot fetched at u == 6 of the previous iteration (u == 2 of this one): younger operations
+                // 4 + 6 + 4 + 9 + 4 = 27 (4 + 4 + 4 + 9 + 4 = 25)
+                if (u == 3U) asm volatile("s_waitcnt vmcnt(27)" : "+v"(raw[1].hd), "+v"(raw[1].qs[0]), "+v"(raw[1].qs[1]), "+v"(raw[1].qs[2]), "+v"(raw[1].qs[3]) : : "memory");
+                if (u == 7U) asm volatile("s_waitcnt vmcnt(25)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]) : : "memory");
+                if (s < last) stage_weights((s + 1U) >> 2, (u + 1U) & 3U, raw[((u + 1U) >> 2) & 1U].hd, raw[((u + 1U) >> 2) & 1U].qs[(u + 1U) & 3U]);
+                if (u == 2U) fetch(b0 + 2U, raw[0]);
+                if (u == 6U) fetch(b0 + 3U, raw[1]);
+                // the token copy of step s + 1 was issued in step s - 2; younger operations: a fetch in that step, then
+                // the whole of steps s - 1 and s
+                const uint32_t per_step[8] = {6, 4, 9, 4, 4, 4, 9, 4}, fetch_after[8] = {0, 0, 5, 0, 0, 0, 5, 0};
+                switch (fetch_after[(u + 6U) & 7U] + per_step[(u + 7U) & 7U] + per_step[u]) {   // a constant once the loop is unrolled
+                case 8: wait_copies<8>(); break;
+                case 10: wait_copies<10>(); break;
+                case 13: wait_copies<13>(); break;
+                case 15: wait_copies<15>(); break;
+                default: wait_copies<0>(); break;
+                }
+                pf_barrier();
+            }
+        }
+        return;
+    }
+
+    // ---- multipliers: wave (wr, wc) owns tile rows 64 wr .. + 64 (two tiles of 32 features) x tokens 64 wc .. + 64
+    floatx16 acc[2][2], part[2][2];                // [token tile][feature tile]
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int n = 0; n < 2; ++n)
 #pragma unroll
-            for (int j = 0; j < 16; ++j) acc[i][n][j] = 0.0F;
-    const uint32_t wr = wave >> 1, wc = wave & 1U;
-
-    const uint32_t arow = lane & 31U, kq = (lane >> 5) * 16U;     // MFMA operand role: row / token lane & 31, 8 halves at k = 8 (lane / 32)
-    PfRaw raw;
-    if (loader) {
-        fetch(0, raw);
-        stage(0, raw, 0);
-        if (steps > 1U) fetch(1, raw);
-    }
-    __syncthreads();
-    for (uint32_t s = 0; s < steps; ++s) {
-        const uint32_t buf = s & 1U;
-        if (loader) {
-            if (s + 1U < steps) {
-                stage(s + 1U, raw, buf ^ 1U);                 // operands fetched during the previous step
-                if (s + 2U < steps) fetch(s + 2U, raw);       // in flight during the next step
-            }
-        } else {
-            const uint8_t* ta = tile_a[buf][0] + (64U * wr + arow) * kPfPitch + kq;
-            const uint8_t* tl = tile_a[buf][1] + (64U * wr + arow) * kPfPitch + kq;
-            const uint8_t* tb = tile_b[buf] + (64U * wc + arow) * kPfPitch + kq;
+            for (int j = 0; j < 16; ++j) { acc[i][n][j] = 0.0F; part[i][n][j] = 0.0F; }
+    const uint32_t wr = wave >> 1, wc = wave & 1U, l31 = lane & 31U, upper = lane >> 5;
+    const uint32_t trow = (64U * wc + l31) * 128U, frow = (64U * wr + l31) * 128U, sw = l31 & 7U;
+    uint32_t piece_at[4];
 #pragma unroll
-            for (uint32_t ks = 0; ks < 4U; ++ks) {
-                half8 b[2], wl[2], wh[2];
+    for (uint32_t ks = 0; ks < 4U; ++ks) piece_at[ks] = ((2U * ks + upper) ^ sw) << 4;
+    // token tiles of this wave that hold any row of the item (the others are neither read nor multiplied)
+    const uint32_t live_tiles = count > 64U * wc ? (count - 64U * wc + 31U) / 32U : 0U;
+    pf_barrier();
+    for (uint32_t s0 = 0; s0 < steps8; s0 += 4U) {
+        if (s0 >= steps) {                                    // idle steps of an odd K: keep the barrier count of the loaders
 #pragma unroll
-                for (uint32_t i = 0; i < 2U; ++i) {
-                    b[i] = *reinterpret_cast<const half8*>(tb + i * 32U * kPfPitch + 32U * ks);
-                    wl[i] = *reinterpret_cast<const half8*>(tl + i * 32U * kPfPitch + 32U * ks);
-                    wh[i] = *reinterpret_cast<const half8*>(ta + i * 32U * kPfPitch + 32U * ks);
-                }
-                // low planes first: consecutive MFMAs never wait for each other's accumulator
-#pragma unroll
-                for (uint32_t i = 0; i < 2U; ++i)
-#pragma unroll
-                    for (uint32_t n = 0; n < 2U; ++n) acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wl[i], b[n], acc[i][n], 0, 0, 0);
-#pragma unroll
-                for (uint32_t i = 0; i < 2U; ++i)
-#pragma unroll
-                    for (uint32_t n = 0; n < 2U; ++n) acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[i], b[n], acc[i][n], 0, 0, 0);
-            }
+            for (uint32_t p = 0; p < 4U; ++p) pf_barrier();
+            continue;
         }
-        __syncthreads();
+#pragma unroll
+        for (uint32_t p = 0; p < 4U; ++p) {
+            const uint32_t s = s0 + p;
+            const pf_lds* tok = tok_stage[p] + trow;
+            const uint8_t* wt = w_tile[s & 1U] + frow;
+            // the operands of k-step ks + 1 are read during the MFMAs of ks
+            const auto k_steps = [&](auto tiles_constant) {
+                constexpr uint32_t NT = decltype(tiles_constant)::value;
+                half8 x[2][NT], w[2][2];
+                const auto read = [&](uint32_t ks, half8 (&xs)[NT], half8 (&ws)[2]) {
+#pragma unroll
+                    for (uint32_t i = 0; i < NT; ++i) xs[i] = *reinterpret_cast<const __attribute__((address_space(3))) half8*>(tok + i * 32U * 128U + piece_at[ks]);
+#pragma unroll
+                    for (uint32_t n = 0; n < 2U; ++n) ws[n] = *reinterpret_cast<const half8*>(wt + n * 32U * 128U + piece_at[ks]);
+                };
+                read(0, x[0], w[0]);
+#pragma unroll
+                for (uint32_t ks = 0; ks < 4U; ++ks) {
+                    if (ks < 3U) read(ks + 1U, x[(ks + 1U) & 1U], w[(ks + 1U) & 1U]);
+                    __builtin_amdgcn_sched_barrier(0);        // the reads of ks + 1 stay ahead of the MFMAs of ks
+#pragma unroll
+                    for (uint32_t i = 0; i < NT; ++i)
+#pragma unroll
+                        for (uint32_t n = 0; n < 2U; ++n) part[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks & 1U][i], w[ks & 1U][n], part[i][n], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            if (live_tiles >= 2U) k_steps(std::integral_constant<uint32_t, 2>{});
+            else if (live_tiles == 1U) k_steps(std::integral_constant<uint32_t, 1>{});
+            if (p == 3U) {
+                // end of a super-block: running sum += d * P, P = 0
+                const uint32_t b = s >> 2;
+                const float d[2] = {d_scale[b & 1U][64U * wr + l31], d_scale[b & 1U][64U * wr + 32U + l31]};
+#pragma unroll
+                for (uint32_t i = 0; i < 2U; ++i)
+#pragma unroll
+                    for (uint32_t n = 0; n < 2U; ++n)
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) {
+                            acc[i][n][j] = __builtin_fmaf(d[n], part[i][n][j], acc[i][n][j]);
+                            part[i][n][j] = 0.0F;
+                        }
+                if (((b & 1U) || b + 1U == blocks) && live_tiles != 0) {
+                    // end of a group of 16 sub-blocks: running sum += S hi * M hi + S lo * M hi + S hi * M lo
+                    const uint32_t g = b >> 1;
+                    const pf_lds* st = s_tile + (g & 1U) * (kPfTile * 64U) + (64U * wc + l31) * 64U + 16U * upper;
+                    const uint8_t* mt = m_tile[g & 1U] + (64U * wr + l31) * 64U + 16U * upper;
+                    half8 sh[2], sl[2], mh[2], ml[2];
+#pragma unroll
+                    for (uint32_t i = 0; i < 2U; ++i) {
+                        sh[i] = *reinterpret_cast<const __attribute__((address_space(3))) half8*>(st + i * 32U * 64U);
+                        sl[i] = *reinterpret_cast<const __attribute__((address_space(3))) half8*>(st + i * 32U * 64U + 32U);
+                        mh[i] = *reinterpret_cast<const half8*>(mt + i * 32U * 64U);
+                        ml[i] = *reinterpret_cast<const half8*>(mt + i * 32U * 64U + 32U);
+                    }
+#pragma unroll
+                    for (uint32_t i = 0; i < 2U; ++i)
+#pragma unroll
+                        for (uint32_t n = 0; n < 2U; ++n) {
+                            acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sh[i], mh[n], acc[i][n], 0, 0, 0);
+                            acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sl[i], mh[n], acc[i][n], 0, 0, 0);
+                            acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sh[i], ml[n], acc[i][n], 0, 0, 0);
+                        }
+                }
+            }
+            pf_barrier();
+        }
     }
-    if (loader) return;
 
-    // C layout of a 32 x 32 tile: lane holds token (lane & 31); register i is weight row 8 (i / 4) + 4 (lane / 32) + i % 4
+    // Result layout of a 32 x 32 tile: the lane holds feature (lane & 31); register j is token 8 (j / 4) + 4 (lane / 32) + j % 4
+    const uint32_t sub_block = (m0 + 32U * wr) / 32U;         // MODE 0: the wave's 32 h values of a token are one sub-block of the down product
 #pragma unroll
-    for (uint32_t nt = 0; nt < 2U; ++nt) {
-        const uint32_t n = 64U * wc + 32U * nt + (lane & 31U);
-        const bool live = n < count;
-        if (MODE == 0) {
-            bool bad = false;
+    for (uint32_t i = 0; i < 2U; ++i) {
 #pragma unroll
-            for (uint32_t i4 = 0; i4 < 4U; ++i4) {
-                float hv[4];
-#pragma unroll
-                for (uint32_t j = 0; j < 4U; ++j) {
-                    const float g = acc[0][nt][4 * i4 + j], u = acc[1][nt][4 * i4 + j];
-                    hv[j] = (g / (1.0F + declared_exp(-g))) * u;
-                    bad = bad || !(finite_f(g) && finite_f(u) && finite_f(hv[j]));
-                }
+        for (uint32_t j = 0; j < 16U; ++j) {
+            const uint32_t n = 64U * wc + 32U * i + 8U * (j / 4U) + 4U * upper + (j & 3U);
+            const bool live = n < count;
+            if (MODE == 0) {
+                const float g = acc[i][0][j], u = acc[i][1][j];
+                const float hv = (g / (1.0F + declared_exp(-g))) * u;
+                const _Float16 h16 = static_cast<_Float16>(hv);
+                float sum = live ? static_cast<float>(h16) : 0.0F;
+                sum += xor1_f(sum); sum += xor2_f(sum); sum += xor4_f(sum); sum += xor8_f(sum); sum += xor16_f(sum);
                 if (live) {
-                    const uint32_t row = m0 + 32U * wr + 8U * i4 + 4U * (lane >> 5);
-                    u32x2 packed = {pack_half2(hv[0], hv[1]), pack_half2(hv[2], hv[3])};
-                    *reinterpret_cast<u32x2*>(a.h + static_cast<size_t>(begin + n) * a.features + row) = packed;
+                    a.h[static_cast<size_t>(begin + n) * a.features + m0 + 32U * wr + l31] = h16;
+                    if (l31 == 0) {
+                        _Float16* sums = reinterpret_cast<_Float16*>(a.h_sums + static_cast<size_t>(begin + n) * pf_sum_row_bytes(a.features));
+                        split_half(sum, sums[sub_block], sums[pf_sum_slots(a.features) + sub_block]);
+                    }
+                    if (!(finite_f(g) && finite_f(u) && finite_f(hv))) {
+                        atomicOr(&a.status[order[begin + n] / a.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                        atomicOr(a.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                    }
                 }
+            } else if (live) {
+                float* out = a.rawdots + static_cast<size_t>(order[begin + n]) * a.features + m0 + 64U * wr + l31;
+                out[0] = acc[i][0][j];
+                out[32] = acc[i][1][j];
             }
-            if (live && bad) {
-                atomicOr(&a.status[order[begin + n] / a.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
-                atomicOr(a.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
-            }
-        } else if (live) {
-            float* out = a.rawdots + static_cast<size_t>(order[begin + n]) * a.features + m0 + 64U * wr;
-#pragma unroll
-            for (uint32_t m = 0; m < 2U; ++m)
-#pragma unroll
-                for (uint32_t i4 = 0; i4 < 4U; ++i4)
-                    *reinterpret_cast<f32x4*>(out + 32U * m + 8U * i4 + 4U * (lane >> 5)) =
-                        f32x4{acc[m][nt][4 * i4], acc[m][nt][4 * i4 + 1], acc[m][nt][4 * i4 + 2], acc[m][nt][4 * i4 + 3]};
         }
     }
 }

@@ -890,6 +890,10 @@ int32_t mi355_moe_route(const mi355_route_policy* p, const void* x, uint32_t kin
     return MI355_OK;
 }
 
+size_t mi355_moe_prefill_f16_workspace_bytes(uint32_t hidden, uint32_t ffn, uint32_t rows, uint32_t top_k) {
+    return pf_workspace_bytes(hidden, ffn, rows, top_k);
+}
+
 size_t mi355_moe_plan_words(uint32_t experts, uint32_t rows, uint32_t top_k) {
     return plan_tickets_at(experts, rows * top_k) + kPlanTicketWords;
 }
@@ -986,21 +990,28 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     STRIX_REQUIRE(r->input_stride % 16U == 0 && aligned(r->input, 16), "moe prefill: input rows must be 16-byte aligned");
     STRIX_REQUIRE(r->h_f16 && aligned(r->h_f16, 16), "moe prefill: h_f16 workspace is null or misaligned");
     STRIX_REQUIRE(rows <= 65535U, "moe prefill: at most 65535 rows per call");
+    STRIX_REQUIRE(wv.hidden % 128U == 0 && wv.ffn % 64U == 0, "moe prefill: hidden must be a multiple of 128, ffn of 64");
     const uint32_t assignments = rows * wv.top_k, bound = plan_item_bound(wv.experts, assignments, kPfTile);
-    STRIX_REQUIRE(bound <= 65535U, "moe prefill: too many work items for one launch");
     hipStream_t st = hs(stream);
     clear_validate_kernel<<<rows, 64, 0, st>>>(r->routes, r->route_weights, wv.experts, wv.top_k, r->status, r->job_status);
     launch_plan(r->routes, wv.experts, assignments, kPfTile, bound, r->plan, st);
     PrefillArgs a{};
     a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.x = static_cast<const uint8_t*>(r->input); a.x_stride = r->input_stride;
-    a.h = static_cast<_Float16*>(r->h_f16); a.rawdots = r->rawdots; a.plan = r->plan; a.experts = wv.experts; a.assignments = assignments;
-    a.status = r->status; a.job_status = r->job_status;
-    const uint32_t items_at = plan_items_at(wv.experts, assignments), order_at = plan_order_at(wv.experts);
+    uint8_t* ws = static_cast<uint8_t*>(r->h_f16);
+    a.h = reinterpret_cast<_Float16*>(ws); a.h_sums = ws + pf_h_bytes(assignments, wv.ffn);
+    uint8_t* x_sums = a.h_sums + static_cast<size_t>(assignments) * pf_sum_row_bytes(wv.ffn);
+    a.x_sums = x_sums;
+    a.rawdots = r->rawdots; a.plan = r->plan; a.experts = wv.experts; a.assignments = assignments;
+    a.status = r->status; a.job_status = r->job_status; a.items = bound;
+    token_sums_kernel<<<rows, 256, 0, st>>>(a.x, a.x_stride, wv.hidden, x_sums);
+    if (pf_sum_slots(wv.ffn) != wv.ffn / 32U) clear_sum_padding_kernel<<<assignments, 64, 0, st>>>(a.h_sums, wv.ffn);
+    const uint32_t items_at = plan_items_at(wv.experts, assignments), order_at = plan_order_at(wv.experts), item_slots = (bound + 7U) / 8U * 8U;
     a.wa = wv.gate; a.wb = wv.up; a.expert_stride = wv.gate_expert_stride; a.row_stride = wv.gate_row_stride; a.k = wv.hidden; a.features = wv.ffn;
-    prefill_f16_kernel<0><<<dim3(wv.ffn / 64U, bound), 512, 0, st>>>(a, items_at, order_at);
+    a.tiles = wv.ffn / 64U;
+    prefill_f16_kernel<0><<<item_slots * a.tiles, 512, 0, st>>>(a, items_at, order_at);
     a.wa = wv.down; a.wb = nullptr; a.expert_stride = wv.down_expert_stride; a.row_stride = wv.down_row_stride; a.k = wv.ffn; a.features = wv.hidden;
-    STRIX_REQUIRE(wv.hidden % 128U == 0, "moe prefill: hidden must be a multiple of 128");
-    prefill_f16_kernel<1><<<dim3(wv.hidden / 128U, bound), 512, 0, st>>>(a, items_at, order_at);
+    a.tiles = wv.hidden / 128U;
+    prefill_f16_kernel<1><<<item_slots * a.tiles, 512, 0, st>>>(a, items_at, order_at);
     STRIX_LAUNCHED("moe prefill f16");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }

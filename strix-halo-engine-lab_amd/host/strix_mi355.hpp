@@ -57,6 +57,9 @@ using Weights = mi355_moe_weights;    // gate / up [experts][ffn][hidden/256 blo
 inline std::size_t plan_words(std::uint32_t experts, std::uint32_t rows, std::uint32_t top_k) {
     return mi355_moe_plan_words(experts, rows, top_k);
 }
+inline std::size_t prefill_f16_workspace_bytes(std::uint32_t hidden, std::uint32_t ffn, std::uint32_t rows, std::uint32_t top_k) {
+    return mi355_moe_prefill_f16_workspace_bytes(hidden, ffn, rows, top_k);
+}
 inline void enqueue_prologue(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) { check(mi355_moe_enqueue_prologue(&w, &r, rows, s)); }
 inline void enqueue_csr(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) { check(mi355_moe_enqueue_csr(&w, &r, rows, s)); }
 inline void enqueue_project(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) { check(mi355_moe_enqueue_project(&w, &r, rows, s)); }
