@@ -164,7 +164,7 @@ def extra_configs(strix, torch, steps, warmup):
         "TFLOPs": (flops_experts + flops_router) / (sec_f16 + sec_route) / 1e12, "experts_TFLOPs": flops_experts / sec_f16 / 1e12,
         "frac_of_fp16_mfma_peak": (flops_experts + flops_router) / (sec_f16 + sec_route) / 2.5e15,
         "experts_frac_of_fp16_mfma_peak": flops_experts / sec_f16 / 2.5e15, "algorithmic_flops": flops_experts + flops_router,
-        "note": "routed experts on fp16 MFMA (weights as fp16 hi + lo, fp32 accumulation) + exact-order router; FAST class, tolerance 2e-3"}
+        "note": "routed experts on fp16 MFMA (exact integer operands sc*q, fp32 block scales, fp32 accumulation) + exact-order router; FAST class, tolerance 2e-3"}
     sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 2, 1)
     out["config4_prefill_T4096_integer_class"] = {
         "ms": sec * 1e3, "TFLOPs": (flops_experts + flops_router) / sec / 1e12, "algorithmic_flops": flops_experts + flops_router,

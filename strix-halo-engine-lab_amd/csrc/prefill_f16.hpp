@@ -215,6 +215,11 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
             asm volatile("global_load_dwordx4 %0, %1, off offset:64" : "=v"(r.qs[2]) : "v"(quants) : "memory");
             asm volatile("global_load_dwordx4 %0, %1, off offset:96" : "=v"(r.qs[3]) : "v"(quants) : "memory");
         };
+        // the two constants of the nibble expansion, kept in registers so that mask-and-merge is one v_and_or_b32
+        // (as immediates the instruction cannot encode them and the compiler emits two)
+        uint32_t nibble_mask, magic_1024;
+        asm volatile("s_mov_b32 %0, 0x000f000f" : "=s"(nibble_mask));
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic_1024));
         // (p = step % 4 and the step's parity are compile-time constants at every call)
         const auto stage_weights = [&](uint32_t b, uint32_t p, const u32x4& hd, const u32x4& quants) {
             const uint32_t sh0 = 16U * (p & 1U), sh1 = sh0 + 8U;
@@ -228,9 +233,9 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
             const half2v mul0 = {c0, c0}, add0 = {n0, n0}, mul1 = {c1, c1}, add1 = {n1, n1};
             const uint32_t qs[4] = {quants.x, quants.y, quants.z, quants.w};
             uint32_t lo[8], hi[8];
-            const auto scaled = [](uint32_t bytes, uint32_t sel, half2v mul, half2v add) {
+            const auto scaled = [&](uint32_t bytes, uint32_t sel, half2v mul, half2v add) {
                 // two nibbles -> (1024 + q) as fp16 bit patterns -> sc q
-                const uint32_t two = (__builtin_amdgcn_perm(0U, bytes, sel) & 0x000f000fU) | 0x64006400U;
+                const uint32_t two = (__builtin_amdgcn_perm(0U, bytes, sel) & nibble_mask) | magic_1024;
                 return __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(half2v, two), mul, add));
             };
 #pragma unroll
@@ -413,6 +418,16 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
 
     // Result layout of a 32 x 32 tile: the lane holds feature (lane & 31); register j is token 8 (j / 4) + 4 (lane / 32) + j % 4
     const uint32_t sub_block = (m0 + 32U * wr) / 32U;         // MODE 0: the wave's 32 h values of a token are one sub-block of the down product
+    uint32_t dest[2][16];                                     // MODE 1: the assignment of every token of the lane, read ahead of all stores
+    if (MODE == 1) {
+#pragma unroll
+        for (uint32_t i = 0; i < 2U; ++i)
+#pragma unroll
+            for (uint32_t j = 0; j < 16U; ++j) {
+                const uint32_t n = 64U * wc + 32U * i + 8U * (j / 4U) + 4U * upper + (j & 3U);
+                dest[i][j] = order[begin + (n < count ? n : count - 1U)];
+            }
+    }
 #pragma unroll
     for (uint32_t i = 0; i < 2U; ++i) {
 #pragma unroll
@@ -437,7 +452,7 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
                     }
                 }
             } else if (live) {
-                float* out = a.rawdots + static_cast<size_t>(order[begin + n]) * a.features + m0 + 64U * wr + l31;
+                float* out = a.rawdots + static_cast<size_t>(dest[i][j]) * a.features + m0 + 64U * wr + l31;
                 out[0] = acc[i][0][j];
                 out[32] = acc[i][1][j];
             }
