@@ -50,6 +50,8 @@ constexpr uint32_t kPfTile = 128;                 // weight rows and tokens per 
 constexpr uint32_t kPfStep = 64;                  // K per step
 constexpr uint32_t kPfTileBytes = kPfTile * 128U; // one step of a tile: 128 rows x 64 halves
 constexpr uint32_t kPfRing = 4;                   // token stages (separate LDS objects: stage = step % 4)
+constexpr uint32_t kPfTokenTiles = 2;                // 32-token tiles per multiplier wave: 8 / kPfTokenTiles multiplier waves
+constexpr uint32_t kPfThreads = 256U + 64U * (8U / kPfTokenTiles);
 constexpr uint32_t kPfTokenAhead = 3;             // steps between a token copy and its use
 
 // sub-block sums of a row: two fp16 planes (hi, lo) of `pf_sum_slots(k)` halves each, the slots past k / 32 zero
@@ -137,7 +139,7 @@ __device__ __forceinline__ uint32_t pf_at(uint32_t row, uint32_t piece) { return
 struct PfRaw { u32x4 hd, qs[4]; };           // one super-block of a weight row: header and the thread's 16 quant bytes of its four steps
 
 template <int MODE>
-__global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_t items_at, uint32_t order_at) {
+__global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, uint32_t items_at, uint32_t order_at) {
     __shared__ __attribute__((aligned(16))) uint8_t tok0[kPfTileBytes];                     // token steps: stage s % 4
     __shared__ __attribute__((aligned(16))) uint8_t tok1[kPfTileBytes];
     __shared__ __attribute__((aligned(16))) uint8_t tok2[kPfTileBytes];
@@ -159,7 +161,7 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
     if (MODE == 1 && (*a.job_status & MI355_STATUS_NONFINITE_PROJECTION)) return;
     const uint32_t* order = a.plan + order_at;
     const bool loader = threadIdx.x < 256U;
-    const uint32_t t = threadIdx.x & 255U, lane = t & 63U, wave = t >> 6;      // index within the role
+    const uint32_t t = loader ? threadIdx.x : threadIdx.x - 256U, lane = t & 63U, wave = t >> 6;      // index within the role
     const uint32_t m0 = tile * (MODE == 0 ? 64U : 128U);
     const uint32_t steps = a.k / kPfStep, blocks = a.k / 256U, steps8 = (steps + 7U) & ~7U;
     const size_t sum_row = pf_sum_row_bytes(a.k);
@@ -325,21 +327,22 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
         return;
     }
 
-    // ---- multipliers: wave (wr, wc) owns tile rows 64 wr .. + 64 (two tiles of 32 features) x tokens 64 wc .. + 64
-    floatx16 acc[2][2], part[2][2];                // [token tile][feature tile]
+    // ---- multipliers: wave (wr, wc) owns tile rows 64 wr .. + 64 (two tiles of 32 features) x tokens TS wc .. + TS
+    constexpr uint32_t TT = kPfTokenTiles, TS = 32U * TT;
+    floatx16 acc[TT][2], part[TT][2];              // [token tile][feature tile]
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < static_cast<int>(TT); ++i)
 #pragma unroll
         for (int n = 0; n < 2; ++n)
 #pragma unroll
             for (int j = 0; j < 16; ++j) { acc[i][n][j] = 0.0F; part[i][n][j] = 0.0F; }
-    const uint32_t wr = wave >> 1, wc = wave & 1U, l31 = lane & 31U, upper = lane >> 5;
-    const uint32_t trow = (64U * wc + l31) * 128U, frow = (64U * wr + l31) * 128U, sw = l31 & 7U;
+    const uint32_t wr = wave / (4U / TT), wc = wave % (4U / TT), l31 = lane & 31U, upper = lane >> 5;
+    const uint32_t trow = (TS * wc + l31) * 128U, frow = (64U * wr + l31) * 128U, sw = l31 & 7U;
     uint32_t piece_at[4];
 #pragma unroll
     for (uint32_t ks = 0; ks < 4U; ++ks) piece_at[ks] = ((2U * ks + upper) ^ sw) << 4;
     // token tiles of this wave that hold any row of the item (the others are neither read nor multiplied)
-    const uint32_t live_tiles = count > 64U * wc ? (count - 64U * wc + 31U) / 32U : 0U;
+    const uint32_t live_tiles = count > TS * wc ? (count - TS * wc + 31U) / 32U : 0U;
     pf_barrier();
     for (uint32_t s0 = 0; s0 < steps8; s0 += 4U) {
         if (s0 >= steps) {                                    // idle steps of an odd K: keep the barrier count of the loaders
@@ -374,14 +377,14 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
                     __builtin_amdgcn_sched_barrier(0);
                 }
             };
-            if (live_tiles >= 2U) k_steps(std::integral_constant<uint32_t, 2>{});
+            if (live_tiles >= TT) k_steps(std::integral_constant<uint32_t, TT>{});
             else if (live_tiles == 1U) k_steps(std::integral_constant<uint32_t, 1>{});
             if (p == 3U) {
                 // end of a super-block: running sum += d * P, P = 0
                 const uint32_t b = s >> 2;
                 const float d[2] = {d_scale[b & 1U][64U * wr + l31], d_scale[b & 1U][64U * wr + 32U + l31]};
 #pragma unroll
-                for (uint32_t i = 0; i < 2U; ++i)
+                for (uint32_t i = 0; i < TT; ++i)
 #pragma unroll
                     for (uint32_t n = 0; n < 2U; ++n)
 #pragma unroll
@@ -392,18 +395,21 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
                 if (((b & 1U) || b + 1U == blocks) && live_tiles != 0) {
                     // end of a group of 16 sub-blocks: running sum += S hi * M hi + S lo * M hi + S hi * M lo
                     const uint32_t g = b >> 1;
-                    const pf_lds* st = s_tile + (g & 1U) * (kPfTile * 64U) + (64U * wc + l31) * 64U + 16U * upper;
+                    const pf_lds* st = s_tile + (g & 1U) * (kPfTile * 64U) + (TS * wc + l31) * 64U + 16U * upper;
                     const uint8_t* mt = m_tile[g & 1U] + (64U * wr + l31) * 64U + 16U * upper;
-                    half8 sh[2], sl[2], mh[2], ml[2];
+                    half8 sh[TT], sl[TT], mh[2], ml[2];
 #pragma unroll
-                    for (uint32_t i = 0; i < 2U; ++i) {
+                    for (uint32_t i = 0; i < TT; ++i) {
                         sh[i] = *reinterpret_cast<const __attribute__((address_space(3))) half8*>(st + i * 32U * 64U);
                         sl[i] = *reinterpret_cast<const __attribute__((address_space(3))) half8*>(st + i * 32U * 64U + 32U);
-                        mh[i] = *reinterpret_cast<const half8*>(mt + i * 32U * 64U);
-                        ml[i] = *reinterpret_cast<const half8*>(mt + i * 32U * 64U + 32U);
                     }
 #pragma unroll
-                    for (uint32_t i = 0; i < 2U; ++i)
+                    for (uint32_t n = 0; n < 2U; ++n) {
+                        mh[n] = *reinterpret_cast<const half8*>(mt + n * 32U * 64U);
+                        ml[n] = *reinterpret_cast<const half8*>(mt + n * 32U * 64U + 32U);
+                    }
+#pragma unroll
+                    for (uint32_t i = 0; i < TT; ++i)
 #pragma unroll
                         for (uint32_t n = 0; n < 2U; ++n) {
                             acc[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sh[i], mh[n], acc[i][n], 0, 0, 0);
@@ -418,21 +424,21 @@ __global__ __launch_bounds__(512) void prefill_f16_kernel(PrefillArgs a, uint32_
 
     // Result layout of a 32 x 32 tile: the lane holds feature (lane & 31); register j is token 8 (j / 4) + 4 (lane / 32) + j % 4
     const uint32_t sub_block = (m0 + 32U * wr) / 32U;         // MODE 0: the wave's 32 h values of a token are one sub-block of the down product
-    uint32_t dest[2][16];                                     // MODE 1: the assignment of every token of the lane, read ahead of all stores
+    uint32_t dest[TT][16];                                     // MODE 1: the assignment of every token of the lane, read ahead of all stores
     if (MODE == 1) {
 #pragma unroll
-        for (uint32_t i = 0; i < 2U; ++i)
+        for (uint32_t i = 0; i < TT; ++i)
 #pragma unroll
             for (uint32_t j = 0; j < 16U; ++j) {
-                const uint32_t n = 64U * wc + 32U * i + 8U * (j / 4U) + 4U * upper + (j & 3U);
+                const uint32_t n = TS * wc + 32U * i + 8U * (j / 4U) + 4U * upper + (j & 3U);
                 dest[i][j] = order[begin + (n < count ? n : count - 1U)];
             }
     }
 #pragma unroll
-    for (uint32_t i = 0; i < 2U; ++i) {
+    for (uint32_t i = 0; i < TT; ++i) {
 #pragma unroll
         for (uint32_t j = 0; j < 16U; ++j) {
-            const uint32_t n = 64U * wc + 32U * i + 8U * (j / 4U) + 4U * upper + (j & 3U);
+            const uint32_t n = TS * wc + 32U * i + 8U * (j / 4U) + 4U * upper + (j & 3U);
             const bool live = n < count;
             if (MODE == 0) {
                 const float g = acc[i][0][j], u = acc[i][1][j];
