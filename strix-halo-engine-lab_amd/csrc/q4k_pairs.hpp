@@ -36,22 +36,25 @@ struct PairArgs {
 };
 
 constexpr uint32_t kPairBlocks = 4;                              // super-blocks per stage
-template <int AL> constexpr uint32_t pair_rows() { return 16U / AL; }
-template <int AL> constexpr uint32_t pair_weight_copies() { return (pair_rows<AL>() * 9U * kPairBlocks + 63U) / 64U; }
-template <int NA, int AL> constexpr uint32_t pair_copies() { return pair_weight_copies<AL>() + NA * AL + 2U * ((NA * AL + 7U) / 8U); }
-template <int NA, int AL> constexpr uint32_t pair_slot_bytes() {
-    return pair_weight_copies<AL>() * 1024U + NA * AL * 1024U + 2U * ((NA * AL + 7U) / 8U) * 1024U;
+// KL = 4 spreads the four super-blocks of a stage over four lanes as well (lane = (al, r, p, k), k in the low two bits):
+// a quarter of the rows and of the instruction stream per wavefront, four times the wavefronts. The lanes of a quad then
+// add their terms to the pair accumulator in super-block order (quad broadcasts), which keeps the reference's sum.
+template <int AL, int KL = 1> constexpr uint32_t pair_rows() { return 16U / (AL * KL); }
+template <int AL, int KL = 1> constexpr uint32_t pair_weight_copies() { return (pair_rows<AL, KL>() * 9U * kPairBlocks + 63U) / 64U; }
+template <int NA, int AL, int KL = 1> constexpr uint32_t pair_copies() { return pair_weight_copies<AL, KL>() + NA * AL + 2U * ((NA * AL + 7U) / 8U); }
+template <int NA, int AL, int KL = 1> constexpr uint32_t pair_slot_bytes() {
+    return pair_weight_copies<AL, KL>() * 1024U + NA * AL * 1024U + 2U * ((NA * AL + 7U) / 8U) * 1024U;
 }
 
-template <int NA, int AL>
+template <int NA, int AL, int KL = 1>
 struct PairSource {
-    static constexpr uint32_t WC = pair_weight_copies<AL>(), B = NA * AL, SC = (B + 7U) / 8U;
+    static constexpr uint32_t WC = pair_weight_copies<AL, KL>(), B = NA * AL, SC = (B + 7U) / 8U;
     const uint8_t* wp[WC];       // weight pieces
     const uint8_t* cp[B];        // activation codes: 16 bytes of row a per lane
     const uint8_t* dp[SC];       // deltas: lane l carries 16 bytes of row l / 8 (+ 8 per further copy)
     const uint8_t* sp[SC];
     __device__ __forceinline__ void init(const uint8_t* rows_base, uint32_t row_stride, const A8Image& img, uint32_t nacts) {
-        const uint32_t lane = threadIdx.x & 63U, total = pair_rows<AL>() * 36U;
+        const uint32_t lane = threadIdx.x & 63U, total = pair_rows<AL, KL>() * 36U;
 #pragma unroll
         for (uint32_t i = 0; i < WC; ++i) {
             uint32_t j = i * 64U + lane;
@@ -100,19 +103,21 @@ struct PairSource {
 };
 
 // The 4 super-blocks of one landed stage: the lane's (row r, pair p) against its NA activation rows.
-template <int NA, int AL>
+template <int NA, int AL, int KL = 1>
 __device__ __forceinline__ void pair_stage_compute(const lds_u8* slot, float (&acc)[NA]) {
     typedef const __attribute__((address_space(3))) u32x4 lds_u32x4;
     typedef const __attribute__((address_space(3))) float lds_f32;
     typedef const __attribute__((address_space(3))) int32_t lds_i32;
-    constexpr uint32_t WC = pair_weight_copies<AL>(), B = NA * AL, SC = (B + 7U) / 8U;
-    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, r = (lane >> 2) & (pair_rows<AL>() - 1U), al = lane / (4U * pair_rows<AL>());
+    constexpr uint32_t WC = pair_weight_copies<AL, KL>(), B = NA * AL, SC = (B + 7U) / 8U, RW = pair_rows<AL, KL>();
+    const uint32_t lane = threadIdx.x & 63U, kl = KL == 4 ? lane & 3U : 0U, pl = KL == 4 ? lane >> 2 : lane;
+    const uint32_t p = pl & 3U, r = (pl >> 2) & (RW - 1U), al = pl / (4U * RW);
     const lds_u8* wrow = slot + r * 576U;
     const lds_u8* codes = slot + 1024U * WC;
     const lds_u8* deltas = slot + 1024U * (WC + B);
     const lds_u8* sums = slot + 1024U * (WC + B + SC);
 #pragma unroll
-    for (uint32_t b = 0; b < kPairBlocks; ++b) {
+    for (uint32_t bb = 0; bb < kPairBlocks / KL; ++bb) {
+        const uint32_t b = KL == 4 ? kl : bb;                  // KL = 4: the lane's own super-block of the stage
         // piece c of the row sits at slot (c + r) % 36
         uint32_t t0 = 9U * b + r, t1 = 9U * b + 1U + 2U * p + r, t2 = t1 + 1U;
         t0 = t0 >= 36U ? t0 - 36U : t0; t1 = t1 >= 36U ? t1 - 36U : t1; t2 = t2 >= 36U ? t2 - 36U : t2;
@@ -155,7 +160,16 @@ __device__ __forceinline__ void pair_stage_compute(const lds_u8* slot, float (&a
             const float u0 = D0 * static_cast<float>(dot0), v0 = M0 * f0;
             const float u1 = D1 * static_cast<float>(dot1), v1 = M1 * f1;
             const float x0 = e0 * (u0 - v0), x1 = e1 * (u1 - v1);
-            acc[i] = acc[i] + (x0 + x1);
+            if constexpr (KL == 4) {
+                // the quad's four terms, super-blocks 0..3 of the stage, in that order
+                const int term = __builtin_bit_cast(int, x0 + x1);
+                acc[i] = acc[i] + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(term, 0x00, 0xF, 0xF, true));
+                acc[i] = acc[i] + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(term, 0x55, 0xF, 0xF, true));
+                acc[i] = acc[i] + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(term, 0xAA, 0xF, 0xF, true));
+                acc[i] = acc[i] + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(term, 0xFF, 0xF, 0xF, true));
+            } else {
+                acc[i] = acc[i] + (x0 + x1);
+            }
             // many activation rows: keep the scheduler from hoisting every later row's operands at once (register pressure)
             if (NA > 2 && (i & 1) == 1) __builtin_amdgcn_sched_barrier(0);
         }
@@ -163,18 +177,18 @@ __device__ __forceinline__ void pair_stage_compute(const lds_u8* slot, float (&a
     }
 }
 
-template <int NA, int AL, int DEPTH>
+template <int NA, int AL, int DEPTH, int KL = 1>
 __global__ __launch_bounds__(64, 2) void q4k_pairs_kernel(PairArgs args) {
-    __shared__ __attribute__((aligned(16))) uint8_t ring0[pair_slot_bytes<NA, AL>()];
-    __shared__ __attribute__((aligned(16))) uint8_t ring1[pair_slot_bytes<NA, AL>()];
-    __shared__ __attribute__((aligned(16))) uint8_t ring2[DEPTH > 2 ? pair_slot_bytes<NA, AL>() : 16];
-    __shared__ __attribute__((aligned(16))) uint8_t ring3[DEPTH > 3 ? pair_slot_bytes<NA, AL>() : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t ring0[pair_slot_bytes<NA, AL, KL>()];
+    __shared__ __attribute__((aligned(16))) uint8_t ring1[pair_slot_bytes<NA, AL, KL>()];
+    __shared__ __attribute__((aligned(16))) uint8_t ring2[DEPTH > 2 ? pair_slot_bytes<NA, AL, KL>() : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t ring3[DEPTH > 3 ? pair_slot_bytes<NA, AL, KL>() : 16];
     lds_u8* const ring[4] = {(lds_u8*)ring0, (lds_u8*)ring1, (lds_u8*)ring2, (lds_u8*)ring3};
     if (args.skip_flag && (*args.skip_flag & args.skip_mask)) return;
-    constexpr uint32_t RW = pair_rows<AL>(), PER = pair_copies<NA, AL>();
+    constexpr uint32_t RW = pair_rows<AL, KL>(), PER = pair_copies<NA, AL, KL>();
     const PairMatrix& m = args.m[blockIdx.y];
     const uint32_t row0 = blockIdx.x * RW, stages = args.blocks / kPairBlocks;
-    PairSource<NA, AL> source;
+    PairSource<NA, AL, KL> source;
     source.init(m.w + static_cast<size_t>(row0) * m.row_stride, static_cast<uint32_t>(m.row_stride), args.img, args.nacts);
     float acc[NA];
 #pragma unroll
@@ -190,18 +204,24 @@ __global__ __launch_bounds__(64, 2) void q4k_pairs_kernel(PairArgs args) {
                 const uint32_t last = b + DEPTH - 1U < stages ? b + DEPTH - 1U : stages;
                 wait_stages_ahead<PER>(last - 1U - b);
                 if (b + DEPTH - 1U < stages) source.start(ring[(s + DEPTH - 1) % DEPTH]);
-                pair_stage_compute<NA, AL>(ring[s], acc);
+                pair_stage_compute<NA, AL, KL>(ring[s], acc);
             }
         }
     }
-    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, r = (lane >> 2) & (RW - 1U), al = lane / (4U * RW);
+    const uint32_t lane = threadIdx.x & 63U, kl = KL == 4 ? lane & 3U : 0U, pl = KL == 4 ? lane >> 2 : lane;
+    const uint32_t p = pl & 3U, r = (pl >> 2) & (RW - 1U), al = pl / (4U * RW);
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
         float v = acc[i];
-        v = v + xor1_f(v);          // acc0 + acc1 | acc2 + acc3
-        v = v + xor2_f(v);          // (acc0 + acc1) + (acc2 + acc3)
+        if constexpr (KL == 4) {    // the pair index is lane bits 2, 3
+            v = v + xor4_f(v);
+            v = v + xor8_f(v);
+        } else {
+            v = v + xor1_f(v);      // acc0 + acc1 | acc2 + acc3
+            v = v + xor2_f(v);      // (acc0 + acc1) + (acc2 + acc3)
+        }
         const uint32_t a = al + AL * i;
-        if (p == 0 && a < args.nacts) m.out[static_cast<size_t>(a) * m.out_stride + row0 + r] = v;
+        if (p == 0 && kl == 0 && a < args.nacts) m.out[static_cast<size_t>(a) * m.out_stride + row0 + r] = v;
     }
 }
 

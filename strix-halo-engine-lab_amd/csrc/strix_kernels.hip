@@ -650,23 +650,24 @@ inline void launch_down_nb(const mi355_moe_weights& w, const mi355_moe_rows& r, 
     }
 }
 // ---- dense matrix (one expert, every row uses it): the pair-per-lane sweep ------------------------------------------
-template <int NA, int AL>
+template <int NA, int AL, int KL = 1>
 inline void launch_pairs_depth(const PairArgs& a, uint32_t matrices, hipStream_t st) {
-    const dim3 grid(a.rows / pair_rows<AL>(), matrices);
+    const dim3 grid(a.rows / pair_rows<AL, KL>(), matrices);
     const uint64_t waves = static_cast<uint64_t>(grid.x) * grid.y;
     // 4 slots when every wavefront of the launch is resident with them and the wait counter can express 3 stages ahead
-    const bool deep = 3U * pair_copies<NA, AL>() <= 63U && waves <= 256ULL * (163840U / (4U * pair_slot_bytes<NA, AL>()));
-    if (deep) q4k_pairs_kernel<NA, AL, 4><<<grid, 64, 0, st>>>(a);
-    else q4k_pairs_kernel<NA, AL, 2><<<grid, 64, 0, st>>>(a);
+    const bool deep = 3U * pair_copies<NA, AL, KL>() <= 63U && waves <= 256ULL * (163840U / (4U * pair_slot_bytes<NA, AL, KL>()));
+    if (deep) q4k_pairs_kernel<NA, AL, 4, KL><<<grid, 64, 0, st>>>(a);
+    else q4k_pairs_kernel<NA, AL, 2, KL><<<grid, 64, 0, st>>>(a);
 }
-// nacts <= 8 activation rows. Matrices with few rows spread every row over two activation lanes when there are >= 4 rows
-// of activations, which doubles the wavefronts and halves each one's instruction stream.
+// nacts <= 8 activation rows. A matrix with few rows gives few wavefronts, each with a long instruction stream (the whole
+// of K): such launches spread every row over more lanes - the four super-blocks of a stage over a quad and, with >= 4
+// activation rows, two activation lanes - which multiplies the wavefronts and divides each one's instruction stream.
 inline void launch_pairs(const PairArgs& a, uint32_t matrices, hipStream_t st) {
     const bool narrow = static_cast<uint64_t>(a.rows) * matrices < 16384U;
-    if (a.nacts <= 1U) launch_pairs_depth<1, 1>(a, matrices, st);
-    else if (a.nacts <= 2U) launch_pairs_depth<2, 1>(a, matrices, st);
-    else if (a.nacts <= 4U) { if (narrow) launch_pairs_depth<2, 2>(a, matrices, st); else launch_pairs_depth<4, 1>(a, matrices, st); }
-    else { if (narrow) launch_pairs_depth<4, 2>(a, matrices, st); else launch_pairs_depth<8, 1>(a, matrices, st); }
+    if (a.nacts <= 1U) { if (narrow) launch_pairs_depth<1, 1, 4>(a, matrices, st); else launch_pairs_depth<1, 1>(a, matrices, st); }
+    else if (a.nacts <= 2U) { if (narrow) launch_pairs_depth<2, 1, 4>(a, matrices, st); else launch_pairs_depth<2, 1>(a, matrices, st); }
+    else if (a.nacts <= 4U) { if (narrow) launch_pairs_depth<2, 2, 4>(a, matrices, st); else launch_pairs_depth<4, 1>(a, matrices, st); }
+    else { if (narrow) launch_pairs_depth<4, 2, 4>(a, matrices, st); else launch_pairs_depth<8, 1>(a, matrices, st); }
 }
 // The dense form needs fp32 gate / up rows as workspace (the optional intermediates views) because a wavefront holds
 // 16 rows, not a whole 32-output SwiGLU group.
