@@ -157,7 +157,10 @@ __global__ __launch_bounds__(256) void quantize_a8_kernel(const uint8_t* x, uint
 // One aligned group of 32 lanes per output row: lane l owns the reference's accumulator lane l (groups g = l, l + 32,
 // ... ascending), then the tree32 butterfly. Up to RB activation rows share one sweep of the weight row.
 // Reference: src/cpu/core/reference.cpp:57-84, src/core/integer_math.hpp:11-13,43-47.
-template <int RB>
+// DW: the weight rows are 4-byte aligned. A block (34 bytes: fp16 scale, 32 codes) is then fetched as nine aligned dwords
+// (two 128-bit loads and one 32-bit load) around its codes and shifted into place, instead of seventeen 16-bit loads.
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+template <int RB, bool DW>
 __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v, uint32_t row0) {
     const uint32_t o = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U;
     if (o >= v.count) return;
@@ -171,8 +174,18 @@ __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v, ui
         const unsigned short* b = reinterpret_cast<const unsigned short*>(wrow + static_cast<size_t>(g) * kQ80Block);
         const float scale = half_bits_to_float(b[0]);
         int w[8];
+        if constexpr (DW) {
+            const uint32_t c0 = g * kQ80Block + 2U, shift = c0 & 3U;          // first code byte: 0 or 2 past a dword boundary
+            const uint32_t* dw = reinterpret_cast<const uint32_t*>(wrow) + (c0 >> 2);
+            const u32x4_a4 lo4 = *reinterpret_cast<const u32x4_a4*>(dw), hi4 = *reinterpret_cast<const u32x4_a4*>(dw + 4);
+            const uint32_t last = dw[shift ? 8 : 7];                          // (an aligned block ends with its eighth dword)
+            const uint32_t d[9] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w, last};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) w[i] = static_cast<int>(static_cast<uint32_t>(b[1 + 2 * i]) | (static_cast<uint32_t>(b[2 + 2 * i]) << 16));
+            for (int i = 0; i < 8; ++i) w[i] = static_cast<int>(__builtin_amdgcn_alignbyte(d[i + 1], d[i], shift));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w[i] = static_cast<int>(static_cast<uint32_t>(b[1 + 2 * i]) | (static_cast<uint32_t>(b[2 + 2 * i]) << 16));
+        }
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             if (static_cast<uint32_t>(r) < nr) {
@@ -838,7 +851,16 @@ int32_t mi355_gemv_q8_0_a8(const mi355_q8a8_view* v, mi355_stream stream) {
     STRIX_REQUIRE(aligned(v->codes, 16) && v->x_stride % 32U == 0 && v->x_stride >= v->in, "Q8_0 product: codes must be 16-byte aligned with x_stride a multiple of 32");
     STRIX_REQUIRE(v->row_bytes >= v->in / 32U * kQ80Block && v->out_stride >= v->count, "Q8_0 product: stride shorter than the row");
     const uint32_t grid = (v->count + 7U) / 8U;
-    for (uint32_t r0 = 0; r0 < v->rows; r0 += 8U) gemv_q8_0_a8_kernel<8><<<grid, 256, 0, hs(stream)>>>(*v, r0);
+    const bool dw = aligned(v->weight, 4) && v->row_bytes % 4U == 0;
+    hipStream_t st = hs(stream);
+    if (v->rows == 1U) { if (dw) gemv_q8_0_a8_kernel<1, true><<<grid, 256, 0, st>>>(*v, 0); else gemv_q8_0_a8_kernel<1, false><<<grid, 256, 0, st>>>(*v, 0); }
+    else if (v->rows == 2U) { if (dw) gemv_q8_0_a8_kernel<2, true><<<grid, 256, 0, st>>>(*v, 0); else gemv_q8_0_a8_kernel<2, false><<<grid, 256, 0, st>>>(*v, 0); }
+    else if (v->rows <= 4U) { if (dw) gemv_q8_0_a8_kernel<4, true><<<grid, 256, 0, st>>>(*v, 0); else gemv_q8_0_a8_kernel<4, false><<<grid, 256, 0, st>>>(*v, 0); }
+    else
+        for (uint32_t r0 = 0; r0 < v->rows; r0 += 8U) {
+            if (dw) gemv_q8_0_a8_kernel<8, true><<<grid, 256, 0, st>>>(*v, r0);
+            else gemv_q8_0_a8_kernel<8, false><<<grid, 256, 0, st>>>(*v, r0);
+        }
     STRIX_LAUNCHED("gemv_q8_0_a8");
     return MI355_OK;
 }

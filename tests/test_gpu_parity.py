@@ -152,6 +152,13 @@ def test_q8_0_gemv_order_fixture_rows_accumulate_and_padding(strix):
     want, _ = orc.gemv_q8_0_a8(wq, c, d, 1024, 19)
     got = out.cpu().numpy()
     assert np.array_equal(bits(got[:, :19]), bits(want)) and np.all(got[:, 19:] == 29.0)
+    # 1, 2 and 3 rows (their own instantiations), and the same weights at a pointer that is only 2-byte aligned
+    shifted = torch.zeros(wq.size + 2, dtype=torch.uint8, device="cuda")
+    shifted[2:] = dev(wq).reshape(-1)
+    for rows in (1, 2, 3):
+        for weight in (dev(wq), shifted[2:]):
+            got = strix.gemv_q8_0_a8(weight, dev(c[:rows]), dev(d[:rows]), 1024, 19).cpu().numpy()
+            assert np.array_equal(bits(got), bits(want[:rows]))
     v = strix.Q8a8View(1, 1, 1, 1, 68, 33, 1, 1, 64, 1, 0)
     assert strix.lib().mi355_gemv_q8_0_a8(C.byref(v), None) == strix.E_INVALID_ARGUMENT
 
