@@ -431,7 +431,7 @@ def exact_weight_layer(x, ids, wts, gate, up, down, H, I, K, base=None):
     return orc.combine(0, wts, ids, raw, base=base), raw
 
 
-@pytest.mark.parametrize("H,I,E,K,T", [(512, 256, 6, 2, 300), (1024, 512, 12, 4, 77), (256, 256, 3, 1, 129)])
+@pytest.mark.parametrize("H,I,E,K,T", [(512, 256, 6, 2, 300), (1024, 512, 12, 4, 77), (256, 256, 3, 1, 129), (768, 1280, 5, 2, 150)])
 def test_prefill_f16_mfma_matches_exact_weight_product(strix, H, I, E, K, T):
     """The fp16 MFMA prefill form against the exact-weight product: tolerance 2e-3 (fp16 activations), both as max abs
     error over the output rms and elementwise on the outputs of at least rms size; the gate / up / down tiles are checked
