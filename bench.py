@@ -128,6 +128,22 @@ def device_q4k(torch, gen, rows_shape, width):
     return w.reshape(rows_shape + (width // 256 * 144,))
 
 
+def extra_config3_small(strix, torch, cfg, steps, warmup):
+    """Config 3 at the other token counts of its family (1 and 4): the same rotating layers, the first rows of their inputs."""
+    out = {}
+    n = len(cfg.layers)
+    for t in (1, 4):
+        def step(i):
+            layer, wr, x = cfg.layers[i % n]
+            layer.run_layer(x[:t], wr)
+        sec = time_steps(torch, step, max(steps, 60), max(warmup, 12))
+        u = statistics.mean(int(torch.unique(strix.route(x[:t], wr, cfg.K)[0]).numel()) for _, wr, x in cfg.layers)
+        nbytes = u * 3 * cfg.I * Q4K_ROW(cfg.H) + cfg.E * cfg.H * 4 + t * (cfg.H * 2 + cfg.H * 4)
+        out[f"config3_moe_decode_T{t}"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                           "algorithmic_bytes": nbytes, "distinct_experts_mean": u}
+    return out
+
+
 def extra_configs(strix, torch, steps, warmup):
     """BASELINE configs 1, 2, 4, 5 on synthetic full-entropy blocks; HBM-bound ones rotate over enough weight sets to stay cold."""
     gen = torch.Generator(device="cuda").manual_seed(11)
@@ -302,8 +318,9 @@ def main():
                      "timing": "HIP events on the launch stream around one back-to-back projection launch per rotating layer"},
     }
     if args.extra:
+        small = extra_config3_small(strix, torch, cfg, args.steps, args.warmup) if args.tokens >= 4 else {}
         del cfg.layers[1:]
-        out["extra"] = extra_configs(strix, torch, args.steps, args.warmup)
+        out["extra"] = {**small, **extra_configs(strix, torch, args.steps, args.warmup)}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_config3(cfg)
     else:

@@ -13,6 +13,7 @@
 #include "device_math.hpp"
 #include "q4k_rows.hpp"
 #include "q4k_pairs.hpp"
+#include "q4k_quads.hpp"
 #include "prefill_f16.hpp"
 #include "route_wave.hpp"
 
@@ -571,6 +572,94 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_
     }
 }
 
+// ---- the smallest decode batches: 16 rows per wavefront, lane = (row, pair) (q4k_quads.hpp) ------------------------------
+#define STRIX_QUAD_SLOTS(DEPTH)                                                                      \
+    __shared__ __attribute__((aligned(16))) uint8_t quad0[4][kQuadSlotBytes];                         \
+    __shared__ __attribute__((aligned(16))) uint8_t quad1[4][kQuadSlotBytes];                         \
+    __shared__ __attribute__((aligned(16))) uint8_t quad2[DEPTH > 2 ? 4 : 1][DEPTH > 2 ? kQuadSlotBytes : 16]; \
+    __shared__ __attribute__((aligned(16))) uint8_t quad3[DEPTH > 3 ? 4 : 1][DEPTH > 3 ? kQuadSlotBytes : 16]; \
+    const uint32_t wave = threadIdx.x >> 6;                                                           \
+    lds_u8* const quad_ring[4] = {(lds_u8*)quad0[wave], (lds_u8*)quad1[wave], (lds_u8*)quad2[DEPTH > 2 ? wave : 0], (lds_u8*)quad3[DEPTH > 3 ? wave : 0]}; \
+    lds_u8* slots[DEPTH];                                                                             \
+    _Pragma("unroll") for (int i = 0; i < DEPTH; ++i) slots[i] = quad_ring[i];
+
+// gate + up + SwiGLU + A8 of one item (one assignment): a 4-wave workgroup per 32-output group, wave = 8 gate rows and the
+// 8 up rows of the same features. Reference: src/cpu/core/routed_expert.cpp:403-427, :147-170.
+template <int DEPTH>
+__global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    STRIX_QUAD_SLOTS(DEPTH)
+    __shared__ float wg_amax[4];
+    __shared__ int wg_sum[4], wg_bad[4];
+    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
+    const uint32_t e = item.x, begin = item.y, end = item.z;
+    if (begin == end) return;
+    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x, groups = w.ffn / 32U;
+    const uint32_t sidx = __builtin_amdgcn_readfirstlane(r.plan[plan_order_at(w.experts) + begin]), row = sidx / w.top_k;
+    const uint32_t f0 = grp * 32U + 8U * wave;
+    const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(f0) * w.gate_row_stride;
+    const uint8_t* gate = w.gate + base;
+    const uint8_t* up = w.up + base;
+    const uint32_t stride = static_cast<uint32_t>(w.gate_row_stride);
+    QuadSource source;
+    source.init([&](uint32_t q) { return q < 8U ? gate + q * stride : up + (q - 8U) * stride; }, r.codes + static_cast<size_t>(row) * w.hidden);
+    lds_u8* const (&sl)[DEPTH] = slots;
+    const float value = sweep_quads<DEPTH>(sl, source, w.hidden / 256U, A8Image{r.codes, r.deltas, r.sums, w.hidden}, row);
+    const float other = __shfl_xor(value, 32);
+    const bool mine = lane < 32U && p == 0;                   // the lane that publishes feature f0 + rr
+    const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
+    const float h = (g / (1.0F + exp_of(w.exp_kind, -g))) * u;
+    const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
+    if (mine) {
+        if (r.gate_out) r.gate_out[at] = g;
+        if (r.up_out) r.up_out[at] = u;
+        if (r.h_out) r.h_out[at] = h;
+    }
+    const int bad = or32_i((mine && !(finite_f(g) && finite_f(u) && finite_f(h))) ? 1 : 0);
+    const float amax_wave = max32(mine ? __builtin_fabsf(h) : 0.0F);
+    if (lane == 0) { wg_amax[wave] = amax_wave; wg_bad[wave] = bad; }
+    __syncthreads();
+    if (wg_bad[0] | wg_bad[1] | wg_bad[2] | wg_bad[3]) {
+        if (threadIdx.x == 0) {
+            atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+        }
+        return;
+    }
+    const float amax = __builtin_fmaxf(__builtin_fmaxf(wg_amax[0], wg_amax[1]), __builtin_fmaxf(wg_amax[2], wg_amax[3]));
+    const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+    const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+    const int code = a8_code(h, dl, tiny);
+    const int sum_wave = sum32_i(mine ? code : 0);
+    if (lane == 0) wg_sum[wave] = sum_wave;
+    if (mine) r.down_codes[at] = static_cast<int8_t>(code);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
+        r.down_sums[static_cast<size_t>(sidx) * groups + grp] = wg_sum[0] + wg_sum[1] + wg_sum[2] + wg_sum[3];
+    }
+}
+
+// down rows of one item: a 4-wave workgroup per 64 outputs, 16 per wave.
+// Reference: src/cpu/core/routed_expert.cpp:429-447, src/moe_a8_down_contract.cpp:146.
+template <int DEPTH>
+__global__ __launch_bounds__(256) void down_quad_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    STRIX_QUAD_SLOTS(DEPTH)
+    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
+    const uint32_t e = item.x, begin = item.y, end = item.z;
+    if (begin == end) return;
+    if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
+    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2;
+    const uint32_t src = __builtin_amdgcn_readfirstlane(r.plan[plan_order_at(w.experts) + begin]);
+    const uint32_t o0 = blockIdx.x * 64U + 16U * wave;
+    const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o0) * w.down_row_stride;
+    const uint32_t stride = static_cast<uint32_t>(w.down_row_stride);
+    QuadSource source;
+    source.init([&](uint32_t q) { return rows + q * stride; }, r.down_codes + static_cast<size_t>(src) * w.ffn);
+    lds_u8* const (&sl)[DEPTH] = slots;
+    const float value = sweep_quads<DEPTH>(sl, source, w.ffn / 256U, A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src);
+    if (p == 0) r.rawdots[static_cast<size_t>(src) * w.hidden + o0 + rr] = value;
+}
+
 // Ordered combine of the slots of one row. Reference: include/strix/moe/combine.hpp:36-59 (fma form),
 // src/ds41_expert_tp.cpp:189-199 (product then add, slots in ascending expert id).
 __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t form) {
@@ -723,6 +812,8 @@ inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uin
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
     else launch_down_nb<4>(w, r, rows, grid, st);
 }
+// Decode batches of one or two tokens (at most this many assignments) run the 16-rows-per-wavefront sweep: see q4k_quads.hpp.
+constexpr uint32_t kQuadMaxItems = 16;
 // An expert's assignments are cut into work items of at most `split` rows: a wave's instruction stream grows with every
 // activation row it serves while its weight stream does not, so wide items finish last; the second read of a split
 // expert's weights comes from the last-level cache. A dense matrix: every row shares one sweep.
@@ -999,8 +1090,15 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     a.quant_blocks = (rows * (wv.hidden / 32U) + 7U) / 8U;
     launch_route_logits(a, hs(stream));
     STRIX_LAUNCHED("moe layer router");
-    launch_project(wv, *r, rows, rows * wv.top_k, hs(stream));       // the fused router planned one item per assignment
-    launch_down(wv, *r, rows, rows * wv.top_k, hs(stream));
+    // the fused router planned one item per assignment
+    const uint32_t items = rows * wv.top_k;
+    if (items <= kQuadMaxItems && wv.experts > 1U) {
+        project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+        down_quad_kernel<4><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+    } else {
+        launch_project(wv, *r, rows, items, hs(stream));
+        launch_down(wv, *r, rows, items, hs(stream));
+    }
     STRIX_LAUNCHED("moe layer experts");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }

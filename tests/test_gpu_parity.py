@@ -302,11 +302,12 @@ def test_config3_moe_decode_layer_shape(strix):
         check_layer_stages(strix, layer, y, ref, want, (c, d, s), ids_ref, w_ref, (gate, up, down, I, {}), H, K, T, 0, 0, TOL_F16)
 
 
-@pytest.mark.parametrize("E,H,I,K,T,order", [(128, 2048, 768, 8, 8, 0), (128, 2048, 768, 8, 1, 0), (160, 1536, 512, 8, 16, 0), (20, 512, 256, 3, 5, 1),
-                                             (64, 1024, 256, 16, 16, 0)])
+@pytest.mark.parametrize("E,H,I,K,T,order", [(128, 2048, 768, 8, 8, 0), (128, 2048, 768, 8, 1, 0), (128, 2048, 768, 8, 2, 0), (160, 1536, 512, 8, 16, 0),
+                                             (20, 512, 256, 3, 5, 1), (64, 1024, 256, 16, 16, 0), (160, 6144, 1280, 8, 2, 0)])
 def test_whole_layer_entry_router_prologue_plan_in_one_launch(strix, E, H, I, K, T, order):
     """mi355_moe_enqueue_layer: ids / weights / scores, the A8 image, the plan-driven experts and the combine must equal
-    the staged entry points bit for bit, twice in a row on the same workspace (the launch tickets return to zero)."""
+    the staged entry points bit for bit, twice in a row on the same workspace (the launch tickets return to zero). Batches of
+    at most 16 assignments run the 16-rows-per-wavefront sweep in the layer entry and the 64-row sweep in the staged one."""
     rng = np.random.default_rng(E + T)
     gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
     wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
