@@ -215,13 +215,17 @@ __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v, ui
 
 // ======================================================================================================== router
 // Plan words (uint32): [0] assignments A = rows * top_k, [1] touched experts U, [2] largest group, [3] launch ticket,
-// [4] work items; [16 ..] offsets[experts + 1]; touched[experts] (ids of the experts with work, ascending); order[A]:
-// assignment indices (row * top_k + slot) grouped by expert, ascending row then slot inside an expert; items[A] x 4 words
-// {expert, begin, end, 0}: the work items of the expert kernels, a touched expert's assignments cut into pieces of at
-// most `split` (zero records after the last item, up to the launch's item bound); 256 ticket / scratch words.
+// [4] work items; [16, 272) ticket / scratch words; offsets[experts + 1]; touched[experts] (ids of the experts with work,
+// ascending); order[A]: assignment indices (row * top_k + slot) grouped by expert, ascending row then slot inside an
+// expert; items[A] x 4 words {expert, begin, end, 0}: the work items of the expert kernels, a touched expert's assignments
+// cut into pieces of at most `split` (zero records after the last item, up to the launch's item bound).
 // Reference: src/hip_moe_q4k_a8_probe.hip:91-147 (stable CSR of (row, slot) by expert).
 __host__ __device__ inline uint32_t pad4(uint32_t v) { return (v + 3U) & ~3U; }
-__host__ __device__ inline uint32_t plan_touched_at(uint32_t experts) { return 16U + pad4(experts + 1U); }
+// ticket / scratch words right after the header, at the same place for every batch size (every launch leaves them zero, and a
+// workspace is reused with varying row counts): [0, 16) row tickets of the fused router, [16, 32) its quantiser tickets,
+// [128, 144) per-row A8 flags of the fused prologue
+constexpr uint32_t kPlanTicketsAt = 16, kPlanTicketWords = 256, kPlanOffsetsAt = kPlanTicketsAt + kPlanTicketWords;
+__host__ __device__ inline uint32_t plan_touched_at(uint32_t experts) { return kPlanOffsetsAt + pad4(experts + 1U); }
 __host__ __device__ inline uint32_t plan_order_at(uint32_t experts) { return plan_touched_at(experts) + pad4(experts); }
 // most work items a plan can hold (layout) and most a launch with pieces of `split` assignments can produce (grid size)
 __host__ __device__ inline uint32_t plan_item_capacity(uint32_t assignments) { return assignments; }
@@ -230,12 +234,9 @@ __host__ __device__ inline uint32_t plan_item_bound(uint32_t experts, uint32_t a
     return assignments < most ? assignments : most;
 }
 __host__ __device__ inline uint32_t plan_items_at(uint32_t experts, uint32_t assignments) { return plan_order_at(experts) + pad4(assignments); }
-__host__ __device__ inline uint32_t plan_tickets_at(uint32_t experts, uint32_t assignments) {
+__host__ __device__ inline uint32_t plan_words_total(uint32_t experts, uint32_t assignments) {
     return plan_items_at(experts, assignments) + 4U * plan_item_capacity(assignments);
 }
-// ticket / scratch words at the end of a plan: [0, 16) row tickets of the fused router, [128, 144) per-row A8 flags of the
-// fused prologue
-constexpr uint32_t kPlanTicketWords = 256;
 
 // Router logits for batches above the decode bound: blocks of 8 experts x 8 rows.
 template <int KIND>
@@ -268,7 +269,7 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
     __shared__ uint32_t flag;
     ChainSlot* const slots[4] = {&slot0, &slot1, &slot2, &slot3};
     const uint32_t bid = blockIdx.x, lane = threadIdx.x, neb = (a.p.experts + 7U) / 8U;
-    uint32_t* tickets = a.plan ? a.plan + plan_tickets_at(a.p.experts, a.rows * a.p.top_k) : nullptr;
+    uint32_t* tickets = a.plan ? a.plan + kPlanTicketsAt : nullptr;
     if (bid < a.route_blocks) {
         const uint32_t row = bid / neb;
         route_chain_block<KIND>(slots, a, row, (bid % neb) * 8U);
@@ -340,8 +341,8 @@ __global__ __launch_bounds__(64) void route_select_kernel(RouteArgs a) {
 // ballot + prefix count (the offsets are already in the plan).
 __global__ __launch_bounds__(64) void plan_order_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
     const uint32_t e = blockIdx.x, lane = threadIdx.x;
-    uint32_t at = plan[16 + e];
-    const uint32_t end = plan[16 + e + 1];
+    uint32_t at = plan[kPlanOffsetsAt + e];
+    const uint32_t end = plan[kPlanOffsetsAt + e + 1];
     uint32_t* order = plan + plan_order_at(experts);
     for (uint32_t a0 = 0; a0 < assignments && at < end; a0 += 64U) {
         const uint32_t a = a0 + lane;
@@ -384,7 +385,7 @@ __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint
         plan[0] = assignments; plan[1] = touched; plan[2] = largest; plan[4] = made;
     }
     __syncthreads();
-    uint32_t* offsets = plan + 16;
+    uint32_t* offsets = plan + kPlanOffsetsAt;
     uint32_t* order = plan + plan_order_at(experts);
     for (uint32_t e = tid; e <= experts; e += 1024U) offsets[e] = count[e];
     if (!fill_order) return;                  // large batches: plan_order_kernel follows
@@ -1009,7 +1010,7 @@ size_t mi355_moe_prefill_f16_workspace_bytes(uint32_t hidden, uint32_t ffn, uint
 }
 
 size_t mi355_moe_plan_words(uint32_t experts, uint32_t rows, uint32_t top_k) {
-    return plan_tickets_at(experts, rows * top_k) + kPlanTicketWords;
+    return plan_words_total(experts, rows * top_k);
 }
 
 int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {

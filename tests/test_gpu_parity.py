@@ -329,7 +329,26 @@ def test_whole_layer_entry_router_prologue_plan_in_one_launch(strix, E, H, I, K,
         assert torch.equal(y, y2) and torch.equal(layer.rawdots[:T], staged.rawdots[:T])
         assert np.all(layer.status[:T].cpu().numpy() == 0)
         n_plan = int(strix.lib().mi355_moe_plan_words(E, 16, K))
-        assert int(layer.plan[3]) == 0 and bool((layer.plan[n_plan - 256:] == 0).all())
+        assert int(layer.plan[3]) == 0 and bool((layer.plan[16:272] == 0).all())      # the ticket words are left zero
+
+
+def test_layer_entry_one_workspace_varying_batch_sizes(strix):
+    """A decode workspace is reused with whatever batch arrives: 8 rows, then 1, 4, 2, 8 on the same MoeLayer must each
+    equal a fresh staged run (the plan's ticket words sit at a place that does not depend on the row count)."""
+    E, H, I, K = 128, 2048, 768, 8
+    rng = np.random.default_rng(77)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
+    wrd = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), 8)
+    staged = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, 8)
+    x = dev(rng.standard_normal((8, H)).astype(np.float16))
+    for rows in (8, 1, 4, 2, 8):
+        y, ids, wts, _ = layer.run_layer(x[:rows], wrd)
+        ids2, wts2, _ = strix.route(x[:rows], wrd, K)
+        assert torch.equal(ids2, ids) and torch.equal(wts2, wts)
+        y2 = staged.run(x[:rows], ids2, wts2)
+        assert torch.equal(y, y2) and torch.equal(layer.rawdots[:rows], staged.rawdots[:rows])
+        assert np.all(layer.status[:rows].cpu().numpy() == 0) and bool((layer.plan[16:272] == 0).all())
 
 
 def test_config5_tp_rank_partial_sums(strix):
