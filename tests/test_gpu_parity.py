@@ -410,6 +410,34 @@ def test_invalid_route_and_nonfinite_projection_fail_closed(strix):
     assert bool((layer.rawdots == -3.0).all())
 
 
+@pytest.mark.parametrize("T", [1, 2, 8])
+def test_layer_entry_nonfinite_input_fails_closed(strix, T):
+    """An infinite input value through the whole-layer entry (the 16-rows-per-wavefront sweep at 1 and 2 rows, the 64-row
+    sweep at 8): the row is flagged (activation and projection bits), publishes nothing, the other rows are unaffected,
+    and the status words equal those of the staged entry points."""
+    E, H, I, K = 16, 512, 256, 4
+    rng = np.random.default_rng(31 + T)
+    gate, up, down = make_layer(rng, H, I, E)
+    wrd = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    good = dev(x.copy())
+    x[T - 1, 5] = np.inf
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), 8)
+    staged = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, 8)
+    want, _, _, _ = layer.run_layer(good, wrd)
+    want = want.clone()
+    layer.output.fill_(-7.0)
+    y, ids, wts, _ = layer.run_layer(dev(x), wrd)
+    st = layer.status[:T].cpu().numpy()
+    assert st[T - 1] & strix.STATUS_NONFINITE_ACTIVATION and st[T - 1] & strix.STATUS_NONFINITE_PROJECTION
+    assert np.all(st[: T - 1] == 0) and bool((y[T - 1] == -7.0).all())
+    assert int(layer.job_status[0]) & strix.STATUS_NONFINITE_PROJECTION
+    assert bool((layer.plan[16:272] == 0).all())
+    # a clean call on the same workspace afterwards is unaffected
+    again, _, _, _ = layer.run_layer(good, wrd)
+    assert torch.equal(again, want) and np.all(layer.status[:T].cpu().numpy() == 0)
+
+
 def test_admission_failures_return_before_any_enqueue(strix):
     H, I, E, K, T = 512, 256, 4, 2, 2
     rng = np.random.default_rng(10)
