@@ -813,8 +813,10 @@ inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uin
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
     else launch_down_nb<4>(w, r, rows, grid, st);
 }
-// Decode batches of one or two tokens (at most this many assignments) run the 16-rows-per-wavefront sweep: see q4k_quads.hpp.
-constexpr uint32_t kQuadMaxItems = 16;
+// Decode batches of at most this many assignments (six tokens at top-8) run the 16-rows-per-wavefront sweep (q4k_quads.hpp),
+// with a 4-slot ring up to 16 assignments and a 2-slot ring above (every workgroup of the launch stays resident); measured
+// at hidden 2048 / ffn 768: faster than the 64-row sweep up to 48 assignments, slower at 64.
+constexpr uint32_t kQuadMaxItems = 48;
 // An expert's assignments are cut into work items of at most `split` rows: a wave's instruction stream grows with every
 // activation row it serves while its weight stream does not, so wide items finish last; the second read of a split
 // expert's weights comes from the last-level cache. A dense matrix: every row shares one sweep.
@@ -1093,9 +1095,16 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     STRIX_LAUNCHED("moe layer router");
     // the fused router planned one item per assignment
     const uint32_t items = rows * wv.top_k;
-    if (items <= kQuadMaxItems && wv.experts > 1U) {
-        project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
-        down_quad_kernel<4><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+    static const int quad_items = env_int("STRIX950_QUAD_ITEMS");   // tuning aid: largest batch (assignments) on the quad sweep
+    const uint32_t quad_max = quad_items > 0 ? static_cast<uint32_t>(quad_items) : kQuadMaxItems;
+    if (items <= quad_max && wv.experts > 1U) {
+        if (items <= 16U) {
+            project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+            down_quad_kernel<4><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+        } else {
+            project_quad_kernel<2><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+            down_quad_kernel<2><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+        }
     } else {
         launch_project(wv, *r, rows, items, hs(stream));
         launch_down(wv, *r, rows, items, hs(stream));

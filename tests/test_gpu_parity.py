@@ -307,7 +307,7 @@ def test_config3_moe_decode_layer_shape(strix):
 def test_whole_layer_entry_router_prologue_plan_in_one_launch(strix, E, H, I, K, T, order):
     """mi355_moe_enqueue_layer: ids / weights / scores, the A8 image, the plan-driven experts and the combine must equal
     the staged entry points bit for bit, twice in a row on the same workspace (the launch tickets return to zero). Batches of
-    at most 16 assignments run the 16-rows-per-wavefront sweep in the layer entry and the 64-row sweep in the staged one."""
+    at most 48 assignments run the 16-rows-per-wavefront sweep in the layer entry and the 64-row sweep in the staged one."""
     rng = np.random.default_rng(E + T)
     gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
     wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
@@ -410,10 +410,9 @@ def test_invalid_route_and_nonfinite_projection_fail_closed(strix):
     assert bool((layer.rawdots == -3.0).all())
 
 
-@pytest.mark.parametrize("T", [1, 2, 8])
+@pytest.mark.parametrize("T", [1, 2, 8, 16])
 def test_layer_entry_nonfinite_input_fails_closed(strix, T):
-    """An infinite input value through the whole-layer entry (the 16-rows-per-wavefront sweep at 1 and 2 rows, the 64-row
-    sweep at 8): the row is flagged (activation and projection bits), publishes nothing, the other rows are unaffected,
+    """An infinite input value through the whole-layer entry (the 16-rows-per-wavefront sweep): the row is flagged (activation and projection bits), publishes nothing, the other rows are unaffected,
     and the status words equal those of the staged entry points."""
     E, H, I, K = 16, 512, 256, 4
     rng = np.random.default_rng(31 + T)
@@ -422,8 +421,7 @@ def test_layer_entry_nonfinite_input_fails_closed(strix, T):
     x = rng.standard_normal((T, H)).astype(np.float16)
     good = dev(x.copy())
     x[T - 1, 5] = np.inf
-    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), 8)
-    staged = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, 8)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), 16)
     want, _, _, _ = layer.run_layer(good, wrd)
     want = want.clone()
     layer.output.fill_(-7.0)
