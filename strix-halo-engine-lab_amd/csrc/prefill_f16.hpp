@@ -26,9 +26,10 @@
 //   * a multiplier wave holds a 64 x 64 quarter (2 x 2 MFMA tiles, A = tokens, B = weights: a lane of the result is
 //     one feature, so d_b is one register per tile row) in two sets of accumulators: P (cleared every super-block) and
 //     the running sum.
-// LDS tiles are [row][64 halves] with a 128-byte pitch and the 16-byte pieces of a row XOR-swizzled by row % 8: a 128-bit
-// LDS access is served eight lanes at a time, and eight consecutive rows then cover all 32 banks for the MFMA operand
-// reads and the loaders' stores, while a copy instruction still writes 1 KB of consecutive LDS. One barrier per step.
+// LDS tiles are [row][64 halves] with a 128-byte pitch and the 16-byte pieces of a row XOR-swizzled by (row / 2) % 8: a
+// 128-bit LDS access is served sixteen lanes at a time over 64 banks, and sixteen consecutive rows then cover all banks for
+// the MFMA operand reads and the loaders' stores (measured: swizzling by row % 8 instead doubles the conflict cycles), while
+// a copy instruction still writes 1 KB of consecutive LDS. One barrier per step.
 //
 // Workgroups are numbered so that the feature tiles of one item run on one XCD (consecutive workgroup ids go round
 // the 8 XCDs): its token rows are then read from HBM once per XCD and served from that XCD's L2 afterwards.
@@ -133,7 +134,7 @@ __device__ __forceinline__ void copy16_to_lds(const uint8_t* src, pf_lds* lds_ba
 }
 
 // byte offset of 16-byte piece `piece` (0..7) of tile row `row`
-__device__ __forceinline__ uint32_t pf_at(uint32_t row, uint32_t piece) { return row * 128U + ((piece ^ (row & 7U)) << 4); }
+__device__ __forceinline__ uint32_t pf_at(uint32_t row, uint32_t piece) { return row * 128U + ((piece ^ ((row >> 1) & 7U)) << 4); }
 
 // the loader's per-step global operands
 struct PfRaw { u32x4 hd, qs[4]; };           // one super-block of a weight row: header and the thread's 16 quant bytes of its four steps
@@ -177,7 +178,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
 #pragma unroll
         for (uint32_t i = 0; i < 4U; ++i) {
             const uint32_t row = 8U * (4U * i + wave) + (lane >> 3), tok = row < count ? row : count - 1U;
-            const uint32_t piece = (lane & 7U) ^ (row & 7U);
+            const uint32_t piece = (lane & 7U) ^ ((row >> 1) & 7U);
             if (MODE == 0) tsrc[i] = a.x + static_cast<size_t>(order[begin + tok] / a.top_k) * a.x_stride + 16U * piece;
             else tsrc[i] = reinterpret_cast<const uint8_t*>(a.h + static_cast<size_t>(begin + tok) * a.k) + 16U * piece;
         }
@@ -337,7 +338,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
 #pragma unroll
             for (int j = 0; j < 16; ++j) { acc[i][n][j] = 0.0F; part[i][n][j] = 0.0F; }
     const uint32_t wr = wave / (4U / TT), wc = wave % (4U / TT), l31 = lane & 31U, upper = lane >> 5;
-    const uint32_t trow = (TS * wc + l31) * 128U, frow = (64U * wr + l31) * 128U, sw = l31 & 7U;
+    const uint32_t trow = (TS * wc + l31) * 128U, frow = (64U * wr + l31) * 128U, sw = (l31 >> 1) & 7U;
     uint32_t piece_at[4];
 #pragma unroll
     for (uint32_t ks = 0; ks < 4U; ++ks) piece_at[ks] = ((2U * ks + upper) ^ sw) << 4;
