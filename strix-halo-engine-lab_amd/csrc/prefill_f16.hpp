@@ -77,7 +77,7 @@ struct PrefillArgs {
     float* rawdots;                               // MODE 1: [assignment][hidden]
     const uint32_t* plan; uint32_t experts, assignments;
     uint32_t* status; uint32_t* job_status;
-    uint32_t tiles, items;                        // feature tiles per item, item bound of the launch
+    uint32_t tiles, items, units;                 // feature tiles per item, item bound of the launch, tiles * items rounded up to 8 items
 };
 
 __device__ __forceinline__ uint32_t pack_half2(float a, float b) {
@@ -152,16 +152,20 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
     pf_lds* const tok_stage[4] = {(pf_lds*)tok0, (pf_lds*)tok1, (pf_lds*)tok2, (pf_lds*)tok3};
     pf_lds* const s_tile = (pf_lds*)s_tile_mem;
 
-    // workgroup -> (item, feature tile): ids i, i + 8, i + 16, ... share an XCD; they walk the tiles of one item first
-    const uint32_t xcd = blockIdx.x & 7U, q = blockIdx.x >> 3;
-    const uint32_t item_index = (q / a.tiles) * 8U + xcd, tile = q % a.tiles;
-    if (item_index >= a.items) return;
-    const uint4 item = *reinterpret_cast<const uint4*>(a.plan + items_at + 4U * item_index);
-    const uint32_t e = item.x, begin = item.y, count = item.z - item.y;
-    if (count == 0) return;
     if (MODE == 1 && (*a.job_status & MI355_STATUS_NONFINITE_PROJECTION)) return;
     const uint32_t* order = a.plan + order_at;
     const bool loader = threadIdx.x < 256U;
+    // A workgroup is persistent: it walks the (item, feature tile) units v = blockIdx.x, blockIdx.x + gridDim.x, ... (gridDim.x a
+    // multiple of 8). Units v, v + 8, v + 16, ... share an XCD and walk the tiles of one item first, so the workgroups of an
+    // XCD work on the same item at the same time. The loaders reach the next unit's prologue (plan and pointer loads, first
+    // copies) while the multipliers are still in the epilogue of the current one: nobody reads LDS after a unit's last barrier.
+    for (uint32_t unit = blockIdx.x; unit < a.units; unit += gridDim.x) {
+    const uint32_t xcd = unit & 7U, q = unit >> 3;
+    const uint32_t item_index = (q / a.tiles) * 8U + xcd, tile = q % a.tiles;
+    if (item_index >= a.items) continue;
+    const uint4 item = *reinterpret_cast<const uint4*>(a.plan + items_at + 4U * item_index);
+    const uint32_t e = item.x, begin = item.y, count = item.z - item.y;
+    if (count == 0) continue;
     const uint32_t t = loader ? threadIdx.x : threadIdx.x - 256U, lane = t & 63U, wave = t >> 6;      // index within the role
     const uint32_t m0 = tile * (MODE == 0 ? 64U : 128U);
     const uint32_t steps = a.k / kPfStep, blocks = a.k / 256U, steps8 = (steps + 7U) & ~7U;
@@ -252,7 +256,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 2U * half + 1U)) = u32x4{lo[4], lo[5], lo[6], lo[7]};
             *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 4U + 2U * half)) = u32x4{hi[0], hi[1], hi[2], hi[3]};
             *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 5U + 2U * half)) = u32x4{hi[4], hi[5], hi[6], hi[7]};
-            if (p == 0) {
+            if (p == 1) {
+                // once per super-block, with its second step: that one is staged while the multipliers run a step without the
+                // end-of-super-block work, and its results are not read before the super-block's last step
                 if (half == 0) d_scale[b & 1U][lrow] = half_bits_to_float(hd.x & 0xffffU);
                 // -(dmin m_j) of this super-block's eight sub-blocks: sub-blocks 8 (b % 2) .. + 8 of the group
                 uint8_t* mrow = m_tile[(b >> 1) & 1U] + lrow * 64U;
@@ -325,7 +331,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                 pf_barrier();
             }
         }
-        return;
+        continue;
     }
 
     // ---- multipliers: wave (wr, wc) owns tile rows 64 wr .. + 64 (two tiles of 32 features) x tokens TS wc .. + TS
@@ -465,6 +471,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             }
         }
     }
+    }   // units
 }
 
 }  // namespace strix950

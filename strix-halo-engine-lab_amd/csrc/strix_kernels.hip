@@ -1138,11 +1138,15 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     if (pf_sum_slots(wv.ffn) != wv.ffn / 32U) clear_sum_padding_kernel<<<assignments, 64, 0, st>>>(a.h_sums, wv.ffn);
     const uint32_t items_at = plan_items_at(wv.experts, assignments), order_at = plan_order_at(wv.experts), item_slots = (bound + 7U) / 8U * 8U;
     a.wa = wv.gate; a.wb = wv.up; a.expert_stride = wv.gate_expert_stride; a.row_stride = wv.gate_row_stride; a.k = wv.hidden; a.features = wv.ffn;
-    a.tiles = wv.ffn / 64U;
-    prefill_f16_kernel<0><<<item_slots * a.tiles, kPfThreads, 0, st>>>(a, items_at, order_at);
+    // persistent workgroups, one per compute unit (the kernel's LDS use allows no second one)
+    int device = 0, cus = 256;
+    if (hipGetDevice(&device) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+    const uint32_t resident = static_cast<uint32_t>(cus > 8 ? cus : 8) & ~7U;
+    a.tiles = wv.ffn / 64U; a.units = item_slots * a.tiles;
+    prefill_f16_kernel<0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     a.wa = wv.down; a.wb = nullptr; a.expert_stride = wv.down_expert_stride; a.row_stride = wv.down_row_stride; a.k = wv.ffn; a.features = wv.hidden;
-    a.tiles = wv.hidden / 128U;
-    prefill_f16_kernel<1><<<item_slots * a.tiles, kPfThreads, 0, st>>>(a, items_at, order_at);
+    a.tiles = wv.hidden / 128U; a.units = item_slots * a.tiles;
+    prefill_f16_kernel<1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     STRIX_LAUNCHED("moe prefill f16");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
