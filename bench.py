@@ -218,6 +218,24 @@ def extra_configs(strix, torch, steps, warmup):
         "frac_of_fp16_mfma_peak": (flops_experts + flops_router) / (sec_f16 + sec_route) / 2.5e15,
         "experts_frac_of_fp16_mfma_peak": flops_experts / sec_f16 / 2.5e15, "algorithmic_flops": flops_experts + flops_router,
         "note": "routed experts on fp16 MFMA (exact integer operands sc*q, fp32 block scales, fp32 accumulation) + exact-order router; FAST class, tolerance 2e-3"}
+    # the always-on shared expert (Q8_0, same intermediate size), integer-dot class: A8 image, gate / up, SwiGLU + A8, down
+    def q8(rows, width):
+        w = torch.randint(0, 256, (rows, width // 32, 34), dtype=torch.uint8, device="cuda", generator=gen)
+        w[..., 1] = (w[..., 1] & 0x03) | 0x14
+        return w.reshape(rows, -1)
+    sg, su, sd = q8(I, H), q8(I, H), q8(H, I)
+
+    def shared(i):
+        c, d, _, _ = strix.quantize_a8(xp)
+        hc, hd, _, _, _ = strix.swiglu_quantize(strix.gemv_q8_0_a8(sg, c, d, H, I), strix.gemv_q8_0_a8(su, c, d, H, I))
+        return strix.gemv_q8_0_a8(sd, hc, hd, I, H)
+    sec_shared = time_steps(torch, shared, 3, 1)
+    flops_shared = 2.0 * T * 3 * I * H
+    out["config4_prefill_T4096_f16_mfma"].update({
+        "shared_expert_ms": sec_shared * 1e3,
+        "with_shared_expert_ms": (sec_f16 + sec_route + sec_shared) * 1e3,
+        "with_shared_expert_TFLOPs": (flops_experts + flops_router + flops_shared) / (sec_f16 + sec_route + sec_shared) / 1e12})
+    del sg, su, sd
     sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 2, 1)
     out["config4_prefill_T4096_integer_class"] = {
         "ms": sec * 1e3, "TFLOPs": (flops_experts + flops_router) / sec / 1e12, "algorithmic_flops": flops_experts + flops_router,

@@ -162,8 +162,8 @@ __global__ __launch_bounds__(256) void quantize_a8_kernel(const uint8_t* x, uint
 // (two 128-bit loads and one 32-bit load) around its codes and shifted into place, instead of seventeen 16-bit loads.
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 template <int RB, bool DW>
-__global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v, uint32_t row0) {
-    const uint32_t o = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U;
+__global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v) {
+    const uint32_t o = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U, row0 = blockIdx.y * RB;
     if (o >= v.count) return;
     const uint32_t groups = v.in / 32U;
     const uint32_t nr = v.rows - row0 < static_cast<uint32_t>(RB) ? v.rows - row0 : static_cast<uint32_t>(RB);
@@ -947,14 +947,19 @@ int32_t mi355_gemv_q8_0_a8(const mi355_q8a8_view* v, mi355_stream stream) {
     const uint32_t grid = (v->count + 7U) / 8U;
     const bool dw = aligned(v->weight, 4) && v->row_bytes % 4U == 0;
     hipStream_t st = hs(stream);
-    if (v->rows == 1U) { if (dw) gemv_q8_0_a8_kernel<1, true><<<grid, 256, 0, st>>>(*v, 0); else gemv_q8_0_a8_kernel<1, false><<<grid, 256, 0, st>>>(*v, 0); }
-    else if (v->rows == 2U) { if (dw) gemv_q8_0_a8_kernel<2, true><<<grid, 256, 0, st>>>(*v, 0); else gemv_q8_0_a8_kernel<2, false><<<grid, 256, 0, st>>>(*v, 0); }
-    else if (v->rows <= 4U) { if (dw) gemv_q8_0_a8_kernel<4, true><<<grid, 256, 0, st>>>(*v, 0); else gemv_q8_0_a8_kernel<4, false><<<grid, 256, 0, st>>>(*v, 0); }
-    else
-        for (uint32_t r0 = 0; r0 < v->rows; r0 += 8U) {
-            if (dw) gemv_q8_0_a8_kernel<8, true><<<grid, 256, 0, st>>>(*v, r0);
-            else gemv_q8_0_a8_kernel<8, false><<<grid, 256, 0, st>>>(*v, r0);
-        }
+    // up to RB activation rows share one sweep of a weight row; more rows are further blocks of the same launch (grid.y)
+    const auto launch = [&](auto rb_constant) {
+        constexpr int RB = decltype(rb_constant)::value;
+        const dim3 g(grid, (v->rows + RB - 1U) / RB);
+        if (dw) gemv_q8_0_a8_kernel<RB, true><<<g, 256, 0, st>>>(*v);
+        else gemv_q8_0_a8_kernel<RB, false><<<g, 256, 0, st>>>(*v);
+    };
+    STRIX_REQUIRE((v->rows + 15U) / 16U <= 65535U, "Q8_0 product: too many rows for one launch");
+    if (v->rows == 1U) launch(std::integral_constant<int, 1>{});
+    else if (v->rows == 2U) launch(std::integral_constant<int, 2>{});
+    else if (v->rows <= 4U) launch(std::integral_constant<int, 4>{});
+    else if (v->rows <= 8U) launch(std::integral_constant<int, 8>{});
+    else launch(std::integral_constant<int, 16>{});            // (32 rows per sweep measured slower: 5.0 vs 4.05 ms on 4096 rows)
     STRIX_LAUNCHED("gemv_q8_0_a8");
     return MI355_OK;
 }
