@@ -120,10 +120,11 @@ class Config3:
         return u * 2 * self.I * Q4K_ROW(self.H) + self.T * self.H * 1.25 + self.T * self.K * self.I * 1.25
 
 
-def device_q4k(torch, gen, rows_shape, width):
-    """Random Q4_K blocks with finite, moderate fp16 d / dmin (every other bit random) - no fp32 staging tensor needed."""
+def device_q4k(torch, gen, rows_shape, width, d_bits=0x13):
+    """Random Q4_K blocks with finite, moderate fp16 d / dmin (every other bit random) - no fp32 staging tensor needed.
+    d_bits = 0x03 keeps d below 2^-11 (weights of a few hundredths), so that a 4096-wide product stays far inside fp16."""
     w = torch.randint(0, 256, rows_shape + (width // 256, 144), dtype=torch.uint8, device="cuda", generator=gen)
-    w[..., 1] = (w[..., 1] & 0x13) | 0x0C
+    w[..., 1] = (w[..., 1] & d_bits) | 0x0C
     w[..., 3] = (w[..., 3] & 0x03) | 0x0C
     return w.reshape(rows_shape + (width // 256 * 144,))
 
@@ -203,7 +204,8 @@ def extra_configs(strix, torch, steps, warmup):
     del layer
     # config 4: 4096-row prefill, hidden 4096, 256 experts top-8 (+ logit bias), intermediate 2048; routed experts + router
     H, I, E, K, T = 4096, 2048, 256, 8, 4096
-    layer = strix.MoeLayer(H, I, E, K, device_q4k(torch, gen, (E, I), H), device_q4k(torch, gen, (E, I), H), device_q4k(torch, gen, (E, H), I), T)
+    layer = strix.MoeLayer(H, I, E, K, device_q4k(torch, gen, (E, I), H, 0x03), device_q4k(torch, gen, (E, I), H, 0x03),
+                           device_q4k(torch, gen, (E, H), I, 0x03), T)
     wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
     bias = torch.randn(E, device="cuda", generator=gen) * 1.5
     xp = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)
@@ -218,7 +220,7 @@ def extra_configs(strix, torch, steps, warmup):
         "frac_of_fp16_mfma_peak": (flops_experts + flops_router) / (sec_f16 + sec_route) / 2.5e15,
         "experts_frac_of_fp16_mfma_peak": flops_experts / sec_f16 / 2.5e15, "algorithmic_flops": flops_experts + flops_router,
         "note": "routed experts on fp16 MFMA (exact integer operands sc*q, fp32 block scales, fp32 accumulation) + exact-order router; FAST class, tolerance 2e-3"}
-    # the always-on shared expert (Q8_0, same intermediate size), integer-dot class: A8 image, gate / up, SwiGLU + A8, down
+    # the always-on shared expert (Q8_0, same intermediate size); first in the integer-dot class: A8 image, gate / up, SwiGLU + A8, down
     def q8(rows, width):
         w = torch.randint(0, 256, (rows, width // 32, 34), dtype=torch.uint8, device="cuda", generator=gen)
         w[..., 1] = (w[..., 1] & 0x03) | 0x14
@@ -229,13 +231,28 @@ def extra_configs(strix, torch, steps, warmup):
         c, d, _, _ = strix.quantize_a8(xp)
         hc, hd, _, _, _ = strix.swiglu_quantize(strix.gemv_q8_0_a8(sg, c, d, H, I), strix.gemv_q8_0_a8(su, c, d, H, I))
         return strix.gemv_q8_0_a8(sd, hc, hd, I, H)
-    sec_shared = time_steps(torch, shared, 3, 1)
+    sec_shared_int = time_steps(torch, shared, 3, 1)
+    # the same expert on the matrix cores: a one-expert layer in the prefill form, its output the base of the routed combine
+    dense = strix.MoeLayer(H, I, 1, 1, sg.reshape(1, I, -1), su.reshape(1, I, -1), sd.reshape(1, H, -1), T, prefill_f16=True,
+                           gate_type=strix.TYPE_Q8_0, down_type=strix.TYPE_Q8_0)
+    zero_ids = torch.zeros((T, 1), dtype=torch.int32, device="cuda")
+    ones = torch.ones((T, 1), dtype=torch.float32, device="cuda")
+    sec_shared = time_steps(torch, lambda i: dense.run_prefill_f16(xp, zero_ids, ones), 10, 3)
+
+    def whole(i):
+        r_ids, r_wts, _ = strix.route(xp, wr, K, bias=bias)
+        return layer.run_prefill_f16(xp, r_ids, r_wts, base=dense.run_prefill_f16(xp, zero_ids, ones))
+    sec_whole = time_steps(torch, whole, 10, 3)
+    if int(layer.status.sum()) or int(dense.status.sum()):
+        raise RuntimeError("config 4: the prefill run set row status bits (non-finite or out-of-range values): the timing is void")
     flops_shared = 2.0 * T * 3 * I * H
     out["config4_prefill_T4096_f16_mfma"].update({
-        "shared_expert_ms": sec_shared * 1e3,
-        "with_shared_expert_ms": (sec_f16 + sec_route + sec_shared) * 1e3,
-        "with_shared_expert_TFLOPs": (flops_experts + flops_router + flops_shared) / (sec_f16 + sec_route + sec_shared) / 1e12})
-    del sg, su, sd
+        "shared_expert_ms": sec_shared * 1e3, "shared_expert_TFLOPs": flops_shared / sec_shared / 1e12,
+        "shared_expert_integer_class_ms": sec_shared_int * 1e3,
+        "with_shared_expert_ms": sec_whole * 1e3,
+        "with_shared_expert_TFLOPs": (flops_experts + flops_router + flops_shared) / sec_whole / 1e12,
+        "with_shared_expert_frac_of_fp16_mfma_peak": (flops_experts + flops_router + flops_shared) / sec_whole / 2.5e15})
+    del sg, su, sd, dense
     sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 2, 1)
     out["config4_prefill_T4096_integer_class"] = {
         "ms": sec * 1e3, "TFLOPs": (flops_experts + flops_router) / sec / 1e12, "algorithmic_flops": flops_experts + flops_router,

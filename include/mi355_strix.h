@@ -40,7 +40,8 @@ enum {
     MI355_STATUS_INVALID_ROUTE = 1,          /* route id >= experts, or non-finite route weight */
     MI355_STATUS_NONFINITE_ACTIVATION = 2,   /* non-finite input activation */
     MI355_STATUS_INVALID_DELTA = 4,
-    MI355_STATUS_NONFINITE_PROJECTION = 8,   /* non-finite gate, up or h; the down phase of the job is skipped */
+    MI355_STATUS_NONFINITE_PROJECTION = 8,   /* non-finite gate, up or h (the fp16 prefill form: h beyond fp16 too); the down
+                                                phase of the job is skipped and its merge publishes no row */
     MI355_STATUS_AGGREGATE = 16              /* merged output failed the commit threshold */
 };
 
@@ -129,7 +130,7 @@ typedef struct mi355_moe_weights {
     uint32_t hidden;      /* multiple of 256 */
     uint32_t ffn;         /* intermediate rows computed by this call (a TP rank: its share), multiple of 256 */
     uint32_t experts, top_k;
-    uint32_t gate_type, down_type;                    /* MI355_TYPE_Q4_K */
+    uint32_t gate_type, down_type;                    /* MI355_TYPE_Q4_K (mi355_moe_enqueue_prefill_f16: or MI355_TYPE_Q8_0) */
     const uint8_t *gate, *up, *down;                  /* GGUF order [experts][ffn][hidden/256], [experts][hidden][ffn/256] */
     uint64_t gate_expert_stride, gate_row_stride;     /* bytes; 0 = dense GGUF order. 16-byte multiples */
     uint64_t down_expert_stride, down_row_stride;     /* a TP rank reads the first ffn/256 blocks of each down row */
@@ -165,7 +166,8 @@ int32_t mi355_moe_enqueue_csr(const mi355_moe_weights*, const mi355_moe_rows*, u
 int32_t mi355_moe_enqueue_project(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, mi355_stream);
 /* down: rawdots[row][slot][hidden]; skipped on the device when any row reported a non-finite projection. */
 int32_t mi355_moe_enqueue_down(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, mi355_stream);
-/* merge: ordered combine of the slots (+ base) into output; form = MI355_COMBINE_*. */
+/* merge: ordered combine of the slots (+ base) into output; form = MI355_COMBINE_*. A flagged row, and every row of a job
+ * whose down phase was skipped, is left unwritten. */
 int32_t mi355_moe_enqueue_merge(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, uint32_t form,
                                 mi355_stream);
 /* prologue + csr + project + down + merge. */
@@ -191,7 +193,11 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* policy, const float* r
  * the library's tolerance (2e-3 of the output rms), NOT the integer-dot class's bits: a caller opts in by calling this
  * entry point. Runs: status clear + route validation, expert plan, gate/up + SwiGLU, down, ordered combine.
  * Requires input_kind = MI355_INPUT_F16, rows->h_f16 (see mi355_moe_prefill_f16_workspace_bytes), hidden % 256 == 0,
- * ffn % 256 == 0. */
+ * ffn % 256 == 0.
+ * gate_type and down_type may each be MI355_TYPE_Q4_K or MI355_TYPE_Q8_0 here (w = d * code, src/ggml_dequant.cpp:84-87: the
+ * codes are the exact operands, d is applied in fp32 to every block's product). An always-on shared expert
+ * (src/hip_shared_expert_launcher.hip) is a layer with experts = top_k = 1, every route id 0 and every route weight 1; its
+ * output is the next call's rows->base. A row whose h leaves the fp16 range is reported as MI355_STATUS_NONFINITE_PROJECTION. */
 int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, uint32_t combine_form,
                                       mi355_stream);
 

@@ -178,11 +178,12 @@ class MoeLayer:
     Rows / Weights bundle, include/strix/cuda/qwen_moe.hpp:55-93)."""
 
     def __init__(self, hidden, ffn, experts, top_k, gate, up, down, max_rows, exp_kind=EXP_GFX1151, intermediates=False,
-                 gate_expert_stride=0, gate_row_stride=0, down_expert_stride=0, down_row_stride=0, prefill_f16=False):
+                 gate_expert_stride=0, gate_row_stride=0, down_expert_stride=0, down_row_stride=0, prefill_f16=False,
+                 gate_type=TYPE_Q4_K, down_type=TYPE_Q4_K):
         dev = gate.device
         self.hidden, self.ffn, self.experts, self.top_k, self.max_rows = hidden, ffn, experts, top_k, max_rows
         self.gate, self.up, self.down = gate, up, down
-        self.w = MoeWeights(hidden, ffn, experts, top_k, TYPE_Q4_K, TYPE_Q4_K, gate.data_ptr(), up.data_ptr(), down.data_ptr(),
+        self.w = MoeWeights(hidden, ffn, experts, top_k, gate_type, down_type, gate.data_ptr(), up.data_ptr(), down.data_ptr(),
                             gate_expert_stride, gate_row_stride, down_expert_stride, down_row_stride, exp_kind)
         n = max_rows * top_k
         z = lambda shape, dt: torch.zeros(shape, dtype=dt, device=dev)

@@ -138,8 +138,11 @@ __device__ __forceinline__ uint32_t pf_at(uint32_t row, uint32_t piece) { return
 
 // the loader's per-step global operands
 struct PfRaw { u32x4 hd, qs[4]; };           // one super-block of a weight row: header and the thread's 16 quant bytes of its four steps
+struct PfRaw8 { u32x4 a, b; uint32_t c; };   // one Q8_0 block of a weight row as nine aligned words
 
-template <int MODE>
+// FMT 0: Q4_K weights, FMT 1: Q8_0 weights (one fp16 d per 32 codes and no minimum, src/ggml_dequant.cpp:84-87: the codes
+// are exact fp16 integers, a step is two blocks, and d is applied in fp32 to the product of each block).
+template <int MODE, int FMT>
 __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, uint32_t items_at, uint32_t order_at) {
     __shared__ __attribute__((aligned(16))) uint8_t tok0[kPfTileBytes];                     // token steps: stage s % 4
     __shared__ __attribute__((aligned(16))) uint8_t tok1[kPfTileBytes];
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
     __shared__ __attribute__((aligned(16))) uint8_t w_tile[2][kPfTileBytes];                // sc q of one step
     __shared__ __attribute__((aligned(16))) uint8_t s_tile_mem[2][kPfTile * 64U];           // [token][hi 16 | lo 16] sums of 16 sub-blocks
     __shared__ __attribute__((aligned(16))) uint8_t m_tile[2][kPfTile * 64U];               // [feature][hi 16 | lo 16] -(dmin m)
-    __shared__ float d_scale[2][kPfTile];                                                   // d of one super-block
+    __shared__ float d_scale[2][2U * kPfTile];                                              // d of one super-block (Q4_K: the first 128) or of a step's two blocks (Q8_0)
     pf_lds* const tok_stage[4] = {(pf_lds*)tok0, (pf_lds*)tok1, (pf_lds*)tok2, (pf_lds*)tok3};
     pf_lds* const s_tile = (pf_lds*)s_tile_mem;
 
@@ -168,7 +171,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
     if (count == 0) continue;
     const uint32_t t = loader ? threadIdx.x : threadIdx.x - 256U, lane = t & 63U, wave = t >> 6;      // index within the role
     const uint32_t m0 = tile * (MODE == 0 ? 64U : 128U);
-    const uint32_t steps = a.k / kPfStep, blocks = a.k / 256U, steps8 = (steps + 7U) & ~7U;
+    const uint32_t steps = a.k / kPfStep, blocks = a.k / 256U, steps8 = FMT == 0 ? (steps + 7U) & ~7U : steps;   // K is a multiple of 256: steps of 4
     const size_t sum_row = pf_sum_row_bytes(a.k);
 
     if (loader) {
@@ -196,15 +199,82 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             ssrc[c] = base + 16U * (part & 1U) + (part >> 1) * (sum_row / 2U);
         }
         const uint32_t last = steps - 1U, last_block = blocks - 1U, last_group = (blocks + 1U) / 2U - 1U;
-        // Every memory operation below is issued unconditionally (indices past the end are clamped: such copies land in
-        // stages nobody reads any more), so the number of operations between an issue and the point that needs its data
-        // is a compile-time constant and the waits are plain s_waitcnt vmcnt(n) of this code's own: the compiler is not
-        // told about these operations, whose bookkeeping across loop iterations it resolves by waiting for all of them.
+        // (memory operations are issued unconditionally, indices past the end clamped: see below)
         const auto copy_tokens = [&](uint32_t s, pf_lds* stage) {          // 4 operations: step s -> its stage
             const uint32_t sc = s < last ? s : last;
 #pragma unroll
             for (uint32_t i = 0; i < 4U; ++i) copy16_to_lds(tsrc[i] + static_cast<size_t>(sc) * 128U, stage + 1024U * (4U * i + wave));
         };
+        if constexpr (FMT == 1) {
+            // ---- Q8_0: the thread owns block 2 s + half of every step (34 bytes at a 2-byte boundary). Rows start at 4-byte
+            // boundaries, so block `half` starts 2 half bytes past one: nine aligned words cover it. For half 0 they are the
+            // words from the block's start (d in the low half of the first, codes from byte 2: every code word straddles two);
+            // for half 1 eight words from the first code and the word before them (d in its high half).
+            const uint8_t* pa = wrow + 34U * half + 2U * half;
+            const uint8_t* pc = half ? pa - 4 : pa + 32;
+            const uint32_t straddle = half ? 0U : 2U;
+            const auto fetch8 = [&](uint32_t s, PfRaw8& r) {                 // 3 operations
+                const uint32_t off = 68U * (s < last ? s : last);
+                const uint8_t* qa = pa + off;
+                const uint8_t* qc = pc + off;
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.a) : "v"(qa) : "memory");
+                asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(r.b) : "v"(qa) : "memory");
+                asm volatile("global_load_dword %0, %1, off" : "=v"(r.c) : "v"(qc) : "memory");
+            };
+            uint32_t bias_bits;                                              // per half: 0x6400 | 0x80: 1024 + (code ^ 0x80) = 1152 + code
+            asm volatile("v_mov_b32 %0, 0x64806480" : "=v"(bias_bits));
+            const _Float16 minus = static_cast<_Float16>(-1152.0F);
+            const half2v minus2 = {minus, minus};
+            const auto stage8 = [&](uint32_t s, const PfRaw8& r) {
+                const uint32_t seq[9] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, half ? r.b.w : r.c};
+                uint32_t out[16];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t codes = __builtin_amdgcn_alignbyte(seq[j + 1], seq[j], straddle);
+                    // two signed bytes -> the fp16 integers: 0x6400 | (byte ^ 0x80) is 1152 + code
+                    const uint32_t lo = __builtin_amdgcn_perm(0U, codes, 0x0c010c00U) ^ bias_bits;
+                    const uint32_t hi = __builtin_amdgcn_perm(0U, codes, 0x0c030c02U) ^ bias_bits;
+                    out[2 * j] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2v, lo) + minus2);
+                    out[2 * j + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2v, hi) + minus2);
+                }
+                uint8_t* tile_w = w_tile[s & 1U];
+#pragma unroll
+                for (uint32_t i = 0; i < 4U; ++i)
+                    *reinterpret_cast<u32x4*>(tile_w + pf_at(lrow, 4U * half + i)) = u32x4{out[4 * i], out[4 * i + 1], out[4 * i + 2], out[4 * i + 3]};
+                d_scale[s & 1U][kPfTile * half + lrow] = half_bits_to_float(half ? r.c >> 16 : r.a.x & 0xffffU);
+            };
+            // Schedule of one step: token copy of step + 3 (4 operations), fetch of step + 4 into the slot used up by the
+            // previous step's staging (3 operations), stage step + 1 (fetched three steps ago: 21 younger operations),
+            // wait for the token copy of step + 1 (issued two steps ago, ahead of that step's fetch: 3 + 14), barrier. The
+            // prologue issues the sequence of three steps before the first.
+            PfRaw8 raw[4];
+            fetch8(0, raw[0]);
+            copy_tokens(0, tok_stage[0]); fetch8(1, raw[1]);
+            copy_tokens(1, tok_stage[1]); fetch8(2, raw[2]);
+            copy_tokens(2, tok_stage[2]); fetch8(3, raw[3]);
+            // younger than the first token copy (and than the first fetch before it): 3 + 7 + 7
+            asm volatile("s_waitcnt vmcnt(17)" : "+v"(raw[0].a), "+v"(raw[0].b), "+v"(raw[0].c) : : "memory");
+            stage8(0, raw[0]);
+            pf_barrier();
+            for (uint32_t s0 = 0; s0 < steps; s0 += 4U) {
+#pragma unroll
+                for (uint32_t u = 0; u < 4U; ++u) {
+                    const uint32_t s = s0 + u;
+                    copy_tokens(s + kPfTokenAhead, tok_stage[(u + kPfTokenAhead) & 3U]);
+                    fetch8(s + 4U, raw[u]);
+                    PfRaw8& next = raw[(u + 1U) & 3U];
+                    asm volatile("s_waitcnt vmcnt(21)" : "+v"(next.a), "+v"(next.b), "+v"(next.c) : : "memory");
+                    if (s < last) stage8(s + 1U, next);
+                    wait_copies<17>();
+                    pf_barrier();
+                }
+            }
+            continue;
+        }
+        // Every memory operation below is issued unconditionally (indices past the end are clamped: such copies land in
+        // stages nobody reads any more), so the number of operations between an issue and the point that needs its data
+        // is a compile-time constant and the waits are plain s_waitcnt vmcnt(n) of this code's own: the compiler is not
+        // told about these operations, whose bookkeeping across loop iterations it resolves by waiting for all of them.
         const auto copy_sums = [&](uint32_t g) {                           // 2 operations: 16 sub-blocks of group g -> s_tile[g % 2]
             const uint32_t gc = g < last_group ? g : last_group;
 #pragma unroll
@@ -373,6 +443,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                     for (uint32_t n = 0; n < 2U; ++n) ws[n] = *reinterpret_cast<const half8*>(wt + n * 32U * 128U + piece_at[ks]);
                 };
                 read(0, x[0], w[0]);
+                float d8[2][2];                               // Q8_0: d of the step's two blocks for the wave's two feature tiles
+                if (FMT == 1) {
+#pragma unroll
+                    for (uint32_t g = 0; g < 2U; ++g)
+#pragma unroll
+                        for (uint32_t n = 0; n < 2U; ++n) d8[g][n] = d_scale[s & 1U][kPfTile * g + 64U * wr + 32U * n + l31];
+                }
 #pragma unroll
                 for (uint32_t ks = 0; ks < 4U; ++ks) {
                     if (ks < 3U) read(ks + 1U, x[(ks + 1U) & 1U], w[(ks + 1U) & 1U]);
@@ -380,13 +457,28 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
 #pragma unroll
                     for (uint32_t i = 0; i < NT; ++i)
 #pragma unroll
-                        for (uint32_t n = 0; n < 2U; ++n) part[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks & 1U][i], w[ks & 1U][n], part[i][n], 0, 0, 0);
+                        for (uint32_t n = 0; n < 2U; ++n) {
+                            if (FMT == 1 && (ks & 1U) == 0) {     // first half of a block: the product starts from zero
+                                const floatx16 zero = {0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F};
+                                part[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks & 1U][i], w[ks & 1U][n], zero, 0, 0, 0);
+                            } else {
+                                part[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks & 1U][i], w[ks & 1U][n], part[i][n], 0, 0, 0);
+                            }
+                        }
                     __builtin_amdgcn_sched_barrier(0);
+                    if (FMT == 1 && (ks & 1U)) {                  // end of a block: running sum += d * product
+#pragma unroll
+                        for (uint32_t i = 0; i < NT; ++i)
+#pragma unroll
+                            for (uint32_t n = 0; n < 2U; ++n)
+#pragma unroll
+                                for (int j = 0; j < 16; ++j) acc[i][n][j] = __builtin_fmaf(d8[ks >> 1][n], part[i][n][j], acc[i][n][j]);
+                    }
                 }
             };
             if (live_tiles >= TT) k_steps(std::integral_constant<uint32_t, TT>{});
             else if (live_tiles == 1U) k_steps(std::integral_constant<uint32_t, 1>{});
-            if (p == 3U) {
+            if (FMT == 0 && p == 3U) {
                 // end of a super-block: running sum += d * P, P = 0
                 const uint32_t b = s >> 2;
                 const float d[2] = {d_scale[b & 1U][64U * wr + l31], d_scale[b & 1U][64U * wr + 32U + l31]};
@@ -459,7 +551,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                         _Float16* sums = reinterpret_cast<_Float16*>(a.h_sums + static_cast<size_t>(begin + n) * pf_sum_row_bytes(a.features));
                         split_half(sum, sums[sub_block], sums[pf_sum_slots(a.features) + sub_block]);
                     }
-                    if (!(finite_f(g) && finite_f(u) && finite_f(hv))) {
+                    if (!(finite_f(g) && finite_f(u) && finite_f(static_cast<float>(h16)))) {     // h beyond fp16 counts as non-finite
                         atomicOr(&a.status[order[begin + n] / a.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
                         atomicOr(a.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
                     }

@@ -337,16 +337,30 @@ __global__ __launch_bounds__(64) void route_select_kernel(RouteArgs a) {
 // ======================================================================================================== expert plan
 // (layout of the plan words: see the router section above)
 
-// Stable order of a large batch: one wave per expert walks the assignments in order, 64 at a time, and places its own by
-// ballot + prefix count (the offsets are already in the plan).
-__global__ __launch_bounds__(64) void plan_order_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
-    const uint32_t e = blockIdx.x, lane = threadIdx.x;
-    uint32_t at = plan[kPlanOffsetsAt + e];
-    const uint32_t end = plan[kPlanOffsetsAt + e + 1];
-    uint32_t* order = plan + plan_order_at(experts);
-    for (uint32_t a0 = 0; a0 < assignments && at < end; a0 += 64U) {
+// Stable order of a large batch: one 16-wave workgroup per expert. Every wave owns a contiguous sixteenth of the assignments:
+// it first counts its own assignments of the expert (ballot + population count, 64 at a time), the counts of the waves before
+// it give its first position, and a second walk places them in index order (the offsets are already in the plan).
+__global__ __launch_bounds__(1024) void plan_order_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
+    __shared__ uint32_t wave_count[16];
+    const uint32_t e = blockIdx.x, lane = threadIdx.x & 63U, wave = threadIdx.x >> 6;
+    const uint32_t first = plan[kPlanOffsetsAt + e], end = plan[kPlanOffsetsAt + e + 1];
+    if (first == end) return;                                   // uniform over the workgroup
+    const uint32_t per = ((assignments + 15U) / 16U + 63U) & ~63U;
+    const uint32_t lo = wave * per < assignments ? wave * per : assignments, hi = lo + per < assignments ? lo + per : assignments;
+    uint32_t mine_total = 0;
+    for (uint32_t a0 = lo; a0 < hi; a0 += 64U) {
         const uint32_t a = a0 + lane;
-        const bool mine = a < assignments && routes[a] == e;
+        mine_total += static_cast<uint32_t>(__popcll(__ballot(a < hi && routes[a] == e)));
+    }
+    if (lane == 0) wave_count[wave] = mine_total;
+    __syncthreads();
+    uint32_t at = first;
+    for (uint32_t w = 0; w < wave; ++w) at += wave_count[w];
+    const uint32_t stop = at + mine_total;
+    uint32_t* order = plan + plan_order_at(experts);
+    for (uint32_t a0 = lo; a0 < hi && at < stop; a0 += 64U) {
+        const uint32_t a = a0 + lane;
+        const bool mine = a < hi && routes[a] == e;
         const uint64_t votes = __ballot(mine);
         if (mine) order[at + __popcll(votes & ((1ULL << lane) - 1ULL))] = a;
         at += static_cast<uint32_t>(__popcll(votes));
@@ -669,8 +683,9 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, mi355_m
     __shared__ uint32_t row_failed;
     const uint32_t row = blockIdx.y, o = blockIdx.x * 256U + threadIdx.x;
     if (threadIdx.x == 0) {
-        // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is this kernel's own)
-        row_failed = r.status[row] & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE);
+        // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is this kernel's own), and
+        // neither does any row of a job whose down phase was skipped (its unweighted outputs are not this job's)
+        row_failed = (r.status[row] & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE)) | (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION);
         for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
         if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
             for (uint32_t i = 1; i < w.top_k; ++i)
@@ -797,9 +812,11 @@ inline void launch_down_dense(const mi355_moe_weights& w, const mi355_moe_rows& 
 
 inline void launch_plan(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t split, uint32_t bound, uint32_t* plan,
                         hipStream_t st) {
-    const bool large = assignments > 4096U;
+    // plan_kernel's own order fill is one thread per expert walking every assignment: fine for a decode batch, far too slow
+    // beyond a few hundred assignments (4096 assignments of one expert: 0.55 ms), where a wave per expert does it instead
+    const bool large = assignments > 256U;
     plan_kernel<<<1, 1024, 0, st>>>(routes, experts, assignments, split, bound, large ? 0U : 1U, plan);
-    if (large) plan_order_kernel<<<experts, 64, 0, st>>>(routes, experts, assignments, plan);
+    if (large) plan_order_kernel<<<experts, 1024, 0, st>>>(routes, experts, assignments, plan);
 }
 inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     if (dense_pairs_ok(w, rows) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
@@ -831,26 +848,38 @@ inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
 }
 
 // ======================================================================================================== admission
-int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv) {
+// bytes of a GGUF row of k weights (k a multiple of 256)
+inline uint64_t moe_row_bytes(uint32_t type, uint32_t k) {
+    return type == MI355_TYPE_Q8_0 ? static_cast<uint64_t>(k / 32U) * kQ80Block : static_cast<uint64_t>(k / 256U) * kQ4kBlock;
+}
+
+// q8_0_too: the matrix-core prefill form also takes Q8_0 expert tensors (a dense shared expert is experts = top_k = 1)
+int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, bool q8_0_too = false) {
     STRIX_REQUIRE(w && r, "moe: null weights or rows");
     STRIX_REQUIRE(rows > 0, "moe: rows must be positive");
-    STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K, "moe: gate/up weights must be Q4_K (type 12)");
-    if (w->down_type != MI355_TYPE_Q4_K) return fail(MI355_E_UNSUPPORTED, "moe: down weights must be Q4_K (type 12)");
+    if (q8_0_too) {
+        STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || w->gate_type == MI355_TYPE_Q8_0, "moe prefill: gate/up weights must be Q4_K (type 12) or Q8_0 (type 8)");
+        if (w->down_type != MI355_TYPE_Q4_K && w->down_type != MI355_TYPE_Q8_0)
+            return fail(MI355_E_UNSUPPORTED, "moe prefill: down weights must be Q4_K (type 12) or Q8_0 (type 8)");
+    } else {
+        STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K, "moe: gate/up weights must be Q4_K (type 12)");
+        if (w->down_type != MI355_TYPE_Q4_K) return fail(MI355_E_UNSUPPORTED, "moe: down weights must be Q4_K (type 12)");
+    }
     STRIX_REQUIRE(w->hidden >= 256 && w->hidden % 256U == 0, "moe: hidden must be a positive multiple of 256");
     STRIX_REQUIRE(w->ffn >= 256 && w->ffn % 256U == 0, "moe: ffn must be a positive multiple of 256");
     STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
     STRIX_REQUIRE(w->top_k > 0 && w->top_k <= kRouteMaxTopK && w->top_k <= w->experts, "moe: top_k must be within 1..16 and <= experts");
     STRIX_REQUIRE(static_cast<uint64_t>(rows) * w->top_k < (1ULL << 31), "moe: too many assignments");
     wv = *w;
-    if (wv.gate_row_stride == 0) wv.gate_row_stride = static_cast<uint64_t>(w->hidden / 256U) * kQ4kBlock;
+    if (wv.gate_row_stride == 0) wv.gate_row_stride = moe_row_bytes(w->gate_type, w->hidden);
     if (wv.gate_expert_stride == 0) wv.gate_expert_stride = wv.gate_row_stride * w->ffn;
-    if (wv.down_row_stride == 0) wv.down_row_stride = static_cast<uint64_t>(w->ffn / 256U) * kQ4kBlock;
+    if (wv.down_row_stride == 0) wv.down_row_stride = moe_row_bytes(w->down_type, w->ffn);
     if (wv.down_expert_stride == 0) wv.down_expert_stride = wv.down_row_stride * w->hidden;
     STRIX_REQUIRE(wv.gate_row_stride % 16U == 0 && wv.gate_expert_stride % 16U == 0 && wv.down_row_stride % 16U == 0 &&
                   wv.down_expert_stride % 16U == 0, "moe: weight strides must be multiples of 16 bytes");
     STRIX_REQUIRE(wv.gate_row_stride < (1ULL << 27) && wv.down_row_stride < (1ULL << 27), "moe: weight row stride must be below 128 MiB");
-    STRIX_REQUIRE(wv.gate_row_stride >= static_cast<uint64_t>(w->hidden / 256U) * kQ4kBlock &&
-                  wv.down_row_stride >= static_cast<uint64_t>(w->ffn / 256U) * kQ4kBlock, "moe: weight row stride shorter than the row");
+    STRIX_REQUIRE(wv.gate_row_stride >= moe_row_bytes(w->gate_type, w->hidden) &&
+                  wv.down_row_stride >= moe_row_bytes(w->down_type, w->ffn), "moe: weight row stride shorter than the row");
     STRIX_REQUIRE(w->gate && w->up && w->down && aligned(w->gate, 16) && aligned(w->up, 16) && aligned(w->down, 16),
                   "moe: weight pointers must be non-null and 16-byte aligned");
     STRIX_REQUIRE(w->exp_kind <= MI355_EXP_DECLARED, "moe: unknown exp kind");
@@ -1055,7 +1084,7 @@ int32_t mi355_moe_enqueue_down(const mi355_moe_weights* w, const mi355_moe_rows*
 
 int32_t mi355_moe_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
     mi355_moe_weights wv;
-    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    if (const int32_t rc = check_moe(w, r, rows, wv, true)) return rc;      // the merge reads no weights: either tensor type
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe merge: unknown combine form");
     STRIX_REQUIRE(rows <= 65535U, "moe merge: at most 65535 rows per call");
     merge_kernel<<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(wv, *r, form);
@@ -1120,7 +1149,7 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
 
 int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
     mi355_moe_weights wv;
-    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    if (const int32_t rc = check_moe(w, r, rows, wv, true)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe prefill: unknown combine form");
     STRIX_REQUIRE(r->input && r->input_kind == MI355_INPUT_F16, "moe prefill: the fp16 form takes fp16 input rows");
     STRIX_REQUIRE(r->input_stride % 16U == 0 && aligned(r->input, 16), "moe prefill: input rows must be 16-byte aligned");
@@ -1148,10 +1177,12 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     if (hipGetDevice(&device) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
     const uint32_t resident = static_cast<uint32_t>(cus > 8 ? cus : 8) & ~7U;
     a.tiles = wv.ffn / 64U; a.units = item_slots * a.tiles;
-    prefill_f16_kernel<0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    if (wv.gate_type == MI355_TYPE_Q8_0) prefill_f16_kernel<0, 1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    else prefill_f16_kernel<0, 0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     a.wa = wv.down; a.wb = nullptr; a.expert_stride = wv.down_expert_stride; a.row_stride = wv.down_row_stride; a.k = wv.ffn; a.features = wv.hidden;
     a.tiles = wv.hidden / 128U; a.units = item_slots * a.tiles;
-    prefill_f16_kernel<1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    if (wv.down_type == MI355_TYPE_Q8_0) prefill_f16_kernel<1, 1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    else prefill_f16_kernel<1, 0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     STRIX_LAUNCHED("moe prefill f16");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }

@@ -13,10 +13,11 @@ from test_gpu_parity import TOL_F16, bits, dev, rel_err
 pytestmark = pytest.mark.gpu
 
 
-def device_q4k(gen, rows_shape, width):
-    """Random Q4_K blocks with finite, moderate fp16 d / dmin (every other bit of a block is random)."""
+def device_q4k(gen, rows_shape, width, d_bits=0x13):
+    """Random Q4_K blocks with finite, moderate fp16 d / dmin (every other bit of a block is random); d_bits = 0x03 keeps d
+    below 2^-11, so that h of a 4096-wide product stays far inside fp16."""
     w = torch.randint(0, 256, rows_shape + (width // 256, 144), dtype=torch.uint8, device="cuda", generator=gen)
-    w[..., 1] = (w[..., 1] & 0x13) | 0x0C
+    w[..., 1] = (w[..., 1] & d_bits) | 0x0C
     w[..., 3] = (w[..., 3] & 0x03) | 0x0C
     return w.reshape(rows_shape + (width // 256 * 144,))
 
@@ -127,3 +128,47 @@ def test_config4_prefill_full_size(strix):
     base_n = base.cpu().numpy()
     assert np.array_equal(bits(base_n[sel]), bits(b_ref))
     check_rows(layer, y, sel, xn, ids_ref, w_ref, gate.cpu().numpy(), up.cpu().numpy(), down.cpu().numpy(), H, I, K, 0, base=base_n)
+
+
+def test_config4_prefill_f16_mfma_full_size(strix):
+    """BASELINE config 4 in the matrix-core class: router, the Q8_0 shared expert as a one-expert prefill layer whose output is
+    the base of the routed combine, the 256 Q4_K routed experts. 12 random rows are checked against the exact-weight product
+    in float64 (shared expert output, unweighted routed outputs and the final rows) with the stated tolerance 2e-3, as max
+    abs error over the reference rms and elementwise on the outputs of at least rms size."""
+    H, I, E, K, T = 4096, 2048, 256, 8, 4096
+    gen = torch.Generator(device="cuda").manual_seed(40)
+    gate, up, down = device_q4k(gen, (E, I), H, 0x03), device_q4k(gen, (E, I), H, 0x03), device_q4k(gen, (E, H), I, 0x03)
+    sg, su, sd = device_q8_0(gen, I, H), device_q8_0(gen, I, H), device_q8_0(gen, H, I)
+    wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
+    bias = torch.randn(E, device="cuda", generator=gen) * 1.5
+    x = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)
+    ids, wts, _ = strix.route(x, wr, K, bias=bias)
+    dense = strix.MoeLayer(H, I, 1, 1, sg.reshape(1, I, -1), su.reshape(1, I, -1), sd.reshape(1, H, -1), T, prefill_f16=True,
+                           gate_type=strix.TYPE_Q8_0, down_type=strix.TYPE_Q8_0)
+    base = dense.run_prefill_f16(x, torch.zeros((T, 1), dtype=torch.int32, device="cuda"), torch.ones((T, 1), dtype=torch.float32, device="cuda"))
+    layer = strix.MoeLayer(H, I, E, K, gate, up, down, T, prefill_f16=True)
+    y = layer.run_prefill_f16(x, ids, wts, base=base).cpu().numpy()
+    assert int(layer.status.sum()) == 0 and int(dense.status.sum()) == 0
+    sel = np.sort(np.random.default_rng(45).choice(T, 12, replace=False))
+    xs = x.cpu().numpy()[sel].astype(np.float64)
+    ids_n, w_n = ids.cpu().numpy()[sel].astype(np.int64), wts.cpu().numpy()[sel]
+
+    def ffn(rows, wg, wu, wd, qtype):
+        g = rows @ orc.dequant_rows(qtype, wg, H).astype(np.float64).T
+        u = rows @ orc.dequant_rows(qtype, wu, H).astype(np.float64).T
+        return ((g / (1.0 + np.exp(-g))) * u) @ orc.dequant_rows(qtype, wd, I).astype(np.float64).T
+
+    def close(got, ref):
+        rms = np.sqrt(np.mean(ref ** 2))
+        assert np.max(np.abs(got - ref)) / rms < TOL_F16
+        big = np.abs(ref) >= rms
+        assert np.max(np.abs(got[big] - ref[big]) / np.abs(ref[big])) < TOL_F16
+
+    base_ref = ffn(xs, sg.cpu().numpy(), su.cpu().numpy(), sd.cpu().numpy(), orc.Q8_0)
+    close(base.cpu().numpy()[sel], base_ref)
+    raw_ref = np.zeros((len(sel), K, H))
+    for e in np.unique(ids_n):
+        r, k = np.nonzero(ids_n == e)
+        raw_ref[r, k] = ffn(xs[r], gate[e].cpu().numpy(), up[e].cpu().numpy(), down[e].cpu().numpy(), orc.Q4_K)
+    close(layer.rawdots.cpu().numpy()[sel], raw_ref)
+    close(y[sel], base_ref + np.einsum("tk,tkh->th", w_n.astype(np.float64), raw_ref))

@@ -461,20 +461,89 @@ def test_admission_failures_return_before_any_enqueue(strix):
 
 
 # ------------------------------------------------------------------------------------------- prefill on the matrix cores
-def exact_weight_layer(x, ids, wts, gate, up, down, H, I, K, base=None):
+def exact_weight_layer(x, ids, wts, gate, up, down, H, I, K, base=None, gate_type=orc.Q4_K, down_type=orc.Q4_K):
     """Exact-weight (BASE class) evaluation of the routed experts in float64 from the decoder's fp32 weights."""
     T = x.shape[0]
     raw = np.zeros((T, K, H), np.float32)
     x64 = x.astype(np.float64)
     for e in np.unique(ids):
-        wg = orc.dequant_rows(orc.Q4_K, gate[e], H).astype(np.float64)
-        wu = orc.dequant_rows(orc.Q4_K, up[e], H).astype(np.float64)
-        wd = orc.dequant_rows(orc.Q4_K, down[e], I).astype(np.float64)
+        wg = orc.dequant_rows(gate_type, gate[e], H).astype(np.float64)
+        wu = orc.dequant_rows(gate_type, up[e], H).astype(np.float64)
+        wd = orc.dequant_rows(down_type, down[e], I).astype(np.float64)
         rows, slots = np.nonzero(ids == e)
         g, u = x64[rows] @ wg.T, x64[rows] @ wu.T
         h = (g / (1.0 + np.exp(-g))) * u
         raw[rows, slots] = (h @ wd.T).astype(np.float32)
     return orc.combine(0, wts, ids, raw, base=base), raw
+
+
+def random_q8_0(rng, shape_rows, width):
+    """Q8_0 rows of random bytes (every code incl. -128) with small finite scales of either sign."""
+    w = rng.integers(0, 256, shape_rows + (width // 32 * 34,), dtype=np.uint8)
+    w[..., 1::34] = (w[..., 1::34] & 0x83) | 0x20        # |d| in [2^-7, 2^-6)
+    return w
+
+
+@pytest.mark.parametrize("H,I,E,K,T,gate_type,down_type,random_bytes", [
+    (512, 256, 1, 1, 300, orc.Q8_0, orc.Q8_0, False),       # a dense (shared) expert: one expert, every row routed to it
+    (768, 1280, 3, 2, 150, orc.Q8_0, orc.Q8_0, False),
+    (256, 512, 1, 1, 129, orc.Q8_0, orc.Q8_0, True),
+    (512, 512, 4, 2, 200, orc.Q8_0, orc.Q4_K, False),
+    (512, 256, 4, 2, 90, orc.Q4_K, orc.Q8_0, False)])
+def test_prefill_f16_mfma_q8_0_tensors(strix, H, I, E, K, T, gate_type, down_type, random_bytes):
+    """The matrix-core prefill form with Q8_0 expert tensors (the always-on shared expert is experts = top_k = 1 with weight 1)
+    against the exact-weight product, tolerance 2e-3 as for Q4_K: max abs error over the output rms, and elementwise on the
+    outputs of at least rms size, for the unweighted down outputs and the combined output."""
+    rng = np.random.default_rng(7 * H + T)
+    def tensor(qtype, rows, width):
+        if random_bytes:
+            return random_q8_0(rng, (E, rows), width)
+        return orc.quantize_rows(qtype, (rng.standard_normal((E, rows, width)) * 0.02).astype(np.float32))
+    gate, up, down = tensor(gate_type, I, H), tensor(gate_type, I, H), tensor(down_type, H, I)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    if E == 1:
+        ids_ref, w_ref = np.zeros((T, 1), np.int64), np.ones((T, 1), np.float32)
+    else:
+        wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+        ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, prefill_f16=True, gate_type=gate_type, down_type=down_type)
+    y = layer.run_prefill_f16(dev(x), dev(ids_ref.astype(np.int32)), dev(w_ref)).cpu().numpy()
+    want, raw_ref = exact_weight_layer(x, ids_ref, w_ref, gate, up, down, H, I, K, gate_type=gate_type, down_type=down_type)
+    for got, ref in ((layer.rawdots[:T].cpu().numpy(), raw_ref), (y, want)):
+        ref64 = ref.astype(np.float64)
+        rms = np.sqrt(np.mean(ref64 ** 2))
+        assert np.max(np.abs(got - ref64)) / rms < TOL_F16
+        big = np.abs(ref64) >= rms
+        assert np.max(np.abs(got[big] - ref64[big]) / np.abs(ref64[big])) < TOL_F16
+    assert np.all(layer.status[:T].cpu().numpy() == 0)
+    # the decode entries keep refusing Q8_0 expert tensors
+    with pytest.raises(strix.StrixError):
+        layer.run(dev(x[:1]), dev(ids_ref[:1].astype(np.int32)), dev(w_ref[:1]))
+
+
+def test_prefill_f16_h_beyond_fp16_fails_closed(strix):
+    """The prefill form keeps h in fp16: a row whose h leaves the fp16 range is flagged as a non-finite projection, the job's
+    down phase is skipped, the merge publishes no row, and a clean call on the same buffers afterwards is unaffected."""
+    H, I, E, K, T = 512, 256, 4, 2, 40
+    rng = np.random.default_rng(77)
+    gate, up, down = make_layer(rng, H, I, E)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    ids, w, _, _ = orc.route(x.astype(np.float32), wr, K)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, prefill_f16=True)
+    want = layer.run_prefill_f16(dev(x), dev(ids.astype(np.int32)), dev(w)).clone()
+    assert int(layer.status.sum()) == 0
+    loud = x.copy()
+    loud[3] *= 4096.0                                       # gate and up of row 3 grow 4096-fold: h far beyond 65504
+    layer.output.fill_(-7.0)
+    layer.rawdots.fill_(-3.0)
+    y = layer.run_prefill_f16(dev(loud), dev(ids.astype(np.int32)), dev(w))
+    st = layer.status[:T].cpu().numpy()
+    assert st[3] & strix.STATUS_NONFINITE_PROJECTION and np.all(np.delete(st, 3) == 0)
+    assert int(layer.job_status[0]) & strix.STATUS_NONFINITE_PROJECTION
+    assert bool((layer.rawdots == -3.0).all()) and bool((y == -7.0).all())
+    again = layer.run_prefill_f16(dev(x), dev(ids.astype(np.int32)), dev(w))
+    assert torch.equal(again, want) and int(layer.status.sum()) == 0
 
 
 @pytest.mark.parametrize("H,I,E,K,T", [(512, 256, 6, 2, 300), (1024, 512, 12, 4, 77), (256, 256, 3, 1, 129), (768, 1280, 5, 2, 150)])
