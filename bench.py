@@ -145,6 +145,61 @@ def extra_config3_small(strix, torch, cfg, steps, warmup):
     return out
 
 
+def extra_config3_executor_formats(strix, torch, cfg, steps, warmup, with_cpu):
+    """Config 3 (T rows) with the down tensors in the reference host executor's own format (Q8_0 blocks of 32): the workload
+    the compiled reference can run itself. GPU: the whole layer; CPU: the reference's Executor (its best ISA, every host
+    thread) on the expert job of layer 0 (A8 rows in, rawdots out: no router, no combine)."""
+    H, I, E, K, T = cfg.H, cfg.I, cfg.E, cfg.K, cfg.T
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    layers = []
+    for layer, wr, x in cfg.layers:
+        w8 = torch.randint(0, 256, (E * H, I // 32, 34), dtype=torch.uint8, device="cuda", generator=gen)
+        w8[..., 1] = (w8[..., 1] & 0x03) | 0x14
+        layers.append((strix.MoeLayer(H, I, E, K, layer.gate, layer.up, w8.reshape(E, H, -1), T, down_type=strix.TYPE_Q8_0), wr, x))
+    n = len(layers)
+
+    def step(i):
+        layer, wr, x = layers[i % n]
+        layer.run_layer(x, wr)
+    sec = time_steps(torch, step, max(steps, 60), max(warmup, 12))
+    entry = {"us": sec * 1e6, "down_format": "Q8_0 (34-byte blocks of 32), four chains per row"}
+    if with_cpu:
+        import ctypes as C
+        import orc
+        R = orc.ref()
+        if R is not None:
+            layer, wr, x = layers[0]
+            xn = x.cpu().numpy().astype(np.float32)
+            ids, _, _, _ = orc.route(xn, wr.cpu().numpy(), K)
+            c, d, s, _ = orc.quantize_a8(xn)
+            gate, up, down = (t.cpu().numpy() for t in (layer.gate, layer.up, layer.down))
+            asg = np.array([[t, k, ids[t, k]] for t in range(T) for k in range(K)], np.uint32)
+            raw, status = np.zeros((T, K, H), np.float32), np.zeros(T, np.uint32)
+            threads = orc.lib().orc_max_threads()
+            R.ref_executor_run.restype = C.c_int
+            pool = C.c_void_p(R.ref_executor_create(threads, 1))
+
+            def run():
+                return R.ref_executor_run(pool, H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down.ctypes.data_as(orc.u8p), 0,
+                                          c.ctypes.data_as(orc.i8p), d.ctypes.data_as(orc.f32p), s.ctypes.data_as(orc.i32p), T,
+                                          asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
+                                          status.ctypes.data_as(orc.u32p))
+            if run() == 0:
+                times, t_end = [], time.perf_counter() + 5.0
+                while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
+                    t0 = time.perf_counter()
+                    run()
+                    times.append(time.perf_counter() - t0)
+                layer.run_layer(x, wr)
+                torch.cuda.synchronize()
+                entry["cpu_reference"] = {"value": statistics.median(times) * 1e6, "unit": "us/expert job", "cores": threads, "kind": "reference",
+                                          "isa": R.ref_executor_isa(pool).decode(),
+                                          "sample": f"the reference's own Executor on layer 0's expert job, median of {len(times)} passes",
+                                          "rawdots_equal_gpu_bits": bool(np.array_equal(raw.view(np.uint32), layer.rawdots[:T].cpu().numpy().view(np.uint32)))}
+            R.ref_executor_destroy(pool)
+    return {f"config3_moe_decode_T{T}_q8_0_down": entry}
+
+
 def extra_configs(strix, torch, steps, warmup):
     """BASELINE configs 1, 2, 4, 5 on synthetic full-entropy blocks; HBM-bound ones rotate over enough weight sets to stay cold."""
     gen = torch.Generator(device="cuda").manual_seed(11)
@@ -354,6 +409,7 @@ def main():
     }
     if args.extra:
         small = extra_config3_small(strix, torch, cfg, args.steps, args.warmup) if args.tokens >= 4 else {}
+        small.update(extra_config3_executor_formats(strix, torch, cfg, args.steps, args.warmup, not args.no_cpu))
         del cfg.layers[1:]
         out["extra"] = {**small, **extra_configs(strix, torch, args.steps, args.warmup)}
     if not args.no_cpu:

@@ -136,13 +136,32 @@ void ref_down_row_q8_0(const std::uint8_t* wrow, std::uint32_t groups, const std
     ex::detail::scalar_kernels().down[1](wrow, groups, &codes, &deltas, &sums, 1, out);
 }
 
-// Whole routed-expert job (Q4_K gate/up, Q8_0 down; the host executor has no Q4_K down), empty exp tables.
-// assignments: count x {row, slot, expert}. executor_threads == 0: reference_run (scalar oracle); otherwise the pool.
+void ref_down_row_q5_1(const std::uint8_t* wrow, std::uint32_t groups, const std::int8_t* codes, const float* deltas,
+                       const std::int32_t* sums, float* out) {
+    ex::detail::scalar_kernels().down[0](wrow, groups, &codes, &deltas, &sums, 1, out);
+}
+
+// Whole routed-expert job (Q4_K gate/up; down Q8_0, or Q5_1 when down_q5_1 != 0; the host executor has no Q4_K down),
+// empty exp tables. assignments: count x {row, slot, expert}. executor_threads == 0: reference_run (scalar oracle);
+// otherwise the pool.
+int ref_routed_expert_run_fmt(std::uint32_t hidden, std::uint32_t ffn, const std::uint8_t* gate, const std::uint8_t* up,
+                              const std::uint8_t* down, int down_q5_1, const std::int8_t* codes, const float* deltas,
+                              const std::int32_t* sums, std::uint32_t rows, const std::uint32_t* assignments,
+                              std::uint32_t count, float* rawdots, std::uint64_t rawdot_row_stride, std::uint32_t* status,
+                              unsigned executor_threads, int allow_simd);
 int ref_routed_expert_run(std::uint32_t hidden, std::uint32_t ffn, const std::uint8_t* gate, const std::uint8_t* up,
                           const std::uint8_t* down_q8_0, const std::int8_t* codes, const float* deltas,
                           const std::int32_t* sums, std::uint32_t rows, const std::uint32_t* assignments,
                           std::uint32_t count, float* rawdots, std::uint64_t rawdot_row_stride, std::uint32_t* status,
                           unsigned executor_threads, int allow_simd) {
+    return ref_routed_expert_run_fmt(hidden, ffn, gate, up, down_q8_0, 0, codes, deltas, sums, rows, assignments, count, rawdots,
+                                     rawdot_row_stride, status, executor_threads, allow_simd);
+}
+int ref_routed_expert_run_fmt(std::uint32_t hidden, std::uint32_t ffn, const std::uint8_t* gate, const std::uint8_t* up,
+                              const std::uint8_t* down_q8_0, int down_q5_1, const std::int8_t* codes, const float* deltas,
+                              const std::int32_t* sums, std::uint32_t rows, const std::uint32_t* assignments,
+                              std::uint32_t count, float* rawdots, std::uint64_t rawdot_row_stride, std::uint32_t* status,
+                              unsigned executor_threads, int allow_simd) {
     return guarded([&] {
         std::vector<ex::RowA8> row_views(rows);
         for (std::uint32_t r = 0; r < rows; ++r)
@@ -150,7 +169,7 @@ int ref_routed_expert_run(std::uint32_t hidden, std::uint32_t ffn, const std::ui
         std::vector<ex::Assignment> as(count);
         for (std::uint32_t a = 0; a < count; ++a) as[a] = {assignments[3 * a], assignments[3 * a + 1], assignments[3 * a + 2]};
         ex::Job job;
-        job.weights = {gate, up, down_q8_0, ex::GateFormat::q4_k, ex::DownFormat::q8_0, {hidden, ffn}};
+        job.weights = {gate, up, down_q8_0, ex::GateFormat::q4_k, down_q5_1 ? ex::DownFormat::q5_1 : ex::DownFormat::q8_0, {hidden, ffn}};
         job.rows = row_views.data(); job.assignments = as.data(); job.count = count;
         job.rawdots = rawdots; job.rawdot_row_stride = rawdot_row_stride; job.status = status;
         if (executor_threads == 0) ex::reference_run(job, empty_table_exp());
@@ -163,6 +182,24 @@ void* ref_executor_create(unsigned threads, int allow_simd) {
     try { return new ex::Executor(threads, empty_table_exp(), allow_simd != 0); } catch (const std::exception& e) { g_error = e.what(); return nullptr; }
 }
 const char* ref_executor_isa(void* pool) { return static_cast<ex::Executor*>(pool)->isa(); }
+// One job on the persistent pool (arguments as ref_routed_expert_run_fmt).
+int ref_executor_run(void* pool, std::uint32_t hidden, std::uint32_t ffn, const std::uint8_t* gate, const std::uint8_t* up,
+                     const std::uint8_t* down, int down_q5_1, const std::int8_t* codes, const float* deltas, const std::int32_t* sums,
+                     std::uint32_t rows, const std::uint32_t* assignments, std::uint32_t count, float* rawdots,
+                     std::uint64_t rawdot_row_stride, std::uint32_t* status) {
+    return guarded([&] {
+        std::vector<ex::RowA8> row_views(rows);
+        for (std::uint32_t r = 0; r < rows; ++r)
+            row_views[r] = {codes + std::size_t{r} * hidden, deltas + std::size_t{r} * (hidden / 32), sums + std::size_t{r} * (hidden / 32)};
+        std::vector<ex::Assignment> as(count);
+        for (std::uint32_t a = 0; a < count; ++a) as[a] = {assignments[3 * a], assignments[3 * a + 1], assignments[3 * a + 2]};
+        ex::Job job;
+        job.weights = {gate, up, down, ex::GateFormat::q4_k, down_q5_1 ? ex::DownFormat::q5_1 : ex::DownFormat::q8_0, {hidden, ffn}};
+        job.rows = row_views.data(); job.assignments = as.data(); job.count = count;
+        job.rawdots = rawdots; job.rawdot_row_stride = rawdot_row_stride; job.status = status;
+        static_cast<ex::Executor*>(pool)->run(job);
+    });
+}
 void ref_executor_destroy(void* pool) { delete static_cast<ex::Executor*>(pool); }
 
 // Router policy (softmax scores with a Math trait, then selection and weights).

@@ -298,6 +298,29 @@ float orc_q8_0_down_row_a8(const uint8_t* wrow, uint32_t groups, const int8_t* c
     return s01 + s23;
 }
 
+/* src/cpu/core/routed_expert.cpp:110-144 with Q51: block = fp16 d, fp16 m, 32 fifth bits, 16 nibble bytes; weight k is
+ * nibble k % 16 (low halves for k < 16, high halves after) plus bit k of the fifth-bit word; the minimum enters through the
+ * group's code sum. */
+float orc_q5_1_down_row_a8(const uint8_t* wrow, uint32_t groups, const int8_t* codes, const float* deltas, const int32_t* sums) {
+    float acc[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+    for (uint32_t g = 0; g < groups; ++g) {
+        const uint8_t* blk = wrow + (size_t)g * ORC_Q5_1_BLOCK;
+        const float d = orc_half_to_float(le16(blk)), m = orc_half_to_float(le16(blk + 2));
+        const uint32_t fifth = (uint32_t)blk[4] | ((uint32_t)blk[5] << 8) | ((uint32_t)blk[6] << 16) | ((uint32_t)blk[7] << 24);
+        int dot = 0;
+        for (uint32_t k = 0; k < 32; ++k) {
+            const uint8_t byte = blk[8 + (k & 15U)];
+            const int q = (int)(k < 16 ? (byte & 15U) : (byte >> 4)) | (int)(((fifth >> k) & 1U) << 4);
+            dot += (int)codes[32 * g + k] * q;
+        }
+        const float first = d * (float)dot;
+        const float combined = first + (m * (float)sums[g]);
+        acc[g % 4] = acc[g % 4] + (deltas[g] * combined);
+    }
+    const float s01 = acc[0] + acc[1], s23 = acc[2] + acc[3];
+    return s01 + s23;
+}
+
 /* ------------------------------------------------------------------ exp / SwiGLU */
 /* src/cpu/core/routed_expert.cpp:248-261 with v_exp = float(exp2(double(a))) (:212-216; the probe-table
  * corrections of :217-226 need tables that are not in the reference tree, so none apply here). */
@@ -467,6 +490,7 @@ void orc_routed_down(const orc_expert_weights* w, const orc_expert_job* job, int
             const int32_t* s = job->h_sums + (size_t)a * groups;
             float value;
             if (w->down_type == ORC_Q4_K) value = orc_q4k_row_a8(wrow, ffn / 256, c, d, s);   /* src/moe_a8_down_contract.cpp:146 */
+            else if (w->down_type == ORC_Q5_1) value = orc_q5_1_down_row_a8(wrow, groups, c, d, s);
             else value = orc_q8_0_down_row_a8(wrow, groups, c, d);
             job->rawdots[(size_t)a * hidden + o] = value;
         }

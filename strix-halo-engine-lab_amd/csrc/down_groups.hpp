@@ -1,0 +1,118 @@
+// Down rows in the formats of the reference's host executor: Q8_0 and Q5_1 blocks of 32 weights against the A8 image of h
+// (src/cpu/core/routed_expert.cpp:110-144, "down (Q5_1 | Q8_0, groups of 32, chain j 0..3 owns groups g = 4c + j, c
+// ascending)", src/cpu/core/routed_expert.hpp:13). Per group: an exact int32 dot, first = d * float(dot),
+// Q5_1: combined = first + (m * float(sum of the group's codes)), chain[g % 4] += delta_g * combined; the row's value is
+// (chain0 + chain1) + (chain2 + chain3).
+//
+// The four chains of a row are independent, so a wavefront holds 16 output rows with lane = (row, chain): a lane walks
+// its chain's groups in ascending order and two quad exchanges form the value, bit for bit the sequential result. A
+// 256-thread workgroup covers 64 output rows of one plan item (an expert and up to `split` of its assignments); every
+// weight block a lane loads is used for up to four assignments before the next one is fetched.
+//
+// Block addresses. Q8_0 blocks are 34 bytes, so a row's blocks alternate between 4-byte and 2-byte alignment; the chain
+// index fixes which (g = 4c + j is odd exactly when j is). A lane reads nine aligned words: for even j the words from the
+// block's start (d in the low half of the first, every code word straddling two of them), for odd j the eight words from the
+// first code and the word before them (d in its high half). Q5_1 blocks are 24 bytes (fp16 d, fp16 m, 32 fifth bits, 16
+// bytes of nibbles; weight k is nibble k % 16 of the low (k < 16) or high halves plus bit k of the fifth-bit word) and
+// always 8-byte aligned.
+#pragma once
+#include "device_math.hpp"
+#include "q4k_rows.hpp"
+
+namespace strix950 {
+
+constexpr uint32_t kDownGroupsRows = 64;       // output rows per workgroup (4 waves x 16)
+constexpr uint32_t kDownGroupsAssignments = 4; // assignments per weight pass
+
+// FMT 0: Q8_0, FMT 1: Q5_1. Loads the lane's block and returns d, m and the eight words of signed / 5-bit codes in the
+// order of the activation codes.
+template <int FMT>
+__device__ __forceinline__ void load_group_block(const uint8_t* block, uint32_t odd, float& d, float& m, uint32_t (&q)[8]) {
+    typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+    if (FMT == 0) {
+        const uint8_t* first = block + 2U * odd;                              // odd: the first code, even: the block's start
+        const u32x4_a4 a = *reinterpret_cast<const u32x4_a4*>(first), b = *reinterpret_cast<const u32x4_a4*>(first + 16);
+        const uint32_t c = *reinterpret_cast<const uint32_t*>(odd ? first - 4 : first + 32);
+        const uint32_t seq[9] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w, c};
+        const uint32_t straddle = odd ? 0U : 2U;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = __builtin_amdgcn_alignbyte(i == 7 && odd ? seq[7] : seq[i + 1], seq[i], straddle);
+        d = half_bits_to_float(odd ? c >> 16 : a.x & 0xffffU);
+        m = 0.0F;
+    } else {
+        const u32x2_a4 head = *reinterpret_cast<const u32x2_a4*>(block);
+        const u32x4_a4 nib = *reinterpret_cast<const u32x4_a4*>(block + 8);
+        d = half_bits_to_float(head.x & 0xffffU);
+        m = half_bits_to_float(head.x >> 16);
+        const uint32_t fifth = head.y, n[4] = {nib.x, nib.y, nib.z, nib.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // four bits of the fifth-bit word -> bit 4 of four bytes: the product places bit b at 8 b (the shifted copies
+            // of a 4-bit value do not overlap, so nothing carries)
+            const uint32_t lo5 = (((fifth >> (4 * i)) & 15U) * 0x00204081U & 0x01010101U) << 4;
+            const uint32_t hi5 = (((fifth >> (16 + 4 * i)) & 15U) * 0x00204081U & 0x01010101U) << 4;
+            q[i] = (n[i] & 0x0f0f0f0fU) | lo5;
+            q[4 + i] = ((n[i] >> 4) & 0x0f0f0f0fU) | hi5;
+        }
+    }
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments,
+                                                          uint32_t items_at, uint32_t order_at) {
+    typedef uint32_t u32x4_g __attribute__((ext_vector_type(4)));
+    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * blockIdx.y);
+    const uint32_t e = item.x, begin = item.y, end = item.z;
+    if (begin == end) return;
+    if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
+    const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, j = lane & 3U, odd = j & 1U;
+    const uint32_t o = blockIdx.x * kDownGroupsRows + 16U * wave + (lane >> 2);
+    const uint32_t groups = w.ffn / 32U, per_chain = groups / 4U;
+    constexpr uint32_t kBlock = FMT == 0 ? 34U : 24U;
+    const uint8_t* wrow = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o) * w.down_row_stride + kBlock * j;
+    const uint32_t* order = r.plan + order_at;
+    for (uint32_t c0 = begin; c0 < end; c0 += kDownGroupsAssignments) {
+        const uint32_t na = end - c0 < kDownGroupsAssignments ? end - c0 : kDownGroupsAssignments;
+        uint32_t src[kDownGroupsAssignments];
+        float chain[kDownGroupsAssignments];
+#pragma unroll
+        for (uint32_t a = 0; a < kDownGroupsAssignments; ++a) {
+            src[a] = order[c0 + (a < na ? a : na - 1U)];
+            chain[a] = 0.0F;
+        }
+#pragma unroll 2
+        for (uint32_t c = 0; c < per_chain; ++c) {
+            const uint32_t g = 4U * c + j;
+            float d, m;
+            uint32_t q[8];
+            load_group_block<FMT>(wrow + static_cast<size_t>(c) * (4U * kBlock), odd, d, m, q);
+#pragma unroll
+            for (uint32_t a = 0; a < kDownGroupsAssignments; ++a) {
+                if (a < na) {                                     // uniform over the workgroup
+                    const u32x4_g* codes = reinterpret_cast<const u32x4_g*>(r.down_codes + static_cast<size_t>(src[a]) * w.ffn + 32U * g);
+                    const u32x4_g c_lo = codes[0], c_hi = codes[1];
+                    const uint32_t cw[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+                    int dot = 0;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) dot = __builtin_amdgcn_sdot4(static_cast<int>(q[i]), static_cast<int>(cw[i]), dot, false);
+                    const float first = d * static_cast<float>(dot);
+                    float combined = first;
+                    if (FMT == 1) combined = first + (m * static_cast<float>(r.down_sums[static_cast<size_t>(src[a]) * groups + g]));
+                    chain[a] = chain[a] + (r.down_deltas[static_cast<size_t>(src[a]) * groups + g] * combined);
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t a = 0; a < kDownGroupsAssignments; ++a) {
+            if (a < na) {
+                float v = chain[a];
+                v = v + xor1_f(v);          // chain0 + chain1 | chain2 + chain3
+                v = v + xor2_f(v);          // (chain0 + chain1) + (chain2 + chain3)
+                if (j == 0) r.rawdots[static_cast<size_t>(src[a]) * w.hidden + o] = v;
+            }
+        }
+    }
+}
+
+}  // namespace strix950

@@ -14,6 +14,7 @@
 #include "q4k_rows.hpp"
 #include "q4k_pairs.hpp"
 #include "q4k_quads.hpp"
+#include "down_groups.hpp"
 #include "prefill_f16.hpp"
 #include "route_wave.hpp"
 
@@ -825,6 +826,13 @@ inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, 
     else launch_project_nb<4>(w, r, rows, grid, st);
 }
 inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+    if (w.down_type != MI355_TYPE_Q4_K) {      // the host executor's formats: blocks of 32, four chains per row
+        const uint32_t assignments = rows * w.top_k, items_at = plan_items_at(w.experts, assignments), order_at = plan_order_at(w.experts);
+        const dim3 grid(w.hidden / kDownGroupsRows, umax);
+        if (w.down_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+        else down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+        return;
+    }
     if (dense_pairs_ok(w, rows)) return launch_down_dense(w, r, rows, st);
     const dim3 grid(w.hidden / 64U, umax);
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
@@ -850,21 +858,24 @@ inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
 // ======================================================================================================== admission
 // bytes of a GGUF row of k weights (k a multiple of 256)
 inline uint64_t moe_row_bytes(uint32_t type, uint32_t k) {
-    return type == MI355_TYPE_Q8_0 ? static_cast<uint64_t>(k / 32U) * kQ80Block : static_cast<uint64_t>(k / 256U) * kQ4kBlock;
+    if (type == MI355_TYPE_Q8_0) return static_cast<uint64_t>(k / 32U) * kQ80Block;
+    if (type == MI355_TYPE_Q5_1) return static_cast<uint64_t>(k / 32U) * 24U;
+    return static_cast<uint64_t>(k / 256U) * kQ4kBlock;
 }
 
-// q8_0_too: the matrix-core prefill form also takes Q8_0 expert tensors (a dense shared expert is experts = top_k = 1)
-int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, bool q8_0_too = false) {
+// Tensor formats by arithmetic class. Integer-dot entries: Q4_K gate/up; down Q4_K, or the host executor's Q8_0 / Q5_1
+// (src/cpu/core/routed_expert.hpp:28). The matrix-core prefill form: Q4_K or Q8_0 for either (a dense shared expert is
+// experts = top_k = 1). The merge reads no weights.
+enum MoeClass { kIntegerClass, kPrefillClass, kAnyClass };
+int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, MoeClass cls = kIntegerClass) {
     STRIX_REQUIRE(w && r, "moe: null weights or rows");
     STRIX_REQUIRE(rows > 0, "moe: rows must be positive");
-    if (q8_0_too) {
-        STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || w->gate_type == MI355_TYPE_Q8_0, "moe prefill: gate/up weights must be Q4_K (type 12) or Q8_0 (type 8)");
-        if (w->down_type != MI355_TYPE_Q4_K && w->down_type != MI355_TYPE_Q8_0)
-            return fail(MI355_E_UNSUPPORTED, "moe prefill: down weights must be Q4_K (type 12) or Q8_0 (type 8)");
-    } else {
-        STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K, "moe: gate/up weights must be Q4_K (type 12)");
-        if (w->down_type != MI355_TYPE_Q4_K) return fail(MI355_E_UNSUPPORTED, "moe: down weights must be Q4_K (type 12)");
-    }
+    const bool gate_q8 = w->gate_type == MI355_TYPE_Q8_0, down_q8 = w->down_type == MI355_TYPE_Q8_0, down_q51 = w->down_type == MI355_TYPE_Q5_1;
+    STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || (gate_q8 && cls != kIntegerClass),
+                  cls == kIntegerClass ? "moe: gate/up weights must be Q4_K (type 12)" : "moe prefill: gate/up weights must be Q4_K (type 12) or Q8_0 (type 8)");
+    if (!(w->down_type == MI355_TYPE_Q4_K || down_q8 || (down_q51 && cls != kPrefillClass)))
+        return fail(MI355_E_UNSUPPORTED, cls == kPrefillClass ? "moe prefill: down weights must be Q4_K (type 12) or Q8_0 (type 8)"
+                                                               : "moe: down weights must be Q4_K (type 12), Q8_0 (type 8) or Q5_1 (type 7)");
     STRIX_REQUIRE(w->hidden >= 256 && w->hidden % 256U == 0, "moe: hidden must be a positive multiple of 256");
     STRIX_REQUIRE(w->ffn >= 256 && w->ffn % 256U == 0, "moe: ffn must be a positive multiple of 256");
     STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
@@ -1084,7 +1095,7 @@ int32_t mi355_moe_enqueue_down(const mi355_moe_weights* w, const mi355_moe_rows*
 
 int32_t mi355_moe_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
     mi355_moe_weights wv;
-    if (const int32_t rc = check_moe(w, r, rows, wv, true)) return rc;      // the merge reads no weights: either tensor type
+    if (const int32_t rc = check_moe(w, r, rows, wv, kAnyClass)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe merge: unknown combine form");
     STRIX_REQUIRE(rows <= 65535U, "moe merge: at most 65535 rows per call");
     merge_kernel<<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(wv, *r, form);
@@ -1134,10 +1145,12 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     if (items <= quad_max && wv.experts > 1U) {
         if (items <= 16U) {
             project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
-            down_quad_kernel<4><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+            if (wv.down_type != MI355_TYPE_Q4_K) launch_down(wv, *r, rows, items, hs(stream));
+            else down_quad_kernel<4><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
         } else {
             project_quad_kernel<2><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
-            down_quad_kernel<2><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+            if (wv.down_type != MI355_TYPE_Q4_K) launch_down(wv, *r, rows, items, hs(stream));
+            else down_quad_kernel<2><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
         }
     } else {
         launch_project(wv, *r, rows, items, hs(stream));
@@ -1149,7 +1162,7 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
 
 int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
     mi355_moe_weights wv;
-    if (const int32_t rc = check_moe(w, r, rows, wv, true)) return rc;
+    if (const int32_t rc = check_moe(w, r, rows, wv, kPrefillClass)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe prefill: unknown combine form");
     STRIX_REQUIRE(r->input && r->input_kind == MI355_INPUT_F16, "moe prefill: the fp16 form takes fp16 input rows");
     STRIX_REQUIRE(r->input_stride % 16U == 0 && aligned(r->input, 16), "moe prefill: input rows must be 16-byte aligned");

@@ -9,8 +9,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 
-Q8_0, Q4_K = 8, 12
-Q8_0_BLOCK, Q4_K_BLOCK = 34, 144
+Q5_1, Q8_0, Q4_K = 7, 8, 12
+Q5_1_BLOCK, Q8_0_BLOCK, Q4_K_BLOCK = 24, 34, 144
 EXP_GFX1151, EXP_DECLARED = 0, 1
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
 COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
@@ -105,6 +105,7 @@ def _declare(L):
     L.orc_q4k_row_a8.restype = C.c_float
     L.orc_q4k_row_a8_contract_form.restype = C.c_float
     L.orc_q8_0_down_row_a8.restype = C.c_float
+    L.orc_q5_1_down_row_a8.restype = C.c_float
     L.orc_expf_gfx1151.restype = C.c_float
     L.orc_expf_gfx1151.argtypes = [C.c_float]
     L.orc_declared_exp.restype = C.c_float
@@ -115,6 +116,8 @@ def _declare(L):
 
 # ---------------------------------------------------------------- numpy-level helpers
 def row_bytes(qtype, elements):
+    if qtype == Q5_1:
+        return elements // 32 * Q5_1_BLOCK
     return elements // 32 * Q8_0_BLOCK if qtype == Q8_0 else elements // 256 * Q4_K_BLOCK
 
 
@@ -182,6 +185,32 @@ def q8_0_down_row_a8(wrow, codes, deltas):
     wrow = np.ascontiguousarray(wrow, np.uint8)
     return np.float32(lib().orc_q8_0_down_row_a8(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q8_0_BLOCK), _ptr(codes, i8p),
                                                  _ptr(deltas, f32p)))
+
+
+def q5_1_down_row_a8(wrow, codes, deltas, sums):
+    wrow = np.ascontiguousarray(wrow, np.uint8)
+    return np.float32(lib().orc_q5_1_down_row_a8(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q5_1_BLOCK), _ptr(codes, i8p),
+                                                 _ptr(deltas, f32p), _ptr(sums, i32p)))
+
+
+def random_q5_1(rng, shape_rows, width):
+    """Q5_1 rows of random bytes (every nibble and fifth bit) with finite fp16 d and m of either sign around 2^-6."""
+    w = rng.integers(0, 256, tuple(shape_rows) + (width // 32 * Q5_1_BLOCK,), dtype=np.uint8)
+    w[..., 1::Q5_1_BLOCK] = (w[..., 1::Q5_1_BLOCK] & 0x83) | 0x20
+    w[..., 3::Q5_1_BLOCK] = (w[..., 3::Q5_1_BLOCK] & 0x83) | 0x20
+    return w
+
+
+def dequant_q5_1_rows(raw, width):
+    """ggml Q5_1: x_k = d * q_k + m, q_k = nibble | fifth bit << 4 (the layout of src/cpu/core/routed_expert.cpp:121-131)."""
+    raw = np.ascontiguousarray(raw, np.uint8).reshape(-1, width // 32, Q5_1_BLOCK)
+    d = raw[..., 0:2].copy().view(np.float16).astype(np.float32)
+    m = raw[..., 2:4].copy().view(np.float16).astype(np.float32)
+    fifth = raw[..., 4:8].copy().view(np.uint32)
+    nib = raw[..., 8:24]
+    k = np.arange(32)
+    q = np.where(k < 16, nib[..., k % 16] & 15, nib[..., k % 16] >> 4).astype(np.uint32) | (((fifth >> k) & 1) << 4)
+    return (d * q.astype(np.float32) + m).reshape(raw.shape[0], width)
 
 
 def swiglu_quantize(g, u, exp_kind=EXP_GFX1151):

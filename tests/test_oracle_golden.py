@@ -528,13 +528,16 @@ def test_combine_forms_and_commit_threshold():
 def _tiny_layer(rng, H, I, E, T, K, down_type):
     gate = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32))
     up = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32))
-    down = orc.quantize_rows(down_type, (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32))
+    if down_type == orc.Q5_1:
+        down = orc.random_q5_1(rng, (E, H), I)
+    else:
+        down = orc.quantize_rows(down_type, (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32))
     x = rng.standard_normal((T, H)).astype(np.float16).astype(np.float32)
     ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.uint32)
     return gate, up, down, x, ids
 
 
-@pytest.mark.parametrize("down_type", [orc.Q4_K, orc.Q8_0])
+@pytest.mark.parametrize("down_type", [orc.Q4_K, orc.Q8_0, orc.Q5_1])
 def test_routed_experts_against_double_precision_dequant_reference(down_type):
     """Brute force: A8-quantise explicitly, dequantise weights with the (separately pinned) block decoders, sum in
     double. The declared fp32 chain must agree to fp32 accumulation accuracy; a dropped term or a wrong index is O(1)."""
@@ -556,7 +559,8 @@ def test_routed_experts_against_double_precision_dequant_reference(down_type):
             ha = r.h_codes[a].astype(np.float64) * np.repeat(r.h_deltas[a].astype(np.float64), 32)
             hd = r.gate[a].astype(np.float64) / (1 + np.exp(-r.gate[a].astype(np.float64))) * r.up[a].astype(np.float64)
             assert np.max(np.abs(ha - hd)) <= np.abs(hd).reshape(-1, 32).max(-1).repeat(32).max() / 127 * 0.51 + 1e-9
-            D = orc.dequant_rows(down_type, down[e], I).astype(np.float64) @ ha
+            wd = orc.dequant_q5_1_rows(down[e], I) if down_type == orc.Q5_1 else orc.dequant_rows(down_type, down[e], I)
+            D = wd.astype(np.float64) @ ha
             assert np.max(np.abs(r.rawdots[t, k] - D)) < 2e-5 * max(1, np.abs(D).max())
     # the down phase alone, from the same h image, gives the same bits (stage-by-stage form used by the GPU tests)
     r2 = orc.routed_experts(H, I, K, gate, up, down, down_type, codes, deltas, sums, ids, down_only_from=(r.h_codes, r.h_deltas, r.h_sums))
@@ -684,6 +688,10 @@ def test_ref_q4k_row_and_down_row_bits_at_config_widths():
         R.ref_down_row_q8_0(w8.ctypes.data_as(orc.u8p), width // 32, codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
                             sums[0].ctypes.data_as(orc.i32p), C.byref(out))
         assert bits(orc.q8_0_down_row_a8(w8, codes[0], deltas[0])) == bits(np.float32(out.value))
+        w5 = orc.random_q5_1(rng, (1,), width)[0]
+        R.ref_down_row_q5_1(w5.ctypes.data_as(orc.u8p), width // 32, codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
+                            sums[0].ctypes.data_as(orc.i32p), C.byref(out))
+        assert bits(orc.q5_1_down_row_a8(w5, codes[0], deltas[0], sums[0])) == bits(np.float32(out.value))
 
 
 @needs_ref
@@ -716,6 +724,19 @@ def test_ref_whole_routed_expert_job_bits():
                                      status.ctypes.data_as(orc.u32p), threads, simd)
         assert rc == 0, R.ref_last_error()
         assert np.array_equal(bits(raw), bits(mine.rawdots)) and np.all(status == 0)
+    # the executor's other down format: Q5_1 (random blocks: the reference has no writer for it either)
+    down5 = orc.random_q5_1(rng, (E, H), I)
+    mine5 = orc.routed_experts(H, I, K, gate, up, down5, orc.Q5_1, codes, deltas, sums, ids)
+    assert not np.array_equal(bits(mine5.rawdots), bits(mine.rawdots))
+    for threads, simd in ((0, 0), (3, 1)):
+        raw = np.zeros((T, K, H), np.float32)
+        status = np.zeros(T, np.uint32)
+        rc = R.ref_routed_expert_run_fmt(H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down5.ctypes.data_as(orc.u8p), 1,
+                                         codes.ctypes.data_as(orc.i8p), deltas.ctypes.data_as(orc.f32p), sums.ctypes.data_as(orc.i32p), T,
+                                         asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
+                                         status.ctypes.data_as(orc.u32p), threads, simd)
+        assert rc == 0, R.ref_last_error()
+        assert np.array_equal(bits(raw), bits(mine5.rawdots)) and np.all(status == 0)
 
 
 @needs_ref
