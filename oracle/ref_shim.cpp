@@ -131,6 +131,12 @@ void ref_gate_row_q4k(const std::uint8_t* wrow, std::uint32_t blocks, const std:
     const ex::RowA8* rows[1] = {&row};
     ex::detail::scalar_kernels().gate[0](wrow, blocks, rows, 1, out);
 }
+void ref_gate_row_q5k(const std::uint8_t* wrow, std::uint32_t blocks, const std::int8_t* codes, const float* deltas,
+                      const std::int32_t* sums, float* out) {
+    const ex::RowA8 row{codes, deltas, sums};
+    const ex::RowA8* rows[1] = {&row};
+    ex::detail::scalar_kernels().gate[1](wrow, blocks, rows, 1, out);
+}
 void ref_down_row_q8_0(const std::uint8_t* wrow, std::uint32_t groups, const std::int8_t* codes, const float* deltas,
                        const std::int32_t* sums, float* out) {
     ex::detail::scalar_kernels().down[1](wrow, groups, &codes, &deltas, &sums, 1, out);
@@ -141,7 +147,8 @@ void ref_down_row_q5_1(const std::uint8_t* wrow, std::uint32_t groups, const std
     ex::detail::scalar_kernels().down[0](wrow, groups, &codes, &deltas, &sums, 1, out);
 }
 
-// Whole routed-expert job (Q4_K gate/up; down Q8_0, or Q5_1 when down_q5_1 != 0; the host executor has no Q4_K down),
+// Whole routed-expert job (gate/up Q4_K, or Q5_K when bit 1 of down_q5_1 is set; down Q8_0, or Q5_1 when bit 0 of down_q5_1
+// is set; the host executor has no Q4_K down),
 // empty exp tables. assignments: count x {row, slot, expert}. executor_threads == 0: reference_run (scalar oracle);
 // otherwise the pool.
 int ref_routed_expert_run_fmt(std::uint32_t hidden, std::uint32_t ffn, const std::uint8_t* gate, const std::uint8_t* up,
@@ -169,7 +176,8 @@ int ref_routed_expert_run_fmt(std::uint32_t hidden, std::uint32_t ffn, const std
         std::vector<ex::Assignment> as(count);
         for (std::uint32_t a = 0; a < count; ++a) as[a] = {assignments[3 * a], assignments[3 * a + 1], assignments[3 * a + 2]};
         ex::Job job;
-        job.weights = {gate, up, down_q8_0, ex::GateFormat::q4_k, down_q5_1 ? ex::DownFormat::q5_1 : ex::DownFormat::q8_0, {hidden, ffn}};
+        job.weights = {gate, up, down_q8_0, (down_q5_1 & 2) ? ex::GateFormat::q5_k : ex::GateFormat::q4_k,
+                       (down_q5_1 & 1) ? ex::DownFormat::q5_1 : ex::DownFormat::q8_0, {hidden, ffn}};
         job.rows = row_views.data(); job.assignments = as.data(); job.count = count;
         job.rawdots = rawdots; job.rawdot_row_stride = rawdot_row_stride; job.status = status;
         if (executor_threads == 0) ex::reference_run(job, empty_table_exp());
@@ -194,7 +202,8 @@ int ref_executor_run(void* pool, std::uint32_t hidden, std::uint32_t ffn, const 
         std::vector<ex::Assignment> as(count);
         for (std::uint32_t a = 0; a < count; ++a) as[a] = {assignments[3 * a], assignments[3 * a + 1], assignments[3 * a + 2]};
         ex::Job job;
-        job.weights = {gate, up, down, ex::GateFormat::q4_k, down_q5_1 ? ex::DownFormat::q5_1 : ex::DownFormat::q8_0, {hidden, ffn}};
+        job.weights = {gate, up, down, (down_q5_1 & 2) ? ex::GateFormat::q5_k : ex::GateFormat::q4_k,
+                       (down_q5_1 & 1) ? ex::DownFormat::q5_1 : ex::DownFormat::q8_0, {hidden, ffn}};
         job.rows = row_views.data(); job.assignments = as.data(); job.count = count;
         job.rawdots = rawdots; job.rawdot_row_stride = rawdot_row_stride; job.status = status;
         static_cast<ex::Executor*>(pool)->run(job);

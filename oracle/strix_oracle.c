@@ -253,6 +253,37 @@ float orc_q4k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, 
     return s01 + s23;
 }
 
+/* src/cpu/core/routed_expert.cpp:73-108 with Q5K: 176-byte blocks (d, dmin, 12 factor bytes as in Q4_K, 32 fifth-bit bytes
+ * - bit j of byte k belongs to element k of sub-block j -, 128 nibble bytes); q = nibble | fifth bit << 4. */
+float orc_q5k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,
+                     const int32_t* sums) {
+    float acc[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+    for (uint32_t b = 0; b < blocks; ++b) {
+        const uint8_t* blk = wrow + (size_t)b * ORC_Q5_K_BLOCK;
+        const float d = orc_half_to_float(le16(blk)), dm = orc_half_to_float(le16(blk + 2));
+        float x[8];
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t p = j >> 1, hi = j & 1;
+            int dot = 0;
+            for (uint32_t k = 0; k < 32; ++k) {
+                const uint8_t byte = blk[48 + 32 * p + k];
+                int q = hi ? (byte >> 4) : (byte & 15);
+                q |= ((blk[16 + k] >> j) & 1) << 4;
+                dot += (int)codes[256 * b + 32 * j + k] * q;
+            }
+            const float D = d * (float)orc_q4k_factor_words(blk, j, 0);
+            const float DM = dm * (float)orc_q4k_factor_words(blk, j, 1);
+            const float u = D * (float)dot;
+            const float v = DM * (float)sums[8 * b + j];
+            const float t = u - v;
+            x[j] = deltas[8 * b + j] * t;
+        }
+        for (uint32_t p = 0; p < 4; ++p) acc[p] = acc[p] + (x[2 * p] + x[2 * p + 1]);
+    }
+    const float s01 = acc[0] + acc[1], s23 = acc[2] + acc[3];
+    return s01 + s23;
+}
+
 float orc_q4k_row_a8_contract_form(const uint8_t* wrow, uint32_t blocks, const int8_t* codes,
                                    const float* deltas, const int32_t* sums) {
     float acc[4] = {0.0F, 0.0F, 0.0F, 0.0F};
@@ -513,8 +544,13 @@ int orc_routed_experts(const orc_expert_weights* w, const orc_expert_job* job, i
             float g[32], u[32], h[32];
             for (uint32_t l = 0; l < 32; ++l) {
                 const uint32_t o = grp * 32 + l;
-                g[l] = orc_q4k_row_a8(gate_row_ptr(w, w->gate, expert, o), blocks, codes, deltas, sums);
-                u[l] = orc_q4k_row_a8(gate_row_ptr(w, w->up, expert, o), blocks, codes, deltas, sums);
+                if (w->gate_type == ORC_Q5_K) {
+                    g[l] = orc_q5k_row_a8(gate_row_ptr(w, w->gate, expert, o), blocks, codes, deltas, sums);
+                    u[l] = orc_q5k_row_a8(gate_row_ptr(w, w->up, expert, o), blocks, codes, deltas, sums);
+                } else {
+                    g[l] = orc_q4k_row_a8(gate_row_ptr(w, w->gate, expert, o), blocks, codes, deltas, sums);
+                    u[l] = orc_q4k_row_a8(gate_row_ptr(w, w->up, expert, o), blocks, codes, deltas, sums);
+                }
             }
             if (job->gate_out) memcpy(job->gate_out + (size_t)a * ffn + grp * 32, g, sizeof g);
             if (job->up_out) memcpy(job->up_out + (size_t)a * ffn + grp * 32, u, sizeof u);

@@ -49,6 +49,28 @@ struct QuadSource {
     }
 };
 
+// The pair term of a super-block from its header words and the two integer dots (sub-blocks 2p, 2p + 1):
+// x_j = delta_j * (d * sc_j * float(dot_j) - dmin * m_j * float(sum_j)), returned as x_2p + x_(2p+1). e0 / e1: the group
+// deltas, f0 / f1: the group sums as floats. Reference: src/cpu/core/routed_expert.cpp:87-104 (the same for Q4_K and Q5_K).
+__device__ __forceinline__ float quad_pair_term(const u32x4& hd, uint32_t p, int dot0, int dot1, float e0, float e1, float f0, float f1) {
+    // 6-bit scale / min of sub-blocks 2p, 2p + 1 (src/cpu/core/routed_expert.cpp:65-71); branch-free choice between the two
+    // packings (pairs 0, 1: 6 low bits; pairs 2, 3: 4 + 2 split bits)
+    const uint32_t sh0 = 16U * (p & 1U), sh1 = sh0 + 8U;
+    const uint32_t fa0 = (hd.y >> sh0) & 255U, fb0 = (hd.z >> sh0) & 255U, fc0 = (hd.w >> sh0) & 255U;
+    const uint32_t fa1 = (hd.y >> sh1) & 255U, fb1 = (hd.z >> sh1) & 255U, fc1 = (hd.w >> sh1) & 255U;
+    const uint32_t lowmask = 0U - static_cast<uint32_t>(p < 2U);
+    const auto pick = [lowmask](uint32_t lo6, uint32_t split) { return split ^ ((lo6 ^ split) & lowmask); };
+    const uint32_t s0 = pick(fa0 & 63U, (fc0 & 15U) | ((fa0 >> 6) << 4)), m0 = pick(fb0 & 63U, (fc0 >> 4) | ((fb0 >> 6) << 4));
+    const uint32_t s1 = pick(fa1 & 63U, (fc1 & 15U) | ((fa1 >> 6) << 4)), m1 = pick(fb1 & 63U, (fc1 >> 4) | ((fb1 >> 6) << 4));
+    const float d = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
+    const float D0 = d * static_cast<float>(s0), M0 = dm * static_cast<float>(m0);
+    const float D1 = d * static_cast<float>(s1), M1 = dm * static_cast<float>(m1);
+    const float u0 = D0 * static_cast<float>(dot0), v0 = M0 * f0;
+    const float u1 = D1 * static_cast<float>(dot1), v1 = M1 * f1;
+    const float x0 = e0 * (u0 - v0), x1 = e1 * (u1 - v1);
+    return x0 + x1;
+}
+
 // One super-block (index kb along K): the lane's pair of its row. vd / vf: the activation row's group deltas / sums,
 // group 8 (kb % 8) + j in lane 8 (kb % 8) + j.
 __device__ __forceinline__ void quad_block_compute(const lds_u8* slot, uint32_t kb, float vd, float vf, float& acc) {
@@ -66,24 +88,9 @@ __device__ __forceinline__ void quad_block_compute(const lds_u8* slot, uint32_t 
         dot0 = __builtin_amdgcn_sdot4(static_cast<int>(w[k] & 0x0f0f0f0fU), static_cast<int>(cw[k]), dot0, false);
         dot1 = __builtin_amdgcn_sdot4(static_cast<int>((w[k] >> 4) & 0x0f0f0f0fU), static_cast<int>(cw[8 + k]), dot1, false);
     }
-    // 6-bit scale / min of sub-blocks 2p, 2p + 1 (src/cpu/core/routed_expert.cpp:65-71); branch-free choice between the two
-    // packings (pairs 0, 1: 6 low bits; pairs 2, 3: 4 + 2 split bits)
-    const uint32_t sh0 = 16U * (p & 1U), sh1 = sh0 + 8U;
-    const uint32_t fa0 = (hd.y >> sh0) & 255U, fb0 = (hd.z >> sh0) & 255U, fc0 = (hd.w >> sh0) & 255U;
-    const uint32_t fa1 = (hd.y >> sh1) & 255U, fb1 = (hd.z >> sh1) & 255U, fc1 = (hd.w >> sh1) & 255U;
-    const uint32_t lowmask = 0U - static_cast<uint32_t>(p < 2U);
-    const auto pick = [lowmask](uint32_t lo6, uint32_t split) { return split ^ ((lo6 ^ split) & lowmask); };
-    const uint32_t s0 = pick(fa0 & 63U, (fc0 & 15U) | ((fa0 >> 6) << 4)), m0 = pick(fb0 & 63U, (fc0 >> 4) | ((fb0 >> 6) << 4));
-    const uint32_t s1 = pick(fa1 & 63U, (fc1 & 15U) | ((fa1 >> 6) << 4)), m1 = pick(fb1 & 63U, (fc1 >> 4) | ((fb1 >> 6) << 4));
-    const float d = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
-    const float D0 = d * static_cast<float>(s0), M0 = dm * static_cast<float>(m0);
-    const float D1 = d * static_cast<float>(s1), M1 = dm * static_cast<float>(m1);
     const int from = static_cast<int>((kb & 7U) * 8U + 2U * p);
     const float e0 = __shfl(vd, from), e1 = __shfl(vd, from + 1), f0 = __shfl(vf, from), f1 = __shfl(vf, from + 1);
-    const float u0 = D0 * static_cast<float>(dot0), v0 = M0 * f0;
-    const float u1 = D1 * static_cast<float>(dot1), v1 = M1 * f1;
-    const float x0 = e0 * (u0 - v0), x1 = e1 * (u1 - v1);
-    acc = acc + (x0 + x1);
+    acc = acc + quad_pair_term(hd, p, dot0, dot1, e0, e1, f0, f1);
 }
 
 // Whole sweep of the wave's 16 rows against activation row `row` of `img`; every lane of a quad returns the row's value.

@@ -15,6 +15,7 @@
 #include "q4k_pairs.hpp"
 #include "q4k_quads.hpp"
 #include "down_groups.hpp"
+#include "q5k_quads.hpp"
 #include "prefill_f16.hpp"
 #include "route_wave.hpp"
 
@@ -655,6 +656,56 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
     }
 }
 
+// The same for Q5_K gate / up tensors (q5k_quads.hpp), for every assignment of the item in turn.
+__global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+    __shared__ float wg_amax[4];
+    __shared__ int wg_sum[4], wg_bad[4];
+    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
+    const uint32_t e = item.x, begin = item.y, end = item.z;
+    const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x, groups = w.ffn / 32U;
+    const uint32_t f0 = grp * 32U + 8U * wave;
+    const uint8_t* wrow = (lane < 32U ? w.gate : w.up) + static_cast<size_t>(e) * w.gate_expert_stride +
+                          static_cast<size_t>(f0 + (rr & 7U)) * w.gate_row_stride;
+    const bool mine = lane < 32U && p == 0;                   // the lane that publishes feature f0 + rr
+    for (uint32_t a = begin; a < end; ++a) {
+        const uint32_t sidx = __builtin_amdgcn_readfirstlane(r.plan[plan_order_at(w.experts) + a]), row = sidx / w.top_k;
+        const float value = sweep_q5k_row(wrow, w.hidden / 256U, A8Image{r.codes, r.deltas, r.sums, w.hidden}, row, p);
+        const float other = __shfl_xor(value, 32);
+        const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
+        const float h = (g / (1.0F + exp_of(w.exp_kind, -g))) * u;
+        const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
+        if (mine) {
+            if (r.gate_out) r.gate_out[at] = g;
+            if (r.up_out) r.up_out[at] = u;
+            if (r.h_out) r.h_out[at] = h;
+        }
+        const int bad = or32_i((mine && !(finite_f(g) && finite_f(u) && finite_f(h))) ? 1 : 0);
+        const float amax_wave = max32(mine ? __builtin_fabsf(h) : 0.0F);
+        __syncthreads();                                          // the previous assignment's reads of the shared words are done
+        if (lane == 0) { wg_amax[wave] = amax_wave; wg_bad[wave] = bad; }
+        __syncthreads();
+        if (wg_bad[0] | wg_bad[1] | wg_bad[2] | wg_bad[3]) {      // uniform over the workgroup
+            if (threadIdx.x == 0) {
+                atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            }
+            continue;
+        }
+        const float amax = __builtin_fmaxf(__builtin_fmaxf(wg_amax[0], wg_amax[1]), __builtin_fmaxf(wg_amax[2], wg_amax[3]));
+        const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+        const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+        const int code = a8_code(h, dl, tiny);
+        const int sum_wave = sum32_i(mine ? code : 0);
+        if (lane == 0) wg_sum[wave] = sum_wave;
+        if (mine) r.down_codes[at] = static_cast<int8_t>(code);
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
+            r.down_sums[static_cast<size_t>(sidx) * groups + grp] = wg_sum[0] + wg_sum[1] + wg_sum[2] + wg_sum[3];
+        }
+    }
+}
+
 // down rows of one item: a 4-wave workgroup per 64 outputs, 16 per wave.
 // Reference: src/cpu/core/routed_expert.cpp:429-447, src/moe_a8_down_contract.cpp:146.
 template <int DEPTH>
@@ -791,7 +842,8 @@ inline void launch_pairs(const PairArgs& a, uint32_t matrices, hipStream_t st) {
 // The dense form needs fp32 gate / up rows as workspace (the optional intermediates views) because a wavefront holds
 // 16 rows, not a whole 32-output SwiGLU group.
 inline bool dense_pairs_ok(const mi355_moe_weights& w, uint32_t rows) {
-    return w.experts == 1U && w.top_k == 1U && rows <= 8U && (w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0 &&
+    return w.gate_type == MI355_TYPE_Q4_K && w.down_type == MI355_TYPE_Q4_K &&
+           w.experts == 1U && w.top_k == 1U && rows <= 8U && (w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0 &&
            w.gate_row_stride < (1ULL << 24) && w.down_row_stride < (1ULL << 24);
 }
 inline void launch_project_dense(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, hipStream_t st) {
@@ -820,6 +872,10 @@ inline void launch_plan(const uint32_t* routes, uint32_t experts, uint32_t assig
     if (large) plan_order_kernel<<<experts, 1024, 0, st>>>(routes, experts, assignments, plan);
 }
 inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+    if (w.gate_type == MI355_TYPE_Q5_K) {
+        project_q5k_kernel<<<dim3(w.ffn / 32U, umax), 256, 0, st>>>(w, r, rows * w.top_k);
+        return;
+    }
     if (dense_pairs_ok(w, rows) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
     const dim3 grid(w.ffn / 32U, umax);
     if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
@@ -860,19 +916,20 @@ inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
 inline uint64_t moe_row_bytes(uint32_t type, uint32_t k) {
     if (type == MI355_TYPE_Q8_0) return static_cast<uint64_t>(k / 32U) * kQ80Block;
     if (type == MI355_TYPE_Q5_1) return static_cast<uint64_t>(k / 32U) * 24U;
+    if (type == MI355_TYPE_Q5_K) return static_cast<uint64_t>(k / 256U) * kQ5kBlock;
     return static_cast<uint64_t>(k / 256U) * kQ4kBlock;
 }
 
-// Tensor formats by arithmetic class. Integer-dot entries: Q4_K gate/up; down Q4_K, or the host executor's Q8_0 / Q5_1
-// (src/cpu/core/routed_expert.hpp:28). The matrix-core prefill form: Q4_K or Q8_0 for either (a dense shared expert is
+// Tensor formats by arithmetic class. Integer-dot entries: gate/up Q4_K or Q5_K; down Q4_K, or the host executor's Q8_0 /
+// Q5_1 (src/cpu/core/routed_expert.hpp:27-28). The matrix-core prefill form: Q4_K or Q8_0 for either (a dense shared expert is
 // experts = top_k = 1). The merge reads no weights.
 enum MoeClass { kIntegerClass, kPrefillClass, kAnyClass };
 int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, MoeClass cls = kIntegerClass) {
     STRIX_REQUIRE(w && r, "moe: null weights or rows");
     STRIX_REQUIRE(rows > 0, "moe: rows must be positive");
     const bool gate_q8 = w->gate_type == MI355_TYPE_Q8_0, down_q8 = w->down_type == MI355_TYPE_Q8_0, down_q51 = w->down_type == MI355_TYPE_Q5_1;
-    STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || (gate_q8 && cls != kIntegerClass),
-                  cls == kIntegerClass ? "moe: gate/up weights must be Q4_K (type 12)" : "moe prefill: gate/up weights must be Q4_K (type 12) or Q8_0 (type 8)");
+    STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || (gate_q8 && cls != kIntegerClass) || (w->gate_type == MI355_TYPE_Q5_K && cls != kPrefillClass),
+                  cls == kPrefillClass ? "moe prefill: gate/up weights must be Q4_K (type 12) or Q8_0 (type 8)" : "moe: gate/up weights must be Q4_K (type 12) or Q5_K (type 13)");
     if (!(w->down_type == MI355_TYPE_Q4_K || down_q8 || (down_q51 && cls != kPrefillClass)))
         return fail(MI355_E_UNSUPPORTED, cls == kPrefillClass ? "moe prefill: down weights must be Q4_K (type 12) or Q8_0 (type 8)"
                                                                : "moe: down weights must be Q4_K (type 12), Q8_0 (type 8) or Q5_1 (type 7)");
@@ -1144,11 +1201,13 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     const uint32_t quad_max = quad_items > 0 ? static_cast<uint32_t>(quad_items) : kQuadMaxItems;
     if (items <= quad_max && wv.experts > 1U) {
         if (items <= 16U) {
-            project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+            if (wv.gate_type != MI355_TYPE_Q4_K) launch_project(wv, *r, rows, items, hs(stream));
+            else project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
             if (wv.down_type != MI355_TYPE_Q4_K) launch_down(wv, *r, rows, items, hs(stream));
             else down_quad_kernel<4><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
         } else {
-            project_quad_kernel<2><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
+            if (wv.gate_type != MI355_TYPE_Q4_K) launch_project(wv, *r, rows, items, hs(stream));
+            else project_quad_kernel<2><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
             if (wv.down_type != MI355_TYPE_Q4_K) launch_down(wv, *r, rows, items, hs(stream));
             else down_quad_kernel<2><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
         }

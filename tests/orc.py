@@ -9,8 +9,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 
-Q5_1, Q8_0, Q4_K = 7, 8, 12
-Q5_1_BLOCK, Q8_0_BLOCK, Q4_K_BLOCK = 24, 34, 144
+Q5_1, Q8_0, Q4_K, Q5_K = 7, 8, 12, 13
+Q5_1_BLOCK, Q8_0_BLOCK, Q4_K_BLOCK, Q5_K_BLOCK = 24, 34, 144, 176
 EXP_GFX1151, EXP_DECLARED = 0, 1
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
 COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
@@ -103,6 +103,7 @@ def _declare(L):
     L.orc_float_to_half.argtypes = [C.c_float]
     L.orc_q4k_factor_words.restype = C.c_uint
     L.orc_q4k_row_a8.restype = C.c_float
+    L.orc_q5k_row_a8.restype = C.c_float
     L.orc_q4k_row_a8_contract_form.restype = C.c_float
     L.orc_q8_0_down_row_a8.restype = C.c_float
     L.orc_q5_1_down_row_a8.restype = C.c_float
@@ -118,6 +119,8 @@ def _declare(L):
 def row_bytes(qtype, elements):
     if qtype == Q5_1:
         return elements // 32 * Q5_1_BLOCK
+    if qtype == Q5_K:
+        return elements // 256 * Q5_K_BLOCK
     return elements // 32 * Q8_0_BLOCK if qtype == Q8_0 else elements // 256 * Q4_K_BLOCK
 
 
@@ -191,6 +194,40 @@ def q5_1_down_row_a8(wrow, codes, deltas, sums):
     wrow = np.ascontiguousarray(wrow, np.uint8)
     return np.float32(lib().orc_q5_1_down_row_a8(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q5_1_BLOCK), _ptr(codes, i8p),
                                                  _ptr(deltas, f32p), _ptr(sums, i32p)))
+
+
+def q5k_row_a8(wrow, codes, deltas, sums):
+    wrow = np.ascontiguousarray(wrow, np.uint8)
+    return np.float32(lib().orc_q5k_row_a8(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q5_K_BLOCK), _ptr(codes, i8p), _ptr(deltas, f32p),
+                                           _ptr(sums, i32p)))
+
+
+def random_q5_k(rng, shape_rows, width):
+    """Q5_K rows of random bytes (factors, fifth bits, nibbles) with positive fp16 d and dmin around 2^-11."""
+    w = rng.integers(0, 256, tuple(shape_rows) + (width // 256 * Q5_K_BLOCK,), dtype=np.uint8)
+    w[..., 1::Q5_K_BLOCK] = (w[..., 1::Q5_K_BLOCK] & 0x03) | 0x10
+    w[..., 3::Q5_K_BLOCK] = (w[..., 3::Q5_K_BLOCK] & 0x03) | 0x10
+    return w
+
+
+def dequant_q5_k_rows(raw, width):
+    """ggml Q5_K: x = d * sc_j * q - dmin * m_j, q = nibble | fifth bit << 4 (layout of src/cpu/core/routed_expert.cpp:73-108;
+    factors as in Q4_K, src/cpu/core/routed_expert.cpp:65-71)."""
+    raw = np.ascontiguousarray(raw, np.uint8).reshape(-1, width // 256, Q5_K_BLOCK)
+    d = raw[..., 0:2].copy().view(np.float16).astype(np.float32)[..., 0]
+    dm = raw[..., 2:4].copy().view(np.float16).astype(np.float32)[..., 0]
+    sc_bytes = raw[..., 4:16].astype(np.uint32)
+    out = np.zeros(raw.shape[:2] + (256,), np.float32)
+    for j in range(8):
+        if j < 4:
+            sc, mn = sc_bytes[..., j] & 63, sc_bytes[..., 4 + j] & 63
+        else:
+            sc = (sc_bytes[..., 4 + j] & 15) | ((sc_bytes[..., j - 4] >> 6) << 4)
+            mn = (sc_bytes[..., 4 + j] >> 4) | ((sc_bytes[..., j] >> 6) << 4)
+        byte = raw[..., 48 + 32 * (j // 2): 48 + 32 * (j // 2) + 32].astype(np.uint32)
+        q = ((byte >> 4) if j & 1 else (byte & 15)) | (((raw[..., 16:48].astype(np.uint32) >> j) & 1) << 4)
+        out[..., 32 * j: 32 * j + 32] = (d * sc.astype(np.float32))[..., None] * q.astype(np.float32) - (dm * mn.astype(np.float32))[..., None]
+    return out.reshape(raw.shape[0], width)
 
 
 def random_q5_1(rng, shape_rows, width):
@@ -268,18 +305,18 @@ class ExpertResult:
 
 def routed_experts(hidden, ffn, top_k, gate, up, down, down_type, codes, deltas, sums, ids, exp_kind=EXP_GFX1151,
                    gate_expert_stride=None, gate_row_stride=None, down_expert_stride=None, down_row_stride=None,
-                   threads=0, want_intermediates=True, down_only_from=None):
+                   threads=0, want_intermediates=True, down_only_from=None, gate_type=Q4_K):
     """gate/up/down: uint8 arrays holding every expert (GGUF order unless strides are given).
     down_only_from: (h_codes, h_deltas, h_sums) -> run the down phase alone on that image."""
     gate = np.ascontiguousarray(gate, np.uint8)
     up = np.ascontiguousarray(up, np.uint8)
     down = np.ascontiguousarray(down, np.uint8)
     rows = codes.shape[0]
-    grb = gate_row_stride or hidden // 256 * Q4_K_BLOCK
+    grb = gate_row_stride or row_bytes(gate_type, hidden)
     geb = gate_expert_stride or grb * ffn
     drb = down_row_stride or row_bytes(down_type, ffn)
     deb = down_expert_stride or drb * hidden
-    w = ExpertWeights(hidden, ffn, 0, top_k, Q4_K, down_type, gate.ctypes.data, up.ctypes.data, down.ctypes.data,
+    w = ExpertWeights(hidden, ffn, 0, top_k, gate_type, down_type, gate.ctypes.data, up.ctypes.data, down.ctypes.data,
                       geb, grb, deb, drb, exp_kind)
     ids = np.ascontiguousarray(ids, np.uint32)
     n = rows * top_k

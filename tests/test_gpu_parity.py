@@ -384,25 +384,37 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
 
 
 # ------------------------------------------------------------------------------------------- the host executor's down formats
-@pytest.mark.parametrize("down_type,H,I,E,K,T,entry", [
-    (orc.Q8_0, 512, 256, 6, 3, 5, "staged"),          # the shape of the compiled reference's own whole-job check
-    (orc.Q5_1, 512, 256, 6, 3, 5, "staged"),
-    (orc.Q8_0, 2048, 768, 128, 8, 8, "layer"),        # config 3's layer with the executor's down format
-    (orc.Q5_1, 2048, 768, 128, 8, 1, "layer"),
-    (orc.Q5_1, 1024, 1280, 16, 4, 40, "staged"),      # plan items of up to four assignments
-    (orc.Q8_0, 768, 512, 5, 2, 23, "layer")])
-def test_down_rows_in_the_host_executor_formats(strix, down_type, H, I, E, K, T, entry):
-    """Q4_K gate/up with Q8_0 or Q5_1 down: the formats of the reference's host executor (src/cpu/core/routed_expert.hpp:28).
+@pytest.mark.parametrize("gate_type,down_type,H,I,E,K,T,entry", [
+    (orc.Q4_K, orc.Q8_0, 512, 256, 6, 3, 5, "staged"),          # the shape of the compiled reference's own whole-job check
+    (orc.Q4_K, orc.Q5_1, 512, 256, 6, 3, 5, "staged"),
+    (orc.Q5_K, orc.Q8_0, 512, 256, 6, 3, 5, "staged"),
+    (orc.Q4_K, orc.Q8_0, 2048, 768, 128, 8, 8, "layer"),        # config 3's layer with the executor's down format
+    (orc.Q4_K, orc.Q5_1, 2048, 768, 128, 8, 1, "layer"),
+    (orc.Q5_K, orc.Q5_1, 2048, 768, 128, 8, 8, "layer"),
+    (orc.Q5_K, orc.Q4_K, 2048, 768, 128, 8, 2, "layer"),        # Q5_K gate/up in front of Q4_K down rows
+    (orc.Q4_K, orc.Q5_1, 1024, 1280, 16, 4, 40, "staged"),      # plan items of up to four assignments
+    (orc.Q5_K, orc.Q8_0, 1024, 1280, 16, 4, 40, "staged"),
+    (orc.Q5_K, orc.Q8_0, 768, 512, 1, 1, 6, "staged"),          # a dense layer: the plan is still built
+    (orc.Q4_K, orc.Q8_0, 768, 512, 5, 2, 23, "layer")])
+def test_down_rows_in_the_host_executor_formats(strix, gate_type, down_type, H, I, E, K, T, entry):
+    """The formats of the reference's host executor (src/cpu/core/routed_expert.hpp:27-28): gate/up Q4_K or Q5_K, down Q8_0 or Q5_1.
     Device rawdots == the oracle's down rows on the device's own h image, bit for bit; the combine likewise; and, when the
     compiled reference is present and the device's h codes equal the oracle's, == reference_run's rawdots bit for bit."""
     import ctypes as C
-    rng = np.random.default_rng(3 * H + T + down_type)
-    gate, up, _ = make_layer(rng, H, I, E)
-    down = orc.random_q5_1(rng, (E, H), I) if down_type == orc.Q5_1 else orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32))
+    rng = np.random.default_rng(3 * H + T + down_type + gate_type)
+    gate, up, down4 = make_layer(rng, H, I, E)
+    if gate_type == orc.Q5_K:
+        gate, up = orc.random_q5_k(rng, (E, I), H), orc.random_q5_k(rng, (E, I), H)
+    if down_type == orc.Q5_1:
+        down = orc.random_q5_1(rng, (E, H), I)
+    elif down_type == orc.Q8_0:
+        down = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32))
+    else:
+        down = down4
     x = rng.standard_normal((T, H)).astype(np.float16)
     wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
     ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
-    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, intermediates=True, down_type=down_type)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, intermediates=True, gate_type=gate_type, down_type=down_type)
     if entry == "layer":
         y, ids, wts, _ = layer.run_layer(dev(x), dev(wr))
         assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
@@ -411,10 +423,13 @@ def test_down_rows_in_the_host_executor_formats(strix, down_type, H, I, E, K, T,
         y = layer.run(dev(x), dev(ids_ref.astype(np.int32)), dev(w_ref)).cpu().numpy()
     n = T * K
     c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
-    ref = orc.routed_experts(H, I, K, gate, up, down, down_type, c, d, s, ids_ref)
+    ref = orc.routed_experts(H, I, K, gate, up, down, down_type, c, d, s, ids_ref, gate_type=gate_type)
     assert np.array_equal(bits(layer.gate_out[:n].cpu().numpy()), bits(ref.gate))
+    assert np.array_equal(bits(layer.up_out[:n].cpu().numpy()), bits(ref.up))
     dc, dd_, ds = layer.down_codes[:n].cpu().numpy(), layer.down_deltas[:n].cpu().numpy(), layer.down_sums[:n].cpu().numpy()
-    ref_down = orc.routed_experts(H, I, K, gate, up, down, down_type, c, d, s, ids_ref, down_only_from=(dc, dd_, ds))
+    hc, hd, hs, _ = orc.quantize_a8(layer.h_out[:n].cpu().numpy(), tiny_rule=True)
+    assert np.array_equal(dc, hc) and np.array_equal(bits(dd_), bits(hd)) and np.array_equal(ds, hs)
+    ref_down = orc.routed_experts(H, I, K, gate, up, down, down_type, c, d, s, ids_ref, down_only_from=(dc, dd_, ds), gate_type=gate_type)
     raw_dev = layer.rawdots[:T].cpu().numpy()
     assert np.array_equal(bits(raw_dev), bits(ref_down.rawdots))
     assert np.array_equal(bits(y), bits(orc.combine(0, w_ref, ids_ref, raw_dev)))
@@ -422,12 +437,12 @@ def test_down_rows_in_the_host_executor_formats(strix, down_type, H, I, E, K, T,
     a, e = rel_err(y, orc.combine(0, w_ref, ids_ref, ref.rawdots))
     assert a < TOL_F16 and e < TOL_F16, (a, e)
     R = orc.ref()
-    if R is not None and np.array_equal(dc, ref.h_codes) and np.array_equal(bits(dd_), bits(ref.h_deltas)):
+    if R is not None and down_type != orc.Q4_K and np.array_equal(dc, ref.h_codes) and np.array_equal(bits(dd_), bits(ref.h_deltas)):
         asg = np.array([[t, k, ids_ref[t, k]] for t in range(T) for k in range(K)], np.uint32)
         raw = np.zeros((T, K, H), np.float32)
         status = np.zeros(T, np.uint32)
         rc = R.ref_routed_expert_run_fmt(H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down.ctypes.data_as(orc.u8p),
-                                         int(down_type == orc.Q5_1), c.ctypes.data_as(orc.i8p), d.ctypes.data_as(orc.f32p),
+                                         int(down_type == orc.Q5_1) + 2 * int(gate_type == orc.Q5_K), c.ctypes.data_as(orc.i8p), d.ctypes.data_as(orc.f32p),
                                          s.ctypes.data_as(orc.i32p), T, asg.ctypes.data_as(orc.u32p), n, raw.ctypes.data_as(orc.f32p),
                                          C.c_uint64(K * H), status.ctypes.data_as(orc.u32p), 0, 0)
         assert rc == 0, R.ref_last_error()
@@ -496,7 +511,7 @@ def test_admission_failures_return_before_any_enqueue(strix):
     x = dev(rng.standard_normal((T, H)).astype(np.float16))
     ids, w = dev(np.zeros((T, K), np.int32)), dev(np.ones((T, K), np.float32))
     layer.output.fill_(5.0)
-    for field, value in (("hidden", 500), ("ffn", 100), ("top_k", 17), ("gate_type", 13), ("gate", 8)):
+    for field, value in (("hidden", 500), ("ffn", 100), ("top_k", 17), ("gate_type", 14), ("gate", 8)):
         saved = getattr(layer.w, field)
         setattr(layer.w, field, value)
         with pytest.raises(strix.StrixError) as err:

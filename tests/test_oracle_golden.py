@@ -570,6 +570,23 @@ def test_routed_experts_against_double_precision_dequant_reference(down_type):
     assert np.array_equal(bits(r1.rawdots), bits(r.rawdots)) and np.array_equal(r1.h_codes, r.h_codes)
 
 
+def test_q5k_gate_rows_against_double_precision_dequant_reference():
+    """Brute force for the Q5_K gate/up row: dequantise with a numpy statement of the block layout, sum in double."""
+    rng = np.random.default_rng(15)
+    H = 768
+    w = orc.random_q5_k(rng, (40,), H)
+    x = rng.standard_normal((3, H)).astype(np.float32)
+    codes, deltas, sums, _ = orc.quantize_a8(x)
+    xa = codes.astype(np.float64) * np.repeat(deltas.astype(np.float64), 32, axis=1)
+    want = xa @ orc.dequant_q5_k_rows(w, H).astype(np.float64).T
+    got = np.array([[orc.q5k_row_a8(w[o], codes[t], deltas[t], sums[t]) for o in range(40)] for t in range(3)])
+    assert np.max(np.abs(got - want)) < 2e-5 * np.abs(want).max()
+    # the fifth bits matter: clearing them changes every row
+    w4 = w.copy().reshape(40, -1, 176)
+    w4[..., 16:48] = 0
+    assert np.all(np.array([orc.q5k_row_a8(w4[o].reshape(-1), codes[0], deltas[0], sums[0]) for o in range(40)]) != got[0])
+
+
 def test_routed_experts_nonfinite_row_sets_status_and_skips_down():
     rng = np.random.default_rng(14)
     H, I, E, T, K = 256, 128, 3, 2, 2
@@ -688,6 +705,10 @@ def test_ref_q4k_row_and_down_row_bits_at_config_widths():
         R.ref_down_row_q8_0(w8.ctypes.data_as(orc.u8p), width // 32, codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
                             sums[0].ctypes.data_as(orc.i32p), C.byref(out))
         assert bits(orc.q8_0_down_row_a8(w8, codes[0], deltas[0])) == bits(np.float32(out.value))
+        wk = orc.random_q5_k(rng, (1,), width)[0]
+        R.ref_gate_row_q5k(wk.ctypes.data_as(orc.u8p), width // 256, codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
+                           sums[0].ctypes.data_as(orc.i32p), C.byref(out))
+        assert bits(orc.q5k_row_a8(wk, codes[0], deltas[0], sums[0])) == bits(np.float32(out.value))
         w5 = orc.random_q5_1(rng, (1,), width)[0]
         R.ref_down_row_q5_1(w5.ctypes.data_as(orc.u8p), width // 32, codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
                             sums[0].ctypes.data_as(orc.i32p), C.byref(out))
@@ -737,6 +758,19 @@ def test_ref_whole_routed_expert_job_bits():
                                          status.ctypes.data_as(orc.u32p), threads, simd)
         assert rc == 0, R.ref_last_error()
         assert np.array_equal(bits(raw), bits(mine5.rawdots)) and np.all(status == 0)
+    # the executor's other gate/up format: Q5_K (random blocks), with either down format
+    gate5, up5 = orc.random_q5_k(rng, (E, I), H), orc.random_q5_k(rng, (E, I), H)
+    for down_t, down_w, flags in ((orc.Q8_0, down, 2), (orc.Q5_1, down5, 3)):
+        mine_k = orc.routed_experts(H, I, K, gate5, up5, down_w, down_t, codes, deltas, sums, ids, gate_type=orc.Q5_K)
+        for threads, simd in ((0, 0), (3, 1)):
+            raw = np.zeros((T, K, H), np.float32)
+            status = np.zeros(T, np.uint32)
+            rc = R.ref_routed_expert_run_fmt(H, I, gate5.ctypes.data_as(orc.u8p), up5.ctypes.data_as(orc.u8p), down_w.ctypes.data_as(orc.u8p), flags,
+                                             codes.ctypes.data_as(orc.i8p), deltas.ctypes.data_as(orc.f32p), sums.ctypes.data_as(orc.i32p), T,
+                                             asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
+                                             status.ctypes.data_as(orc.u32p), threads, simd)
+            assert rc == 0, R.ref_last_error()
+            assert np.array_equal(bits(raw), bits(mine_k.rawdots)) and np.all(status == 0)
 
 
 @needs_ref
