@@ -45,7 +45,7 @@ enum {
     MI355_STATUS_AGGREGATE = 16              /* merged output failed the commit threshold */
 };
 
-enum { MI355_TYPE_Q5_1 = 7, MI355_TYPE_Q8_0 = 8, MI355_TYPE_Q4_K = 12, MI355_TYPE_Q5_K = 13 };              /* ggml tensor type ids */
+enum { MI355_TYPE_Q5_1 = 7, MI355_TYPE_Q8_0 = 8, MI355_TYPE_Q4_K = 12, MI355_TYPE_Q5_K = 13, MI355_TYPE_Q6_K = 14 };              /* ggml tensor type ids */
 enum { MI355_INPUT_F32 = 0, MI355_INPUT_F16 = 1, MI355_INPUT_BF16 = 2 };
 enum { MI355_LOGITS_FMA_ASCENDING = 0, MI355_LOGITS_LANE32_BUTTERFLY = 1 };
 enum { MI355_COMBINE_FMA_SLOT_ORDER = 0, MI355_COMBINE_MULADD_ASCENDING_EXPERT = 1 };
@@ -124,17 +124,18 @@ int32_t mi355_moe_route(const mi355_route_policy* policy, const void* x, uint32_
  * (include/strix/cuda/qwen_moe.hpp:55-110: Rows / Weights, enqueue_prologue / csr / project / down / merge) and
  * computes what strix::cpu::expert::reference_run computes (src/cpu/core/routed_expert.cpp:264-300) with Q4_K or Q5_K gate/up
  * and Q4_K down (down rows by the gate/up row contract: src/moe_a8_down_contract.cpp:146) or the host executor's own down
- * formats, Q8_0 and Q5_1 blocks of 32 (src/cpu/core/routed_expert.hpp:28, routed_expert.cpp:110-144). The single-row C1 forms of
+ * formats, Q8_0 and Q5_1 blocks of 32 (src/cpu/core/routed_expert.hpp:28, routed_expert.cpp:110-144), or Q6_K down rows
+ * (src/moe_a8_down_contract.cpp:18-37, 147-158). The single-row C1 forms of
  * include/strix/hip_moe_q4k_a8_probe.hpp:12 and include/strix/hip_moe_a8_down.hpp:11-30 are rows = 1.
  */
 typedef struct mi355_moe_weights {
     uint32_t hidden;      /* multiple of 256 */
     uint32_t ffn;         /* intermediate rows computed by this call (a TP rank: its share), multiple of 256 */
     uint32_t experts, top_k;
-    uint32_t gate_type, down_type;                    /* gate/up MI355_TYPE_Q4_K or Q5_K; down Q4_K, Q8_0 or Q5_1
+    uint32_t gate_type, down_type;                    /* gate/up MI355_TYPE_Q4_K or Q5_K; down Q4_K, Q8_0, Q5_1 or Q6_K
                                                          (mi355_moe_enqueue_prefill_f16: Q4_K or Q8_0 for either) */
     const uint8_t *gate, *up, *down;                  /* GGUF order [experts][ffn][hidden/256], [experts][hidden][ffn/256 or ffn/32 blocks] */
-    uint64_t gate_expert_stride, gate_row_stride;     /* bytes; 0 = dense GGUF order. 16-byte multiples */
+    uint64_t gate_expert_stride, gate_row_stride;     /* bytes; 0 = dense GGUF order. 16-byte multiples (Q6_K down: 2) */
     uint64_t down_expert_stride, down_row_stride;     /* a TP rank reads the first ffn/256 blocks of each down row */
     uint32_t exp_kind;                                /* MI355_EXP_* used by SiLU */
 } mi355_moe_weights;

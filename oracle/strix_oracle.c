@@ -352,6 +352,35 @@ float orc_q5_1_down_row_a8(const uint8_t* wrow, uint32_t groups, const int8_t* c
     return s01 + s23;
 }
 
+/* src/moe_a8_down_contract.cpp:18-37 (group term) and :147-158 (row): 210-byte blocks = 128 nibble bytes, 64 bytes of bit
+ * pairs, 16 signed scales (one per 16 weights), fp16 d. */
+float orc_q6k_down_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas) {
+    float accum[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+    for (uint32_t block = 0; block < blocks; ++block) {
+        const uint8_t* b = wrow + (size_t)block * ORC_Q6_K_BLOCK;
+        const float d = orc_half_to_float(le16(b + 208));
+        for (uint32_t pair = 0; pair < 4; ++pair) {
+            float c[2];
+            for (uint32_t k = 0; k < 2; ++k) {
+                const uint32_t g = block * 8 + pair * 2 + k, j = g % 8, half = j / 4, quarter = j % 4;
+                int64_t part[2] = {0, 0};
+                for (uint32_t i = 0; i < 32; ++i) {
+                    const uint32_t low = (b[half * 64 + (quarter & 1) * 32 + i] >> (quarter >= 2 ? 4 : 0)) & 15U;
+                    const uint32_t high = (b[128 + half * 32 + i] >> (2 * quarter)) & 3U;
+                    part[i / 16] += (int64_t)codes[g * 32 + i] * ((int)(low | (high << 4)) - 32);
+                }
+                const int64_t s0 = (int8_t)b[192 + 2 * j], s1 = (int8_t)b[193 + 2 * j];
+                const int64_t integer = s0 * part[0] + s1 * part[1];
+                c[k] = deltas[g] * (d * (float)integer);
+            }
+            const float paired = c[0] + c[1];
+            accum[pair] = accum[pair] + paired;
+        }
+    }
+    const float left = accum[0] + accum[1], right = accum[2] + accum[3];
+    return left + right;
+}
+
 /* ------------------------------------------------------------------ exp / SwiGLU */
 /* src/cpu/core/routed_expert.cpp:248-261 with v_exp = float(exp2(double(a))) (:212-216; the probe-table
  * corrections of :217-226 need tables that are not in the reference tree, so none apply here). */
@@ -522,6 +551,7 @@ void orc_routed_down(const orc_expert_weights* w, const orc_expert_job* job, int
             float value;
             if (w->down_type == ORC_Q4_K) value = orc_q4k_row_a8(wrow, ffn / 256, c, d, s);   /* src/moe_a8_down_contract.cpp:146 */
             else if (w->down_type == ORC_Q5_1) value = orc_q5_1_down_row_a8(wrow, groups, c, d, s);
+            else if (w->down_type == ORC_Q6_K) value = orc_q6k_down_row_a8(wrow, ffn / 256, c, d);
             else value = orc_q8_0_down_row_a8(wrow, groups, c, d);
             job->rawdots[(size_t)a * hidden + o] = value;
         }

@@ -12,7 +12,7 @@
  *
  * Pinning status (what checks each function besides this text):
  *   half/Q8_0/Q4_K decode, scale/min unpack, Q8_0 writer, A8 quantiser, Q8_0xA8 product order,
- *   Q4_KxA8 and Q5_KxA8 rows, Q8_0 and Q5_1 down rows, router selection/weights, combine: pinned by the literal vectors and
+ *   Q4_KxA8 and Q5_KxA8 rows, Q8_0, Q5_1 and Q6_K down rows, router selection/weights, combine: pinned by the literal vectors and
  *   invariants of the reference's own tests (tests/golden/) and, where it builds, bitwise against the
  *   compiled reference (oracle/_ref).
  *   orc_expf_gfx1151: pinned only against the reference function run with EMPTY correction tables;
@@ -35,8 +35,8 @@
 extern "C" {
 #endif
 
-enum { ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13 };          /* ggml type ids */
-enum { ORC_Q5_1_BLOCK = 24, ORC_Q8_0_BLOCK = 34, ORC_Q4_K_BLOCK = 144, ORC_Q5_K_BLOCK = 176 };
+enum { ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };          /* ggml type ids */
+enum { ORC_Q5_1_BLOCK = 24, ORC_Q8_0_BLOCK = 34, ORC_Q4_K_BLOCK = 144, ORC_Q5_K_BLOCK = 176, ORC_Q6_K_BLOCK = 210 };
 enum { ORC_STATUS_INVALID_ROUTE = 1, ORC_STATUS_NONFINITE_ACTIVATION = 2, ORC_STATUS_INVALID_DELTA = 4,
        ORC_STATUS_NONFINITE_PROJECTION = 8 };
 enum { ORC_EXP_GFX1151_NOTABLE = 0, ORC_EXP_DECLARED = 1 };
@@ -86,6 +86,7 @@ float orc_q4k_row_a8_contract_form(const uint8_t* wrow, uint32_t blocks, const i
                                    const float* deltas, const int32_t* sums);
 /* Q8_0 down row, groups mod 4 (src/cpu/core/routed_expert.cpp:110-144 with Q51 = false). */
 float orc_q8_0_down_row_a8(const uint8_t* wrow, uint32_t groups, const int8_t* codes, const float* deltas);
+float orc_q6k_down_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas);
 float orc_q5_1_down_row_a8(const uint8_t* wrow, uint32_t groups, const int8_t* codes, const float* deltas, const int32_t* sums);
 
 /* ---- exp / SwiGLU ---------------------------------------------------------------------------- */
@@ -122,7 +123,7 @@ void orc_combine(int form, uint32_t rows, uint32_t top_k, uint32_t width, const 
 /* ---- routed expert layer (src/cpu/core/routed_expert.cpp:264-300 generalised to Q4_K / Q8_0 down) - */
 typedef struct {
     uint32_t hidden, ffn, experts, top_k;   /* ffn = intermediate rows computed here (rank-local for a TP shard) */
-    uint32_t gate_type, down_type;          /* ORC_Q4_K or ORC_Q5_K gate/up; ORC_Q4_K, ORC_Q8_0 or ORC_Q5_1 down */
+    uint32_t gate_type, down_type;          /* ORC_Q4_K or ORC_Q5_K gate/up; ORC_Q4_K, ORC_Q8_0, ORC_Q5_1 or ORC_Q6_K down */
     const uint8_t *gate, *up, *down;
     uint64_t gate_expert_stride, gate_row_stride;   /* bytes */
     uint64_t down_expert_stride, down_row_stride;   /* bytes; a rank reads the first ffn/blk blocks of each row */

@@ -10,7 +10,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmi355_strix.so")
 
-TYPE_Q5_1, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q5_K = 7, 8, 12, 13
+TYPE_Q5_1, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K = 7, 8, 12, 13, 14
 INPUT_F32, INPUT_F16, INPUT_BF16 = 0, 1, 2
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
 COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1

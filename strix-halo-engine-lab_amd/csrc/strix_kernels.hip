@@ -16,6 +16,7 @@
 #include "q4k_quads.hpp"
 #include "down_groups.hpp"
 #include "q5k_quads.hpp"
+#include "q6k_quads.hpp"
 #include "prefill_f16.hpp"
 #include "route_wave.hpp"
 
@@ -882,11 +883,12 @@ inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, 
     else launch_project_nb<4>(w, r, rows, grid, st);
 }
 inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
-    if (w.down_type != MI355_TYPE_Q4_K) {      // the host executor's formats: blocks of 32, four chains per row
+    if (w.down_type != MI355_TYPE_Q4_K) {      // Q8_0 / Q5_1 (blocks of 32, four chains per row) and Q6_K (pairs per super-block)
         const uint32_t assignments = rows * w.top_k, items_at = plan_items_at(w.experts, assignments), order_at = plan_order_at(w.experts);
         const dim3 grid(w.hidden / kDownGroupsRows, umax);
         if (w.down_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
-        else down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+        else if (w.down_type == MI355_TYPE_Q5_1) down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+        else down_q6k_kernel<<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         return;
     }
     if (dense_pairs_ok(w, rows)) return launch_down_dense(w, r, rows, st);
@@ -917,22 +919,24 @@ inline uint64_t moe_row_bytes(uint32_t type, uint32_t k) {
     if (type == MI355_TYPE_Q8_0) return static_cast<uint64_t>(k / 32U) * kQ80Block;
     if (type == MI355_TYPE_Q5_1) return static_cast<uint64_t>(k / 32U) * 24U;
     if (type == MI355_TYPE_Q5_K) return static_cast<uint64_t>(k / 256U) * kQ5kBlock;
+    if (type == MI355_TYPE_Q6_K) return static_cast<uint64_t>(k / 256U) * kQ6kBlock;
     return static_cast<uint64_t>(k / 256U) * kQ4kBlock;
 }
 
-// Tensor formats by arithmetic class. Integer-dot entries: gate/up Q4_K or Q5_K; down Q4_K, or the host executor's Q8_0 /
-// Q5_1 (src/cpu/core/routed_expert.hpp:27-28). The matrix-core prefill form: Q4_K or Q8_0 for either (a dense shared expert is
+// Tensor formats by arithmetic class. Integer-dot entries: gate/up Q4_K or Q5_K; down Q4_K, the host executor's Q8_0 /
+// Q5_1 (src/cpu/core/routed_expert.hpp:27-28) or Q6_K (src/moe_a8_down_contract.cpp:147). The matrix-core prefill form: Q4_K or Q8_0 for either (a dense shared expert is
 // experts = top_k = 1). The merge reads no weights.
 enum MoeClass { kIntegerClass, kPrefillClass, kAnyClass };
 int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, MoeClass cls = kIntegerClass) {
     STRIX_REQUIRE(w && r, "moe: null weights or rows");
     STRIX_REQUIRE(rows > 0, "moe: rows must be positive");
-    const bool gate_q8 = w->gate_type == MI355_TYPE_Q8_0, down_q8 = w->down_type == MI355_TYPE_Q8_0, down_q51 = w->down_type == MI355_TYPE_Q5_1;
+    const bool gate_q8 = w->gate_type == MI355_TYPE_Q8_0, down_q8 = w->down_type == MI355_TYPE_Q8_0;
+    const bool down_q51 = w->down_type == MI355_TYPE_Q5_1 || w->down_type == MI355_TYPE_Q6_K;      // integer class only
     STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || (gate_q8 && cls != kIntegerClass) || (w->gate_type == MI355_TYPE_Q5_K && cls != kPrefillClass),
                   cls == kPrefillClass ? "moe prefill: gate/up weights must be Q4_K (type 12) or Q8_0 (type 8)" : "moe: gate/up weights must be Q4_K (type 12) or Q5_K (type 13)");
     if (!(w->down_type == MI355_TYPE_Q4_K || down_q8 || (down_q51 && cls != kPrefillClass)))
         return fail(MI355_E_UNSUPPORTED, cls == kPrefillClass ? "moe prefill: down weights must be Q4_K (type 12) or Q8_0 (type 8)"
-                                                               : "moe: down weights must be Q4_K (type 12), Q8_0 (type 8) or Q5_1 (type 7)");
+                                                               : "moe: down weights must be Q4_K (type 12), Q8_0 (type 8), Q5_1 (type 7) or Q6_K (type 14)");
     STRIX_REQUIRE(w->hidden >= 256 && w->hidden % 256U == 0, "moe: hidden must be a positive multiple of 256");
     STRIX_REQUIRE(w->ffn >= 256 && w->ffn % 256U == 0, "moe: ffn must be a positive multiple of 256");
     STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
@@ -943,8 +947,9 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
     if (wv.gate_expert_stride == 0) wv.gate_expert_stride = wv.gate_row_stride * w->ffn;
     if (wv.down_row_stride == 0) wv.down_row_stride = moe_row_bytes(w->down_type, w->ffn);
     if (wv.down_expert_stride == 0) wv.down_expert_stride = wv.down_row_stride * w->hidden;
-    STRIX_REQUIRE(wv.gate_row_stride % 16U == 0 && wv.gate_expert_stride % 16U == 0 && wv.down_row_stride % 16U == 0 &&
-                  wv.down_expert_stride % 16U == 0, "moe: weight strides must be multiples of 16 bytes");
+    const uint32_t down_unit = w->down_type == MI355_TYPE_Q6_K ? 2U : 16U;        // Q6_K blocks are 210 bytes
+    STRIX_REQUIRE(wv.gate_row_stride % 16U == 0 && wv.gate_expert_stride % 16U == 0 && wv.down_row_stride % down_unit == 0 &&
+                  wv.down_expert_stride % down_unit == 0, "moe: weight strides must be multiples of 16 bytes (Q6_K down: 2)");
     STRIX_REQUIRE(wv.gate_row_stride < (1ULL << 27) && wv.down_row_stride < (1ULL << 27), "moe: weight row stride must be below 128 MiB");
     STRIX_REQUIRE(wv.gate_row_stride >= moe_row_bytes(w->gate_type, w->hidden) &&
                   wv.down_row_stride >= moe_row_bytes(w->down_type, w->ffn), "moe: weight row stride shorter than the row");

@@ -9,8 +9,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 
-Q5_1, Q8_0, Q4_K, Q5_K = 7, 8, 12, 13
-Q5_1_BLOCK, Q8_0_BLOCK, Q4_K_BLOCK, Q5_K_BLOCK = 24, 34, 144, 176
+Q5_1, Q8_0, Q4_K, Q5_K, Q6_K = 7, 8, 12, 13, 14
+Q5_1_BLOCK, Q8_0_BLOCK, Q4_K_BLOCK, Q5_K_BLOCK, Q6_K_BLOCK = 24, 34, 144, 176, 210
 EXP_GFX1151, EXP_DECLARED = 0, 1
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
 COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
@@ -104,6 +104,7 @@ def _declare(L):
     L.orc_q4k_factor_words.restype = C.c_uint
     L.orc_q4k_row_a8.restype = C.c_float
     L.orc_q5k_row_a8.restype = C.c_float
+    L.orc_q6k_down_row_a8.restype = C.c_float
     L.orc_q4k_row_a8_contract_form.restype = C.c_float
     L.orc_q8_0_down_row_a8.restype = C.c_float
     L.orc_q5_1_down_row_a8.restype = C.c_float
@@ -121,6 +122,8 @@ def row_bytes(qtype, elements):
         return elements // 32 * Q5_1_BLOCK
     if qtype == Q5_K:
         return elements // 256 * Q5_K_BLOCK
+    if qtype == Q6_K:
+        return elements // 256 * Q6_K_BLOCK
     return elements // 32 * Q8_0_BLOCK if qtype == Q8_0 else elements // 256 * Q4_K_BLOCK
 
 
@@ -227,6 +230,34 @@ def dequant_q5_k_rows(raw, width):
         byte = raw[..., 48 + 32 * (j // 2): 48 + 32 * (j // 2) + 32].astype(np.uint32)
         q = ((byte >> 4) if j & 1 else (byte & 15)) | (((raw[..., 16:48].astype(np.uint32) >> j) & 1) << 4)
         out[..., 32 * j: 32 * j + 32] = (d * sc.astype(np.float32))[..., None] * q.astype(np.float32) - (dm * mn.astype(np.float32))[..., None]
+    return out.reshape(raw.shape[0], width)
+
+
+def q6k_down_row_a8(wrow, codes, deltas):
+    wrow = np.ascontiguousarray(wrow, np.uint8)
+    return np.float32(lib().orc_q6k_down_row_a8(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q6_K_BLOCK), _ptr(codes, i8p), _ptr(deltas, f32p)))
+
+
+def random_q6_k(rng, shape_rows, width):
+    """Q6_K rows of random bytes (nibbles, bit pairs, signed scales) with fp16 d of either sign around 2^-13."""
+    w = rng.integers(0, 256, tuple(shape_rows) + (width // 256 * Q6_K_BLOCK,), dtype=np.uint8)
+    w[..., 209::Q6_K_BLOCK] = (w[..., 209::Q6_K_BLOCK] & 0x83) | 0x08
+    return w
+
+
+def dequant_q6_k_rows(raw, width):
+    """ggml dequantize_row_q6_K: x = d * scale[16-weight group] * (q - 32), element layout of src/moe_a8_down_contract.cpp:20-29."""
+    raw = np.ascontiguousarray(raw, np.uint8).reshape(-1, width // 256, Q6_K_BLOCK)
+    d = raw[..., 208:210].copy().view(np.float16).astype(np.float32)[..., 0]
+    scales = raw[..., 192:208].view(np.int8).astype(np.float32)
+    out = np.zeros(raw.shape[:2] + (256,), np.float32)
+    for j in range(8):
+        half, quarter = j // 4, j % 4
+        ql = raw[..., half * 64 + (quarter & 1) * 32: half * 64 + (quarter & 1) * 32 + 32].astype(np.int32)
+        qh = raw[..., 128 + half * 32: 128 + half * 32 + 32].astype(np.int32)
+        q = (((ql >> (4 if quarter >= 2 else 0)) & 15) | (((qh >> (2 * quarter)) & 3) << 4)) - 32
+        sc = np.repeat(scales[..., 2 * j: 2 * j + 2], 16, axis=-1)
+        out[..., 32 * j: 32 * j + 32] = d[..., None] * sc * q.astype(np.float32)
     return out.reshape(raw.shape[0], width)
 
 

@@ -395,6 +395,9 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
     (orc.Q4_K, orc.Q5_1, 1024, 1280, 16, 4, 40, "staged"),      # plan items of up to four assignments
     (orc.Q5_K, orc.Q8_0, 1024, 1280, 16, 4, 40, "staged"),
     (orc.Q5_K, orc.Q8_0, 768, 512, 1, 1, 6, "staged"),          # a dense layer: the plan is still built
+    (orc.Q4_K, orc.Q6_K, 512, 768, 6, 3, 5, "staged"),          # Q6_K down (src/moe_a8_down_contract.cpp:147): odd block count, 2-byte aligned rows
+    (orc.Q5_K, orc.Q6_K, 2048, 768, 128, 8, 8, "layer"),
+    (orc.Q4_K, orc.Q6_K, 1024, 1280, 16, 4, 40, "staged"),
     (orc.Q4_K, orc.Q8_0, 768, 512, 5, 2, 23, "layer")])
 def test_down_rows_in_the_host_executor_formats(strix, gate_type, down_type, H, I, E, K, T, entry):
     """The formats of the reference's host executor (src/cpu/core/routed_expert.hpp:27-28): gate/up Q4_K or Q5_K, down Q8_0 or Q5_1.
@@ -407,6 +410,8 @@ def test_down_rows_in_the_host_executor_formats(strix, gate_type, down_type, H, 
         gate, up = orc.random_q5_k(rng, (E, I), H), orc.random_q5_k(rng, (E, I), H)
     if down_type == orc.Q5_1:
         down = orc.random_q5_1(rng, (E, H), I)
+    elif down_type == orc.Q6_K:
+        down = orc.random_q6_k(rng, (E, H), I)
     elif down_type == orc.Q8_0:
         down = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32))
     else:
@@ -437,7 +442,7 @@ def test_down_rows_in_the_host_executor_formats(strix, gate_type, down_type, H, 
     a, e = rel_err(y, orc.combine(0, w_ref, ids_ref, ref.rawdots))
     assert a < TOL_F16 and e < TOL_F16, (a, e)
     R = orc.ref()
-    if R is not None and down_type != orc.Q4_K and np.array_equal(dc, ref.h_codes) and np.array_equal(bits(dd_), bits(ref.h_deltas)):
+    if R is not None and down_type in (orc.Q8_0, orc.Q5_1) and np.array_equal(dc, ref.h_codes) and np.array_equal(bits(dd_), bits(ref.h_deltas)):
         asg = np.array([[t, k, ids_ref[t, k]] for t in range(T) for k in range(K)], np.uint32)
         raw = np.zeros((T, K, H), np.float32)
         status = np.zeros(T, np.uint32)
@@ -518,7 +523,7 @@ def test_admission_failures_return_before_any_enqueue(strix):
             layer.run(x, ids, w)
         assert err.value.code == strix.E_INVALID_ARGUMENT
         setattr(layer.w, field, saved)
-    layer.w.down_type = 14
+    layer.w.down_type = 2
     with pytest.raises(strix.StrixError) as err:
         layer.run(x, ids, w)
     assert err.value.code == strix.E_UNSUPPORTED

@@ -587,6 +587,30 @@ def test_q5k_gate_rows_against_double_precision_dequant_reference():
     assert np.all(np.array([orc.q5k_row_a8(w4[o].reshape(-1), codes[0], deltas[0], sums[0]) for o in range(40)]) != got[0])
 
 
+def test_q6k_down_rows_against_the_contract_and_double_precision():
+    """Q6_K down row: bitwise against the compiled reference's contract oracle (evaluate_down_row, type 14) where it is built,
+    and against a float64 sum over a numpy statement of the block layout."""
+    import ctypes as C
+    rng = np.random.default_rng(16)
+    for width in (256, 768, 1280, 1536):                     # the contract oracle admits K-quant rows up to 1536
+        w = orc.random_q6_k(rng, (12,), width)
+        x = (rng.standard_normal((2, width)) * 3.0).astype(np.float32)
+        codes, deltas, sums, _ = orc.quantize_a8(x, tiny_rule=True)
+        got = np.array([[orc.q6k_down_row_a8(w[o], codes[t], deltas[t]) for o in range(12)] for t in range(2)])
+        xa = codes.astype(np.float64) * np.repeat(deltas.astype(np.float64), 32, axis=1)
+        want = xa @ orc.dequant_q6_k_rows(w, width).astype(np.float64).T
+        assert np.max(np.abs(got - want)) < 2e-5 * np.abs(want).max()
+        R = orc.ref()
+        if R is not None:
+            out = C.c_float(0)
+            for t in range(2):
+                for o in range(12):
+                    assert R.ref_evaluate_down_row(w[o].ctypes.data_as(orc.u8p), C.c_size_t(w[o].size), codes[t].ctypes.data_as(orc.i8p),
+                                                   deltas[t].ctypes.data_as(orc.f32p), sums[t].ctypes.data_as(orc.i32p), C.c_size_t(width), 14,
+                                                   C.byref(out)) == 0, R.ref_last_error()
+                    assert bits(np.float32(got[t, o])) == bits(np.float32(out.value))
+
+
 def test_routed_experts_nonfinite_row_sets_status_and_skips_down():
     rng = np.random.default_rng(14)
     H, I, E, T, K = 256, 128, 3, 2, 2
