@@ -145,59 +145,84 @@ def extra_config3_small(strix, torch, cfg, steps, warmup):
     return out
 
 
+def device_blocks(torch, gen, rows, blocks, block_bytes, scale_bytes, high):
+    """Random quantized blocks [rows][blocks * block_bytes] whose fp16 scale fields (high bytes at `scale_bytes`) are small and finite."""
+    w = torch.randint(0, 256, (rows, blocks, block_bytes), dtype=torch.uint8, device="cuda", generator=gen)
+    for at in scale_bytes:
+        w[..., at] = (w[..., at] & 0x03) | high
+    return w.reshape(rows, -1)
+
+
 def extra_config3_executor_formats(strix, torch, cfg, steps, warmup, with_cpu):
-    """Config 3 (T rows) with the down tensors in the reference host executor's own format (Q8_0 blocks of 32): the workload
-    the compiled reference can run itself. GPU: the whole layer; CPU: the reference's Executor (its best ISA, every host
-    thread) on the expert job of layer 0 (A8 rows in, rawdots out: no router, no combine)."""
+    """Config 3 (T rows) with the expert tensors in the other formats of the path: the reference host executor's own
+    (gate/up Q4_K or Q5_K, down Q8_0 or Q5_1), which the compiled reference can run itself, and Q6_K down rows. GPU: the whole
+    layer; CPU: the reference's Executor (its best ISA, every host thread) on the expert job of layer 0 (A8 rows in, rawdots
+    out: no router, no combine)."""
     H, I, E, K, T = cfg.H, cfg.I, cfg.E, cfg.K, cfg.T
     gen = torch.Generator(device="cuda").manual_seed(5)
-    layers = []
-    for layer, wr, x in cfg.layers:
-        w8 = torch.randint(0, 256, (E * H, I // 32, 34), dtype=torch.uint8, device="cuda", generator=gen)
-        w8[..., 1] = (w8[..., 1] & 0x03) | 0x14
-        layers.append((strix.MoeLayer(H, I, E, K, layer.gate, layer.up, w8.reshape(E, H, -1), T, down_type=strix.TYPE_Q8_0), wr, x))
-    n = len(layers)
+    out = {}
+    combos = (("q4_k_gate_q8_0_down", strix.TYPE_Q4_K, strix.TYPE_Q8_0, 0), ("q5_k_gate_q5_1_down", strix.TYPE_Q5_K, strix.TYPE_Q5_1, 3),
+              ("q4_k_gate_q6_k_down", strix.TYPE_Q4_K, strix.TYPE_Q6_K, None))
+    for name, gate_type, down_type, ref_flags in combos:
+        layers = []
+        for layer, wr, x in cfg.layers:
+            if gate_type == strix.TYPE_Q5_K:
+                gate, up = (device_blocks(torch, gen, E * I, H // 256, 176, (1, 3), 0x10).reshape(E, I, -1) for _ in range(2))
+            else:
+                gate, up = layer.gate, layer.up
+            if down_type == strix.TYPE_Q8_0:
+                down = device_blocks(torch, gen, E * H, I // 32, 34, (1,), 0x14)
+            elif down_type == strix.TYPE_Q5_1:
+                down = device_blocks(torch, gen, E * H, I // 32, 24, (1, 3), 0x14)
+            else:
+                down = device_blocks(torch, gen, E * H, I // 256, 210, (209,), 0x08)
+            layers.append((strix.MoeLayer(H, I, E, K, gate, up, down.reshape(E, H, -1), T, gate_type=gate_type, down_type=down_type), wr, x))
+        n = len(layers)
 
-    def step(i):
-        layer, wr, x = layers[i % n]
-        layer.run_layer(x, wr)
-    sec = time_steps(torch, step, max(steps, 60), max(warmup, 12))
-    entry = {"us": sec * 1e6, "down_format": "Q8_0 (34-byte blocks of 32), four chains per row"}
-    if with_cpu:
-        import ctypes as C
-        import orc
-        R = orc.ref()
-        if R is not None:
-            layer, wr, x = layers[0]
-            xn = x.cpu().numpy().astype(np.float32)
-            ids, _, _, _ = orc.route(xn, wr.cpu().numpy(), K)
-            c, d, s, _ = orc.quantize_a8(xn)
-            gate, up, down = (t.cpu().numpy() for t in (layer.gate, layer.up, layer.down))
-            asg = np.array([[t, k, ids[t, k]] for t in range(T) for k in range(K)], np.uint32)
-            raw, status = np.zeros((T, K, H), np.float32), np.zeros(T, np.uint32)
-            threads = orc.lib().orc_max_threads()
-            R.ref_executor_run.restype = C.c_int
-            pool = C.c_void_p(R.ref_executor_create(threads, 1))
+        def step(i):
+            layer, wr, x = layers[i % n]
+            layer.run_layer(x, wr)
+        sec = time_steps(torch, step, max(steps, 60), max(warmup, 12))
+        entry = {"us": sec * 1e6}
+        if int(sum(int(l.status.sum()) for l, _, _ in layers)):
+            raise RuntimeError(f"{name}: a run set row status bits: the timing is void")
+        if with_cpu and ref_flags is not None:
+            import ctypes as C
+            import orc
+            R = orc.ref()
+            if R is not None:
+                layer, wr, x = layers[0]
+                xn = x.cpu().numpy().astype(np.float32)
+                ids, _, _, _ = orc.route(xn, wr.cpu().numpy(), K)
+                c, d, s, _ = orc.quantize_a8(xn)
+                gate, up, down = (t.cpu().numpy() for t in (layer.gate, layer.up, layer.down))
+                asg = np.array([[t, k, ids[t, k]] for t in range(T) for k in range(K)], np.uint32)
+                raw, status = np.zeros((T, K, H), np.float32), np.zeros(T, np.uint32)
+                threads = orc.lib().orc_max_threads()
+                R.ref_executor_run.restype = C.c_int
+                pool = C.c_void_p(R.ref_executor_create(threads, 1))
 
-            def run():
-                return R.ref_executor_run(pool, H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down.ctypes.data_as(orc.u8p), 0,
-                                          c.ctypes.data_as(orc.i8p), d.ctypes.data_as(orc.f32p), s.ctypes.data_as(orc.i32p), T,
-                                          asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
-                                          status.ctypes.data_as(orc.u32p))
-            if run() == 0:
-                times, t_end = [], time.perf_counter() + 5.0
-                while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
-                    t0 = time.perf_counter()
-                    run()
-                    times.append(time.perf_counter() - t0)
-                layer.run_layer(x, wr)
-                torch.cuda.synchronize()
-                entry["cpu_reference"] = {"value": statistics.median(times) * 1e6, "unit": "us/expert job", "cores": threads, "kind": "reference",
-                                          "isa": R.ref_executor_isa(pool).decode(),
-                                          "sample": f"the reference's own Executor on layer 0's expert job, median of {len(times)} passes",
-                                          "rawdots_equal_gpu_bits": bool(np.array_equal(raw.view(np.uint32), layer.rawdots[:T].cpu().numpy().view(np.uint32)))}
-            R.ref_executor_destroy(pool)
-    return {f"config3_moe_decode_T{T}_q8_0_down": entry}
+                def run():
+                    return R.ref_executor_run(pool, H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down.ctypes.data_as(orc.u8p),
+                                              ref_flags, c.ctypes.data_as(orc.i8p), d.ctypes.data_as(orc.f32p), s.ctypes.data_as(orc.i32p), T,
+                                              asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
+                                              status.ctypes.data_as(orc.u32p))
+                if run() == 0:
+                    times, t_end = [], time.perf_counter() + 4.0
+                    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
+                        t0 = time.perf_counter()
+                        run()
+                        times.append(time.perf_counter() - t0)
+                    layer.run_layer(x, wr)
+                    torch.cuda.synchronize()
+                    entry["cpu_reference"] = {"value": statistics.median(times) * 1e6, "unit": "us/expert job", "cores": threads, "kind": "reference",
+                                              "isa": R.ref_executor_isa(pool).decode(),
+                                              "sample": f"the reference's own Executor on layer 0's expert job, median of {len(times)} passes",
+                                              "rawdots_equal_gpu_bits": bool(np.array_equal(raw.view(np.uint32), layer.rawdots[:T].cpu().numpy().view(np.uint32)))}
+                R.ref_executor_destroy(pool)
+        out[f"config3_moe_decode_T{T}_{name}"] = entry
+        del layers
+    return out
 
 
 def extra_configs(strix, torch, steps, warmup):
