@@ -792,14 +792,8 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate,
 // ======================================================================================================== dispatch
 // Up to 4 (routed experts) or 8 (dense matrix) activation rows share one sweep of an expert's weights; an expert with
 // more assignments is swept again for the rest.
-inline int env_int(const char* name) {
-    const char* v = std::getenv(name);
-    return v && *v ? std::atoi(v) : 0;
-}
 // Ring depth: the deepest of 4, 3, 2 at which every workgroup of the launch is resident at once (LDS is what limits it).
 inline int ring_depth(uint64_t waves, int nbmax) {
-    static const int env_depth = env_int("STRIX950_DEPTH");   // tuning aid: 2, 3 or 4 overrides the heuristic
-    if (env_depth >= 2 && env_depth <= 4) return env_depth;
     for (int d = 4; d > 2; --d)
         if (waves <= 256ULL * (163840U / (static_cast<uint32_t>(d) * slot_bytes(nbmax)))) return d;
     return 2;
@@ -904,9 +898,7 @@ constexpr uint32_t kQuadMaxItems = 48;
 // activation row it serves while its weight stream does not, so wide items finish last; the second read of a split
 // expert's weights comes from the last-level cache. A dense matrix: every row shares one sweep.
 inline uint32_t plan_split(const mi355_moe_weights& w, uint32_t rows) {
-    static const int env_split = env_int("STRIX950_SPLIT");   // tuning aid: 1..4 overrides the heuristic for routed experts
     if (w.experts == 1U) return 8;
-    if (env_split >= 1 && env_split <= 4) return static_cast<uint32_t>(env_split);
     return rows <= kFusedMaxRows ? 1U : 4U;
 }
 inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
@@ -1202,9 +1194,7 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     STRIX_LAUNCHED("moe layer router");
     // the fused router planned one item per assignment
     const uint32_t items = rows * wv.top_k;
-    static const int quad_items = env_int("STRIX950_QUAD_ITEMS");   // tuning aid: largest batch (assignments) on the quad sweep
-    const uint32_t quad_max = quad_items > 0 ? static_cast<uint32_t>(quad_items) : kQuadMaxItems;
-    if (items <= quad_max && wv.experts > 1U) {
+    if (items <= kQuadMaxItems && wv.experts > 1U) {
         if (items <= 16U) {
             if (wv.gate_type != MI355_TYPE_Q4_K) launch_project(wv, *r, rows, items, hs(stream));
             else project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
