@@ -458,7 +458,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                     for (uint32_t i = 0; i < NT; ++i)
 #pragma unroll
                         for (uint32_t n = 0; n < 2U; ++n) {
-                            if (FMT == 1 && (ks & 1U) == 0) {     // first half of a block: the product starts from zero
+                            if ((FMT == 1 && (ks & 1U) == 0) || (FMT == 0 && p == 0 && ks == 0)) {   // first MFMA of a block's product: it starts from zero
                                 const floatx16 zero = {0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F};
                                 part[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks & 1U][i], w[ks & 1U][n], zero, 0, 0, 0);
                             } else {
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             if (live_tiles >= TT) k_steps(std::integral_constant<uint32_t, TT>{});
             else if (live_tiles == 1U) k_steps(std::integral_constant<uint32_t, 1>{});
             if (FMT == 0 && p == 3U) {
-                // end of a super-block: running sum += d * P, P = 0
+                // end of a super-block: running sum += d * P (the next super-block's first MFMA starts P from zero)
                 const uint32_t b = s >> 2;
                 const float d[2] = {d_scale[b & 1U][64U * wr + l31], d_scale[b & 1U][64U * wr + 32U + l31]};
 #pragma unroll
@@ -487,10 +487,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
 #pragma unroll
                     for (uint32_t n = 0; n < 2U; ++n)
 #pragma unroll
-                        for (int j = 0; j < 16; ++j) {
-                            acc[i][n][j] = __builtin_fmaf(d[n], part[i][n][j], acc[i][n][j]);
-                            part[i][n][j] = 0.0F;
-                        }
+                        for (int j = 0; j < 16; ++j) acc[i][n][j] = __builtin_fmaf(d[n], part[i][n][j], acc[i][n][j]);   // (tiles with no live row keep P = 0)
                 if (((b & 1U) || b + 1U == blocks) && live_tiles != 0) {
                     // end of a group of 16 sub-blocks: running sum += S hi * M hi + S lo * M hi + S hi * M lo
                     const uint32_t g = b >> 1;

@@ -934,6 +934,8 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
     STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
     STRIX_REQUIRE(w->top_k > 0 && w->top_k <= kRouteMaxTopK && w->top_k <= w->experts, "moe: top_k must be within 1..16 and <= experts");
     STRIX_REQUIRE(static_cast<uint64_t>(rows) * w->top_k < (1ULL << 31), "moe: too many assignments");
+    // plan items are one grid dimension of the expert launches
+    STRIX_REQUIRE(cls != kIntegerClass || item_bound(*w, rows) <= 65535U, "moe: too many work items for one call (experts + rows * top_k / 4 must stay below 65536)");
     wv = *w;
     if (wv.gate_row_stride == 0) wv.gate_row_stride = moe_row_bytes(w->gate_type, w->hidden);
     if (wv.gate_expert_stride == 0) wv.gate_expert_stride = wv.gate_row_stride * w->ffn;

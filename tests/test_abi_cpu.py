@@ -48,6 +48,36 @@ def test_host_admission_needs_no_device(lib):
     assert b"pair-ascending-sb-tree4" in lib.mi355_numerical_identity(12, 0)
 
 
+def test_expert_tensor_format_admission_on_the_host(lib):
+    """Which tensor formats each arithmetic class admits, and the work-item limit, decided on the host before any device call
+    (every pointer below is a dummy: a call that fails admission dereferences none of them and enqueues nothing)."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("strix_pkg", os.path.join(ROOT, "strix-halo-engine-lab_amd", "__init__.py"))
+    pkg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(pkg)
+    lib.mi355_last_error.restype = C.c_char_p
+    rows = pkg.MoeRows()
+
+    def weights(gate_type, down_type, experts=8, top_k=2):
+        return pkg.MoeWeights(512, 256, experts, top_k, gate_type, down_type, 0, 0, 0, 0, 0, 0, 0, 0)
+    # formats no class takes: an argument error (gate/up) or "unsupported" (down) before the null weight pointers are looked at
+    for entry in (lib.mi355_moe_enqueue, lib.mi355_moe_enqueue_prefill_f16):
+        assert entry(C.byref(weights(14, 12)), C.byref(rows), 4, 0, None) == -1 and b"gate/up" in lib.mi355_last_error()
+        assert entry(C.byref(weights(12, 2)), C.byref(rows), 4, 0, None) == -2 and b"down" in lib.mi355_last_error()
+    # per class: Q8_0 gate/up only in the prefill form; Q5_K gate/up and Q5_1 / Q6_K down only in the integer class
+    assert lib.mi355_moe_enqueue(C.byref(weights(8, 8)), C.byref(rows), 4, 0, None) == -1 and b"gate/up" in lib.mi355_last_error()
+    assert lib.mi355_moe_enqueue_prefill_f16(C.byref(weights(13, 12)), C.byref(rows), 4, 0, None) == -1 and b"gate/up" in lib.mi355_last_error()
+    for down in (7, 14):
+        assert lib.mi355_moe_enqueue_prefill_f16(C.byref(weights(12, down)), C.byref(rows), 4, 0, None) == -2
+    # admitted formats get as far as the pointer checks
+    for gate, down in ((12, 12), (13, 8), (12, 7), (13, 14)):
+        assert lib.mi355_moe_enqueue(C.byref(weights(gate, down)), C.byref(rows), 4, 0, None) == -1
+        assert b"weight pointers" in lib.mi355_last_error()
+    # more plan items than a launch dimension holds
+    assert lib.mi355_moe_enqueue(C.byref(weights(12, 12, experts=256, top_k=16)), C.byref(rows), 65535, 0, None) == -1
+    assert b"too many work items" in lib.mi355_last_error()
+
+
 def test_product_path_never_references_the_oracle():
     """The oracle is test infrastructure: nothing under the package may import, link or call it."""
     pkg = os.path.join(ROOT, "strix-halo-engine-lab_amd")

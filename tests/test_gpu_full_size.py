@@ -172,3 +172,41 @@ def test_config4_prefill_f16_mfma_full_size(strix):
         raw_ref[r, k] = ffn(xs[r], gate[e].cpu().numpy(), up[e].cpu().numpy(), down[e].cpu().numpy(), orc.Q4_K)
     close(layer.rawdots.cpu().numpy()[sel], raw_ref)
     close(y[sel], base_ref + np.einsum("tk,tkh->th", w_n.astype(np.float64), raw_ref))
+
+
+def test_config4_size_with_the_host_executor_formats(strix):
+    """Config 4's shape (4096 rows, 256 experts top-8, 32,768 assignments in plan items of up to four) with Q5_K gate/up and
+    Q8_0 down tensors, integer class: the device's gate / up rows and rawdots of 16 random rows against the oracle, bit for bit
+    (rawdots on the device's own h image), and the combine of those rows."""
+    H, I, E, K, T = 4096, 2048, 256, 8, 4096
+    gen = torch.Generator(device="cuda").manual_seed(41)
+
+    def blocks(rows, count, size, scale_bytes, high):
+        w = torch.randint(0, 256, (rows, count, size), dtype=torch.uint8, device="cuda", generator=gen)
+        for at in scale_bytes:
+            w[..., at] = (w[..., at] & 0x03) | high
+        return w.reshape(rows, -1)
+    gate, up = (blocks(E * I, H // 256, 176, (1, 3), 0x0C).reshape(E, I, -1) for _ in range(2))
+    down = blocks(E * H, I // 32, 34, (1,), 0x14).reshape(E, H, -1)
+    wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
+    x = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)
+    layer = strix.MoeLayer(H, I, E, K, gate, up, down, T, intermediates=True, gate_type=strix.TYPE_Q5_K, down_type=strix.TYPE_Q8_0)
+    y, ids, wts, _ = layer.run_layer(x, wr)
+    y = y.cpu().numpy()
+    assert int(layer.status.sum()) == 0
+    sel = np.sort(np.random.default_rng(46).choice(T, 16, replace=False))
+    xs = x.cpu().numpy()[sel].astype(np.float32)
+    ids_n, w_n = ids.cpu().numpy()[sel].astype(np.uint32), wts.cpu().numpy()[sel]
+    ids_ref, w_ref, _, _ = orc.route(xs, wr.cpu().numpy(), K)
+    assert np.array_equal(ids_n, ids_ref) and np.array_equal(bits(w_n), bits(w_ref))
+    c, d, s, _ = orc.quantize_a8(xs)
+    g_np, u_np, d_np = gate.cpu().numpy(), up.cpu().numpy(), down.cpu().numpy()
+    ref = orc.routed_experts(H, I, K, g_np, u_np, d_np, orc.Q8_0, c, d, s, ids_ref, gate_type=orc.Q5_K)
+    slots = (sel[:, None] * K + np.arange(K)[None, :]).reshape(-1)
+    assert np.array_equal(bits(layer.gate_out.cpu().numpy()[slots]), bits(ref.gate))
+    assert np.array_equal(bits(layer.up_out.cpu().numpy()[slots]), bits(ref.up))
+    dc, dd, ds = (t.cpu().numpy()[slots] for t in (layer.down_codes, layer.down_deltas, layer.down_sums))
+    ref_down = orc.routed_experts(H, I, K, g_np, u_np, d_np, orc.Q8_0, c, d, s, ids_ref, gate_type=orc.Q5_K, down_only_from=(dc, dd, ds))
+    raw_dev = layer.rawdots.cpu().numpy()[sel]
+    assert np.array_equal(bits(raw_dev), bits(ref_down.rawdots))
+    assert np.array_equal(bits(y[sel]), bits(orc.combine(0, w_ref, ids_ref, raw_dev)))
