@@ -52,6 +52,7 @@ __global__ __launch_bounds__(256) void down_q6k_kernel(mi355_moe_weights w, mi35
             src[a] = order[c0 + (a < na ? a : na - 1U)];
             acc[a] = 0.0F;
         }
+#pragma unroll 2
         for (uint32_t b = 0; b < blocks; ++b) {
             const uint8_t* blk = wrow + static_cast<size_t>(b) * kQ6kBlock;
             uint32_t ql[16], qh[8];
