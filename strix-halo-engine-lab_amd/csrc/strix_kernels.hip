@@ -370,49 +370,81 @@ __global__ __launch_bounds__(1024) void plan_order_kernel(const uint32_t* routes
     }
 }
 
+// Exclusive prefix sum of one value per thread over a 1024-thread workgroup (16 waves); `total` is the sum over all threads.
+// wave_totals: 16 shared words of the caller's, not reused before its next barrier.
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* wave_totals, uint32_t& total) {
+    const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6;
+    uint32_t x = v;
+#pragma unroll
+    for (uint32_t d = 1; d < 64U; d <<= 1) {
+        const uint32_t below = __shfl_up(x, d);
+        if (lane >= d) x += below;
+    }
+    if (lane == 63U) wave_totals[wave] = x;
+    __syncthreads();
+    uint32_t base = 0, sum = 0;
+    for (uint32_t w = 0; w < 16U; ++w) {
+        const uint32_t t = wave_totals[w];
+        base += w < wave ? t : 0U;
+        sum += t;
+    }
+    total = sum;
+    return base + x - v;
+}
+
+// The expert plan in one workgroup: thread e owns expert e (counts by shared-memory atomics, three prefix sums for the
+// offsets, the item numbers and the touched list, then its own items and - for a small batch - its own stretch of the order).
 __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t split,
                                                     uint32_t item_bound, uint32_t fill_order, uint32_t* plan) {
-    __shared__ uint32_t count[kRouteMaxExperts + 1];
-    const uint32_t tid = threadIdx.x;
-    for (uint32_t e = tid; e <= experts; e += 1024U) count[e] = 0;
+    __shared__ uint32_t count[kRouteMaxExperts];
+    __shared__ uint32_t wave_totals[3][16];
+    __shared__ uint32_t wave_largest[16];
+    __shared__ uint32_t small_routes[256];                 // fill_order: at most 256 assignments
+    const uint32_t tid = threadIdx.x, lane = tid & 63U, wave = tid >> 6;
+    count[tid] = 0;
     __syncthreads();
     for (uint32_t a = tid; a < assignments; a += 1024U) {
         const uint32_t e = routes[a];
+        if (fill_order) small_routes[a] = e;
         if (e < experts) atomicAdd(&count[e], 1U);
     }
     __syncthreads();
-    if (tid == 0) {
-        uint32_t run = 0, touched = 0, largest = 0, made = 0;
-        uint32_t* touched_ids = plan + plan_touched_at(experts);
-        uint32_t* items = plan + plan_items_at(experts, assignments);
-        for (uint32_t e = 0; e < experts; ++e) {
-            const uint32_t c = count[e];
-            count[e] = run;
-            if (c != 0) {
-                for (uint32_t b = 0; b < c; b += split, ++made) {
-                    items[4U * made] = e; items[4U * made + 1U] = run + b; items[4U * made + 2U] = run + (b + split < c ? b + split : c); items[4U * made + 3U] = 0;
-                }
-                touched_ids[touched++] = e;
-            }
-            run += c;
-            largest = c > largest ? c : largest;
-        }
-        for (uint32_t u = made; u < item_bound; ++u) { items[4U * u] = 0; items[4U * u + 1U] = 0; items[4U * u + 2U] = 0; items[4U * u + 3U] = 0; }
-        count[experts] = run;
-        plan[0] = assignments; plan[1] = touched; plan[2] = largest; plan[4] = made;
+    const uint32_t c = tid < experts ? count[tid] : 0U, pieces = (c + split - 1U) / split;
+    uint32_t run, made, touched;
+    const uint32_t first = block_exclusive_scan(c, wave_totals[0], run);
+    const uint32_t item_from = block_exclusive_scan(pieces, wave_totals[1], made);
+    const uint32_t touched_from = block_exclusive_scan(c != 0 ? 1U : 0U, wave_totals[2], touched);
+    uint32_t largest = c;
+#pragma unroll
+    for (int d = 32; d; d >>= 1) {
+        const uint32_t other = __shfl_xor(largest, d);
+        largest = other > largest ? other : largest;
     }
+    if (lane == 0) wave_largest[wave] = largest;
     __syncthreads();
     uint32_t* offsets = plan + kPlanOffsetsAt;
+    uint32_t* touched_ids = plan + plan_touched_at(experts);
     uint32_t* order = plan + plan_order_at(experts);
-    for (uint32_t e = tid; e <= experts; e += 1024U) offsets[e] = count[e];
-    if (!fill_order) return;                  // large batches: plan_order_kernel follows
-    for (uint32_t e = tid; e < experts; e += 1024U) {
-        const uint32_t end = e + 1 <= experts ? count[e + 1] : 0;
-        uint32_t at = count[e];
-        if (at == end) continue;
-        for (uint32_t a = 0; a < assignments && at < end; ++a)
-            if (routes[a] == e) order[at++] = a;
+    uint32_t* items = plan + plan_items_at(experts, assignments);
+    if (tid < experts) {
+        offsets[tid] = first;
+        if (c != 0) {
+            touched_ids[touched_from] = tid;
+            for (uint32_t b = 0, k = item_from; b < c; b += split, ++k)
+                *reinterpret_cast<uint4*>(items + 4U * k) = make_uint4(tid, first + b, first + (b + split < c ? b + split : c), 0U);
+        }
     }
+    for (uint32_t u = made + tid; u < item_bound; u += 1024U) *reinterpret_cast<uint4*>(items + 4U * u) = make_uint4(0U, 0U, 0U, 0U);
+    if (tid == 0) {
+        uint32_t most = 0;
+        for (uint32_t w = 0; w < 16U; ++w) most = wave_largest[w] > most ? wave_largest[w] : most;
+        offsets[experts] = run;
+        plan[0] = assignments; plan[1] = touched; plan[2] = most; plan[4] = made;
+    }
+    if (!fill_order || tid >= experts || c == 0) return;   // large batches: plan_order_kernel follows
+    uint32_t at = first;
+    for (uint32_t a = 0; a < assignments; ++a)
+        if (small_routes[a] == tid) order[at++] = a;
 }
 
 __global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* routes, const float* route_weights, uint32_t experts,
