@@ -383,6 +383,55 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
         assert 1e-4 < rel_err(layer.gate_out[:T].cpu().numpy(), g_exact)[0] < 5e-2
 
 
+# ------------------------------------------------------------------------------------------- the expert plan
+@pytest.mark.parametrize("E,K,T", [(6, 3, 5), (128, 8, 8), (128, 8, 16), (16, 4, 40), (1024, 16, 16), (1, 1, 7), (256, 8, 500), (3, 2, 300)])
+def test_expert_plan_words(strix, E, K, T):
+    """The plan written by mi355_moe_enqueue_csr (the stable CSR of (row, slot) by expert, src/hip_moe_q4k_a8_probe.hip:91-147):
+    header counts, offsets, touched ids, order and work items against a numpy statement, for one-workgroup plans (up to 256
+    assignments) and for the wave-per-expert order of larger ones; a route id out of range belongs to no expert."""
+    H, I = 256, 256
+    rng = np.random.default_rng(E + T)
+    one = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((1, 1, H)) * 0.02).astype(np.float32))
+    gate = np.ascontiguousarray(np.broadcast_to(one, (E, I, one.shape[-1])))
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(gate), dev(gate), T)
+    ids = np.stack([rng.permutation(E)[:K] if E >= K else np.zeros(K, np.int64) for _ in range(T)]).astype(np.int32)
+    if E > 1:
+        ids[T // 2, 0] = E + 5                                   # invalid: flagged by the prologue, skipped by the plan
+    x = dev(rng.standard_normal((T, H)).astype(np.float16))
+    w = dev(np.ones((T, K), np.float32))
+    layer.plan.fill_(-1)
+    layer.plan[16:272] = 0
+    layer.stage("csr", x, dev(ids), w)
+    plan = layer.plan.cpu().numpy().view(np.uint32)
+    flat = ids.reshape(-1).astype(np.int64)
+    A = T * K
+    split = 8 if E == 1 else (1 if T <= 16 else 4)
+    valid = flat < E
+    counts = np.bincount(flat[valid], minlength=E)
+    offsets = np.concatenate([[0], np.cumsum(counts)])
+    pad4 = lambda v: (v + 3) & ~3
+    offsets_at = 272
+    touched_at = offsets_at + pad4(E + 1)
+    order_at = touched_at + pad4(E)
+    items_at = order_at + pad4(A)
+    touched = np.nonzero(counts)[0]
+    assert plan[0] == A and plan[1] == touched.size and plan[2] == counts.max()
+    assert np.array_equal(plan[offsets_at: offsets_at + E + 1], offsets)
+    assert np.array_equal(plan[touched_at: touched_at + touched.size], touched)
+    order = np.argsort(np.where(valid, flat, E), kind="stable")[: int(valid.sum())]
+    assert np.array_equal(plan[order_at: order_at + order.size], order)
+    want_items = []
+    for e in touched:
+        for b in range(0, counts[e], split):
+            want_items.append((e, offsets[e] + b, offsets[e] + min(b + split, counts[e]), 0))
+    assert plan[4] == len(want_items)
+    got_items = plan[items_at: items_at + 4 * len(want_items)].reshape(-1, 4)
+    assert np.array_equal(got_items, np.array(want_items, np.uint32).reshape(-1, 4))
+    bound = min(A, E + A // split)
+    assert np.all(plan[items_at + 4 * len(want_items): items_at + 4 * bound] == 0)     # zero records up to the launch's item bound
+    assert np.all(plan[16:272] == 0)
+
+
 # ------------------------------------------------------------------------------------------- the host executor's down formats
 @pytest.mark.parametrize("gate_type,down_type,H,I,E,K,T,entry", [
     (orc.Q4_K, orc.Q8_0, 512, 256, 6, 3, 5, "staged"),          # the shape of the compiled reference's own whole-job check
