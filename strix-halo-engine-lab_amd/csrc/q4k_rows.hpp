@@ -30,7 +30,8 @@ namespace strix950 {
 constexpr uint32_t kWaveRows = 64;
 constexpr uint32_t kStageBytes = kWaveRows * 144U;   // 9,216
 constexpr uint32_t kStagePieces = 9;                 // global_load_lds instructions per stage (576 pieces / 64 lanes)
-// a ring slot: the stage's weights + its codes of up to nbmax (4 or 8) activation rows
+// a ring slot: the stage's weights + its codes of up to nbmax (4 or 8) activation rows; a codes copy always writes four
+// rows (1 KB), so only a sweep with narrow codes copies may use slot_bytes(1)
 __host__ __device__ constexpr uint32_t slot_bytes(int nbmax) { return kStageBytes + 256U * static_cast<uint32_t>(nbmax); }
 typedef __attribute__((address_space(3))) uint8_t lds_u8;      // ring slots are addressed in the LDS address space
 template <int NA> constexpr uint32_t stage_copies() { return kStagePieces + (NA + 3) / 4; }   // copy instructions per stage
@@ -66,8 +67,11 @@ struct StageSource {
     }
     // start the copy of the next super-block of all 64 rows (and of the activation rows' codes) into one ring slot,
     // then step to the block after it
-    template <int NA>
+    // A codes copy moves four activation rows (1 KB: lanes 16 a .. 16 a + 15 move row a). NARROW (NA == 1 only): just the
+    // first sixteen lanes take part, so the slot ends 256 bytes after the weights (slot_bytes(1)) instead of 1 KB after them.
+    template <int NA, bool NARROW = false>
     __device__ __forceinline__ void start(lds_u8* slot) {
+        static_assert(!NARROW || NA == 1, "a narrow codes copy serves one activation row");
 #pragma unroll
         for (uint32_t i = 0; i < kStagePieces; ++i) {
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)piece[i],
@@ -76,8 +80,9 @@ struct StageSource {
         }
 #pragma unroll
         for (int h = 0; h < (NA + 3) / 4; ++h) {
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)act_piece[h],
-                                             (__attribute__((address_space(3))) void*)(slot + kStageBytes + 1024U * h), 16, 0, 0);
+            if (!NARROW || (threadIdx.x & 63U) < 16U)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)act_piece[h],
+                                                 (__attribute__((address_space(3))) void*)(slot + kStageBytes + 1024U * h), 16, 0, 0);
             act_piece[h] += 256;
         }
     }
@@ -193,7 +198,7 @@ __device__ __forceinline__ void block_compute(const lds_u8* slot, uint32_t kb, c
 // Whole sweep: K = blocks super-blocks of the 64 rows described by `source` against the NA rows of `act`.
 // value[a] = the lane's row against activation row a. `slots` are DEPTH separate LDS buffers of slot_bytes().
 // On entry nothing is in flight; on exit every copy has landed and been consumed.
-template <int NA, int DEPTH>
+template <int NA, int DEPTH, bool NARROW = false>
 __device__ __forceinline__ void sweep_rows(lds_u8* const (&slots)[DEPTH], StageSource source, uint32_t blocks,
                                            const ActRows<NA>& act, float (&value)[NA]) {
     const uint32_t lane = threadIdx.x & 63U;
@@ -208,7 +213,7 @@ __device__ __forceinline__ void sweep_rows(lds_u8* const (&slots)[DEPTH], StageS
     source.init_act<NA>(act.codes, act.width, act.lane_row);
 #pragma unroll
     for (int s = 0; s < DEPTH - 1; ++s)
-        if (static_cast<uint32_t>(s) < blocks) source.start<NA>(slots[s]);
+        if (static_cast<uint32_t>(s) < blocks) source.start<NA, NARROW>(slots[s]);
     for (uint32_t b0 = 0; b0 < blocks; b0 += DEPTH) {
 #pragma unroll
         for (int s = 0; s < DEPTH; ++s) {
@@ -225,7 +230,7 @@ __device__ __forceinline__ void sweep_rows(lds_u8* const (&slots)[DEPTH], StageS
                 // started so far: stages 0 .. min(blocks, b + DEPTH - 1) - 1; stage b must have landed
                 const uint32_t last = b + DEPTH - 1U < blocks ? b + DEPTH - 1U : blocks;
                 wait_stages_ahead<stage_copies<NA>()>(last - 1U - b);
-                if (b + DEPTH - 1U < blocks) source.start<NA>(slots[(s + DEPTH - 1) % DEPTH]);
+                if (b + DEPTH - 1U < blocks) source.start<NA, NARROW>(slots[(s + DEPTH - 1) % DEPTH]);
                 block_compute<NA>(slots[s], b, vd, vf, acc);
             }
         }

@@ -792,6 +792,61 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, mi355_m
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
+// Down rows and the ordered combine of a decode batch in one launch: a workgroup owns (row, 64 output columns) and has one
+// wave per slot of the row, wave k sweeping the down rows of the expert in slot k (the plan holds one item per assignment,
+// in assignment order); the waves leave their 64 values in LDS and wave 0 folds them exactly as merge_kernel does. Only
+// waves of one workgroup exchange data, so nothing depends on the visibility of another workgroup's stores.
+// Reference: src/cpu/core/routed_expert.cpp:429-447, src/moe_a8_down_contract.cpp:146, include/strix/moe/combine.hpp:36-59.
+constexpr uint32_t kDownMergeSlots = 8;        // top_k bound: 8 waves x 2 ring slots fill the LDS of a compute unit
+__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments, uint32_t form) {
+    __shared__ __attribute__((aligned(16))) uint8_t rings[kDownMergeSlots][2][slot_bytes(1)];
+    __shared__ float slot_value[kDownMergeSlots][64];
+    __shared__ uint32_t slot_order[kDownMergeSlots];
+    __shared__ float slot_weight[kDownMergeSlots];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, row = blockIdx.y, o = blockIdx.x * 64U + lane;
+    if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;            // the whole job: no down rows, nothing published
+    const uint32_t a = row * w.top_k + wave;
+    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * a);
+    const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
+    float value = 0.0F;
+    if (begin != end) {                                                        // (an invalid route has no item: its row is flagged)
+        const uint32_t* order = r.plan + plan_order_at(w.experts);
+        const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
+        const uint32_t stride = static_cast<uint32_t>(w.down_row_stride);
+        StageSource source;
+        source.init([&](uint32_t q) { return rows + q * stride; });
+        lds_u8* const slots[2] = {(lds_u8*)rings[wave][0], (lds_u8*)rings[wave][1]};
+        const uint32_t src[1] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(order[begin]))}, lane_rows[1] = {order[begin]};
+        const ActRows<1> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src, lane_rows);
+        float swept[1];
+        sweep_rows<1, 2, true>(slots, source, w.ffn / 256U, act, swept);      // narrow codes copies: the slots are slot_bytes(1)
+        value = swept[0];
+        r.rawdots[static_cast<size_t>(src[0]) * w.hidden + o] = value;
+    }
+    slot_value[wave][lane] = value;
+    if (threadIdx.x == 0) {
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
+        if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
+            for (uint32_t i = 1; i < w.top_k; ++i)
+                for (uint32_t j = i; j > 0 && r.routes[row * w.top_k + slot_order[j]] < r.routes[row * w.top_k + slot_order[j - 1]]; --j) {
+                    const uint32_t t = slot_order[j]; slot_order[j] = slot_order[j - 1]; slot_order[j - 1] = t;
+                }
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights[row * w.top_k + slot_order[k]];
+    }
+    __syncthreads();
+    // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is the combine's own)
+    if (wave != 0 || (r.status[row] & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
+    float acc = 0.0F;
+    for (uint32_t k = 0; k < w.top_k; ++k) {
+        const float ev = slot_value[slot_order[k]][lane];
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], ev, acc);
+        else acc = acc + slot_weight[k] * ev;
+    }
+    const float y = r.base ? acc + r.base[static_cast<size_t>(row) * w.hidden + o] : acc;
+    if (!finite_f(y)) atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
+}
+
 // SwiGLU + A8 re-quantisation of dense gate/up rows. Reference: src/cpu/core/routed_expert.cpp:147-170.
 __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate, const float* up, uint32_t ffn, uint32_t exp_kind,
                                                               int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
@@ -935,6 +990,12 @@ inline uint32_t plan_split(const mi355_moe_weights& w, uint32_t rows) {
 }
 inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
     return plan_item_bound(w.experts, rows * w.top_k, plan_split(w, rows));
+}
+
+inline uint32_t compute_units() {
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    return cus > 0 ? static_cast<uint32_t>(cus) : 0U;
 }
 
 // ======================================================================================================== admission
@@ -1242,6 +1303,15 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
         }
     } else {
         launch_project(wv, *r, rows, items, hs(stream));
+        // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
+        // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
+        // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
+        if (wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
+            (wv.hidden / 64U) * rows <= compute_units()) {
+            down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, hs(stream)>>>(wv, *r, items, form);
+            STRIX_LAUNCHED("moe layer experts + combine");
+            return MI355_OK;
+        }
         launch_down(wv, *r, rows, items, hs(stream));
     }
     STRIX_LAUNCHED("moe layer experts");

@@ -383,6 +383,28 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
         assert 1e-4 < rel_err(layer.gate_out[:T].cpu().numpy(), g_exact)[0] < 5e-2
 
 
+@pytest.mark.parametrize("combine", [0, 1])
+def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine):
+    """A decode batch whose (row, 64 columns) workgroups are all resident takes the down rows and the ordered combine in one
+    launch (a wave per slot): output, rawdots and status words must equal the staged entry points' bit for bit, for both
+    combine forms and with a base term."""
+    E, H, I, K, T = 32, 1024, 512, 8, 8
+    rng = np.random.default_rng(91 + combine)
+    gate, up, down = make_layer(rng, H, I, E)
+    x = dev(rng.standard_normal((T, H)).astype(np.float16))
+    wr = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
+    base = dev(rng.standard_normal((T, H)).astype(np.float32))
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T)
+    y, ids, wts, _ = layer.run_layer(x, wr, base=base, combine=combine)
+    y, raw = y.clone(), layer.rawdots[:T].clone()
+    assert int(layer.status.sum()) == 0
+    staged = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, T)
+    want = staged.run(x, ids.clone(), wts.clone(), base=base, combine=combine)
+    assert torch.equal(raw, staged.rawdots[:T]) and torch.equal(y, want)
+    ids_n, w_n = ids.cpu().numpy().astype(np.uint32), wts.cpu().numpy()
+    assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine(combine, w_n, ids_n, raw.cpu().numpy(), base=base.cpu().numpy())))
+
+
 # ------------------------------------------------------------------------------------------- the expert plan
 @pytest.mark.parametrize("E,K,T", [(6, 3, 5), (128, 8, 8), (128, 8, 16), (16, 4, 40), (1024, 16, 16), (1, 1, 7), (256, 8, 500), (3, 2, 300)])
 def test_expert_plan_words(strix, E, K, T):
