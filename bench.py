@@ -269,6 +269,13 @@ def extra_configs(strix, torch, steps, warmup):
         out[f"config2_dense_q4k_ffn_B{B}"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
                                               "algorithmic_bytes": nbytes}
     del layers
+    # RMSNorm in front of the block (the third entry of the reference's CPU kernel table): 4096 rows of 4096 fp32
+    xn = torch.randn((4096, 4096), device="cuda", generator=gen)
+    wn = torch.randn(4096, device="cuda", generator=gen)
+    sec = time_steps(torch, lambda i: strix.rmsnorm_f32(xn, wn), max(steps // 4, 10), max(warmup // 4, 3))
+    nbytes = 2 * xn.numel() * 4 + wn.numel() * 4
+    out["rmsnorm_f32_4096x4096"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS, "algorithmic_bytes": nbytes}
+    del xn, wn
     # config 5: expert-TP rank 0 of 2, 16 rows, hidden 6144, 160 experts top-8, intermediate 2560 / 2
     H, I, E, K, T = 6144, 2560, 160, 8, 16
     grb, drb = H // 256 * 144, I // 256 * 144

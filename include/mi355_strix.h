@@ -74,6 +74,15 @@ int32_t mi355_quantize_weight_rows(uint32_t weight_type, const float* x, uint32_
                                    void* out, mi355_stream stream);
 
 /* ------------------------------------------------------------------------------------------------------
+ * RMSNorm of fp32 rows. Replaces strix::cpu::Kernels::rmsnorm_f32 (src/cpu/core/backend.hpp:71-72,
+ * src/cpu/core/reference.cpp:86-103): ReductionOrder::lane_strided_fma_lds_halving with 256 lanes for n >= 512 and 128
+ * below (backend.hpp:91): lane l runs the fma chain over x[l], x[l + L], ..., the partial sums are halved pairwise
+ * (l, l + h), r = 1 / sqrt(sum / n + eps), y = (x * r) * w (w may be NULL: y = x * r). Rows are dense: [rows][n].
+ */
+int32_t mi355_rmsnorm_f32(const float* x, const float* w, uint32_t n, float eps, float* y, uint32_t rows,
+                          mi355_stream stream);
+
+/* ------------------------------------------------------------------------------------------------------
  * A8 activation quantiser. Replaces strix::cpu::Kernels::quantize_a8 (src/cpu/core/backend.hpp:68-69,
  * src/cpu/core/reference.cpp:35-55): groups of 32, delta = amax / 127 (1 for an all-zero group or amax < 2^-119),
  * code = rint(x / delta) clamped to +-127, per-group code sums. width % 32 != 0 -> MI355_E_INVALID_ARGUMENT before any

@@ -99,6 +99,9 @@ void ref_q8_0_quantize_group(const float* v, float* d, std::int8_t* q) {
 int ref_quantize_a8(const float* x, std::size_t width, std::int8_t* codes, float* deltas, std::int32_t* sums) {
     return guarded([&] { strix::cpu::reference_kernels().quantize_a8(x, width, codes, deltas, sums); });
 }
+int ref_rmsnorm_f32(const float* x, const float* w, unsigned n, float eps, float* y, unsigned rows) {
+    return guarded([&] { strix::cpu::reference_kernels().rmsnorm_f32(x, w, n, eps, y, rows, strix::cpu::Stream{}); });
+}
 int ref_gemv_q8_0_a8(const strix::cpu::Q8a8View* view) {
     return guarded([&] { strix::cpu::reference_kernels().gemv_q8_0_a8(*view, strix::cpu::Stream{}); });
 }

@@ -224,6 +224,26 @@ int orc_gemv_q8_0_a8(const orc_q8a8_view* v, int threads) {
     return 0;
 }
 
+/* ------------------------------------------------------------------ RMSNorm */
+/* src/cpu/core/reference.cpp:86-103; lane count src/cpu/core/backend.hpp:91. */
+void orc_rmsnorm_f32(const float* x, const float* w, uint32_t n, float eps, float* y, uint32_t rows) {
+    const uint32_t lanes = n >= 512 ? 256U : 128U;
+    float partial[256];
+    for (uint32_t row = 0; row < rows; ++row) {
+        const float* xr = x + (size_t)row * n;
+        float* yr = y + (size_t)row * n;
+        for (uint32_t lane = 0; lane < lanes; ++lane) {
+            float a = 0.0F;
+            for (uint32_t i = lane; i < n; i += lanes) a = fmaf(xr[i], xr[i], a);
+            partial[lane] = a;
+        }
+        for (uint32_t h = lanes / 2; h > 0; h >>= 1)
+            for (uint32_t lane = 0; lane < h; ++lane) partial[lane] = partial[lane] + partial[lane + h];
+        const float r = 1.0F / sqrtf(partial[0] / (float)n + eps);
+        for (uint32_t i = 0; i < n; ++i) yr[i] = w ? (xr[i] * r) * w[i] : xr[i] * r;
+    }
+}
+
 /* ------------------------------------------------------------------ Q4_K x A8 row */
 float orc_q4k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,
                      const int32_t* sums) {

@@ -11,7 +11,7 @@
  * without fast-math: every float operation below is one IEEE-754 binary32 round-to-nearest operation.
  *
  * Pinning status (what checks each function besides this text):
- *   half/Q8_0/Q4_K decode, scale/min unpack, Q8_0 writer, A8 quantiser, Q8_0xA8 product order,
+ *   half/Q8_0/Q4_K decode, scale/min unpack, Q8_0 writer, A8 quantiser, RMSNorm, Q8_0xA8 product order,
  *   Q4_KxA8 and Q5_KxA8 rows, Q8_0, Q5_1 and Q6_K down rows, router selection/weights, combine: pinned by the literal vectors and
  *   invariants of the reference's own tests (tests/golden/) and, where it builds, bitwise against the
  *   compiled reference (oracle/_ref).
@@ -77,6 +77,7 @@ typedef struct {
 int orc_gemv_q8_0_a8(const orc_q8a8_view* view, int threads);   /* -1: in % 32 != 0, nothing written */
 
 /* ---- Q4_K x A8 row (src/cpu/core/routed_expert.cpp:73-108 == src/moe_q4k_a8_contract.cpp:126-140) */
+void orc_rmsnorm_f32(const float* x, const float* w, uint32_t n, float eps, float* y, uint32_t rows);
 float orc_q4k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,
                      const int32_t* sums);
 float orc_q5k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,

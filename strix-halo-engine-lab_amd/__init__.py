@@ -81,7 +81,7 @@ EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi3
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
            "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
-           "mi355_swiglu_quantize"]
+           "mi355_swiglu_quantize", "mi355_rmsnorm_f32"]
 
 
 def require_gpu():
@@ -138,6 +138,14 @@ def quantize_a8(x, want_sums=True):
     check(lib().mi355_quantize_a8(_p(x), input_kind(x), rows, width, C.c_uint64(x.stride(0) * x.element_size()), _p(codes),
                                   _p(deltas), _p(sums), _p(status), _stream()))
     return codes, deltas, sums, status
+
+
+def rmsnorm_f32(x, weight=None, eps=1e-6):
+    """RMSNorm of fp32 rows in the reference's reduction order (strix::cpu::Kernels::rmsnorm_f32)."""
+    assert x.dim() == 2 and x.is_contiguous() and x.dtype == torch.float32
+    y = torch.empty_like(x)
+    check(lib().mi355_rmsnorm_f32(_p(x), _p(weight), x.shape[1], C.c_float(eps), _p(y), x.shape[0], _stream()))
+    return y
 
 
 def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False, row_bytes_=None, out_stride=None):

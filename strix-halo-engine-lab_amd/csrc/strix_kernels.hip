@@ -134,6 +134,27 @@ __global__ __launch_bounds__(64) void quantize_q4_k_rows_kernel(const float* x, 
 }
 
 // ======================================================================================================== A8 quantiser
+// RMSNorm of fp32 rows in the reference's declared order (src/cpu/core/reference.cpp:86-103, lane count
+// src/cpu/core/backend.hpp:91): lane l of L = 256 (n >= 512) or 128 runs the fma chain over x[l], x[l + L], ...; the L partial
+// sums are halved in LDS (partial[l] += partial[l + h], h = L/2 .. 1); r = 1 / sqrt(sum / n + eps); y = (x * r) * w.
+// One workgroup of L threads per row: the lanes' strided chains are coalesced reads as they stand.
+__global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* x, const float* w, uint32_t n, float eps, float* y) {
+    __shared__ float partial[256];
+    const uint32_t lanes = blockDim.x, lane = threadIdx.x;
+    const float* xr = x + static_cast<size_t>(blockIdx.x) * n;
+    float* yr = y + static_cast<size_t>(blockIdx.x) * n;
+    float a = 0.0F;
+    for (uint32_t i = lane; i < n; i += lanes) a = __builtin_fmaf(xr[i], xr[i], a);
+    partial[lane] = a;
+    for (uint32_t h = lanes / 2U; h > 0; h >>= 1) {
+        __syncthreads();
+        if (lane < h) partial[lane] = partial[lane] + partial[lane + h];
+    }
+    __syncthreads();
+    const float r = 1.0F / __builtin_sqrtf(partial[0] / static_cast<float>(n) + eps);
+    for (uint32_t i = lane; i < n; i += lanes) yr[i] = w ? (xr[i] * r) * w[i] : xr[i] * r;
+}
+
 // One aligned group of 32 lanes per 32-value group; 8 groups per 256-thread block.
 // Reference: src/cpu/core/reference.cpp:35-55.
 template <int KIND>
@@ -1122,6 +1143,15 @@ int32_t mi355_quantize_a8(const void* x, uint32_t kind, uint32_t rows, uint32_t 
     else if (kind == MI355_INPUT_F16) quantize_a8_kernel<1><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, sums, status);
     else quantize_a8_kernel<2><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, sums, status);
     STRIX_LAUNCHED("quantize_a8");
+    return MI355_OK;
+}
+
+int32_t mi355_rmsnorm_f32(const float* x, const float* w, uint32_t n, float eps, float* y, uint32_t rows, mi355_stream stream) {
+    if (rows == 0 || n == 0) return MI355_OK;
+    STRIX_REQUIRE(x && y, "rmsnorm: null pointer");
+    STRIX_REQUIRE(rows <= 0x7fffffffU, "rmsnorm: too many rows");
+    rmsnorm_f32_kernel<<<rows, n >= 512U ? 256 : 128, 0, hs(stream)>>>(x, w, n, eps, y);
+    STRIX_LAUNCHED("rmsnorm_f32");
     return MI355_OK;
 }
 

@@ -36,6 +36,10 @@ struct Kernels {
                                 sums, nullptr, s.stream));
     }
     static void gemv_q8_0_a8(const Q8a8View& v, const Stream& s = {}) { check(mi355_gemv_q8_0_a8(&v, s.stream)); }
+    // x, y: device fp32 [rows][n]; w: device fp32 [n] or null (the signature of strix::cpu::Kernels::rmsnorm_f32)
+    static void rmsnorm_f32(const float* x, const float* w, unsigned n, float eps, float* y, unsigned rows, const Stream& s = {}) {
+        check(mi355_rmsnorm_f32(x, w, n, eps, y, rows, s.stream));
+    }
 };
 
 // ---------------------------------------------------------------------------------------------- router

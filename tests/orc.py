@@ -117,6 +117,14 @@ def _declare(L):
 
 
 # ---------------------------------------------------------------- numpy-level helpers
+def rmsnorm_f32(x, w=None, eps=1e-6):
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty_like(x)
+    wp = None if w is None else _ptr(np.ascontiguousarray(w, np.float32), f32p)
+    lib().orc_rmsnorm_f32(_ptr(x, f32p), wp, C.c_uint32(x.shape[1]), C.c_float(eps), _ptr(y, f32p), C.c_uint32(x.shape[0]))
+    return y
+
+
 def row_bytes(qtype, elements):
     if qtype == Q5_1:
         return elements // 32 * Q5_1_BLOCK

@@ -38,6 +38,18 @@ def random_q4k(rng, shape_rows, width):
     return w
 
 
+# ------------------------------------------------------------------------------------------- RMSNorm
+@pytest.mark.parametrize("n,rows", [(64, 3), (511, 2), (512, 5), (2048, 8), (4096, 300), (6144, 16)])
+def test_rmsnorm_bit_exact(strix, n, rows):
+    """mi355_rmsnorm_f32 against the oracle (itself bitwise equal to the compiled reference kernel table): the lane-strided
+    fma chains, the halving tree, the correctly rounded 1 / sqrt and the two products, bit for bit."""
+    rng = np.random.default_rng(n + rows)
+    x = (rng.standard_normal((rows, n)) * 3.0).astype(np.float32)
+    w = rng.standard_normal(n).astype(np.float32)
+    assert np.array_equal(bits(strix.rmsnorm_f32(dev(x), dev(w)).cpu().numpy()), bits(orc.rmsnorm_f32(x, w)))
+    assert np.array_equal(bits(strix.rmsnorm_f32(dev(x), None, eps=1e-5).cpu().numpy()), bits(orc.rmsnorm_f32(x, None, 1e-5)))
+
+
 # ------------------------------------------------------------------------------------------- block decode / writers
 @pytest.mark.parametrize("qtype,width", [(orc.Q8_0, 4096), (orc.Q4_K, 2048), (orc.Q4_K, 5120)])
 def test_dequantised_weights_bit_exact(strix, qtype, width):

@@ -740,6 +740,27 @@ def test_ref_q4k_row_and_down_row_bits_at_config_widths():
 
 
 @needs_ref
+def test_ref_rmsnorm_bits():
+    """RMSNorm (lane-strided fma chains, halving tree): the restatement against the compiled reference kernel table, bit for
+    bit, for both lane counts, with and without the weight vector; and against float64 to 1e-6."""
+    import ctypes as C
+    R = orc.ref()
+    rng = np.random.default_rng(27)
+    for n, rows in ((64, 3), (511, 2), (512, 2), (2048, 4), (5120, 2), (6144, 1)):
+        x = (rng.standard_normal((rows, n)) * rng.choice([1e-3, 1.0, 50.0])).astype(np.float32)
+        w = rng.standard_normal(n).astype(np.float32)
+        for weight in (w, None):
+            mine = orc.rmsnorm_f32(x, weight, 1e-6)
+            theirs = np.empty_like(x)
+            wp = None if weight is None else weight.ctypes.data_as(orc.f32p)
+            assert R.ref_rmsnorm_f32(x.ctypes.data_as(orc.f32p), wp, n, C.c_float(1e-6), theirs.ctypes.data_as(orc.f32p), rows) == 0, R.ref_last_error()
+            assert np.array_equal(bits(mine), bits(theirs))
+            x64 = x.astype(np.float64)
+            want = x64 / np.sqrt(np.mean(x64 ** 2, axis=1, keepdims=True) + 1e-6) * (1.0 if weight is None else weight.astype(np.float64))
+            assert np.max(np.abs(mine - want)) <= 2e-6 * np.max(np.abs(want))
+
+
+@needs_ref
 def test_ref_exp_functions_bits():
     R = orc.ref()
     rng = np.random.default_rng(23)
