@@ -37,7 +37,20 @@ def layer_case(seed, H, I, E, T, K):
     return gate, up, down, x, ids
 
 
+def format_layer_case(seed, H, I, E, T, K):
+    """The host executor's other formats: Q5_K gate/up and Q5_1 down blocks of random bytes."""
+    rng = np.random.default_rng(seed)
+    gate, up = orc.random_q5_k(rng, (E, I), H), orc.random_q5_k(rng, (E, I), H)
+    down = orc.random_q5_1(rng, (E, H), I)
+    x = rng.standard_normal((T, H)).astype(np.float16).astype(np.float32)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.uint32)
+    return gate, up, down, x, ids
+
+
 LAYER_CASES = [(101, 2048, 768, 3, 2, 2), (102, 2560, 640, 2, 3, 2), (103, 512, 256, 6, 4, 3)]
+FORMAT_LAYER_CASES = [(111, 1024, 512, 4, 3, 2), (112, 2048, 768, 3, 2, 2)]
+Q6K_WIDTHS = [256, 768, 1280, 1536]
+RMSNORM_CASES = [(401, 64, 3), (402, 511, 2), (403, 2048, 4), (404, 6144, 2)]
 ROW_WIDTHS = [2048, 768, 4096, 5120, 6144, 1280, 27648]
 GEMV_CASES = [(201, 4096, 64, 2), (202, 1024, 33, 3)]
 
@@ -79,6 +92,35 @@ def main():
         assert R.ref_gemv_q8_0_a8(C.byref(v)) == 0
         out[f"gemv_{seed}_bits"] = y.view(np.uint32)
         out[f"gemv_{seed}_a8_codes_crc"] = np.array([int(np.bitwise_xor.reduce(codes.view(np.uint8).astype(np.uint32) * np.arange(1, codes.size + 1, dtype=np.uint32).reshape(codes.shape), axis=None))], np.uint32)
+    for seed, H, I, E, T, K in FORMAT_LAYER_CASES:
+        gate, up, down, x, ids = format_layer_case(seed, H, I, E, T, K)
+        codes, deltas, sums, _ = orc.quantize_a8(x)
+        asg = np.array([[t, k, ids[t, k]] for t in range(T) for k in range(K)], np.uint32)
+        raw = np.zeros((T, K, H), np.float32)
+        status = np.zeros(T, np.uint32)
+        rc = R.ref_routed_expert_run_fmt(H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down.ctypes.data_as(orc.u8p), 3,
+                                         codes.ctypes.data_as(orc.i8p), deltas.ctypes.data_as(orc.f32p), sums.ctypes.data_as(orc.i32p), T,
+                                         asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
+                                         status.ctypes.data_as(orc.u32p), 0, 0)
+        assert rc == 0
+        out[f"format_layer_{seed}_rawdots_bits"] = raw.view(np.uint32)
+    rng = np.random.default_rng(310)
+    vals = []
+    for width in Q6K_WIDTHS:
+        w = orc.random_q6_k(rng, (1,), width)[0]
+        x = (rng.standard_normal((1, width)) * 3.0).astype(np.float32)
+        codes, deltas, sums, _ = orc.quantize_a8(x, tiny_rule=True)
+        assert R.ref_evaluate_down_row(w.ctypes.data_as(orc.u8p), C.c_size_t(w.size), codes[0].ctypes.data_as(orc.i8p), deltas[0].ctypes.data_as(orc.f32p),
+                                       sums[0].ctypes.data_as(orc.i32p), C.c_size_t(width), 14, C.byref(o)) == 0
+        vals.append(o.value)
+    out["q6k_down_rows_bits"] = np.array(vals, np.float32).view(np.uint32)
+    for seed, n, rows in RMSNORM_CASES:
+        rng = np.random.default_rng(seed)
+        x = (rng.standard_normal((rows, n)) * 2.0).astype(np.float32)
+        w = rng.standard_normal(n).astype(np.float32)
+        y = np.empty_like(x)
+        assert R.ref_rmsnorm_f32(x.ctypes.data_as(orc.f32p), w.ctypes.data_as(orc.f32p), n, C.c_float(1e-6), y.ctypes.data_as(orc.f32p), rows) == 0
+        out[f"rmsnorm_{seed}_bits"] = y.view(np.uint32)
     np.savez_compressed(os.path.join(HERE, "ref_vectors.npz"), **out)
     print("wrote", {k: v.shape for k, v in out.items()})
 

@@ -875,3 +875,21 @@ def test_committed_reference_vectors():
         codes, deltas, sums, _ = orc.quantize_a8(x)
         y, _ = orc.gemv_q8_0_a8(w, codes, deltas, width, count, threads=2)
         assert np.array_equal(bits(y), gold[f"gemv_{seed}_bits"])
+    for seed, H, I, E, T, K in mk.FORMAT_LAYER_CASES:                      # Q5_K gate/up + Q5_1 down whole jobs
+        gate, up, down, x, ids = mk.format_layer_case(seed, H, I, E, T, K)
+        codes, deltas, sums, _ = orc.quantize_a8(x)
+        r = orc.routed_experts(H, I, K, gate, up, down, orc.Q5_1, codes, deltas, sums, ids, want_intermediates=False, gate_type=orc.Q5_K)
+        assert np.array_equal(bits(r.rawdots), gold[f"format_layer_{seed}_rawdots_bits"]), seed
+    rng = np.random.default_rng(310)
+    vals = []
+    for width in mk.Q6K_WIDTHS:
+        w = orc.random_q6_k(rng, (1,), width)[0]
+        x = (rng.standard_normal((1, width)) * 3.0).astype(np.float32)
+        codes, deltas, sums, _ = orc.quantize_a8(x, tiny_rule=True)
+        vals.append(orc.q6k_down_row_a8(w, codes[0], deltas[0]))
+    assert np.array_equal(bits(np.array(vals, np.float32)), gold["q6k_down_rows_bits"])
+    for seed, n, rows in mk.RMSNORM_CASES:
+        rng = np.random.default_rng(seed)
+        x = (rng.standard_normal((rows, n)) * 2.0).astype(np.float32)
+        w = rng.standard_normal(n).astype(np.float32)
+        assert np.array_equal(bits(orc.rmsnorm_f32(x, w, 1e-6)), gold[f"rmsnorm_{seed}_bits"])
