@@ -974,9 +974,23 @@ inline void launch_plan(const uint32_t* routes, uint32_t experts, uint32_t assig
     plan_kernel<<<1, 1024, 0, st>>>(routes, experts, assignments, split, bound, large ? 0U : 1U, plan);
     if (large) plan_order_kernel<<<experts, 1024, 0, st>>>(routes, experts, assignments, plan);
 }
+// Decode batches of at most this many assignments (six tokens at top-8) run the 16-rows-per-wavefront sweep (q4k_quads.hpp),
+// with a 4-slot ring up to 16 assignments and a 2-slot ring above (every workgroup of the launch stays resident); measured
+// at hidden 2048 / ffn 768: faster than the 64-row sweep up to 48 assignments, slower at 64. Such a batch is planned one
+// assignment per item (the fused router's plan, and the staged plan with pieces of one).
+constexpr uint32_t kQuadMaxItems = 48;
+inline bool quad_sweep(const mi355_moe_weights& w, uint32_t rows) {
+    return rows <= kFusedMaxRows && rows * w.top_k <= kQuadMaxItems && w.experts > 1U;
+}
 inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     if (w.gate_type == MI355_TYPE_Q5_K) {
         project_q5k_kernel<<<dim3(w.ffn / 32U, umax), 256, 0, st>>>(w, r, rows * w.top_k);
+        return;
+    }
+    if (quad_sweep(w, rows)) {
+        const uint32_t items = rows * w.top_k;
+        if (items <= 16U) project_quad_kernel<4><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, r, items);
+        else project_quad_kernel<2><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, r, items);
         return;
     }
     if (dense_pairs_ok(w, rows) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
@@ -993,15 +1007,17 @@ inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uin
         else down_q6k_kernel<<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         return;
     }
+    if (quad_sweep(w, rows)) {
+        const uint32_t items = rows * w.top_k;
+        if (items <= 16U) down_quad_kernel<4><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
+        else down_quad_kernel<2><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
+        return;
+    }
     if (dense_pairs_ok(w, rows)) return launch_down_dense(w, r, rows, st);
     const dim3 grid(w.hidden / 64U, umax);
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
     else launch_down_nb<4>(w, r, rows, grid, st);
 }
-// Decode batches of at most this many assignments (six tokens at top-8) run the 16-rows-per-wavefront sweep (q4k_quads.hpp),
-// with a 4-slot ring up to 16 assignments and a 2-slot ring above (every workgroup of the launch stays resident); measured
-// at hidden 2048 / ffn 768: faster than the 64-row sweep up to 48 assignments, slower at 64.
-constexpr uint32_t kQuadMaxItems = 48;
 // An expert's assignments are cut into work items of at most `split` rows: a wave's instruction stream grows with every
 // activation row it serves while its weight stream does not, so wide items finish last; the second read of a split
 // expert's weights comes from the last-level cache. A dense matrix: every row shares one sweep.
@@ -1319,31 +1335,17 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     STRIX_LAUNCHED("moe layer router");
     // the fused router planned one item per assignment
     const uint32_t items = rows * wv.top_k;
-    if (items <= kQuadMaxItems && wv.experts > 1U) {
-        if (items <= 16U) {
-            if (wv.gate_type != MI355_TYPE_Q4_K) launch_project(wv, *r, rows, items, hs(stream));
-            else project_quad_kernel<4><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
-            if (wv.down_type != MI355_TYPE_Q4_K) launch_down(wv, *r, rows, items, hs(stream));
-            else down_quad_kernel<4><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
-        } else {
-            if (wv.gate_type != MI355_TYPE_Q4_K) launch_project(wv, *r, rows, items, hs(stream));
-            else project_quad_kernel<2><<<dim3(wv.ffn / 32U, items), 256, 0, hs(stream)>>>(wv, *r, items);
-            if (wv.down_type != MI355_TYPE_Q4_K) launch_down(wv, *r, rows, items, hs(stream));
-            else down_quad_kernel<2><<<dim3(wv.hidden / 64U, items), 256, 0, hs(stream)>>>(wv, *r, items);
-        }
-    } else {
-        launch_project(wv, *r, rows, items, hs(stream));
-        // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
-        // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
-        // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
-        if (wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
-            (wv.hidden / 64U) * rows <= compute_units()) {
-            down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, hs(stream)>>>(wv, *r, items, form);
-            STRIX_LAUNCHED("moe layer experts + combine");
-            return MI355_OK;
-        }
-        launch_down(wv, *r, rows, items, hs(stream));
+    launch_project(wv, *r, rows, items, hs(stream));
+    // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
+    // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
+    // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
+    if (!quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
+        (wv.hidden / 64U) * rows <= compute_units()) {
+        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, hs(stream)>>>(wv, *r, items, form);
+        STRIX_LAUNCHED("moe layer experts + combine");
+        return MI355_OK;
     }
+    launch_down(wv, *r, rows, items, hs(stream));
     STRIX_LAUNCHED("moe layer experts");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
