@@ -6,6 +6,7 @@
 
 #include <cmath>
 #include <cstdio>
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <string>
@@ -1029,10 +1030,18 @@ inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
     return plan_item_bound(w.experts, rows * w.top_k, plan_split(w, rows));
 }
 
+// compute units of the current device (0 if the runtime cannot say); remembered per device ordinal
 inline uint32_t compute_units() {
+    static std::atomic<uint32_t> known[64];
     int device = 0, cus = 0;
-    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
-    return cus > 0 ? static_cast<uint32_t>(cus) : 0U;
+    if (hipGetDevice(&device) != hipSuccess || device < 0) return 0;
+    if (device < 64) {
+        const uint32_t seen = known[device].load(std::memory_order_relaxed);
+        if (seen != 0) return seen;
+    }
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) return 0;
+    if (device < 64) known[device].store(static_cast<uint32_t>(cus), std::memory_order_relaxed);
+    return static_cast<uint32_t>(cus);
 }
 
 // ======================================================================================================== admission
@@ -1376,9 +1385,8 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     const uint32_t items_at = plan_items_at(wv.experts, assignments), order_at = plan_order_at(wv.experts), item_slots = (bound + 7U) / 8U * 8U;
     a.wa = wv.gate; a.wb = wv.up; a.expert_stride = wv.gate_expert_stride; a.row_stride = wv.gate_row_stride; a.k = wv.hidden; a.features = wv.ffn;
     // persistent workgroups, one per compute unit (the kernel's LDS use allows no second one)
-    int device = 0, cus = 256;
-    if (hipGetDevice(&device) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
-    const uint32_t resident = static_cast<uint32_t>(cus > 8 ? cus : 8) & ~7U;
+    const uint32_t cus = compute_units();
+    const uint32_t resident = (cus > 8U ? cus : 256U) & ~7U;
     a.tiles = wv.ffn / 64U; a.units = item_slots * a.tiles;
     if (wv.gate_type == MI355_TYPE_Q8_0) prefill_f16_kernel<0, 1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     else prefill_f16_kernel<0, 0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
