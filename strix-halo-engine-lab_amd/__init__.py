@@ -187,7 +187,7 @@ class MoeLayer:
 
     def __init__(self, hidden, ffn, experts, top_k, gate, up, down, max_rows, exp_kind=EXP_GFX1151, intermediates=False,
                  gate_expert_stride=0, gate_row_stride=0, down_expert_stride=0, down_row_stride=0, prefill_f16=False,
-                 gate_type=TYPE_Q4_K, down_type=TYPE_Q4_K):
+                 gate_type=TYPE_Q4_K, down_type=TYPE_Q4_K, output_stride=None):
         dev = gate.device
         self.hidden, self.ffn, self.experts, self.top_k, self.max_rows = hidden, ffn, experts, top_k, max_rows
         self.gate, self.up, self.down = gate, up, down
@@ -199,7 +199,8 @@ class MoeLayer:
         self.status, self.job_status = z(max_rows, torch.int32), z(4, torch.int32)
         self.down_codes, self.down_deltas, self.down_sums = z((n, ffn), torch.int8), z((n, ffn // 32), torch.float32), z((n, ffn // 32), torch.int32)
         self.rawdots = z((max_rows, top_k, hidden), torch.float32)
-        self.output = z((max_rows, hidden), torch.float32)
+        self.output_stride = output_stride or hidden          # floats between output rows (>= hidden)
+        self.output = z((max_rows, self.output_stride), torch.float32)[:, :hidden]
         self.gate_out = z((n, ffn), torch.float32) if intermediates else None
         self.up_out = z((n, ffn), torch.float32) if intermediates else None
         self.h_out = z((n, ffn), torch.float32) if intermediates else None
@@ -215,7 +216,7 @@ class MoeLayer:
                              self.codes.data_ptr(), self.deltas.data_ptr(), self.sums.data_ptr(), self.status.data_ptr(),
                              _p(self.gate_out).value or 0, _p(self.up_out).value or 0, _p(self.h_out).value or 0,
                              self.down_codes.data_ptr(), self.down_deltas.data_ptr(), self.down_sums.data_ptr(),
-                             self.rawdots.data_ptr(), 0 if base is None else base.data_ptr(), self.output.data_ptr(), self.hidden,
+                             self.rawdots.data_ptr(), 0 if base is None else base.data_ptr(), self.output.data_ptr(), self.output_stride,
                              self.plan.data_ptr(), self.job_status.data_ptr(), _p(self.h_f16).value or 0)
 
     def run(self, x, ids, weights, base=None, combine=COMBINE_FMA_SLOT):

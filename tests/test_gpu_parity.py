@@ -417,6 +417,35 @@ def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine):
     assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine(combine, w_n, ids_n, raw.cpu().numpy(), base=base.cpu().numpy())))
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T", [2, 8, 20])
+def test_layer_entry_input_kinds_and_output_stride(strix, dtype, T):
+    """fp32 and bf16 input rows (the fp16 kind is the default of the other tests) through the whole-layer entry - quad sweep,
+    row sweep with the fused down + combine, and the staged path of a larger batch - with output rows 64 floats apart from
+    their width: router ids / weights and the output against the oracle on the same values, bit for bit; the padding between
+    output rows is never written."""
+    E, H, I, K = 16, 512, 256, 4
+    rng = np.random.default_rng(5 + T)
+    gate, up, down = make_layer(rng, H, I, E)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    xt = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(getattr(torch, dtype))
+    x32 = xt.to(torch.float32).numpy()                          # the values the device sees, exactly
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, output_stride=H + 64)
+    full = layer.output.as_strided((T, H + 64), (H + 64, 1))
+    full.fill_(-7.0)
+    y, ids, wts, _ = layer.run_layer(xt.cuda(), dev(wr))
+    ids_ref, w_ref, _, _ = orc.route(x32, wr, K)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    c, d, s, _ = orc.quantize_a8(x32)
+    assert np.array_equal(layer.codes[:T].cpu().numpy(), c) and np.array_equal(bits(layer.deltas[:T].cpu().numpy()), bits(d))
+    raw_dev = layer.rawdots[:T].cpu().numpy()
+    assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine(0, w_ref, ids_ref, raw_dev)))
+    ref = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref)
+    a, e = rel_err(y.cpu().numpy(), orc.combine(0, w_ref, ids_ref, ref.rawdots))
+    assert a < TOL_F16 and e < TOL_F16
+    assert bool((full[:, H:] == -7.0).all()) and int(layer.status.sum()) == 0
+
+
 # ------------------------------------------------------------------------------------------- the expert plan
 @pytest.mark.parametrize("E,K,T", [(6, 3, 5), (128, 8, 8), (128, 8, 16), (16, 4, 40), (1024, 16, 16), (1, 1, 7), (256, 8, 500), (3, 2, 300)])
 def test_expert_plan_words(strix, E, K, T):
