@@ -142,7 +142,7 @@ typedef struct mi355_moe_weights {
     uint32_t ffn;         /* intermediate rows computed by this call (a TP rank: its share), multiple of 256 */
     uint32_t experts, top_k;
     uint32_t gate_type, down_type;                    /* gate/up MI355_TYPE_Q4_K or Q5_K; down Q4_K, Q8_0, Q5_1 or Q6_K
-                                                         (mi355_moe_enqueue_prefill_f16: Q4_K or Q8_0 for either) */
+                                                         (mi355_moe_enqueue_prefill_f16: Q4_K, Q5_K or Q8_0 for either) */
     const uint8_t *gate, *up, *down;                  /* GGUF order [experts][ffn][hidden/256], [experts][hidden][ffn/256 or ffn/32 blocks] */
     uint64_t gate_expert_stride, gate_row_stride;     /* bytes; 0 = dense GGUF order. 16-byte multiples (Q6_K down: 2) */
     uint64_t down_expert_stride, down_row_stride;     /* a TP rank reads the first ffn/256 blocks of each down row */
@@ -206,8 +206,9 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* policy, const float* r
  * entry point. Runs: status clear + route validation, expert plan, gate/up + SwiGLU, down, ordered combine.
  * Requires input_kind = MI355_INPUT_F16, rows->h_f16 (see mi355_moe_prefill_f16_workspace_bytes), hidden % 256 == 0,
  * ffn % 256 == 0.
- * gate_type and down_type may each be MI355_TYPE_Q4_K or MI355_TYPE_Q8_0 here (w = d * code, src/ggml_dequant.cpp:84-87: the
- * codes are the exact operands, d is applied in fp32 to every block's product). An always-on shared expert
+ * gate_type and down_type may each be MI355_TYPE_Q4_K, MI355_TYPE_Q5_K (the nibble plus a fifth bit: sc * q stays an exact
+ * fp16 integer) or MI355_TYPE_Q8_0 here (w = d * code, src/ggml_dequant.cpp:84-87: the codes are the exact operands, d is
+ * applied in fp32 to every block's product). An always-on shared expert
  * (src/hip_shared_expert_launcher.hip) is a layer with experts = top_k = 1, every route id 0 and every route weight 1; its
  * output is the next call's rows->base. A row whose h leaves the fp16 range is reported as MI355_STATUS_NONFINITE_PROJECTION. */
 int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, uint32_t combine_form,

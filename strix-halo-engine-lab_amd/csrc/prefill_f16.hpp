@@ -137,10 +137,12 @@ __device__ __forceinline__ void copy16_to_lds(const uint8_t* src, pf_lds* lds_ba
 __device__ __forceinline__ uint32_t pf_at(uint32_t row, uint32_t piece) { return row * 128U + ((piece ^ ((row >> 1) & 7U)) << 4); }
 
 // the loader's per-step global operands
-struct PfRaw { u32x4 hd, qs[4]; };           // one super-block of a weight row: header and the thread's 16 quant bytes of its four steps
+struct PfRaw { u32x4 hd, qs[4], fifth; };    // one super-block of a weight row: header, the thread's 16 quant bytes of its four steps, Q5_K: their fifth bits
 struct PfRaw8 { u32x4 a, b; uint32_t c; };   // one Q8_0 block of a weight row as nine aligned words
 
-// FMT 0: Q4_K weights, FMT 1: Q8_0 weights (one fp16 d per 32 codes and no minimum, src/ggml_dequant.cpp:84-87: the codes
+// FMT 0: Q4_K weights; FMT 2: Q5_K weights (the same block with 32 fifth-bit bytes after the factors, bit j of byte k for
+// element k of sub-block j: q = nibble | bit << 4, sc q <= 1953 is still an exact fp16 integer); FMT 1: Q8_0 weights (one
+// fp16 d per 32 codes and no minimum, src/ggml_dequant.cpp:84-87: the codes
 // are exact fp16 integers, a step is two blocks, and d is applied in fp32 to the product of each block).
 template <int MODE, int FMT>
 __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, uint32_t items_at, uint32_t order_at) {
@@ -171,7 +173,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
     if (count == 0) continue;
     const uint32_t t = loader ? threadIdx.x : threadIdx.x - 256U, lane = t & 63U, wave = t >> 6;      // index within the role
     const uint32_t m0 = tile * (MODE == 0 ? 64U : 128U);
-    const uint32_t steps = a.k / kPfStep, blocks = a.k / 256U, steps8 = FMT == 0 ? (steps + 7U) & ~7U : steps;   // K is a multiple of 256: steps of 4
+    const uint32_t steps = a.k / kPfStep, blocks = a.k / 256U, steps8 = FMT != 1 ? (steps + 7U) & ~7U : steps;   // K is a multiple of 256: steps of 4
     const size_t sum_row = pf_sum_row_bytes(a.k);
 
     if (loader) {
@@ -283,9 +285,15 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
         };
         // 5 operations: a super-block's header and the thread's 16 quant bytes of each of its four steps, issued together
         // (they touch the same two or three cache lines)
+        constexpr uint32_t kBlockBytes = FMT == 2 ? 176U : 144U, kQuantsAt = FMT == 2 ? 48U : 16U;
+        constexpr uint32_t kFetchOps = FMT == 2 ? 6U : 5U;                 // operations of one fetch (Q5_K: + the fifth bits)
         const auto fetch = [&](uint32_t b, PfRaw& r) {
-            const uint8_t* blk = wrow + static_cast<size_t>(b < last_block ? b : last_block) * 144U;
-            const uint8_t* quants = blk + 16U + 16U * half;
+            const uint8_t* blk = wrow + static_cast<size_t>(b < last_block ? b : last_block) * kBlockBytes;
+            const uint8_t* quants = blk + kQuantsAt + 16U * half;
+            if (FMT == 2) {
+                const uint8_t* bits = blk + 16U + 16U * half;              // fifth bits of elements 16 half .. + 16 of every sub-block
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.fifth) : "v"(bits) : "memory");
+            }
             asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.hd) : "v"(blk) : "memory");
             asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.qs[0]) : "v"(quants) : "memory");
             asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=v"(r.qs[1]) : "v"(quants) : "memory");
@@ -295,10 +303,11 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
         // the two constants of the nibble expansion, kept in registers so that mask-and-merge is one v_and_or_b32
         // (as immediates the instruction cannot encode them and the compiler emits two)
         uint32_t nibble_mask, magic_1024;
-        asm volatile("s_mov_b32 %0, 0x000f000f" : "=s"(nibble_mask));
+        if (FMT == 2) asm volatile("s_mov_b32 %0, 0x001f001f" : "=s"(nibble_mask));
+        else asm volatile("s_mov_b32 %0, 0x000f000f" : "=s"(nibble_mask));
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic_1024));
         // (p = step % 4 and the step's parity are compile-time constants at every call)
-        const auto stage_weights = [&](uint32_t b, uint32_t p, const u32x4& hd, const u32x4& quants) {
+        const auto stage_weights = [&](uint32_t b, uint32_t p, const u32x4& hd, const u32x4& quants, const u32x4& fifth) {
             const uint32_t sh0 = 16U * (p & 1U), sh1 = sh0 + 8U;
             const uint32_t fa0 = (hd.y >> sh0) & 255U, fc0 = (hd.w >> sh0) & 255U;
             const uint32_t fa1 = (hd.y >> sh1) & 255U, fc1 = (hd.w >> sh1) & 255U;
@@ -309,6 +318,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             const _Float16 n0 = static_cast<_Float16>(-1024.0F * static_cast<float>(s0)), n1 = static_cast<_Float16>(-1024.0F * static_cast<float>(s1));
             const half2v mul0 = {c0, c0}, add0 = {n0, n0}, mul1 = {c1, c1}, add1 = {n1, n1};
             const uint32_t qs[4] = {quants.x, quants.y, quants.z, quants.w};
+            const uint32_t q5[4] = {fifth.x, fifth.y, fifth.z, fifth.w};
             uint32_t lo[8], hi[8];
             const auto scaled = [&](uint32_t bytes, uint32_t sel, half2v mul, half2v add) {
                 // two nibbles -> (1024 + q) as fp16 bit patterns -> sc q
@@ -317,7 +327,11 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             };
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const uint32_t w = qs[i], w4 = w >> 4;
+                uint32_t w = qs[i], w4 = w >> 4;
+                if (FMT == 2) {      // nibble | fifth bit << 4 per byte (sub-block 2p: bit 2p of the fifth-bit byte, 2p + 1: the next)
+                    w = (w & 0x0f0f0f0fU) | (((q5[i] >> (2U * p)) & 0x01010101U) << 4);
+                    w4 = (w4 & 0x0f0f0f0fU) | (((q5[i] >> (2U * p + 1U)) & 0x01010101U) << 4);
+                }
                 lo[2 * i] = scaled(w, 0x0c010c00U, mul0, add0); lo[2 * i + 1] = scaled(w, 0x0c030c02U, mul0, add0);
                 hi[2 * i] = scaled(w4, 0x0c010c00U, mul1, add1); hi[2 * i + 1] = scaled(w4, 0x0c030c02U, mul1, add1);
             }
@@ -370,9 +384,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
         copy_tokens(1, tok_stage[1]);
         fetch(1, raw[1]);
         copy_tokens(2, tok_stage[2]);
-        // younger than the first token copy: 4 + 5 + 4; the first fetch is older still
-        asm volatile("s_waitcnt vmcnt(13)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]) : : "memory");
-        stage_weights(0, 0, raw[0].hd, raw[0].qs[0]);
+        // younger than the first token copy: 4 + a fetch + 4; the first fetch is older still
+        if (FMT == 2) asm volatile("s_waitcnt vmcnt(14)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]), "+v"(raw[0].fifth) : : "memory");
+        else asm volatile("s_waitcnt vmcnt(13)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]) : : "memory");
+        stage_weights(0, 0, raw[0].hd, raw[0].qs[0], raw[0].fifth);
         pf_barrier();
         for (uint32_t s0 = 0; s0 < steps8; s0 += 8U) {
             const uint32_t b0 = s0 >> 2;
@@ -382,20 +397,27 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                 if (u == 0) copy_sums((s >> 3) + 1U);
                 copy_tokens(s + kPfTokenAhead, tok_stage[(u + kPfTokenAhead) & 3U]);
                 // the slot fetched at u == 6 of the previous iteration (u == 2 of this one): younger operations
-                // 4 + 6 + 4 + 9 + 4 = 27 (4 + 4 + 4 + 9 + 4 = 25)
-                if (u == 3U) asm volatile("s_waitcnt vmcnt(27)" : "+v"(raw[1].hd), "+v"(raw[1].qs[0]), "+v"(raw[1].qs[1]), "+v"(raw[1].qs[2]), "+v"(raw[1].qs[3]) : : "memory");
-                if (u == 7U) asm volatile("s_waitcnt vmcnt(25)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]) : : "memory");
-                if (s < last) stage_weights((s + 1U) >> 2, (u + 1U) & 3U, raw[((u + 1U) >> 2) & 1U].hd, raw[((u + 1U) >> 2) & 1U].qs[(u + 1U) & 3U]);
+                // 4 + 6 + 4 + (4 + a fetch) + 4 = 27 with 5 operations per fetch (4 + 4 + 4 + (4 + a fetch) + 4 = 25); Q5_K: one more
+                if (FMT == 2) {
+                    if (u == 3U) asm volatile("s_waitcnt vmcnt(28)" : "+v"(raw[1].hd), "+v"(raw[1].qs[0]), "+v"(raw[1].qs[1]), "+v"(raw[1].qs[2]), "+v"(raw[1].qs[3]), "+v"(raw[1].fifth) : : "memory");
+                    if (u == 7U) asm volatile("s_waitcnt vmcnt(26)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]), "+v"(raw[0].fifth) : : "memory");
+                } else {
+                    if (u == 3U) asm volatile("s_waitcnt vmcnt(27)" : "+v"(raw[1].hd), "+v"(raw[1].qs[0]), "+v"(raw[1].qs[1]), "+v"(raw[1].qs[2]), "+v"(raw[1].qs[3]) : : "memory");
+                    if (u == 7U) asm volatile("s_waitcnt vmcnt(25)" : "+v"(raw[0].hd), "+v"(raw[0].qs[0]), "+v"(raw[0].qs[1]), "+v"(raw[0].qs[2]), "+v"(raw[0].qs[3]) : : "memory");
+                }
+                if (s < last) stage_weights((s + 1U) >> 2, (u + 1U) & 3U, raw[((u + 1U) >> 2) & 1U].hd, raw[((u + 1U) >> 2) & 1U].qs[(u + 1U) & 3U], raw[((u + 1U) >> 2) & 1U].fifth);
                 if (u == 2U) fetch(b0 + 2U, raw[0]);
                 if (u == 6U) fetch(b0 + 3U, raw[1]);
                 // the token copy of step s + 1 was issued in step s - 2; younger operations: a fetch in that step, then
                 // the whole of steps s - 1 and s
-                const uint32_t per_step[8] = {6, 4, 9, 4, 4, 4, 9, 4}, fetch_after[8] = {0, 0, 5, 0, 0, 0, 5, 0};
+                const uint32_t per_step[8] = {6, 4, 4 + kFetchOps, 4, 4, 4, 4 + kFetchOps, 4}, fetch_after[8] = {0, 0, kFetchOps, 0, 0, 0, kFetchOps, 0};
                 switch (fetch_after[(u + 6U) & 7U] + per_step[(u + 7U) & 7U] + per_step[u]) {   // a constant once the loop is unrolled
                 case 8: wait_copies<8>(); break;
                 case 10: wait_copies<10>(); break;
                 case 13: wait_copies<13>(); break;
+                case 14: wait_copies<14>(); break;
                 case 15: wait_copies<15>(); break;
+                case 16: wait_copies<16>(); break;
                 default: wait_copies<0>(); break;
                 }
                 pf_barrier();
@@ -458,7 +480,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                     for (uint32_t i = 0; i < NT; ++i)
 #pragma unroll
                         for (uint32_t n = 0; n < 2U; ++n) {
-                            if ((FMT == 1 && (ks & 1U) == 0) || (FMT == 0 && p == 0 && ks == 0)) {   // first MFMA of a block's product: it starts from zero
+                            if ((FMT == 1 && (ks & 1U) == 0) || (FMT != 1 && p == 0 && ks == 0)) {   // first MFMA of a block's product: it starts from zero
                                 const floatx16 zero = {0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F, 0.0F};
                                 part[i][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks & 1U][i], w[ks & 1U][n], zero, 0, 0, 0);
                             } else {
@@ -478,7 +500,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             };
             if (live_tiles >= TT) k_steps(std::integral_constant<uint32_t, TT>{});
             else if (live_tiles == 1U) k_steps(std::integral_constant<uint32_t, 1>{});
-            if (FMT == 0 && p == 3U) {
+            if (FMT != 1 && p == 3U) {
                 // end of a super-block: running sum += d * P (the next super-block's first MFMA starts P from zero)
                 const uint32_t b = s >> 2;
                 const float d[2] = {d_scale[b & 1U][64U * wr + l31], d_scale[b & 1U][64U * wr + 32U + l31]};

@@ -1055,18 +1055,18 @@ inline uint64_t moe_row_bytes(uint32_t type, uint32_t k) {
 }
 
 // Tensor formats by arithmetic class. Integer-dot entries: gate/up Q4_K or Q5_K; down Q4_K, the host executor's Q8_0 /
-// Q5_1 (src/cpu/core/routed_expert.hpp:27-28) or Q6_K (src/moe_a8_down_contract.cpp:147). The matrix-core prefill form: Q4_K or Q8_0 for either (a dense shared expert is
-// experts = top_k = 1). The merge reads no weights.
+// Q5_1 (src/cpu/core/routed_expert.hpp:27-28) or Q6_K (src/moe_a8_down_contract.cpp:147). The matrix-core prefill form: Q4_K, Q5_K or Q8_0 for either (a dense shared
+// expert is experts = top_k = 1). The merge reads no weights.
 enum MoeClass { kIntegerClass, kPrefillClass, kAnyClass };
 int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, MoeClass cls = kIntegerClass) {
     STRIX_REQUIRE(w && r, "moe: null weights or rows");
     STRIX_REQUIRE(rows > 0, "moe: rows must be positive");
     const bool gate_q8 = w->gate_type == MI355_TYPE_Q8_0, down_q8 = w->down_type == MI355_TYPE_Q8_0;
     const bool down_q51 = w->down_type == MI355_TYPE_Q5_1 || w->down_type == MI355_TYPE_Q6_K;      // integer class only
-    STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || (gate_q8 && cls != kIntegerClass) || (w->gate_type == MI355_TYPE_Q5_K && cls != kPrefillClass),
-                  cls == kPrefillClass ? "moe prefill: gate/up weights must be Q4_K (type 12) or Q8_0 (type 8)" : "moe: gate/up weights must be Q4_K (type 12) or Q5_K (type 13)");
-    if (!(w->down_type == MI355_TYPE_Q4_K || down_q8 || (down_q51 && cls != kPrefillClass)))
-        return fail(MI355_E_UNSUPPORTED, cls == kPrefillClass ? "moe prefill: down weights must be Q4_K (type 12) or Q8_0 (type 8)"
+    STRIX_REQUIRE(w->gate_type == MI355_TYPE_Q4_K || w->gate_type == MI355_TYPE_Q5_K || (gate_q8 && cls != kIntegerClass),
+                  cls == kPrefillClass ? "moe prefill: gate/up weights must be Q4_K (type 12), Q5_K (type 13) or Q8_0 (type 8)" : "moe: gate/up weights must be Q4_K (type 12) or Q5_K (type 13)");
+    if (!(w->down_type == MI355_TYPE_Q4_K || down_q8 || (down_q51 && cls != kPrefillClass) || (w->down_type == MI355_TYPE_Q5_K && cls != kIntegerClass)))
+        return fail(MI355_E_UNSUPPORTED, cls == kPrefillClass ? "moe prefill: down weights must be Q4_K (type 12), Q5_K (type 13) or Q8_0 (type 8)"
                                                                : "moe: down weights must be Q4_K (type 12), Q8_0 (type 8), Q5_1 (type 7) or Q6_K (type 14)");
     STRIX_REQUIRE(w->hidden >= 256 && w->hidden % 256U == 0, "moe: hidden must be a positive multiple of 256");
     STRIX_REQUIRE(w->ffn >= 256 && w->ffn % 256U == 0, "moe: ffn must be a positive multiple of 256");
@@ -1389,10 +1389,12 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     const uint32_t resident = (cus > 8U ? cus : 256U) & ~7U;
     a.tiles = wv.ffn / 64U; a.units = item_slots * a.tiles;
     if (wv.gate_type == MI355_TYPE_Q8_0) prefill_f16_kernel<0, 1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    else if (wv.gate_type == MI355_TYPE_Q5_K) prefill_f16_kernel<0, 2><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     else prefill_f16_kernel<0, 0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     a.wa = wv.down; a.wb = nullptr; a.expert_stride = wv.down_expert_stride; a.row_stride = wv.down_row_stride; a.k = wv.ffn; a.features = wv.hidden;
     a.tiles = wv.hidden / 128U; a.units = item_slots * a.tiles;
     if (wv.down_type == MI355_TYPE_Q8_0) prefill_f16_kernel<1, 1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    else if (wv.down_type == MI355_TYPE_Q5_K) prefill_f16_kernel<1, 2><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     else prefill_f16_kernel<1, 0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
     STRIX_LAUNCHED("moe prefill f16");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);

@@ -145,6 +145,12 @@ def float_to_half(value):
 
 def dequant_rows(qtype, packed, elements):
     """packed: uint8 [rows][row_bytes] -> float32 [rows][elements]."""
+    if qtype == Q5_K:
+        return dequant_q5_k_rows(packed, elements)
+    if qtype == Q5_1:
+        return dequant_q5_1_rows(packed, elements)
+    if qtype == Q6_K:
+        return dequant_q6_k_rows(packed, elements)
     packed = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1, row_bytes(qtype, elements))
     out = np.empty((packed.shape[0], elements), np.float32)
     fn = lib().orc_dequant_q8_0_row if qtype == Q8_0 else lib().orc_dequant_q4_k_row
@@ -211,6 +217,38 @@ def q5k_row_a8(wrow, codes, deltas, sums):
     wrow = np.ascontiguousarray(wrow, np.uint8)
     return np.float32(lib().orc_q5k_row_a8(_ptr(wrow, u8p), C.c_uint32(wrow.size // Q5_K_BLOCK), _ptr(codes, i8p), _ptr(deltas, f32p),
                                            _ptr(sums, i32p)))
+
+
+def quantize_q5_k_rows(x):
+    """A plain min / max Q5_K writer for tests (the reference has none): float32 [..., width] -> uint8 [..., width / 256 * 176].
+    Per sub-block scale = (max - min0) / 31 and offset = -min0 (min0 = min(min, 0)), d = max scale / 63, dmin = max offset / 63
+    as fp16, 6-bit factors and 5-bit codes by round-to-nearest against the fp16 values; packed as the decoders expect."""
+    x = np.ascontiguousarray(x, np.float32)
+    lead, width = x.shape[:-1], x.shape[-1]
+    v = x.reshape(-1, width // 256, 8, 32).astype(np.float64)
+    mn = np.minimum(v.min(-1), 0.0)
+    scale = (v.max(-1) - mn) / 31.0
+    d = (scale.max(-1) / 63.0).astype(np.float16)
+    dm = ((-mn).max(-1) / 63.0).astype(np.float16)
+    d64, dm64 = d.astype(np.float64), dm.astype(np.float64)
+    sc = np.where(d64[..., None] > 0, np.rint(scale / np.where(d64 > 0, d64, 1.0)[..., None]), 0).clip(0, 63).astype(np.uint32)
+    m = np.where(dm64[..., None] > 0, np.rint(-mn / np.where(dm64 > 0, dm64, 1.0)[..., None]), 0).clip(0, 63).astype(np.uint32)
+    step = d64[..., None] * sc
+    q = np.where(step[..., None] > 0, np.rint((v + (dm64[..., None] * m)[..., None]) / np.where(step > 0, step, 1.0)[..., None]), 0).clip(0, 31).astype(np.uint32)
+    out = np.zeros(v.shape[:2] + (Q5_K_BLOCK,), np.uint8)
+    out[..., 0:2] = d.view(np.uint8).reshape(d.shape + (2,))
+    out[..., 2:4] = dm.view(np.uint8).reshape(dm.shape + (2,))
+    for j in range(4):
+        out[..., 4 + j] = (sc[..., j] & 63) | ((sc[..., j + 4] >> 4) << 6)
+        out[..., 8 + j] = (m[..., j] & 63) | ((m[..., j + 4] >> 4) << 6)
+        out[..., 12 + j] = (sc[..., j + 4] & 15) | ((m[..., j + 4] & 15) << 4)
+    fifth = np.zeros(v.shape[:2] + (32,), np.uint32)
+    for j in range(8):
+        fifth |= (q[..., j, :] >> 4) << j
+    out[..., 16:48] = fifth.astype(np.uint8)
+    for p in range(4):
+        out[..., 48 + 32 * p: 80 + 32 * p] = ((q[..., 2 * p, :] & 15) | ((q[..., 2 * p + 1, :] & 15) << 4)).astype(np.uint8)
+    return out.reshape(lead + (width // 256 * Q5_K_BLOCK,))
 
 
 def random_q5_k(rng, shape_rows, width):

@@ -64,14 +64,17 @@ def test_expert_tensor_format_admission_on_the_host(lib):
     for entry in (lib.mi355_moe_enqueue, lib.mi355_moe_enqueue_prefill_f16):
         assert entry(C.byref(weights(14, 12)), C.byref(rows), 4, 0, None) == -1 and b"gate/up" in lib.mi355_last_error()
         assert entry(C.byref(weights(12, 2)), C.byref(rows), 4, 0, None) == -2 and b"down" in lib.mi355_last_error()
-    # per class: Q8_0 gate/up only in the prefill form; Q5_K gate/up and Q5_1 / Q6_K down only in the integer class
+    # per class: Q8_0 gate/up and Q5_K down only in the prefill form; Q5_1 / Q6_K down only in the integer class
     assert lib.mi355_moe_enqueue(C.byref(weights(8, 8)), C.byref(rows), 4, 0, None) == -1 and b"gate/up" in lib.mi355_last_error()
-    assert lib.mi355_moe_enqueue_prefill_f16(C.byref(weights(13, 12)), C.byref(rows), 4, 0, None) == -1 and b"gate/up" in lib.mi355_last_error()
+    assert lib.mi355_moe_enqueue(C.byref(weights(12, 13)), C.byref(rows), 4, 0, None) == -2          # Q5_K down: prefill form only
     for down in (7, 14):
         assert lib.mi355_moe_enqueue_prefill_f16(C.byref(weights(12, down)), C.byref(rows), 4, 0, None) == -2
     # admitted formats get as far as the pointer checks
     for gate, down in ((12, 12), (13, 8), (12, 7), (13, 14)):
         assert lib.mi355_moe_enqueue(C.byref(weights(gate, down)), C.byref(rows), 4, 0, None) == -1
+        assert b"weight pointers" in lib.mi355_last_error()
+    for gate, down in ((12, 12), (13, 13), (8, 8), (13, 8), (8, 12)):
+        assert lib.mi355_moe_enqueue_prefill_f16(C.byref(weights(gate, down)), C.byref(rows), 4, 0, None) == -1
         assert b"weight pointers" in lib.mi355_last_error()
     # more plan items than a launch dimension holds
     assert lib.mi355_moe_enqueue(C.byref(weights(12, 12, experts=256, top_k=16)), C.byref(rows), 65535, 0, None) == -1

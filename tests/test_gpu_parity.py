@@ -673,14 +673,19 @@ def random_q8_0(rng, shape_rows, width):
     (768, 1280, 3, 2, 150, orc.Q8_0, orc.Q8_0, False),
     (256, 512, 1, 1, 129, orc.Q8_0, orc.Q8_0, True),
     (512, 512, 4, 2, 200, orc.Q8_0, orc.Q4_K, False),
-    (512, 256, 4, 2, 90, orc.Q4_K, orc.Q8_0, False)])
+    (512, 256, 4, 2, 90, orc.Q4_K, orc.Q8_0, False),
+    (512, 256, 4, 2, 300, orc.Q5_K, orc.Q4_K, False),       # Q5_K (fifth bits in use): even, odd and single super-block counts
+    (768, 1280, 3, 2, 150, orc.Q5_K, orc.Q5_K, False),
+    (256, 512, 5, 1, 129, orc.Q4_K, orc.Q5_K, False)])
 def test_prefill_f16_mfma_q8_0_tensors(strix, H, I, E, K, T, gate_type, down_type, random_bytes):
     """The matrix-core prefill form with Q8_0 expert tensors (the always-on shared expert is experts = top_k = 1 with weight 1)
     against the exact-weight product, tolerance 2e-3 as for Q4_K: max abs error over the output rms, and elementwise on the
     outputs of at least rms size, for the unweighted down outputs and the combined output."""
     rng = np.random.default_rng(7 * H + T)
     def tensor(qtype, rows, width):
-        if random_bytes:
+        if qtype == orc.Q5_K:      # written from normal weights (random bytes give a heavy-tailed h whose fp16 rounding alone exceeds the bar)
+            return orc.quantize_q5_k_rows((rng.standard_normal((E, rows, width)) * 0.02).astype(np.float32))
+        if random_bytes and qtype == orc.Q8_0:
             return random_q8_0(rng, (E, rows), width)
         return orc.quantize_rows(qtype, (rng.standard_normal((E, rows, width)) * 0.02).astype(np.float32))
     gate, up, down = tensor(gate_type, I, H), tensor(gate_type, I, H), tensor(down_type, H, I)

@@ -570,6 +570,18 @@ def test_routed_experts_against_double_precision_dequant_reference(down_type):
     assert np.array_equal(bits(r1.rawdots), bits(r.rawdots)) and np.array_equal(r1.h_codes, r.h_codes)
 
 
+def test_q5k_test_writer_round_trip():
+    """The tests' own Q5_K writer: decoding what it wrote returns the input to within half a code step, and the fifth bits are
+    in use (codes above 15 exist)."""
+    rng = np.random.default_rng(17)
+    x = (rng.standard_normal((6, 1024)) * 0.02).astype(np.float32)
+    packed = orc.quantize_q5_k_rows(x)
+    assert packed.shape == (6, 4 * 176) and packed.reshape(6, 4, 176)[..., 16:48].any()
+    back = orc.dequant_q5_k_rows(packed, 1024)
+    step = (x.reshape(6, 4, 8, 32).max(-1) - np.minimum(x.reshape(6, 4, 8, 32).min(-1), 0)) / 31
+    assert np.max(np.abs(back - x).reshape(6, 4, 8, 32) / (step[..., None] + 1e-12)) < 1.6
+
+
 def test_q5k_gate_rows_against_double_precision_dequant_reference():
     """Brute force for the Q5_K gate/up row: dequantise with a numpy statement of the block layout, sum in double."""
     rng = np.random.default_rng(15)
