@@ -1024,7 +1024,13 @@ inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uin
 // expert's weights comes from the last-level cache. A dense matrix: every row shares one sweep.
 inline uint32_t plan_split(const mi355_moe_weights& w, uint32_t rows) {
     if (w.experts == 1U) return 8;
-    return rows <= kFusedMaxRows ? 1U : 4U;
+    if (rows > kFusedMaxRows) return 4U;
+    if (quad_sweep(w, rows)) return 1U;       // the 16-rows-per-wavefront sweep serves one assignment per item
+    // decode batches: one item per assignment while an expert's gate + up rows are a few MB (the second sweep of an expert
+    // that two rows chose is a cache hit and the short instruction streams finish sooner); larger experts are swept once
+    // for every two rows that chose them (hidden 6144, ffn 1280, 16 rows: 384 -> 351 us)
+    const uint64_t sweep_bytes = 2ULL * w.ffn * (w.hidden / 256U) * kQ4kBlock;
+    return sweep_bytes >= (4ULL << 20) ? 2U : 1U;
 }
 inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
     return plan_item_bound(w.experts, rows * w.top_k, plan_split(w, rows));
@@ -1331,7 +1337,7 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     float* weights = const_cast<float*>(r->route_weights);
     if (const int32_t rc = check_route(p, r->input, r->input_kind, wv.hidden, r->input_stride, router_weight, ids, weights, scores)) return rc;
     STRIX_REQUIRE(p->experts == wv.experts && p->top_k == wv.top_k, "moe layer: router policy and expert tensors disagree on experts / top_k");
-    if (rows > kFusedMaxRows) {      // large batches: router, then the staged prologue / plan
+    if (rows > kFusedMaxRows || plan_split(wv, rows) != 1U) {      // large batches: router, then the staged prologue / plan
         if (const int32_t rc = mi355_moe_route(p, r->input, r->input_kind, rows, wv.hidden, r->input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
         return mi355_moe_enqueue(w, r, rows, form, stream);
     }

@@ -736,7 +736,10 @@ def test_prefill_f16_h_beyond_fp16_fails_closed(strix):
     assert torch.equal(again, want) and int(layer.status.sum()) == 0
 
 
-@pytest.mark.parametrize("H,I,E,K,T", [(512, 256, 6, 2, 300), (1024, 512, 12, 4, 77), (256, 256, 3, 1, 129), (768, 1280, 5, 2, 150)])
+@pytest.mark.parametrize("H,I,E,K,T", [(512, 256, 6, 2, 300), (1024, 512, 12, 4, 77), (256, 256, 3, 1, 129), (768, 1280, 5, 2, 150),
+                                       # many experts chosen by few rows each (plan items of 1 to 32 rows: token tiles with no
+                                       # live row beside one that has some), 3 / 5 / 8 super-blocks per row
+                                       (768, 1280, 16, 4, 60), (512, 256, 40, 8, 33), (256, 256, 24, 2, 9), (2048, 768, 64, 8, 100)])
 def test_prefill_f16_mfma_matches_exact_weight_product(strix, H, I, E, K, T):
     """The fp16 MFMA prefill form against the exact-weight product: tolerance 2e-3 (fp16 activations), both as max abs
     error over the output rms and elementwise on the outputs of at least rms size; the gate / up / down tiles are checked
