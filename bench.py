@@ -229,6 +229,18 @@ def extra_configs(strix, torch, steps, warmup):
     """BASELINE configs 1, 2, 4, 5 on synthetic full-entropy blocks; HBM-bound ones rotate over enough weight sets to stay cold."""
     gen = torch.Generator(device="cuda").manual_seed(11)
     out = {}
+    # what the machine gives vendor kernels (not this library's code): a 1 GiB device copy and a large fp16 GEMM, as the
+    # practical ceilings next to the published peaks the fractions below are quoted against
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    sec = time_steps(torch, lambda i: dst.copy_(src), 10, 3)
+    out["probe_device_copy_1GiB"] = {"GBps_read_plus_write": 2.0 * src.numel() / sec / 1e9, "frac_of_hbm_peak": 2.0 * src.numel() / sec / 1e9 / HBM_PEAK_GBPS}
+    del src, dst
+    ga = torch.randn((8192, 8192), device="cuda", generator=gen).to(torch.float16)
+    gb = torch.randn((8192, 8192), device="cuda", generator=gen).to(torch.float16)
+    sec = time_steps(torch, lambda i: torch.matmul(ga, gb), 10, 3)
+    out["probe_fp16_gemm_8192_vendor_library"] = {"TFLOPs": 2.0 * 8192 ** 3 / sec / 1e12, "frac_of_fp16_mfma_peak": 2.0 * 8192 ** 3 / sec / 2.5e15}
+    del ga, gb
     # config 1: Q8_0 4096 x 4096 GEMV, one fp32 row
     n = 4096
     sets = []
