@@ -191,7 +191,10 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights*, const mi355_moe_rows*, uint3
  * and weights), scores is a [rows][experts] workspace and output. For rows <= 16 the router, the A8 prologue and the expert
  * plan run in ONE launch (the workgroup that completes a row's logits also selects its experts and writes the row's work
  * items: one item per assignment, in assignment order; the CSR fields of the plan are not written), followed by project,
- * down and merge (down and merge share a launch when the batch is small enough for every workgroup to be resident). rows->plan must be zero-filled once when it is allocated; every launch leaves its ticket words zero, and
+ * down and merge (down and merge share a launch when the batch is small enough for every workgroup to be resident). Where an
+ * expert's gate + up rows exceed 4 MB (and the batch is too large for the 16-rows-per-wavefront sweep) such a batch goes the
+ * staged way instead - router, prologue, plan with up to two rows per work item - so that two rows that chose one expert
+ * share one sweep of its weights; the results are the same bits. rows->plan must be zero-filled once when it is allocated; every launch leaves its ticket words zero, and
  * they sit at a fixed place, so one workspace serves calls with any row count up to the one it was sized for. */
 int32_t mi355_moe_enqueue_layer(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
                                 float* scores, const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows,

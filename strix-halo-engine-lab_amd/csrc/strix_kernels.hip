@@ -1337,7 +1337,7 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     float* weights = const_cast<float*>(r->route_weights);
     if (const int32_t rc = check_route(p, r->input, r->input_kind, wv.hidden, r->input_stride, router_weight, ids, weights, scores)) return rc;
     STRIX_REQUIRE(p->experts == wv.experts && p->top_k == wv.top_k, "moe layer: router policy and expert tensors disagree on experts / top_k");
-    if (rows > kFusedMaxRows || plan_split(wv, rows) != 1U) {      // large batches: router, then the staged prologue / plan
+    if (rows > kFusedMaxRows || plan_split(wv, rows) != 1U) {      // large batches, and decode batches over large experts (shared sweeps): router, then the staged prologue / plan
         if (const int32_t rc = mi355_moe_route(p, r->input, r->input_kind, rows, wv.hidden, r->input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
         return mi355_moe_enqueue(w, r, rows, form, stream);
     }
