@@ -314,6 +314,29 @@ def test_config3_moe_decode_layer_shape(strix):
         check_layer_stages(strix, layer, y, ref, want, (c, d, s), ids_ref, w_ref, (gate, up, down, I, {}), H, K, T, 0, 0, TOL_F16)
 
 
+def test_layer_entry_shared_sweeps_over_large_experts(strix):
+    """A decode batch over experts whose gate + up rows exceed 4 MB (here 4.7 MB) and too large for the 16-rows-per-wavefront
+    sweep (64 assignments) is planned with up to two rows per work item: every expert is chosen by several rows, so items of
+    two rows and of one row both occur. Stage by stage against the oracle, through the layer entry and the staged one."""
+    E, H, I, K, T = 12, 2048, 2048, 4, 16
+    rng = np.random.default_rng(77)
+    gate, up, down = make_layer(rng, H, I, E)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, intermediates=True)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    ref = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref)
+    want = orc.combine(0, w_ref, ids_ref, ref.rawdots)
+    y, ids, wts, _ = layer.run_layer(dev(x), dev(wr))
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    items = int(layer.plan[4])
+    assert T * K // 2 <= items < T * K                     # shared sweeps: fewer work items than assignments
+    check_layer_stages(strix, layer, y.cpu().numpy(), ref, want, (c, d, s), ids_ref, w_ref, (gate, up, down, I, {}), H, K, T, 0, 0, TOL_F16)
+    y2 = layer.run(dev(x), ids, wts)
+    assert torch.equal(y2, y)
+
+
 @pytest.mark.parametrize("E,H,I,K,T,order", [(128, 2048, 768, 8, 8, 0), (128, 2048, 768, 8, 1, 0), (128, 2048, 768, 8, 2, 0), (160, 1536, 512, 8, 16, 0),
                                              (20, 512, 256, 3, 5, 1), (64, 1024, 256, 16, 16, 0), (160, 6144, 1280, 8, 2, 0)])
 def test_whole_layer_entry_router_prologue_plan_in_one_launch(strix, E, H, I, K, T, order):
