@@ -49,7 +49,9 @@ enum { MI355_TYPE_Q5_1 = 7, MI355_TYPE_Q8_0 = 8, MI355_TYPE_Q4_K = 12, MI355_TYP
 enum { MI355_INPUT_F32 = 0, MI355_INPUT_F16 = 1, MI355_INPUT_BF16 = 2 };
 enum { MI355_LOGITS_FMA_ASCENDING = 0, MI355_LOGITS_LANE32_BUTTERFLY = 1 };
 enum { MI355_COMBINE_FMA_SLOT_ORDER = 0, MI355_COMBINE_MULADD_ASCENDING_EXPERT = 1 };
-enum { MI355_EXP_GFX1151 = 0, MI355_EXP_DECLARED = 1 };
+enum { MI355_EXP_GFX1151 = 0, MI355_EXP_DECLARED = 1,
+       MI355_EXP_LIBM = 2 };   /* router softmax only: the C library's expf as the reference's router test oracle uses it
+                                  (tests/hip_moe_route_launcher_tests.hip:329), restated in double precision on the device */
 
 const char* mi355_last_error(void);
 const char* mi355_version(void);
@@ -121,6 +123,10 @@ typedef struct mi355_route_policy {
     uint32_t logits_order;            /* MI355_LOGITS_* */
     float renorm_eps, scale;
     uint32_t renormalize;
+    uint32_t renorm_single;           /* the weights are renormalised when renormalize && (top_k > 1 || renorm_single)
+                                         (include/strix/moe/route_policy.hpp:146) */
+    uint32_t exp_kind;                /* Math::exp of the softmax: MI355_EXP_DECLARED (include/strix/ds41_moe.hpp:38-54),
+                                         MI355_EXP_LIBM or MI355_EXP_GFX1151 */
 } mi355_route_policy;
 /* x: [rows] activations (input_kind), row r at x + r * x_stride_bytes. router_weight: fp32 [experts][hidden].
  * logit_bias: fp32 [experts] or NULL. ids / weights: [rows][top_k]. scores: [rows][experts] workspace AND output. */
@@ -146,7 +152,12 @@ typedef struct mi355_moe_weights {
     const uint8_t *gate, *up, *down;                  /* GGUF order [experts][ffn][hidden/256], [experts][hidden][ffn/256 or ffn/32 blocks] */
     uint64_t gate_expert_stride, gate_row_stride;     /* bytes; 0 = dense GGUF order. 16-byte multiples (Q6_K down: 2) */
     uint64_t down_expert_stride, down_row_stride;     /* a TP rank reads the first ffn/256 blocks of each down row */
-    uint32_t exp_kind;                                /* MI355_EXP_* used by SiLU */
+    uint32_t exp_kind;                                /* MI355_EXP_GFX1151 or MI355_EXP_DECLARED, used by SiLU */
+    float swiglu_limit;                               /* the SwiGLU clamp trait (include/strix/moe/activation_policy.hpp:22-24,
+                                                         DownRequest::swiglu_limit include/strix/moe_a8_down_contract.hpp:45):
+                                                         finite L > 0: g = min(g, L), u = clamp(u, -L, L) before silu(g) * u, the
+                                                         fail-closed check stays on the raw projections; +infinity (or 0, the
+                                                         zero-initialised default) = no clamp; anything else is rejected */
 } mi355_moe_weights;
 
 typedef struct mi355_moe_rows {
@@ -161,7 +172,10 @@ typedef struct mi355_moe_rows {
     const float* base;               /* optional [rows][hidden] added by the merge (shared expert output) */
     float* output; uint64_t output_stride;            /* [rows][hidden] fp32, stride in floats */
     uint32_t* plan;                  /* mi355_moe_plan_words(experts, rows, top_k) words, 16-byte aligned */
-    uint32_t* job_status;            /* 1 word: OR of every row's status (decides whether the down phase runs) */
+    uint32_t* job_status;            /* 1 word of job-wide flags: MI355_STATUS_NONFINITE_PROJECTION when any row's gate, up or h
+                                        was non-finite (the down phase is then skipped and no row is published). An invalid
+                                        route or a non-finite input flags only its own row (status[row]); the reference's
+                                        summary word fails the whole job for those too */
     void* h_f16;                     /* optional workspace of mi355_moe_prefill_f16_workspace_bytes() bytes, 16-byte aligned,
                                         used only by mi355_moe_enqueue_prefill_f16 (h in fp16 and sub-block sums) */
 } mi355_moe_rows;
@@ -219,9 +233,10 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights*, const mi355_moe_
 
 /* SwiGLU + A8 re-quantisation of h for a dense gate/up pair (the shared expert and the dense FFN):
  * gate / up: fp32 [rows][ffn]; writes h codes / deltas / sums as above and optionally h values.
- * Replaces enqueue_down_activation_quantize (include/strix/hip_moe_a8_down.hpp:18) for rows of gate|up. */
+ * Replaces enqueue_down_activation_quantize (include/strix/hip_moe_a8_down.hpp:18) for rows of gate|up.
+ * swiglu_limit: as mi355_moe_weights::swiglu_limit. */
 int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows, uint32_t ffn, uint32_t exp_kind,
-                              int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
+                              float swiglu_limit, int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
                               mi355_stream stream);
 
 #ifdef __cplusplus

@@ -7,6 +7,7 @@
 #include "cpu/core/routed_expert_kernels.hpp"
 #include "strix/ds41_moe.hpp"
 #include "strix/ggml_dequant.hpp"
+#include "strix/moe/activation_policy.hpp"
 #include "strix/moe/combine.hpp"
 #include "strix/moe/route_policy.hpp"
 #include "strix/moe_a8_down_contract.hpp"
@@ -231,6 +232,23 @@ int ref_route_select(std::uint32_t experts, std::uint32_t top_k, float renorm_ep
         strix::moe::route_select_ref(p, std::span<const float>(scores, experts), {}, std::span<std::uint32_t>(ids, top_k),
                                      std::span<float>(weights, top_k));
     });
+}
+// The same with the policy's renorm_single field given (top_k = 1 renormalises only when it is set).
+int ref_route_select_policy(std::uint32_t experts, std::uint32_t top_k, float renorm_eps, float scale, int renormalize, int renorm_single,
+                            const float* scores, std::uint32_t* ids, float* weights) {
+    return guarded([&] {
+        strix::moe::RoutePolicy p;
+        p.score = strix::moe::RouteScore::softmax; p.selection_bias = false; p.key = strix::moe::RouteKey::float_serial;
+        p.order = strix::moe::RouteOrder::selection; p.experts = experts; p.top_k = top_k;
+        p.renormalize = renormalize != 0; p.renorm_single = renorm_single != 0; p.renorm_eps = renorm_eps; p.scale = scale;
+        strix::moe::route_select_ref(p, std::span<const float>(scores, experts), {}, std::span<std::uint32_t>(ids, top_k),
+                                     std::span<float>(weights, top_k));
+    });
+}
+// The SwiGLU clamp trait.
+void ref_swiglu_clamp(float gate, float up, float limit, float* gate_out, float* up_out) {
+    const auto c = strix::moe::swiglu_clamp(gate, up, limit);
+    *gate_out = c.gate; *up_out = c.up;
 }
 int ref_combine_fma(std::uint32_t rows, std::uint32_t top_k, std::uint32_t width, const float* w, const float* eo,
                     const float* base, float* y) {

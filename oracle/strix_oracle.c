@@ -438,15 +438,25 @@ float orc_declared_exp(float x) {
     return (p * float_of((uint32_t)(k1 + 127) << 23)) * float_of((uint32_t)(k2 + 127) << 23);
 }
 
-static float exp_of(int kind, float x) { return kind == ORC_EXP_DECLARED ? orc_declared_exp(x) : orc_expf_gfx1151(x); }
+static float exp_of(int kind, float x) {
+    return kind == ORC_EXP_DECLARED ? orc_declared_exp(x) : kind == ORC_EXP_LIBM ? expf(x) : orc_expf_gfx1151(x);
+}
 
 int orc_swiglu_quantize(int exp_kind, const float* g, const float* u, int8_t* codes, float* delta, int32_t* sum,
                         float* h_out) {
+    return orc_swiglu_quantize_clamped(exp_kind, INFINITY, g, u, codes, delta, sum, h_out);
+}
+
+int orc_swiglu_quantize_clamped(int exp_kind, float limit, const float* g, const float* u, int8_t* codes, float* delta,
+                                int32_t* sum, float* h_out) {
     float hv[32];
     int bad = 0;
     for (int l = 0; l < 32; ++l) {
-        const float ex = exp_of(exp_kind, -g[l]);
-        hv[l] = (g[l] / (1.0F + ex)) * u[l];
+        /* include/strix/moe/activation_policy.hpp:22-24 */
+        const float gc = g[l] > limit ? limit : g[l];
+        const float uc = u[l] < -limit ? -limit : (u[l] > limit ? limit : u[l]);
+        const float ex = exp_of(exp_kind, -gc);
+        hv[l] = (gc / (1.0F + ex)) * uc;
         bad |= !is_finite(g[l]) || !is_finite(u[l]) || !is_finite(hv[l]);
     }
     if (h_out) for (int l = 0; l < 32; ++l) h_out[l] = hv[l];
@@ -488,7 +498,8 @@ void orc_route_select(const orc_route_policy* p, const float* scores, uint32_t* 
     const float denominator = sum + p->renorm_eps;
     for (uint32_t k = 0; k < p->top_k; ++k) {
         const float s = scores[ids[k]];
-        weights[k] = (p->renormalize ? s / denominator : s) * p->scale;
+        const int renorm = p->renormalize && (p->top_k > 1U || p->renorm_single);
+        weights[k] = (renorm ? s / denominator : s) * p->scale;
     }
 }
 
@@ -604,7 +615,7 @@ int orc_routed_experts(const orc_expert_weights* w, const orc_expert_job* job, i
             }
             if (job->gate_out) memcpy(job->gate_out + (size_t)a * ffn + grp * 32, g, sizeof g);
             if (job->up_out) memcpy(job->up_out + (size_t)a * ffn + grp * 32, u, sizeof u);
-            const int ok = orc_swiglu_quantize(w->exp_kind, g, u, hc + (size_t)a * ffn + grp * 32,
+            const int ok = orc_swiglu_quantize_clamped(w->exp_kind, w->swiglu_limit == 0.0F ? INFINITY : w->swiglu_limit, g, u, hc + (size_t)a * ffn + grp * 32,
                                                hd + (size_t)a * groups + grp, hs + (size_t)a * groups + grp, h);
             if (job->h_out) memcpy(job->h_out + (size_t)a * ffn + grp * 32, h, sizeof h);
             if (!ok) {

@@ -39,7 +39,8 @@ enum { ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 }
 enum { ORC_Q5_1_BLOCK = 24, ORC_Q8_0_BLOCK = 34, ORC_Q4_K_BLOCK = 144, ORC_Q5_K_BLOCK = 176, ORC_Q6_K_BLOCK = 210 };
 enum { ORC_STATUS_INVALID_ROUTE = 1, ORC_STATUS_NONFINITE_ACTIVATION = 2, ORC_STATUS_INVALID_DELTA = 4,
        ORC_STATUS_NONFINITE_PROJECTION = 8 };
-enum { ORC_EXP_GFX1151_NOTABLE = 0, ORC_EXP_DECLARED = 1 };
+enum { ORC_EXP_GFX1151_NOTABLE = 0, ORC_EXP_DECLARED = 1,
+       ORC_EXP_LIBM = 2 };   /* expf of the C library: the Math::exp of the reference's router test oracle (tests/hip_moe_route_launcher_tests.hip:329) */
 enum { ORC_LOGITS_FMA_ASCENDING = 0, ORC_LOGITS_LANE32_BUTTERFLY = 1 };
 enum { ORC_COMBINE_FMA_SLOT_ORDER = 0, ORC_COMBINE_MULADD_ASCENDING_EXPERT = 1 };
 
@@ -98,6 +99,11 @@ float orc_declared_exp(float x);     /* include/strix/ds41_moe.hpp:38-54 */
  * h_out (optional) receives the 32 h values. src/cpu/core/routed_expert.cpp:147-170. */
 int orc_swiglu_quantize(int exp_kind, const float* g, const float* u, int8_t* codes, float* delta,
                         int32_t* sum, float* h_out);
+/* The same with the SwiGLU clamp trait (include/strix/moe/activation_policy.hpp:22-24; producer body
+ * src/hip_moe_q4k_a8_probe.hip:594-621): g = min(g, limit), u = clamp(u, -limit, limit) before silu(g) * u, the finite check
+ * stays on the raw g and u. limit = +infinity clamps nothing. */
+int orc_swiglu_quantize_clamped(int exp_kind, float limit, const float* g, const float* u, int8_t* codes, float* delta,
+                                int32_t* sum, float* h_out);
 
 /* ---- router (include/strix/moe/route_policy.hpp:99-156; logits tests/hip_moe_route_launcher_tests.hip:281-330) */
 typedef struct {
@@ -107,6 +113,7 @@ typedef struct {
     float renorm_eps;       /* Qwen launcher 0, policy default 1e-20 */
     float scale;
     int renormalize;
+    int renorm_single;      /* renormalise when renormalize && (top_k > 1 || renorm_single), include/strix/moe/route_policy.hpp:146 */
 } orc_route_policy;
 /* x [rows][hidden] fp32, w [experts][hidden] fp32, logit_bias [experts] or NULL (added to the logit).
  * ids/weights [rows][top_k]; scores (optional) [rows][experts]; logits (optional) [rows][experts]. */
@@ -129,6 +136,7 @@ typedef struct {
     uint64_t gate_expert_stride, gate_row_stride;   /* bytes */
     uint64_t down_expert_stride, down_row_stride;   /* bytes; a rank reads the first ffn/blk blocks of each row */
     int exp_kind;
+    float swiglu_limit;     /* clamp trait; +infinity or 0 = none */
 } orc_expert_weights;
 typedef struct {
     /* inputs */

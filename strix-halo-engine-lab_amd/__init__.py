@@ -14,7 +14,7 @@ TYPE_Q5_1, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K = 7, 8, 12, 13, 14
 INPUT_F32, INPUT_F16, INPUT_BF16 = 0, 1, 2
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
 COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
-EXP_GFX1151, EXP_DECLARED = 0, 1
+EXP_GFX1151, EXP_DECLARED, EXP_LIBM = 0, 1, 2
 STATUS_INVALID_ROUTE, STATUS_NONFINITE_ACTIVATION, STATUS_INVALID_DELTA, STATUS_NONFINITE_PROJECTION, STATUS_AGGREGATE = 1, 2, 4, 8, 16
 E_INVALID_ARGUMENT, E_UNSUPPORTED, E_HIP = -1, -2, -3
 Q8_0_BLOCK, Q4_K_BLOCK = 34, 144
@@ -34,7 +34,8 @@ class Q8a8View(C.Structure):
 
 class RoutePolicy(C.Structure):
     _fields_ = [("experts", C.c_uint32), ("top_k", C.c_uint32), ("logits_order", C.c_uint32),
-                ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_uint32)]
+                ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_uint32),
+                ("renorm_single", C.c_uint32), ("exp_kind", C.c_uint32)]
 
 
 class MoeWeights(C.Structure):
@@ -42,7 +43,8 @@ class MoeWeights(C.Structure):
                 ("gate_type", C.c_uint32), ("down_type", C.c_uint32),
                 ("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p),
                 ("gate_expert_stride", C.c_uint64), ("gate_row_stride", C.c_uint64),
-                ("down_expert_stride", C.c_uint64), ("down_row_stride", C.c_uint64), ("exp_kind", C.c_uint32)]
+                ("down_expert_stride", C.c_uint64), ("down_row_stride", C.c_uint64), ("exp_kind", C.c_uint32),
+                ("swiglu_limit", C.c_float)]
 
 
 class MoeRows(C.Structure):
@@ -158,10 +160,11 @@ def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False,
     return out
 
 
-def route(x, router_weight, top_k, bias=None, logits_order=LOGITS_FMA, renorm_eps=0.0, scale=1.0, renormalize=True):
+def route(x, router_weight, top_k, bias=None, logits_order=LOGITS_FMA, renorm_eps=0.0, scale=1.0, renormalize=True, renorm_single=True,
+          exp_kind=EXP_DECLARED):
     rows, hidden = x.shape
     experts = router_weight.shape[0]
-    p = RoutePolicy(experts, top_k, logits_order, renorm_eps, scale, int(renormalize))
+    p = RoutePolicy(experts, top_k, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single), exp_kind)
     ids = torch.empty((rows, top_k), dtype=torch.int32, device=x.device)
     weights = torch.empty((rows, top_k), dtype=torch.float32, device=x.device)
     scores = torch.empty((rows, experts), dtype=torch.float32, device=x.device)
@@ -170,14 +173,14 @@ def route(x, router_weight, top_k, bias=None, logits_order=LOGITS_FMA, renorm_ep
     return ids, weights, scores
 
 
-def swiglu_quantize(gate, up, exp_kind=EXP_GFX1151):
+def swiglu_quantize(gate, up, exp_kind=EXP_GFX1151, swiglu_limit=float("inf")):
     rows, ffn = gate.shape
     codes = torch.zeros((rows, ffn), dtype=torch.int8, device=gate.device)
     deltas = torch.zeros((rows, ffn // 32), dtype=torch.float32, device=gate.device)
     sums = torch.zeros((rows, ffn // 32), dtype=torch.int32, device=gate.device)
     h = torch.zeros((rows, ffn), dtype=torch.float32, device=gate.device)
     status = torch.zeros(rows, dtype=torch.int32, device=gate.device)
-    check(lib().mi355_swiglu_quantize(_p(gate), _p(up), rows, ffn, exp_kind, _p(codes), _p(deltas), _p(sums), _p(h), _p(status), _stream()))
+    check(lib().mi355_swiglu_quantize(_p(gate), _p(up), rows, ffn, exp_kind, C.c_float(swiglu_limit), _p(codes), _p(deltas), _p(sums), _p(h), _p(status), _stream()))
     return codes, deltas, sums, h, status
 
 
@@ -187,12 +190,12 @@ class MoeLayer:
 
     def __init__(self, hidden, ffn, experts, top_k, gate, up, down, max_rows, exp_kind=EXP_GFX1151, intermediates=False,
                  gate_expert_stride=0, gate_row_stride=0, down_expert_stride=0, down_row_stride=0, prefill_f16=False,
-                 gate_type=TYPE_Q4_K, down_type=TYPE_Q4_K, output_stride=None):
+                 gate_type=TYPE_Q4_K, down_type=TYPE_Q4_K, output_stride=None, swiglu_limit=float("inf")):
         dev = gate.device
         self.hidden, self.ffn, self.experts, self.top_k, self.max_rows = hidden, ffn, experts, top_k, max_rows
         self.gate, self.up, self.down = gate, up, down
         self.w = MoeWeights(hidden, ffn, experts, top_k, gate_type, down_type, gate.data_ptr(), up.data_ptr(), down.data_ptr(),
-                            gate_expert_stride, gate_row_stride, down_expert_stride, down_row_stride, exp_kind)
+                            gate_expert_stride, gate_row_stride, down_expert_stride, down_row_stride, exp_kind, swiglu_limit)
         n = max_rows * top_k
         z = lambda shape, dt: torch.zeros(shape, dtype=dt, device=dev)
         self.codes, self.deltas, self.sums = z((max_rows, hidden), torch.int8), z((max_rows, hidden // 32), torch.float32), z((max_rows, hidden // 32), torch.int32)
@@ -231,7 +234,7 @@ class MoeLayer:
         return self.output[:rows]
 
     def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,
-                  scale=1.0, renormalize=True):
+                  scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED):
         """Router + experts + combine through mi355_moe_enqueue_layer. Returns (output, ids, weights, scores)."""
         rows = x.shape[0]
         if not hasattr(self, "ids") or self.ids.shape[0] < rows:
@@ -239,7 +242,7 @@ class MoeLayer:
             self.route_w = torch.zeros((self.max_rows, self.top_k), dtype=torch.float32, device=x.device)
             self.scores = torch.zeros((self.max_rows, self.experts), dtype=torch.float32, device=x.device)
         _, rv = self.rows_view(x, self.ids, self.route_w, base)
-        p = RoutePolicy(self.experts, self.top_k, logits_order, renorm_eps, scale, int(renormalize))
+        p = RoutePolicy(self.experts, self.top_k, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single), exp_kind)
         check(lib().mi355_moe_enqueue_layer(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), C.byref(self.w), C.byref(rv), rows,
                                             combine, _stream()))
         return self.output[:rows], self.ids[:rows], self.route_w[:rows], self.scores[:rows]

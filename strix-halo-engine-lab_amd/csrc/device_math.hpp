@@ -90,7 +90,45 @@ __device__ __forceinline__ float expf_gfx1151(float x) {
     if (f_of(0x42b17218U) < x) y = f_of(0x7f800000U);
     return y;
 }
-__device__ __forceinline__ float exp_of(uint32_t kind, float x) { return kind == 1U ? declared_exp(x) : expf_gfx1151(x); }
+// The C library's single-precision exp as the reference's router test oracle calls it (std::exp on a float,
+// tests/hip_moe_route_launcher_tests.hip:329): z = x * 32 / ln 2 in double, k = round(z) by the 1.5 * 2^52 shift, r = z - k,
+// 2^(k / 32) from a 32-entry table with k's upper bits added to the exponent, a cubic in r, one rounding to float.
+// Every operation is a double-precision IEEE operation, so the bits are the host library's wherever its own result is
+// not within a few double ulps of a float rounding boundary.
+__device__ __forceinline__ float expf_libm(float x) {
+    static constexpr unsigned long long kTab[32] = {
+        0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
+        0x3fef72b83c7d517bULL, 0x3fef54873168b9aaULL, 0x3fef387a6e756238ULL, 0x3fef1e9df51fdee1ULL,
+        0x3fef06fe0a31b715ULL, 0x3feef1a7373aa9cbULL, 0x3feedea64c123422ULL, 0x3feece086061892dULL,
+        0x3feebfdad5362a27ULL, 0x3feeb42b569d4f82ULL, 0x3feeab07dd485429ULL, 0x3feea47eb03a5585ULL,
+        0x3feea09e667f3bcdULL, 0x3fee9f75e8ec5f74ULL, 0x3feea11473eb0187ULL, 0x3feea589994cce13ULL,
+        0x3feeace5422aa0dbULL, 0x3feeb737b0cdc5e5ULL, 0x3feec49182a3f090ULL, 0x3feed503b23e255dULL,
+        0x3feee89f995ad3adULL, 0x3feeff76f2fb5e47ULL, 0x3fef199bdd85529cULL, 0x3fef3720dcef9069ULL,
+        0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL};
+    if (!(x == x)) return x + x;
+    if (x > 0x1.62e42ep6F) return f_of(0x7f800000U);
+    if (x < -0x1.9fe368p6F) return 0.0F;
+    const double z = (0x1.71547652b82fep+0 * 32.0) * static_cast<double>(x);
+    double kd = z + 0x1.8p+52;
+    const unsigned long long ki = __builtin_bit_cast(unsigned long long, kd);
+    kd = kd - 0x1.8p+52;
+    const double r = z - kd;
+    const double s = __builtin_bit_cast(double, kTab[ki % 32U] + (ki << 47));
+    const double c01 = (0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0) * r + (0x1.ebfce50fac4f3p-3 / 32.0 / 32.0);
+    const double r2 = r * r;
+    double y = (0x1.62e42ff0c52d6p-1 / 32.0) * r + 1.0;
+    y = c01 * r2 + y;
+    y = y * s;
+    return static_cast<float>(y);
+}
+__device__ __forceinline__ float exp_of(uint32_t kind, float x) { return kind == 1U ? declared_exp(x) : kind == 2U ? expf_libm(x) : expf_gfx1151(x); }
+
+// The SwiGLU clamp trait (include/strix/moe/activation_policy.hpp:22-24): gate from above, up on both sides; NaN passes
+// through; limit = +infinity clamps nothing (every comparison is false).
+__device__ __forceinline__ void swiglu_clamp(float& g, float& u, float limit) {
+    g = g > limit ? limit : g;
+    u = u < -limit ? -limit : (u > limit ? limit : u);
+}
 
 // ---- cross-lane moves inside a 64-wide wavefront ----------------------------------------------------------------
 // lane ^ 1 and lane ^ 2 are DPP quad permutes (no LDS traffic); wider distances go through the swizzle crossbar.

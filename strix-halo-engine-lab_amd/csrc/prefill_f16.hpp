@@ -70,6 +70,7 @@ struct PrefillArgs {
     uint32_t k;                                   // K = hidden (MODE 0) or ffn (MODE 1), multiple of 256
     uint32_t features;                            // ffn (MODE 0) or hidden (MODE 1)
     uint32_t top_k, exp_kind;
+    float swiglu_limit;                           // the clamp trait of the SwiGLU epilogue (+infinity: none)
     const uint8_t* x; uint64_t x_stride;          // MODE 0: fp16 token rows (bytes); MODE 1: unused
     _Float16* h;                                  // [assignments in plan order][ffn] fp16: written by MODE 0, read by MODE 1
     uint8_t* h_sums;                              // [assignments in plan order] sub-block sums of h: written by MODE 0, read by MODE 1
@@ -560,7 +561,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             const bool live = n < count;
             if (MODE == 0) {
                 const float g = acc[i][0][j], u = acc[i][1][j];
-                const float hv = (g / (1.0F + declared_exp(-g))) * u;
+                float gc = g, uc = u;
+                swiglu_clamp(gc, uc, a.swiglu_limit);
+                const float hv = (gc / (1.0F + declared_exp(-gc))) * uc;
                 const _Float16 h16 = static_cast<_Float16>(hv);
                 float sum = live ? static_cast<float>(h16) : 0.0F;
                 sum += xor1_f(sum); sum += xor2_f(sum); sum += xor4_f(sum); sum += xor8_f(sum); sum += xor16_f(sum);

@@ -442,7 +442,7 @@ __device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const Rou
 #pragma unroll
     for (uint32_t i = 0; i < PER; ++i) {
         const uint32_t e = lane + 64U * i;
-        if (e < E) p_lds[e] = declared_exp(v[i] - m);
+        if (e < E) p_lds[e] = exp_of(a.p.exp_kind, v[i] - m);
     }
     __syncthreads();
     // denominator: ascending expert order from 0, computed by every lane (LDS broadcast reads, 16 values fetched ahead)
@@ -495,7 +495,8 @@ __device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const Rou
     const float den = sum + a.p.renorm_eps;
     if (lane < K) {
         a.ids[static_cast<size_t>(row) * K + lane] = my_id;
-        a.weights[static_cast<size_t>(row) * K + lane] = (a.p.renormalize ? my_v / den : my_v) * a.p.scale;
+        const bool renorm = a.p.renormalize && (K > 1U || a.p.renorm_single);      // include/strix/moe/route_policy.hpp:146
+        a.weights[static_cast<size_t>(row) * K + lane] = (renorm ? my_v / den : my_v) * a.p.scale;
     }
     __syncthreads();
     return my_id;

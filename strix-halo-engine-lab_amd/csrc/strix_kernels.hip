@@ -245,21 +245,21 @@ __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v) {
 // expert; items[A] x 4 words {expert, begin, end, 0}: the work items of the expert kernels, a touched expert's assignments
 // cut into pieces of at most `split` (zero records after the last item, up to the launch's item bound).
 // Reference: src/hip_moe_q4k_a8_probe.hip:91-147 (stable CSR of (row, slot) by expert).
-__host__ __device__ inline uint32_t pad4(uint32_t v) { return (v + 3U) & ~3U; }
+__host__ __device__ constexpr uint32_t pad4(uint32_t v) { return (v + 3U) & ~3U; }
 // ticket / scratch words right after the header, at the same place for every batch size (every launch leaves them zero, and a
 // workspace is reused with varying row counts): [0, 16) row tickets of the fused router, [16, 32) its quantiser tickets,
 // [128, 144) per-row A8 flags of the fused prologue
 constexpr uint32_t kPlanTicketsAt = 16, kPlanTicketWords = 256, kPlanOffsetsAt = kPlanTicketsAt + kPlanTicketWords;
-__host__ __device__ inline uint32_t plan_touched_at(uint32_t experts) { return kPlanOffsetsAt + pad4(experts + 1U); }
-__host__ __device__ inline uint32_t plan_order_at(uint32_t experts) { return plan_touched_at(experts) + pad4(experts); }
+__host__ __device__ constexpr uint32_t plan_touched_at(uint32_t experts) { return kPlanOffsetsAt + pad4(experts + 1U); }
+__host__ __device__ constexpr uint32_t plan_order_at(uint32_t experts) { return plan_touched_at(experts) + pad4(experts); }
 // most work items a plan can hold (layout) and most a launch with pieces of `split` assignments can produce (grid size)
-__host__ __device__ inline uint32_t plan_item_capacity(uint32_t assignments) { return assignments; }
+__host__ __device__ constexpr uint32_t plan_item_capacity(uint32_t assignments) { return assignments; }
 __host__ __device__ inline uint32_t plan_item_bound(uint32_t experts, uint32_t assignments, uint32_t split) {
     const uint32_t most = experts + assignments / split;
     return assignments < most ? assignments : most;
 }
-__host__ __device__ inline uint32_t plan_items_at(uint32_t experts, uint32_t assignments) { return plan_order_at(experts) + pad4(assignments); }
-__host__ __device__ inline uint32_t plan_words_total(uint32_t experts, uint32_t assignments) {
+__host__ __device__ constexpr uint32_t plan_items_at(uint32_t experts, uint32_t assignments) { return plan_order_at(experts) + pad4(assignments); }
+__host__ __device__ constexpr uint32_t plan_words_total(uint32_t experts, uint32_t assignments) {
     return plan_items_at(experts, assignments) + 4U * plan_item_capacity(assignments);
 }
 
@@ -511,7 +511,9 @@ __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], con
     for (int a = 0; a < NA; ++a) {
         const float other = __shfl_xor(value[a], 32);
         const float g = lane < 32U ? value[a] : other, u = lane < 32U ? other : value[a];
-        const float h = (g / (1.0F + exp_of(w.exp_kind, -g))) * u;
+        float gc = g, uc = u;
+        swiglu_clamp(gc, uc, w.swiglu_limit);
+        const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
         const size_t at = static_cast<size_t>(sidx[a]) * w.ffn + grp * 32U + o;
         if (lane < 32U) {
             if (r.gate_out) r.gate_out[at] = g;
@@ -561,7 +563,7 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void project_wave_kernel(mi3
     const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U) * w.gate_row_stride;
     const uint8_t* gate = w.gate + base;
     const uint8_t* up = w.up + base;
-    const uint32_t stride = static_cast<uint32_t>(w.gate_row_stride);
+    const size_t stride = w.gate_row_stride;       // (64-bit: row * stride passes 2^32 for rows of 64 MiB and more)
     StageSource source;
     source.init([&](uint32_t row) { return row < 32U ? gate + row * stride : up + (row - 32U) * stride; });
     lds_u8* const (&sl)[DEPTH] = slots;
@@ -618,7 +620,7 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_
     if (end - begin > 1U) __builtin_amdgcn_s_setprio(3);     // as in the projection: the longest instruction streams issue first
     const uint32_t* order = r.plan + plan_order_at(w.experts);
     const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
-    const uint32_t stride = static_cast<uint32_t>(w.down_row_stride);
+    const size_t stride = w.down_row_stride;
     StageSource source;
     source.init([&](uint32_t row) { return rows + row * stride; });
     lds_u8* const (&sl)[DEPTH] = slots;
@@ -671,7 +673,7 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
     const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(f0) * w.gate_row_stride;
     const uint8_t* gate = w.gate + base;
     const uint8_t* up = w.up + base;
-    const uint32_t stride = static_cast<uint32_t>(w.gate_row_stride);
+    const size_t stride = w.gate_row_stride;
     QuadSource source;
     source.init([&](uint32_t q) { return q < 8U ? gate + q * stride : up + (q - 8U) * stride; }, r.codes + static_cast<size_t>(row) * w.hidden);
     lds_u8* const (&sl)[DEPTH] = slots;
@@ -679,7 +681,9 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
     const float other = __shfl_xor(value, 32);
     const bool mine = lane < 32U && p == 0;                   // the lane that publishes feature f0 + rr
     const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
-    const float h = (g / (1.0F + exp_of(w.exp_kind, -g))) * u;
+    float gc = g, uc = u;
+    swiglu_clamp(gc, uc, w.swiglu_limit);
+    const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
     const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
     if (mine) {
         if (r.gate_out) r.gate_out[at] = g;
@@ -727,7 +731,9 @@ __global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, m
         const float value = sweep_q5k_row(wrow, w.hidden / 256U, A8Image{r.codes, r.deltas, r.sums, w.hidden}, row, p);
         const float other = __shfl_xor(value, 32);
         const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
-        const float h = (g / (1.0F + exp_of(w.exp_kind, -g))) * u;
+        float gc = g, uc = u;
+        swiglu_clamp(gc, uc, w.swiglu_limit);
+        const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
         const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
         if (mine) {
             if (r.gate_out) r.gate_out[at] = g;
@@ -774,7 +780,7 @@ __global__ __launch_bounds__(256) void down_quad_kernel(mi355_moe_weights w, mi3
     const uint32_t src = __builtin_amdgcn_readfirstlane(r.plan[plan_order_at(w.experts) + begin]);
     const uint32_t o0 = blockIdx.x * 64U + 16U * wave;
     const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o0) * w.down_row_stride;
-    const uint32_t stride = static_cast<uint32_t>(w.down_row_stride);
+    const size_t stride = w.down_row_stride;
     QuadSource source;
     source.init([&](uint32_t q) { return rows + q * stride; }, r.down_codes + static_cast<size_t>(src) * w.ffn);
     lds_u8* const (&sl)[DEPTH] = slots;
@@ -834,7 +840,7 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
     if (begin != end) {                                                        // (an invalid route has no item: its row is flagged)
         const uint32_t* order = r.plan + plan_order_at(w.experts);
         const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
-        const uint32_t stride = static_cast<uint32_t>(w.down_row_stride);
+        const size_t stride = w.down_row_stride;
         StageSource source;
         source.init([&](uint32_t q) { return rows + q * stride; });
         lds_u8* const slots[2] = {(lds_u8*)rings[wave][0], (lds_u8*)rings[wave][1]};
@@ -870,15 +876,17 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
 }
 
 // SwiGLU + A8 re-quantisation of dense gate/up rows. Reference: src/cpu/core/routed_expert.cpp:147-170.
-__global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate, const float* up, uint32_t ffn, uint32_t exp_kind,
+__global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate, const float* up, uint32_t ffn, uint32_t exp_kind, float limit,
                                                               int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
                                                               uint32_t* job_status) {
     const uint32_t row = blockIdx.y, groups = ffn / 32U, grp = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U;
     if (grp >= groups) return;
     const size_t at = static_cast<size_t>(row) * ffn + grp * 32U + l;
     const float g = gate[at], u = up[at];
-    const float ex = exp_of(exp_kind, -g);
-    const float hv = (g / (1.0F + ex)) * u;
+    float gc = g, uc = u;
+    swiglu_clamp(gc, uc, limit);
+    const float ex = exp_of(exp_kind, -gc);
+    const float hv = (gc / (1.0F + ex)) * uc;
     if (h_out) h_out[at] = hv;
     const int bad = or32_i((finite_f(g) && finite_f(u) && finite_f(hv)) ? 0 : 1);
     if (bad) {
@@ -956,7 +964,7 @@ inline void launch_project_dense(const mi355_moe_weights& w, const mi355_moe_row
     a.m[1] = PairMatrix{w.up, w.gate_row_stride, r.up_out, w.ffn};
     a.rows = w.ffn; a.blocks = w.hidden / 256U; a.img = A8Image{r.codes, r.deltas, r.sums, w.hidden}; a.nacts = rows;
     launch_pairs(a, 2, st);
-    swiglu_quantize_kernel<<<dim3((w.ffn / 32U + 7U) / 8U, rows), 256, 0, st>>>(r.gate_out, r.up_out, w.ffn, w.exp_kind, r.down_codes, r.down_deltas,
+    swiglu_quantize_kernel<<<dim3((w.ffn / 32U + 7U) / 8U, rows), 256, 0, st>>>(r.gate_out, r.up_out, w.ffn, w.exp_kind, w.swiglu_limit, r.down_codes, r.down_deltas,
                                                                                 r.down_sums, r.h_out, r.status, r.job_status);
 }
 inline void launch_down_dense(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, hipStream_t st) {
@@ -1079,6 +1087,8 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
     STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
     STRIX_REQUIRE(w->top_k > 0 && w->top_k <= kRouteMaxTopK && w->top_k <= w->experts, "moe: top_k must be within 1..16 and <= experts");
     STRIX_REQUIRE(static_cast<uint64_t>(rows) * w->top_k < (1ULL << 31), "moe: too many assignments");
+    // rows are one grid dimension of the prologue and of the merge: every entry refuses a larger batch before its first launch
+    STRIX_REQUIRE(rows <= 65535U, "moe: at most 65535 rows per call");
     // plan items are one grid dimension of the expert launches
     STRIX_REQUIRE(cls != kIntegerClass || item_bound(*w, rows) <= 65535U, "moe: too many work items for one call (experts + rows * top_k / 4 must stay below 65536)");
     wv = *w;
@@ -1095,6 +1105,9 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
     STRIX_REQUIRE(w->gate && w->up && w->down && aligned(w->gate, 16) && aligned(w->up, 16) && aligned(w->down, 16),
                   "moe: weight pointers must be non-null and 16-byte aligned");
     STRIX_REQUIRE(w->exp_kind <= MI355_EXP_DECLARED, "moe: unknown exp kind");
+    // the clamp trait: +infinity (or the zero-initialised 0) = none, else finite and positive (src/moe_a8_down_contract.cpp:57)
+    if (wv.swiglu_limit == 0.0F) wv.swiglu_limit = INFINITY;
+    STRIX_REQUIRE(wv.swiglu_limit > 0.0F, "moe: swiglu_limit must be +infinity (none) or finite and positive");
     STRIX_REQUIRE(r->routes && r->route_weights && r->codes && r->deltas && r->sums && r->status && r->down_codes && r->down_deltas &&
                   r->down_sums && r->rawdots && r->output && r->plan && r->job_status, "moe: a required row view is null");
     STRIX_REQUIRE(aligned(r->codes, 16) && aligned(r->down_codes, 16) && aligned(r->plan, 16) && aligned(r->rawdots, 16) &&
@@ -1222,6 +1235,7 @@ int32_t check_route(const mi355_route_policy* p, const void* x, uint32_t kind, u
                   "route policy: need 0 < top_k <= experts, experts <= 1024, top_k <= 16");
     STRIX_REQUIRE(hidden > 0 && hidden <= kRouteMaxHidden && hidden % 32U == 0, "route: hidden must be a multiple of 32 within 16384");
     STRIX_REQUIRE(kind <= MI355_INPUT_BF16 && p->logits_order <= MI355_LOGITS_LANE32_BUTTERFLY, "route: unknown input kind or logits order");
+    STRIX_REQUIRE(p->exp_kind <= MI355_EXP_LIBM, "route policy: unknown exp kind");
     STRIX_REQUIRE(aligned(wr, 16) && aligned(x, 16) && x_stride % 16U == 0, "route: router weight, activations and their row stride must be 16-byte aligned");
     return MI355_OK;
 }
@@ -1379,7 +1393,7 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     clear_validate_kernel<<<rows, 64, 0, st>>>(r->routes, r->route_weights, wv.experts, wv.top_k, r->status, r->job_status);
     launch_plan(r->routes, wv.experts, assignments, kPfTile, bound, r->plan, st);
     PrefillArgs a{};
-    a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.x = static_cast<const uint8_t*>(r->input); a.x_stride = r->input_stride;
+    a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.swiglu_limit = wv.swiglu_limit; a.x = static_cast<const uint8_t*>(r->input); a.x_stride = r->input_stride;
     uint8_t* ws = static_cast<uint8_t*>(r->h_f16);
     a.h = reinterpret_cast<_Float16*>(ws); a.h_sums = ws + pf_h_bytes(assignments, wv.ffn);
     uint8_t* x_sums = a.h_sums + static_cast<size_t>(assignments) * pf_sum_row_bytes(wv.ffn);
@@ -1406,14 +1420,16 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
 
-int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows, uint32_t ffn, uint32_t exp_kind, int8_t* codes,
-                              float* deltas, int32_t* sums, float* h_out, uint32_t* status, mi355_stream stream) {
+int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows, uint32_t ffn, uint32_t exp_kind, float swiglu_limit,
+                              int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status, mi355_stream stream) {
     STRIX_REQUIRE(ffn % 32U == 0, "swiglu: ffn must be a multiple of 32");
     STRIX_REQUIRE(exp_kind <= MI355_EXP_DECLARED, "swiglu: unknown exp kind");
+    if (swiglu_limit == 0.0F) swiglu_limit = INFINITY;
+    STRIX_REQUIRE(swiglu_limit > 0.0F, "swiglu: swiglu_limit must be +infinity (none) or finite and positive");
     if (rows == 0 || ffn == 0) return MI355_OK;
     STRIX_REQUIRE(gate && up && codes && deltas && sums, "swiglu: null pointer");
     STRIX_REQUIRE(rows <= 65535U, "swiglu: at most 65535 rows per call");
-    swiglu_quantize_kernel<<<dim3((ffn / 32U + 7U) / 8U, rows), 256, 0, hs(stream)>>>(gate, up, ffn, exp_kind, codes, deltas, sums, h_out, status, nullptr);
+    swiglu_quantize_kernel<<<dim3((ffn / 32U + 7U) / 8U, rows), 256, 0, hs(stream)>>>(gate, up, ffn, exp_kind, swiglu_limit, codes, deltas, sums, h_out, status, nullptr);
     STRIX_LAUNCHED("swiglu_quantize");
     return MI355_OK;
 }

@@ -93,9 +93,9 @@ inline void enqueue_layer(const moe_route::Policy& policy, const float* router_w
 
 // SwiGLU + A8 re-quantisation of dense gate | up rows (enqueue_down_activation_quantize, include/strix/hip_moe_a8_down.hpp:18).
 inline void enqueue_down_activation_quantize(const float* gate, const float* up, std::uint32_t rows, std::uint32_t ffn,
-                                             std::uint32_t exp_kind, std::int8_t* codes, float* deltas, std::int32_t* sums,
-                                             float* h_out, std::uint32_t* status, mi355_stream s) {
-    check(mi355_swiglu_quantize(gate, up, rows, ffn, exp_kind, codes, deltas, sums, h_out, status, s));
+                                             std::uint32_t exp_kind, float swiglu_limit, std::int8_t* codes, float* deltas,
+                                             std::int32_t* sums, float* h_out, std::uint32_t* status, mi355_stream s) {
+    check(mi355_swiglu_quantize(gate, up, rows, ffn, exp_kind, swiglu_limit, codes, deltas, sums, h_out, status, s));
 }
 
 }  // namespace strix::mi355

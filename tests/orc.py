@@ -11,7 +11,7 @@ ORACLE_DIR = os.path.join(ROOT, "oracle")
 
 Q5_1, Q8_0, Q4_K, Q5_K, Q6_K = 7, 8, 12, 13, 14
 Q5_1_BLOCK, Q8_0_BLOCK, Q4_K_BLOCK, Q5_K_BLOCK, Q6_K_BLOCK = 24, 34, 144, 176, 210
-EXP_GFX1151, EXP_DECLARED = 0, 1
+EXP_GFX1151, EXP_DECLARED, EXP_LIBM = 0, 1, 2
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
 COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
 
@@ -78,7 +78,7 @@ class Q8a8View(C.Structure):
 
 class RoutePolicy(C.Structure):
     _fields_ = [("experts", C.c_uint32), ("top_k", C.c_uint32), ("logits_order", C.c_int), ("exp_kind", C.c_int),
-                ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_int)]
+                ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_int), ("renorm_single", C.c_int)]
 
 
 class ExpertWeights(C.Structure):
@@ -86,7 +86,8 @@ class ExpertWeights(C.Structure):
                 ("gate_type", C.c_uint32), ("down_type", C.c_uint32),
                 ("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p),
                 ("gate_expert_stride", C.c_uint64), ("gate_row_stride", C.c_uint64),
-                ("down_expert_stride", C.c_uint64), ("down_row_stride", C.c_uint64), ("exp_kind", C.c_int)]
+                ("down_expert_stride", C.c_uint64), ("down_row_stride", C.c_uint64), ("exp_kind", C.c_int),
+                ("swiglu_limit", C.c_float)]
 
 
 class ExpertJob(C.Structure):
@@ -327,25 +328,25 @@ def dequant_q5_1_rows(raw, width):
     return (d * q.astype(np.float32) + m).reshape(raw.shape[0], width)
 
 
-def swiglu_quantize(g, u, exp_kind=EXP_GFX1151):
+def swiglu_quantize(g, u, exp_kind=EXP_GFX1151, limit=float("inf")):
     g = np.ascontiguousarray(g, np.float32)
     u = np.ascontiguousarray(u, np.float32)
     codes = np.zeros(32, np.int8)
     delta = C.c_float(0)
     s = C.c_int32(0)
     h = np.zeros(32, np.float32)
-    ok = lib().orc_swiglu_quantize(exp_kind, _ptr(g, f32p), _ptr(u, f32p), _ptr(codes, i8p), C.byref(delta), C.byref(s),
-                                   _ptr(h, f32p))
+    ok = lib().orc_swiglu_quantize_clamped(exp_kind, C.c_float(limit), _ptr(g, f32p), _ptr(u, f32p), _ptr(codes, i8p), C.byref(delta),
+                                           C.byref(s), _ptr(h, f32p))
     return ok, codes, np.float32(delta.value), s.value, h
 
 
 def route(x, w, top_k, bias=None, logits_order=LOGITS_FMA, exp_kind=EXP_DECLARED, renorm_eps=0.0, scale=1.0,
-          renormalize=True, threads=0):
+          renormalize=True, threads=0, renorm_single=True):
     x = np.ascontiguousarray(x, np.float32)
     w = np.ascontiguousarray(w, np.float32)
     rows, hidden = x.shape
     experts = w.shape[0]
-    p = RoutePolicy(experts, top_k, logits_order, exp_kind, renorm_eps, scale, int(renormalize))
+    p = RoutePolicy(experts, top_k, logits_order, exp_kind, renorm_eps, scale, int(renormalize), int(renorm_single))
     ids = np.zeros((rows, top_k), np.uint32)
     weights = np.zeros((rows, top_k), np.float32)
     scores = np.zeros((rows, experts), np.float32)
@@ -356,9 +357,9 @@ def route(x, w, top_k, bias=None, logits_order=LOGITS_FMA, exp_kind=EXP_DECLARED
     return ids, weights, scores, logits
 
 
-def route_select(scores, top_k, renorm_eps=0.0, scale=1.0, renormalize=True):
+def route_select(scores, top_k, renorm_eps=0.0, scale=1.0, renormalize=True, renorm_single=True):
     scores = np.ascontiguousarray(scores, np.float32)
-    p = RoutePolicy(scores.size, top_k, 0, 0, renorm_eps, scale, int(renormalize))
+    p = RoutePolicy(scores.size, top_k, 0, 0, renorm_eps, scale, int(renormalize), int(renorm_single))
     ids = np.zeros(top_k, np.uint32)
     weights = np.zeros(top_k, np.float32)
     lib().orc_route_select(C.byref(p), _ptr(scores, f32p), _ptr(ids, u32p), _ptr(weights, f32p))
@@ -382,7 +383,7 @@ class ExpertResult:
 
 def routed_experts(hidden, ffn, top_k, gate, up, down, down_type, codes, deltas, sums, ids, exp_kind=EXP_GFX1151,
                    gate_expert_stride=None, gate_row_stride=None, down_expert_stride=None, down_row_stride=None,
-                   threads=0, want_intermediates=True, down_only_from=None, gate_type=Q4_K):
+                   threads=0, want_intermediates=True, down_only_from=None, gate_type=Q4_K, swiglu_limit=float("inf")):
     """gate/up/down: uint8 arrays holding every expert (GGUF order unless strides are given).
     down_only_from: (h_codes, h_deltas, h_sums) -> run the down phase alone on that image."""
     gate = np.ascontiguousarray(gate, np.uint8)
@@ -394,7 +395,7 @@ def routed_experts(hidden, ffn, top_k, gate, up, down, down_type, codes, deltas,
     drb = down_row_stride or row_bytes(down_type, ffn)
     deb = down_expert_stride or drb * hidden
     w = ExpertWeights(hidden, ffn, 0, top_k, gate_type, down_type, gate.ctypes.data, up.ctypes.data, down.ctypes.data,
-                      geb, grb, deb, drb, exp_kind)
+                      geb, grb, deb, drb, exp_kind, swiglu_limit)
     ids = np.ascontiguousarray(ids, np.uint32)
     n = rows * top_k
     r = ExpertResult()

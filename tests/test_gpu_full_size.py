@@ -56,9 +56,11 @@ def check_rows(layer, y, sel, x, ids_ref, w_ref, gate, up, down, H, ffn, K, comb
     assert np.all(layer.status.cpu().numpy()[sel] == 0)
 
 
-def test_config2_dense_q4k_ffn_full_size(strix):
-    """BASELINE config 2: Q4_K FFN 27648 x 5120 (gate, up) and 5120 x 27648 (down), 8 fp16 rows, every row checked."""
-    H, I, T = 5120, 27648, 8
+@pytest.mark.parametrize("T", [1, 4, 8])
+def test_config2_dense_q4k_ffn_full_size(strix, T):
+    """BASELINE config 2: Q4_K FFN 27648 x 5120 (gate, up) and 5120 x 27648 (down), 1 / 4 / 8 fp16 rows (each batch size runs its
+    own instantiation of the dense sweep), every row checked."""
+    H, I = 5120, 27648
     gen = torch.Generator(device="cuda").manual_seed(2)
     gate, up, down = device_q4k(gen, (1, I), H), device_q4k(gen, (1, I), H), device_q4k(gen, (1, H), I)
     x = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)

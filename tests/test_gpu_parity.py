@@ -205,6 +205,34 @@ def test_router_exact_ties_lane32_order_and_policy_constants(strix):
     assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(sc.cpu().numpy()), bits(s_ref))
 
 
+@pytest.mark.parametrize("experts,hidden,rows", [(128, 2048, 8), (256, 4096, 40)])
+def test_router_with_the_c_library_exp(strix, experts, hidden, rows):
+    """Math::exp = expf of the C library, the exp of the reference's router test oracle (tests/hip_moe_route_launcher_tests.hip:329):
+    ids, weights and scores equal the oracle's (whose exp is the host library's expf) bit for bit, for the decode and the batch
+    router and through the fused layer entry."""
+    rng = np.random.default_rng(experts + 1)
+    x = rng.standard_normal((rows, hidden)).astype(np.float16)
+    wr = (rng.standard_normal((experts, hidden)) * 0.05).astype(np.float32)
+    ids, wts, scores = strix.route(dev(x), dev(wr), 8, exp_kind=strix.EXP_LIBM)
+    ids_ref, w_ref, s_ref, _ = orc.route(x.astype(np.float32), wr, 8, exp_kind=orc.EXP_LIBM)
+    assert np.array_equal(bits(scores.cpu().numpy()), bits(s_ref))
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    _, _, s_declared, _ = orc.route(x.astype(np.float32), wr, 8, exp_kind=orc.EXP_DECLARED)
+    assert not np.array_equal(bits(s_declared), bits(s_ref))      # the policy field is not ignored
+
+
+def test_router_single_expert_renormalisation(strix):
+    """top_k = 1: the weight is renormalised only when the policy's renorm_single is set (include/strix/moe/route_policy.hpp:146)."""
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((5, 512)).astype(np.float16)
+    wr = (rng.standard_normal((24, 512)) * 0.05).astype(np.float32)
+    for single in (False, True):
+        ids, wts, _ = strix.route(dev(x), dev(wr), 1, renorm_eps=1e-20, scale=2.5, renorm_single=single)
+        ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, 1, renorm_eps=1e-20, scale=2.5, renorm_single=single)
+        assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    assert float(wts[0, 0]) == 2.5
+
+
 # ------------------------------------------------------------------------------------------- routed experts, stage by stage
 def make_layer(rng, H, I, E, full_entropy=False):
     if full_entropy:
@@ -290,6 +318,56 @@ def test_moe_layer_declared_exp_is_bit_exact_end_to_end(strix):
     assert np.array_equal(layer.down_codes[:T * K].cpu().numpy(), ref.h_codes)
     assert np.array_equal(bits(layer.h_out[:T * K].cpu().numpy()), bits(ref.h))
     assert np.array_equal(bits(y), bits(want))
+
+
+@pytest.mark.parametrize("H,I,E,K,T,gate_q5k", [(1024, 512, 8, 4, 9, False), (1024, 512, 8, 4, 2, False), (512, 256, 6, 2, 5, True)])
+def test_swiglu_clamp_trait_in_every_projection_kernel(strix, H, I, E, K, T, gate_q5k):
+    """The SwiGLU clamp (include/strix/moe/activation_policy.hpp:22-24) in the 64-row sweep (9 rows), the 16-row sweep (2 rows)
+    and the Q5_K projection: with the declared exp every bit of h, of its A8 image and of the layer output equals the oracle's,
+    the limit actually binds, and gate_out / up_out keep the RAW projections."""
+    rng = np.random.default_rng(H + T)
+    limit = 0.02
+    if gate_q5k:
+        gate, up = orc.random_q5_k(rng, (E, I), H), orc.random_q5_k(rng, (E, I), H)
+        down = make_layer(rng, H, I, E)[2]
+    else:
+        gate, up, down = make_layer(rng, H, I, E)
+    gt = orc.Q5_K if gate_q5k else orc.Q4_K
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, exp_kind=1, intermediates=True, swiglu_limit=limit,
+                           gate_type=strix.TYPE_Q5_K if gate_q5k else strix.TYPE_Q4_K)
+    y = layer.run(dev(x), dev(ids_ref.astype(np.int32)), dev(w_ref)).cpu().numpy()
+    ref = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref, exp_kind=1, swiglu_limit=limit, gate_type=gt)
+    free = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref, exp_kind=1, gate_type=gt)
+    n = T * K
+    assert np.array_equal(bits(layer.gate_out[:n].cpu().numpy()), bits(ref.gate)) and np.array_equal(bits(ref.gate), bits(free.gate))
+    assert np.array_equal(bits(layer.up_out[:n].cpu().numpy()), bits(ref.up))
+    assert np.array_equal(bits(layer.h_out[:n].cpu().numpy()), bits(ref.h)) and not np.array_equal(bits(ref.h), bits(free.h))
+    assert np.array_equal(layer.down_codes[:n].cpu().numpy(), ref.h_codes) and np.array_equal(bits(layer.down_deltas[:n].cpu().numpy()), bits(ref.h_deltas))
+    assert np.array_equal(bits(y), bits(orc.combine(0, w_ref, ids_ref, ref.rawdots)))
+    assert np.all(layer.status[:T].cpu().numpy() == 0)
+    # the dense entry of the same producer
+    g_d, u_d = layer.gate_out[:n].clone(), layer.up_out[:n].clone()
+    hc, hd, hs, hv, st = strix.swiglu_quantize(g_d, u_d, exp_kind=1, swiglu_limit=limit)
+    assert np.array_equal(hc.cpu().numpy(), ref.h_codes) and np.array_equal(bits(hv.cpu().numpy()), bits(ref.h)) and int(st.sum()) == 0
+
+
+def test_swiglu_clamp_admission(strix):
+    rng = np.random.default_rng(2)
+    gate, up, down = make_layer(rng, 256, 256, 2)
+    x = dev(rng.standard_normal((1, 256)).astype(np.float16))
+    ids, w = dev(np.zeros((1, 1), np.int32)), dev(np.ones((1, 1), np.float32))
+    for bad in (-1.0, float("nan")):
+        layer = strix.MoeLayer(256, 256, 2, 1, dev(gate), dev(up), dev(down), 1, swiglu_limit=bad)
+        with pytest.raises(strix.StrixError) as err:
+            layer.run(x, ids, w)
+        assert err.value.code == strix.E_INVALID_ARGUMENT and "swiglu_limit" in str(err.value)
+    for none in (0.0, float("inf")):          # 0 (the zero-initialised struct) and +infinity both mean "no clamp"
+        layer = strix.MoeLayer(256, 256, 2, 1, dev(gate), dev(up), dev(down), 1, swiglu_limit=none)
+        layer.run(x, ids, w)
 
 
 def test_config3_moe_decode_layer_shape(strix):
@@ -396,7 +474,7 @@ def test_config5_tp_rank_partial_sums(strix):
         check_layer_stages(strix, *out[:7], out[7], H, K, T, 1, 0, TOL_F16)
 
 
-@pytest.mark.parametrize("H,I,batches", [(1280, 1792, (1, 4, 8)), (1024, 2048, (1, 2, 3, 4, 5, 8))])
+@pytest.mark.parametrize("H,I,batches", [(1280, 1792, (1, 4, 5, 6, 7, 8)), (1024, 2048, (1, 2, 3, 4, 5, 8))])
 def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
     """BASELINE config 2 structure at reduced size: a dense Q4_K FFN is the one-expert, top-1, weight-1 layer. The second
     shape (row lengths that are multiples of 4 super-blocks) runs the pair-per-lane dense sweep, the first the row-per-lane
@@ -619,8 +697,10 @@ def test_invalid_route_and_nonfinite_projection_fail_closed(strix):
 
 @pytest.mark.parametrize("T", [1, 2, 8, 16])
 def test_layer_entry_nonfinite_input_fails_closed(strix, T):
-    """An infinite input value through the whole-layer entry (the 16-rows-per-wavefront sweep): the row is flagged (activation and projection bits), publishes nothing, the other rows are unaffected,
-    and the status words equal those of the staged entry points."""
+    """An infinite input value through the whole-layer entry: the row is flagged (activation and projection bits) and the job
+    status word carries the non-finite-projection bit, so the down phase of the WHOLE job is skipped and NO row is published -
+    the healthy rows keep status 0 and their previous output, and the caller must read job_status to know that. The ticket
+    words are left zero and a clean call on the same workspace afterwards is unaffected."""
     E, H, I, K = 16, 512, 256, 4
     rng = np.random.default_rng(31 + T)
     gate, up, down = make_layer(rng, H, I, E)
@@ -635,7 +715,7 @@ def test_layer_entry_nonfinite_input_fails_closed(strix, T):
     y, ids, wts, _ = layer.run_layer(dev(x), wrd)
     st = layer.status[:T].cpu().numpy()
     assert st[T - 1] & strix.STATUS_NONFINITE_ACTIVATION and st[T - 1] & strix.STATUS_NONFINITE_PROJECTION
-    assert np.all(st[: T - 1] == 0) and bool((y[T - 1] == -7.0).all())
+    assert np.all(st[: T - 1] == 0) and bool((y[:T] == -7.0).all())          # nothing of the job is published
     assert int(layer.job_status[0]) & strix.STATUS_NONFINITE_PROJECTION
     assert bool((layer.plan[16:272] == 0).all())
     # a clean call on the same workspace afterwards is unaffected

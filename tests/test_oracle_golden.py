@@ -858,6 +858,118 @@ def test_ref_router_policy_and_combine_bits():
     assert np.array_equal(bits(y), bits(y_ref))
 
 
+@needs_ref
+def test_ref_router_libm_exp_scores_and_single_expert_renormalisation():
+    """Math::exp = the C library's expf (the reference's router test oracle) and the policy's renorm_single field, both
+    against the compiled reference policy functions."""
+    import ctypes as C
+    R = orc.ref()
+    rng = np.random.default_rng(31)
+    for experts in (128, 257):
+        z = (rng.standard_normal(experts) * 2.5).astype(np.float32)
+        s_ref = np.zeros(experts, np.float32)
+        assert R.ref_route_scores_softmax(z.ctypes.data_as(orc.f32p), C.c_size_t(experts), s_ref.ctypes.data_as(orc.f32p), 1) == 0
+        _, _, scores, _ = orc.route(np.ones((1, 1), np.float32), z[:, None].copy(), 4, exp_kind=orc.EXP_LIBM)
+        assert np.array_equal(bits(scores[0]), bits(s_ref))
+        _, _, declared, _ = orc.route(np.ones((1, 1), np.float32), z[:, None].copy(), 4, exp_kind=orc.EXP_DECLARED)
+        assert not np.array_equal(bits(declared[0]), bits(s_ref))          # the two Math traits differ in bits
+        for top_k in (1, 2):
+            for renormalize in (0, 1):
+                for single in (0, 1):
+                    ids_ref, w_ref = np.zeros(top_k, np.uint32), np.zeros(top_k, np.float32)
+                    assert R.ref_route_select_policy(experts, top_k, C.c_float(1e-20), C.c_float(2.5), renormalize, single,
+                                                     s_ref.ctypes.data_as(orc.f32p), ids_ref.ctypes.data_as(orc.u32p),
+                                                     w_ref.ctypes.data_as(orc.f32p)) == 0
+                    ids, w = orc.route_select(s_ref, top_k, renorm_eps=1e-20, scale=2.5, renormalize=bool(renormalize), renorm_single=bool(single))
+                    assert np.array_equal(ids, ids_ref) and np.array_equal(bits(w), bits(w_ref)), (top_k, renormalize, single)
+    # top_k = 1: the weight is s * scale unless renorm_single is set (then s / (s + eps) * scale)
+    ids, w = orc.route_select(s_ref, 1, renorm_eps=0.0, scale=2.0, renormalize=True, renorm_single=False)
+    assert bits(w)[0] == bits(np.float32(s_ref[ids[0]] * np.float32(2.0)))
+    ids, w = orc.route_select(s_ref, 1, renorm_eps=0.0, scale=2.0, renormalize=True, renorm_single=True)
+    assert w[0] == np.float32(2.0)
+
+
+def libm_expf_restated(x):
+    """The algorithm the device uses for Math::exp = expf (csrc/device_math.hpp expf_libm), in numpy double precision."""
+    import struct
+    tab = np.array([struct.unpack("<Q", struct.pack("<d", 2.0 ** (i / 32.0)))[0] - (i << 47) for i in range(32)], np.uint64)
+    xd = x.astype(np.float64)
+    z = (float.fromhex("0x1.71547652b82fep+0") * 32.0) * xd
+    kd = z + float.fromhex("0x1.8p+52")
+    ki = kd.view(np.uint64)
+    kd = kd - float.fromhex("0x1.8p+52")
+    r = z - kd
+    s = (tab[(ki % np.uint64(32)).astype(np.int64)] + (ki << np.uint64(47))).view(np.float64)
+    c01 = (float.fromhex("0x1.c6af84b912394p-5") / 32.0 / 32.0 / 32.0) * r + (float.fromhex("0x1.ebfce50fac4f3p-3") / 32.0 / 32.0)
+    y = (float.fromhex("0x1.62e42ff0c52d6p-1") / 32.0) * r + 1.0
+    y = c01 * (r * r) + y
+    return (y * s).astype(np.float32)
+
+
+def test_libm_expf_restatement_equals_the_c_library():
+    """Two million arguments over the softmax range (x <= 0) and beyond: the table-and-cubic algorithm in double precision
+    gives the C library's bits (the table entries are the correctly rounded 2^(i/32), checked against Python's pow here)."""
+    import ctypes as C
+    libm = C.CDLL("libm.so.6")
+    libm.expf.restype, libm.expf.argtypes = C.c_float, [C.c_float]
+    rng = np.random.default_rng(41)
+    x = np.concatenate([-rng.random(1_200_000) * 40.0, rng.standard_normal(500_000) * 6.0, rng.uniform(-87.0, 88.0, 300_000)]).astype(np.float32)
+    got = libm_expf_restated(x)
+    sample = rng.choice(x.size, 60_000, replace=False)
+    want = np.array([libm.expf(float(v)) for v in x[sample]], np.float32)
+    assert np.array_equal(bits(got[sample]), bits(want))
+    # the oracle's EXP_LIBM softmax is that function: one-expert-hot rows give exp(z - max) / sum directly
+    z = np.array([0.0, -1.5, -7.25, -30.0], np.float32)
+    _, _, scores, _ = orc.route(np.ones((1, 1), np.float32), z[:, None].copy(), 1, exp_kind=orc.EXP_LIBM)
+    p = libm_expf_restated(z)
+    total = np.float32(0.0)
+    for v in p:
+        total = np.float32(total + v)
+    assert np.array_equal(bits(scores[0]), bits((p / total).astype(np.float32)))
+
+
+def test_swiglu_clamp_trait():
+    """The clamp acts on the projections before silu(g) * u (gate from above only, up on both sides), a huge limit is no
+    clamp bit for bit, and the fail-closed check stays on the RAW projections (an infinite gate that the clamp would hide
+    still fails)."""
+    rng = np.random.default_rng(43)
+    g = (rng.standard_normal(32) * 6.0).astype(np.float32)
+    u = (rng.standard_normal(32) * 6.0).astype(np.float32)
+    L = 2.5
+    for kind in (orc.EXP_GFX1151, orc.EXP_DECLARED):
+        plain = orc.swiglu_quantize(g, u, kind)
+        huge = orc.swiglu_quantize(g, u, kind, limit=1e30)
+        assert huge[0] == plain[0] == 1 and np.array_equal(huge[1], plain[1]) and bits(huge[2]) == bits(plain[2]) and np.array_equal(bits(huge[4]), bits(plain[4]))
+        clamped = orc.swiglu_quantize(g, u, kind, limit=L)
+        by_hand = orc.swiglu_quantize(np.minimum(g, np.float32(L)), np.clip(u, -np.float32(L), np.float32(L)), kind)
+        assert np.array_equal(clamped[1], by_hand[1]) and bits(clamped[2]) == bits(by_hand[2]) and clamped[3] == by_hand[3]
+        assert np.array_equal(bits(clamped[4]), bits(by_hand[4])) and not np.array_equal(clamped[1], plain[1])
+        low = g.copy(); low[3] = -40.0          # the gate is not clamped from below
+        assert orc.swiglu_quantize(low, u, kind, limit=L)[4][3] == orc.swiglu_quantize(low, np.clip(u, -L, L).astype(np.float32), kind)[4][3]
+        bad = g.copy(); bad[7] = np.inf
+        assert orc.swiglu_quantize(bad, u, kind, limit=L)[0] == 0
+    R = orc.ref()
+    if R is not None:
+        import ctypes as C
+        R.ref_swiglu_clamp.argtypes = [C.c_float, C.c_float, C.c_float, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+        for gv, uv in ((3.0, -9.0), (-8.0, 9.0), (float("nan"), 1.0), (1.0, float("nan")), (2.5, 2.5), (float("inf"), float("-inf"))):
+            a, b = C.c_float(0), C.c_float(0)
+            R.ref_swiglu_clamp(gv, uv, L, C.byref(a), C.byref(b))
+            want_g = gv if not gv > L else L
+            want_u = -L if uv < -L else (L if uv > L else uv)
+            assert (math.isnan(a.value) and math.isnan(want_g)) or a.value == want_g
+            assert (math.isnan(b.value) and math.isnan(want_u)) or b.value == want_u
+            # and the oracle applies exactly that pair: h of a one-value group
+            gg, uu = np.zeros(32, np.float32), np.zeros(32, np.float32)
+            gg[0], uu[0] = gv, uv
+            ok, _, _, _, h = orc.swiglu_quantize(gg, uu, orc.EXP_DECLARED, limit=L)
+            if math.isfinite(gv) and math.isfinite(uv):
+                hh = orc.swiglu_quantize(np.full(32, a.value, np.float32) * (np.arange(32) == 0), np.full(32, b.value, np.float32) * (np.arange(32) == 0), orc.EXP_DECLARED)[4]
+                assert ok == 1 and bits(h)[0] == bits(hh)[0]
+            else:
+                assert ok == 0
+
+
 # ---------------------------------------------------------------- committed reference-generated vectors
 def test_committed_reference_vectors():
     """tests/golden/ref_vectors.npz holds outputs the compiled reference produced (tests/golden/make_ref_vectors.py);
