@@ -214,6 +214,20 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* policy, const float* r
                                 float* scores, const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows,
                                 uint32_t combine_form, mi355_stream);
 
+/* mi355_moe_enqueue_layer with every work buffer inside the library. It has no counterpart in the reference: it is for
+ * callers that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation). The caller passes only inputs and outputs: the policy, router and expert tensors, the input rows, and the
+ * row outputs routes / route_weights [rows][top_k], status [rows], output [rows][output_stride] (base: optional [rows][hidden]).
+ * Router scores, the A8 images, the expert plan, the unweighted down outputs and the job status word live in a device array
+ * of about 5.1 MB that is part of the library image (each device the library runs on holds its own copy until the process
+ * ends). Limits: rows <= 16, top_k <= 8, hidden <= 8192, ffn <= 4096, experts <= 1024; beyond them the call returns
+ * MI355_E_INVALID_ARGUMENT. The call allocates nothing and computes the same bits as mi355_moe_enqueue_layer. Every call on
+ * a device shares that device's array: two calls that overlap on one device (different streams or threads) race. */
+int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
+                                       const mi355_moe_weights*, const void* input, uint32_t input_kind, uint64_t input_stride,
+                                       uint32_t rows, uint32_t* routes, float* route_weights, uint32_t* status, const float* base,
+                                       float* output, uint64_t output_stride, uint32_t combine_form, mi355_stream);
+
 /* The routed experts of a prefill batch on the matrix cores - the path's FAST arithmetic class (the reference's
  * bit-changing MMA forms: include/strix/cuda/qwen_moe.hpp:100-101 moe_mma, known_rows::enqueue_prefill
  * include/strix/hip_moe_q4k_a8_known_rows.hpp:109-111). The integers sc * q of the Q4_K blocks (exact in fp16) are multiplied

@@ -82,7 +82,7 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32"]
 
 
@@ -246,6 +246,15 @@ class MoeLayer:
         check(lib().mi355_moe_enqueue_layer(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), C.byref(self.w), C.byref(rv), rows,
                                             combine, _stream()))
         return self.output[:rows], self.ids[:rows], self.route_w[:rows], self.scores[:rows]
+
+    def run_layer_static(self, x, router_weight, ids, route_w, status, output, bias=None, base=None, combine=COMBINE_FMA_SLOT):
+        """mi355_moe_enqueue_layer_static: the work buffers are the library's own; only inputs and outputs are passed."""
+        rows = x.shape[0]
+        p = RoutePolicy(self.experts, self.top_k, LOGITS_FMA, 0.0, 1.0, 1, 1, EXP_DECLARED)
+        check(lib().mi355_moe_enqueue_layer_static(C.byref(p), _p(router_weight), _p(bias), C.byref(self.w), _p(x), input_kind(x),
+                                                   C.c_uint64(x.stride(0) * x.element_size()), rows, _p(ids), _p(route_w), _p(status), _p(base),
+                                                   _p(output), C.c_uint64(output.stride(0)), combine, _stream()))
+        return output[:rows]
 
     def stage(self, name, x, ids, weights, base=None, combine=COMBINE_FMA_SLOT):
         rows, rv = self.rows_view(x, ids, weights, base)

@@ -1434,4 +1434,72 @@ int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows,
     return MI355_OK;
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// mi355_moe_enqueue_layer for callers that cannot allocate: every work buffer of the layer (router scores, the A8 images
+// of the input and of h, the expert plan, the unweighted down outputs, the job status word) lives in a file-scope device
+// array of a fixed size instead of caller memory. Each device holds its own copy of that array; its address on a device is
+// looked up once (hipGetSymbolAddress with that device current) and kept, and only that address - never the array's name -
+// is handed to kernels.
+namespace {
+constexpr uint32_t kStaticRows = 16, kStaticTopK = 8, kStaticHidden = 8192, kStaticFfn = 4096, kStaticExperts = 1024;
+constexpr uint32_t kStaticAssignments = kStaticRows * kStaticTopK;
+constexpr size_t align256(size_t v) { return (v + 255U) & ~static_cast<size_t>(255U); }
+constexpr size_t kStaticPlanAt = 0;
+constexpr size_t kStaticJobAt = kStaticPlanAt + align256(4U * static_cast<size_t>(plan_words_total(kStaticExperts, kStaticAssignments)));
+constexpr size_t kStaticScoresAt = kStaticJobAt + 256U;
+constexpr size_t kStaticCodesAt = kStaticScoresAt + align256(4U * static_cast<size_t>(kStaticRows) * kStaticExperts);
+constexpr size_t kStaticDeltasAt = kStaticCodesAt + align256(static_cast<size_t>(kStaticRows) * kStaticHidden);
+constexpr size_t kStaticSumsAt = kStaticDeltasAt + align256(4U * static_cast<size_t>(kStaticRows) * (kStaticHidden / 32U));
+constexpr size_t kStaticDownCodesAt = kStaticSumsAt + align256(4U * static_cast<size_t>(kStaticRows) * (kStaticHidden / 32U));
+constexpr size_t kStaticDownDeltasAt = kStaticDownCodesAt + align256(static_cast<size_t>(kStaticAssignments) * kStaticFfn);
+constexpr size_t kStaticDownSumsAt = kStaticDownDeltasAt + align256(4U * static_cast<size_t>(kStaticAssignments) * (kStaticFfn / 32U));
+constexpr size_t kStaticRawdotsAt = kStaticDownSumsAt + align256(4U * static_cast<size_t>(kStaticAssignments) * (kStaticFfn / 32U));
+constexpr size_t kStaticBytes = kStaticRawdotsAt + align256(4U * static_cast<size_t>(kStaticAssignments) * kStaticHidden);    // about 5.1 MB
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];     // zero at load: the plan's ticket words start at zero
+namespace {
+std::atomic<unsigned char*> g_scratch_of_device[64];
+// the array's address on the current device (looked up on the first call there); nullptr with the reason in g_error
+unsigned char* scratch_on_current_device() {
+    int device = -1;
+    const hipError_t e0 = hipGetDevice(&device);
+    if (e0 != hipSuccess) { hip_fail(e0, "static workspace: hipGetDevice"); return nullptr; }
+    if (device < 0 || device >= 64) { fail(MI355_E_UNSUPPORTED, "static workspace: device ordinal beyond 63"); return nullptr; }
+    unsigned char* known = g_scratch_of_device[device].load(std::memory_order_acquire);
+    if (known) return known;
+    void* found = nullptr;
+    const hipError_t e1 = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (e1 != hipSuccess || !found) { hip_fail(e1, "static workspace: hipGetSymbolAddress"); return nullptr; }
+    g_scratch_of_device[device].store(static_cast<unsigned char*>(found), std::memory_order_release);   // (a racing first call stores the same address)
+    return static_cast<unsigned char*>(found);
+}
+}  // namespace
+
+int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float* router_weight, const float* logit_bias,
+                                       const mi355_moe_weights* w, const void* input, uint32_t input_kind, uint64_t input_stride,
+                                       uint32_t rows, uint32_t* routes, float* route_weights, uint32_t* status, const float* base,
+                                       float* output, uint64_t output_stride, uint32_t form, mi355_stream stream) {
+    STRIX_REQUIRE(p && w, "moe layer (static workspace): null policy or weights");
+    STRIX_REQUIRE(rows >= 1U && rows <= kStaticRows, "moe layer (static workspace): rows must be within 1..16");
+    STRIX_REQUIRE(w->top_k >= 1U && w->top_k <= kStaticTopK, "moe layer (static workspace): top_k must be within 1..8");
+    STRIX_REQUIRE(w->hidden <= kStaticHidden && w->ffn <= kStaticFfn && w->experts <= kStaticExperts,
+                  "moe layer (static workspace): hidden <= 8192, ffn <= 4096 and experts <= 1024 are the limits of the built-in workspace");
+    STRIX_REQUIRE(routes && route_weights && status && output && input, "moe layer (static workspace): null row view");
+    unsigned char* ws = scratch_on_current_device();
+    if (!ws) return g_error.rfind("static workspace: device", 0) == 0 ? MI355_E_UNSUPPORTED : MI355_E_HIP;
+    mi355_moe_rows r{};
+    r.input = input; r.input_kind = input_kind; r.input_stride = input_stride;
+    r.routes = routes; r.route_weights = route_weights; r.status = status; r.base = base; r.output = output; r.output_stride = output_stride;
+    r.plan = reinterpret_cast<uint32_t*>(ws + kStaticPlanAt);
+    r.job_status = reinterpret_cast<uint32_t*>(ws + kStaticJobAt);
+    r.codes = reinterpret_cast<int8_t*>(ws + kStaticCodesAt);
+    r.deltas = reinterpret_cast<float*>(ws + kStaticDeltasAt);
+    r.sums = reinterpret_cast<int32_t*>(ws + kStaticSumsAt);
+    r.down_codes = reinterpret_cast<int8_t*>(ws + kStaticDownCodesAt);
+    r.down_deltas = reinterpret_cast<float*>(ws + kStaticDownDeltasAt);
+    r.down_sums = reinterpret_cast<int32_t*>(ws + kStaticDownSumsAt);
+    r.rawdots = reinterpret_cast<float*>(ws + kStaticRawdotsAt);
+    return mi355_moe_enqueue_layer(p, router_weight, logit_bias, reinterpret_cast<float*>(ws + kStaticScoresAt), w, &r, rows, form, stream);
+}
+
 }  // extern "C"

@@ -107,6 +107,10 @@ def test_every_layer_entry_refuses_an_oversized_batch_before_its_first_launch(li
     # the clamp trait is validated with the rest of the weights
     bad = pkg.MoeWeights(512, 256, 8, 1, 12, 12, 0x1000, 0x2000, 0x3000, 0, 0, 0, 0, 0, -2.0)
     assert lib.mi355_moe_enqueue(C.byref(bad), C.byref(rows), 4, 0, None) == -1 and b"swiglu_limit" in lib.mi355_last_error()
+    # the entry with a built-in workspace states its limits
+    assert lib.mi355_moe_enqueue_layer_static(C.byref(policy), C.c_void_p(0x5000), None, C.byref(w), C.c_void_p(0x4000), 1, C.c_uint64(1024), 17,
+                                              C.c_void_p(0x4000), C.c_void_p(0x4000), C.c_void_p(0x4000), None, C.c_void_p(0x4000), C.c_uint64(512), 0, None) == -1
+    assert b"1..16" in lib.mi355_last_error()
 
 
 def test_product_path_never_references_the_oracle():

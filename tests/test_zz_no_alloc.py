@@ -1,0 +1,49 @@
+"""The allocation-free layer entry (mi355_moe_enqueue_layer_static) against mi355_moe_enqueue_layer: same bits, on two calls in
+a row, the second with a smaller input; and its size limits are refused before anything runs."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(strix, H, I, E, K, T, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    q = lambda shape: strix.quantize_weight_rows(strix.TYPE_Q4_K, torch.randn(shape, generator=g, device="cuda") * 0.02)
+    gate, up, down = q((E, I, H)), q((E, I, H)), q((E, H, I))
+    wr = torch.randn((E, H), generator=g, device="cuda") * 0.02
+    x = torch.randn((T, H), generator=g, device="cuda").to(torch.float16)
+    return strix.MoeLayer(H, I, E, K, gate, up, down, T), wr, x
+
+
+@pytest.mark.parametrize("H,I,E,K,T,T2", [(2048, 768, 128, 8, 8, 3), (1024, 512, 16, 4, 16, 1), (6144, 1280, 160, 8, 16, 5)])
+def test_static_workspace_layer_equals_the_caller_workspace_layer(strix, H, I, E, K, T, T2):
+    layer, wr, x = _layer(strix, H, I, E, K, T, seed=H + T)
+    for rows in (T, T2):                       # two calls in a row, the second with fewer rows
+        xs = x[:rows].contiguous()
+        want, ids, wts, _ = layer.run_layer(xs, wr)
+        want, ids, wts = want.clone(), ids.clone(), wts.clone()
+        want_status = layer.status[:rows].clone()
+        ids2 = torch.full((rows, K), -1, dtype=torch.int32, device="cuda")
+        wts2 = torch.full((rows, K), -1.0, dtype=torch.float32, device="cuda")
+        status2 = torch.full((rows,), 77, dtype=torch.int32, device="cuda")
+        out2 = torch.full((rows, H), -7.0, dtype=torch.float32, device="cuda")
+        got = layer.run_layer_static(xs, wr, ids2, wts2, status2, out2)
+        torch.cuda.synchronize()
+        assert torch.equal(ids2, ids)
+        assert np.array_equal(wts2.cpu().numpy().view(np.uint32), wts.cpu().numpy().view(np.uint32))
+        assert torch.equal(status2, want_status) and int(status2.sum()) == 0
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.cpu().numpy().view(np.uint32))
+
+
+def test_static_workspace_layer_refuses_sizes_beyond_its_limits(strix):
+    layer, wr, x = _layer(strix, 1024, 512, 16, 4, 17, seed=5)
+    ids = torch.zeros((17, 4), dtype=torch.int32, device="cuda")
+    wts = torch.zeros((17, 4), dtype=torch.float32, device="cuda")
+    status = torch.zeros(17, dtype=torch.int32, device="cuda")
+    out = torch.full((17, 1024), -7.0, dtype=torch.float32, device="cuda")
+    with pytest.raises(strix.StrixError) as err:
+        layer.run_layer_static(x, wr, ids, wts, status, out)
+    assert err.value.code == strix.E_INVALID_ARGUMENT and "1..16" in str(err.value)
+    torch.cuda.synchronize()
+    assert bool((out == -7.0).all())
