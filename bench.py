@@ -9,7 +9,9 @@ tokens), as consecutive layers of a model do.
 
 Prints ONE JSON line. `value` = microseconds per layer (lower is better). `roofline` prices the dominant kernel (gate/up
 projection) by its algorithmic bytes against the 8 TB/s HBM peak, from HIP events recorded around that kernel on its own
-stream inside this run. `cpu_baseline` times the CPU oracle (a port of the reference's CPU path) on the same layer."""
+stream inside this run. `prefill` is the metric's second figure: BASELINE config 4 (4096 rows) on the matrix cores, TFLOP/s against
+the fp16 MFMA peak. `cpu_baseline` times the CPU oracle (a port of the reference's CPU path) on the same layer, with the
+compiled reference's own Executor beside it where that library was built, the host CPU model and its read-bandwidth ceiling."""
 import argparse
 import json
 import os
@@ -24,6 +26,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0     # MI355X published HBM3E peak
+MFMA_F16_PEAK_FLOPS = 2.5e15     # MI355X published dense fp16 MFMA peak
 # HBM bytes per launch of the gate/up kernel on the default workload, from two rocprofv3 --pmc passes (FETCH_SIZE scaled
 # x2.000, WRITE_SIZE x1.000 by a 256 MiB device copy in the same runs): profiles/project_wave_kernel_config3_moe_decode_T8.txt
 PROJECT_TRAFFIC_BYTES_DEFAULT = 99_892_019 + 147_661
@@ -38,6 +41,7 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8)
     ap.add_argument("--layers", type=int, default=6, help="independent layers rotated through (cold-cache working set)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the config-4 prefill leg")
     ap.add_argument("--extra", action="store_true",
                     help="also time BASELINE configs 1, 2, 4 and 5 (reported under 'extra'; the headline value stays config 3)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -225,6 +229,60 @@ def extra_config3_executor_formats(strix, torch, cfg, steps, warmup, with_cpu):
     return out
 
 
+def prefill_config4(strix, torch, gen, keep=False, reps=10):
+    """BASELINE config 4: 4096 fp16 rows, hidden 4096, 256 routed Q4_K experts top-8 (router logits + N(0, 1.5) per-expert bias:
+    Zipf-like load) of intermediate 2048, plus the always-on shared Q8_0 expert; router + shared expert + routed experts +
+    ordered combine on the matrix cores (mi355_moe_enqueue_prefill_f16: exact integer operands, fp32 block scales and
+    accumulation). FLOPs: the algorithmic 2 x rows x (8 + 1) x 3 x 2048 x 4096 + the router's."""
+    H, I, E, K, T = 4096, 2048, 256, 8, 4096
+    gate, up, down = (device_q4k(torch, gen, (E, I), H, 0x03), device_q4k(torch, gen, (E, I), H, 0x03), device_q4k(torch, gen, (E, H), I, 0x03))
+    wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
+    bias = torch.randn(E, device="cuda", generator=gen) * 1.5
+    xp = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)
+    layer = strix.MoeLayer(H, I, E, K, gate, up, down, T, prefill_f16=True)
+    flops_experts, flops_router, flops_shared = 2.0 * T * K * 3 * I * H, 2.0 * T * E * H, 2.0 * T * 3 * I * H
+    ids, wts, _ = strix.route(xp, wr, K, bias=bias)
+    sec_route = time_steps(torch, lambda i: strix.route(xp, wr, K, bias=bias), 5, 2)
+    sec_f16 = time_steps(torch, lambda i: layer.run_prefill_f16(xp, ids, wts), reps, 3)
+
+    def q8(rows, width):
+        w = torch.randint(0, 256, (rows, width // 32, 34), dtype=torch.uint8, device="cuda", generator=gen)
+        w[..., 1] = (w[..., 1] & 0x03) | 0x14
+        return w.reshape(rows, -1)
+    sg, su, sd = q8(I, H), q8(I, H), q8(H, I)
+    # the shared expert: a one-expert layer in the same prefill form, its output the base of the routed combine
+    dense = strix.MoeLayer(H, I, 1, 1, sg.reshape(1, I, -1), su.reshape(1, I, -1), sd.reshape(1, H, -1), T, prefill_f16=True,
+                           gate_type=strix.TYPE_Q8_0, down_type=strix.TYPE_Q8_0)
+    zero_ids = torch.zeros((T, 1), dtype=torch.int32, device="cuda")
+    ones = torch.ones((T, 1), dtype=torch.float32, device="cuda")
+    sec_shared = time_steps(torch, lambda i: dense.run_prefill_f16(xp, zero_ids, ones), reps, 3)
+
+    def whole(i):
+        r_ids, r_wts, _ = strix.route(xp, wr, K, bias=bias)
+        return layer.run_prefill_f16(xp, r_ids, r_wts, base=dense.run_prefill_f16(xp, zero_ids, ones))
+    sec_whole = time_steps(torch, whole, reps, 3)
+    if int(layer.status.sum()) or int(dense.status.sum()):
+        raise RuntimeError("config 4: the prefill run set row status bits (non-finite or out-of-range values): the timing is void")
+    total = flops_experts + flops_router + flops_shared
+    out = {
+        "workload": "BASELINE config 4: 4096 fp16 rows, hidden 4096, 256 routed Q4_K experts top-8 (biased router) + 1 shared Q8_0 expert, intermediate 2048",
+        "ms": sec_whole * 1e3, "TFLOPs": total / sec_whole / 1e12, "frac": total / sec_whole / MFMA_F16_PEAK_FLOPS, "peak": MFMA_F16_PEAK_FLOPS / 1e12,
+        "unit": "TFLOP/s", "bound": "mfma", "dtype": "f16 operands, f32 accumulation", "algorithmic_flops": total,
+        "kernel": "prefill_f16_kernel (gate/up + SwiGLU, then down) of the routed experts",
+        "experts_ms": sec_f16 * 1e3, "experts_TFLOPs": flops_experts / sec_f16 / 1e12, "experts_frac": flops_experts / sec_f16 / MFMA_F16_PEAK_FLOPS,
+        "router_ms": sec_route * 1e3, "shared_expert_ms": sec_shared * 1e3, "shared_expert_TFLOPs": flops_shared / sec_shared / 1e12,
+        "note": "FAST class (fp16 MFMA on exact integer operands sc*q, fp32 block scales and accumulation), tolerance 2e-3 against the exact-weight product; router exact-order"}
+    if keep:
+        # the same expert in the integer-dot class (A8 image, gate / up, SwiGLU + A8, down), for the comparison in --extra
+        def shared(i):
+            c, d, _, _ = strix.quantize_a8(xp)
+            hc, hd, _, _, _ = strix.swiglu_quantize(strix.gemv_q8_0_a8(sg, c, d, H, I), strix.gemv_q8_0_a8(su, c, d, H, I))
+            return strix.gemv_q8_0_a8(sd, hc, hd, I, H)
+        out["shared_expert_integer_class_ms"] = time_steps(torch, shared, 3, 1) * 1e3
+        return out, layer, xp, wr, bias
+    return out
+
+
 def extra_configs(strix, torch, steps, warmup):
     """BASELINE configs 1, 2, 4, 5 on synthetic full-entropy blocks; HBM-bound ones rotate over enough weight sets to stay cold."""
     gen = torch.Generator(device="cuda").manual_seed(11)
@@ -301,57 +359,11 @@ def extra_configs(strix, torch, steps, warmup):
     out["config5_tp_rank_shard_T16"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
                                         "algorithmic_bytes": nbytes, "distinct_experts_mean": u}
     del layer
-    # config 4: 4096-row prefill, hidden 4096, 256 experts top-8 (+ logit bias), intermediate 2048; routed experts + router
+    # config 4 (the 4096-row prefill) on the matrix cores, and the same work in the bit-exact integer-dot class
+    pf, layer, xp, wr, bias = prefill_config4(strix, torch, gen, keep=True)
+    out["config4_prefill_T4096_f16_mfma"] = pf
     H, I, E, K, T = 4096, 2048, 256, 8, 4096
-    layer = strix.MoeLayer(H, I, E, K, device_q4k(torch, gen, (E, I), H, 0x03), device_q4k(torch, gen, (E, I), H, 0x03),
-                           device_q4k(torch, gen, (E, H), I, 0x03), T)
-    wr = torch.randn((E, H), device="cuda", generator=gen) * 0.02
-    bias = torch.randn(E, device="cuda", generator=gen) * 1.5
-    xp = torch.randn((T, H), device="cuda", generator=gen).to(torch.float16)
-    layer = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, T, prefill_f16=True)
     flops_experts, flops_router = 2.0 * T * K * 3 * I * H, 2.0 * T * E * H
-    ids, wts, _ = strix.route(xp, wr, K, bias=bias)
-    sec_route = time_steps(torch, lambda i: strix.route(xp, wr, K, bias=bias), 5, 2)
-    sec_f16 = time_steps(torch, lambda i: layer.run_prefill_f16(xp, ids, wts), 10, 3)
-    out["config4_prefill_T4096_f16_mfma"] = {
-        "ms": (sec_f16 + sec_route) * 1e3, "experts_ms": sec_f16 * 1e3, "router_ms": sec_route * 1e3,
-        "TFLOPs": (flops_experts + flops_router) / (sec_f16 + sec_route) / 1e12, "experts_TFLOPs": flops_experts / sec_f16 / 1e12,
-        "frac_of_fp16_mfma_peak": (flops_experts + flops_router) / (sec_f16 + sec_route) / 2.5e15,
-        "experts_frac_of_fp16_mfma_peak": flops_experts / sec_f16 / 2.5e15, "algorithmic_flops": flops_experts + flops_router,
-        "note": "routed experts on fp16 MFMA (exact integer operands sc*q, fp32 block scales, fp32 accumulation) + exact-order router; FAST class, tolerance 2e-3"}
-    # the always-on shared expert (Q8_0, same intermediate size); first in the integer-dot class: A8 image, gate / up, SwiGLU + A8, down
-    def q8(rows, width):
-        w = torch.randint(0, 256, (rows, width // 32, 34), dtype=torch.uint8, device="cuda", generator=gen)
-        w[..., 1] = (w[..., 1] & 0x03) | 0x14
-        return w.reshape(rows, -1)
-    sg, su, sd = q8(I, H), q8(I, H), q8(H, I)
-
-    def shared(i):
-        c, d, _, _ = strix.quantize_a8(xp)
-        hc, hd, _, _, _ = strix.swiglu_quantize(strix.gemv_q8_0_a8(sg, c, d, H, I), strix.gemv_q8_0_a8(su, c, d, H, I))
-        return strix.gemv_q8_0_a8(sd, hc, hd, I, H)
-    sec_shared_int = time_steps(torch, shared, 3, 1)
-    # the same expert on the matrix cores: a one-expert layer in the prefill form, its output the base of the routed combine
-    dense = strix.MoeLayer(H, I, 1, 1, sg.reshape(1, I, -1), su.reshape(1, I, -1), sd.reshape(1, H, -1), T, prefill_f16=True,
-                           gate_type=strix.TYPE_Q8_0, down_type=strix.TYPE_Q8_0)
-    zero_ids = torch.zeros((T, 1), dtype=torch.int32, device="cuda")
-    ones = torch.ones((T, 1), dtype=torch.float32, device="cuda")
-    sec_shared = time_steps(torch, lambda i: dense.run_prefill_f16(xp, zero_ids, ones), 10, 3)
-
-    def whole(i):
-        r_ids, r_wts, _ = strix.route(xp, wr, K, bias=bias)
-        return layer.run_prefill_f16(xp, r_ids, r_wts, base=dense.run_prefill_f16(xp, zero_ids, ones))
-    sec_whole = time_steps(torch, whole, 10, 3)
-    if int(layer.status.sum()) or int(dense.status.sum()):
-        raise RuntimeError("config 4: the prefill run set row status bits (non-finite or out-of-range values): the timing is void")
-    flops_shared = 2.0 * T * 3 * I * H
-    out["config4_prefill_T4096_f16_mfma"].update({
-        "shared_expert_ms": sec_shared * 1e3, "shared_expert_TFLOPs": flops_shared / sec_shared / 1e12,
-        "shared_expert_integer_class_ms": sec_shared_int * 1e3,
-        "with_shared_expert_ms": sec_whole * 1e3,
-        "with_shared_expert_TFLOPs": (flops_experts + flops_router + flops_shared) / sec_whole / 1e12,
-        "with_shared_expert_frac_of_fp16_mfma_peak": (flops_experts + flops_router + flops_shared) / sec_whole / 2.5e15})
-    del sg, su, sd, dense
     sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 2, 1)
     out["config4_prefill_T4096_integer_class"] = {
         "ms": sec * 1e3, "TFLOPs": (flops_experts + flops_router) / sec / 1e12, "algorithmic_flops": flops_experts + flops_router,
@@ -368,6 +380,73 @@ def time_steps(torch, fn, steps, warmup):
         fn(warmup + i)
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps
+
+
+def host_cpu_info(threads):
+    """Host CPU model, the vector ISA flags that matter to the reference's CPU kernels, and a plain multi-thread read-bandwidth
+    ceiling (method of the reference's scripts/bench/residency/cpu_expert_bench.cpp:131-147)."""
+    import ctypes as C
+    import orc
+    model, flags = "unknown", set()
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name") and model == "unknown":
+                model = line.split(":", 1)[1].strip()
+            if line.startswith("flags") and not flags:
+                flags = set(line.split(":", 1)[1].split())
+    except OSError:
+        pass
+    isa = [f for f in ("avx2", "avx_vnni", "avx512f", "avx512bw", "avx512_vnni", "amx_int8") if f in flags]
+    buf = np.ones(1 << 27, np.uint64)      # 1 GiB
+    L = orc.lib()
+    L.orc_read_seconds.restype = C.c_double
+    L.orc_read_seconds.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
+    L.orc_read_seconds(buf.ctypes.data, buf.size, 1, threads, None)
+    sec = L.orc_read_seconds(buf.ctypes.data, buf.size, 4, threads, None) / 4.0
+    return {"cpu_model": model, "isa_flags": isa, "read_bandwidth_GBps": buf.nbytes / sec / 1e9, "read_bandwidth_threads": threads}
+
+
+def reference_executor_config3(cfg, torch, strix, budget_s=4.0):
+    """The compiled reference's own Executor (its best ISA, every host thread) on layer 0's expert job of the same geometry with
+    the down tensors in Q8_0 - the executor has no Q4_K down rows (src/cpu/core/routed_expert.hpp:28), so the gate/up tensors,
+    tokens and routes are the workload's and only the down tensor's format differs. None where oracle/_ref was not built."""
+    import ctypes as C
+    import orc
+    R = orc.ref()
+    if R is None:
+        return None
+    layer, wr, x = cfg.layers[0]
+    H, I, E, K, T = cfg.H, cfg.I, cfg.E, cfg.K, cfg.T
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    down = device_blocks(torch, gen, E * H, I // 32, 34, (1,), 0x14).cpu().numpy()
+    gate, up = layer.gate.cpu().numpy(), layer.up.cpu().numpy()
+    xn = x.cpu().numpy().astype(np.float32)
+    ids, _, _, _ = orc.route(xn, wr.cpu().numpy(), K)
+    c, d, s, _ = orc.quantize_a8(xn)
+    asg = np.array([[t, k, ids[t, k]] for t in range(T) for k in range(K)], np.uint32)
+    raw, status = np.zeros((T, K, H), np.float32), np.zeros(T, np.uint32)
+    threads = orc.lib().orc_max_threads()
+    R.ref_executor_run.restype = C.c_int
+    pool = C.c_void_p(R.ref_executor_create(threads, 1))
+
+    def run():
+        return R.ref_executor_run(pool, H, I, gate.ctypes.data_as(orc.u8p), up.ctypes.data_as(orc.u8p), down.ctypes.data_as(orc.u8p), 0,
+                                  c.ctypes.data_as(orc.i8p), d.ctypes.data_as(orc.f32p), s.ctypes.data_as(orc.i32p), T,
+                                  asg.ctypes.data_as(orc.u32p), T * K, raw.ctypes.data_as(orc.f32p), C.c_uint64(K * H),
+                                  status.ctypes.data_as(orc.u32p))
+    out = None
+    if run() == 0:
+        times, t_end = [], time.perf_counter() + budget_s
+        while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
+            t0 = time.perf_counter()
+            run()
+            times.append(time.perf_counter() - t0)
+        out = {"value": statistics.median(times) * 1e6, "unit": "us/expert job", "cores": threads, "kind": "reference",
+               "isa": R.ref_executor_isa(pool).decode(),
+               "sample": f"the reference's Executor on layer 0's expert job (gate/up/SwiGLU/down of {T * K} assignments; no router, no combine) "
+                         f"with the workload's Q4_K gate/up tensors and a Q8_0 down tensor, median of {len(times)} passes"}
+    R.ref_executor_destroy(pool)
+    return out
 
 
 def cpu_baseline_config3(cfg, budget_s=12.0):
@@ -394,7 +473,8 @@ def cpu_baseline_config3(cfg, budget_s=12.0):
     med = statistics.median(times)
     return {"value": med * 1e6, "unit": "us/layer", "cores": threads, "kind": "port",
             "sample": f"layer 0 of the same config-3 workload (T={T}), median of {len(times)} passes after one warm-up; "
-                      "scalar C restatement of the reference CPU path, OpenMP over (assignment, 32-output group) and (assignment, output)"}
+                      "C restatement of the reference CPU path (group dots vectorised by the compiler for the host ISA, the fp32 chain scalar), "
+                      "OpenMP over (assignment, 32-output group) and (assignment, output)"}
 
 
 def main():
@@ -457,8 +537,17 @@ def main():
         small.update(extra_config3_executor_formats(strix, torch, cfg, args.steps, args.warmup, not args.no_cpu))
         del cfg.layers[1:]
         out["extra"] = {**small, **extra_configs(strix, torch, args.steps, args.warmup)}
+    if args.extra:
+        out["prefill"] = out["extra"]["config4_prefill_T4096_f16_mfma"]
+    elif not args.no_prefill:
+        # the second target of the metric: the 4096-row prefill on the matrix cores (BASELINE config 4, whole layer)
+        del cfg.layers[1:]
+        torch.cuda.empty_cache()
+        out["prefill"] = prefill_config4(strix, torch, torch.Generator(device="cuda").manual_seed(11))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_config3(cfg)
+        out["cpu_baseline"]["reference_executor"] = reference_executor_config3(cfg, torch, strix)
+        out["cpu_baseline"]["host"] = host_cpu_info(out["cpu_baseline"]["cores"])
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -22,6 +22,22 @@ static inline int is_finite(float x) { return (bits_of(x) & 0x7f800000U) != 0x7f
 static inline uint16_t le16(const uint8_t* p) { return (uint16_t)(p[0] | ((unsigned)p[1] << 8)); }
 static inline uint32_t le32(const uint8_t* p) { uint32_t v; memcpy(&v, p, 4); return v; }
 
+/* Plain multi-thread read of a buffer (sum of its 64-bit words), seconds for `reps` passes: the host's memory-read ceiling
+ * next to the CPU baseline (method of the reference's scripts/bench/residency/cpu_expert_bench.cpp:131-147). */
+double orc_read_seconds(const uint64_t* buffer, size_t words, int reps, int threads, uint64_t* checksum) {
+    uint64_t total = 0;
+    const double t0 = omp_get_wtime();
+    for (int r = 0; r < reps; ++r) {
+        uint64_t sum = 0;
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static) reduction(+ : sum)
+        for (size_t i = 0; i < words; ++i) sum += buffer[i];
+        total += sum;
+    }
+    const double t1 = omp_get_wtime();
+    if (checksum) *checksum = total;
+    return t1 - t0;
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();
@@ -245,6 +261,23 @@ void orc_rmsnorm_f32(const float* x, const float* w, uint32_t n, float eps, floa
 }
 
 /* ------------------------------------------------------------------ Q4_K x A8 row */
+/* The exact int32 group dots of one super-block (dot[j] = sum_k code * nibble, sub-block j = 2p low / 2p + 1 high nibbles of
+ * bytes 32p .. 32p + 31). Integer arithmetic only, so the compiler may vectorise it for whatever the host offers (the clones
+ * are picked at load time); the fp32 chain around it stays scalar and in the declared order. */
+__attribute__((target_clones("arch=skylake-avx512", "avx2", "default"), optimize("O3")))
+static void q4k_block_dots(const uint8_t* qs, const int8_t* codes, int dot[8]) {
+    for (uint32_t p = 0; p < 4; ++p) {
+        int lo = 0, hi = 0;
+        for (uint32_t k = 0; k < 32; ++k) {
+            const uint8_t byte = qs[32 * p + k];
+            lo += (int)codes[64 * p + k] * (int)(byte & 15);
+            hi += (int)codes[64 * p + 32 + k] * (int)(byte >> 4);
+        }
+        dot[2 * p] = lo;
+        dot[2 * p + 1] = hi;
+    }
+}
+
 float orc_q4k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,
                      const int32_t* sums) {
     float acc[4] = {0.0F, 0.0F, 0.0F, 0.0F};
@@ -252,14 +285,10 @@ float orc_q4k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, 
         const uint8_t* blk = wrow + (size_t)b * ORC_Q4_K_BLOCK;
         const float d = orc_half_to_float(le16(blk)), dm = orc_half_to_float(le16(blk + 2));
         float x[8];
+        int dots[8];
+        q4k_block_dots(blk + 16, codes + 256 * b, dots);
         for (uint32_t j = 0; j < 8; ++j) {
-            const uint32_t p = j >> 1, hi = j & 1;
-            int dot = 0;
-            for (uint32_t k = 0; k < 32; ++k) {
-                const uint8_t byte = blk[16 + 32 * p + k];
-                const int q = hi ? (byte >> 4) : (byte & 15);
-                dot += (int)codes[256 * b + 32 * j + k] * q;
-            }
+            const int dot = dots[j];
             const float D = d * (float)orc_q4k_factor_words(blk, j, 0);
             const float DM = dm * (float)orc_q4k_factor_words(blk, j, 1);
             const float u = D * (float)dot;

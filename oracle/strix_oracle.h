@@ -166,6 +166,8 @@ void orc_base_linear(uint32_t type, const uint8_t* weight, uint64_t row_stride, 
 float orc_lane_dot(const float* a, const float* b, size_t n);
 
 int orc_max_threads(void);
+/* seconds for `reps` multi-thread read passes over a buffer of 64-bit words (host memory-read ceiling) */
+double orc_read_seconds(const uint64_t* buffer, size_t words, int reps, int threads, uint64_t* checksum);
 
 #ifdef __cplusplus
 }
