@@ -59,7 +59,10 @@ constexpr uint32_t kPfTokenAhead = 3;             // steps between a token copy 
 __host__ __device__ constexpr uint32_t pf_sum_slots(uint32_t k) { return (k / 32U + 15U) & ~15U; }
 __host__ __device__ constexpr size_t pf_sum_row_bytes(uint32_t k) { return 4U * static_cast<size_t>(pf_sum_slots(k)); }
 // bytes of the fp16 workspace: h [assignments][ffn], sums of h [assignments], sums of the input rows [rows]
-__host__ __device__ constexpr size_t pf_h_bytes(uint32_t assignments, uint32_t ffn) { return 2U * static_cast<size_t>(assignments) * ffn; }
+// (two fp16 planes: h = hi + lo)
+// (one plane holds a tile of 128 rows more than the assignments: the down kernel reads whole tiles of rows)
+__host__ __device__ constexpr size_t pf_h_plane_bytes(uint32_t assignments, uint32_t ffn) { return 2U * (static_cast<size_t>(assignments) + 128U) * ffn; }
+__host__ __device__ constexpr size_t pf_h_bytes(uint32_t assignments, uint32_t ffn) { return 2U * pf_h_plane_bytes(assignments, ffn); }
 __host__ __device__ constexpr size_t pf_workspace_bytes(uint32_t hidden, uint32_t ffn, uint32_t rows, uint32_t top_k) {
     return pf_h_bytes(rows * top_k, ffn) + static_cast<size_t>(rows) * top_k * pf_sum_row_bytes(ffn) + static_cast<size_t>(rows) * pf_sum_row_bytes(hidden);
 }
@@ -73,6 +76,8 @@ struct PrefillArgs {
     float swiglu_limit;                           // the clamp trait of the SwiGLU epilogue (+infinity: none)
     const uint8_t* x; uint64_t x_stride;          // MODE 0: fp16 token rows (bytes); MODE 1: unused
     _Float16* h;                                  // [assignments in plan order][ffn] fp16: written by MODE 0, read by MODE 1
+    _Float16* h_lo;                               // the same shape: fp16(h - fp16(h)), so that hi + lo carries h to 22 bits
+    uint32_t lo_pass;                             // MODE 1 of prefill_f16_kernel: multiply the lo plane and ADD to the outputs (second pass)
     uint8_t* h_sums;                              // [assignments in plan order] sub-block sums of h: written by MODE 0, read by MODE 1
     const uint8_t* x_sums;                        // [rows] sub-block sums of the input rows (MODE 0)
     float* rawdots;                               // MODE 1: [assignment][hidden]
@@ -190,7 +195,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
             const uint32_t row = 8U * (4U * i + wave) + (lane >> 3), tok = row < count ? row : count - 1U;
             const uint32_t piece = (lane & 7U) ^ ((row >> 1) & 7U);
             if (MODE == 0) tsrc[i] = a.x + static_cast<size_t>(order[begin + tok] / a.top_k) * a.x_stride + 16U * piece;
-            else tsrc[i] = reinterpret_cast<const uint8_t*>(a.h + static_cast<size_t>(begin + tok) * a.k) + 16U * piece;
+            else tsrc[i] = reinterpret_cast<const uint8_t*>((a.lo_pass ? a.h_lo : a.h) + static_cast<size_t>(begin + tok) * a.k) + 16U * piece;
         }
         // ---- sums side: copy c of a group moves pieces 256 c + t; piece = (token, part): part 0, 1 = hi, part 2, 3 = lo
         const uint8_t* ssrc[2];
@@ -511,7 +516,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                     for (uint32_t n = 0; n < 2U; ++n)
 #pragma unroll
                         for (int j = 0; j < 16; ++j) acc[i][n][j] = __builtin_fmaf(d[n], part[i][n][j], acc[i][n][j]);   // (tiles with no live row keep P = 0)
-                if (((b & 1U) || b + 1U == blocks) && live_tiles != 0) {
+                if (((b & 1U) || b + 1U == blocks) && live_tiles != 0 && !(MODE == 1 && a.lo_pass)) {
                     // end of a group of 16 sub-blocks: running sum += S hi * M hi + S lo * M hi + S hi * M lo
                     const uint32_t g = b >> 1;
                     const pf_lds* st = s_tile + (g & 1U) * (kPfTile * 64U) + (TS * wc + l31) * 64U + 16U * upper;
@@ -565,10 +570,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                 swiglu_clamp(gc, uc, a.swiglu_limit);
                 const float hv = (gc / (1.0F + declared_exp(-gc))) * uc;
                 const _Float16 h16 = static_cast<_Float16>(hv);
-                float sum = live ? static_cast<float>(h16) : 0.0F;
+                const _Float16 h16_lo = static_cast<_Float16>(hv - static_cast<float>(h16));
+                float sum = live ? static_cast<float>(h16) + static_cast<float>(h16_lo) : 0.0F;
                 sum += xor1_f(sum); sum += xor2_f(sum); sum += xor4_f(sum); sum += xor8_f(sum); sum += xor16_f(sum);
                 if (live) {
                     a.h[static_cast<size_t>(begin + n) * a.features + m0 + 32U * wr + l31] = h16;
+                    a.h_lo[static_cast<size_t>(begin + n) * a.features + m0 + 32U * wr + l31] = h16_lo;
                     if (l31 == 0) {
                         _Float16* sums = reinterpret_cast<_Float16*>(a.h_sums + static_cast<size_t>(begin + n) * pf_sum_row_bytes(a.features));
                         split_half(sum, sums[sub_block], sums[pf_sum_slots(a.features) + sub_block]);
@@ -580,8 +587,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                 }
             } else if (live) {
                 float* out = a.rawdots + static_cast<size_t>(dest[i][j]) * a.features + m0 + 64U * wr + l31;
-                out[0] = acc[i][0][j];
-                out[32] = acc[i][1][j];
+                if (a.lo_pass) { out[0] += acc[i][0][j]; out[32] += acc[i][1][j]; }
+                else { out[0] = acc[i][0][j]; out[32] = acc[i][1][j]; }
             }
         }
     }

@@ -19,6 +19,7 @@
 #include "q5k_quads.hpp"
 #include "q6k_quads.hpp"
 #include "prefill_f16.hpp"
+#include "prefill_reg.hpp"
 #include "route_wave.hpp"
 
 namespace strix950 {
@@ -1395,7 +1396,8 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     PrefillArgs a{};
     a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.swiglu_limit = wv.swiglu_limit; a.x = static_cast<const uint8_t*>(r->input); a.x_stride = r->input_stride;
     uint8_t* ws = static_cast<uint8_t*>(r->h_f16);
-    a.h = reinterpret_cast<_Float16*>(ws); a.h_sums = ws + pf_h_bytes(assignments, wv.ffn);
+    a.h = reinterpret_cast<_Float16*>(ws); a.h_lo = reinterpret_cast<_Float16*>(ws + pf_h_plane_bytes(assignments, wv.ffn));
+    a.h_sums = ws + pf_h_bytes(assignments, wv.ffn);
     uint8_t* x_sums = a.h_sums + static_cast<size_t>(assignments) * pf_sum_row_bytes(wv.ffn);
     a.x_sums = x_sums;
     a.rawdots = r->rawdots; a.plan = r->plan; a.experts = wv.experts; a.assignments = assignments;
@@ -1403,19 +1405,38 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     token_sums_kernel<<<rows, 256, 0, st>>>(a.x, a.x_stride, wv.hidden, x_sums);
     if (pf_sum_slots(wv.ffn) != wv.ffn / 32U) clear_sum_padding_kernel<<<assignments, 64, 0, st>>>(a.h_sums, wv.ffn);
     const uint32_t items_at = plan_items_at(wv.experts, assignments), order_at = plan_order_at(wv.experts), item_slots = (bound + 7U) / 8U * 8U;
-    a.wa = wv.gate; a.wb = wv.up; a.expert_stride = wv.gate_expert_stride; a.row_stride = wv.gate_row_stride; a.k = wv.hidden; a.features = wv.ffn;
-    // persistent workgroups, one per compute unit (the kernel's LDS use allows no second one)
+    // persistent workgroups, one per compute unit (the kernels' LDS use allows no second one)
     const uint32_t cus = compute_units();
     const uint32_t resident = (cus > 8U ? cus : 256U) & ~7U;
-    a.tiles = wv.ffn / 64U; a.units = item_slots * a.tiles;
-    if (wv.gate_type == MI355_TYPE_Q8_0) prefill_f16_kernel<0, 1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
-    else if (wv.gate_type == MI355_TYPE_Q5_K) prefill_f16_kernel<0, 2><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
-    else prefill_f16_kernel<0, 0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    const auto grid_of = [&](uint32_t units) { return units < resident ? units : resident; };
+    // gate / up + SwiGLU. Q4_K tensors: every wave expands its own rows in registers (prefill_reg.hpp); Q5_K / Q8_0: the loader /
+    // multiplier kernel (prefill_f16.hpp). Both leave h as two fp16 planes and its sub-block sums.
+    a.wa = wv.gate; a.wb = wv.up; a.expert_stride = wv.gate_expert_stride; a.row_stride = wv.gate_row_stride; a.k = wv.hidden; a.features = wv.ffn;
+    a.lo_pass = 0;
+    if (wv.gate_type == MI355_TYPE_Q4_K && wv.ffn % 128U == 0) {
+        a.tiles = wv.ffn / 128U; a.units = item_slots * a.tiles;
+        prefill_reg_kernel<0><<<grid_of(a.units), kRgThreads, 0, st>>>(a, items_at, order_at);
+    } else {
+        a.tiles = wv.ffn / 64U; a.units = item_slots * a.tiles;
+        if (wv.gate_type == MI355_TYPE_Q8_0) prefill_f16_kernel<0, 1><<<grid_of(a.units), kPfThreads, 0, st>>>(a, items_at, order_at);
+        else if (wv.gate_type == MI355_TYPE_Q5_K) prefill_f16_kernel<0, 2><<<grid_of(a.units), kPfThreads, 0, st>>>(a, items_at, order_at);
+        else prefill_f16_kernel<0, 0><<<grid_of(a.units), kPfThreads, 0, st>>>(a, items_at, order_at);
+    }
+    // down rows: h enters as hi + lo. The register-operand kernel multiplies both planes in one sweep of the weights; the loader /
+    // multiplier kernel runs a second pass over the lo plane that adds to the first pass's outputs.
     a.wa = wv.down; a.wb = nullptr; a.expert_stride = wv.down_expert_stride; a.row_stride = wv.down_row_stride; a.k = wv.ffn; a.features = wv.hidden;
-    a.tiles = wv.hidden / 128U; a.units = item_slots * a.tiles;
-    if (wv.down_type == MI355_TYPE_Q8_0) prefill_f16_kernel<1, 1><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
-    else if (wv.down_type == MI355_TYPE_Q5_K) prefill_f16_kernel<1, 2><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
-    else prefill_f16_kernel<1, 0><<<a.units < resident ? a.units : resident, kPfThreads, 0, st>>>(a, items_at, order_at);
+    if (wv.down_type == MI355_TYPE_Q4_K && wv.hidden % 256U == 0) {
+        a.tiles = wv.hidden / 256U; a.units = item_slots * a.tiles;
+        prefill_reg_kernel<1><<<grid_of(a.units), kRgThreads, 0, st>>>(a, items_at, order_at);
+    } else {
+        a.tiles = wv.hidden / 128U; a.units = item_slots * a.tiles;
+        for (uint32_t pass = 0; pass < 2U; ++pass) {
+            a.lo_pass = pass;
+            if (wv.down_type == MI355_TYPE_Q8_0) prefill_f16_kernel<1, 1><<<grid_of(a.units), kPfThreads, 0, st>>>(a, items_at, order_at);
+            else if (wv.down_type == MI355_TYPE_Q5_K) prefill_f16_kernel<1, 2><<<grid_of(a.units), kPfThreads, 0, st>>>(a, items_at, order_at);
+            else prefill_f16_kernel<1, 0><<<grid_of(a.units), kPfThreads, 0, st>>>(a, items_at, order_at);
+        }
+    }
     STRIX_LAUNCHED("moe prefill f16");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }

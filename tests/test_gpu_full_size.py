@@ -163,7 +163,7 @@ def test_config4_prefill_f16_mfma_full_size(strix):
     def close(got, ref):
         rms = np.sqrt(np.mean(ref ** 2))
         assert np.max(np.abs(got - ref)) / rms < TOL_F16
-        big = np.abs(ref) >= rms
+        big = np.abs(ref) > 1e-2 * rms
         assert np.max(np.abs(got[big] - ref[big]) / np.abs(ref[big])) < TOL_F16
 
     base_ref = ffn(xs, sg.cpu().numpy(), su.cpu().numpy(), sd.cpu().numpy(), orc.Q8_0)

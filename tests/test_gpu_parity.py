@@ -779,17 +779,26 @@ def random_q8_0(rng, shape_rows, width):
     (512, 256, 4, 2, 90, orc.Q4_K, orc.Q8_0, False),
     (512, 256, 4, 2, 300, orc.Q5_K, orc.Q4_K, False),       # Q5_K (fifth bits in use): even, odd and single super-block counts
     (768, 1280, 3, 2, 150, orc.Q5_K, orc.Q5_K, False),
-    (256, 512, 5, 1, 129, orc.Q4_K, orc.Q5_K, False)])
+    (256, 512, 5, 1, 129, orc.Q4_K, orc.Q5_K, False),
+    # blocks of random bytes: every factor, minimum and code value occurs and h has a heavy tail (h carried as a single fp16
+    # misses the bar on these: the largest error reaches 4e-3 of the rms; as hi + lo it stays near 1e-5)
+    (512, 512, 4, 2, 300, orc.Q4_K, orc.Q4_K, True),
+    (1024, 768, 6, 2, 200, orc.Q5_K, orc.Q5_K, True),
+    (768, 512, 3, 2, 150, orc.Q4_K, orc.Q5_K, True),
+    (512, 1024, 1, 1, 140, orc.Q5_K, orc.Q8_0, True)])
 def test_prefill_f16_mfma_q8_0_tensors(strix, H, I, E, K, T, gate_type, down_type, random_bytes):
-    """The matrix-core prefill form with Q8_0 expert tensors (the always-on shared expert is experts = top_k = 1 with weight 1)
-    against the exact-weight product, tolerance 2e-3 as for Q4_K: max abs error over the output rms, and elementwise on the
-    outputs of at least rms size, for the unweighted down outputs and the combined output."""
+    """The matrix-core prefill form with Q8_0 / Q5_K / mixed expert tensors (the always-on shared expert is experts = top_k = 1
+    with weight 1) against the exact-weight product, tolerance 2e-3 as for Q4_K: max abs error over the output rms, and
+    elementwise on every output above a hundredth of the rms, for the unweighted down outputs and the combined output."""
     rng = np.random.default_rng(7 * H + T)
     def tensor(qtype, rows, width):
-        if qtype == orc.Q5_K:      # written from normal weights (random bytes give a heavy-tailed h whose fp16 rounding alone exceeds the bar)
+        if random_bytes:
+            w = {orc.Q8_0: random_q8_0, orc.Q4_K: random_q4k, orc.Q5_K: orc.random_q5_k}[qtype](rng, (E, rows), width)
+            if qtype == orc.Q4_K:
+                w[..., 1::144] &= 0x0F          # d below 2^-11: h of these products stays inside fp16
+            return w
+        if qtype == orc.Q5_K:
             return orc.quantize_q5_k_rows((rng.standard_normal((E, rows, width)) * 0.02).astype(np.float32))
-        if random_bytes and qtype == orc.Q8_0:
-            return random_q8_0(rng, (E, rows), width)
         return orc.quantize_rows(qtype, (rng.standard_normal((E, rows, width)) * 0.02).astype(np.float32))
     gate, up, down = tensor(gate_type, I, H), tensor(gate_type, I, H), tensor(down_type, H, I)
     x = rng.standard_normal((T, H)).astype(np.float16)
@@ -805,7 +814,7 @@ def test_prefill_f16_mfma_q8_0_tensors(strix, H, I, E, K, T, gate_type, down_typ
         ref64 = ref.astype(np.float64)
         rms = np.sqrt(np.mean(ref64 ** 2))
         assert np.max(np.abs(got - ref64)) / rms < TOL_F16
-        big = np.abs(ref64) >= rms
+        big = np.abs(ref64) > 1e-2 * rms
         assert np.max(np.abs(got[big] - ref64[big]) / np.abs(ref64[big])) < TOL_F16
     assert np.all(layer.status[:T].cpu().numpy() == 0)
     # the integer-class entries keep refusing Q8_0 gate / up tensors
@@ -860,7 +869,7 @@ def test_prefill_f16_mfma_matches_exact_weight_product(strix, H, I, E, K, T):
         ref64 = ref.astype(np.float64)
         rms = np.sqrt(np.mean(ref64 ** 2))
         assert np.max(np.abs(got - ref64)) / rms < TOL_F16                       # max abs error over the output rms
-        big = np.abs(ref64) >= rms                                               # elementwise relative error of the rms-sized outputs
+        big = np.abs(ref64) > 1e-2 * rms                                         # elementwise relative error above a hundredth of the rms
         assert np.max(np.abs(got[big] - ref64[big]) / np.abs(ref64[big])) < TOL_F16
     assert np.all(layer.status[:T].cpu().numpy() == 0)
     e0 = int(ids_ref[0, 0])
