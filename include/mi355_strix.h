@@ -253,6 +253,74 @@ int32_t mi355_swiglu_quantize(const float* gate, const float* up, uint32_t rows,
                               float swiglu_limit, int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
                               mi355_stream stream);
 
+/* ------------------------------------------------------------------------------------------------------
+ * The reference's A8 request / bindings boundary (the HIP entry points this library replaces). Field for field:
+ *   mi355_device_bytes      = DeviceBytes                  include/strix/moe_q4k_a8_contract.hpp:117
+ *   mi355_a8_shape          = Shape                        include/strix/moe_q4k_a8_contract.hpp:104
+ *   mi355_a8_request        = Request                      include/strix/moe_q4k_a8_contract.hpp:105-116
+ *   mi355_a8_bindings       = Bindings                     include/strix/moe_q4k_a8_contract.hpp:118-120
+ *   mi355_a8_down_shape / _request / _bindings = DownShape / DownRequest / DownBindings   include/strix/moe_a8_down_contract.hpp:39-52
+ *   mi355_slot_merge_tail   = SlotMergeTail                include/strix/hip_moe_a8_down.hpp:21-29
+ * (std::string_view becomes a NUL-terminated string, bool a uint32_t, InputKind one of MI355_INPUT_*.)
+ * mi355_a8_validate / mi355_a8_validate_down are the reference's validate / validate_down (src/moe_q4k_a8_contract.cpp:343-372,
+ * src/moe_a8_down_contract.cpp:53-82): pure host admission - enabled, the exact numerical identity string of this library
+ * (mi355_numerical_identity), bounded dimensions, every view non-null, aligned (16 bytes; down routes / status words: 4) and of EXACTLY the required byte size, every mutable view disjoint from every other view (down:
+ * all views pairwise disjoint). Bounds are this library's, wider than the reference's: hidden % 256 <= 16384, rows % 32 <=
+ * 16384 (down: intermediate % 128, K-quant % 256), experts <= 1024, top_k <= 16, and logical_rows 1..16: the per-row views
+ * (input, routes, codes, deltas, sums, output; down: intermediates, routes, codes, deltas, sums, rawdots) then hold that many
+ * contiguous single-row extents, status stays one shared word. Every enqueue validates the whole bundle before its first
+ * launch and, as in the reference, never allocates, synchronises, resets or reads back; status words are sticky (OR only).
+ */
+typedef struct mi355_device_bytes { uintptr_t address; uint64_t bytes; } mi355_device_bytes;
+typedef struct mi355_a8_shape { uint32_t hidden, rows, experts, top_k, logical_rows; } mi355_a8_shape;      /* rows = expert intermediate size */
+typedef struct mi355_a8_request {
+    uint32_t enabled;
+    const char* approved_numerical_identity;      /* must equal mi355_numerical_identity(gate_type, 0) */
+    uint32_t input;                               /* MI355_INPUT_BF16, MI355_INPUT_F32 (the reference's kinds) or MI355_INPUT_F16 */
+    mi355_a8_shape shape;
+    uint32_t gate_type, up_type;                  /* 12 or 13, equal */
+    uint32_t fused_gate_up;                       /* must be 0 */
+    float swiglu_limit;                           /* must be +infinity here: the clamp belongs to the down producer */
+} mi355_a8_request;
+typedef struct mi355_a8_bindings { mi355_device_bytes input, gate, up, routes, codes, deltas, sums, status, output; } mi355_a8_bindings;
+int32_t mi355_a8_validate(const mi355_a8_request*, const mi355_a8_bindings*);
+/* enqueue_probe (include/strix/hip_moe_q4k_a8_probe.hpp:12): route check, A8 image of the input row(s), gate and up rows of
+ * the chosen experts: output[((row * top_k + slot) * 2 + which) * shape.rows + i] fp32 (which 0 = gate, 1 = up), bitwise
+ * the reference row contract (src/moe_q4k_a8_contract.cpp:126-140). */
+int32_t mi355_a8_enqueue_probe(const mi355_a8_request*, const mi355_a8_bindings*, mi355_stream);
+
+typedef struct mi355_a8_down_shape { uint32_t hidden, intermediate, experts, top_k; } mi355_a8_down_shape;
+typedef struct mi355_a8_down_request {
+    uint32_t enabled;
+    const char* approved_numerical_identity;      /* must equal mi355_numerical_identity(weight_type, 1) */
+    mi355_a8_down_shape shape;
+    uint32_t weight_type;                         /* 7 (Q5_1), 8 (Q8_0), 12 (Q4_K) or 14 (Q6_K) */
+    float swiglu_limit;                           /* +infinity (none) or finite > 0: the clamped producer */
+} mi355_a8_down_request;
+/* intermediates: per (row, slot) [gate I | up I] fp32 (the probe's output); the producer replaces ONLY gate with h. */
+typedef struct mi355_a8_down_bindings {
+    mi355_device_bytes intermediates, weights, routes, codes, deltas, sums, rawdots, status, aggregate_status;   /* aggregate_status may be {0, 0} */
+} mi355_a8_down_bindings;
+int32_t mi355_a8_validate_down(const mi355_a8_down_request*, const mi355_a8_down_bindings*, uint32_t logical_rows);
+/* enqueue_down_activation_quantize (include/strix/hip_moe_a8_down.hpp:18): h = silu(g) * u (clamp trait applied first) and its
+ * A8 image; invalid route -> status |= 1, non-finite g / u / h -> status |= 8, either -> aggregate_status |= 16.
+ * exp_kind: MI355_EXP_* of the SiLU (the reference's device expf is MI355_EXP_GFX1151). */
+int32_t mi355_a8_enqueue_down_activation_quantize(const mi355_a8_down_request*, const mi355_a8_down_bindings*, uint32_t logical_rows,
+                                                  uint32_t exp_kind, mi355_stream);
+/* enqueue_down_rawdots (include/strix/hip_moe_a8_down.hpp:19): rawdots[(row * top_k + slot) * hidden + o], unweighted. */
+int32_t mi355_a8_enqueue_down_rawdots(const mi355_a8_down_request*, const mi355_a8_down_bindings*, uint32_t logical_rows, mi355_stream);
+/* The same for one row, then the ordered expert-slot merge, the finite / commit test and the first-error record
+ * (include/strix/moe_slot_merge.hpp:1-12,47-55; src/hip_moe_q4k_a8_probe.hip:825-897): accumulation[o] = fma chain over the slots
+ * from +0 in slot order; any |value| with bits >= 0x7f800000 (bf16_commit: >= 0x7f7f8000, i.e. also what rounds to bf16
+ * infinity) fails the step: status |= 8 and nothing is committed; a clean step stores output (fp32, or bf16 round to nearest
+ * even when output_bf16); record = DeferredMoeFirstError {domain, bits} keeps the first non-zero status. tickets is accepted
+ * for signature parity and left untouched (the merge is a launch of its own here). */
+typedef struct mi355_slot_merge_tail {
+    uint32_t* tickets; const float* route_weights; float* accumulation; void* output;
+    uint32_t output_bf16, bf16_commit; void* record; uint32_t domain;
+} mi355_slot_merge_tail;
+int32_t mi355_a8_enqueue_down_rawdots_merge(const mi355_a8_down_request*, const mi355_a8_down_bindings*, const mi355_slot_merge_tail*, mi355_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -246,6 +246,39 @@ int ref_route_select_policy(std::uint32_t experts, std::uint32_t top_k, float re
     });
 }
 // The SwiGLU clamp trait.
+// validate / validate_down of the two A8 contracts (src/moe_q4k_a8_contract.cpp:343-372, src/moe_a8_down_contract.cpp:53-82):
+// 0 = admitted, -1 = refused (ref_last_error holds the reason). views: nine {address, bytes} pairs in the order of Bindings /
+// DownBindings.
+int ref_a8_validate(int enabled, const char* identity, int input_fp32, std::uint32_t hidden, std::uint32_t rows, std::uint32_t experts,
+                    std::uint32_t top_k, std::uint32_t logical_rows, std::uint32_t gate_type, std::uint32_t up_type, int fused, float limit,
+                    const std::uint64_t* views) {
+    a8::Request q;
+    q.enabled = enabled != 0; q.approved_numerical_identity = identity ? std::string_view(identity) : std::string_view();
+    q.input = input_fp32 ? a8::InputKind::fp32 : a8::InputKind::bf16;
+    q.shape = a8::Shape{hidden, rows, experts, top_k, logical_rows};
+    q.gate_type = gate_type; q.up_type = up_type; q.fused_gate_up = fused != 0; q.swiglu_limit = limit;
+    a8::DeviceBytes v[9];
+    for (int i = 0; i < 9; ++i) v[i] = a8::DeviceBytes{static_cast<std::uintptr_t>(views[2 * i]), views[2 * i + 1]};
+    const a8::Bindings b{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
+    return guarded([&] { a8::validate(q, b); });
+}
+int ref_a8_validate_down(int enabled, const char* identity, std::uint32_t hidden, std::uint32_t intermediate, std::uint32_t experts,
+                         std::uint32_t top_k, std::uint32_t weight_type, float limit, const std::uint64_t* views) {
+    a8::DownRequest q;
+    q.enabled = enabled != 0; q.approved_numerical_identity = identity ? std::string_view(identity) : std::string_view();
+    q.shape = a8::DownShape{hidden, intermediate, experts, top_k};
+    q.weight_type = weight_type; q.swiglu_limit = limit;
+    a8::DeviceBytes v[9];
+    for (int i = 0; i < 9; ++i) v[i] = a8::DeviceBytes{static_cast<std::uintptr_t>(views[2 * i]), views[2 * i + 1]};
+    const a8::DownBindings b{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
+    return guarded([&] { a8::validate_down(q, b); });
+}
+const char* ref_a8_identity(std::uint32_t type, int down) {
+    static std::string held;
+    try { held = std::string(down ? a8::down_numerical_identity(type) : a8::numerical_identity_for_gate_type(type)); } catch (const std::exception&) { held.clear(); }
+    return held.c_str();
+}
+
 void ref_swiglu_clamp(float gate, float up, float limit, float* gate_out, float* up_out) {
     const auto c = strix::moe::swiglu_clamp(gate, up, limit);
     *gate_out = c.gate; *up_out = c.up;

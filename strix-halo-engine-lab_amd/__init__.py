@@ -57,6 +57,46 @@ class MoeRows(C.Structure):
                 ("plan", C.c_void_p), ("job_status", C.c_void_p), ("h_f16", C.c_void_p)]
 
 
+class DeviceBytes(C.Structure):
+    _fields_ = [("address", C.c_size_t), ("bytes", C.c_uint64)]
+
+
+class A8Shape(C.Structure):
+    _fields_ = [("hidden", C.c_uint32), ("rows", C.c_uint32), ("experts", C.c_uint32), ("top_k", C.c_uint32), ("logical_rows", C.c_uint32)]
+
+
+class A8Request(C.Structure):
+    _fields_ = [("enabled", C.c_uint32), ("approved_numerical_identity", C.c_char_p), ("input", C.c_uint32), ("shape", A8Shape),
+                ("gate_type", C.c_uint32), ("up_type", C.c_uint32), ("fused_gate_up", C.c_uint32), ("swiglu_limit", C.c_float)]
+
+
+class A8Bindings(C.Structure):
+    _fields_ = [(n, DeviceBytes) for n in ("input", "gate", "up", "routes", "codes", "deltas", "sums", "status", "output")]
+
+
+class A8DownShape(C.Structure):
+    _fields_ = [("hidden", C.c_uint32), ("intermediate", C.c_uint32), ("experts", C.c_uint32), ("top_k", C.c_uint32)]
+
+
+class A8DownRequest(C.Structure):
+    _fields_ = [("enabled", C.c_uint32), ("approved_numerical_identity", C.c_char_p), ("shape", A8DownShape), ("weight_type", C.c_uint32),
+                ("swiglu_limit", C.c_float)]
+
+
+class A8DownBindings(C.Structure):
+    _fields_ = [(n, DeviceBytes) for n in ("intermediates", "weights", "routes", "codes", "deltas", "sums", "rawdots", "status", "aggregate_status")]
+
+
+class SlotMergeTail(C.Structure):
+    _fields_ = [("tickets", C.c_void_p), ("route_weights", C.c_void_p), ("accumulation", C.c_void_p), ("output", C.c_void_p),
+                ("output_bf16", C.c_uint32), ("bf16_commit", C.c_uint32), ("record", C.c_void_p), ("domain", C.c_uint32)]
+
+
+def device_bytes(t):
+    """DeviceBytes of a tensor (None: the empty view)."""
+    return DeviceBytes(0, 0) if t is None else DeviceBytes(t.data_ptr(), t.numel() * t.element_size())
+
+
 _lib = None
 
 
@@ -83,7 +123,8 @@ EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi3
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
            "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
-           "mi355_swiglu_quantize", "mi355_rmsnorm_f32"]
+           "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe",
+           "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge"]
 
 
 def require_gpu():
@@ -182,6 +223,68 @@ def swiglu_quantize(gate, up, exp_kind=EXP_GFX1151, swiglu_limit=float("inf")):
     status = torch.zeros(rows, dtype=torch.int32, device=gate.device)
     check(lib().mi355_swiglu_quantize(_p(gate), _p(up), rows, ffn, exp_kind, C.c_float(swiglu_limit), _p(codes), _p(deltas), _p(sums), _p(h), _p(status), _stream()))
     return codes, deltas, sums, h, status
+
+
+class A8Decode:
+    """The reference's single-row A8 pipeline over the request / bindings entry points (include/strix/hip_moe_q4k_a8_probe.hpp:12,
+    include/strix/hip_moe_a8_down.hpp:18-30): probe -> down_activation_quantize -> down_rawdots (+ slot merge). Owns the views the
+    reference's caller owns (every one an allocation of its own, so the bundle is disjoint and 256-byte aligned) for up to
+    `rows` logical rows. gate / up / down: uint8 device tensors holding every expert in GGUF order."""
+
+    def __init__(self, hidden, intermediate, experts, top_k, gate, up, down, rows=1, gate_type=TYPE_Q4_K, down_type=TYPE_Q4_K, input_dtype=torch.bfloat16,
+                 swiglu_limit=float("inf")):
+        self.H, self.I, self.E, self.K, self.R = hidden, intermediate, experts, top_k, rows
+        self.gate_type, self.down_type, self.limit = gate_type, down_type, swiglu_limit
+        self.gate, self.up, self.down = gate, up, down
+        d = gate.device
+        z = lambda shape, dt: torch.zeros(shape, dtype=dt, device=d)
+        self.input = z((rows, hidden), input_dtype)
+        self.routes = z((rows, top_k), torch.int32)
+        self.codes, self.deltas, self.sums = z((rows, hidden), torch.int8), z((rows, hidden // 32), torch.float32), z((rows, hidden // 32), torch.int32)
+        self.status, self.aggregate = z(1, torch.int32), z(1, torch.int32)
+        self.intermediates = z((rows, top_k, 2, intermediate), torch.float32)      # the probe's output = the down producer's input
+        self.h_codes = z((rows, top_k, intermediate), torch.int8)
+        self.h_deltas, self.h_sums = z((rows, top_k, intermediate // 32), torch.float32), z((rows, top_k, intermediate // 32), torch.int32)
+        self.rawdots = z((rows, top_k, hidden), torch.float32)
+        self.probe_identity = lib().mi355_numerical_identity(gate_type, 0)
+        self.down_identity = lib().mi355_numerical_identity(down_type, 1)
+
+    def request(self, rows=None):
+        return A8Request(1, self.probe_identity, input_kind(self.input), A8Shape(self.H, self.I, self.E, self.K, rows or self.R), self.gate_type,
+                         self.gate_type, 0, float("inf"))
+
+    def bindings(self, rows=None):
+        n = rows or self.R
+        return A8Bindings(device_bytes(self.input[:n]), device_bytes(self.gate), device_bytes(self.up), device_bytes(self.routes[:n]),
+                          device_bytes(self.codes[:n]), device_bytes(self.deltas[:n]), device_bytes(self.sums[:n]), device_bytes(self.status),
+                          device_bytes(self.intermediates[:n]))
+
+    def down_request(self):
+        return A8DownRequest(1, self.down_identity, A8DownShape(self.H, self.I, self.E, self.K), self.down_type, self.limit)
+
+    def down_bindings(self, rows=None, aggregate=True):
+        n = rows or self.R
+        return A8DownBindings(device_bytes(self.intermediates[:n]), device_bytes(self.down), device_bytes(self.routes[:n]), device_bytes(self.h_codes[:n]),
+                              device_bytes(self.h_deltas[:n]), device_bytes(self.h_sums[:n]), device_bytes(self.rawdots[:n]), device_bytes(self.status),
+                              device_bytes(self.aggregate if aggregate else None))
+
+    def enqueue_probe(self, rows=None):
+        q, b = self.request(rows), self.bindings(rows)
+        check(lib().mi355_a8_enqueue_probe(C.byref(q), C.byref(b), _stream()))
+
+    def enqueue_down_activation_quantize(self, rows=None, exp_kind=EXP_GFX1151):
+        q, b = self.down_request(), self.down_bindings(rows)
+        check(lib().mi355_a8_enqueue_down_activation_quantize(C.byref(q), C.byref(b), rows or self.R, exp_kind, _stream()))
+
+    def enqueue_down_rawdots(self, rows=None):
+        q, b = self.down_request(), self.down_bindings(rows)
+        check(lib().mi355_a8_enqueue_down_rawdots(C.byref(q), C.byref(b), rows or self.R, _stream()))
+
+    def enqueue_down_rawdots_merge(self, route_weights, accumulation, output, record, domain=1, bf16_commit=False):
+        """One row: rawdots, then the ordered slot merge, commit test and first-error record (SlotMergeTail)."""
+        q, b = self.down_request(), self.down_bindings(1)
+        tail = SlotMergeTail(None, _p(route_weights), _p(accumulation), _p(output), int(output.dtype == torch.bfloat16), int(bf16_commit), _p(record), domain)
+        check(lib().mi355_a8_enqueue_down_rawdots_merge(C.byref(q), C.byref(b), C.byref(tail), _stream()))
 
 
 class MoeLayer:

@@ -1,0 +1,310 @@
+// The reference's A8 request / bindings boundary on this library's kernels: host admission (pure: no allocation, no device
+// call, no buffer touched) and the single-row ("C1") entry points with up to 16 logical rows.
+//   Request / Shape / Bindings / validate     include/strix/moe_q4k_a8_contract.hpp:104-122, src/moe_q4k_a8_contract.cpp:343-372
+//   enqueue_probe                             include/strix/hip_moe_q4k_a8_probe.hpp:8-12
+//   DownRequest / DownBindings / validate_down include/strix/moe_a8_down_contract.hpp:40-54, src/moe_a8_down_contract.cpp:53-82
+//   enqueue_down_activation_quantize / enqueue_down_rawdots (+ SlotMergeTail)   include/strix/hip_moe_a8_down.hpp:11-30
+// Differences from the reference, all widening: the geometry caps (hidden 2560, rows 1536, experts 512) are this library's
+// (hidden <= 16384, intermediate <= 16384, experts <= 1024, top_k <= 16), fp16 input is a third input kind, and
+// shape.logical_rows may be 1..16 with the per-row views holding that many contiguous single-row extents (the reference's
+// union form without its plan view: an expert chosen by two rows is simply read twice).
+// Status words are the caller's and sticky: nothing here clears them, bits are OR-ed in.
+#pragma once
+
+namespace strix950 {
+
+constexpr uint32_t kA8MaxHidden = 16384, kA8MaxIntermediate = 16384, kA8MaxLogicalRows = 16;
+
+inline bool a8_identity_matches(const char* given, uint32_t type, int down) {
+    const char* mine = mi355_numerical_identity(type, down);
+    return given != nullptr && mine[0] != 0 && std::strcmp(given, mine) == 0;
+}
+inline bool a8_overlap(const mi355_device_bytes& x, const mi355_device_bytes& y) {
+    return !(x.address + x.bytes <= y.address || y.address + y.bytes <= x.address);
+}
+inline bool a8_clamp_ok(float limit) { return limit == INFINITY || (std::isfinite(limit) && limit > 0.0F); }
+
+// gate / up row bytes per 256 weights (src/moe_q4k_a8_contract.cpp:352-354: Q4_K 144, Q5_K 176)
+inline uint64_t a8_gate_block_bytes(uint32_t type) { return type == MI355_TYPE_Q5_K ? 176U : 144U; }
+
+int32_t a8_validate(const mi355_a8_request* q, const mi355_a8_bindings* b) {
+    STRIX_REQUIRE(q && b, "A8 probe: null request or bindings");
+    STRIX_REQUIRE(q->enabled && a8_identity_matches(q->approved_numerical_identity, q->gate_type, 0),
+                  "A8 probe requires explicit matching numerical identity approval (mi355_numerical_identity(gate_type, 0))");
+    const mi355_a8_shape& s = q->shape;
+    STRIX_REQUIRE(s.hidden >= 256 && s.hidden <= kA8MaxHidden && s.hidden % 256U == 0 && s.rows > 0 && s.rows <= kA8MaxIntermediate &&
+                  s.rows % 32U == 0 && s.experts > 0 && s.experts <= kRouteMaxExperts && s.top_k > 0 && s.top_k <= kRouteMaxTopK &&
+                  s.logical_rows >= 1 && s.logical_rows <= kA8MaxLogicalRows,
+                  "A8 probe admits hidden % 256 (<= 16384), rows % 32 (<= 16384), experts <= 1024, top_k <= 16, logical_rows 1..16 only");
+    STRIX_REQUIRE(q->input <= MI355_INPUT_BF16, "A8 probe: input storage unsupported");
+    STRIX_REQUIRE(q->gate_type == q->up_type && !q->fused_gate_up && (q->gate_type == MI355_TYPE_Q4_K || q->gate_type == MI355_TYPE_Q5_K),
+                  "A8 probe requires separate matching type 12 or type 13 gate / up tensors");
+    STRIX_REQUIRE(q->swiglu_limit == INFINITY, "A8 probe: a finite SwiGLU clamp belongs to the down producer (DownRequest), not to the projection");
+    const uint64_t R = s.logical_rows;
+    const uint64_t weight_bytes = static_cast<uint64_t>(s.experts) * s.rows * (s.hidden / 256U) * a8_gate_block_bytes(q->gate_type);
+    const mi355_device_bytes views[9] = {b->input, b->gate, b->up, b->routes, b->codes, b->deltas, b->sums, b->status, b->output};
+    const uint64_t required[9] = {R * s.hidden * (q->input == MI355_INPUT_F32 ? 4U : 2U), weight_bytes, weight_bytes, R * s.top_k * 4ULL,
+                                  R * s.hidden, R * (s.hidden / 32U) * 4ULL, R * (s.hidden / 32U) * 4ULL, 4,
+                                  R * s.top_k * 2ULL * s.rows * 4ULL};
+    for (size_t i = 0; i < 9; ++i) {
+        STRIX_REQUIRE(views[i].address != 0 && views[i].address % 16U == 0 && views[i].bytes == required[i] &&
+                      views[i].bytes <= UINTPTR_MAX - views[i].address, "A8 probe device view address / alignment / exact byte size invalid");
+        // every mutable view (codes, deltas, sums, status, output) is disjoint from every other view; gate and up are separate
+        for (size_t j = 0; j < i; ++j)
+            if (i >= 4 || (i == 2 && j == 1))
+                STRIX_REQUIRE(!a8_overlap(views[i], views[j]), "A8 probe mutable views and separate gate / up must not overlap");
+    }
+    return MI355_OK;
+}
+
+inline uint64_t a8_down_row_bytes(uint32_t type, uint32_t intermediate) {        // src/moe_a8_down_contract.cpp:47-52
+    if (type == MI355_TYPE_Q4_K) return static_cast<uint64_t>(intermediate / 256U) * 144U;
+    if (type == MI355_TYPE_Q6_K) return static_cast<uint64_t>(intermediate / 256U) * 210U;
+    return static_cast<uint64_t>(intermediate / 32U) * (type == MI355_TYPE_Q5_1 ? 24U : 34U);
+}
+
+int32_t a8_validate_down(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t logical_rows) {
+    STRIX_REQUIRE(q && b, "A8 down: null request or bindings");
+    if (!(q->weight_type == MI355_TYPE_Q4_K || q->weight_type == MI355_TYPE_Q6_K || q->weight_type == MI355_TYPE_Q5_1 || q->weight_type == MI355_TYPE_Q8_0))
+        return fail(MI355_E_UNSUPPORTED, "A8 down weights must be Q5_1 (7), Q8_0 (8), Q4_K (12) or Q6_K (14)");
+    STRIX_REQUIRE(q->enabled && a8_identity_matches(q->approved_numerical_identity, q->weight_type, 1),
+                  "A8 down requires explicit matching numerical identity (mi355_numerical_identity(weight_type, 1))");
+    STRIX_REQUIRE(a8_clamp_ok(q->swiglu_limit), "A8 down SwiGLU clamp limit must be +infinity (none) or finite positive");
+    const mi355_a8_down_shape& s = q->shape;
+    const bool kq = q->weight_type == MI355_TYPE_Q4_K || q->weight_type == MI355_TYPE_Q6_K;
+    STRIX_REQUIRE(s.hidden > 0 && s.hidden <= kA8MaxHidden && s.hidden % 64U == 0 && s.intermediate > 0 && s.intermediate <= kA8MaxIntermediate &&
+                  s.intermediate % (kq ? 256U : 128U) == 0 && s.experts > 0 && s.experts <= kRouteMaxExperts && s.top_k > 0 && s.top_k <= kRouteMaxTopK &&
+                  logical_rows >= 1 && logical_rows <= kA8MaxLogicalRows,
+                  "A8 down admits hidden % 64, intermediate % 128 (K-quant: % 256), experts <= 1024, top_k <= 16, rows 1..16 only");
+    const uint64_t R = logical_rows, groups = static_cast<uint64_t>(s.top_k) * (s.intermediate / 32U);
+    const mi355_device_bytes views[9] = {b->intermediates, b->weights, b->routes, b->codes, b->deltas, b->sums, b->rawdots, b->status, b->aggregate_status};
+    const uint64_t bytes[9] = {R * s.top_k * 2ULL * s.intermediate * 4ULL,
+                               static_cast<uint64_t>(s.experts) * s.hidden * a8_down_row_bytes(q->weight_type, s.intermediate),
+                               R * s.top_k * 4ULL, R * s.top_k * static_cast<uint64_t>(s.intermediate), R * groups * 4ULL, R * groups * 4ULL,
+                               R * s.top_k * static_cast<uint64_t>(s.hidden) * 4ULL, 4, 4};
+    // the weight tensor starts on 16 bytes in every class (the reference asks that of Q4_K only and 2 bytes of the others,
+    // src/moe_a8_down_contract.cpp:72-73; the kernels here read words and quads relative to the tensor's start)
+    const unsigned align[9] = {16, 16, 4, 16, 16, 16, 16, 4, 4};
+    for (size_t i = 0; i < 9; ++i) {
+        if (i == 8 && views[i].address == 0 && views[i].bytes == 0) continue;     // the aggregate word is optional
+        STRIX_REQUIRE(views[i].address != 0 && views[i].address % align[i] == 0 && views[i].bytes == bytes[i] &&
+                      bytes[i] <= UINTPTR_MAX - views[i].address, "A8 down view alignment / address / exact extent invalid");
+        for (size_t j = 0; j < i; ++j) STRIX_REQUIRE(!a8_overlap(views[i], views[j]), "A8 down views must be disjoint");
+    }
+    return MI355_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------- kernels
+// Route check + A8 image of the input rows of the probe (src/hip_moe_q4k_a8_probe.hip:41-90: validation and quantizer of one
+// row; here blockIdx.y = logical row). Block x quantises 8 groups of 32; block (0, row) also checks the row's routes.
+template <int KIND>
+__global__ __launch_bounds__(256) void a8_probe_prologue_kernel(const uint8_t* x, uint32_t hidden, const uint32_t* routes, uint32_t experts,
+                                                                uint32_t top_k, int8_t* codes, float* deltas, int32_t* sums, uint32_t* status) {
+    const uint32_t r = blockIdx.y, groups = hidden / 32U, g = blockIdx.x * 8U + (threadIdx.x >> 5), j = threadIdx.x & 31U;
+    if (blockIdx.x == 0 && threadIdx.x < top_k && routes[r * top_k + threadIdx.x] >= experts) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+    if (g >= groups) return;
+    const float v = load_activation<KIND>(x + static_cast<size_t>(r) * hidden * (KIND == 0 ? 4U : 2U), g * 32U + j);
+    const float amax = max32(__builtin_fabsf(v));
+    const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+    const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+    const int code = a8_code(v, delta, tiny);
+    const int sum = sum32_i(code);
+    const int bad = or32_i(finite_f(v) ? 0 : 1);
+    codes[static_cast<size_t>(r) * hidden + g * 32U + j] = static_cast<int8_t>(code);
+    if (j == 0) {
+        deltas[static_cast<size_t>(r) * groups + g] = delta;
+        sums[static_cast<size_t>(r) * groups + g] = sum;
+        if (bad) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
+    }
+}
+
+// The down producer (src/hip_moe_q4k_a8_probe.hip:594-621): intermediates hold, per assignment, [gate I | up I]; h replaces the
+// gate half, its A8 image goes to codes / deltas / sums [assignment][I]. One half-wave per group of 32.
+__global__ __launch_bounds__(256) void a8_down_activation_kernel(float* intermediates, const uint32_t* routes, uint32_t experts, uint32_t width,
+                                                                 uint32_t exp_kind, float limit, int8_t* codes, float* deltas, int32_t* sums,
+                                                                 uint32_t* status, uint32_t* aggregate) {
+    const uint32_t a = blockIdx.y, groups = width / 32U, grp = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U;
+    if (grp >= groups) return;
+    if (routes[a] >= experts) {
+        if (l == 0) { atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE)); if (aggregate) atomicOr(aggregate, static_cast<uint32_t>(MI355_STATUS_AGGREGATE)); }
+        return;
+    }
+    const size_t at = static_cast<size_t>(a) * 2U * width + grp * 32U + l;
+    const float g = intermediates[at], u = intermediates[at + width];
+    float gc = g, uc = u;
+    swiglu_clamp(gc, uc, limit);
+    const float hv = (gc / (1.0F + exp_of(exp_kind, -gc))) * uc;
+    if (or32_i((finite_f(g) && finite_f(u) && finite_f(hv)) ? 0 : 1)) {
+        if (l == 0) { atomicOr(status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION)); if (aggregate) atomicOr(aggregate, static_cast<uint32_t>(MI355_STATUS_AGGREGATE)); }
+        return;
+    }
+    const float amax = max32(__builtin_fabsf(hv));
+    const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+    const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+    const int code = a8_code(hv, dl, tiny);
+    const int sum = sum32_i(code);
+    intermediates[at] = hv;
+    codes[static_cast<size_t>(a) * width + grp * 32U + l] = static_cast<int8_t>(code);
+    if (l == 0) { deltas[static_cast<size_t>(a) * groups + grp] = dl; sums[static_cast<size_t>(a) * groups + grp] = sum; }
+}
+
+// Expert-slot merge, commit and first-error record of one row after its rawdots (include/strix/moe_slot_merge.hpp:47-55,
+// src/hip_moe_q4k_a8_probe.hip:825-897): per output +0, then fma(route_weight[slot], rawdots[slot][o], acc) in slot order (nothing
+// is written when the status was already set or a route is invalid); a value at or above the commit threshold (bf16
+// commit: 0x7f7f8000, the finite values that round to bf16 infinity included) fails the whole step: status |= 8 and no output
+// is committed; the record keeps the first non-zero status of the stream. One 1024-thread workgroup.
+struct SlotMergeArgs {
+    const float* rawdots; const uint32_t* routes; uint32_t* status; uint32_t hidden, experts, top_k;
+    const float* route_weights; float* accumulation; void* output; uint32_t output_bf16, bf16_commit; uint32_t* record; uint32_t domain;
+};
+__global__ __launch_bounds__(1024) void a8_slot_merge_kernel(SlotMergeArgs t) {
+    __shared__ uint32_t flagged, invalid;
+    if (threadIdx.x == 0) { flagged = 0; invalid = 0; }
+    __syncthreads();
+    const uint32_t initial = *t.status;
+    if (threadIdx.x < t.top_k && t.routes[threadIdx.x] >= t.experts) invalid = 1;
+    __syncthreads();
+    if (initial == 0U) {
+        const bool written = invalid == 0;
+        for (uint32_t o = threadIdx.x; o < t.hidden; o += 1024U) {
+            float current = 0.0F;
+            if (written) {
+                for (uint32_t k = 0; k < t.top_k; ++k) current = __builtin_fmaf(t.route_weights[k], t.rawdots[static_cast<size_t>(k) * t.hidden + o], current);
+                t.accumulation[o] = current;
+            }
+            const float value = written ? current : t.accumulation[o];
+            if ((b_of(value) & 0x7fffffffU) >= (t.bf16_commit ? 0x7f7f8000U : 0x7f800000U)) flagged = 1;
+        }
+    }
+    __syncthreads();
+    const uint32_t final_status = initial | (flagged ? 8U : 0U);
+    if (final_status == 0U)
+        for (uint32_t o = threadIdx.x; o < t.hidden; o += 1024U) {
+            const uint32_t bits = b_of(t.accumulation[o]);
+            if (t.output_bf16) static_cast<unsigned short*>(t.output)[o] = static_cast<unsigned short>((bits + 0x7fffU + ((bits >> 16) & 1U)) >> 16);
+            else static_cast<float*>(t.output)[o] = f_of(bits);
+        }
+    if (threadIdx.x == 0) {
+        if (flagged) atomicOr(t.status, 8U);
+        // DeferredMoeFirstError {domain, bits}: the first non-zero status of the stream stays (include/strix/deferred_moe_status.hpp:19-26)
+        if (final_status != 0U && t.record[0] == 0U) { t.record[1] = final_status; t.record[0] = t.domain; }
+    }
+}
+
+inline RowsK a8_rows(const mi355_moe_weights& w) {
+    RowsK r{};
+    r.slot_stride = w.ffn;
+    return r;
+}
+
+}  // namespace strix950
+
+using namespace strix950;
+
+extern "C" {
+
+int32_t mi355_a8_validate(const mi355_a8_request* q, const mi355_a8_bindings* b) { return a8_validate(q, b); }
+int32_t mi355_a8_validate_down(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t logical_rows) {
+    return a8_validate_down(q, b, logical_rows);
+}
+
+int32_t mi355_a8_enqueue_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, mi355_stream stream) {
+    if (const int32_t rc = a8_validate(q, b)) return rc;          // the whole bundle is validated before the first enqueue
+    const mi355_a8_shape& s = q->shape;
+    hipStream_t st = hs(stream);
+    const uint32_t R = s.logical_rows, groups = s.hidden / 32U;
+    const uint8_t* x = reinterpret_cast<const uint8_t*>(b->input.address);
+    uint32_t* status = reinterpret_cast<uint32_t*>(b->status.address);
+    const dim3 pgrid((groups + 7U) / 8U, R);
+    const auto prologue = [&](auto kind) {
+        a8_probe_prologue_kernel<decltype(kind)::value><<<pgrid, 256, 0, st>>>(x, s.hidden, reinterpret_cast<const uint32_t*>(b->routes.address), s.experts, s.top_k,
+            reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), status);
+    };
+    if (q->input == MI355_INPUT_F32) prologue(std::integral_constant<int, 0>{});
+    else if (q->input == MI355_INPUT_F16) prologue(std::integral_constant<int, 1>{});
+    else prologue(std::integral_constant<int, 2>{});
+    mi355_moe_weights w{};
+    w.hidden = s.hidden; w.ffn = s.rows; w.experts = s.experts; w.top_k = s.top_k; w.gate_type = q->gate_type; w.down_type = MI355_TYPE_Q4_K;
+    w.gate = reinterpret_cast<const uint8_t*>(b->gate.address); w.up = reinterpret_cast<const uint8_t*>(b->up.address);
+    w.gate_row_stride = moe_row_bytes(q->gate_type, s.hidden); w.gate_expert_stride = w.gate_row_stride * s.rows;
+    w.exp_kind = MI355_EXP_GFX1151; w.swiglu_limit = INFINITY;
+    // projection only: output[(assignment * 2 + which) * rows + row], no plan (item i = assignment i), no image of h
+    RowsK r = a8_rows(w);
+    r.routes = reinterpret_cast<const uint32_t*>(b->routes.address);
+    r.codes = reinterpret_cast<int8_t*>(b->codes.address); r.deltas = reinterpret_cast<float*>(b->deltas.address); r.sums = reinterpret_cast<int32_t*>(b->sums.address);
+    r.status = status; r.job_status = status;
+    r.gate_out = reinterpret_cast<float*>(b->output.address); r.up_out = r.gate_out + s.rows; r.slot_stride = 2ULL * s.rows;
+    const uint32_t items = R * s.top_k;
+    if (q->gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
+    else if (items <= 16U) project_quad_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
+    else if (items <= kQuadMaxItems) project_quad_kernel<2><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
+    else launch_project_nb<4>(w, r, R, dim3(s.rows / 32U, items), st);
+    STRIX_LAUNCHED("A8 probe");
+    return MI355_OK;
+}
+
+int32_t mi355_a8_enqueue_down_activation_quantize(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t logical_rows,
+                                                  uint32_t exp_kind, mi355_stream stream) {
+    if (const int32_t rc = a8_validate_down(q, b, logical_rows)) return rc;
+    STRIX_REQUIRE(exp_kind <= MI355_EXP_DECLARED, "A8 down: unknown exp kind");
+    const mi355_a8_down_shape& s = q->shape;
+    const uint32_t items = logical_rows * s.top_k;
+    a8_down_activation_kernel<<<dim3((s.intermediate / 32U + 7U) / 8U, items), 256, 0, hs(stream)>>>(
+        reinterpret_cast<float*>(b->intermediates.address), reinterpret_cast<const uint32_t*>(b->routes.address), s.experts, s.intermediate, exp_kind, q->swiglu_limit,
+        reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address),
+        reinterpret_cast<uint32_t*>(b->status.address), reinterpret_cast<uint32_t*>(b->aggregate_status.address));
+    STRIX_LAUNCHED("A8 down activation");
+    return MI355_OK;
+}
+
+namespace {
+int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t logical_rows, hipStream_t st) {
+    const mi355_a8_down_shape& s = q->shape;
+    mi355_moe_weights w{};
+    w.hidden = s.hidden; w.ffn = s.intermediate; w.experts = s.experts; w.top_k = s.top_k; w.gate_type = MI355_TYPE_Q4_K; w.down_type = q->weight_type;
+    w.down = reinterpret_cast<const uint8_t*>(b->weights.address);
+    w.down_row_stride = a8_down_row_bytes(q->weight_type, s.intermediate); w.down_expert_stride = w.down_row_stride * s.hidden;
+    w.swiglu_limit = INFINITY;
+    RowsK r = a8_rows(w);
+    r.routes = reinterpret_cast<const uint32_t*>(b->routes.address);
+    r.down_codes = reinterpret_cast<int8_t*>(b->codes.address); r.down_deltas = reinterpret_cast<float*>(b->deltas.address);
+    r.down_sums = reinterpret_cast<int32_t*>(b->sums.address); r.rawdots = reinterpret_cast<float*>(b->rawdots.address);
+    r.status = reinterpret_cast<uint32_t*>(b->status.address);
+    r.job_status = r.status;        // a non-finite projection recorded by the producer (bit 8) skips the rows, as in the layer entries
+    const uint32_t items = logical_rows * s.top_k;
+    if (q->weight_type != MI355_TYPE_Q4_K) {
+        const dim3 grid(s.hidden / kDownGroupsRows, items);
+        if (q->weight_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
+        else if (q->weight_type == MI355_TYPE_Q5_1) down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
+        else down_q6k_kernel<<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
+    } else if (items <= 16U) down_quad_kernel<4><<<dim3(s.hidden / 64U, items), 256, 0, st>>>(w, r, items);
+    else if (items <= kQuadMaxItems) down_quad_kernel<2><<<dim3(s.hidden / 64U, items), 256, 0, st>>>(w, r, items);
+    else launch_down_nb<4>(w, r, logical_rows, dim3(s.hidden / 64U, items), st);
+    return MI355_OK;
+}
+}  // namespace
+
+int32_t mi355_a8_enqueue_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t logical_rows, mi355_stream stream) {
+    if (const int32_t rc = a8_validate_down(q, b, logical_rows)) return rc;
+    a8_down_rawdots(q, b, logical_rows, hs(stream));
+    STRIX_LAUNCHED("A8 down rawdots");
+    return MI355_OK;
+}
+
+int32_t mi355_a8_enqueue_down_rawdots_merge(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, const mi355_slot_merge_tail* tail,
+                                            mi355_stream stream) {
+    if (const int32_t rc = a8_validate_down(q, b, 1)) return rc;
+    STRIX_REQUIRE(tail && tail->route_weights && tail->accumulation && tail->output && tail->record && q->shape.hidden % 64U == 0 && q->shape.top_k <= 16U,
+                  "A8 down slot-merge tail requires weights, accumulation, output, record, H % 64 == 0, K <= 16");
+    a8_down_rawdots(q, b, 1, hs(stream));
+    SlotMergeArgs t{};
+    t.rawdots = reinterpret_cast<const float*>(b->rawdots.address); t.routes = reinterpret_cast<const uint32_t*>(b->routes.address);
+    t.status = reinterpret_cast<uint32_t*>(b->status.address); t.hidden = q->shape.hidden; t.experts = q->shape.experts; t.top_k = q->shape.top_k;
+    t.route_weights = tail->route_weights; t.accumulation = tail->accumulation; t.output = tail->output; t.output_bf16 = tail->output_bf16;
+    t.bf16_commit = tail->bf16_commit; t.record = static_cast<uint32_t*>(tail->record); t.domain = tail->domain;
+    a8_slot_merge_kernel<<<1, 1024, 0, hs(stream)>>>(t);
+    STRIX_LAUNCHED("A8 down rawdots + slot merge");
+    return MI355_OK;
+}
+
+}  // extern "C"

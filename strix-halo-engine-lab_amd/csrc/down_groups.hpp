@@ -59,11 +59,11 @@ __device__ __forceinline__ void load_group_block(const uint8_t* block, uint32_t 
 }
 
 template <int FMT>
-__global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments,
+__global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments,
                                                           uint32_t items_at, uint32_t order_at) {
     typedef uint32_t u32x4_g __attribute__((ext_vector_type(4)));
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * blockIdx.y);
-    const uint32_t e = item.x, begin = item.y, end = item.z;
+    const WorkItem item = work_item(w, r, items_at, blockIdx.y);
+    const uint32_t e = item.e, begin = item.begin, end = item.end;
     if (begin == end) return;
     if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
     const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, j = lane & 3U, odd = j & 1U;
@@ -71,14 +71,13 @@ __global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, m
     const uint32_t groups = w.ffn / 32U, per_chain = groups / 4U;
     constexpr uint32_t kBlock = FMT == 0 ? 34U : 24U;
     const uint8_t* wrow = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o) * w.down_row_stride + kBlock * j;
-    const uint32_t* order = r.plan + order_at;
     for (uint32_t c0 = begin; c0 < end; c0 += kDownGroupsAssignments) {
         const uint32_t na = end - c0 < kDownGroupsAssignments ? end - c0 : kDownGroupsAssignments;
         uint32_t src[kDownGroupsAssignments];
         float chain[kDownGroupsAssignments];
 #pragma unroll
         for (uint32_t a = 0; a < kDownGroupsAssignments; ++a) {
-            src[a] = order[c0 + (a < na ? a : na - 1U)];
+            src[a] = ordered(r, order_at, c0 + (a < na ? a : na - 1U));
             chain[a] = 0.0F;
         }
 #pragma unroll 2

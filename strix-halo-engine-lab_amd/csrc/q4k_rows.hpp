@@ -24,6 +24,7 @@
 // Reference arithmetic: src/cpu/core/routed_expert.cpp:73-108 == src/moe_q4k_a8_contract.cpp:126-140.
 #pragma once
 #include "device_math.hpp"
+#include "mi355_strix.h"
 
 namespace strix950 {
 
@@ -36,6 +37,24 @@ __host__ __device__ constexpr uint32_t slot_bytes(int nbmax) { return kStageByte
 typedef __attribute__((address_space(3))) uint8_t lds_u8;      // ring slots are addressed in the LDS address space
 template <int NA> constexpr uint32_t stage_copies() { return kStagePieces + (NA + 3) / 4; }   // copy instructions per stage
 
+
+// The kernels' view of the per-row buffers: the public bundle plus what only some entry points vary.
+struct RowsK : mi355_moe_rows {
+    uint64_t slot_stride;     // floats between the rows of consecutive assignments in gate_out / up_out / h_out (dense: ffn)
+};
+// One work item of an expert launch: assignments [begin, end) of the plan order belong to expert e. Without a plan
+// (plan == nullptr) item i is assignment i alone, its expert read from the routes: the single-row forms of the reference
+// entry points (include/strix/hip_moe_q4k_a8_probe.hpp:12, include/strix/hip_moe_a8_down.hpp:11-30) bring no plan view.
+struct WorkItem { uint32_t e, begin, end; };
+__device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const RowsK& r, uint32_t items_at, uint32_t index) {
+    if (r.plan) {
+        const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * index);
+        return {item.x, item.y, item.z};
+    }
+    const uint32_t e = r.routes[index];
+    return {e, index, e < w.experts ? index + 1U : index};      // an invalid route has no item (its row is flagged)
+}
+__device__ __forceinline__ uint32_t ordered(const RowsK& r, uint32_t order_at, uint32_t i) { return r.plan ? r.plan[order_at + i] : i; }
 
 struct A8Image {                             // device A8 image: codes [rows][width], deltas / sums [rows][width / 32]
     const int8_t* codes;

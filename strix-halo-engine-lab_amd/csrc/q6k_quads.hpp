@@ -30,26 +30,25 @@ __device__ __forceinline__ void load_words_2aligned(const uint8_t* at, uint32_t 
     for (int i = 0; i < N; ++i) out[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
 }
 
-__global__ __launch_bounds__(256) void down_q6k_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments,
+__global__ __launch_bounds__(256) void down_q6k_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments,
                                                        uint32_t items_at, uint32_t order_at) {
     typedef uint32_t u32x4_g __attribute__((ext_vector_type(4)));
     constexpr uint32_t NA = 4;
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * blockIdx.y);
-    const uint32_t e = item.x, begin = item.y, end = item.z;
+    const WorkItem item = work_item(w, r, items_at, blockIdx.y);
+    const uint32_t e = item.e, begin = item.begin, end = item.end;
     if (begin == end) return;
     if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
     const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, p = lane & 3U, half = p >> 1, odd = p & 1U;
     const uint32_t o = blockIdx.x * 64U + 16U * wave + (lane >> 2);
     const uint32_t groups = w.ffn / 32U, blocks = w.ffn / 256U;
     const uint8_t* wrow = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o) * w.down_row_stride;
-    const uint32_t* order = r.plan + order_at;
     for (uint32_t c0 = begin; c0 < end; c0 += NA) {
         const uint32_t na = end - c0 < NA ? end - c0 : NA;
         uint32_t src[NA];
         float acc[NA];
 #pragma unroll
         for (uint32_t a = 0; a < NA; ++a) {
-            src[a] = order[c0 + (a < na ? a : na - 1U)];
+            src[a] = ordered(r, order_at, c0 + (a < na ? a : na - 1U));
             acc[a] = 0.0F;
         }
 #pragma unroll 2

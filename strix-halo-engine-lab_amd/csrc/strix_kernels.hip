@@ -492,18 +492,18 @@ __global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* rout
 // Reference: src/cpu/core/routed_expert.cpp:403-427 (gate item), :147-170 (swiglu_quantize).
 template <int NA, int DEPTH>
 __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
-                                              const mi355_moe_rows& r, uint32_t grp, const uint32_t* order, uint32_t c0) {
+                                              const RowsK& r, uint32_t grp, uint32_t order_at, uint32_t c0) {
     const uint32_t lane = threadIdx.x & 63U, o = lane & 31U, groups = w.ffn / 32U;
     uint32_t sidx[NA], src[NA], lane_rows[(NA + 3) / 4];
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
-        sidx[a] = __builtin_amdgcn_readfirstlane(order[c0 + a]);
+        sidx[a] = __builtin_amdgcn_readfirstlane(ordered(r, order_at, c0 + a));
         src[a] = sidx[a] / w.top_k;
     }
 #pragma unroll
     for (int h = 0; h < (NA + 3) / 4; ++h) {
         const uint32_t a = 4U * h + (lane >> 4);
-        lane_rows[h] = order[c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)] / w.top_k;
+        lane_rows[h] = ordered(r, order_at, c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)) / w.top_k;
     }
     const ActRows<NA> act(A8Image{r.codes, r.deltas, r.sums, w.hidden}, src, lane_rows);
     float value[NA];
@@ -516,11 +516,13 @@ __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], con
         swiglu_clamp(gc, uc, w.swiglu_limit);
         const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
         const size_t at = static_cast<size_t>(sidx[a]) * w.ffn + grp * 32U + o;
+        const size_t at_out = static_cast<size_t>(sidx[a]) * r.slot_stride + grp * 32U + o;
         if (lane < 32U) {
-            if (r.gate_out) r.gate_out[at] = g;
-            if (r.up_out) r.up_out[at] = u;
-            if (r.h_out) r.h_out[at] = h;
+            if (r.gate_out) r.gate_out[at_out] = g;
+            if (r.up_out) r.up_out[at_out] = u;
+            if (r.h_out) r.h_out[at_out] = h;
         }
+        if (!r.down_codes) continue;                      // projection only (the probe form): no A8 image of h
         if (or32_i((finite_f(g) && finite_f(u) && finite_f(h)) ? 0 : 1)) {
             if (lane == 0) {
                 atomicOr(&r.status[sidx[a] / w.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
@@ -552,14 +554,14 @@ __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], con
 
 // NBMAX = most activation rows sharing one sweep of the weights (4 for routed experts, 8 for a dense matrix).
 template <int NBMAX, int DEPTH>
-__global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void project_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+__global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void project_wave_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments) {
     STRIX_RING_SLOTS(DEPTH, NBMAX)
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
-    const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
+    const uint32_t e = __builtin_amdgcn_readfirstlane(item.e), begin = __builtin_amdgcn_readfirstlane(item.begin), end = __builtin_amdgcn_readfirstlane(item.end);
     if (begin == end) return;
     // a wave that serves several activation rows has the longest instruction stream of the launch: let it issue first
     if (end - begin > 1U) __builtin_amdgcn_s_setprio(3);
-    const uint32_t* order = r.plan + plan_order_at(w.experts);
+    const uint32_t order_at = plan_order_at(w.experts);
     const uint32_t grp = blockIdx.x;
     const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U) * w.gate_row_stride;
     const uint8_t* gate = w.gate + base;
@@ -571,17 +573,17 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void project_wave_kernel(mi3
     for (uint32_t c0 = begin; c0 < end;) {
         const uint32_t left = end - c0, na = left < static_cast<uint32_t>(NBMAX) ? left : static_cast<uint32_t>(NBMAX);
         switch (na) {
-        case 1: project_chunk<1, DEPTH>(sl, source, w, r, grp, order, c0); break;
-        case 2: project_chunk<2, DEPTH>(sl, source, w, r, grp, order, c0); break;
-        case 3: project_chunk<3, DEPTH>(sl, source, w, r, grp, order, c0); break;
-        case 4: project_chunk<4, DEPTH>(sl, source, w, r, grp, order, c0); break;
+        case 1: project_chunk<1, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
+        case 2: project_chunk<2, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
+        case 3: project_chunk<3, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
+        case 4: project_chunk<4, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
         default:
             if constexpr (NBMAX == 8) {
                 switch (na) {
-                case 5: project_chunk<5, DEPTH>(sl, source, w, r, grp, order, c0); break;
-                case 6: project_chunk<6, DEPTH>(sl, source, w, r, grp, order, c0); break;
-                case 7: project_chunk<7, DEPTH>(sl, source, w, r, grp, order, c0); break;
-                default: project_chunk<8, DEPTH>(sl, source, w, r, grp, order, c0); break;
+                case 5: project_chunk<5, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
+                case 6: project_chunk<6, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
+                case 7: project_chunk<7, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
+                default: project_chunk<8, DEPTH>(sl, source, w, r, grp, order_at, c0); break;
                 }
             }
             break;
@@ -594,14 +596,14 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void project_wave_kernel(mi3
 // Reference: src/cpu/core/routed_expert.cpp:429-447 (down item), src/moe_a8_down_contract.cpp:146 (Q4_K down row).
 template <int NA, int DEPTH>
 __device__ __forceinline__ void down_chunk(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
-                                           const mi355_moe_rows& r, const uint32_t* order, uint32_t c0) {
+                                           const RowsK& r, uint32_t order_at, uint32_t c0) {
     uint32_t src[NA], lane_rows[(NA + 3) / 4];
 #pragma unroll
-    for (int a = 0; a < NA; ++a) src[a] = __builtin_amdgcn_readfirstlane(order[c0 + a]);
+    for (int a = 0; a < NA; ++a) src[a] = __builtin_amdgcn_readfirstlane(ordered(r, order_at, c0 + a));
 #pragma unroll
     for (int h = 0; h < (NA + 3) / 4; ++h) {
         const uint32_t a = 4U * h + ((threadIdx.x & 63U) >> 4);
-        lane_rows[h] = order[c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)];
+        lane_rows[h] = ordered(r, order_at, c0 + (a < static_cast<uint32_t>(NA) ? a : 0U));
     }
     const ActRows<NA> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src, lane_rows);
     float value[NA];
@@ -612,14 +614,14 @@ __device__ __forceinline__ void down_chunk(lds_u8* const (&slots)[DEPTH], const 
 }
 
 template <int NBMAX, int DEPTH>
-__global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+__global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments) {
     STRIX_RING_SLOTS(DEPTH, NBMAX)
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
-    const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
+    const uint32_t e = __builtin_amdgcn_readfirstlane(item.e), begin = __builtin_amdgcn_readfirstlane(item.begin), end = __builtin_amdgcn_readfirstlane(item.end);
     if (begin == end) return;
     if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
     if (end - begin > 1U) __builtin_amdgcn_s_setprio(3);     // as in the projection: the longest instruction streams issue first
-    const uint32_t* order = r.plan + plan_order_at(w.experts);
+    const uint32_t order_at = plan_order_at(w.experts);
     const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
     const size_t stride = w.down_row_stride;
     StageSource source;
@@ -628,17 +630,17 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_
     for (uint32_t c0 = begin; c0 < end;) {
         const uint32_t left = end - c0, na = left < static_cast<uint32_t>(NBMAX) ? left : static_cast<uint32_t>(NBMAX);
         switch (na) {
-        case 1: down_chunk<1, DEPTH>(sl, source, w, r, order, c0); break;
-        case 2: down_chunk<2, DEPTH>(sl, source, w, r, order, c0); break;
-        case 3: down_chunk<3, DEPTH>(sl, source, w, r, order, c0); break;
-        case 4: down_chunk<4, DEPTH>(sl, source, w, r, order, c0); break;
+        case 1: down_chunk<1, DEPTH>(sl, source, w, r, order_at, c0); break;
+        case 2: down_chunk<2, DEPTH>(sl, source, w, r, order_at, c0); break;
+        case 3: down_chunk<3, DEPTH>(sl, source, w, r, order_at, c0); break;
+        case 4: down_chunk<4, DEPTH>(sl, source, w, r, order_at, c0); break;
         default:
             if constexpr (NBMAX == 8) {
                 switch (na) {
-                case 5: down_chunk<5, DEPTH>(sl, source, w, r, order, c0); break;
-                case 6: down_chunk<6, DEPTH>(sl, source, w, r, order, c0); break;
-                case 7: down_chunk<7, DEPTH>(sl, source, w, r, order, c0); break;
-                default: down_chunk<8, DEPTH>(sl, source, w, r, order, c0); break;
+                case 5: down_chunk<5, DEPTH>(sl, source, w, r, order_at, c0); break;
+                case 6: down_chunk<6, DEPTH>(sl, source, w, r, order_at, c0); break;
+                case 7: down_chunk<7, DEPTH>(sl, source, w, r, order_at, c0); break;
+                default: down_chunk<8, DEPTH>(sl, source, w, r, order_at, c0); break;
                 }
             }
             break;
@@ -661,15 +663,15 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_
 // gate + up + SwiGLU + A8 of one item (one assignment): a 4-wave workgroup per 32-output group, wave = 8 gate rows and the
 // 8 up rows of the same features. Reference: src/cpu/core/routed_expert.cpp:403-427, :147-170.
 template <int DEPTH>
-__global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+__global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments) {
     STRIX_QUAD_SLOTS(DEPTH)
     __shared__ float wg_amax[4];
     __shared__ int wg_sum[4], wg_bad[4];
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
-    const uint32_t e = item.x, begin = item.y, end = item.z;
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
+    const uint32_t e = item.e, begin = item.begin, end = item.end;
     if (begin == end) return;
     const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x, groups = w.ffn / 32U;
-    const uint32_t sidx = __builtin_amdgcn_readfirstlane(r.plan[plan_order_at(w.experts) + begin]), row = sidx / w.top_k;
+    const uint32_t sidx = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), begin)), row = sidx / w.top_k;
     const uint32_t f0 = grp * 32U + 8U * wave;
     const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(f0) * w.gate_row_stride;
     const uint8_t* gate = w.gate + base;
@@ -686,11 +688,13 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
     swiglu_clamp(gc, uc, w.swiglu_limit);
     const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
     const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
+    const size_t at_out = static_cast<size_t>(sidx) * r.slot_stride + f0 + rr;
     if (mine) {
-        if (r.gate_out) r.gate_out[at] = g;
-        if (r.up_out) r.up_out[at] = u;
-        if (r.h_out) r.h_out[at] = h;
+        if (r.gate_out) r.gate_out[at_out] = g;
+        if (r.up_out) r.up_out[at_out] = u;
+        if (r.h_out) r.h_out[at_out] = h;
     }
+    if (!r.down_codes) return;                            // projection only (the probe form): no A8 image of h
     const int bad = or32_i((mine && !(finite_f(g) && finite_f(u) && finite_f(h))) ? 1 : 0);
     const float amax_wave = max32(mine ? __builtin_fabsf(h) : 0.0F);
     if (lane == 0) { wg_amax[wave] = amax_wave; wg_bad[wave] = bad; }
@@ -717,18 +721,18 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
 }
 
 // The same for Q5_K gate / up tensors (q5k_quads.hpp), for every assignment of the item in turn.
-__global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+__global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments) {
     __shared__ float wg_amax[4];
     __shared__ int wg_sum[4], wg_bad[4];
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
-    const uint32_t e = item.x, begin = item.y, end = item.z;
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
+    const uint32_t e = item.e, begin = item.begin, end = item.end;
     const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x, groups = w.ffn / 32U;
     const uint32_t f0 = grp * 32U + 8U * wave;
     const uint8_t* wrow = (lane < 32U ? w.gate : w.up) + static_cast<size_t>(e) * w.gate_expert_stride +
                           static_cast<size_t>(f0 + (rr & 7U)) * w.gate_row_stride;
     const bool mine = lane < 32U && p == 0;                   // the lane that publishes feature f0 + rr
     for (uint32_t a = begin; a < end; ++a) {
-        const uint32_t sidx = __builtin_amdgcn_readfirstlane(r.plan[plan_order_at(w.experts) + a]), row = sidx / w.top_k;
+        const uint32_t sidx = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), a)), row = sidx / w.top_k;
         const float value = sweep_q5k_row(wrow, w.hidden / 256U, A8Image{r.codes, r.deltas, r.sums, w.hidden}, row, p);
         const float other = __shfl_xor(value, 32);
         const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
@@ -736,11 +740,13 @@ __global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, m
         swiglu_clamp(gc, uc, w.swiglu_limit);
         const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
         const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
+        const size_t at_out = static_cast<size_t>(sidx) * r.slot_stride + f0 + rr;
         if (mine) {
-            if (r.gate_out) r.gate_out[at] = g;
-            if (r.up_out) r.up_out[at] = u;
-            if (r.h_out) r.h_out[at] = h;
+            if (r.gate_out) r.gate_out[at_out] = g;
+            if (r.up_out) r.up_out[at_out] = u;
+            if (r.h_out) r.h_out[at_out] = h;
         }
+        if (!r.down_codes) continue;                      // projection only (the probe form): no A8 image of h
         const int bad = or32_i((mine && !(finite_f(g) && finite_f(u) && finite_f(h))) ? 1 : 0);
         const float amax_wave = max32(mine ? __builtin_fabsf(h) : 0.0F);
         __syncthreads();                                          // the previous assignment's reads of the shared words are done
@@ -771,14 +777,14 @@ __global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, m
 // down rows of one item: a 4-wave workgroup per 64 outputs, 16 per wave.
 // Reference: src/cpu/core/routed_expert.cpp:429-447, src/moe_a8_down_contract.cpp:146.
 template <int DEPTH>
-__global__ __launch_bounds__(256) void down_quad_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments) {
+__global__ __launch_bounds__(256) void down_quad_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments) {
     STRIX_QUAD_SLOTS(DEPTH)
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * blockIdx.y);
-    const uint32_t e = item.x, begin = item.y, end = item.z;
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
+    const uint32_t e = item.e, begin = item.begin, end = item.end;
     if (begin == end) return;
     if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;
     const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2;
-    const uint32_t src = __builtin_amdgcn_readfirstlane(r.plan[plan_order_at(w.experts) + begin]);
+    const uint32_t src = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), begin));
     const uint32_t o0 = blockIdx.x * 64U + 16U * wave;
     const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o0) * w.down_row_stride;
     const size_t stride = w.down_row_stride;
@@ -791,7 +797,7 @@ __global__ __launch_bounds__(256) void down_quad_kernel(mi355_moe_weights w, mi3
 
 // Ordered combine of the slots of one row. Reference: include/strix/moe/combine.hpp:36-59 (fma form),
 // src/ds41_expert_tp.cpp:189-199 (product then add, slots in ascending expert id).
-__global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t form) {
+__global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, RowsK r, uint32_t form) {
     __shared__ uint32_t slot_order[16];
     __shared__ float slot_weight[16];
     __shared__ uint32_t row_failed;
@@ -827,7 +833,7 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, mi355_m
 // waves of one workgroup exchange data, so nothing depends on the visibility of another workgroup's stores.
 // Reference: src/cpu/core/routed_expert.cpp:429-447, src/moe_a8_down_contract.cpp:146, include/strix/moe/combine.hpp:36-59.
 constexpr uint32_t kDownMergeSlots = 8;        // top_k bound: 8 waves x 2 ring slots fill the LDS of a compute unit
-__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_moe_weights w, mi355_moe_rows r, uint32_t assignments, uint32_t form) {
+__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
     __shared__ __attribute__((aligned(16))) uint8_t rings[kDownMergeSlots][2][slot_bytes(1)];
     __shared__ float slot_value[kDownMergeSlots][64];
     __shared__ uint32_t slot_order[kDownMergeSlots];
@@ -835,17 +841,17 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, row = blockIdx.y, o = blockIdx.x * 64U + lane;
     if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;            // the whole job: no down rows, nothing published
     const uint32_t a = row * w.top_k + wave;
-    const uint4 item = *reinterpret_cast<const uint4*>(r.plan + plan_items_at(w.experts, assignments) + 4U * a);
-    const uint32_t e = __builtin_amdgcn_readfirstlane(item.x), begin = __builtin_amdgcn_readfirstlane(item.y), end = __builtin_amdgcn_readfirstlane(item.z);
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), a);
+    const uint32_t e = __builtin_amdgcn_readfirstlane(item.e), begin = __builtin_amdgcn_readfirstlane(item.begin), end = __builtin_amdgcn_readfirstlane(item.end);
     float value = 0.0F;
     if (begin != end) {                                                        // (an invalid route has no item: its row is flagged)
-        const uint32_t* order = r.plan + plan_order_at(w.experts);
+        const uint32_t first = ordered(r, plan_order_at(w.experts), begin);
         const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
         const size_t stride = w.down_row_stride;
         StageSource source;
         source.init([&](uint32_t q) { return rows + q * stride; });
         lds_u8* const slots[2] = {(lds_u8*)rings[wave][0], (lds_u8*)rings[wave][1]};
-        const uint32_t src[1] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(order[begin]))}, lane_rows[1] = {order[begin]};
+        const uint32_t src[1] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(first))}, lane_rows[1] = {first};
         const ActRows<1> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src, lane_rows);
         float swept[1];
         sweep_rows<1, 2, true>(slots, source, w.ffn / 256U, act, swept);      // narrow codes copies: the slots are slot_bytes(1)
@@ -917,7 +923,7 @@ inline int ring_depth(uint64_t waves, int nbmax) {
     return 2;
 }
 template <int NBMAX>
-inline void launch_project_nb(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, dim3 grid, hipStream_t st) {
+inline void launch_project_nb(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, dim3 grid, hipStream_t st) {
     switch (ring_depth(static_cast<uint64_t>(grid.x) * grid.y, NBMAX)) {
     case 4: project_wave_kernel<NBMAX, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
     case 3: project_wave_kernel<NBMAX, 3><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
@@ -925,7 +931,7 @@ inline void launch_project_nb(const mi355_moe_weights& w, const mi355_moe_rows& 
     }
 }
 template <int NBMAX>
-inline void launch_down_nb(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, dim3 grid, hipStream_t st) {
+inline void launch_down_nb(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, dim3 grid, hipStream_t st) {
     switch (ring_depth(static_cast<uint64_t>(grid.x) * grid.y, NBMAX)) {
     case 4: down_wave_kernel<NBMAX, 4><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
     case 3: down_wave_kernel<NBMAX, 3><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
@@ -959,7 +965,7 @@ inline bool dense_pairs_ok(const mi355_moe_weights& w, uint32_t rows) {
            w.experts == 1U && w.top_k == 1U && rows <= 8U && (w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0 &&
            w.gate_row_stride < (1ULL << 24) && w.down_row_stride < (1ULL << 24);
 }
-inline void launch_project_dense(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, hipStream_t st) {
+inline void launch_project_dense(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, hipStream_t st) {
     PairArgs a{};
     a.m[0] = PairMatrix{w.gate, w.gate_row_stride, r.gate_out, w.ffn};
     a.m[1] = PairMatrix{w.up, w.gate_row_stride, r.up_out, w.ffn};
@@ -968,7 +974,7 @@ inline void launch_project_dense(const mi355_moe_weights& w, const mi355_moe_row
     swiglu_quantize_kernel<<<dim3((w.ffn / 32U + 7U) / 8U, rows), 256, 0, st>>>(r.gate_out, r.up_out, w.ffn, w.exp_kind, w.swiglu_limit, r.down_codes, r.down_deltas,
                                                                                 r.down_sums, r.h_out, r.status, r.job_status);
 }
-inline void launch_down_dense(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, hipStream_t st) {
+inline void launch_down_dense(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, hipStream_t st) {
     PairArgs a{};
     a.m[0] = PairMatrix{w.down, w.down_row_stride, r.rawdots, w.hidden};
     a.rows = w.hidden; a.blocks = w.ffn / 256U; a.img = A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}; a.nacts = rows;
@@ -992,7 +998,7 @@ constexpr uint32_t kQuadMaxItems = 48;
 inline bool quad_sweep(const mi355_moe_weights& w, uint32_t rows) {
     return rows <= kFusedMaxRows && rows * w.top_k <= kQuadMaxItems && w.experts > 1U;
 }
-inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     if (w.gate_type == MI355_TYPE_Q5_K) {
         project_q5k_kernel<<<dim3(w.ffn / 32U, umax), 256, 0, st>>>(w, r, rows * w.top_k);
         return;
@@ -1008,7 +1014,7 @@ inline void launch_project(const mi355_moe_weights& w, const mi355_moe_rows& r, 
     if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
     else launch_project_nb<4>(w, r, rows, grid, st);
 }
-inline void launch_down(const mi355_moe_weights& w, const mi355_moe_rows& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st) {
     if (w.down_type != MI355_TYPE_Q4_K) {      // Q8_0 / Q5_1 (blocks of 32, four chains per row) and Q6_K (pairs per super-block)
         const uint32_t assignments = rows * w.top_k, items_at = plan_items_at(w.experts, assignments), order_at = plan_order_at(w.experts);
         const dim3 grid(w.hidden / kDownGroupsRows, umax);
@@ -1057,6 +1063,14 @@ inline uint32_t compute_units() {
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) return 0;
     if (device < 64) known[device].store(static_cast<uint32_t>(cus), std::memory_order_relaxed);
     return static_cast<uint32_t>(cus);
+}
+
+// the kernels' view of a dense row bundle
+inline RowsK rows_k(const mi355_moe_rows& r, const mi355_moe_weights& w) {
+    RowsK k{};
+    static_cast<mi355_moe_rows&>(k) = r;
+    k.slot_stride = w.ffn;
+    return k;
 }
 
 // ======================================================================================================== admission
@@ -1128,14 +1142,34 @@ const char* mi355_last_error(void) { return g_error.c_str(); }
 const char* mi355_version(void) { return "mi355-strix 0.1 (gfx950)"; }
 
 const char* mi355_numerical_identity(uint32_t weight_type, int down) {
-    // The reference's identity strings name wave32; the arithmetic clauses are the ones implemented here.
-    if (weight_type == MI355_TYPE_Q4_K && !down)
-        return "strix-moe-q4k-a8g32-probe-v2:f32-div-rne:g32-sym127-zero1-finite-noflush:"
-               "dot-s8xu8-i32:combine-separate-f32:pair-ascending-sb-tree4:writer-c0:wave64-gfx950";
+    // Identity strings are the admission tokens of the reference's contracts (include/strix/moe_q4k_a8_contract.hpp:24-29,
+    // include/strix/moe_a8_down_contract.hpp:9-28); a caller hands over the token of the arithmetic it approved. The tokens are
+    // returned verbatim because the bits are the same: "wave32" in the probe tokens names the reference's reduction tree
+    // (pairs ascending, four super-block partials folded by a two-level tree), which the 64-lane kernels here reproduce.
+    if (!down) {
+        if (weight_type == MI355_TYPE_Q4_K)
+            return "strix-moe-q4k-a8g32-probe-v2:f32-div-rne:g32-sym127-zero1-finite-noflush:"
+                   "dot-s8xu8-i32:combine-separate-f32:pair-ascending-sb-tree4:writer-c0:wave32:proj-nonfinite=propagate-unqualified";
+        if (weight_type == MI355_TYPE_Q5_K)
+            return "strix-moe-q5k-a8g32-probe-v1:f32-div-rne:g32-sym127-zero1-finite-noflush:"
+                   "dot-s8xu5qh-i32:combine-separate-f32:pair-ascending-sb-tree4:writer-c0:wave32:proj-nonfinite=propagate-unqualified";
+        if (weight_type == MI355_TYPE_Q8_0) return "cpu-q8a8-tree32@1";
+        return "";
+    }
     if (weight_type == MI355_TYPE_Q4_K)
         return "q4k-a8g32-down-v1:s8xu4-i32:delta*((d*(sc*I))-(dmin*(m*S))):pair-ascending-sb-tree4:"
                "silu-div-expf-times-up:g32-sym127-f32delta-rne:tiny-lt2^-119-zero1:raw-slot-major:finite-failclosed";
-    if (weight_type == MI355_TYPE_Q8_0) return "cpu-q8a8-tree32@1";
+    if (weight_type == MI355_TYPE_Q6_K)
+        return "q6k-a8g32-down-v1:s8xs8-i32:delta*(d*(s0*I0+s1*I1)):pair-ascending-sb-tree4:"
+               "silu-div-expf-times-up:g32-sym127-f32delta-rne:tiny-lt2^-119-zero1:raw-slot-major:finite-failclosed";
+    if (weight_type == MI355_TYPE_Q5_1)
+        return "q51-a8g32-down-v1:s8xu5-i32:delta*(d*S+m*C):separate-f32:"
+               "silu-div-expf-times-up:g32-sym127-f32delta-rne:tiny-lt2^-119-zero1:"
+               "blocks-mod4-ascending:tree-xor1-xor2:raw-slot-major:finite-failclosed";
+    if (weight_type == MI355_TYPE_Q8_0)
+        return "q80-a8g32-down-v1:s8xs8-i32:delta*(d*S):separate-f32:"
+               "silu-div-expf-times-up:g32-sym127-f32delta-rne:tiny-lt2^-119-zero1:"
+               "blocks-mod4-ascending:tree-xor1-xor2:raw-slot-major:finite-failclosed";
     return "";
 }
 
@@ -1305,7 +1339,7 @@ int32_t mi355_moe_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows* 
 int32_t mi355_moe_enqueue_project(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    launch_project(wv, *r, rows, item_bound(wv, rows), hs(stream));
+    launch_project(wv, rows_k(*r, wv), rows, item_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe project");
     return MI355_OK;
 }
@@ -1313,7 +1347,7 @@ int32_t mi355_moe_enqueue_project(const mi355_moe_weights* w, const mi355_moe_ro
 int32_t mi355_moe_enqueue_down(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    launch_down(wv, *r, rows, item_bound(wv, rows), hs(stream));
+    launch_down(wv, rows_k(*r, wv), rows, item_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe down");
     return MI355_OK;
 }
@@ -1323,7 +1357,7 @@ int32_t mi355_moe_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows
     if (const int32_t rc = check_moe(w, r, rows, wv, kAnyClass)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe merge: unknown combine form");
     STRIX_REQUIRE(rows <= 65535U, "moe merge: at most 65535 rows per call");
-    merge_kernel<<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(wv, *r, form);
+    merge_kernel<<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(wv, rows_k(*r, wv), form);
     STRIX_LAUNCHED("moe merge");
     return MI355_OK;
 }
@@ -1365,17 +1399,17 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     STRIX_LAUNCHED("moe layer router");
     // the fused router planned one item per assignment
     const uint32_t items = rows * wv.top_k;
-    launch_project(wv, *r, rows, items, hs(stream));
+    launch_project(wv, rows_k(*r, wv), rows, items, hs(stream));
     // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
     // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
     // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
     if (!quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
         (wv.hidden / 64U) * rows <= compute_units()) {
-        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, hs(stream)>>>(wv, *r, items, form);
+        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, hs(stream)>>>(wv, rows_k(*r, wv), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
-    launch_down(wv, *r, rows, items, hs(stream));
+    launch_down(wv, rows_k(*r, wv), rows, items, hs(stream));
     STRIX_LAUNCHED("moe layer experts");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
@@ -1524,3 +1558,5 @@ int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float*
 }
 
 }  // extern "C"
+
+#include "a8_contract.hpp"

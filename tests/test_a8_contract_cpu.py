@@ -1,0 +1,237 @@
+"""Host admission of the A8 request / bindings boundary (mi355_a8_validate, mi355_a8_validate_down) against the compiled
+reference's validate / validate_down (src/moe_q4k_a8_contract.cpp:343-372, src/moe_a8_down_contract.cpp:53-82) on the same
+requests. Pure host code on both sides: the device addresses are made-up numbers that nothing dereferences."""
+import ctypes as C
+import importlib.util
+import math
+import os
+import random
+
+import pytest
+
+import orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "strix-halo-engine-lab_amd", "libmi355_strix.so")
+INF = math.inf
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    spec = importlib.util.spec_from_file_location("strix_pkg_a8", os.path.join(ROOT, "strix-halo-engine-lab_amd", "__init__.py"))
+    m = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(m)
+    return m
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        import __graft_entry__
+        __graft_entry__.build()
+    L = C.CDLL(LIB)
+    L.mi355_numerical_identity.restype = C.c_char_p
+    L.mi355_last_error.restype = C.c_char_p
+    return L
+
+
+@pytest.fixture(scope="module")
+def ref():
+    r = orc.ref()
+    if not r:
+        pytest.skip("oracle/_ref was not built (no reference tree at build time)")
+    r.ref_a8_identity.restype = C.c_char_p
+    return r
+
+
+def test_identity_tokens_are_the_reference_tokens(lib, ref):
+    for type_, down in ((12, 0), (13, 0), (12, 1), (14, 1), (7, 1), (8, 1)):
+        assert lib.mi355_numerical_identity(type_, down) == ref.ref_a8_identity(type_, down), (type_, down)
+        assert len(lib.mi355_numerical_identity(type_, down)) > 40
+
+
+def probe_required(hidden, rows, experts, top_k, R, gate_type, fp32):
+    wb = experts * rows * (hidden // 256) * (176 if gate_type == 13 else 144)
+    return [R * hidden * (4 if fp32 else 2), wb, wb, R * top_k * 4, R * hidden, R * (hidden // 32) * 4, R * (hidden // 32) * 4, 4,
+            R * top_k * 2 * rows * 4]
+
+
+def down_row_bytes(type_, inter):
+    return {12: inter // 256 * 144, 14: inter // 256 * 210, 7: inter // 32 * 24, 8: inter // 32 * 34}[type_]
+
+
+def down_required(hidden, inter, experts, top_k, R, type_):
+    groups = top_k * (inter // 32)
+    return [R * top_k * 2 * inter * 4, experts * hidden * down_row_bytes(type_, inter), R * top_k * 4, R * top_k * inter, R * groups * 4,
+            R * groups * 4, R * top_k * hidden * 4, 4, 4]
+
+
+def lay_out(required, base=0x7000_0000_0000):
+    """Nine disjoint 256-aligned views of exactly the required sizes."""
+    views, at = [], base
+    for n in required:
+        views.append([at, n])
+        at += (n + 255) // 256 * 256 + 256
+    return views
+
+
+def call_probe(lib, ref, pkg, q, views):
+    """(mine, reference) admission of one request: True = admitted."""
+    ident = q["identity"]
+    req = pkg.A8Request(q["enabled"], ident, pkg.INPUT_F32 if q["fp32"] else pkg.INPUT_BF16,
+                        pkg.A8Shape(q["hidden"], q["rows"], q["experts"], q["top_k"], q["R"]), q["gate"], q["up"], q["fused"], q["limit"])
+    b = pkg.A8Bindings(*[pkg.DeviceBytes(a, n) for a, n in views])
+    mine = lib.mi355_a8_validate(C.byref(req), C.byref(b)) == 0
+    flat = (C.c_uint64 * 18)(*[v for pair in views for v in pair])
+    theirs = ref.ref_a8_validate(q["enabled"], ident, int(q["fp32"]), q["hidden"], q["rows"], q["experts"], q["top_k"], q["R"], q["gate"], q["up"],
+                                 q["fused"], C.c_float(q["limit"]), flat) == 0
+    return mine, theirs
+
+
+def call_down(lib, ref, pkg, q, views, R=1):
+    req = pkg.A8DownRequest(q["enabled"], q["identity"], pkg.A8DownShape(q["hidden"], q["inter"], q["experts"], q["top_k"]), q["type"], q["limit"])
+    b = pkg.A8DownBindings(*[pkg.DeviceBytes(a, n) for a, n in views])
+    mine = lib.mi355_a8_validate_down(C.byref(req), C.byref(b), R) == 0
+    flat = (C.c_uint64 * 18)(*[v for pair in views for v in pair])
+    theirs = ref.ref_a8_validate_down(q["enabled"], q["identity"], q["hidden"], q["inter"], q["experts"], q["top_k"], q["type"], C.c_float(q["limit"]),
+                                      flat) == 0
+    return mine, theirs
+
+
+def probe_request(lib, **over):
+    q = dict(enabled=1, fp32=False, hidden=2048, rows=768, experts=128, top_k=8, R=1, gate=12, up=12, fused=0, limit=INF)
+    q.update(over)
+    q.setdefault("identity", lib.mi355_numerical_identity(q["gate"], 0))
+    return q
+
+
+def down_request(lib, **over):
+    q = dict(enabled=1, hidden=2048, inter=768, experts=128, top_k=8, type=12, limit=INF)
+    q.update(over)
+    q.setdefault("identity", lib.mi355_numerical_identity(q["type"], 1))
+    return q
+
+
+def test_probe_admission_agrees_with_the_reference(lib, ref, pkg):
+    """Inside the reference's geometry caps the two admit and refuse the same requests: identity, enable flag, dimensions,
+    tensor types, exact extents, alignment, overlap of a mutable view with any other view."""
+    rng = random.Random(5)
+    good = probe_request(lib)
+    views = lay_out(probe_required(2048, 768, 128, 8, 1, 12, False))
+    assert call_probe(lib, ref, pkg, good, views) == (True, True)
+    cases = [dict(enabled=0), dict(identity=b"something else"), dict(identity=None), dict(identity=lib.mi355_numerical_identity(13, 0)),
+             dict(hidden=0), dict(hidden=2048 + 128), dict(rows=0), dict(rows=48), dict(experts=0), dict(top_k=0), dict(top_k=17),
+             dict(gate=13), dict(up=13), dict(gate=13, up=13), dict(gate=13, up=13, identity=lib.mi355_numerical_identity(13, 0)),
+             dict(gate=8, up=8), dict(fused=1), dict(fp32=True), dict(R=0)]
+    for over in cases:
+        q = probe_request(lib, **over) if "identity" in over else probe_request(lib, **over, identity=good["identity"])
+        req = probe_required(max(q["hidden"], 0), q["rows"], q["experts"], q["top_k"], max(q["R"], 1), q["gate"], q["fp32"])
+        mine, theirs = call_probe(lib, ref, pkg, q, lay_out(req))
+        assert mine == theirs, (over, lib.mi355_last_error())
+    seen = {True: 0, False: 0}
+    for _ in range(400):
+        hidden, rows, experts, top_k = rng.choice([256, 1024, 2560]), rng.choice([32, 96, 768, 1536]), rng.choice([1, 7, 512]), rng.choice([1, 4, 16])
+        gate = rng.choice([12, 13])
+        q = probe_request(lib, hidden=hidden, rows=rows, experts=experts, top_k=top_k, gate=gate, up=gate, fp32=rng.random() < 0.5)
+        v = lay_out(probe_required(hidden, rows, experts, top_k, 1, gate, q["fp32"]))
+        kind = rng.randrange(6)
+        i = rng.randrange(9)
+        if kind == 1:
+            v[i][1] += rng.choice([-1, 1, 16, -16])          # not the exact extent
+        elif kind == 2:
+            v[i][0] += rng.choice([1, 2, 4, 8])              # misaligned
+        elif kind == 3:
+            v[i][0] = 0                                      # null
+        elif kind == 4:
+            j = rng.randrange(9)                             # view i starts inside view j
+            if j != i:
+                v[i][0] = v[j][0] + (rng.randrange(v[j][1]) // 16) * 16
+        elif kind == 5:
+            j = rng.randrange(9)                             # view i ends inside view j (or just touches it)
+            if j != i:
+                v[i][0] = v[j][0] - v[i][1] + rng.choice([0, 16]) - (v[j][0] - v[i][1]) % 16
+        mine, theirs = call_probe(lib, ref, pkg, q, v)
+        assert mine == theirs, (q, kind, i, v, lib.mi355_last_error())
+        seen[mine] += 1
+    assert seen[True] > 60 and seen[False] > 120
+
+
+def test_probe_admission_beyond_the_reference_caps(lib, ref, pkg):
+    """What this library widens, and only that: hidden / rows / experts beyond 2560 / 1536 / 512, fp16 input and up to 16
+    logical rows are admitted here and refused by the reference; a finite clamp is refused (it belongs to the down producer)."""
+    for over in (dict(hidden=4096), dict(rows=2048), dict(experts=1024), dict(R=4), dict(R=16)):
+        q = probe_request(lib, **over)
+        v = lay_out(probe_required(q["hidden"], q["rows"], q["experts"], q["top_k"], q["R"], 12, False))
+        assert call_probe(lib, ref, pkg, q, v) == (True, False), over
+    for over in (dict(hidden=16384 + 256), dict(rows=16384 + 32), dict(experts=1025), dict(R=17)):
+        q = probe_request(lib, **over)
+        v = lay_out(probe_required(q["hidden"], q["rows"], q["experts"], q["top_k"], q["R"], 12, False))
+        assert call_probe(lib, ref, pkg, q, v) == (False, False), over
+    q = probe_request(lib, limit=10.0)
+    mine, _ = call_probe(lib, ref, pkg, q, lay_out(probe_required(2048, 768, 128, 8, 1, 12, False)))
+    assert not mine and b"clamp" in lib.mi355_last_error()
+    # the per-row views of R rows are R single-row extents: a bundle sized for one row is refused for four
+    q = probe_request(lib, R=4)
+    mine, _ = call_probe(lib, ref, pkg, q, lay_out(probe_required(2048, 768, 128, 8, 1, 12, False)))
+    assert not mine
+    # fp16 input (kind 1) has the extent of bf16
+    req = pkg.A8Request(1, q["identity"], pkg.INPUT_F16, pkg.A8Shape(2048, 768, 128, 8, 1), 12, 12, 0, INF)
+    b = pkg.A8Bindings(*[pkg.DeviceBytes(a, n) for a, n in lay_out(probe_required(2048, 768, 128, 8, 1, 12, False))])
+    assert lib.mi355_a8_validate(C.byref(req), C.byref(b)) == 0
+    req.input = 3
+    assert lib.mi355_a8_validate(C.byref(req), C.byref(b)) != 0
+
+
+def test_down_admission_agrees_with_the_reference(lib, ref, pkg):
+    rng = random.Random(9)
+    good = down_request(lib)
+    assert call_down(lib, ref, pkg, good, lay_out(down_required(2048, 768, 128, 8, 1, 12))) == (True, True)
+    for over in (dict(enabled=0), dict(identity=b"x"), dict(identity=None), dict(identity=lib.mi355_numerical_identity(14, 1)), dict(limit=0.0),
+                 dict(limit=-1.0), dict(limit=-INF), dict(limit=math.nan), dict(limit=10.0), dict(hidden=0), dict(hidden=2048 + 32), dict(inter=0),
+                 dict(inter=768 + 128), dict(experts=0), dict(top_k=0), dict(top_k=17)):
+        q = down_request(lib, **over) if "identity" in over else down_request(lib, **over, identity=good["identity"])
+        v = lay_out(down_required(q["hidden"], q["inter"], q["experts"], q["top_k"], 1, 12))
+        mine, theirs = call_down(lib, ref, pkg, q, v)
+        assert mine == theirs, (over, lib.mi355_last_error())
+    seen = {True: 0, False: 0}
+    for _ in range(500):
+        type_ = rng.choice([12, 14, 7, 8])
+        kq = type_ in (12, 14)
+        hidden, experts = rng.choice([64, 2048, 2560]), rng.choice([1, 60, 512])
+        inter = rng.choice([256, 768, 1536] if kq else [128, 384, 640])
+        top_k = rng.choice([1, 8, 16] if kq else [1, 8, 10, 11])
+        q = down_request(lib, hidden=hidden, inter=inter, experts=experts, top_k=top_k, type=type_, limit=rng.choice([INF, 7.0]))
+        v = lay_out(down_required(hidden, inter, experts, top_k, 1, type_))
+        kind, i = rng.randrange(7), rng.randrange(9)
+        if kind == 1:
+            v[i][1] += rng.choice([-1, 1, 16, -16])
+        elif kind == 2:
+            if i == 1 and type_ != 12:
+                continue                                     # this library asks 16 bytes of every weight tensor, the reference 2
+            v[i][0] += rng.choice([1, 2, 4, 8])
+        elif kind == 3:
+            v[i] = [0, 0] if i == 8 and rng.random() < 0.5 else [0, v[i][1]]      # the aggregate word is optional
+        elif kind == 4:
+            j = rng.randrange(9)
+            if j != i:
+                v[i][0] = v[j][0] + (rng.randrange(v[j][1]) // 16) * 16
+        elif kind == 5:
+            j = rng.randrange(9)
+            if j != i:
+                v[i][0] = v[j][0] - v[i][1] + rng.choice([0, 16]) - (v[j][0] - v[i][1]) % 16
+        mine, theirs = call_down(lib, ref, pkg, q, v)
+        if not kq and top_k == 11:
+            assert not theirs and (mine or kind not in (0, 6)), (q, kind)      # K <= 10 is the reference's cap for these classes, 16 here
+            continue
+        assert mine == theirs, (q, kind, i, v, lib.mi355_last_error())
+        seen[mine] += 1
+    assert seen[True] > 80 and seen[False] > 120
+    # other weight types are not this library's (the reference also knows 20 and 42)
+    q = down_request(lib, type=13, identity=good["identity"])
+    mine, theirs = call_down(lib, ref, pkg, q, lay_out(down_required(2048, 768, 128, 8, 1, 12)))
+    assert (mine, theirs) == (False, False)
+    # logical rows: R single-row extents per row view, 1..16
+    for R, ok in ((4, True), (16, True), (0, False), (17, False)):
+        q = down_request(lib)
+        mine, _ = call_down(lib, ref, pkg, q, lay_out(down_required(2048, 768, 128, 8, max(R, 1), 12)), R=R)
+        assert mine == ok, R
