@@ -134,6 +134,10 @@ int32_t mi355_moe_route(const mi355_route_policy* policy, const void* x, uint32_
                         uint32_t hidden, uint64_t x_stride_bytes, const float* router_weight, const float* logit_bias,
                         uint32_t* ids, float* weights, float* scores, mi355_stream stream);
 
+/* The host executor's per-row A8 image and assignment (RowA8, Assignment: src/cpu/core/routed_expert.hpp:41-49), device pointers. */
+typedef struct mi355_row_a8 { const int8_t* codes; const float* deltas; const int32_t* sums; } mi355_row_a8;
+typedef struct mi355_expert_assignment { uint32_t row, slot, expert; } mi355_expert_assignment;
+
 /* ------------------------------------------------------------------------------------------------------
  * Routed experts. The whole-layer form follows the reference's host API for one MoE layer
  * (include/strix/cuda/qwen_moe.hpp:55-110: Rows / Weights, enqueue_prologue / csr / project / down / merge) and
@@ -320,6 +324,75 @@ typedef struct mi355_slot_merge_tail {
     uint32_t output_bf16, bf16_commit; void* record; uint32_t domain;
 } mi355_slot_merge_tail;
 int32_t mi355_a8_enqueue_down_rawdots_merge(const mi355_a8_down_request*, const mi355_a8_down_bindings*, const mi355_slot_merge_tail*, mi355_stream);
+
+/* ------------------------------------------------------------------------------------------------------
+ * The strided form of the per-row views: the reference's multi-row entry binds every view as Strided<T>{base, stride in
+ * bytes}, row r at base + r * stride (Rows, include/strix/cuda/qwen_moe.hpp:34-37,55-76 = the views of the HIP
+ * KnownMoePrefillPrepared, src/hip_moe_experts_launcher.hip:2884-2904); a caller that holds such buffers binds them here
+ * without a copy. Field for field Rows, with this library's plan words in the place of the reference's Csr views and the
+ * job word (the reference's csr.summary[0]) named. Per row: input [hidden] (input_kind; the reference: bf16), routes
+ * [top_k], route_weights [top_k], codes [hidden], deltas / sums [hidden / 32], status [1], intermediates [top_k][2][ffn]
+ * (h in the place of gate | up; base may be null), accumulation [>= hidden floats], down_codes [top_k][ffn], down_deltas /
+ * down_sums [top_k][ffn / 32], rawdots [top_k][hidden], output [hidden] (output_kind: MI355_INPUT_BF16 as in the reference,
+ * or MI355_INPUT_F32). Every base and stride is a multiple of 16 bytes (routes, route_weights, status: 4).
+ * Stages, same names and order as the reference (include/strix/cuda/qwen_moe.hpp:96-110):
+ *   prologue  zero accumulation[0 .. clear_words), check the routes (bad id or non-finite weight: status = 1, row not
+ *             quantised), A8 image of the input with the probe contract's quantiser (no tiny-group rule; non-finite value:
+ *             bit 2; delta underflow: bit 4), image stored for a clean row only, status OVERWRITTEN
+ *   csr       the expert plan; job_status = OR of every row's status
+ *   project / down   the integer-class expert kernels (bitwise mi355_moe_enqueue_project / _down)
+ *   merge     nothing for a failed job or row; accumulation[o] = fma chain over the slots in slot order from +0; a value whose
+ *             magnitude bits reach 0x7f7f8000 (bf16 output; fp32 output: 0x7f800000) sets bit 8 in the row and the job
+ *   commit    record = DeferredMoeFirstError {domain, bits} of the first failed row (a record already set stays,
+ *             include/strix/deferred_moe_status.hpp:19-26); a failed job commits nothing; else output = accumulation
+ *             (bf16: round to nearest even)
+ */
+typedef struct mi355_strided { void* base; uint64_t stride; } mi355_strided;
+typedef struct mi355_moe_rows_strided {
+    mi355_strided input, routes, route_weights, codes, deltas, sums, status, intermediates, accumulation,
+                  down_codes, down_deltas, down_sums, rawdots, output;
+    uint32_t* plan;              /* mi355_moe_plan_words(experts, rows, top_k) words, 16-byte aligned */
+    uint32_t* job_status;        /* one word */
+    uint32_t input_kind, output_kind;
+} mi355_moe_rows_strided;
+int32_t mi355_moe_strided_enqueue_prologue(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, uint32_t clear_words, mi355_stream);
+int32_t mi355_moe_strided_enqueue_csr(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, mi355_stream);
+int32_t mi355_moe_strided_enqueue_project(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, mi355_stream);
+int32_t mi355_moe_strided_enqueue_down(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, mi355_stream);
+int32_t mi355_moe_strided_enqueue_merge(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, mi355_stream);
+int32_t mi355_moe_strided_enqueue_commit(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, uint32_t* record, uint32_t domain,
+                                         mi355_stream);
+/* prologue + csr + project + down + merge + commit (enqueue, include/strix/cuda/qwen_moe.hpp:107) */
+int32_t mi355_moe_strided_enqueue(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, uint32_t clear_words, uint32_t* record,
+                                  uint32_t domain, mi355_stream);
+
+/* ------------------------------------------------------------------------------------------------------
+ * The job form of the host executor (strix::cpu::expert::Job / LayerWeights / Executor, src/cpu/core/routed_expert.hpp:28-61,
+ * 79-95): a list of (row, slot, expert) assignments over per-row A8 images, every pointer device memory.
+ * rawdots[row * rawdot_row_stride + slot * hidden + o] receives the unweighted down rows; a non-finite gate / up / h value
+ * ORs 1 (kNonfinite) into status[row] and the job then computes no down row at all (src/cpu/core/routed_expert.cpp:403-447,
+ * 461). The executor object owns the A8 image of h for up to max_assignments assignments of up to max_ffn values
+ * (allocated at create, as the host Executor owns its scratch); run allocates nothing and does not synchronise. Expert ids
+ * are trusted, as on the host. One job at a time per executor.
+ */
+typedef struct mi355_layer_weights {
+    const uint8_t* gate; const uint8_t* up; const uint8_t* down;      /* GGUF order: gate / up [experts][ffn][hidden / 256], down [experts][hidden][ffn / 32] */
+    uint32_t gate_format;        /* GateFormat: 0 = Q4_K, 1 = Q5_K */
+    uint32_t down_format;        /* DownFormat: 0 = Q5_1, 1 = Q8_0 */
+    uint32_t hidden, ffn;        /* Shape: hidden % 256, ffn % 128 */
+} mi355_layer_weights;
+typedef struct mi355_expert_job {
+    mi355_layer_weights weights;
+    const mi355_row_a8* rows;                    /* indexed by assignment.row */
+    const mi355_expert_assignment* assignments;
+    uint32_t count;
+    float* rawdots;
+    uint64_t rawdot_row_stride;                  /* in floats */
+    uint32_t* status;                            /* per row, OR-ed */
+} mi355_expert_job;
+void* mi355_executor_create(uint32_t max_assignments, uint32_t max_ffn, uint32_t exp_kind);      /* NULL on failure (mi355_last_error) */
+int32_t mi355_executor_run(void* executor, const mi355_expert_job* job, mi355_stream);
+void mi355_executor_destroy(void* executor);
 
 #ifdef __cplusplus
 }

@@ -92,6 +92,34 @@ class SlotMergeTail(C.Structure):
                 ("output_bf16", C.c_uint32), ("bf16_commit", C.c_uint32), ("record", C.c_void_p), ("domain", C.c_uint32)]
 
 
+class Strided(C.Structure):
+    _fields_ = [("base", C.c_void_p), ("stride", C.c_uint64)]
+
+
+class MoeRowsStrided(C.Structure):
+    _fields_ = [(n, Strided) for n in ("input", "routes", "route_weights", "codes", "deltas", "sums", "status", "intermediates", "accumulation",
+                                        "down_codes", "down_deltas", "down_sums", "rawdots", "output")] + \
+               [("plan", C.c_void_p), ("job_status", C.c_void_p), ("input_kind", C.c_uint32), ("output_kind", C.c_uint32)]
+
+
+class RowA8(C.Structure):
+    _fields_ = [("codes", C.c_void_p), ("deltas", C.c_void_p), ("sums", C.c_void_p)]
+
+
+class ExpertAssignment(C.Structure):
+    _fields_ = [("row", C.c_uint32), ("slot", C.c_uint32), ("expert", C.c_uint32)]
+
+
+class LayerWeights(C.Structure):
+    _fields_ = [("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p), ("gate_format", C.c_uint32), ("down_format", C.c_uint32),
+                ("hidden", C.c_uint32), ("ffn", C.c_uint32)]
+
+
+class ExpertJob(C.Structure):
+    _fields_ = [("weights", LayerWeights), ("rows", C.c_void_p), ("assignments", C.c_void_p), ("count", C.c_uint32), ("rawdots", C.c_void_p),
+                ("rawdot_row_stride", C.c_uint64), ("status", C.c_void_p)]
+
+
 def device_bytes(t):
     """DeviceBytes of a tensor (None: the empty view)."""
     return DeviceBytes(0, 0) if t is None else DeviceBytes(t.data_ptr(), t.numel() * t.element_size())
@@ -109,6 +137,23 @@ def lib():
         L = C.CDLL(LIB_PATH)
         L.mi355_last_error.restype = C.c_char_p
         L.mi355_version.restype = C.c_char_p
+        # every pointer parameter is declared: an undeclared Python integer would be passed as a 32-bit C int
+        P, U = C.c_void_p, C.c_uint32
+        for name in ("prologue", "csr", "project", "down", "merge"):
+            getattr(L, "mi355_moe_strided_enqueue_" + name).argtypes = [P, P, U] + ([U] if name == "prologue" else []) + [P]
+        L.mi355_moe_strided_enqueue_commit.argtypes = [P, P, U, P, U, P]
+        L.mi355_moe_strided_enqueue.argtypes = [P, P, U, U, P, U, P]
+        L.mi355_a8_validate.argtypes = [P, P]
+        L.mi355_a8_validate_down.argtypes = [P, P, U]
+        L.mi355_a8_enqueue_probe.argtypes = [P, P, P]
+        L.mi355_a8_enqueue_down_activation_quantize.argtypes = [P, P, U, U, P]
+        L.mi355_a8_enqueue_down_rawdots.argtypes = [P, P, U, P]
+        L.mi355_a8_enqueue_down_rawdots_merge.argtypes = [P, P, P, P]
+        L.mi355_executor_create.argtypes = [U, U, U]
+        L.mi355_executor_create.restype = C.c_void_p
+        L.mi355_executor_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.mi355_executor_destroy.argtypes = [C.c_void_p]
+        L.mi355_executor_destroy.restype = None
         L.mi355_numerical_identity.restype = C.c_char_p
         L.mi355_numerical_identity.argtypes = [C.c_uint32, C.c_int]
         L.mi355_moe_plan_words.restype = C.c_size_t
@@ -124,7 +169,10 @@ EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi3
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
            "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe",
-           "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge"]
+           "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
+           "mi355_moe_strided_enqueue_prologue", "mi355_moe_strided_enqueue_csr", "mi355_moe_strided_enqueue_project", "mi355_moe_strided_enqueue_down",
+           "mi355_moe_strided_enqueue_merge", "mi355_moe_strided_enqueue_commit", "mi355_moe_strided_enqueue", "mi355_executor_create",
+           "mi355_executor_run", "mi355_executor_destroy"]
 
 
 def require_gpu():
@@ -285,6 +333,27 @@ class A8Decode:
         q, b = self.down_request(), self.down_bindings(1)
         tail = SlotMergeTail(None, _p(route_weights), _p(accumulation), _p(output), int(output.dtype == torch.bfloat16), int(bf16_commit), _p(record), domain)
         check(lib().mi355_a8_enqueue_down_rawdots_merge(C.byref(q), C.byref(b), C.byref(tail), _stream()))
+
+
+class Executor:
+    """The host executor's object on the GPU (strix::cpu::expert::Executor, src/cpu/core/routed_expert.hpp:79-95): create once,
+    run(job) per step, destroy. Workspace for max_assignments x max_ffn is allocated at construction; run allocates nothing."""
+
+    def __init__(self, max_assignments, max_ffn, exp_kind=EXP_GFX1151):
+        self.handle = lib().mi355_executor_create(max_assignments, max_ffn, exp_kind)
+        if not self.handle:
+            raise StrixError(E_INVALID_ARGUMENT, lib().mi355_last_error().decode())
+
+    def run(self, job):
+        check(lib().mi355_executor_run(self.handle, C.byref(job), _stream()))
+
+    def close(self):
+        if self.handle:
+            lib().mi355_executor_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        self.close()
 
 
 class MoeLayer:

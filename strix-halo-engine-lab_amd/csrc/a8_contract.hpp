@@ -103,18 +103,23 @@ __global__ __launch_bounds__(256) void a8_probe_prologue_kernel(const uint8_t* x
     const uint32_t r = blockIdx.y, groups = hidden / 32U, g = blockIdx.x * 8U + (threadIdx.x >> 5), j = threadIdx.x & 31U;
     if (blockIdx.x == 0 && threadIdx.x < top_k && routes[r * top_k + threadIdx.x] >= experts) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
     if (g >= groups) return;
-    const float v = load_activation<KIND>(x + static_cast<size_t>(r) * hidden * (KIND == 0 ? 4U : 2U), g * 32U + j);
-    const float amax = max32(__builtin_fabsf(v));
-    const bool tiny = amax > 0.0F && amax < 0x1p-119F;
-    const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
-    const int code = a8_code(v, delta, tiny);
-    const int sum = sum32_i(code);
+    // the probe contract's quantiser ("g32-sym127-zero1-finite-noflush", src/moe_q4k_a8_contract.cpp:67-91): delta = amax / 127
+    // with no tiny-group rule; a non-finite value is flagged and taken as 0, a delta that underflows to 0 is flagged and taken as 1
+    float v = load_activation<KIND>(x + static_cast<size_t>(r) * hidden * (KIND == 0 ? 4U : 2U), g * 32U + j);
     const int bad = or32_i(finite_f(v) ? 0 : 1);
+    if (!finite_f(v)) v = 0.0F;
+    const float amax = max32(__builtin_fabsf(v));
+    float delta = amax == 0.0F ? 1.0F : amax / 127.0F;
+    const bool underflow = !(delta > 0.0F) || !finite_f(delta);
+    if (underflow) delta = 1.0F;
+    const int code = a8_code(v, delta, false);
+    const int sum = sum32_i(code);
     codes[static_cast<size_t>(r) * hidden + g * 32U + j] = static_cast<int8_t>(code);
     if (j == 0) {
         deltas[static_cast<size_t>(r) * groups + g] = delta;
         sums[static_cast<size_t>(r) * groups + g] = sum;
         if (bad) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
+        if (underflow) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_DELTA));
     }
 }
 
@@ -191,10 +196,9 @@ __global__ __launch_bounds__(1024) void a8_slot_merge_kernel(SlotMergeArgs t) {
     }
 }
 
+// the bundle of the single-row entry points: no plan, no job word of its own, R contiguous single-row extents per view
 inline RowsK a8_rows(const mi355_moe_weights& w) {
-    RowsK r{};
-    r.slot_stride = w.ffn;
-    return r;
+    return rows_k(mi355_moe_rows{}, w);
 }
 
 }  // namespace strix950
@@ -231,9 +235,11 @@ int32_t mi355_a8_enqueue_probe(const mi355_a8_request* q, const mi355_a8_binding
     // projection only: output[(assignment * 2 + which) * rows + row], no plan (item i = assignment i), no image of h
     RowsK r = a8_rows(w);
     r.routes = reinterpret_cast<const uint32_t*>(b->routes.address);
-    r.codes = reinterpret_cast<int8_t*>(b->codes.address); r.deltas = reinterpret_cast<float*>(b->deltas.address); r.sums = reinterpret_cast<int32_t*>(b->sums.address);
+    r.in = dense_image(reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), s.hidden);
     r.status = status; r.job_status = status;
+    r.status_rs = 0;                // one shared status word
     r.gate_out = reinterpret_cast<float*>(b->output.address); r.up_out = r.gate_out + s.rows; r.slot_stride = 2ULL * s.rows;
+    r.inter_rs = 4ULL * s.top_k * r.slot_stride;
     const uint32_t items = R * s.top_k;
     if (q->gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else if (items <= 16U) project_quad_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
@@ -267,9 +273,10 @@ int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bind
     w.swiglu_limit = INFINITY;
     RowsK r = a8_rows(w);
     r.routes = reinterpret_cast<const uint32_t*>(b->routes.address);
-    r.down_codes = reinterpret_cast<int8_t*>(b->codes.address); r.down_deltas = reinterpret_cast<float*>(b->deltas.address);
-    r.down_sums = reinterpret_cast<int32_t*>(b->sums.address); r.rawdots = reinterpret_cast<float*>(b->rawdots.address);
+    r.h = dense_image(reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), s.intermediate);
+    r.rawdots = reinterpret_cast<float*>(b->rawdots.address);
     r.status = reinterpret_cast<uint32_t*>(b->status.address);
+    r.status_rs = 0;
     r.job_status = r.status;        // a non-finite projection recorded by the producer (bit 8) skips the rows, as in the layer entries
     const uint32_t items = logical_rows * s.top_k;
     if (q->weight_type != MI355_TYPE_Q4_K) {

@@ -75,10 +75,16 @@ __global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, R
         const uint32_t na = end - c0 < kDownGroupsAssignments ? end - c0 : kDownGroupsAssignments;
         uint32_t src[kDownGroupsAssignments];
         float chain[kDownGroupsAssignments];
+        const int8_t* h_codes[kDownGroupsAssignments];
+        const float* h_deltas[kDownGroupsAssignments];
+        const int32_t* h_sums[kDownGroupsAssignments];
 #pragma unroll
         for (uint32_t a = 0; a < kDownGroupsAssignments; ++a) {
             src[a] = ordered(r, order_at, c0 + (a < na ? a : na - 1U));
             chain[a] = 0.0F;
+            h_codes[a] = r.h.codes_of(src[a]);
+            h_deltas[a] = r.h.deltas_of(src[a]);
+            h_sums[a] = r.h.sums_of(src[a]);
         }
 #pragma unroll 2
         for (uint32_t c = 0; c < per_chain; ++c) {
@@ -89,7 +95,7 @@ __global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, R
 #pragma unroll
             for (uint32_t a = 0; a < kDownGroupsAssignments; ++a) {
                 if (a < na) {                                     // uniform over the workgroup
-                    const u32x4_g* codes = reinterpret_cast<const u32x4_g*>(r.down_codes + static_cast<size_t>(src[a]) * w.ffn + 32U * g);
+                    const u32x4_g* codes = reinterpret_cast<const u32x4_g*>(h_codes[a] + 32U * g);
                     const u32x4_g c_lo = codes[0], c_hi = codes[1];
                     const uint32_t cw[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
                     int dot = 0;
@@ -97,8 +103,8 @@ __global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, R
                     for (int i = 0; i < 8; ++i) dot = __builtin_amdgcn_sdot4(static_cast<int>(q[i]), static_cast<int>(cw[i]), dot, false);
                     const float first = d * static_cast<float>(dot);
                     float combined = first;
-                    if (FMT == 1) combined = first + (m * static_cast<float>(r.down_sums[static_cast<size_t>(src[a]) * groups + g]));
-                    chain[a] = chain[a] + (r.down_deltas[static_cast<size_t>(src[a]) * groups + g] * combined);
+                    if (FMT == 1) combined = first + (m * static_cast<float>(h_sums[a][g]));
+                    chain[a] = chain[a] + (h_deltas[a][g] * combined);
                 }
             }
         }
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(256) void down_groups_kernel(mi355_moe_weights w, R
                 float v = chain[a];
                 v = v + xor1_f(v);          // chain0 + chain1 | chain2 + chain3
                 v = v + xor2_f(v);          // (chain0 + chain1) + (chain2 + chain3)
-                if (j == 0) r.rawdots[static_cast<size_t>(src[a]) * w.hidden + o] = v;
+                if (j == 0) r.rawdots_of(src[a], w.hidden)[o] = v;
             }
         }
     }

@@ -67,13 +67,13 @@ struct PairSource {
 #pragma unroll
         for (uint32_t a = 0; a < B; ++a) {
             const uint32_t row = a < nacts ? a : 0U;
-            cp[a] = reinterpret_cast<const uint8_t*>(img.codes) + static_cast<size_t>(row) * img.width + 16U * lane;
+            cp[a] = reinterpret_cast<const uint8_t*>(img.codes_of(row)) + 16U * lane;
         }
 #pragma unroll
         for (uint32_t i = 0; i < SC; ++i) {
             const uint32_t a = 8U * i + (lane >> 3), row = a < nacts ? a : 0U;
-            dp[i] = reinterpret_cast<const uint8_t*>(img.deltas + static_cast<size_t>(row) * groups) + 16U * (lane & 7U);
-            sp[i] = reinterpret_cast<const uint8_t*>(img.sums + static_cast<size_t>(row) * groups) + 16U * (lane & 7U);
+            dp[i] = reinterpret_cast<const uint8_t*>(img.deltas_of(row)) + 16U * (lane & 7U);
+            sp[i] = reinterpret_cast<const uint8_t*>(img.sums_of(row)) + 16U * (lane & 7U);
         }
     }
     // slot: [weights WC KiB][codes B KiB][deltas SC KiB][sums SC KiB]

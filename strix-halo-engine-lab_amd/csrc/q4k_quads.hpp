@@ -97,8 +97,8 @@ __device__ __forceinline__ void quad_block_compute(const lds_u8* slot, uint32_t 
 template <int DEPTH>
 __device__ __forceinline__ float sweep_quads(lds_u8* const (&slots)[DEPTH], QuadSource source, uint32_t blocks, const A8Image& img, uint32_t row) {
     const uint32_t lane = threadIdx.x & 63U, groups = img.width / 32U;
-    const float* deltas = img.deltas + static_cast<size_t>(row) * groups;
-    const int32_t* sums = img.sums + static_cast<size_t>(row) * groups;
+    const float* deltas = img.deltas_of(row);
+    const int32_t* sums = img.sums_of(row);
     float acc = 0.0F, vd = 0.0F, vf = 0.0F;
 #pragma unroll
     for (int s = 0; s < DEPTH - 1; ++s)

@@ -38,30 +38,113 @@ typedef __attribute__((address_space(3))) uint8_t lds_u8;      // ring slots are
 template <int NA> constexpr uint32_t stage_copies() { return kStagePieces + (NA + 3) / 4; }   // copy instructions per stage
 
 
-// The kernels' view of the per-row buffers: the public bundle plus what only some entry points vary.
+// The A8 image of a set of rows: int8 codes [width] and, per group of 32, an fp32 delta and the int32 sum of the codes.
+// Image i lives at codes + (i / per_row) * codes_rs + (i % per_row) * width bytes (deltas / sums likewise, width / 32 words per
+// image): per_row = 1 is one image per logical row (the input rows; every dense buffer, whose stride is then the image
+// size), per_row = top_k the images of h inside strided per-row views (one per slot). With `table` set, image i is where
+// table[i] points (the host executor's RowA8, src/cpu/core/routed_expert.hpp:41-45).
+struct A8Image {
+    const int8_t* codes;
+    const float* deltas;
+    const int32_t* sums;
+    uint32_t width;
+    uint32_t per_row;
+    uint64_t codes_rs, deltas_rs, sums_rs;        // bytes between logical rows
+    const mi355_row_a8* table;
+    __device__ __forceinline__ void split(uint32_t i, uint32_t& q, uint32_t& s) const {
+        if (per_row == 1U) { q = i; s = 0; } else { q = i / per_row; s = i - q * per_row; }
+    }
+    __device__ __forceinline__ const int8_t* codes_of(uint32_t i) const {
+        if (table) return table[i].codes;
+        uint32_t q, s;
+        split(i, q, s);
+        return reinterpret_cast<const int8_t*>(reinterpret_cast<const uint8_t*>(codes) + q * codes_rs + static_cast<size_t>(s) * width);
+    }
+    __device__ __forceinline__ const float* deltas_of(uint32_t i) const {
+        if (table) return table[i].deltas;
+        uint32_t q, s;
+        split(i, q, s);
+        return reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(deltas) + q * deltas_rs) + static_cast<size_t>(s) * (width / 32U);
+    }
+    __device__ __forceinline__ const int32_t* sums_of(uint32_t i) const {
+        if (table) return table[i].sums;
+        uint32_t q, s;
+        split(i, q, s);
+        return reinterpret_cast<const int32_t*>(reinterpret_cast<const uint8_t*>(sums) + q * sums_rs) + static_cast<size_t>(s) * (width / 32U);
+    }
+};
+// one image per row, rows back to back
+__host__ __device__ inline A8Image dense_image(const int8_t* codes, const float* deltas, const int32_t* sums, uint32_t width) {
+    return A8Image{codes, deltas, sums, width, 1U, width, width / 8U, width / 8U, nullptr};
+}
+
+// The kernels' view of the per-row buffers: the public bundle plus what only some entry points vary. An assignment index
+// i (row-major: i = row * top_k + slot, or, in the job form, the position in the job's assignment list) resolves to
+// (row, slot) by place(); the per-assignment fields then sit at base + row * <field>_rs + slot * <slot extent> bytes. The
+// dense bundles give <field>_rs = top_k * <slot extent>, so every address is the dense one.
 struct RowsK : mi355_moe_rows {
-    uint64_t slot_stride;     // floats between the rows of consecutive assignments in gate_out / up_out / h_out (dense: ffn)
+    uint64_t slot_stride;     // floats between the slots of a row in gate_out / up_out / h_out (dense: ffn)
+    A8Image in, h;            // the images of the input rows and of h
+    uint64_t routes_rs, route_weights_rs, status_rs, inter_rs, rawdots_rs, base_rs;      // bytes between logical rows
+    const mi355_expert_assignment* assignments;      // job form (src/cpu/core/routed_expert.hpp:47-49): item i = assignments[i]
+    uint32_t top_k;
+    uint32_t nonfinite_bit;   // what a non-finite gate / up / h value ORs into its row's status (8; the host executor's job: 1)
+
+    __device__ __forceinline__ void place(uint32_t i, uint32_t& row, uint32_t& slot) const {
+        if (assignments) { row = assignments[i].row; slot = assignments[i].slot; }
+        else { row = i / top_k; slot = i - row * top_k; }
+    }
+    __device__ __forceinline__ uint32_t row_of(uint32_t i) const { return assignments ? assignments[i].row : i / top_k; }
+    __device__ __forceinline__ const uint32_t* routes_of(uint32_t row) const {
+        return reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(routes) + row * routes_rs);
+    }
+    __device__ __forceinline__ const float* route_weights_of(uint32_t row) const {
+        return reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(route_weights) + row * route_weights_rs);
+    }
+    __device__ __forceinline__ uint32_t* status_of(uint32_t row) const {
+        return reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(status) + row * status_rs);
+    }
+    __device__ __forceinline__ const float* base_of(uint32_t row) const {
+        return reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(base) + row * base_rs);
+    }
+    // the `hidden` unweighted outputs of assignment i
+    __device__ __forceinline__ float* rawdots_of(uint32_t i, uint32_t hidden) const {
+        uint32_t row, slot;
+        place(i, row, slot);
+        return reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(rawdots) + row * rawdots_rs) + static_cast<size_t>(slot) * hidden;
+    }
+    // element 0 of assignment i in one of gate_out / up_out / h_out (null stays null)
+    __device__ __forceinline__ float* inter_of(float* field, uint32_t i) const {
+        if (!field) return nullptr;
+        uint32_t row, slot;
+        place(i, row, slot);
+        return reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(field) + row * inter_rs) + slot * slot_stride;
+    }
+    // the writable image of h of assignment i
+    __device__ __forceinline__ int8_t* h_codes_of(uint32_t i) const { return const_cast<int8_t*>(h.codes_of(i)); }
+    __device__ __forceinline__ float* h_deltas_of(uint32_t i) const { return const_cast<float*>(h.deltas_of(i)); }
+    __device__ __forceinline__ int32_t* h_sums_of(uint32_t i) const { return const_cast<int32_t*>(h.sums_of(i)); }
 };
 // One work item of an expert launch: assignments [begin, end) of the plan order belong to expert e. Without a plan
-// (plan == nullptr) item i is assignment i alone, its expert read from the routes: the single-row forms of the reference
-// entry points (include/strix/hip_moe_q4k_a8_probe.hpp:12, include/strix/hip_moe_a8_down.hpp:11-30) bring no plan view.
+// (plan == nullptr) item i is assignment i alone, its expert read from the routes (or from the job's list): the single-row
+// forms of the reference entry points (include/strix/hip_moe_q4k_a8_probe.hpp:12, include/strix/hip_moe_a8_down.hpp:11-30) and
+// the host executor's Job bring no plan view.
 struct WorkItem { uint32_t e, begin, end; };
 __device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const RowsK& r, uint32_t items_at, uint32_t index) {
     if (r.plan) {
         const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * index);
         return {item.x, item.y, item.z};
     }
-    const uint32_t e = r.routes[index];
+    uint32_t e;
+    if (r.assignments) e = r.assignments[index].expert;
+    else {
+        uint32_t row, slot;
+        r.place(index, row, slot);
+        e = r.routes_of(row)[slot];
+    }
     return {e, index, e < w.experts ? index + 1U : index};      // an invalid route has no item (its row is flagged)
 }
 __device__ __forceinline__ uint32_t ordered(const RowsK& r, uint32_t order_at, uint32_t i) { return r.plan ? r.plan[order_at + i] : i; }
-
-struct A8Image {                             // device A8 image: codes [rows][width], deltas / sums [rows][width / 32]
-    const int8_t* codes;
-    const float* deltas;
-    const int32_t* sums;
-    uint32_t width;
-};
 
 // Per-lane source pointers of the nine pieces the lane copies in every stage. row_ptr(r) = first byte of row r (0..63).
 struct StageSource {
@@ -78,11 +161,11 @@ struct StageSource {
     }
     // lane_row[h] = index (into the A8 image) of activation row 4 h + lane / 16, any valid row where that is >= NA
     template <int NA>
-    __device__ __forceinline__ void init_act(const int8_t* codes, uint32_t width, const uint32_t (&lane_row)[(NA + 3) / 4]) {
+    __device__ __forceinline__ void init_act(const A8Image& img, const uint32_t (&lane_row)[(NA + 3) / 4]) {
         const uint32_t lane = threadIdx.x & 63U;
 #pragma unroll
         for (int h = 0; h < (NA + 3) / 4; ++h)
-            act_piece[h] = reinterpret_cast<const uint8_t*>(codes) + static_cast<size_t>(lane_row[h]) * width + 16U * (lane & 15U);
+            act_piece[h] = reinterpret_cast<const uint8_t*>(img.codes_of(lane_row[h])) + 16U * (lane & 15U);
     }
     // start the copy of the next super-block of all 64 rows (and of the activation rows' codes) into one ring slot,
     // then step to the block after it
@@ -137,22 +220,21 @@ __device__ __forceinline__ void q4k_factors(const u32x4& hd, uint32_t& sc, uint3
 // Uniform view of the NA activation rows of one sweep (row bases, wave-uniform).
 template <int NA>
 struct ActRows {
-    const int8_t* codes;                       // image base
-    uint32_t width;
+    A8Image img;
     uint32_t lane_row[(NA + 3) / 4];           // per lane: image row of activation row 4 h + lane / 16 (see StageSource::init_act)
     const float* deltas[NA];
     const int32_t* sums[NA];
     uint32_t groups;                           // per activation row
     // row[a]: image row of activation row a (any lane's value is taken); lane_rows: the per-lane rows for the code copies
     __device__ __forceinline__ ActRows(const A8Image& img, const uint32_t (&row)[NA], const uint32_t (&lane_rows)[(NA + 3) / 4])
-        : codes(img.codes), width(img.width), groups(img.width / 32U) {
+        : img(img), groups(img.width / 32U) {
 #pragma unroll
         for (int h = 0; h < (NA + 3) / 4; ++h) lane_row[h] = lane_rows[h];
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             const uint32_t r = __builtin_amdgcn_readfirstlane(row[a]);
-            deltas[a] = img.deltas + static_cast<size_t>(r) * groups;
-            sums[a] = img.sums + static_cast<size_t>(r) * groups;
+            deltas[a] = img.deltas_of(r);
+            sums[a] = img.sums_of(r);
         }
     }
 };
@@ -229,7 +311,7 @@ __device__ __forceinline__ void sweep_rows(lds_u8* const (&slots)[DEPTH], StageS
     float vd[NA], vf[NA];
 #pragma unroll
     for (int a = 0; a < NA; ++a) vd[a] = vf[a] = 0.0F;
-    source.init_act<NA>(act.codes, act.width, act.lane_row);
+    source.init_act<NA>(act.img, act.lane_row);
 #pragma unroll
     for (int s = 0; s < DEPTH - 1; ++s)
         if (static_cast<uint32_t>(s) < blocks) source.start<NA, NARROW>(slots[s]);

@@ -17,9 +17,9 @@ constexpr uint32_t kQ5kBlock = 176;
 // The value of one weight row against activation row `row` of `img`, for the lane's pair p; every lane of a quad returns it.
 __device__ __forceinline__ float sweep_q5k_row(const uint8_t* wrow, uint32_t blocks, const A8Image& img, uint32_t row, uint32_t p) {
     const uint32_t groups = img.width / 32U;
-    const u32x4* codes = reinterpret_cast<const u32x4*>(img.codes + static_cast<size_t>(row) * img.width + 64U * p);
-    const float2* deltas = reinterpret_cast<const float2*>(img.deltas + static_cast<size_t>(row) * groups + 2U * p);
-    const int2* sums = reinterpret_cast<const int2*>(img.sums + static_cast<size_t>(row) * groups + 2U * p);
+    const u32x4* codes = reinterpret_cast<const u32x4*>(img.codes_of(row) + 64U * p);
+    const float2* deltas = reinterpret_cast<const float2*>(img.deltas_of(row) + 2U * p);
+    const int2* sums = reinterpret_cast<const int2*>(img.sums_of(row) + 2U * p);
     float acc = 0.0F;
 #pragma unroll 4
     for (uint32_t b = 0; b < blocks; ++b) {     // four blocks of loads in flight: 52 -> 35 us at hidden 2048, 64 assignments

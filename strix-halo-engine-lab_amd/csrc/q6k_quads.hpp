@@ -46,10 +46,14 @@ __global__ __launch_bounds__(256) void down_q6k_kernel(mi355_moe_weights w, Rows
         const uint32_t na = end - c0 < NA ? end - c0 : NA;
         uint32_t src[NA];
         float acc[NA];
+        const int8_t* h_codes[NA];
+        const float* h_deltas[NA];
 #pragma unroll
         for (uint32_t a = 0; a < NA; ++a) {
             src[a] = ordered(r, order_at, c0 + (a < na ? a : na - 1U));
             acc[a] = 0.0F;
+            h_codes[a] = r.h.codes_of(src[a]);
+            h_deltas[a] = r.h.deltas_of(src[a]);
         }
 #pragma unroll 2
         for (uint32_t b = 0; b < blocks; ++b) {
@@ -76,8 +80,8 @@ __global__ __launch_bounds__(256) void down_q6k_kernel(mi355_moe_weights w, Rows
 #pragma unroll
             for (uint32_t a = 0; a < NA; ++a) {
                 if (a < na) {                                     // uniform over the workgroup
-                    const u32x4_g* codes = reinterpret_cast<const u32x4_g*>(r.down_codes + static_cast<size_t>(src[a]) * w.ffn + 256U * b + 64U * p);
-                    const float2 delta = *reinterpret_cast<const float2*>(r.down_deltas + static_cast<size_t>(src[a]) * groups + 8U * b + 2U * p);
+                    const u32x4_g* codes = reinterpret_cast<const u32x4_g*>(h_codes[a] + 256U * b + 64U * p);
+                    const float2 delta = *reinterpret_cast<const float2*>(h_deltas[a] + 8U * b + 2U * p);
                     float term[2];
 #pragma unroll
                     for (uint32_t k = 0; k < 2U; ++k) {
@@ -102,7 +106,7 @@ __global__ __launch_bounds__(256) void down_q6k_kernel(mi355_moe_weights w, Rows
                 float v = acc[a];
                 v = v + xor1_f(v);          // acc0 + acc1 | acc2 + acc3
                 v = v + xor2_f(v);          // (acc0 + acc1) + (acc2 + acc3)
-                if (p == 0) r.rawdots[static_cast<size_t>(src[a]) * w.hidden + o] = v;
+                if (p == 0) r.rawdots_of(src[a], w.hidden)[o] = v;
             }
         }
     }

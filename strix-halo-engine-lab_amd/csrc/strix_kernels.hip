@@ -363,10 +363,23 @@ __global__ __launch_bounds__(64) void route_select_kernel(RouteArgs a) {
 // ======================================================================================================== expert plan
 // (layout of the plan words: see the router section above)
 
+// The routes of a batch as the plan kernels read them: assignment a = row a / top_k, slot a % top_k, rows `rs` bytes apart.
+struct RoutesView {
+    const uint32_t* base;
+    uint64_t rs;
+    uint32_t top_k;
+    __device__ __forceinline__ uint32_t at(uint32_t a) const {
+        if (rs == 4ULL * top_k) return base[a];
+        const uint32_t row = a / top_k;
+        return reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(base) + row * rs)[a - row * top_k];
+    }
+};
+inline RoutesView dense_routes(const uint32_t* routes, uint32_t top_k) { return RoutesView{routes, 4ULL * top_k, top_k}; }
+
 // Stable order of a large batch: one 16-wave workgroup per expert. Every wave owns a contiguous sixteenth of the assignments:
 // it first counts its own assignments of the expert (ballot + population count, 64 at a time), the counts of the waves before
 // it give its first position, and a second walk places them in index order (the offsets are already in the plan).
-__global__ __launch_bounds__(1024) void plan_order_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
+__global__ __launch_bounds__(1024) void plan_order_kernel(RoutesView routes, uint32_t experts, uint32_t assignments, uint32_t* plan) {
     __shared__ uint32_t wave_count[16];
     const uint32_t e = blockIdx.x, lane = threadIdx.x & 63U, wave = threadIdx.x >> 6;
     const uint32_t first = plan[kPlanOffsetsAt + e], end = plan[kPlanOffsetsAt + e + 1];
@@ -376,7 +389,7 @@ __global__ __launch_bounds__(1024) void plan_order_kernel(const uint32_t* routes
     uint32_t mine_total = 0;
     for (uint32_t a0 = lo; a0 < hi; a0 += 64U) {
         const uint32_t a = a0 + lane;
-        mine_total += static_cast<uint32_t>(__popcll(__ballot(a < hi && routes[a] == e)));
+        mine_total += static_cast<uint32_t>(__popcll(__ballot(a < hi && routes.at(a) == e)));
     }
     if (lane == 0) wave_count[wave] = mine_total;
     __syncthreads();
@@ -386,7 +399,7 @@ __global__ __launch_bounds__(1024) void plan_order_kernel(const uint32_t* routes
     uint32_t* order = plan + plan_order_at(experts);
     for (uint32_t a0 = lo; a0 < hi && at < stop; a0 += 64U) {
         const uint32_t a = a0 + lane;
-        const bool mine = a < hi && routes[a] == e;
+        const bool mine = a < hi && routes.at(a) == e;
         const uint64_t votes = __ballot(mine);
         if (mine) order[at + __popcll(votes & ((1ULL << lane) - 1ULL))] = a;
         at += static_cast<uint32_t>(__popcll(votes));
@@ -417,7 +430,7 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* w
 
 // The expert plan in one workgroup: thread e owns expert e (counts by shared-memory atomics, three prefix sums for the
 // offsets, the item numbers and the touched list, then its own items and - for a small batch - its own stretch of the order).
-__global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t split,
+__global__ __launch_bounds__(1024) void plan_kernel(RoutesView routes, uint32_t experts, uint32_t assignments, uint32_t split,
                                                     uint32_t item_bound, uint32_t fill_order, uint32_t* plan) {
     __shared__ uint32_t count[kRouteMaxExperts];
     __shared__ uint32_t wave_totals[3][16];
@@ -427,7 +440,7 @@ __global__ __launch_bounds__(1024) void plan_kernel(const uint32_t* routes, uint
     count[tid] = 0;
     __syncthreads();
     for (uint32_t a = tid; a < assignments; a += 1024U) {
-        const uint32_t e = routes[a];
+        const uint32_t e = routes.at(a);
         if (fill_order) small_routes[a] = e;
         if (e < experts) atomicAdd(&count[e], 1U);
     }
@@ -493,19 +506,19 @@ __global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* rout
 template <int NA, int DEPTH>
 __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
                                               const RowsK& r, uint32_t grp, uint32_t order_at, uint32_t c0) {
-    const uint32_t lane = threadIdx.x & 63U, o = lane & 31U, groups = w.ffn / 32U;
+    const uint32_t lane = threadIdx.x & 63U, o = lane & 31U;
     uint32_t sidx[NA], src[NA], lane_rows[(NA + 3) / 4];
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
         sidx[a] = __builtin_amdgcn_readfirstlane(ordered(r, order_at, c0 + a));
-        src[a] = sidx[a] / w.top_k;
+        src[a] = r.row_of(sidx[a]);
     }
 #pragma unroll
     for (int h = 0; h < (NA + 3) / 4; ++h) {
         const uint32_t a = 4U * h + (lane >> 4);
-        lane_rows[h] = ordered(r, order_at, c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)) / w.top_k;
+        lane_rows[h] = r.row_of(ordered(r, order_at, c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)));
     }
-    const ActRows<NA> act(A8Image{r.codes, r.deltas, r.sums, w.hidden}, src, lane_rows);
+    const ActRows<NA> act(r.in, src, lane_rows);
     float value[NA];
     sweep_rows<NA, DEPTH>(slots, source, w.hidden / 256U, act, value);
 #pragma unroll
@@ -515,17 +528,16 @@ __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], con
         float gc = g, uc = u;
         swiglu_clamp(gc, uc, w.swiglu_limit);
         const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
-        const size_t at = static_cast<size_t>(sidx[a]) * w.ffn + grp * 32U + o;
-        const size_t at_out = static_cast<size_t>(sidx[a]) * r.slot_stride + grp * 32U + o;
+        const uint32_t at_out = grp * 32U + o;
         if (lane < 32U) {
-            if (r.gate_out) r.gate_out[at_out] = g;
-            if (r.up_out) r.up_out[at_out] = u;
-            if (r.h_out) r.h_out[at_out] = h;
+            if (r.gate_out) r.inter_of(r.gate_out, sidx[a])[at_out] = g;
+            if (r.up_out) r.inter_of(r.up_out, sidx[a])[at_out] = u;
+            if (r.h_out) r.inter_of(r.h_out, sidx[a])[at_out] = h;
         }
-        if (!r.down_codes) continue;                      // projection only (the probe form): no A8 image of h
+        if (!r.h.codes) continue;                         // projection only (the probe form): no A8 image of h
         if (or32_i((finite_f(g) && finite_f(u) && finite_f(h)) ? 0 : 1)) {
             if (lane == 0) {
-                atomicOr(&r.status[sidx[a] / w.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                atomicOr(r.status_of(src[a]), r.nonfinite_bit);
                 atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
             }
         } else {
@@ -534,10 +546,10 @@ __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], con
             const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
             const int code = a8_code(h, dl, tiny);
             const int sum = sum32_i(code);
-            if (lane < 32U) r.down_codes[at] = static_cast<int8_t>(code);
+            if (lane < 32U) r.h_codes_of(sidx[a])[at_out] = static_cast<int8_t>(code);
             if (lane == 0) {
-                r.down_deltas[static_cast<size_t>(sidx[a]) * groups + grp] = dl;
-                r.down_sums[static_cast<size_t>(sidx[a]) * groups + grp] = sum;
+                r.h_deltas_of(sidx[a])[grp] = dl;
+                r.h_sums_of(sidx[a])[grp] = sum;
             }
         }
     }
@@ -605,12 +617,12 @@ __device__ __forceinline__ void down_chunk(lds_u8* const (&slots)[DEPTH], const 
         const uint32_t a = 4U * h + ((threadIdx.x & 63U) >> 4);
         lane_rows[h] = ordered(r, order_at, c0 + (a < static_cast<uint32_t>(NA) ? a : 0U));
     }
-    const ActRows<NA> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src, lane_rows);
+    const ActRows<NA> act(r.h, src, lane_rows);
     float value[NA];
     sweep_rows<NA, DEPTH>(slots, source, w.ffn / 256U, act, value);
     const uint32_t o = blockIdx.x * 64U + (threadIdx.x & 63U);
 #pragma unroll
-    for (int a = 0; a < NA; ++a) r.rawdots[static_cast<size_t>(src[a]) * w.hidden + o] = value[a];
+    for (int a = 0; a < NA; ++a) r.rawdots_of(src[a], w.hidden)[o] = value[a];
 }
 
 template <int NBMAX, int DEPTH>
@@ -670,38 +682,37 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
     const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
     const uint32_t e = item.e, begin = item.begin, end = item.end;
     if (begin == end) return;
-    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x, groups = w.ffn / 32U;
-    const uint32_t sidx = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), begin)), row = sidx / w.top_k;
+    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x;
+    const uint32_t sidx = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), begin)), row = r.row_of(sidx);
     const uint32_t f0 = grp * 32U + 8U * wave;
     const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(f0) * w.gate_row_stride;
     const uint8_t* gate = w.gate + base;
     const uint8_t* up = w.up + base;
     const size_t stride = w.gate_row_stride;
     QuadSource source;
-    source.init([&](uint32_t q) { return q < 8U ? gate + q * stride : up + (q - 8U) * stride; }, r.codes + static_cast<size_t>(row) * w.hidden);
+    source.init([&](uint32_t q) { return q < 8U ? gate + q * stride : up + (q - 8U) * stride; }, r.in.codes_of(row));
     lds_u8* const (&sl)[DEPTH] = slots;
-    const float value = sweep_quads<DEPTH>(sl, source, w.hidden / 256U, A8Image{r.codes, r.deltas, r.sums, w.hidden}, row);
+    const float value = sweep_quads<DEPTH>(sl, source, w.hidden / 256U, r.in, row);
     const float other = __shfl_xor(value, 32);
     const bool mine = lane < 32U && p == 0;                   // the lane that publishes feature f0 + rr
     const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
     float gc = g, uc = u;
     swiglu_clamp(gc, uc, w.swiglu_limit);
     const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
-    const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
-    const size_t at_out = static_cast<size_t>(sidx) * r.slot_stride + f0 + rr;
+    const uint32_t at_out = f0 + rr;
     if (mine) {
-        if (r.gate_out) r.gate_out[at_out] = g;
-        if (r.up_out) r.up_out[at_out] = u;
-        if (r.h_out) r.h_out[at_out] = h;
+        if (r.gate_out) r.inter_of(r.gate_out, sidx)[at_out] = g;
+        if (r.up_out) r.inter_of(r.up_out, sidx)[at_out] = u;
+        if (r.h_out) r.inter_of(r.h_out, sidx)[at_out] = h;
     }
-    if (!r.down_codes) return;                            // projection only (the probe form): no A8 image of h
+    if (!r.h.codes) return;                               // projection only (the probe form): no A8 image of h
     const int bad = or32_i((mine && !(finite_f(g) && finite_f(u) && finite_f(h))) ? 1 : 0);
     const float amax_wave = max32(mine ? __builtin_fabsf(h) : 0.0F);
     if (lane == 0) { wg_amax[wave] = amax_wave; wg_bad[wave] = bad; }
     __syncthreads();
     if (wg_bad[0] | wg_bad[1] | wg_bad[2] | wg_bad[3]) {
         if (threadIdx.x == 0) {
-            atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            atomicOr(r.status_of(row), r.nonfinite_bit);
             atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
         }
         return;
@@ -712,11 +723,11 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
     const int code = a8_code(h, dl, tiny);
     const int sum_wave = sum32_i(mine ? code : 0);
     if (lane == 0) wg_sum[wave] = sum_wave;
-    if (mine) r.down_codes[at] = static_cast<int8_t>(code);
+    if (mine) r.h_codes_of(sidx)[at_out] = static_cast<int8_t>(code);
     __syncthreads();
     if (threadIdx.x == 0) {
-        r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
-        r.down_sums[static_cast<size_t>(sidx) * groups + grp] = wg_sum[0] + wg_sum[1] + wg_sum[2] + wg_sum[3];
+        r.h_deltas_of(sidx)[grp] = dl;
+        r.h_sums_of(sidx)[grp] = wg_sum[0] + wg_sum[1] + wg_sum[2] + wg_sum[3];
     }
 }
 
@@ -726,27 +737,26 @@ __global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, R
     __shared__ int wg_sum[4], wg_bad[4];
     const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
     const uint32_t e = item.e, begin = item.begin, end = item.end;
-    const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x, groups = w.ffn / 32U;
+    const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x;
     const uint32_t f0 = grp * 32U + 8U * wave;
     const uint8_t* wrow = (lane < 32U ? w.gate : w.up) + static_cast<size_t>(e) * w.gate_expert_stride +
                           static_cast<size_t>(f0 + (rr & 7U)) * w.gate_row_stride;
     const bool mine = lane < 32U && p == 0;                   // the lane that publishes feature f0 + rr
     for (uint32_t a = begin; a < end; ++a) {
-        const uint32_t sidx = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), a)), row = sidx / w.top_k;
-        const float value = sweep_q5k_row(wrow, w.hidden / 256U, A8Image{r.codes, r.deltas, r.sums, w.hidden}, row, p);
+        const uint32_t sidx = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), a)), row = r.row_of(sidx);
+        const float value = sweep_q5k_row(wrow, w.hidden / 256U, r.in, row, p);
         const float other = __shfl_xor(value, 32);
         const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
         float gc = g, uc = u;
         swiglu_clamp(gc, uc, w.swiglu_limit);
         const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
-        const size_t at = static_cast<size_t>(sidx) * w.ffn + f0 + rr;
-        const size_t at_out = static_cast<size_t>(sidx) * r.slot_stride + f0 + rr;
+        const uint32_t at_out = f0 + rr;
         if (mine) {
-            if (r.gate_out) r.gate_out[at_out] = g;
-            if (r.up_out) r.up_out[at_out] = u;
-            if (r.h_out) r.h_out[at_out] = h;
+            if (r.gate_out) r.inter_of(r.gate_out, sidx)[at_out] = g;
+            if (r.up_out) r.inter_of(r.up_out, sidx)[at_out] = u;
+            if (r.h_out) r.inter_of(r.h_out, sidx)[at_out] = h;
         }
-        if (!r.down_codes) continue;                      // projection only (the probe form): no A8 image of h
+        if (!r.h.codes) continue;                         // projection only (the probe form): no A8 image of h
         const int bad = or32_i((mine && !(finite_f(g) && finite_f(u) && finite_f(h))) ? 1 : 0);
         const float amax_wave = max32(mine ? __builtin_fabsf(h) : 0.0F);
         __syncthreads();                                          // the previous assignment's reads of the shared words are done
@@ -754,7 +764,7 @@ __global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, R
         __syncthreads();
         if (wg_bad[0] | wg_bad[1] | wg_bad[2] | wg_bad[3]) {      // uniform over the workgroup
             if (threadIdx.x == 0) {
-                atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                atomicOr(r.status_of(row), r.nonfinite_bit);
                 atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
             }
             continue;
@@ -765,11 +775,11 @@ __global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, R
         const int code = a8_code(h, dl, tiny);
         const int sum_wave = sum32_i(mine ? code : 0);
         if (lane == 0) wg_sum[wave] = sum_wave;
-        if (mine) r.down_codes[at] = static_cast<int8_t>(code);
+        if (mine) r.h_codes_of(sidx)[at_out] = static_cast<int8_t>(code);
         __syncthreads();
         if (threadIdx.x == 0) {
-            r.down_deltas[static_cast<size_t>(sidx) * groups + grp] = dl;
-            r.down_sums[static_cast<size_t>(sidx) * groups + grp] = wg_sum[0] + wg_sum[1] + wg_sum[2] + wg_sum[3];
+            r.h_deltas_of(sidx)[grp] = dl;
+            r.h_sums_of(sidx)[grp] = wg_sum[0] + wg_sum[1] + wg_sum[2] + wg_sum[3];
         }
     }
 }
@@ -789,10 +799,10 @@ __global__ __launch_bounds__(256) void down_quad_kernel(mi355_moe_weights w, Row
     const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(o0) * w.down_row_stride;
     const size_t stride = w.down_row_stride;
     QuadSource source;
-    source.init([&](uint32_t q) { return rows + q * stride; }, r.down_codes + static_cast<size_t>(src) * w.ffn);
+    source.init([&](uint32_t q) { return rows + q * stride; }, r.h.codes_of(src));
     lds_u8* const (&sl)[DEPTH] = slots;
-    const float value = sweep_quads<DEPTH>(sl, source, w.ffn / 256U, A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src);
-    if (p == 0) r.rawdots[static_cast<size_t>(src) * w.hidden + o0 + rr] = value;
+    const float value = sweep_quads<DEPTH>(sl, source, w.ffn / 256U, r.h, src);
+    if (p == 0) r.rawdots_of(src, w.hidden)[o0 + rr] = value;
 }
 
 // Ordered combine of the slots of one row. Reference: include/strix/moe/combine.hpp:36-59 (fma form),
@@ -805,25 +815,25 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, RowsK r
     if (threadIdx.x == 0) {
         // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is this kernel's own), and
         // neither does any row of a job whose down phase was skipped (its unweighted outputs are not this job's)
-        row_failed = (r.status[row] & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE)) | (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION);
+        row_failed = (*r.status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE)) | (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION);
         for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
         if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
             for (uint32_t i = 1; i < w.top_k; ++i)
-                for (uint32_t j = i; j > 0 && r.routes[row * w.top_k + slot_order[j]] < r.routes[row * w.top_k + slot_order[j - 1]]; --j) {
+                for (uint32_t j = i; j > 0 && r.routes_of(row)[slot_order[j]] < r.routes_of(row)[slot_order[j - 1]]; --j) {
                     const uint32_t t = slot_order[j]; slot_order[j] = slot_order[j - 1]; slot_order[j - 1] = t;
                 }
-        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights[row * w.top_k + slot_order[k]];
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights_of(row)[slot_order[k]];
     }
     __syncthreads();
     if (o >= w.hidden || row_failed) return;
     float acc = 0.0F;
     for (uint32_t k = 0; k < w.top_k; ++k) {
-        const float e = r.rawdots[(static_cast<size_t>(row) * w.top_k + slot_order[k]) * w.hidden + o];
+        const float e = r.rawdots_of(row * w.top_k + slot_order[k], w.hidden)[o];
         if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], e, acc);
         else acc = acc + slot_weight[k] * e;
     }
-    const float y = r.base ? acc + r.base[static_cast<size_t>(row) * w.hidden + o] : acc;
-    if (!finite_f(y)) atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    const float y = r.base ? acc + r.base_of(row)[o] : acc;
+    if (!finite_f(y)) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
@@ -852,33 +862,33 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
         source.init([&](uint32_t q) { return rows + q * stride; });
         lds_u8* const slots[2] = {(lds_u8*)rings[wave][0], (lds_u8*)rings[wave][1]};
         const uint32_t src[1] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(first))}, lane_rows[1] = {first};
-        const ActRows<1> act(A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}, src, lane_rows);
+        const ActRows<1> act(r.h, src, lane_rows);
         float swept[1];
         sweep_rows<1, 2, true>(slots, source, w.ffn / 256U, act, swept);      // narrow codes copies: the slots are slot_bytes(1)
         value = swept[0];
-        r.rawdots[static_cast<size_t>(src[0]) * w.hidden + o] = value;
+        r.rawdots_of(src[0], w.hidden)[o] = value;
     }
     slot_value[wave][lane] = value;
     if (threadIdx.x == 0) {
         for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
         if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
             for (uint32_t i = 1; i < w.top_k; ++i)
-                for (uint32_t j = i; j > 0 && r.routes[row * w.top_k + slot_order[j]] < r.routes[row * w.top_k + slot_order[j - 1]]; --j) {
+                for (uint32_t j = i; j > 0 && r.routes_of(row)[slot_order[j]] < r.routes_of(row)[slot_order[j - 1]]; --j) {
                     const uint32_t t = slot_order[j]; slot_order[j] = slot_order[j - 1]; slot_order[j - 1] = t;
                 }
-        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights[row * w.top_k + slot_order[k]];
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights_of(row)[slot_order[k]];
     }
     __syncthreads();
     // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is the combine's own)
-    if (wave != 0 || (r.status[row] & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
+    if (wave != 0 || (*r.status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
     float acc = 0.0F;
     for (uint32_t k = 0; k < w.top_k; ++k) {
         const float ev = slot_value[slot_order[k]][lane];
         if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], ev, acc);
         else acc = acc + slot_weight[k] * ev;
     }
-    const float y = r.base ? acc + r.base[static_cast<size_t>(row) * w.hidden + o] : acc;
-    if (!finite_f(y)) atomicOr(&r.status[row], static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    const float y = r.base ? acc + r.base_of(row)[o] : acc;
+    if (!finite_f(y)) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
@@ -913,13 +923,39 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate,
     }
 }
 
+// A property of the current device, asked once per device ordinal (0 if the runtime cannot say).
+inline uint32_t device_property(hipDeviceAttribute_t what, std::atomic<uint32_t> (&known)[64]) {
+    int device = 0, value = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0) return 0;
+    if (device < 64) {
+        const uint32_t seen = known[device].load(std::memory_order_relaxed);
+        if (seen != 0) return seen;
+    }
+    if (hipDeviceGetAttribute(&value, what, device) != hipSuccess || value <= 0) return 0;
+    if (device < 64) known[device].store(static_cast<uint32_t>(value), std::memory_order_relaxed);
+    return static_cast<uint32_t>(value);
+}
+inline uint32_t compute_units() {
+    static std::atomic<uint32_t> known[64];
+    return device_property(hipDeviceAttributeMultiprocessorCount, known);
+}
+// LDS bytes of one compute unit
+inline uint32_t lds_per_unit() {
+    static std::atomic<uint32_t> known[64];
+    return device_property(hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, known);
+}
+// wavefronts of a launch that are all resident at once when each holds `lds_each` bytes of LDS
+inline uint64_t resident_waves(uint32_t lds_each) {
+    return static_cast<uint64_t>(compute_units()) * (lds_per_unit() / lds_each);
+}
+
 // ======================================================================================================== dispatch
 // Up to 4 (routed experts) or 8 (dense matrix) activation rows share one sweep of an expert's weights; an expert with
 // more assignments is swept again for the rest.
 // Ring depth: the deepest of 4, 3, 2 at which every workgroup of the launch is resident at once (LDS is what limits it).
 inline int ring_depth(uint64_t waves, int nbmax) {
     for (int d = 4; d > 2; --d)
-        if (waves <= 256ULL * (163840U / (static_cast<uint32_t>(d) * slot_bytes(nbmax)))) return d;
+        if (waves <= resident_waves(static_cast<uint32_t>(d) * slot_bytes(nbmax))) return d;
     return 2;
 }
 template <int NBMAX>
@@ -938,13 +974,35 @@ inline void launch_down_nb(const mi355_moe_weights& w, const RowsK& r, uint32_t 
     default: down_wave_kernel<NBMAX, 2><<<grid, 64, 0, st>>>(w, r, rows * w.top_k); break;
     }
 }
+inline RowsK rows_k(const mi355_moe_rows& r, const mi355_moe_weights& w) {
+    RowsK k{};
+    static_cast<mi355_moe_rows&>(k) = r;
+    k.slot_stride = w.ffn;
+    k.top_k = w.top_k;
+    k.nonfinite_bit = MI355_STATUS_NONFINITE_PROJECTION;
+    k.in = dense_image(r.codes, r.deltas, r.sums, w.hidden);
+    k.h = dense_image(r.down_codes, r.down_deltas, r.down_sums, w.ffn);
+    k.routes_rs = k.route_weights_rs = 4ULL * w.top_k;
+    k.status_rs = 4;
+    k.inter_rs = 4ULL * w.top_k * w.ffn;
+    k.rawdots_rs = 4ULL * w.top_k * w.hidden;
+    k.base_rs = 4ULL * w.hidden;
+    return k;
+}
+// every per-row view back to back (the layouts of mi355_moe_rows): the forms that read the fields as plain arrays apply
+inline bool dense_rows(const RowsK& k, const mi355_moe_weights& w) {
+    return !k.assignments && !k.in.table && k.in.per_row == 1U && k.in.codes_rs == w.hidden && k.in.deltas_rs == w.hidden / 8U && k.in.sums_rs == w.hidden / 8U &&
+           k.h.per_row == 1U && k.h.codes_rs == w.ffn && k.h.deltas_rs == w.ffn / 8U && k.h.sums_rs == w.ffn / 8U && k.slot_stride == w.ffn &&
+           k.inter_rs == 4ULL * w.top_k * w.ffn && k.rawdots_rs == 4ULL * w.top_k * w.hidden && k.status_rs == 4;
+}
+
 // ---- dense matrix (one expert, every row uses it): the pair-per-lane sweep ------------------------------------------
 template <int NA, int AL, int KL = 1>
 inline void launch_pairs_depth(const PairArgs& a, uint32_t matrices, hipStream_t st) {
     const dim3 grid(a.rows / pair_rows<AL, KL>(), matrices);
     const uint64_t waves = static_cast<uint64_t>(grid.x) * grid.y;
     // 4 slots when every wavefront of the launch is resident with them and the wait counter can express 3 stages ahead
-    const bool deep = 3U * pair_copies<NA, AL, KL>() <= 63U && waves <= 256ULL * (163840U / (4U * pair_slot_bytes<NA, AL, KL>()));
+    const bool deep = 3U * pair_copies<NA, AL, KL>() <= 63U && waves <= resident_waves(4U * pair_slot_bytes<NA, AL, KL>());
     if (deep) q4k_pairs_kernel<NA, AL, 4, KL><<<grid, 64, 0, st>>>(a);
     else q4k_pairs_kernel<NA, AL, 2, KL><<<grid, 64, 0, st>>>(a);
 }
@@ -969,7 +1027,7 @@ inline void launch_project_dense(const mi355_moe_weights& w, const RowsK& r, uin
     PairArgs a{};
     a.m[0] = PairMatrix{w.gate, w.gate_row_stride, r.gate_out, w.ffn};
     a.m[1] = PairMatrix{w.up, w.gate_row_stride, r.up_out, w.ffn};
-    a.rows = w.ffn; a.blocks = w.hidden / 256U; a.img = A8Image{r.codes, r.deltas, r.sums, w.hidden}; a.nacts = rows;
+    a.rows = w.ffn; a.blocks = w.hidden / 256U; a.img = r.in; a.nacts = rows;
     launch_pairs(a, 2, st);
     swiglu_quantize_kernel<<<dim3((w.ffn / 32U + 7U) / 8U, rows), 256, 0, st>>>(r.gate_out, r.up_out, w.ffn, w.exp_kind, w.swiglu_limit, r.down_codes, r.down_deltas,
                                                                                 r.down_sums, r.h_out, r.status, r.job_status);
@@ -977,12 +1035,12 @@ inline void launch_project_dense(const mi355_moe_weights& w, const RowsK& r, uin
 inline void launch_down_dense(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, hipStream_t st) {
     PairArgs a{};
     a.m[0] = PairMatrix{w.down, w.down_row_stride, r.rawdots, w.hidden};
-    a.rows = w.hidden; a.blocks = w.ffn / 256U; a.img = A8Image{r.down_codes, r.down_deltas, r.down_sums, w.ffn}; a.nacts = rows;
+    a.rows = w.hidden; a.blocks = w.ffn / 256U; a.img = r.h; a.nacts = rows;
     a.skip_flag = r.job_status; a.skip_mask = MI355_STATUS_NONFINITE_PROJECTION;
     launch_pairs(a, 1, st);
 }
 
-inline void launch_plan(const uint32_t* routes, uint32_t experts, uint32_t assignments, uint32_t split, uint32_t bound, uint32_t* plan,
+inline void launch_plan(RoutesView routes, uint32_t experts, uint32_t assignments, uint32_t split, uint32_t bound, uint32_t* plan,
                         hipStream_t st) {
     // plan_kernel's own order fill is one thread per expert walking every assignment: fine for a decode batch, far too slow
     // beyond a few hundred assignments (4096 assignments of one expert: 0.55 ms), where a wave per expert does it instead
@@ -1009,7 +1067,7 @@ inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t 
         else project_quad_kernel<2><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, r, items);
         return;
     }
-    if (dense_pairs_ok(w, rows) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
+    if (dense_pairs_ok(w, rows) && dense_rows(r, w) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
     const dim3 grid(w.ffn / 32U, umax);
     if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
     else launch_project_nb<4>(w, r, rows, grid, st);
@@ -1029,7 +1087,7 @@ inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t row
         else down_quad_kernel<2><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
         return;
     }
-    if (dense_pairs_ok(w, rows)) return launch_down_dense(w, r, rows, st);
+    if (dense_pairs_ok(w, rows) && dense_rows(r, w)) return launch_down_dense(w, r, rows, st);
     const dim3 grid(w.hidden / 64U, umax);
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
     else launch_down_nb<4>(w, r, rows, grid, st);
@@ -1049,28 +1107,6 @@ inline uint32_t plan_split(const mi355_moe_weights& w, uint32_t rows) {
 }
 inline uint32_t item_bound(const mi355_moe_weights& w, uint32_t rows) {
     return plan_item_bound(w.experts, rows * w.top_k, plan_split(w, rows));
-}
-
-// compute units of the current device (0 if the runtime cannot say); remembered per device ordinal
-inline uint32_t compute_units() {
-    static std::atomic<uint32_t> known[64];
-    int device = 0, cus = 0;
-    if (hipGetDevice(&device) != hipSuccess || device < 0) return 0;
-    if (device < 64) {
-        const uint32_t seen = known[device].load(std::memory_order_relaxed);
-        if (seen != 0) return seen;
-    }
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) return 0;
-    if (device < 64) known[device].store(static_cast<uint32_t>(cus), std::memory_order_relaxed);
-    return static_cast<uint32_t>(cus);
-}
-
-// the kernels' view of a dense row bundle
-inline RowsK rows_k(const mi355_moe_rows& r, const mi355_moe_weights& w) {
-    RowsK k{};
-    static_cast<mi355_moe_rows&>(k) = r;
-    k.slot_stride = w.ffn;
-    return k;
 }
 
 // ======================================================================================================== admission
@@ -1098,7 +1134,9 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
         return fail(MI355_E_UNSUPPORTED, cls == kPrefillClass ? "moe prefill: down weights must be Q4_K (type 12), Q5_K (type 13) or Q8_0 (type 8)"
                                                                : "moe: down weights must be Q4_K (type 12), Q8_0 (type 8), Q5_1 (type 7) or Q6_K (type 14)");
     STRIX_REQUIRE(w->hidden >= 256 && w->hidden % 256U == 0, "moe: hidden must be a positive multiple of 256");
-    STRIX_REQUIRE(w->ffn >= 256 && w->ffn % 256U == 0, "moe: ffn must be a positive multiple of 256");
+    // K-quant down rows are super-blocks of 256; the executor's block-of-32 formats need four chains of groups (src/cpu/core/routed_expert.hpp:22)
+    const uint32_t ffn_unit = (cls == kIntegerClass && (down_q8 || w->down_type == MI355_TYPE_Q5_1)) ? 128U : 256U;
+    STRIX_REQUIRE(w->ffn >= ffn_unit && w->ffn % ffn_unit == 0, "moe: ffn must be a positive multiple of 256 (Q8_0 / Q5_1 down rows: 128)");
     STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
     STRIX_REQUIRE(w->top_k > 0 && w->top_k <= kRouteMaxTopK && w->top_k <= w->experts, "moe: top_k must be within 1..16 and <= experts");
     STRIX_REQUIRE(static_cast<uint64_t>(rows) * w->top_k < (1ULL << 31), "moe: too many assignments");
@@ -1331,7 +1369,7 @@ int32_t mi355_moe_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_r
 int32_t mi355_moe_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
-    launch_plan(r->routes, wv.experts, rows * wv.top_k, plan_split(wv, rows), item_bound(wv, rows), r->plan, hs(stream));
+    launch_plan(dense_routes(r->routes, wv.top_k), wv.experts, rows * wv.top_k, plan_split(wv, rows), item_bound(wv, rows), r->plan, hs(stream));
     STRIX_LAUNCHED("moe plan");
     return MI355_OK;
 }
@@ -1426,7 +1464,7 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
     const uint32_t assignments = rows * wv.top_k, bound = plan_item_bound(wv.experts, assignments, kPfTile);
     hipStream_t st = hs(stream);
     clear_validate_kernel<<<rows, 64, 0, st>>>(r->routes, r->route_weights, wv.experts, wv.top_k, r->status, r->job_status);
-    launch_plan(r->routes, wv.experts, assignments, kPfTile, bound, r->plan, st);
+    launch_plan(dense_routes(r->routes, wv.top_k), wv.experts, assignments, kPfTile, bound, r->plan, st);
     PrefillArgs a{};
     a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.swiglu_limit = wv.swiglu_limit; a.x = static_cast<const uint8_t*>(r->input); a.x_stride = r->input_stride;
     uint8_t* ws = static_cast<uint8_t*>(r->h_f16);
@@ -1560,3 +1598,4 @@ int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float*
 }  // extern "C"
 
 #include "a8_contract.hpp"
+#include "rows_forms.hpp"
