@@ -124,7 +124,7 @@ inline bool strided_ok(const mi355_strided& v, size_t unit) {
 }
 
 // admission of the strided bundle + the kernels' view of it
-int32_t check_strided(const mi355_moe_weights* w, const mi355_moe_rows_strided* v, uint32_t rows, mi355_moe_weights& wv, RowsK& k) {
+int32_t check_strided(const mi355_moe_weights* w, const mi355_moe_rows_strided* v, uint32_t rows, mi355_moe_weights& wv, RowsK& k, bool need_tensors = true) {
     STRIX_REQUIRE(w && v, "moe strided: null weights or rows");
     mi355_moe_rows shell{};                     // check_moe looks at the dense bundle's pointers: stand-ins that pass its null / alignment tests
     shell.routes = static_cast<const uint32_t*>(v->routes.base); shell.route_weights = static_cast<const float*>(v->route_weights.base);
@@ -133,7 +133,7 @@ int32_t check_strided(const mi355_moe_weights* w, const mi355_moe_rows_strided* 
     shell.down_deltas = static_cast<float*>(v->down_deltas.base); shell.down_sums = static_cast<int32_t*>(v->down_sums.base);
     shell.rawdots = static_cast<float*>(v->rawdots.base); shell.output = static_cast<float*>(v->output.base); shell.output_stride = w->hidden;
     shell.plan = v->plan; shell.job_status = v->job_status;
-    if (const int32_t rc = check_moe(w, &shell, rows, wv)) return rc;
+    if (const int32_t rc = check_moe(w, &shell, rows, wv, kIntegerClass, need_tensors)) return rc;
     STRIX_REQUIRE(v->input_kind <= MI355_INPUT_BF16 && (v->output_kind == MI355_INPUT_BF16 || v->output_kind == MI355_INPUT_F32),
                   "moe strided: input kind must be fp32 / fp16 / bf16, output kind bf16 or fp32");
     // every base and stride is 16-byte aligned (include/strix/cuda/qwen_moe.hpp:34); routes, route weights and status are words
@@ -185,7 +185,7 @@ extern "C" {
 
 int32_t mi355_moe_strided_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_rows_strided* v, uint32_t rows, uint32_t clear_words, mi355_stream stream) {
     mi355_moe_weights wv; RowsK k;
-    if (const int32_t rc = check_strided(w, v, rows, wv, k)) return rc;
+    if (const int32_t rc = check_strided(w, v, rows, wv, k, false)) return rc;
     STRIX_REQUIRE(clear_words * 4ULL <= v->accumulation.stride || rows == 1U, "moe strided prologue: clear_words reaches into the next row's accumulation");
     STRIX_REQUIRE(wv.hidden <= 16384U, "moe strided prologue: hidden beyond 16384");
     const size_t lds = wv.hidden + 8U * (wv.hidden / 32U);
@@ -199,7 +199,7 @@ int32_t mi355_moe_strided_enqueue_prologue(const mi355_moe_weights* w, const mi3
 
 int32_t mi355_moe_strided_enqueue_csr(const mi355_moe_weights* w, const mi355_moe_rows_strided* v, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv; RowsK k;
-    if (const int32_t rc = check_strided(w, v, rows, wv, k)) return rc;
+    if (const int32_t rc = check_strided(w, v, rows, wv, k, false)) return rc;
     hipStream_t st = hs(stream);
     launch_plan(RoutesView{k.routes, k.routes_rs, wv.top_k}, wv.experts, rows * wv.top_k, plan_split(wv, rows), item_bound(wv, rows), v->plan, st);
     strided_job_status_kernel<<<1, 1024, 0, st>>>(v->status, rows, v->job_status);
@@ -225,7 +225,7 @@ int32_t mi355_moe_strided_enqueue_down(const mi355_moe_weights* w, const mi355_m
 
 int32_t mi355_moe_strided_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows_strided* v, uint32_t rows, mi355_stream stream) {
     mi355_moe_weights wv; RowsK k;
-    if (const int32_t rc = check_strided(w, v, rows, wv, k)) return rc;
+    if (const int32_t rc = check_strided(w, v, rows, wv, k, false)) return rc;
     strided_merge_kernel<<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(*v, wv.hidden, wv.experts, wv.top_k);
     STRIX_LAUNCHED("moe strided merge");
     return MI355_OK;
@@ -234,7 +234,7 @@ int32_t mi355_moe_strided_enqueue_merge(const mi355_moe_weights* w, const mi355_
 int32_t mi355_moe_strided_enqueue_commit(const mi355_moe_weights* w, const mi355_moe_rows_strided* v, uint32_t rows, uint32_t* record, uint32_t domain,
                                          mi355_stream stream) {
     mi355_moe_weights wv; RowsK k;
-    if (const int32_t rc = check_strided(w, v, rows, wv, k)) return rc;
+    if (const int32_t rc = check_strided(w, v, rows, wv, k, false)) return rc;
     strided_commit_kernel<<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(*v, wv.hidden, rows, record, domain);
     STRIX_LAUNCHED("moe strided commit");
     return MI355_OK;

@@ -1123,7 +1123,8 @@ inline uint64_t moe_row_bytes(uint32_t type, uint32_t k) {
 // Q5_1 (src/cpu/core/routed_expert.hpp:27-28) or Q6_K (src/moe_a8_down_contract.cpp:147). The matrix-core prefill form: Q4_K, Q5_K or Q8_0 for either (a dense shared
 // expert is experts = top_k = 1). The merge reads no weights.
 enum MoeClass { kIntegerClass, kPrefillClass, kAnyClass };
-int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, MoeClass cls = kIntegerClass) {
+int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, mi355_moe_weights& wv, MoeClass cls = kIntegerClass,
+                  bool need_tensors = true) {
     STRIX_REQUIRE(w && r, "moe: null weights or rows");
     STRIX_REQUIRE(rows > 0, "moe: rows must be positive");
     const bool gate_q8 = w->gate_type == MI355_TYPE_Q8_0, down_q8 = w->down_type == MI355_TYPE_Q8_0;
@@ -1155,7 +1156,8 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
     STRIX_REQUIRE(wv.gate_row_stride < (1ULL << 27) && wv.down_row_stride < (1ULL << 27), "moe: weight row stride must be below 128 MiB");
     STRIX_REQUIRE(wv.gate_row_stride >= moe_row_bytes(w->gate_type, w->hidden) &&
                   wv.down_row_stride >= moe_row_bytes(w->down_type, w->ffn), "moe: weight row stride shorter than the row");
-    STRIX_REQUIRE(w->gate && w->up && w->down && aligned(w->gate, 16) && aligned(w->up, 16) && aligned(w->down, 16),
+    // (a stage that reads no weights is admitted on the geometry alone)
+    STRIX_REQUIRE(!need_tensors || (w->gate && w->up && w->down && aligned(w->gate, 16) && aligned(w->up, 16) && aligned(w->down, 16)),
                   "moe: weight pointers must be non-null and 16-byte aligned");
     STRIX_REQUIRE(w->exp_kind <= MI355_EXP_DECLARED, "moe: unknown exp kind");
     // the clamp trait: +infinity (or the zero-initialised 0) = none, else finite and positive (src/moe_a8_down_contract.cpp:57)

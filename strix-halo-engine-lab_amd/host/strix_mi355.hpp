@@ -1,17 +1,29 @@
-// Header-only C++ mirror of the engine-side interfaces this library replaces, over the C ABI in mi355_strix.h.
-// Same names, argument meaning and error behaviour as the reference, so host code written against the reference reads
-// unchanged:
-//   strix::mi355::Q8a8View / Kernels         <- strix::cpu::Q8a8View / Kernels   (src/cpu/core/backend.hpp:52-73)
-//   strix::mi355::qwen_moe::Rows / Weights / enqueue_prologue .. enqueue_merge / enqueue
-//                                             <- strix::cuda::qwen_moe          (include/strix/cuda/qwen_moe.hpp:55-110)
-//   strix::mi355::moe_route::enqueue          <- the route launcher              (include/strix/hip_moe_route_launcher.hpp:16-30)
-// Admission failures throw std::invalid_argument before anything is enqueued, HIP failures throw std::runtime_error, as
-// the reference's validate() / hip_check do. Every pointer is device memory; nothing here allocates or synchronises.
+// Header-only C++ mirror of the engine-side interfaces this library replaces, over the C ABI in mi355_strix.h: the
+// reference's struct and function names, argument order and error behaviour, so that a call site written against the
+// reference compiles against this namespace after the changes listed here and nothing else:
+//   * namespace strix::mi355 in the place of strix; device memory everywhere (the CPU interfaces below take device pointers);
+//   * a stream argument where the reference has a thread pool or a cudaStream_t (mi355_stream = hipStream_t as void*);
+//   * qwen_moe::Rows carries the model geometry (the reference twin fixes it at compile time, include/strix/cuda/qwen_moe.hpp:27),
+//     its Csr views are this library's plan words, and enqueue_project / enqueue take no amdmath::Tables (the exp kind is in Weights);
+//   * expert::Executor is constructed with its capacity (max assignments, max ffn) instead of a thread count.
+// Interfaces:
+//   cpu::Q8a8View / Stream / Kernels            src/cpu/core/backend.hpp:52-73
+//   moe_q4k_a8::Request .. Bindings, validate, enqueue_probe                          include/strix/moe_q4k_a8_contract.hpp:101-122,
+//                                                                                     include/strix/hip_moe_q4k_a8_probe.hpp:12
+//   moe_q4k_a8::DownRequest .. DownBindings, validate_down, enqueue_down_*, SlotMergeTail   include/strix/moe_a8_down_contract.hpp:39-54,
+//                                                                                     include/strix/hip_moe_a8_down.hpp:11-30
+//   qwen_moe::Strided / Rows / Weights, enqueue_prologue .. enqueue_commit, enqueue   include/strix/cuda/qwen_moe.hpp:34-110
+//   expert::LayerWeights / RowA8 / Assignment / Job / Executor                        src/cpu/core/routed_expert.hpp:28-95
+//   moe_route::enqueue                                                                the policy of include/strix/moe_core/route_policy.hpp
+// Admission failures throw std::invalid_argument before anything is enqueued, HIP failures throw std::runtime_error, as the
+// reference's check / hip_check do. Nothing here allocates (Executor's constructor aside) or synchronises.
 #pragma once
 #include <cstddef>
 #include <cstdint>
+#include <limits>
 #include <stdexcept>
 #include <string>
+#include <string_view>
 
 #include "mi355_strix.h"
 
@@ -25,22 +37,273 @@ inline void check(std::int32_t rc) {
 }
 
 // ---------------------------------------------------------------------------------------------- dense kernel table
+namespace cpu {
 using Q8a8View = mi355_q8a8_view;                       // field for field strix::cpu::Q8a8View
-struct Stream { mi355_stream stream = nullptr; };       // the reference's Stream carries a thread count; here a HIP stream
-
+struct Stream { mi355_stream stream = nullptr; };       // the reference's Stream carries the worker pool; here the HIP stream
+// The kernel table: the three entries of strix::cpu::Kernels with their signatures. quantize_a8 and gemv_q8_0_a8 throw
+// std::invalid_argument for a width / in not divisible by 32 before writing any output; zero width is allowed.
 struct Kernels {
-    // x: device fp32 [width]. Throws std::invalid_argument for width % 32 != 0 before any write; sums may be null.
-    static void quantize_a8(const float* x, std::size_t width, std::int8_t* codes, float* deltas, std::int32_t* sums,
-                            const Stream& s = {}) {
-        check(mi355_quantize_a8(x, MI355_INPUT_F32, 1, static_cast<std::uint32_t>(width), width * sizeof(float), codes, deltas,
-                                sums, nullptr, s.stream));
-    }
-    static void gemv_q8_0_a8(const Q8a8View& v, const Stream& s = {}) { check(mi355_gemv_q8_0_a8(&v, s.stream)); }
-    // x, y: device fp32 [rows][n]; w: device fp32 [n] or null (the signature of strix::cpu::Kernels::rmsnorm_f32)
-    static void rmsnorm_f32(const float* x, const float* w, unsigned n, float eps, float* y, unsigned rows, const Stream& s = {}) {
-        check(mi355_rmsnorm_f32(x, w, n, eps, y, rows, s.stream));
-    }
+    void (*quantize_a8)(const float* x, std::size_t width, std::int8_t* codes, float* deltas, std::int32_t* sums);
+    void (*gemv_q8_0_a8)(const Q8a8View& v, const Stream& s);
+    void (*rmsnorm_f32)(const float* x, const float* w, unsigned n, float eps, float* y, unsigned rows, const Stream& s);
 };
+inline const Kernels& mi355_kernels() noexcept {
+    static const Kernels table{
+        [](const float* x, std::size_t width, std::int8_t* codes, float* deltas, std::int32_t* sums) {
+            check(mi355_quantize_a8(x, MI355_INPUT_F32, 1, static_cast<std::uint32_t>(width), width * sizeof(float), codes, deltas, sums, nullptr, nullptr));
+        },
+        [](const Q8a8View& v, const Stream& s) { check(mi355_gemv_q8_0_a8(&v, s.stream)); },
+        [](const float* x, const float* w, unsigned n, float eps, float* y, unsigned rows, const Stream& s) {
+            check(mi355_rmsnorm_f32(x, w, n, eps, y, rows, s.stream));
+        }};
+    return table;
+}
+}  // namespace cpu
+
+// ---------------------------------------------------------------------------------------------- A8 request / bindings
+namespace moe_q4k_a8 {
+inline constexpr float kSwigluNoClamp = std::numeric_limits<float>::infinity();
+inline constexpr unsigned invalid_route = 1U, nonfinite_activation = 2U, invalid_delta = 4U;
+inline constexpr std::uint32_t down_invalid_route = 1, down_nonfinite_activation = 8, down_aggregate_error = 16;
+
+enum class InputKind { bf16, fp32, fp16 };              // the reference has bf16 and fp32
+struct Shape { std::uint32_t hidden = 256, rows = 32, experts = 1, top_k = 1, logical_rows = 1; };
+struct Request {
+    bool enabled = false;
+    std::string_view approved_numerical_identity;
+    InputKind input = InputKind::bf16;
+    Shape shape;
+    std::uint32_t gate_type = 12, up_type = 12;
+    bool fused_gate_up = false;
+    float swiglu_limit = kSwigluNoClamp;
+};
+struct DeviceBytes { std::uintptr_t address = 0; std::uint64_t bytes = 0; };
+struct Bindings { DeviceBytes input, gate, up, routes, codes, deltas, sums, status, output; };
+
+[[nodiscard]] inline std::string_view numerical_identity_for_gate_type(std::uint32_t gate_type) {
+    const char* id = mi355_numerical_identity(gate_type, 0);
+    if (!id[0]) throw std::invalid_argument("A8 gate/up requires type12 or type13");
+    return id;
+}
+[[nodiscard]] inline std::string_view down_numerical_identity(std::uint32_t weight_type) {
+    const char* id = mi355_numerical_identity(weight_type, 1);
+    if (!id[0]) throw std::invalid_argument("A8 down weights must be type 7, 8, 12 or 14");
+    return id;
+}
+
+namespace detail {
+inline mi355_device_bytes c(const DeviceBytes& v) { return mi355_device_bytes{v.address, v.bytes}; }
+struct CRequest { std::string identity; mi355_a8_request q; };
+inline void fill(const Request& r, CRequest& out) {
+    out.identity = std::string(r.approved_numerical_identity);
+    out.q = mi355_a8_request{r.enabled ? 1U : 0U, out.identity.c_str(),
+                             r.input == InputKind::bf16 ? MI355_INPUT_BF16 : r.input == InputKind::fp32 ? MI355_INPUT_F32 : MI355_INPUT_F16,
+                             mi355_a8_shape{r.shape.hidden, r.shape.rows, r.shape.experts, r.shape.top_k, r.shape.logical_rows},
+                             r.gate_type, r.up_type, r.fused_gate_up ? 1U : 0U, r.swiglu_limit};
+}
+inline mi355_a8_bindings c(const Bindings& b) {
+    return mi355_a8_bindings{c(b.input), c(b.gate), c(b.up), c(b.routes), c(b.codes), c(b.deltas), c(b.sums), c(b.status), c(b.output)};
+}
+}  // namespace detail
+
+// Pure host admission; no allocation, HIP call or buffer mutation.
+inline void validate(const Request& request, const Bindings& bindings) {
+    detail::CRequest q; detail::fill(request, q);
+    const mi355_a8_bindings b = detail::c(bindings);
+    check(mi355_a8_validate(&q.q, &b));
+}
+inline void enqueue_probe(const Request& request, const Bindings& bindings, mi355_stream stream = nullptr) {
+    detail::CRequest q; detail::fill(request, q);
+    const mi355_a8_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_probe(&q.q, &b, stream));
+}
+
+struct DownShape { std::uint32_t hidden = 0, intermediate = 0, experts = 0, top_k = 0; };
+struct DownRequest {
+    bool enabled = false;
+    std::string_view approved_numerical_identity;
+    DownShape shape;
+    std::uint32_t weight_type = 7;
+    float swiglu_limit = kSwigluNoClamp;
+};
+struct DownBindings { DeviceBytes intermediates, weights, routes, codes, deltas, sums, rawdots, status, aggregate_status; };
+struct SlotMergeTail {
+    std::uint32_t* tickets = nullptr;
+    const float* route_weights = nullptr;
+    float* accumulation = nullptr;
+    void* output = nullptr;
+    bool output_bf16 = false, bf16_commit = false;
+    void* record = nullptr;  // DeferredMoeFirstError {domain, bits}
+    std::uint32_t domain = 0;
+};
+namespace detail {
+struct CDownRequest { std::string identity; mi355_a8_down_request q; };
+inline void fill(const DownRequest& r, CDownRequest& out) {
+    out.identity = std::string(r.approved_numerical_identity);
+    out.q = mi355_a8_down_request{r.enabled ? 1U : 0U, out.identity.c_str(),
+                                  mi355_a8_down_shape{r.shape.hidden, r.shape.intermediate, r.shape.experts, r.shape.top_k}, r.weight_type, r.swiglu_limit};
+}
+inline mi355_a8_down_bindings c(const DownBindings& b) {
+    return mi355_a8_down_bindings{c(b.intermediates), c(b.weights), c(b.routes), c(b.codes), c(b.deltas), c(b.sums), c(b.rawdots), c(b.status),
+                                  c(b.aggregate_status)};
+}
+}  // namespace detail
+inline void validate_down(const DownRequest& request, const DownBindings& bindings) {
+    detail::CDownRequest q; detail::fill(request, q);
+    const mi355_a8_down_bindings b = detail::c(bindings);
+    check(mi355_a8_validate_down(&q.q, &b, 1));
+}
+// The SiLU's expf is the gfx1151 device function's host twin, as in the reference's kernels.
+inline void enqueue_down_activation_quantize(const DownRequest& request, const DownBindings& bindings, mi355_stream stream) {
+    detail::CDownRequest q; detail::fill(request, q);
+    const mi355_a8_down_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_down_activation_quantize(&q.q, &b, 1, MI355_EXP_GFX1151, stream));
+}
+inline void enqueue_down_rawdots(const DownRequest& request, const DownBindings& bindings, mi355_stream stream) {
+    detail::CDownRequest q; detail::fill(request, q);
+    const mi355_a8_down_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_down_rawdots(&q.q, &b, 1, stream));
+}
+inline void enqueue_down_rawdots(const DownRequest& request, const DownBindings& bindings, const SlotMergeTail& tail, mi355_stream stream) {
+    detail::CDownRequest q; detail::fill(request, q);
+    const mi355_a8_down_bindings b = detail::c(bindings);
+    const mi355_slot_merge_tail t{tail.tickets, tail.route_weights, tail.accumulation, tail.output, tail.output_bf16 ? 1U : 0U, tail.bf16_commit ? 1U : 0U,
+                                  tail.record, tail.domain};
+    check(mi355_a8_enqueue_down_rawdots_merge(&q.q, &b, &t, stream));
+}
+}  // namespace moe_q4k_a8
+
+// ---------------------------------------------------------------------------------------------- strided multi-row layer
+namespace qwen_moe {
+inline constexpr std::uint32_t invalid_route = 1, nonfinite_activation = 2, invalid_delta = 4, projection_nonfinite = 8;
+inline constexpr std::uint32_t type_q5_1 = 7, type_q8_0 = 8, type_q4_k = 12, type_q5_k = 13, type_q6_k = 14;
+// Row r of a view lives at base + r * stride (bytes). Every base and stride must be 16-byte aligned (routes, route weights
+// and status: 4).
+template <class T> struct Strided { T* base = nullptr; std::uint64_t stride = 0; };
+struct Geometry { std::uint32_t hidden = 0, ffn = 0, experts = 0, top_k = 0; };
+struct Csr { std::uint32_t* plan = nullptr; std::uint32_t* summary = nullptr; };   // plan: mi355_moe_plan_words(); summary: one word (the job status)
+struct Rows {
+    Strided<const std::uint16_t> input;        // BF16 [hidden]
+    Strided<const std::uint32_t> routes;       // [top_k]
+    Strided<const float> route_weights;        // [top_k]
+    Strided<std::int8_t> codes;                // [hidden]
+    Strided<float> deltas;                     // [hidden / 32]
+    Strided<std::int32_t> sums;                // [hidden / 32]
+    Strided<std::uint32_t> status;             // [1]
+    Strided<float> intermediates;              // [top_k * 2 * ffn]: h | u per slot; base may be null (not written)
+    Strided<float> accumulation;               // [clear_words >= hidden]: zeroed by the prologue, merge result
+    Strided<std::int8_t> down_codes;           // [top_k * ffn]
+    Strided<float> down_deltas;                // [top_k * ffn / 32]
+    Strided<std::int32_t> down_sums;           // [top_k * ffn / 32]
+    Strided<float> rawdots;                    // [top_k * hidden]
+    Strided<std::uint16_t> output;             // BF16 [hidden]
+    Csr csr;
+    Geometry geometry;
+};
+struct Weights {
+    std::uint32_t gate_type = type_q4_k;       // 12 or 13 (gate and up share it)
+    const std::uint8_t* gate = nullptr;        // [experts][ffn][hidden/256 blocks]
+    const std::uint8_t* up = nullptr;
+    std::uint32_t down_type = type_q5_1;       // 7, 8, 12 or 14
+    const std::uint8_t* down = nullptr;        // [experts][hidden][ffn/32 blocks] (K-quants: ffn/256 super-blocks)
+    std::uint32_t exp_kind = MI355_EXP_GFX1151;
+    float swiglu_limit = std::numeric_limits<float>::infinity();
+};
+namespace detail {
+template <class T> inline mi355_strided c(const Strided<T>& v) { return mi355_strided{const_cast<void*>(static_cast<const void*>(v.base)), v.stride}; }
+inline mi355_moe_rows_strided c(const Rows& r) {
+    mi355_moe_rows_strided v{};
+    v.input = c(r.input); v.routes = c(r.routes); v.route_weights = c(r.route_weights); v.codes = c(r.codes); v.deltas = c(r.deltas); v.sums = c(r.sums);
+    v.status = c(r.status); v.intermediates = c(r.intermediates); v.accumulation = c(r.accumulation); v.down_codes = c(r.down_codes);
+    v.down_deltas = c(r.down_deltas); v.down_sums = c(r.down_sums); v.rawdots = c(r.rawdots); v.output = c(r.output);
+    v.plan = r.csr.plan; v.job_status = r.csr.summary; v.input_kind = MI355_INPUT_BF16; v.output_kind = MI355_INPUT_BF16;
+    return v;
+}
+// (the stages that read no weights are admitted on the geometry alone: default Weights)
+inline mi355_moe_weights c(const Rows& r, const Weights& w) {
+    mi355_moe_weights m{};
+    m.hidden = r.geometry.hidden; m.ffn = r.geometry.ffn; m.experts = r.geometry.experts; m.top_k = r.geometry.top_k;
+    m.gate_type = w.gate_type; m.down_type = w.down_type; m.gate = w.gate; m.up = w.up; m.down = w.down;
+    m.exp_kind = w.exp_kind; m.swiglu_limit = w.swiglu_limit;
+    return m;
+}
+}  // namespace detail
+inline void enqueue_prologue(const Rows& r, std::uint32_t rows, std::uint32_t clear_words, mi355_stream s) {
+    const auto v = detail::c(r); const auto m = detail::c(r, Weights{});
+    check(mi355_moe_strided_enqueue_prologue(&m, &v, rows, clear_words, s));
+}
+inline void enqueue_csr(const Rows& r, std::uint32_t rows, mi355_stream s) {
+    const auto v = detail::c(r); const auto m = detail::c(r, Weights{});
+    check(mi355_moe_strided_enqueue_csr(&m, &v, rows, s));
+}
+inline void enqueue_project(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) {
+    const auto v = detail::c(r); const auto m = detail::c(r, w);
+    check(mi355_moe_strided_enqueue_project(&m, &v, rows, s));
+}
+inline void enqueue_down(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) {
+    const auto v = detail::c(r); const auto m = detail::c(r, w);
+    check(mi355_moe_strided_enqueue_down(&m, &v, rows, s));
+}
+inline void enqueue_merge(const Rows& r, std::uint32_t rows, mi355_stream s) {
+    const auto v = detail::c(r); const auto m = detail::c(r, Weights{});
+    check(mi355_moe_strided_enqueue_merge(&m, &v, rows, s));
+}
+// record: optional device DeferredMoeFirstError {domain, bits}; the domain is the reference's DeferredMoeDomain::q4k_a8 (2)
+inline void enqueue_commit(const Rows& r, std::uint32_t rows, std::uint32_t* record, mi355_stream s) {
+    const auto v = detail::c(r); const auto m = detail::c(r, Weights{});
+    check(mi355_moe_strided_enqueue_commit(&m, &v, rows, record, 2U, s));
+}
+// prologue + csr + project + down + merge + commit
+inline void enqueue(const Rows& r, std::uint32_t rows, std::uint32_t clear_words, const Weights& w, std::uint32_t* record, mi355_stream s) {
+    const auto v = detail::c(r); const auto m = detail::c(r, w);
+    check(mi355_moe_strided_enqueue(&m, &v, rows, clear_words, record, 2U, s));
+}
+}  // namespace qwen_moe
+
+// ---------------------------------------------------------------------------------------------- host executor's job
+namespace expert {
+enum class GateFormat : std::uint8_t { q4_k, q5_k };
+enum class DownFormat : std::uint8_t { q5_1, q8_0 };
+struct Shape { std::uint32_t hidden = 0, ffn = 0; };
+struct LayerWeights {
+    const std::uint8_t* gate = nullptr;
+    const std::uint8_t* up = nullptr;
+    const std::uint8_t* down = nullptr;
+    GateFormat gate_format = GateFormat::q4_k;
+    DownFormat down_format = DownFormat::q5_1;
+    Shape shape;
+};
+using RowA8 = mi355_row_a8;                    // codes, deltas, sums (device pointers)
+using Assignment = mi355_expert_assignment;    // row, slot, expert
+inline constexpr std::uint32_t kNonfinite = 1U;
+struct Job {
+    LayerWeights weights;
+    const RowA8* rows = nullptr;               // device array, indexed by Assignment::row
+    const Assignment* assignments = nullptr;   // device array
+    std::uint32_t count = 0;
+    float* rawdots = nullptr;                  // rawdots[row * rawdot_row_stride + slot * hidden + o]
+    std::uint64_t rawdot_row_stride = 0;       // in floats
+    std::uint32_t* status = nullptr;           // per row, OR-ed
+};
+class Executor {
+public:
+    Executor(std::uint32_t max_assignments, std::uint32_t max_ffn, std::uint32_t exp_kind = MI355_EXP_GFX1151)
+        : handle_(mi355_executor_create(max_assignments, max_ffn, exp_kind)) {
+        if (!handle_) throw std::invalid_argument(mi355_last_error());
+    }
+    ~Executor() { mi355_executor_destroy(handle_); }
+    Executor(const Executor&) = delete;
+    Executor& operator=(const Executor&) = delete;
+    void run(const Job& job, mi355_stream stream = nullptr) {
+        const mi355_expert_job j{mi355_layer_weights{job.weights.gate, job.weights.up, job.weights.down, static_cast<std::uint32_t>(job.weights.gate_format),
+                                                     static_cast<std::uint32_t>(job.weights.down_format), job.weights.shape.hidden, job.weights.shape.ffn},
+                                 job.rows, job.assignments, job.count, job.rawdots, job.rawdot_row_stride, job.status};
+        check(mi355_executor_run(handle_, &j, stream));
+    }
+private:
+    void* handle_;
+};
+}  // namespace expert
 
 // ---------------------------------------------------------------------------------------------- router
 namespace moe_route {
@@ -48,54 +311,8 @@ using Policy = mi355_route_policy;
 inline void enqueue(const Policy& policy, const void* x, std::uint32_t input_kind, std::uint32_t rows, std::uint32_t hidden,
                     std::uint64_t x_stride_bytes, const float* router_weight, const float* logit_bias, std::uint32_t* ids,
                     float* weights, float* scores, mi355_stream stream) {
-    check(mi355_moe_route(&policy, x, input_kind, rows, hidden, x_stride_bytes, router_weight, logit_bias, ids, weights, scores,
-                          stream));
+    check(mi355_moe_route(&policy, x, input_kind, rows, hidden, x_stride_bytes, router_weight, logit_bias, ids, weights, scores, stream));
 }
 }  // namespace moe_route
-
-// ---------------------------------------------------------------------------------------------- routed experts
-namespace qwen_moe {
-using Rows = mi355_moe_rows;          // per-row views: input, routes, route_weights, A8 image, status, h image, rawdots, output
-using Weights = mi355_moe_weights;    // gate / up [experts][ffn][hidden/256 blocks], down [experts][hidden][ffn/256 blocks]
-
-inline std::size_t plan_words(std::uint32_t experts, std::uint32_t rows, std::uint32_t top_k) {
-    return mi355_moe_plan_words(experts, rows, top_k);
-}
-inline std::size_t prefill_f16_workspace_bytes(std::uint32_t hidden, std::uint32_t ffn, std::uint32_t rows, std::uint32_t top_k) {
-    return mi355_moe_prefill_f16_workspace_bytes(hidden, ffn, rows, top_k);
-}
-inline void enqueue_prologue(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) { check(mi355_moe_enqueue_prologue(&w, &r, rows, s)); }
-inline void enqueue_csr(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) { check(mi355_moe_enqueue_csr(&w, &r, rows, s)); }
-inline void enqueue_project(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) { check(mi355_moe_enqueue_project(&w, &r, rows, s)); }
-inline void enqueue_down(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s) { check(mi355_moe_enqueue_down(&w, &r, rows, s)); }
-inline void enqueue_merge(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s,
-                          std::uint32_t form = MI355_COMBINE_FMA_SLOT_ORDER) {
-    check(mi355_moe_enqueue_merge(&w, &r, rows, form, s));
-}
-// prologue + csr + project + down + merge
-inline void enqueue(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s,
-                    std::uint32_t form = MI355_COMBINE_FMA_SLOT_ORDER) {
-    check(mi355_moe_enqueue(&w, &r, rows, form, s));
-}
-// the routed experts of a prefill batch on fp16 MFMA (FAST class: follows the exact-weight product to 2e-3, not the
-// integer-dot bits); needs r.h_f16 and fp16 input rows
-inline void enqueue_prefill_f16(const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s,
-                                std::uint32_t form = MI355_COMBINE_FMA_SLOT_ORDER) {
-    check(mi355_moe_enqueue_prefill_f16(&w, &r, rows, form, s));
-}
-// router + the layer; r.routes / r.route_weights receive the selection
-inline void enqueue_layer(const moe_route::Policy& policy, const float* router_weight, const float* logit_bias, float* scores,
-                          const Rows& r, std::uint32_t rows, const Weights& w, mi355_stream s,
-                          std::uint32_t form = MI355_COMBINE_FMA_SLOT_ORDER) {
-    check(mi355_moe_enqueue_layer(&policy, router_weight, logit_bias, scores, &w, &r, rows, form, s));
-}
-}  // namespace qwen_moe
-
-// SwiGLU + A8 re-quantisation of dense gate | up rows (enqueue_down_activation_quantize, include/strix/hip_moe_a8_down.hpp:18).
-inline void enqueue_down_activation_quantize(const float* gate, const float* up, std::uint32_t rows, std::uint32_t ffn,
-                                             std::uint32_t exp_kind, float swiglu_limit, std::int8_t* codes, float* deltas,
-                                             std::int32_t* sums, float* h_out, std::uint32_t* status, mi355_stream s) {
-    check(mi355_swiglu_quantize(gate, up, rows, ffn, exp_kind, swiglu_limit, codes, deltas, sums, h_out, status, s));
-}
 
 }  // namespace strix::mi355

@@ -1,0 +1,277 @@
+// Calls the library on the GPU through the C++ mirror of the reference's interfaces (strix_mi355.hpp) and checks the bits
+// against the CPU oracle (liboracle.so, the checker). Built by __graft_entry__.build() with hipcc as host C++; run as a child
+// process by tests/test_gpu_cpp_mirror.py. Exit status = number of failed checks.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "strix_mi355.hpp"
+extern "C" {
+#include "strix_oracle.h"
+}
+
+namespace m = strix::mi355;
+
+static int failures = 0;
+static void expect(bool ok, const char* what) {
+    std::printf("%s %s\n", ok ? "PASS" : "FAIL", what);
+    std::fflush(stdout);
+    if (!ok) ++failures;
+}
+static void hip(hipError_t e, const char* what) {
+    if (e != hipSuccess) { std::printf("HIP error in %s: %s\n", what, hipGetErrorString(e)); std::exit(100); }
+}
+template <class T> struct Dev {                        // a device array with its host copy
+    T* p = nullptr;
+    size_t n = 0;
+    explicit Dev(size_t count) : n(count) { hip(hipMalloc(reinterpret_cast<void**>(&p), (count ? count : 1) * sizeof(T)), "hipMalloc"); hip(hipMemset(p, 0, (count ? count : 1) * sizeof(T)), "hipMemset"); }
+    explicit Dev(const std::vector<T>& h) : Dev(h.size()) { put(h); }
+    ~Dev() { (void)hipFree(p); }
+    Dev(const Dev&) = delete;
+    void put(const std::vector<T>& h) { hip(hipMemcpy(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice), "H2D"); }
+    std::vector<T> get() const { std::vector<T> h(n); hip(hipMemcpy(h.data(), p, n * sizeof(T), hipMemcpyDeviceToHost), "D2H"); return h; }
+    m::moe_q4k_a8::DeviceBytes bytes() const { return {reinterpret_cast<std::uintptr_t>(p), static_cast<std::uint64_t>(n * sizeof(T))}; }
+};
+template <class T> static bool same_bits(const std::vector<T>& a, const std::vector<T>& b) {
+    return a.size() == b.size() && std::memcmp(a.data(), b.data(), a.size() * sizeof(T)) == 0;
+}
+static std::uint16_t bf16_rne(float f) {
+    std::uint32_t b; std::memcpy(&b, &f, 4);
+    return static_cast<std::uint16_t>((b + 0x7fffU + ((b >> 16) & 1U)) >> 16);
+}
+static float bf16_value(std::uint16_t h) { const std::uint32_t b = static_cast<std::uint32_t>(h) << 16; float f; std::memcpy(&f, &b, 4); return f; }
+
+constexpr std::uint32_t H = 512, I = 256, E = 4, K = 2, T = 3;
+static std::mt19937 rng(12345);
+static std::vector<float> normal(size_t n, float scale) {
+    std::normal_distribution<float> d(0.0F, scale);
+    std::vector<float> v(n);
+    for (auto& x : v) x = d(rng);
+    return v;
+}
+static std::vector<std::uint8_t> q4k_tensor(size_t rows, std::uint32_t width, float scale) {
+    std::vector<std::uint8_t> out(rows * (width / 256) * 144);
+    const std::vector<float> w = normal(rows * width, scale);
+    for (size_t r = 0; r < rows; ++r) orc_quantize_q4_k_row(w.data() + r * width, width, out.data() + r * (width / 256) * 144);
+    return out;
+}
+static std::vector<std::uint8_t> q8_0_tensor(size_t rows, std::uint32_t width, float scale) {
+    std::vector<std::uint8_t> out(rows * (width / 32) * 34);
+    const std::vector<float> w = normal(rows * width, scale);
+    for (size_t r = 0; r < rows; ++r) orc_quantize_q8_0_row(w.data() + r * width, width, out.data() + r * (width / 32) * 34);
+    return out;
+}
+
+// ----------------------------------------------------------------------------------------------- the dense kernel table
+static void kernel_table() {
+    const m::cpu::Kernels& k = m::cpu::mi355_kernels();
+    const std::uint32_t width = 1024, count = 96;
+    const std::vector<float> x = normal(width, 1.0F);
+    Dev<float> dx(x), dd(width / 32), dy(width), dout(count);
+    Dev<std::int8_t> dc(width);
+    Dev<std::int32_t> ds(width / 32);
+    k.quantize_a8(dx.p, width, dc.p, dd.p, ds.p);
+    std::vector<std::int8_t> c(width); std::vector<float> d(width / 32); std::vector<std::int32_t> s(width / 32);
+    orc_quantize_a8(x.data(), width, c.data(), d.data(), s.data(), 1);
+    expect(same_bits(dc.get(), c) && same_bits(dd.get(), d) && same_bits(ds.get(), s), "Kernels::quantize_a8 == oracle");
+    const std::vector<std::uint8_t> w = q8_0_tensor(count, width, 0.05F);
+    Dev<std::uint8_t> dw(w);
+    const m::cpu::Q8a8View view{dw.p, dc.p, dd.p, dout.p, width / 32 * 34, width, count, 1, width, count, 0};
+    k.gemv_q8_0_a8(view, m::cpu::Stream{});
+    std::vector<float> want(count);
+    const orc_q8a8_view ov{w.data(), c.data(), d.data(), want.data(), width / 32 * 34, width, count, 1, width, count, 0};
+    orc_gemv_q8_0_a8(&ov, 1);
+    expect(same_bits(dout.get(), want), "Kernels::gemv_q8_0_a8 == oracle");
+    const std::vector<float> g = normal(width, 1.0F);
+    Dev<float> dg(g);
+    k.rmsnorm_f32(dx.p, dg.p, width, 1e-6F, dy.p, 1, m::cpu::Stream{});
+    std::vector<float> yn(width);
+    orc_rmsnorm_f32(x.data(), g.data(), width, 1e-6F, yn.data(), 1);
+    expect(same_bits(dy.get(), yn), "Kernels::rmsnorm_f32 == oracle");
+    bool threw = false;
+    try { k.quantize_a8(dx.p, 33, dc.p, dd.p, ds.p); } catch (const std::invalid_argument&) { threw = true; }
+    expect(threw, "Kernels::quantize_a8 throws std::invalid_argument for width % 32 != 0");
+}
+
+// ----------------------------------------------------------------------------------------------- one expert layer, three ways
+struct Layer {
+    std::vector<std::uint8_t> gate = q4k_tensor(size_t(E) * I, H, 0.05F), up = q4k_tensor(size_t(E) * I, H, 0.05F);
+    std::vector<std::uint8_t> down = q4k_tensor(size_t(E) * H, I, 0.05F), down8 = q8_0_tensor(size_t(E) * H, I, 0.05F);
+    std::vector<std::uint16_t> x;                          // bf16 rows
+    std::vector<float> x32;
+    std::vector<std::uint32_t> routes{1, 3, 0, 2, 3, 1};   // [T][K]
+    std::vector<float> weights{0.75F, 0.25F, 0.5F, 0.5F, 0.125F, 0.875F};
+    std::vector<std::int8_t> c; std::vector<float> d; std::vector<std::int32_t> s;
+    Layer() : c(T * H), d(T * H / 32), s(T * H / 32) {
+        const std::vector<float> raw = normal(T * H, 1.0F);
+        for (float v : raw) { x.push_back(bf16_rne(v)); x32.push_back(bf16_value(x.back())); }
+        for (std::uint32_t t = 0; t < T; ++t) orc_quantize_a8(x32.data() + t * H, H, c.data() + t * H, d.data() + t * (H / 32), s.data() + t * (H / 32), 0);
+    }
+    // the oracle's whole job with the given down tensor
+    struct Result { std::vector<float> gate, up, h, rawdots; std::vector<std::int8_t> hc; std::vector<float> hd; std::vector<std::int32_t> hs; };
+    Result oracle(const std::vector<std::uint8_t>& down_tensor, std::uint32_t down_type) const {
+        Result r;
+        const size_t n = size_t(T) * K;
+        r.gate.resize(n * I); r.up.resize(n * I); r.h.resize(n * I); r.rawdots.resize(n * H); r.hc.resize(n * I); r.hd.resize(n * I / 32); r.hs.resize(n * I / 32);
+        std::vector<std::uint32_t> status(T);
+        const std::uint64_t grb = H / 256 * 144, drb = down_type == 12 ? I / 256 * 144 : I / 32 * 34;
+        const orc_expert_weights w{H, I, E, K, 12, down_type, gate.data(), up.data(), down_tensor.data(), grb * I, grb, drb * H, drb, 0, INFINITY};
+        const orc_expert_job job{c.data(), d.data(), s.data(), routes.data(), T, r.gate.data(), r.up.data(), r.h.data(), r.hc.data(), r.hd.data(), r.hs.data(),
+                                 r.rawdots.data(), status.data()};
+        orc_routed_experts(&w, &job, 1);
+        return r;
+    }
+};
+
+static void a8_single_row(const Layer& L) {
+    namespace a8 = m::moe_q4k_a8;
+    const Layer::Result ref = L.oracle(L.down, 12);
+    Dev<std::uint8_t> gate(L.gate), up(L.up), down(L.down);
+    Dev<std::uint16_t> input(std::vector<std::uint16_t>(L.x.begin(), L.x.begin() + H));
+    Dev<std::uint32_t> routes(std::vector<std::uint32_t>(L.routes.begin(), L.routes.begin() + K)), status(1), aggregate(1), record(2);
+    Dev<std::int8_t> codes(H), hcodes(K * I);
+    Dev<float> deltas(H / 32), output(K * 2 * I), hdeltas(K * I / 32), rawdots(K * H), acc(H), route_w(std::vector<float>(L.weights.begin(), L.weights.begin() + K));
+    Dev<std::int32_t> sums(H / 32), hsums(K * I / 32);
+    Dev<std::uint16_t> y(H);
+    a8::Request q;
+    q.enabled = true; q.approved_numerical_identity = a8::numerical_identity_for_gate_type(12); q.input = a8::InputKind::bf16;
+    q.shape = a8::Shape{H, I, E, K, 1};
+    const a8::Bindings b{input.bytes(), gate.bytes(), up.bytes(), routes.bytes(), codes.bytes(), deltas.bytes(), sums.bytes(), status.bytes(), output.bytes()};
+    a8::validate(q, b);
+    a8::enqueue_probe(q, b, nullptr);
+    const std::vector<float> out = output.get();
+    bool ok = true;
+    for (std::uint32_t k = 0; k < K; ++k)
+        ok = ok && std::memcmp(out.data() + (k * 2) * I, ref.gate.data() + k * I, I * 4) == 0 && std::memcmp(out.data() + (k * 2 + 1) * I, ref.up.data() + k * I, I * 4) == 0;
+    expect(ok, "moe_q4k_a8::enqueue_probe: output[(slot * 2 + which) * rows + i] == oracle gate / up rows");
+    a8::DownRequest dq;
+    dq.enabled = true; dq.approved_numerical_identity = a8::down_numerical_identity(12); dq.shape = a8::DownShape{H, I, E, K}; dq.weight_type = 12;
+    const a8::DownBindings db{output.bytes(), down.bytes(), routes.bytes(), hcodes.bytes(), hdeltas.bytes(), hsums.bytes(), rawdots.bytes(), status.bytes(), aggregate.bytes()};
+    a8::validate_down(dq, db);
+    a8::enqueue_down_activation_quantize(dq, db, nullptr);
+    expect(same_bits(hcodes.get(), std::vector<std::int8_t>(ref.hc.begin(), ref.hc.begin() + K * I)) &&
+           same_bits(hdeltas.get(), std::vector<float>(ref.hd.begin(), ref.hd.begin() + K * I / 32)), "moe_q4k_a8::enqueue_down_activation_quantize == oracle h image");
+    a8::SlotMergeTail tail;
+    tail.route_weights = route_w.p; tail.accumulation = acc.p; tail.output = y.p; tail.output_bf16 = true; tail.bf16_commit = true; tail.record = record.p; tail.domain = 2;
+    a8::enqueue_down_rawdots(dq, db, tail, nullptr);
+    expect(same_bits(rawdots.get(), std::vector<float>(ref.rawdots.begin(), ref.rawdots.begin() + K * H)), "moe_q4k_a8::enqueue_down_rawdots (merge tail) rawdots == oracle");
+    std::vector<float> want(H);
+    orc_combine(0, 1, K, H, L.weights.data(), L.routes.data(), ref.rawdots.data(), nullptr, want.data());
+    std::vector<std::uint16_t> want16;
+    for (float v : want) want16.push_back(bf16_rne(v));
+    expect(same_bits(acc.get(), want) && same_bits(y.get(), want16) && status.get()[0] == 0 && record.get()[0] == 0, "slot merge tail: accumulation, bf16 output, clean status");
+    bool threw = false;
+    q.approved_numerical_identity = "not the approved arithmetic";
+    try { a8::enqueue_probe(q, b, nullptr); } catch (const std::invalid_argument&) { threw = true; }
+    expect(threw, "moe_q4k_a8::enqueue_probe throws std::invalid_argument without the identity approval");
+}
+
+static void strided_rows(const Layer& L) {
+    namespace qm = m::qwen_moe;
+    const Layer::Result ref = L.oracle(L.down8, 8);
+    Dev<std::uint8_t> gate(L.gate), up(L.up), down(L.down8);
+    // one record of bytes per row holding every view (all strides equal, none dense)
+    const size_t off_in = 0, off_routes = off_in + 2 * H, off_w = off_routes + 16, off_codes = off_w + 16, off_d = off_codes + H, off_s = off_d + H / 8,
+                 off_status = off_s + H / 8, off_inter = off_status + 16, off_acc = off_inter + 8 * K * I, off_hc = off_acc + 4 * H, off_hd = off_hc + K * I,
+                 off_hs = off_hd + K * I / 8, off_raw = off_hs + K * I / 8, off_out = off_raw + 4 * K * H, stride = off_out + 2 * H + 64;
+    std::vector<std::uint8_t> host(T * stride, 0x5A);
+    for (std::uint32_t t = 0; t < T; ++t) {
+        std::memcpy(host.data() + t * stride + off_in, L.x.data() + t * H, 2 * H);
+        std::memcpy(host.data() + t * stride + off_routes, L.routes.data() + t * K, 4 * K);
+        std::memcpy(host.data() + t * stride + off_w, L.weights.data() + t * K, 4 * K);
+    }
+    Dev<std::uint8_t> block(host);
+    Dev<std::uint32_t> plan(mi355_moe_plan_words(E, T, K)), summary(1), record(2);
+    qm::Rows r;
+    const auto at = [&](size_t off) { return block.p + off; };
+    r.input = {reinterpret_cast<const std::uint16_t*>(at(off_in)), stride}; r.routes = {reinterpret_cast<const std::uint32_t*>(at(off_routes)), stride};
+    r.route_weights = {reinterpret_cast<const float*>(at(off_w)), stride}; r.codes = {reinterpret_cast<std::int8_t*>(at(off_codes)), stride};
+    r.deltas = {reinterpret_cast<float*>(at(off_d)), stride}; r.sums = {reinterpret_cast<std::int32_t*>(at(off_s)), stride};
+    r.status = {reinterpret_cast<std::uint32_t*>(at(off_status)), stride}; r.intermediates = {reinterpret_cast<float*>(at(off_inter)), stride};
+    r.accumulation = {reinterpret_cast<float*>(at(off_acc)), stride}; r.down_codes = {reinterpret_cast<std::int8_t*>(at(off_hc)), stride};
+    r.down_deltas = {reinterpret_cast<float*>(at(off_hd)), stride}; r.down_sums = {reinterpret_cast<std::int32_t*>(at(off_hs)), stride};
+    r.rawdots = {reinterpret_cast<float*>(at(off_raw)), stride}; r.output = {reinterpret_cast<std::uint16_t*>(at(off_out)), stride};
+    r.csr = qm::Csr{plan.p, summary.p};
+    r.geometry = qm::Geometry{H, I, E, K};
+    qm::Weights w;
+    w.gate_type = qm::type_q4_k; w.gate = gate.p; w.up = up.p; w.down_type = qm::type_q8_0; w.down = down.p;
+    qm::enqueue_prologue(r, T, H, nullptr);
+    qm::enqueue_csr(r, T, nullptr);
+    qm::enqueue_project(r, T, w, nullptr);
+    qm::enqueue_down(r, T, w, nullptr);
+    qm::enqueue_merge(r, T, nullptr);
+    qm::enqueue_commit(r, T, record.p, nullptr);
+    const std::vector<std::uint8_t> got = block.get();
+    std::vector<float> want(T * H);
+    orc_combine(0, T, K, H, L.weights.data(), L.routes.data(), ref.rawdots.data(), nullptr, want.data());
+    bool raw_ok = true, out_ok = true, codes_ok = true;
+    for (std::uint32_t t = 0; t < T; ++t) {
+        raw_ok = raw_ok && std::memcmp(got.data() + t * stride + off_raw, ref.rawdots.data() + size_t(t) * K * H, 4 * K * H) == 0;
+        codes_ok = codes_ok && std::memcmp(got.data() + t * stride + off_codes, L.c.data() + t * H, H) == 0 &&
+                   std::memcmp(got.data() + t * stride + off_hc, ref.hc.data() + size_t(t) * K * I, K * I) == 0;
+        for (std::uint32_t o = 0; o < H; ++o) {
+            std::uint16_t v; std::memcpy(&v, got.data() + t * stride + off_out + 2 * o, 2);
+            out_ok = out_ok && v == bf16_rne(want[t * H + o]);
+        }
+    }
+    expect(codes_ok, "qwen_moe strided stages: A8 images of the input and of h == oracle");
+    expect(raw_ok, "qwen_moe strided stages: rawdots == oracle");
+    expect(out_ok && summary.get()[0] == 0 && record.get()[0] == 0, "qwen_moe strided stages: bf16 output == oracle merge, clean job");
+}
+
+static void executor_job(const Layer& L) {
+    namespace ex = m::expert;
+    const Layer::Result ref = L.oracle(L.down8, 8);
+    Dev<std::uint8_t> gate(L.gate), up(L.up), down(L.down8);
+    Dev<std::int8_t> c(L.c);
+    Dev<float> d(L.d);
+    Dev<std::int32_t> s(L.s);
+    std::vector<ex::RowA8> table;
+    for (std::uint32_t t = 0; t < T; ++t) table.push_back(ex::RowA8{c.p + t * H, d.p + t * (H / 32), s.p + t * (H / 32)});
+    std::vector<ex::Assignment> list;
+    for (std::uint32_t t = T; t-- > 0;)                      // rows in descending order: the list is in no particular order
+        for (std::uint32_t k = 0; k < K; ++k) list.push_back(ex::Assignment{t, k, L.routes[t * K + k]});
+    Dev<ex::RowA8> dtable(table);
+    Dev<ex::Assignment> dlist(list);
+    const std::uint64_t row_stride = K * H + 32;
+    Dev<float> raw(T * row_stride);
+    Dev<std::uint32_t> status(T);
+    ex::Job job;
+    job.weights = ex::LayerWeights{gate.p, up.p, down.p, ex::GateFormat::q4_k, ex::DownFormat::q8_0, ex::Shape{H, I}};
+    job.rows = dtable.p; job.assignments = dlist.p; job.count = static_cast<std::uint32_t>(list.size());
+    job.rawdots = raw.p; job.rawdot_row_stride = row_stride; job.status = status.p;
+    ex::Executor pool(64, 256);
+    pool.run(job);
+    const std::vector<float> got = raw.get();
+    bool ok = true;
+    for (std::uint32_t t = 0; t < T; ++t) ok = ok && std::memcmp(got.data() + t * row_stride, ref.rawdots.data() + size_t(t) * K * H, 4 * K * H) == 0;
+    expect(ok && status.get() == std::vector<std::uint32_t>(T, 0U), "expert::Executor::run(Job): rawdots == oracle");
+    bool threw = false;
+    job.count = 65;
+    try { pool.run(job); } catch (const std::invalid_argument&) { threw = true; }
+    expect(threw, "expert::Executor::run throws std::invalid_argument for a job beyond its capacity");
+}
+
+int main() {
+    int devices = 0;
+    if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) { std::printf("no GPU\n"); return 99; }
+    hip(hipSetDevice(0), "hipSetDevice");
+    try {
+        kernel_table();
+        const Layer L;
+        a8_single_row(L);
+        strided_rows(L);
+        executor_job(L);
+    } catch (const std::exception& e) {
+        std::printf("FAIL exception: %s\n", e.what());
+        return 98;
+    }
+    hip(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    std::printf("%d failed\n", failures);
+    return failures;
+}

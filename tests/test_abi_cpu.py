@@ -123,12 +123,11 @@ def test_product_path_never_references_the_oracle():
                 assert "liboracle" not in text and "import orc" not in text and "strix_oracle.h" not in text, f
 
 
-def test_cpp_host_mirror_compiles_against_the_header():
-    """The header-only C++ mirror of the reference interfaces must compile against include/mi355_strix.h with a host compiler."""
-    import subprocess, tempfile
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    with tempfile.NamedTemporaryFile("w", suffix=".cpp", delete=False) as f:
-        f.write('#include "strix_mi355.hpp"\nint main() { return 0; }\n')
-    subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I" + os.path.join(root, "include"),
-                    "-I" + os.path.join(root, "strix-halo-engine-lab_amd", "host"), f.name], check=True)
-    os.unlink(f.name)
+def test_cpp_host_mirror_compiles_and_links():
+    """The C++ mirror of the reference interfaces and the program that drives the GPU through it compile and link against the
+    library (the run is tests/test_gpu_cpp_mirror.py)."""
+    import __graft_entry__
+    if not os.path.exists(LIB):
+        __graft_entry__.build()
+    __graft_entry__.build_cpp_mirror_test()
+    assert os.path.exists(os.path.join(ROOT, "tests", "cpp", "mirror_gpu_test.bin"))

@@ -1,0 +1,21 @@
+"""Runs the hipcc-built C++ program that calls the library through the C++ mirror of the reference's interfaces
+(strix-halo-engine-lab_amd/host/strix_mi355.hpp: cpu::Kernels, moe_q4k_a8::enqueue_probe / enqueue_down_*, qwen_moe::enqueue_*
+on strided Rows, expert::Executor::run(Job)) and checks every result bit for bit against the oracle, in a child process."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "mirror_gpu_test.bin")
+
+
+@pytest.mark.gpu
+def test_cpp_mirror_program_on_the_gpu():
+    assert os.path.exists(BIN), "tests/cpp/mirror_gpu_test.bin is built by __graft_entry__.build()"
+    run = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
+    print(run.stdout)
+    print(run.stderr)
+    assert run.returncode == 0, run.stdout + run.stderr
+    lines = [l for l in run.stdout.splitlines() if l.startswith(("PASS", "FAIL"))]
+    assert len(lines) >= 12 and all(l.startswith("PASS") for l in lines)
