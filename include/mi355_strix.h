@@ -394,6 +394,36 @@ void* mi355_executor_create(uint32_t max_assignments, uint32_t max_ffn, uint32_t
 int32_t mi355_executor_run(void* executor, const mi355_expert_job* job, mi355_stream);
 void mi355_executor_destroy(void* executor);
 
+/* ------------------------------------------------------------------------------------------------------
+ * GGUF v3 container reader and the tensor map of one MoE layer: the data format in front of the path (the reference:
+ * strix::gguf::read_file / FileInfo / TensorInfo, include/strix/gguf_reader.hpp:75-117, src/gguf_reader.cpp; the expert
+ * tensors as src/qwen_moe_prepared.cpp:104-119 names them). Host code only. open() parses and validates the whole index
+ * (version 3, bounded counts, lower-case dotted keys, no duplicate key or tensor name, rank 1..4 with non-zero extents, known
+ * tensor types with a pinned storage geometry, general.alignment a non-zero multiple of 8, zero padding, aligned offsets,
+ * every tensor inside the file, no overlap) and returns NULL with mi355_last_error() set on any violation. offset is the
+ * ABSOLUTE file offset of the tensor's first byte; dims are fastest first, as stored.
+ */
+typedef struct mi355_gguf_tensor { const char* name; uint32_t n_dims; uint64_t dims[4]; uint32_t ggml_type; uint64_t offset, bytes; } mi355_gguf_tensor;
+void* mi355_gguf_open(const char* path);
+void mi355_gguf_close(void* file);
+uint64_t mi355_gguf_tensor_count(const void* file);
+uint64_t mi355_gguf_metadata_count(const void* file);
+uint64_t mi355_gguf_alignment(const void* file);
+uint64_t mi355_gguf_data_offset(const void* file);
+int32_t mi355_gguf_tensor_at(const void* file, uint64_t index, mi355_gguf_tensor* out);
+int32_t mi355_gguf_find_tensor(const void* file, const char* name, mi355_gguf_tensor* out);
+/* kind: 0 unsigned or boolean (*u), 1 signed (*i), 2 floating (*f), 3 string (*text, valid until close), 4 array (*u = length) */
+int32_t mi355_gguf_metadata(const void* file, const char* key, uint32_t* kind, uint64_t* u, int64_t* i, double* f, const char** text);
+/* blk.<layer>.ffn_gate_exps / ffn_up_exps [hidden][ffn][experts], ffn_down_exps [ffn][hidden][experts], ffn_gate_inp F32
+ * [hidden][experts]; optional (bytes == 0 when absent): ffn_norm F32 [hidden], exp_probs_b F32 [experts], the shared expert
+ * ffn_gate_shexp / ffn_up_shexp [hidden][shared_ffn], ffn_down_shexp [shared_ffn][hidden], ffn_gate_inp_shexp F32 [hidden].
+ * The expert tensors' bytes are [experts][rows][blocks], exactly what mi355_moe_weights takes. */
+typedef struct mi355_gguf_moe_layer_map {
+    mi355_gguf_tensor gate, up, down, router, norm, router_bias, shared_gate, shared_up, shared_down, shared_router;
+    uint32_t hidden, ffn, experts, shared_ffn, gate_type, down_type;
+} mi355_gguf_moe_layer_map;
+int32_t mi355_gguf_moe_layer(const void* file, uint32_t layer, mi355_gguf_moe_layer_map* out);
+
 #ifdef __cplusplus
 }
 #endif

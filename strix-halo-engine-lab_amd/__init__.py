@@ -120,6 +120,78 @@ class ExpertJob(C.Structure):
                 ("rawdot_row_stride", C.c_uint64), ("status", C.c_void_p)]
 
 
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 4), ("ggml_type", C.c_uint32), ("offset", C.c_uint64),
+                ("bytes", C.c_uint64)]
+
+
+class GgufMoeLayerMap(C.Structure):
+    _fields_ = [(n, GgufTensor) for n in ("gate", "up", "down", "router", "norm", "router_bias", "shared_gate", "shared_up", "shared_down",
+                                           "shared_router")] + \
+               [(n, C.c_uint32) for n in ("hidden", "ffn", "experts", "shared_ffn", "gate_type", "down_type")]
+
+
+class GgufFile:
+    """A parsed GGUF v3 file (strix::gguf::FileInfo, include/strix/gguf_reader.hpp:89-104): the tensor index, the metadata and the
+    map of a MoE layer. Raises StrixError with the reader's reason for a file it does not admit."""
+
+    def __init__(self, path):
+        self.path = path
+        self.handle = lib().mi355_gguf_open(os.fsencode(path))
+        if not self.handle:
+            raise StrixError(E_INVALID_ARGUMENT, lib().mi355_last_error().decode())
+        self.alignment = lib().mi355_gguf_alignment(self.handle)
+        self.data_offset = lib().mi355_gguf_data_offset(self.handle)
+
+    def close(self):
+        if self.handle:
+            lib().mi355_gguf_close(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        self.close()
+
+    @staticmethod
+    def _info(t):
+        return {"name": t.name.decode(), "dims": [int(t.dims[i]) for i in range(t.n_dims)], "type": int(t.ggml_type), "offset": int(t.offset),
+                "bytes": int(t.bytes)}
+
+    def tensors(self):
+        out = []
+        for i in range(lib().mi355_gguf_tensor_count(self.handle)):
+            t = GgufTensor()
+            check(lib().mi355_gguf_tensor_at(self.handle, i, C.byref(t)))
+            out.append(self._info(t))
+        return out
+
+    def metadata(self, key):
+        kind, u, i, f, text = C.c_uint32(), C.c_uint64(), C.c_int64(), C.c_double(), C.c_char_p()
+        check(lib().mi355_gguf_metadata(self.handle, key.encode(), C.byref(kind), C.byref(u), C.byref(i), C.byref(f), C.byref(text)))
+        return [u.value, i.value, f.value, text.value.decode() if text.value is not None else None, u.value][kind.value]
+
+    def moe_layer_map(self, layer):
+        m = GgufMoeLayerMap()
+        check(lib().mi355_gguf_moe_layer(self.handle, layer, C.byref(m)))
+        return m
+
+    def read(self, t, device=None):
+        """The bytes of a tensor (a GgufTensor of this file) as a uint8 tensor, memory-mapped from the file and uploaded when a
+        device is given."""
+        import numpy as np
+        raw = np.memmap(self.path, dtype=np.uint8, mode="r", offset=int(t.offset), shape=(int(t.bytes),))
+        host = torch.from_numpy(np.array(raw))
+        return host.to(device) if device is not None else host
+
+    def load_moe_layer(self, layer, top_k, max_rows, device="cuda", **layer_options):
+        """One MoE layer of the file on the device: (MoeLayer, router weight fp32 [experts][hidden], norm weight or None, map)."""
+        m = self.moe_layer_map(layer)
+        gate, up, down = (self.read(t, device) for t in (m.gate, m.up, m.down))
+        router = self.read(m.router, device).view(torch.float32).reshape(m.experts, m.hidden)
+        norm = self.read(m.norm, device).view(torch.float32) if m.norm.bytes else None
+        moe = MoeLayer(m.hidden, m.ffn, m.experts, top_k, gate, up, down, max_rows, gate_type=m.gate_type, down_type=m.down_type, **layer_options)
+        return moe, router, norm, m
+
+
 def device_bytes(t):
     """DeviceBytes of a tensor (None: the empty view)."""
     return DeviceBytes(0, 0) if t is None else DeviceBytes(t.data_ptr(), t.numel() * t.element_size())
@@ -149,6 +221,15 @@ def lib():
         L.mi355_a8_enqueue_down_activation_quantize.argtypes = [P, P, U, U, P]
         L.mi355_a8_enqueue_down_rawdots.argtypes = [P, P, U, P]
         L.mi355_a8_enqueue_down_rawdots_merge.argtypes = [P, P, P, P]
+        L.mi355_gguf_open.argtypes, L.mi355_gguf_open.restype = [C.c_char_p], P
+        L.mi355_gguf_close.argtypes, L.mi355_gguf_close.restype = [P], None
+        for name in ("tensor_count", "metadata_count", "alignment", "data_offset"):
+            f = getattr(L, "mi355_gguf_" + name)
+            f.argtypes, f.restype = [P], C.c_uint64
+        L.mi355_gguf_tensor_at.argtypes = [P, C.c_uint64, P]
+        L.mi355_gguf_find_tensor.argtypes = [P, C.c_char_p, P]
+        L.mi355_gguf_metadata.argtypes = [P, C.c_char_p, P, P, P, P, P]
+        L.mi355_gguf_moe_layer.argtypes = [P, U, P]
         L.mi355_executor_create.argtypes = [U, U, U]
         L.mi355_executor_create.restype = C.c_void_p
         L.mi355_executor_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
@@ -172,7 +253,9 @@ EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi3
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
            "mi355_moe_strided_enqueue_prologue", "mi355_moe_strided_enqueue_csr", "mi355_moe_strided_enqueue_project", "mi355_moe_strided_enqueue_down",
            "mi355_moe_strided_enqueue_merge", "mi355_moe_strided_enqueue_commit", "mi355_moe_strided_enqueue", "mi355_executor_create",
-           "mi355_executor_run", "mi355_executor_destroy"]
+           "mi355_executor_run", "mi355_executor_destroy", "mi355_gguf_open", "mi355_gguf_close", "mi355_gguf_tensor_count",
+           "mi355_gguf_metadata_count", "mi355_gguf_alignment", "mi355_gguf_data_offset", "mi355_gguf_tensor_at", "mi355_gguf_find_tensor",
+           "mi355_gguf_metadata", "mi355_gguf_moe_layer"]
 
 
 def require_gpu():

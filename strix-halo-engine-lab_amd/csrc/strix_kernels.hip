@@ -300,11 +300,11 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
         const uint32_t row = bid / neb;
         route_chain_block<KIND>(slots, a, row, (bid % neb) * 8U);
         if (!a.plan) return;
-        // hand-off between workgroups without cache-wide fences: the logits were stored write-through at device scope and
-        // are complete once the wave's store counter drains; the reader loads them at device scope
-        __builtin_amdgcn_s_waitcnt(0);
+        // hand-off between workgroups: the wave's logit stores happen before the barrier, the barrier before lane 0's
+        // ticket increment, which releases them at device scope; the workgroup that takes the row's last ticket acquires with
+        // the same operation, and its other lanes read the logits after the second barrier
         __syncthreads();
-        if (lane == 0) flag = __hip_atomic_fetch_add(&tickets[row], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == neb - 1U;
+        if (lane == 0) flag = __hip_atomic_fetch_add(&tickets[row], 1U, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == neb - 1U;
         __syncthreads();
         if (flag) {
             if (lane == 0) tickets[row] = 0;
@@ -344,9 +344,10 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
             }
         }
         // the row's last quantiser block publishes the row's status word (a row's 32-groups fill whole blocks: hidden % 256 == 0)
+        // (the flag words are read-modify-written by device-scope atomics only; the ticket orders them as above)
         const uint32_t r = g0 / groups;
-        __builtin_amdgcn_s_waitcnt(0);
-        if (lane == 0 && __hip_atomic_fetch_add(&tickets[16U + r], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups / 8U - 1U) {
+        __syncthreads();
+        if (lane == 0 && __hip_atomic_fetch_add(&tickets[16U + r], 1U, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == groups / 8U - 1U) {
             a.status[r] = __hip_atomic_load(flags + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             flags[r] = 0;
             tickets[16U + r] = 0;
@@ -1136,7 +1137,7 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
                                                                : "moe: down weights must be Q4_K (type 12), Q8_0 (type 8), Q5_1 (type 7) or Q6_K (type 14)");
     STRIX_REQUIRE(w->hidden >= 256 && w->hidden % 256U == 0, "moe: hidden must be a positive multiple of 256");
     // K-quant down rows are super-blocks of 256; the executor's block-of-32 formats need four chains of groups (src/cpu/core/routed_expert.hpp:22)
-    const uint32_t ffn_unit = (cls == kIntegerClass && (down_q8 || w->down_type == MI355_TYPE_Q5_1)) ? 128U : 256U;
+    const uint32_t ffn_unit = (cls != kPrefillClass && (down_q8 || w->down_type == MI355_TYPE_Q5_1)) ? 128U : 256U;
     STRIX_REQUIRE(w->ffn >= ffn_unit && w->ffn % ffn_unit == 0, "moe: ffn must be a positive multiple of 256 (Q8_0 / Q5_1 down rows: 128)");
     STRIX_REQUIRE(w->experts > 0 && w->experts <= kRouteMaxExperts, "moe: experts must be within 1..1024");
     STRIX_REQUIRE(w->top_k > 0 && w->top_k <= kRouteMaxTopK && w->top_k <= w->experts, "moe: top_k must be within 1..16 and <= experts");
@@ -1601,3 +1602,4 @@ int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float*
 
 #include "a8_contract.hpp"
 #include "rows_forms.hpp"
+#include "gguf_reader.hpp"
