@@ -127,9 +127,12 @@ typedef struct mi355_route_policy {
                                          (include/strix/moe/route_policy.hpp:146) */
     uint32_t exp_kind;                /* Math::exp of the softmax: MI355_EXP_DECLARED (include/strix/ds41_moe.hpp:38-54),
                                          MI355_EXP_LIBM or MI355_EXP_GFX1151 */
+    uint32_t shared_experts;          /* 0..4 always-on experts behind the routed ones: ids / weights rows are then
+                                         [top_k + shared_experts] wide, slot top_k + s holds expert id experts + s with weight 1
+                                         (the shared expert of a layer stored as one more expert of the same tensors) */
 } mi355_route_policy;
 /* x: [rows] activations (input_kind), row r at x + r * x_stride_bytes. router_weight: fp32 [experts][hidden].
- * logit_bias: fp32 [experts] or NULL. ids / weights: [rows][top_k]. scores: [rows][experts] workspace AND output. */
+ * logit_bias: fp32 [experts] or NULL. ids / weights: [rows][top_k + shared_experts]. scores: [rows][experts] workspace AND output. */
 int32_t mi355_moe_route(const mi355_route_policy* policy, const void* x, uint32_t input_kind, uint32_t rows,
                         uint32_t hidden, uint64_t x_stride_bytes, const float* router_weight, const float* logit_bias,
                         uint32_t* ids, float* weights, float* scores, mi355_stream stream);
@@ -217,6 +220,19 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights*, const mi355_moe_rows*, uint3
 int32_t mi355_moe_enqueue_layer(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
                                 float* scores, const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows,
                                 uint32_t combine_form, mi355_stream);
+
+/* The layer with the RMSNorm of its input inside the first launch (the reference normalises the residual stream in front of
+ * the MoE, src/ops/norm/norm.hpp:40-58, and runs the shared expert beside the routed ones, src/hip_shared_expert_launcher.hip):
+ * rows->input holds the raw rows; the router, the A8 image and the experts see y = (x * r) * norm_weight,
+ * r = 1 / sqrt(mean(x^2) + norm_eps), bit for bit mi355_rmsnorm_f32 (lane-strided fma chains, LDS halving) followed by
+ * mi355_moe_enqueue_layer on y; norm_weight may be NULL (unit scale). normed: fp32 [rows][hidden], receives y (the input of
+ * anything else that reads the normalised rows). For rows <= 16 every workgroup of the router / prologue launch derives its
+ * row's r itself, so no launch is added; larger batches run one norm launch first.
+ * A shared expert stored as expert `experts` of the same tensors is the policy's shared_experts = 1: every row then carries
+ * one more slot with weight 1, its gate / up / down rows are swept once per four rows, and the ordered combine adds it last. */
+int32_t mi355_moe_enqueue_layer_normed(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
+                                       float* scores, const float* norm_weight, float norm_eps, float* normed, const mi355_moe_weights*,
+                                       const mi355_moe_rows*, uint32_t rows, uint32_t combine_form, mi355_stream);
 
 /* mi355_moe_enqueue_layer with every work buffer inside the library. It has no counterpart in the reference: it is for
  * callers that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid

@@ -35,7 +35,7 @@ class Q8a8View(C.Structure):
 class RoutePolicy(C.Structure):
     _fields_ = [("experts", C.c_uint32), ("top_k", C.c_uint32), ("logits_order", C.c_uint32),
                 ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_uint32),
-                ("renorm_single", C.c_uint32), ("exp_kind", C.c_uint32)]
+                ("renorm_single", C.c_uint32), ("exp_kind", C.c_uint32), ("shared_experts", C.c_uint32)]
 
 
 class MoeWeights(C.Structure):
@@ -248,7 +248,7 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
            "mi355_moe_strided_enqueue_prologue", "mi355_moe_strided_enqueue_csr", "mi355_moe_strided_enqueue_project", "mi355_moe_strided_enqueue_down",
@@ -333,12 +333,12 @@ def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False,
 
 
 def route(x, router_weight, top_k, bias=None, logits_order=LOGITS_FMA, renorm_eps=0.0, scale=1.0, renormalize=True, renorm_single=True,
-          exp_kind=EXP_DECLARED):
+          exp_kind=EXP_DECLARED, shared_experts=0):
     rows, hidden = x.shape
     experts = router_weight.shape[0]
-    p = RoutePolicy(experts, top_k, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single), exp_kind)
-    ids = torch.empty((rows, top_k), dtype=torch.int32, device=x.device)
-    weights = torch.empty((rows, top_k), dtype=torch.float32, device=x.device)
+    p = RoutePolicy(experts, top_k, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single), exp_kind, shared_experts)
+    ids = torch.empty((rows, top_k + shared_experts), dtype=torch.int32, device=x.device)
+    weights = torch.empty((rows, top_k + shared_experts), dtype=torch.float32, device=x.device)
     scores = torch.empty((rows, experts), dtype=torch.float32, device=x.device)
     check(lib().mi355_moe_route(C.byref(p), _p(x), input_kind(x), rows, hidden, C.c_uint64(x.stride(0) * x.element_size()),
                                 _p(router_weight), _p(bias), _p(ids), _p(weights), _p(scores), _stream()))
@@ -489,17 +489,29 @@ class MoeLayer:
         return self.output[:rows]
 
     def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,
-                  scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED):
-        """Router + experts + combine through mi355_moe_enqueue_layer. Returns (output, ids, weights, scores)."""
+                  scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED, shared_experts=0, norm=None):
+        """Router + experts + combine through mi355_moe_enqueue_layer. Returns (output, ids, weights, scores).
+        shared_experts: the last `shared_experts` experts of the tensors are always on (the router picks among the others).
+        norm: (weight or None, eps) - the RMSNorm of x runs inside the first launch (mi355_moe_enqueue_layer_normed); the
+        normalised rows are left in self.normed."""
         rows = x.shape[0]
+        if router_weight.shape[0] != self.experts - shared_experts or router_weight.shape[1] != self.hidden:
+            raise StrixError(E_INVALID_ARGUMENT, "the router weight must be [experts - shared_experts][hidden]")
         if not hasattr(self, "ids") or self.ids.shape[0] < rows:
             self.ids = torch.zeros((self.max_rows, self.top_k), dtype=torch.int32, device=x.device)
             self.route_w = torch.zeros((self.max_rows, self.top_k), dtype=torch.float32, device=x.device)
             self.scores = torch.zeros((self.max_rows, self.experts), dtype=torch.float32, device=x.device)
         _, rv = self.rows_view(x, self.ids, self.route_w, base)
-        p = RoutePolicy(self.experts, self.top_k, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single), exp_kind)
-        check(lib().mi355_moe_enqueue_layer(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), C.byref(self.w), C.byref(rv), rows,
-                                            combine, _stream()))
+        p = RoutePolicy(self.experts - shared_experts, self.top_k - shared_experts, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single),
+                        exp_kind, shared_experts)
+        if norm is None:
+            check(lib().mi355_moe_enqueue_layer(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), C.byref(self.w), C.byref(rv), rows,
+                                                combine, _stream()))
+        else:
+            if not hasattr(self, "normed"):
+                self.normed = torch.zeros((self.max_rows, self.hidden), dtype=torch.float32, device=x.device)
+            check(lib().mi355_moe_enqueue_layer_normed(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), _p(norm[0]), C.c_float(norm[1]),
+                                                       _p(self.normed), C.byref(self.w), C.byref(rv), rows, combine, _stream()))
         return self.output[:rows], self.ids[:rows], self.route_w[:rows], self.scores[:rows]
 
     def run_layer_static(self, x, router_weight, ids, route_w, status, output, bias=None, base=None, combine=COMBINE_FMA_SLOT):

@@ -29,7 +29,33 @@ struct RouteArgs {
     // fused decode extras (all null / zero for the plain router)
     int8_t* codes; float* deltas; int32_t* sums; uint32_t* status; uint32_t* job_status; uint32_t* plan;
     uint32_t route_blocks, quant_blocks;
+    // RMSNorm of the input rows inside the launch (norm_on): the router and the A8 image see y = (x * r) * norm_w, r = 1 / sqrt(mean(x^2) + eps)
+    // in the declared order of src/cpu/core/reference.cpp:86-103; normed (optional) receives y as fp32 [rows][hidden]
+    uint32_t norm_on; const float* norm_w; float norm_eps; float* normed;
 };
+
+// r of one row by a 64-thread workgroup, bit for bit rmsnorm_f32_kernel: lane l of L = 256 (n >= 512) or 128 chains
+// fma(x, x, a) over x[l], x[l + L], ...; the L partial sums are halved in LDS; thread t stands for lanes t, t + 64, ...
+template <int KIND>
+__device__ __forceinline__ float row_norm_factor(float* partial /* 256 floats of LDS */, const uint8_t* xrow, uint32_t n, float eps) {
+    const uint32_t t = threadIdx.x & 63U, L = n >= 512U ? 256U : 128U;
+    for (uint32_t l = t; l < L; l += 64U) {
+        float a = 0.0F;
+        for (uint32_t i = l; i < n; i += L) {
+            const float v = load_activation<KIND>(xrow, i);
+            a = __builtin_fmaf(v, v, a);
+        }
+        partial[l] = a;
+    }
+    for (uint32_t h = L / 2U; h > 0; h >>= 1) {
+        __syncthreads();
+        for (uint32_t l = t; l < h; l += 64U) partial[l] = partial[l] + partial[l + h];
+    }
+    __syncthreads();
+    const float r = 1.0F / __builtin_sqrtf(partial[0] / static_cast<float>(n) + eps);
+    __syncthreads();
+    return r;
+}
 
 // ---------------------------------------------------------------------------------------------------- logit chains
 // Logits of 8 experts x 8 rows -> scores[row][expert] (used as the logit workspace). hidden % 32 == 0.
@@ -242,15 +268,25 @@ struct __attribute__((aligned(16))) ChainSlot {
     float w[kChainExperts][kChainPitch];
     float x[kChainChunk];                             // the row's features as fp32
     uint32_t raw[kChainChunk / 2];                    // fp16 / bf16 input as copied (unused for fp32 input)
+    float nw[kChainChunk];                            // the norm weights of the chunk (fused RMSNorm only)
 };
-template <int KIND> constexpr uint32_t chain_copies() { return 2U * kChainExperts + (KIND == 0 ? 2U : 1U); }
+template <int KIND, bool NORM = false> constexpr uint32_t chain_copies() { return 2U * kChainExperts + (KIND == 0 ? 2U : 1U) + (NORM ? 2U : 0U); }
 
 // Start the copy of features [k0, k0 + 512) of 8 router-weight rows and of the activation row. Every chunk issues the
 // same number of copy instructions (the waits count them): lanes past the end of the row re-fetch its last piece into
 // slot positions that are never read.
-template <int KIND>
+template <int KIND, bool NORM = false>
 __device__ __forceinline__ void chain_start(ChainSlot& slot, const RouteArgs& a, uint32_t row, uint32_t e0, uint32_t k0) {
     const uint32_t lane = threadIdx.x & 63U;
+    if constexpr (NORM) {       // (a null norm weight is a unit scale: the router weights stand in and are not used)
+        const float* nsrc = a.norm_w ? a.norm_w : a.wr;
+#pragma unroll
+        for (uint32_t j = 0; j < 2U; ++j) {
+            const uint32_t k = k0 + 256U * j + 4U * lane, kk = k + 4U <= a.hidden ? k : a.hidden - 4U;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(nsrc + kk),
+                                             (__attribute__((address_space(3))) void*)(&slot.nw[256U * j]), 16, 0, 0);
+        }
+    }
 #pragma unroll
     for (uint32_t i = 0; i < kChainExperts; ++i) {
         const uint32_t e = e0 + i < a.p.experts ? e0 + i : a.p.experts - 1U;
@@ -277,8 +313,21 @@ __device__ __forceinline__ void chain_start(ChainSlot& slot, const RouteArgs& a,
     }
 }
 // fp16 / bf16: widen the landed chunk to fp32 (8 features per lane).
-template <int KIND>
-__device__ __forceinline__ void chain_widen(ChainSlot& slot) {
+template <int KIND, bool NORM = false>
+__device__ __forceinline__ void chain_widen(ChainSlot& slot, float factor = 1.0F, bool scaled = false) {
+    if constexpr (KIND == 0 && NORM) {
+        // fp32 rows arrive as they are: scale them in place, y = (x * r) * w
+        const uint32_t lane = threadIdx.x & 63U;
+#pragma unroll
+        for (uint32_t j = 0; j < 2U; ++j) {
+            f32x4 v = *reinterpret_cast<const f32x4*>(&slot.x[256U * j + 4U * lane]);
+            const f32x4 w = *reinterpret_cast<const f32x4*>(&slot.nw[256U * j + 4U * lane]);
+            v.x = v.x * factor; v.y = v.y * factor; v.z = v.z * factor; v.w = v.w * factor;
+            if (scaled) { v.x = v.x * w.x; v.y = v.y * w.y; v.z = v.z * w.z; v.w = v.w * w.w; }
+            *reinterpret_cast<f32x4*>(&slot.x[256U * j + 4U * lane]) = v;
+        }
+        __syncthreads();
+    }
     if constexpr (KIND != 0) {
         const uint32_t lane = threadIdx.x & 63U;
         const u32x4 r = *reinterpret_cast<const u32x4*>(&slot.raw[4U * lane]);
@@ -288,6 +337,13 @@ __device__ __forceinline__ void chain_widen(ChainSlot& slot) {
         for (int q = 0; q < 4; ++q) {
             if constexpr (KIND == 1) { f[2 * q] = half_bits_to_float(h[q] & 0xffffU); f[2 * q + 1] = half_bits_to_float(h[q] >> 16); }
             else { f[2 * q] = f_of(h[q] << 16); f[2 * q + 1] = f_of(h[q] & 0xffff0000U); }
+        }
+        if constexpr (NORM) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                f[q] = f[q] * factor;
+                if (scaled) f[q] = f[q] * slot.nw[8U * lane + q];
+            }
         }
         *reinterpret_cast<f32x4*>(&slot.x[8U * lane]) = f32x4{f[0], f[1], f[2], f[3]};
         *reinterpret_cast<f32x4*>(&slot.x[8U * lane + 4U]) = f32x4{f[4], f[5], f[6], f[7]};
@@ -321,9 +377,9 @@ __device__ __forceinline__ void chain_wait() { __builtin_amdgcn_s_waitcnt((N & 1
 
 // Logits of experts [e0, e0 + 8) for one row -> scores[row][expert] (+ bias), stored for readers in other workgroups of
 // the same launch. hidden % 32 == 0. slots: 4 separate LDS objects.
-template <int KIND>
-__device__ __forceinline__ void route_chain_block(ChainSlot* const (&slots)[4], const RouteArgs& a, uint32_t row, uint32_t e0) {
-    constexpr uint32_t NI = chain_copies<KIND>();
+template <int KIND, bool NORM = false>
+__device__ __forceinline__ void route_chain_block(ChainSlot* const (&slots)[4], const RouteArgs& a, uint32_t row, uint32_t e0, float r = 1.0F) {
+    constexpr uint32_t NI = chain_copies<KIND, NORM>();
     const uint32_t lane = threadIdx.x & 63U, chunks = (a.hidden + kChainChunk - 1U) / kChainChunk;
     const bool butterfly = a.p.logits_order == MI355_LOGITS_LANE32_BUTTERFLY;
     const uint32_t el = lane & 7U;                      // chain form: the lane's expert
@@ -331,7 +387,7 @@ __device__ __forceinline__ void route_chain_block(ChainSlot* const (&slots)[4], 
     float acc = 0.0F, part[4] = {0.0F, 0.0F, 0.0F, 0.0F};
 #pragma unroll
     for (uint32_t s = 0; s < 3U; ++s)
-        if (s < chunks) chain_start<KIND>(*slots[s], a, row, e0, s * kChainChunk);
+        if (s < chunks) chain_start<KIND, NORM>(*slots[s], a, row, e0, s * kChainChunk);
     for (uint32_t c0 = 0; c0 < chunks; c0 += 4U) {
 #pragma unroll
         for (uint32_t s = 0; s < 4U; ++s) {
@@ -342,9 +398,9 @@ __device__ __forceinline__ void route_chain_block(ChainSlot* const (&slots)[4], 
                 if (ahead == 0) chain_wait<0>();
                 else if (ahead == 1) chain_wait<NI>();
                 else chain_wait<2 * NI>();
-                if (c + 3U < chunks) chain_start<KIND>(*slots[(s + 3U) % 4U], a, row, e0, (c + 3U) * kChainChunk);
+                if (c + 3U < chunks) chain_start<KIND, NORM>(*slots[(s + 3U) % 4U], a, row, e0, (c + 3U) * kChainChunk);
                 ChainSlot& slot = *slots[s];
-                chain_widen<KIND>(slot);
+                chain_widen<KIND, NORM>(slot, r, a.norm_w != nullptr);
                 const uint32_t kc = a.hidden - c * kChainChunk < kChainChunk ? a.hidden - c * kChainChunk : kChainChunk;
                 if (!butterfly) {
                     if (kc == kChainChunk) {      // full chunk: straight-line code, operands fetched 16 features ahead
@@ -425,10 +481,10 @@ __device__ __forceinline__ uint64_t key_max_wave(uint64_t key) {        // the w
     const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(key >> 32)), 63));
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
-// Returns, in lane k < top_k, the k-th selected expert.
+// Returns, in lane k < top_k + shared_experts, the expert of slot k.
 template <uint32_t PER>
 __device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const RouteArgs& a, uint32_t row) {
-    const uint32_t lane = threadIdx.x & 63U, E = a.p.experts, K = a.p.top_k;
+    const uint32_t lane = threadIdx.x & 63U, E = a.p.experts, K = a.p.top_k, P = K + a.p.shared_experts;
     float* z = a.scores + static_cast<size_t>(row) * E;
     float v[PER];
     float m = -INFINITY;
@@ -494,9 +550,13 @@ __device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const Rou
     }
     const float den = sum + a.p.renorm_eps;
     if (lane < K) {
-        a.ids[static_cast<size_t>(row) * K + lane] = my_id;
+        a.ids[static_cast<size_t>(row) * P + lane] = my_id;
         const bool renorm = a.p.renormalize && (K > 1U || a.p.renorm_single);      // include/strix/moe/route_policy.hpp:146
-        a.weights[static_cast<size_t>(row) * K + lane] = (renorm ? my_v / den : my_v) * a.p.scale;
+        a.weights[static_cast<size_t>(row) * P + lane] = (renorm ? my_v / den : my_v) * a.p.scale;
+    } else if (lane < P) {      // the always-on experts behind the routed ones: ids experts .. experts + shared - 1, weight 1
+        my_id = E + (lane - K);
+        a.ids[static_cast<size_t>(row) * P + lane] = my_id;
+        a.weights[static_cast<size_t>(row) * P + lane] = 1.0F;
     }
     __syncthreads();
     return my_id;

@@ -285,7 +285,7 @@ __global__ __launch_bounds__(256, 2) void route_batch_kernel(RouteArgs a) {
 // and the block that finishes a row's last 8 experts (row ticket) runs that row's softmax / top-k / weights and writes the
 // row's work items: a decode batch is planned one item per assignment (item i = assignment i, order = identity; the CSR
 // fields of the plan are not written), so nothing waits for the other rows. Every ticket word is left zero.
-template <int KIND>
+template <int KIND, bool NORM = false>
 __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
     __shared__ ChainSlot slot0;
     __shared__ ChainSlot slot1;
@@ -298,7 +298,9 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
     uint32_t* tickets = a.plan ? a.plan + kPlanTicketsAt : nullptr;
     if (bid < a.route_blocks) {
         const uint32_t row = bid / neb;
-        route_chain_block<KIND>(slots, a, row, (bid % neb) * 8U);
+        float r = 1.0F;
+        if constexpr (NORM) r = row_norm_factor<KIND>(sel_p, a.x + row * a.x_stride, a.hidden, a.norm_eps);
+        route_chain_block<KIND, NORM>(slots, a, row, (bid % neb) * 8U, r);
         if (!a.plan) return;
         // hand-off between workgroups: the wave's logit stores happen before the barrier, the barrier before lane 0's
         // ticket increment, which releases them at device scope; the workgroup that takes the row's last ticket acquires with
@@ -308,27 +310,50 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
         __syncthreads();
         if (flag) {
             if (lane == 0) tickets[row] = 0;
+            // The plan of a decode batch. Routed slots: position row * K + slot, one item per assignment. The always-on experts
+            // behind them (slot K + s, chosen by every row): positions rows * K + s * rows + row, one item per four rows, so
+            // their weights are swept once per four rows and not once per row.
             const uint32_t expert = route_select_row(sel_p, a, row);
-            if (lane < a.p.top_k) {
-                const uint32_t assignments = a.rows * a.p.top_k, i = row * a.p.top_k + lane;
-                *reinterpret_cast<uint4*>(a.plan + plan_items_at(a.p.experts, assignments) + 4U * i) = make_uint4(expert, i, i + 1U, 0U);
-                a.plan[plan_order_at(a.p.experts) + i] = i;
-            }
+            const uint32_t K = a.p.top_k, S = a.p.shared_experts, P = K + S, assignments = a.rows * P, all = a.p.experts + S;
+            uint32_t* items = a.plan + plan_items_at(all, assignments);
+            uint32_t* order = a.plan + plan_order_at(all);
+            if (lane < K) {
+                const uint32_t at = row * K + lane;
+                *reinterpret_cast<uint4*>(items + 4U * at) = make_uint4(expert, at, at + 1U, 0U);
+                order[at] = row * P + lane;
+            } else if (lane < P) order[a.rows * K + (lane - K) * a.rows + row] = row * P + lane;
         }
-        if (bid == 0 && lane == 0) {
-            const uint32_t assignments = a.rows * a.p.top_k;
-            *a.job_status = 0;
-            a.plan[0] = assignments; a.plan[1] = 0; a.plan[2] = 1; a.plan[4] = assignments;
+        if (bid == 0) {
+            const uint32_t K = a.p.top_k, S = a.p.shared_experts, P = K + S, assignments = a.rows * P, all = a.p.experts + S;
+            const uint32_t chunks = (a.rows + 3U) / 4U, made = a.rows * K + S * chunks;
+            uint32_t* items = a.plan + plan_items_at(all, assignments);
+            if (lane < S * chunks) {
+                const uint32_t s_ = lane / chunks, c = lane - s_ * chunks, first = a.rows * K + s_ * a.rows + 4U * c;
+                const uint32_t last = 4U * c + 4U < a.rows ? first + 4U : a.rows * K + s_ * a.rows + a.rows;
+                *reinterpret_cast<uint4*>(items + 4U * (a.rows * K + lane)) = make_uint4(a.p.experts + s_, first, last, 0U);
+            }
+            for (uint32_t i = made + lane; i < assignments; i += 64U) *reinterpret_cast<uint4*>(items + 4U * i) = make_uint4(0U, 0U, 0U, 0U);
+            if (lane == 0) {
+                *a.job_status = 0;
+                a.plan[0] = assignments; a.plan[1] = 0; a.plan[2] = S ? 4U : 1U; a.plan[4] = made;
+            }
         }
     } else {
         // A8 prologue (src/cpu/core/reference.cpp:35-55): two groups of 32 at a time, 8 groups per block
         const uint32_t groups = a.hidden / 32U, total = a.rows * groups, g0 = (bid - a.route_blocks) * 8U;
         uint32_t* flags = tickets + 128U;
+        float factor = 1.0F;         // (a block's eight groups belong to one row: hidden % 256 == 0)
+        if constexpr (NORM) factor = row_norm_factor<KIND>(sel_p, a.x + (g0 / groups) * a.x_stride, a.hidden, a.norm_eps);
         for (uint32_t i = 0; i < 8U; i += 2U) {
             const uint32_t g = g0 + i + (lane >> 5), j = lane & 31U;
             if (g < total) {
                 const uint32_t r = g / groups, gi = g % groups;
-                const float v = load_activation<KIND>(a.x + r * a.x_stride, gi * 32U + j);
+                float v = load_activation<KIND>(a.x + r * a.x_stride, gi * 32U + j);
+                if constexpr (NORM) {
+                    v = v * factor;
+                    if (a.norm_w) v = v * a.norm_w[gi * 32U + j];
+                    if (a.normed) a.normed[static_cast<size_t>(r) * a.hidden + gi * 32U + j] = v;
+                }
                 const float amax = max32(__builtin_fabsf(v));
                 const bool tiny = amax > 0.0F && amax < 0x1p-119F;
                 const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
@@ -1057,12 +1082,13 @@ constexpr uint32_t kQuadMaxItems = 48;
 inline bool quad_sweep(const mi355_moe_weights& w, uint32_t rows) {
     return rows <= kFusedMaxRows && rows * w.top_k <= kQuadMaxItems && w.experts > 1U;
 }
-inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+// grouped: the plan's items hold several assignments (the one-assignment sweeps do not apply)
+inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st, bool grouped = false) {
     if (w.gate_type == MI355_TYPE_Q5_K) {
         project_q5k_kernel<<<dim3(w.ffn / 32U, umax), 256, 0, st>>>(w, r, rows * w.top_k);
         return;
     }
-    if (quad_sweep(w, rows)) {
+    if (!grouped && quad_sweep(w, rows)) {
         const uint32_t items = rows * w.top_k;
         if (items <= 16U) project_quad_kernel<4><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, r, items);
         else project_quad_kernel<2><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, r, items);
@@ -1073,7 +1099,7 @@ inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t 
     if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
     else launch_project_nb<4>(w, r, rows, grid, st);
 }
-inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st) {
+inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st, bool grouped = false) {
     if (w.down_type != MI355_TYPE_Q4_K) {      // Q8_0 / Q5_1 (blocks of 32, four chains per row) and Q6_K (pairs per super-block)
         const uint32_t assignments = rows * w.top_k, items_at = plan_items_at(w.experts, assignments), order_at = plan_order_at(w.experts);
         const dim3 grid(w.hidden / kDownGroupsRows, umax);
@@ -1082,7 +1108,7 @@ inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t row
         else down_q6k_kernel<<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         return;
     }
-    if (quad_sweep(w, rows)) {
+    if (!grouped && quad_sweep(w, rows)) {
         const uint32_t items = rows * w.top_k;
         if (items <= 16U) down_quad_kernel<4><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
         else down_quad_kernel<2><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
@@ -1309,6 +1335,8 @@ int32_t check_route(const mi355_route_policy* p, const void* x, uint32_t kind, u
     STRIX_REQUIRE(p && x && wr && ids && weights && scores, "route: null pointer");
     STRIX_REQUIRE(p->experts > 0 && p->experts <= kRouteMaxExperts && p->top_k > 0 && p->top_k <= kRouteMaxTopK && p->top_k <= p->experts,
                   "route policy: need 0 < top_k <= experts, experts <= 1024, top_k <= 16");
+    STRIX_REQUIRE(p->shared_experts <= 4U && p->top_k + p->shared_experts <= kRouteMaxTopK && p->experts + p->shared_experts <= kRouteMaxExperts,
+                  "route policy: at most 4 always-on experts, top_k + shared <= 16, experts + shared <= 1024");
     STRIX_REQUIRE(hidden > 0 && hidden <= kRouteMaxHidden && hidden % 32U == 0, "route: hidden must be a multiple of 32 within 16384");
     STRIX_REQUIRE(kind <= MI355_INPUT_BF16 && p->logits_order <= MI355_LOGITS_LANE32_BUTTERFLY, "route: unknown input kind or logits order");
     STRIX_REQUIRE(p->exp_kind <= MI355_EXP_LIBM, "route policy: unknown exp kind");
@@ -1322,7 +1350,11 @@ void launch_route_logits(RouteArgs& a, hipStream_t st) {
     if (a.rows <= kFusedMaxRows) {
         a.route_blocks = neb * a.rows;
         const uint32_t blocks = a.route_blocks + a.quant_blocks;
-        if (a.kind == MI355_INPUT_F32) route_decode_kernel<0><<<blocks, 64, 0, st>>>(a);
+        if (a.norm_on) {
+            if (a.kind == MI355_INPUT_F32) route_decode_kernel<0, true><<<blocks, 64, 0, st>>>(a);
+            else if (a.kind == MI355_INPUT_F16) route_decode_kernel<1, true><<<blocks, 64, 0, st>>>(a);
+            else route_decode_kernel<2, true><<<blocks, 64, 0, st>>>(a);
+        } else if (a.kind == MI355_INPUT_F32) route_decode_kernel<0><<<blocks, 64, 0, st>>>(a);
         else if (a.kind == MI355_INPUT_F16) route_decode_kernel<1><<<blocks, 64, 0, st>>>(a);
         else route_decode_kernel<2><<<blocks, 64, 0, st>>>(a);
     } else if (a.p.logits_order == MI355_LOGITS_FMA_ASCENDING && (a.rows + kBatchTile - 1U) / kBatchTile <= 65535U) {
@@ -1417,8 +1449,26 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, u
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
 
-int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
-                                const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+}  // extern "C"
+
+namespace {
+// RMSNorm of rows of any input kind into fp32 rows (the staged form of the fused norm): rmsnorm_f32_kernel's order.
+template <int KIND>
+__global__ __launch_bounds__(64) void rmsnorm_rows_kernel(const uint8_t* x, uint64_t x_stride, const float* w, uint32_t n, float eps, float* y) {
+    __shared__ float partial[256];
+    const uint8_t* xr = x + blockIdx.x * x_stride;
+    const float r = row_norm_factor<KIND>(partial, xr, n, eps);
+    float* yr = y + static_cast<size_t>(blockIdx.x) * n;
+    for (uint32_t i = threadIdx.x; i < n; i += 64U) {
+        const float v = load_activation<KIND>(xr, i) * r;
+        yr[i] = w ? v * w[i] : v;
+    }
+}
+
+struct LayerNorm { bool on; const float* weight; float eps; float* normed; };
+
+int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores, const LayerNorm& norm,
+                      const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
@@ -1426,33 +1476,68 @@ int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router
     uint32_t* ids = const_cast<uint32_t*>(r->routes);
     float* weights = const_cast<float*>(r->route_weights);
     if (const int32_t rc = check_route(p, r->input, r->input_kind, wv.hidden, r->input_stride, router_weight, ids, weights, scores)) return rc;
-    STRIX_REQUIRE(p->experts == wv.experts && p->top_k == wv.top_k, "moe layer: router policy and expert tensors disagree on experts / top_k");
+    STRIX_REQUIRE(p->experts + p->shared_experts == wv.experts && p->top_k + p->shared_experts == wv.top_k,
+                  "moe layer: router policy (experts, top_k, always-on experts) and expert tensors disagree on experts / top_k");
+    STRIX_REQUIRE(!norm.on || (norm.normed && aligned(norm.normed, 16) && (!norm.weight || aligned(norm.weight, 16)) && norm.eps >= 0.0F),
+                  "moe layer: the fused RMSNorm needs a 16-byte aligned fp32 [rows][hidden] view for the normalised rows, aligned weights, eps >= 0");
+    hipStream_t st = hs(stream);
     if (rows > kFusedMaxRows || plan_split(wv, rows) != 1U) {      // large batches, and decode batches over large experts (shared sweeps): router, then the staged prologue / plan
-        if (const int32_t rc = mi355_moe_route(p, r->input, r->input_kind, rows, wv.hidden, r->input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
-        return mi355_moe_enqueue(w, r, rows, form, stream);
+        mi355_moe_rows staged = *r;
+        if (norm.on) {
+            const uint8_t* x = static_cast<const uint8_t*>(r->input);
+            if (r->input_kind == MI355_INPUT_F32) rmsnorm_rows_kernel<0><<<rows, 64, 0, st>>>(x, r->input_stride, norm.weight, wv.hidden, norm.eps, norm.normed);
+            else if (r->input_kind == MI355_INPUT_F16) rmsnorm_rows_kernel<1><<<rows, 64, 0, st>>>(x, r->input_stride, norm.weight, wv.hidden, norm.eps, norm.normed);
+            else rmsnorm_rows_kernel<2><<<rows, 64, 0, st>>>(x, r->input_stride, norm.weight, wv.hidden, norm.eps, norm.normed);
+            STRIX_LAUNCHED("moe layer norm");
+            staged.input = norm.normed; staged.input_kind = MI355_INPUT_F32; staged.input_stride = 4ULL * wv.hidden;
+        }
+        if (const int32_t rc = mi355_moe_route(p, staged.input, staged.input_kind, rows, wv.hidden, staged.input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
+        return mi355_moe_enqueue(w, &staged, rows, form, stream);
     }
     RouteArgs a{};
     a.p = *p; a.x = static_cast<const uint8_t*>(r->input); a.kind = r->input_kind; a.x_stride = r->input_stride; a.rows = rows; a.hidden = wv.hidden;
     a.wr = router_weight; a.bias = logit_bias; a.ids = ids; a.weights = weights; a.scores = scores;
     a.codes = r->codes; a.deltas = r->deltas; a.sums = r->sums; a.status = r->status; a.job_status = r->job_status; a.plan = r->plan;
     a.quant_blocks = (rows * (wv.hidden / 32U) + 7U) / 8U;
-    launch_route_logits(a, hs(stream));
+    a.norm_on = norm.on ? 1U : 0U; a.norm_w = norm.weight; a.norm_eps = norm.eps; a.normed = norm.normed;
+    launch_route_logits(a, st);
     STRIX_LAUNCHED("moe layer router");
-    // the fused router planned one item per assignment
+    // the fused router planned one item per routed assignment (and one per four rows of an always-on expert)
     const uint32_t items = rows * wv.top_k;
-    launch_project(wv, rows_k(*r, wv), rows, items, hs(stream));
+    if (p->shared_experts) {       // items of several rows: the 64-row sweeps
+        launch_project(wv, rows_k(*r, wv), rows, items, st, true);
+        STRIX_LAUNCHED("moe layer gate / up");
+        launch_down(wv, rows_k(*r, wv), rows, items, st, true);
+        STRIX_LAUNCHED("moe layer experts");
+        return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+    }
+    launch_project(wv, rows_k(*r, wv), rows, items, st);
     // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
     // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
     // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
     if (!quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
         (wv.hidden / 64U) * rows <= compute_units()) {
-        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, hs(stream)>>>(wv, rows_k(*r, wv), items, form);
+        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
-    launch_down(wv, rows_k(*r, wv), rows, items, hs(stream));
+    launch_down(wv, rows_k(*r, wv), rows, items, st);
     STRIX_LAUNCHED("moe layer experts");
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+}
+}  // namespace
+
+extern "C" {
+
+int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
+                                const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    return enqueue_layer(p, router_weight, logit_bias, scores, LayerNorm{false, nullptr, 0.0F, nullptr}, w, r, rows, form, stream);
+}
+
+int32_t mi355_moe_enqueue_layer_normed(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
+                                       const float* norm_weight, float norm_eps, float* normed, const mi355_moe_weights* w, const mi355_moe_rows* r,
+                                       uint32_t rows, uint32_t form, mi355_stream stream) {
+    return enqueue_layer(p, router_weight, logit_bias, scores, LayerNorm{true, norm_weight, norm_eps, normed}, w, r, rows, form, stream);
 }
 
 int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {

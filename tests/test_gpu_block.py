@@ -1,0 +1,115 @@
+"""The MoE block around the routed experts: the RMSNorm of the input inside the router / prologue launch
+(mi355_moe_enqueue_layer_normed; the reference normalises in front of the MoE, src/ops/norm/norm.hpp:40-58, declared order
+src/cpu/core/reference.cpp:86-103) and the shared expert as an always-on expert of the same launches (policy.shared_experts).
+Bit for bit the oracle composition rmsnorm -> route -> A8 -> experts -> ordered combine."""
+import numpy as np
+import pytest
+import torch
+
+import orc
+from test_gpu_parity import bits, dev, make_layer
+from test_gpu_a8_contract import make_down
+
+pytestmark = pytest.mark.gpu
+DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+def layer_tensors(rng, H, I, E, gate_type, down_type):
+    if gate_type == orc.Q5_K:
+        gate, up = orc.random_q5_k(rng, (E, I), H), orc.random_q5_k(rng, (E, I), H)
+    else:
+        gate = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32))
+        up = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32))
+    return gate, up, make_down(rng, down_type, E, H, I)
+
+
+@pytest.mark.parametrize("kind,H,I,E,K,T,scaled", [
+    ("f16", 2048, 768, 128, 8, 8, True),            # config 3 with the norm in front
+    ("bf16", 2048, 768, 128, 8, 1, True),
+    ("f32", 1024, 512, 16, 4, 16, True),
+    ("f32", 1024, 512, 16, 4, 3, False),            # unit scale (no norm weight)
+    ("bf16", 256, 256, 8, 2, 5, True),              # 128 lanes in the norm's reduction (n < 512)
+    ("f16", 1280, 512, 16, 4, 7, True),             # a last, partial chunk of the router chain (1280 = 2 * 512 + 256)
+    ("f16", 1024, 512, 16, 4, 24, True),            # beyond the fused batch: norm launch, then the staged layer
+    ("bf16", 2048, 768, 128, 8, 40, False)])
+def test_rmsnorm_inside_the_layer_entry(strix, kind, H, I, E, K, T, scaled):
+    rng = np.random.default_rng(H + 3 * T + E)
+    gate, up, down = layer_tensors(rng, H, I, E, orc.Q4_K, orc.Q4_K)
+    x_t = torch.from_numpy((rng.standard_normal((T, H)) * 3.0).astype(np.float32)).to(DT[kind])
+    x32 = x_t.to(torch.float32).numpy()
+    nw = (1.0 + 0.2 * rng.standard_normal(H)).astype(np.float32) if scaled else None
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    eps = 1e-6
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, intermediates=True)
+    y, ids, wts, _ = layer.run_layer(x_t.cuda(), dev(wr), norm=(dev(nw) if scaled else None, eps))
+    torch.cuda.synchronize()
+    want_n = orc.rmsnorm_f32(x32, nw, eps)
+    assert np.array_equal(bits(layer.normed[:T].cpu().numpy()), bits(want_n))
+    ids_ref, w_ref, _, _ = orc.route(want_n, wr, K)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    c, d, s, _ = orc.quantize_a8(want_n)
+    assert np.array_equal(layer.codes[:T].cpu().numpy(), c) and np.array_equal(bits(layer.deltas[:T].cpu().numpy()), bits(d))
+    ref = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref)
+    assert np.array_equal(bits(layer.rawdots[:T].cpu().numpy()), bits(ref.rawdots))
+    assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine(0, w_ref, ids_ref, ref.rawdots)))
+    assert np.all(layer.status[:T].cpu().numpy() == 0)
+    # the standalone kernel gives the same rows
+    if kind == "f32":
+        assert np.array_equal(bits(strix.rmsnorm_f32(x_t.cuda(), dev(nw) if scaled else None, eps).cpu().numpy()), bits(want_n))
+
+
+@pytest.mark.parametrize("gate_type,down_type,H,I,E,K,S,T", [
+    (orc.Q4_K, orc.Q4_K, 2048, 768, 128, 8, 1, 8),       # config 3 plus a shared expert: nine slots, 64 + 2 work items
+    (orc.Q4_K, orc.Q4_K, 1024, 512, 16, 4, 1, 1),
+    (orc.Q4_K, orc.Q4_K, 1024, 512, 16, 4, 1, 6),        # two four-row items for the shared expert, the second of two rows
+    (orc.Q5_K, orc.Q8_0, 1024, 512, 16, 4, 1, 16),
+    (orc.Q4_K, orc.Q6_K, 512, 768, 6, 3, 2, 5),          # two always-on experts
+    (orc.Q4_K, orc.Q5_1, 1024, 384, 8, 2, 1, 9),
+    (orc.Q4_K, orc.Q4_K, 1024, 512, 16, 4, 1, 24)])      # the staged path: router, plan kernel
+def test_shared_expert_as_an_always_on_slot(strix, gate_type, down_type, H, I, E, K, S, T):
+    rng = np.random.default_rng(H + 5 * T + S + down_type)
+    gate, up, down = layer_tensors(rng, H, I, E + S, gate_type, down_type)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    layer = strix.MoeLayer(H, I, E + S, K + S, dev(gate), dev(up), dev(down), T, intermediates=True, gate_type=gate_type, down_type=down_type)
+    y, ids, wts, _ = layer.run_layer(dev(x), dev(wr), shared_experts=S)
+    torch.cuda.synchronize()
+    ids_r, w_r, _, _ = orc.route(x.astype(np.float32), wr, K)
+    ids_ref = np.concatenate([ids_r, np.tile(np.arange(E, E + S, dtype=np.uint32), (T, 1))], axis=1)
+    w_ref = np.concatenate([w_r, np.ones((T, S), np.float32)], axis=1)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    ref = orc.routed_experts(H, I, K + S, gate, up, down, down_type, c, d, s, ids_ref, gate_type=gate_type)
+    n = T * (K + S)
+    assert np.array_equal(bits(layer.gate_out[:n].cpu().numpy()), bits(ref.gate))
+    assert np.array_equal(layer.down_codes[:n].cpu().numpy(), ref.h_codes)
+    assert np.array_equal(bits(layer.rawdots[:T].cpu().numpy()), bits(ref.rawdots))
+    assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine(0, w_ref, ids_ref, ref.rawdots)))
+    assert np.all(layer.status[:T].cpu().numpy() == 0)
+    # the router alone writes the same rows
+    ids2, w2, _ = strix.route(dev(x), dev(wr), K, shared_experts=S)
+    assert np.array_equal(ids2.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(w2.cpu().numpy()), bits(w_ref))
+
+
+def test_block_norm_and_shared_expert_together_and_admission(strix):
+    H, I, E, K, S, T = 2048, 768, 32, 4, 1, 8
+    rng = np.random.default_rng(99)
+    gate, up, down = layer_tensors(rng, H, I, E + S, orc.Q4_K, orc.Q4_K)
+    x = (rng.standard_normal((T, H)) * 2.0).astype(np.float16)
+    nw = (1.0 + 0.2 * rng.standard_normal(H)).astype(np.float32)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    residual = rng.standard_normal((T, H)).astype(np.float32)
+    layer = strix.MoeLayer(H, I, E + S, K + S, dev(gate), dev(up), dev(down), T)
+    y, ids, wts, _ = layer.run_layer(dev(x), dev(wr), shared_experts=S, norm=(dev(nw), 1e-5), base=dev(residual))
+    want_n = orc.rmsnorm_f32(x.astype(np.float32), nw, 1e-5)
+    ids_r, w_r, _, _ = orc.route(want_n, wr, K)
+    ids_ref = np.concatenate([ids_r, np.full((T, 1), E, np.uint32)], axis=1)
+    w_ref = np.concatenate([w_r, np.ones((T, 1), np.float32)], axis=1)
+    c, d, s, _ = orc.quantize_a8(want_n)
+    ref = orc.routed_experts(H, I, K + S, gate, up, down, orc.Q4_K, c, d, s, ids_ref)
+    assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine(0, w_ref, ids_ref, ref.rawdots, base=residual)))
+    # the policy and the tensors must agree on the always-on experts
+    with pytest.raises(strix.StrixError):
+        layer.run_layer(dev(x), dev(wr), shared_experts=0)
+    with pytest.raises(strix.StrixError):
+        strix.route(dev(x), dev(wr), K, shared_experts=5)
