@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0     # MI355X published HBM3E peak
 MFMA_F16_PEAK_FLOPS = 2.5e15     # MI355X published dense fp16 MFMA peak
 # HBM bytes per launch of the gate/up kernel on the default workload, from two rocprofv3 --pmc passes (FETCH_SIZE scaled
 # x2.000, WRITE_SIZE x1.000 by a 256 MiB device copy in the same runs): profiles/project_wave_kernel_config3_moe_decode_T8.txt
-PROJECT_TRAFFIC_BYTES_DEFAULT = 99_892_019 + 147_661
+PROJECT_TRAFFIC_BYTES_DEFAULT = 99_723_264 + 147_466
 Q4K_ROW = lambda k: k // 256 * 144
 
 

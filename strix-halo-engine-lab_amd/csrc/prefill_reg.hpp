@@ -297,8 +297,12 @@ __global__ __launch_bounds__(kRgThreads) void prefill_reg_kernel(PrefillArgs a, 
         for (uint32_t i = 0; i < LIVE; ++i)
 #pragma unroll
             for (uint32_t k = 0; k < 8U; ++k) {
-                const float sent = gate_lane ? acc[i][8U + k] : acc[i][k], got = xor16_f(sent);
-                const float g = gate_lane ? acc[i][k] : got, u = gate_lane ? got : acc[i][8U + k];
+                // (the two registers are named before the per-lane choice: choosing the INDEX per lane instead would make the
+                // compiler walk all sixteen registers of the tile with compare-and-select pairs)
+                float first = acc[i][k], second = acc[i][8U + k];
+                asm volatile("" : "+v"(first), "+v"(second));
+                const float sent = gate_lane ? second : first, got = xor16_f(sent);
+                const float g = gate_lane ? first : got, u = gate_lane ? got : second;
                 const uint32_t r = gate_lane ? k : 8U + k;
                 const uint32_t t = 32U * i + 8U * (r / 4U) + 4U * half + (r & 3U);
                 const bool live = t < count;

@@ -197,6 +197,8 @@ __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v) {
     float lane[RB];
 #pragma unroll
     for (int r = 0; r < RB; ++r) lane[r] = 0.0F;
+    // (unrolled: the loads of four of the lane's groups are in flight together; the accumulation order does not change)
+#pragma unroll 4
     for (uint32_t g = l; g < groups; g += 32U) {
         const unsigned short* b = reinterpret_cast<const unsigned short*>(wrow + static_cast<size_t>(g) * kQ80Block);
         const float scale = half_bits_to_float(b[0]);

@@ -8,6 +8,8 @@
 //   * expert::Executor is constructed with its capacity (max assignments, max ffn) instead of a thread count.
 // Interfaces:
 //   cpu::Q8a8View / Stream / Kernels            src/cpu/core/backend.hpp:52-73
+//   weight::Candidate / Plan / WeightView / KernelArguments / enqueue / enqueue_dense   include/strix/weight/resolve.hpp:67-84,
+//                                                                                     src/cpu/weight/registry.cpp:11-63
 //   moe_q4k_a8::Request .. Bindings, validate, enqueue_probe                          include/strix/moe_q4k_a8_contract.hpp:101-122,
 //                                                                                     include/strix/hip_moe_q4k_a8_probe.hpp:12
 //   moe_q4k_a8::DownRequest .. DownBindings, validate_down, enqueue_down_*, SlotMergeTail   include/strix/moe_a8_down_contract.hpp:39-54,
@@ -24,6 +26,7 @@
 #include <stdexcept>
 #include <string>
 #include <string_view>
+#include <type_traits>
 
 #include "mi355_strix.h"
 
@@ -59,6 +62,90 @@ inline const Kernels& mi355_kernels() noexcept {
     return table;
 }
 }  // namespace cpu
+
+// ---------------------------------------------------------------------------------------------- typed weight-operator registry
+// The checked launch envelope of the reference's weight registry (Candidate / Plan / WeightView / KernelArguments / enqueue,
+// include/strix/weight/types.hpp:18-64, include/strix/weight/resolve.hpp:67-84) with the one registration the CPU backend
+// makes, the raw Q8_0 tree32 product (src/cpu/weight/registry.cpp:11-63, src/cpu/weight/source.hpp:17-38): the same kernel id,
+// storage / arithmetic / image ids, schema and ABI revision, and the same refusals in the same order (a plan that does not
+// select this kernel and arithmetic: unsupported_arithmetic; an envelope of another schema, revision or size: malformed; a
+// null operand: malformed; dimensions or strides: unsupported_shape), Status instead of exceptions. The payload is device
+// memory; output replaces view.out as in the reference's dispatch.
+namespace weight {
+using TensorId = std::uint64_t;
+using KernelId = std::uint64_t;
+struct Id { std::string_view name; std::uint32_t revision; };
+inline bool operator==(Id a, Id b) noexcept { return a.revision == b.revision && a.name == b.name; }
+using FormatId = Id; using ArithmeticId = Id; using ImageId = Id;
+enum class Backend : std::uint8_t { hip, cuda, cpu, intel };
+enum class Exactness : std::uint8_t { legacy_bitwise, operand_exact, fast };
+enum class Strategy : std::uint8_t { native, staged, converted, onfly };
+enum class Error : std::uint8_t { ok, unknown_format, malformed, unsupported_role, unsupported_shape, unsupported_backend, unsupported_arithmetic,
+                                  unavailable_isa, memory_budget, unqualified, stale_source, device_failure };
+struct Status { Error code; std::string detail; explicit operator bool() const { return code == Error::ok; } };
+struct Shape { std::uint64_t dims[4]; std::uint8_t rank; };
+struct WeightView { TensorId tensor; FormatId storage; Shape shape; const std::uint8_t* payload; std::uint64_t payload_bytes; };   // payload: device memory
+struct Candidate { KernelId kernel; FormatId storage; ArithmeticId arithmetic; ImageId image; Backend backend; Strategy strategy; Exactness exactness; };
+struct Plan { Candidate selected; };
+struct KernelArguments { KernelId schema; std::uint32_t abi_revision; const void* data; std::size_t bytes; };
+template <class Args> struct ArgumentTraits;
+template <class Args> KernelArguments arguments(Args& args) {
+    using Type = std::remove_cv_t<Args>;
+    static_assert(std::is_standard_layout_v<Type> && std::is_trivially_copyable_v<Type>);
+    return {ArgumentTraits<Type>::schema, ArgumentTraits<Type>::abi_revision, &args, sizeof(Type)};
+}
+template <class Args> KernelArguments arguments(const Args&&) = delete;
+
+inline constexpr KernelId q8_tree32_kernel = 0x43505501;
+struct DenseArguments { cpu::Q8a8View view; cpu::Stream stream; };
+template <> struct ArgumentTraits<DenseArguments> {
+    static constexpr KernelId schema = q8_tree32_kernel;
+    static constexpr std::uint32_t abi_revision = 2;
+};
+inline const Candidate* candidates(std::size_t& count) noexcept {
+    static const Candidate entries[] = {{q8_tree32_kernel, {"gguf.q8_0", 1}, {"cpu-q8a8-tree32", 1}, {"cpu.q8-raw", 1}, Backend::hip, Strategy::native,
+                                         Exactness::legacy_bitwise}};
+    count = 1;
+    return entries;
+}
+inline Status validate_view(const cpu::Q8a8View& view) {
+    if (!view.weight || !view.codes || !view.deltas || !view.out) return {Error::malformed, "Q8 launch has null operand"};
+    if (!view.in || !view.count || !view.rows || view.in % 32U || view.x_stride % 32U || view.x_stride < view.in ||
+        static_cast<std::uint64_t>(view.in / 32U) * 34U > view.row_bytes || view.out_stride < view.count)
+        return {Error::unsupported_shape, "Q8 launch dimensions/strides"};
+    return {Error::ok, {}};
+}
+// weight: [count][in] Q8_0 rows (dims fastest first: in, count)
+inline Status validate_q8_shape(const WeightView& weight, std::uint64_t count, std::uint64_t in) {
+    if (!(weight.storage == FormatId{"gguf.q8_0", 1})) return {Error::unknown_format, "weight is not raw Q8_0"};
+    if (weight.shape.rank != 2 || weight.shape.dims[0] != in || weight.shape.dims[1] != count) return {Error::unsupported_shape, "Q8 weight shape differs from the launch"};
+    if (!weight.payload || weight.payload_bytes < count * (in / 32U) * 34U) return {Error::malformed, "Q8 weight payload shorter than its shape"};
+    return {Error::ok, {}};
+}
+inline Status enqueue(const Plan& plan, const WeightView& weight, const KernelArguments& envelope, void* output, void* /*workspace*/, std::size_t /*workspace_bytes*/) {
+    if (plan.selected.kernel != q8_tree32_kernel || !(plan.selected.arithmetic == ArithmeticId{"cpu-q8a8-tree32", 1}) || plan.selected.strategy != Strategy::native)
+        return {Error::unsupported_arithmetic, "the registry only provides the raw Q8_0 tree32 incumbent"};
+    if (envelope.schema != q8_tree32_kernel || envelope.abi_revision != 2 || envelope.bytes != sizeof(DenseArguments) || !envelope.data)
+        return {Error::malformed, "Q8 typed launch schema/ABI"};
+    const DenseArguments& args = *static_cast<const DenseArguments*>(envelope.data);
+    cpu::Q8a8View view = args.view;
+    view.out = static_cast<float*>(output);
+    view.weight = weight.payload;
+    Status status = validate_view(view);
+    if (!status) return status;
+    status = validate_q8_shape(weight, view.count, view.in);
+    if (!status) return status;
+    const std::int32_t rc = mi355_gemv_q8_0_a8(&view, args.stream.stream);
+    if (rc != MI355_OK) return {rc == MI355_E_HIP ? Error::device_failure : Error::unsupported_shape, mi355_last_error()};
+    return {Error::ok, {}};
+}
+inline Status enqueue_dense(const WeightView& weight, const DenseArguments& args) {
+    std::size_t n;
+    Plan plan{candidates(n)[0]};
+    DenseArguments launch = args;
+    return enqueue(plan, weight, arguments(launch), args.view.out, nullptr, 0);
+}
+}  // namespace weight
 
 // ---------------------------------------------------------------------------------------------- A8 request / bindings
 namespace moe_q4k_a8 {

@@ -96,6 +96,31 @@ static void kernel_table() {
     bool threw = false;
     try { k.quantize_a8(dx.p, 33, dc.p, dd.p, ds.p); } catch (const std::invalid_argument&) { threw = true; }
     expect(threw, "Kernels::quantize_a8 throws std::invalid_argument for width % 32 != 0");
+
+    // the same product through the typed registry envelope
+    namespace wt = m::weight;
+    Dev<float> dout2(count);
+    const wt::WeightView weight{7, {"gguf.q8_0", 1}, wt::Shape{{width, count, 0, 0}, 2}, dw.p, w.size()};
+    wt::DenseArguments args{view, m::cpu::Stream{}};
+    args.view.out = dout2.p;
+    expect(static_cast<bool>(wt::enqueue_dense(weight, args)) && same_bits(dout2.get(), want), "weight::enqueue_dense (typed envelope) == oracle");
+    std::size_t n = 0;
+    wt::Plan plan{wt::candidates(n)[0]};
+    wt::KernelArguments envelope = wt::arguments(args);
+    envelope.abi_revision = 1;
+    expect(wt::enqueue(plan, weight, envelope, dout2.p, nullptr, 0).code == wt::Error::malformed, "weight::enqueue refuses an envelope of another ABI revision: malformed");
+    envelope = wt::arguments(args);
+    plan.selected.arithmetic = wt::ArithmeticId{"cpu-q8a8-tree32", 2};
+    expect(wt::enqueue(plan, weight, envelope, dout2.p, nullptr, 0).code == wt::Error::unsupported_arithmetic, "weight::enqueue refuses another arithmetic: unsupported_arithmetic");
+    plan = wt::Plan{wt::candidates(n)[0]};
+    wt::DenseArguments bad = args;
+    bad.view.x_stride = width + 8;
+    envelope = wt::arguments(bad);
+    expect(wt::enqueue(plan, weight, envelope, dout2.p, nullptr, 0).code == wt::Error::unsupported_shape, "weight::enqueue refuses a stride that is no multiple of 32: unsupported_shape");
+    wt::WeightView other = weight;
+    other.shape.dims[1] = count + 1;
+    envelope = wt::arguments(args);
+    expect(wt::enqueue(plan, other, envelope, dout2.p, nullptr, 0).code == wt::Error::unsupported_shape, "weight::enqueue refuses a weight whose shape differs from the launch");
 }
 
 // ----------------------------------------------------------------------------------------------- one expert layer, three ways
