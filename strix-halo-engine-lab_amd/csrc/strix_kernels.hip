@@ -14,6 +14,7 @@
 #include "device_math.hpp"
 #include "q4k_rows.hpp"
 #include "q4k_pairs.hpp"
+#include "q4k_mma.hpp"
 #include "q4k_quads.hpp"
 #include "down_groups.hpp"
 #include "q5k_quads.hpp"
@@ -1037,7 +1038,24 @@ inline void launch_pairs_depth(const PairArgs& a, uint32_t matrices, hipStream_t
 // nacts <= 8 activation rows. A matrix with few rows gives few wavefronts, each with a long instruction stream (the whole
 // of K): such launches spread every row over more lanes - the four super-blocks of a stage over a quad and, with >= 4
 // activation rows, two activation lanes - which multiplies the wavefronts and divides each one's instruction stream.
+// 3..16 activation rows over whole 32-row tiles: the matrix-core sweep (q4k_mma.hpp). A launch with no more workgroups than
+// compute units (few, long rows) runs four stages of a tile at a time (measured at 5120 rows x 27648, 8 rows: 59 -> 33 us;
+// ring depths 2..4 within 2 us of each other in both forms).
+template <int NAL>
+inline void launch_mma_depth(const PairArgs& a, uint32_t matrices, hipStream_t st) {
+    const dim3 grid(a.rows / kMmaRows, matrices);
+    if (static_cast<uint64_t>(grid.x) * grid.y <= compute_units()) q4k_mma_kernel<NAL, 2, 4><<<grid, 1024, 0, st>>>(a);
+    else q4k_mma_kernel<NAL, 3, 1><<<grid, 256, 0, st>>>(a);
+}
+inline bool mma_rows_ok(const PairArgs& a) { return a.nacts >= 3U && a.nacts <= 16U && a.rows % kMmaRows == 0; }
+inline void launch_mma(const PairArgs& a, uint32_t matrices, hipStream_t st) {
+    if (a.nacts <= 4U) launch_mma_depth<2>(a, matrices, st);
+    else if (a.nacts <= 8U) launch_mma_depth<4>(a, matrices, st);
+    else if (a.nacts <= 12U) launch_mma_depth<6>(a, matrices, st);
+    else launch_mma_depth<8>(a, matrices, st);
+}
 inline void launch_pairs(const PairArgs& a, uint32_t matrices, hipStream_t st) {
+    if (mma_rows_ok(a)) return launch_mma(a, matrices, st);
     const bool narrow = static_cast<uint64_t>(a.rows) * matrices < 16384U;
     if (a.nacts <= 1U) { if (narrow) launch_pairs_depth<1, 1, 4>(a, matrices, st); else launch_pairs_depth<1, 1>(a, matrices, st); }
     else if (a.nacts <= 2U) { if (narrow) launch_pairs_depth<2, 1, 4>(a, matrices, st); else launch_pairs_depth<2, 1>(a, matrices, st); }
@@ -1048,7 +1066,8 @@ inline void launch_pairs(const PairArgs& a, uint32_t matrices, hipStream_t st) {
 // 16 rows, not a whole 32-output SwiGLU group.
 inline bool dense_pairs_ok(const mi355_moe_weights& w, uint32_t rows) {
     return w.gate_type == MI355_TYPE_Q4_K && w.down_type == MI355_TYPE_Q4_K &&
-           w.experts == 1U && w.top_k == 1U && rows <= 8U && (w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0 &&
+           w.experts == 1U && w.top_k == 1U && rows <= 16U &&
+           (rows >= 3U || ((w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0)) &&      // the matrix-core sweep takes any length
            w.gate_row_stride < (1ULL << 24) && w.down_row_stride < (1ULL << 24);
 }
 inline void launch_project_dense(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, hipStream_t st) {

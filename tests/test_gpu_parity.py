@@ -474,11 +474,11 @@ def test_config5_tp_rank_partial_sums(strix):
         check_layer_stages(strix, *out[:7], out[7], H, K, T, 1, 0, TOL_F16)
 
 
-@pytest.mark.parametrize("H,I,batches", [(1280, 1792, (1, 4, 5, 6, 7, 8)), (1024, 2048, (1, 2, 3, 4, 5, 8))])
+@pytest.mark.parametrize("H,I,batches", [(1280, 1792, (1, 4, 5, 6, 7, 8, 11, 16)), (1024, 2048, (1, 2, 3, 4, 5, 8, 9, 12, 13))])
 def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
     """BASELINE config 2 structure at reduced size: a dense Q4_K FFN is the one-expert, top-1, weight-1 layer. The second
-    shape (row lengths that are multiples of 4 super-blocks) runs the pair-per-lane dense sweep, the first the row-per-lane
-    sweep; both must give the oracle's bits."""
+    shape (row lengths that are multiples of 4 super-blocks) runs the pair-per-lane dense sweep for 1 and 2 rows, the first the
+    row-per-lane sweep; 3..16 rows run the int8 matrix-core sweep (each of its four widths appears); all must give the oracle's bits."""
     for T in batches:
         rng = np.random.default_rng(20 + T)
         gate, up, down = make_layer(rng, H, I, 1)
