@@ -690,6 +690,8 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void down_wave_kernel(mi355_
     }
 }
 
+#include "q4k_mma_moe.hpp"
+
 // ---- the smallest decode batches: 16 rows per wavefront, lane = (row, pair) (q4k_quads.hpp) ------------------------------
 #define STRIX_QUAD_SLOTS(DEPTH)                                                                      \
     __shared__ __attribute__((aligned(16))) uint8_t quad0[4][kQuadSlotBytes];                         \
@@ -1038,24 +1040,7 @@ inline void launch_pairs_depth(const PairArgs& a, uint32_t matrices, hipStream_t
 // nacts <= 8 activation rows. A matrix with few rows gives few wavefronts, each with a long instruction stream (the whole
 // of K): such launches spread every row over more lanes - the four super-blocks of a stage over a quad and, with >= 4
 // activation rows, two activation lanes - which multiplies the wavefronts and divides each one's instruction stream.
-// 3..16 activation rows over whole 32-row tiles: the matrix-core sweep (q4k_mma.hpp). A launch with no more workgroups than
-// compute units (few, long rows) runs four stages of a tile at a time (measured at 5120 rows x 27648, 8 rows: 59 -> 33 us;
-// ring depths 2..4 within 2 us of each other in both forms).
-template <int NAL>
-inline void launch_mma_depth(const PairArgs& a, uint32_t matrices, hipStream_t st) {
-    const dim3 grid(a.rows / kMmaRows, matrices);
-    if (static_cast<uint64_t>(grid.x) * grid.y <= compute_units()) q4k_mma_kernel<NAL, 2, 4><<<grid, 1024, 0, st>>>(a);
-    else q4k_mma_kernel<NAL, 3, 1><<<grid, 256, 0, st>>>(a);
-}
-inline bool mma_rows_ok(const PairArgs& a) { return a.nacts >= 3U && a.nacts <= 16U && a.rows % kMmaRows == 0; }
-inline void launch_mma(const PairArgs& a, uint32_t matrices, hipStream_t st) {
-    if (a.nacts <= 4U) launch_mma_depth<2>(a, matrices, st);
-    else if (a.nacts <= 8U) launch_mma_depth<4>(a, matrices, st);
-    else if (a.nacts <= 12U) launch_mma_depth<6>(a, matrices, st);
-    else launch_mma_depth<8>(a, matrices, st);
-}
 inline void launch_pairs(const PairArgs& a, uint32_t matrices, hipStream_t st) {
-    if (mma_rows_ok(a)) return launch_mma(a, matrices, st);
     const bool narrow = static_cast<uint64_t>(a.rows) * matrices < 16384U;
     if (a.nacts <= 1U) { if (narrow) launch_pairs_depth<1, 1, 4>(a, matrices, st); else launch_pairs_depth<1, 1>(a, matrices, st); }
     else if (a.nacts <= 2U) { if (narrow) launch_pairs_depth<2, 1, 4>(a, matrices, st); else launch_pairs_depth<2, 1>(a, matrices, st); }
@@ -1066,8 +1051,7 @@ inline void launch_pairs(const PairArgs& a, uint32_t matrices, hipStream_t st) {
 // 16 rows, not a whole 32-output SwiGLU group.
 inline bool dense_pairs_ok(const mi355_moe_weights& w, uint32_t rows) {
     return w.gate_type == MI355_TYPE_Q4_K && w.down_type == MI355_TYPE_Q4_K &&
-           w.experts == 1U && w.top_k == 1U && rows <= 16U &&
-           (rows >= 3U || ((w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0)) &&      // the matrix-core sweep takes any length
+           w.experts == 1U && w.top_k == 1U && rows <= 8U && (w.hidden / 256U) % kPairBlocks == 0 && (w.ffn / 256U) % kPairBlocks == 0 &&
            w.gate_row_stride < (1ULL << 24) && w.down_row_stride < (1ULL << 24);
 }
 inline void launch_project_dense(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, hipStream_t st) {
@@ -1085,6 +1069,53 @@ inline void launch_down_dense(const mi355_moe_weights& w, const RowsK& r, uint32
     a.rows = w.hidden; a.blocks = w.ffn / 256U; a.img = r.h; a.nacts = rows;
     a.skip_flag = r.job_status; a.skip_mask = MI355_STATUS_NONFINITE_PROJECTION;
     launch_pairs(a, 1, st);
+}
+
+// ---- work items of 3..32 rows on the int8 matrix cores (q4k_mma_moe.hpp) ---------------------------------------------
+// A dense Q4_K FFN (one expert, top-1, assignment i = row i) with at least 3 rows, in chunks of the sweep's width.
+inline bool mma_dense(const mi355_moe_weights& w, const RowsK& r, uint32_t rows) {
+    return w.gate_type == MI355_TYPE_Q4_K && w.down_type == MI355_TYPE_Q4_K && w.experts == 1U && w.top_k == 1U && rows >= 3U && !r.assignments;
+}
+// Routed experts of a batch past the decode sizes whose experts hold several rows each on average: the plan cuts an expert's
+// rows into items of this many (0: the vector-ALU sweeps serve the batch).
+// Items of up to four 32-row sweeps: the later sweeps of a tile's weights hit the cache, and an expert with thousands of rows
+// still spreads over many workgroups.
+constexpr uint32_t kMmaItemRows = 128;
+inline uint32_t mma_grouped_split(const mi355_moe_weights& w, uint32_t rows) {
+    if (w.gate_type != MI355_TYPE_Q4_K || w.down_type != MI355_TYPE_Q4_K || w.experts == 1U || rows <= kFusedMaxRows) return 0U;
+    const uint64_t assignments = static_cast<uint64_t>(rows) * w.top_k;
+    return assignments >= 16ULL * w.experts ? kMmaItemRows : assignments >= 4ULL * w.experts ? 16U : 0U;
+}
+template <int NAL>
+inline void launch_mma_project_nal(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t dense, uint32_t items, hipStream_t st) {
+    const dim3 grid(w.ffn / 32U, dense ? (dense + 2U * NAL - 1U) / (2U * NAL) : items);
+    q4k_mma_project_kernel<NAL, (NAL >= 8 ? 2 : 3)><<<grid, 256, 0, st>>>(w, r, rows * w.top_k, dense);
+}
+// A launch with no more workgroups than compute units (few, long rows) runs four stages of a tile at a time (measured at 5120
+// rows x 27648, 8 rows: 59 -> 33 us; ring depths 2..4 within 2 us of each other in both forms).
+template <int NAL>
+inline void launch_mma_down_nal(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t dense, uint32_t items, hipStream_t st) {
+    const dim3 grid(w.hidden / kMmaRows, dense ? (dense + 2U * NAL - 1U) / (2U * NAL) : items);
+    if constexpr (NAL <= 8) {
+        if (static_cast<uint64_t>(grid.x) * grid.y <= compute_units()) {
+            q4k_mma_down_kernel<NAL, 2, 4><<<grid, 1024, 0, st>>>(w, r, rows * w.top_k, dense);
+            return;
+        }
+    }
+    q4k_mma_down_kernel<NAL, (NAL >= 8 ? 2 : 3), 1><<<grid, 256, 0, st>>>(w, r, rows * w.top_k, dense);
+}
+// width: the most rows an item (or the dense batch) holds
+inline void launch_mma_project(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t dense, uint32_t items, uint32_t width, hipStream_t st) {
+    if (width <= 4U) launch_mma_project_nal<2>(w, r, rows, dense, items, st);
+    else if (width <= 8U) launch_mma_project_nal<4>(w, r, rows, dense, items, st);
+    else if (width <= 16U) launch_mma_project_nal<8>(w, r, rows, dense, items, st);
+    else launch_mma_project_nal<16>(w, r, rows, dense, items, st);
+}
+inline void launch_mma_down(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t dense, uint32_t items, uint32_t width, hipStream_t st) {
+    if (width <= 4U) launch_mma_down_nal<2>(w, r, rows, dense, items, st);
+    else if (width <= 8U) launch_mma_down_nal<4>(w, r, rows, dense, items, st);
+    else if (width <= 16U) launch_mma_down_nal<8>(w, r, rows, dense, items, st);
+    else launch_mma_down_nal<16>(w, r, rows, dense, items, st);
 }
 
 inline void launch_plan(RoutesView routes, uint32_t experts, uint32_t assignments, uint32_t split, uint32_t bound, uint32_t* plan,
@@ -1115,6 +1146,8 @@ inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t 
         else project_quad_kernel<2><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, r, items);
         return;
     }
+    if (mma_dense(w, r, rows)) return launch_mma_project(w, r, rows, rows, 0, rows, st);
+    if (const uint32_t split = mma_grouped_split(w, rows); split && r.plan) return launch_mma_project(w, r, rows, 0, umax, split, st);
     if (dense_pairs_ok(w, rows) && dense_rows(r, w) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
     const dim3 grid(w.ffn / 32U, umax);
     if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
@@ -1135,6 +1168,8 @@ inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t row
         else down_quad_kernel<2><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
         return;
     }
+    if (mma_dense(w, r, rows)) return launch_mma_down(w, r, rows, rows, 0, rows, st);
+    if (const uint32_t split = mma_grouped_split(w, rows); split && r.plan) return launch_mma_down(w, r, rows, 0, umax, split, st);
     if (dense_pairs_ok(w, rows) && dense_rows(r, w)) return launch_down_dense(w, r, rows, st);
     const dim3 grid(w.hidden / 64U, umax);
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
@@ -1145,6 +1180,7 @@ inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t row
 // expert's weights comes from the last-level cache. A dense matrix: every row shares one sweep.
 inline uint32_t plan_split(const mi355_moe_weights& w, uint32_t rows) {
     if (w.experts == 1U) return 8;
+    if (const uint32_t split = mma_grouped_split(w, rows)) return split;     // items for the matrix-core sweep
     if (rows > kFusedMaxRows) return 4U;
     if (quad_sweep(w, rows)) return 1U;       // the 16-rows-per-wavefront sweep serves one assignment per item
     // decode batches: one item per assignment while an expert's gate + up rows are a few MB (the second sweep of an expert

@@ -415,6 +415,46 @@ def test_layer_entry_shared_sweeps_over_large_experts(strix):
     assert torch.equal(y2, y)
 
 
+@pytest.mark.parametrize("E,K,T,bias_scale,nonfinite", [(6, 2, 200, 2.0, False), (8, 2, 40, 0.0, False), (5, 3, 97, 1.0, True)])
+def test_batches_past_decode_sizes_run_the_matrix_core_sweep(strix, E, K, T, bias_scale, nonfinite):
+    """Batches whose experts hold at least 4 / 16 rows on average are planned in items of 16 / 128 rows and served by the int8
+    matrix-core sweep in chunks of 16 / 32 rows: a biased router makes one expert's item longer than a sweep (several chunks,
+    the last one ragged and odd) while others hold a row or two. Stage by stage against the oracle - gate, up, the A8 image
+    of h, rawdots bit for bit - through the layer entry and the staged one; with a non-finite weight scale in one expert the
+    rows that chose it are flagged and the down stage is skipped, as on the vector-ALU sweeps."""
+    H, I = 768, 512
+    rng = np.random.default_rng(1000 + T)
+    gate, up, down = make_layer(rng, H, I, E)
+    if nonfinite:
+        gate = gate.copy()
+        gate.reshape(E, I, -1)[1, 7, 0:2] = np.frombuffer(np.float16(np.inf).tobytes(), np.uint8)      # d of one block of expert 1
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(E) * bias_scale).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, intermediates=True)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K, bias=bias)
+    y, ids, wts, _ = layer.run_layer(dev(x), dev(wr), bias=dev(bias))
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    counts = np.bincount(ids_ref.reshape(-1), minlength=E)
+    split = 128 if T * K >= 16 * E else 16
+    assert T * K >= 4 * E and int(layer.plan[4]) == sum(-(-int(c) // split) for c in counts)
+    if bias_scale:
+        assert counts.max() > 32 and counts.max() % 32 not in (0, 31)          # several chunks, a ragged last one
+    if nonfinite:
+        hit = np.any(ids_ref == 1, axis=1)
+        st = layer.status[:T].cpu().numpy()
+        assert hit.any() and not hit.all()
+        assert np.all((st[hit] & strix.STATUS_NONFINITE_PROJECTION) != 0) and np.all(st[~hit] == 0)
+        assert int(layer.job_status[0]) & strix.STATUS_NONFINITE_PROJECTION
+        return
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    ref = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref)
+    want = orc.combine(0, w_ref, ids_ref, ref.rawdots)
+    check_layer_stages(strix, layer, y.cpu().numpy(), ref, want, (c, d, s), ids_ref, w_ref, (gate, up, down, I, {}), H, K, T, 0, 0, TOL_F16)
+    y2 = layer.run(dev(x), ids, wts)
+    assert torch.equal(y2, y)
+
+
 @pytest.mark.parametrize("E,H,I,K,T,order", [(128, 2048, 768, 8, 8, 0), (128, 2048, 768, 8, 1, 0), (128, 2048, 768, 8, 2, 0), (160, 1536, 512, 8, 16, 0),
                                              (20, 512, 256, 3, 5, 1), (64, 1024, 256, 16, 16, 0), (160, 6144, 1280, 8, 2, 0)])
 def test_whole_layer_entry_router_prologue_plan_in_one_launch(strix, E, H, I, K, T, order):
@@ -569,7 +609,9 @@ def test_expert_plan_words(strix, E, K, T):
     plan = layer.plan.cpu().numpy().view(np.uint32)
     flat = ids.reshape(-1).astype(np.int64)
     A = T * K
-    split = 8 if E == 1 else (1 if T <= 16 else 4)
+    # items: 8 rows of a dense matrix; one assignment at decode sizes; past them 128 / 16 rows for the matrix-core sweep when
+    # the experts hold at least 16 / 4 rows on average, else 4
+    split = 8 if E == 1 else (1 if T <= 16 else 128 if A >= 16 * E else 16 if A >= 4 * E else 4)
     valid = flat < E
     counts = np.bincount(flat[valid], minlength=E)
     offsets = np.concatenate([[0], np.cumsum(counts)])
