@@ -367,7 +367,7 @@ def extra_configs(strix, torch, steps, warmup):
     sec = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 2, 1)
     out["config4_prefill_T4096_integer_class"] = {
         "ms": sec * 1e3, "TFLOPs": (flops_experts + flops_router) / sec / 1e12, "algorithmic_flops": flops_experts + flops_router,
-        "note": "same work in the bit-exact integer-dot class on the decode kernels (router included)"}
+        "note": "same work in the bit-exact integer-dot class: int8 matrix-core group dots, the fp32 chain on the vector ALU (router included)"}
     return out
 
 

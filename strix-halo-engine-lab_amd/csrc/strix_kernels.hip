@@ -1111,11 +1111,19 @@ inline void launch_mma_project(const mi355_moe_weights& w, const RowsK& r, uint3
     else if (width <= 16U) launch_mma_project_nal<8>(w, r, rows, dense, items, st);
     else launch_mma_project_nal<16>(w, r, rows, dense, items, st);
 }
+// A dense FFN's gate and up rows as raw values into the intermediates, then the SwiGLU / A8 kernel (5..16 rows, one chunk).
+inline void launch_mma_gate_up(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, hipStream_t st) {
+    const dim3 grid(w.ffn / kMmaRows, 1, 2);
+    if (rows <= 8U) q4k_mma_down_kernel<4, 3, 1, true><<<grid, 256, 0, st>>>(w, r, rows, rows);
+    else q4k_mma_down_kernel<8, 2, 1, true><<<grid, 256, 0, st>>>(w, r, rows, rows);
+    swiglu_quantize_kernel<<<dim3((w.ffn / 32U + 7U) / 8U, rows), 256, 0, st>>>(r.gate_out, r.up_out, w.ffn, w.exp_kind, w.swiglu_limit, r.down_codes, r.down_deltas,
+                                                                                r.down_sums, r.h_out, r.status, r.job_status);
+}
+// (the down rows run best 16 rows to a sweep: 4096 rows over 256 experts, hidden 4096 / ffn 2048: 2.57 ms against 3.03 ms with 32)
 inline void launch_mma_down(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t dense, uint32_t items, uint32_t width, hipStream_t st) {
     if (width <= 4U) launch_mma_down_nal<2>(w, r, rows, dense, items, st);
     else if (width <= 8U) launch_mma_down_nal<4>(w, r, rows, dense, items, st);
-    else if (width <= 16U) launch_mma_down_nal<8>(w, r, rows, dense, items, st);
-    else launch_mma_down_nal<16>(w, r, rows, dense, items, st);
+    else launch_mma_down_nal<8>(w, r, rows, dense, items, st);
 }
 
 inline void launch_plan(RoutesView routes, uint32_t experts, uint32_t assignments, uint32_t split, uint32_t bound, uint32_t* plan,
@@ -1146,7 +1154,10 @@ inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t 
         else project_quad_kernel<2><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, r, items);
         return;
     }
-    if (mma_dense(w, r, rows)) return launch_mma_project(w, r, rows, rows, 0, rows, st);
+    if (mma_dense(w, r, rows)) {
+        if (rows > 4U && rows <= 16U && r.gate_out && r.up_out && dense_rows(r, w)) return launch_mma_gate_up(w, r, rows, st);
+        return launch_mma_project(w, r, rows, rows, 0, rows, st);
+    }
     if (const uint32_t split = mma_grouped_split(w, rows); split && r.plan) return launch_mma_project(w, r, rows, 0, umax, split, st);
     if (dense_pairs_ok(w, rows) && dense_rows(r, w) && r.gate_out && r.up_out) return launch_project_dense(w, r, rows, st);
     const dim3 grid(w.ffn / 32U, umax);
