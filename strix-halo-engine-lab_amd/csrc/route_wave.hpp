@@ -313,6 +313,10 @@ __device__ __forceinline__ void chain_start(ChainSlot& slot, const RouteArgs& a,
     }
 }
 // fp16 / bf16: widen the landed chunk to fp32 (8 features per lane).
+// The widened values are read by other lanes of the same wavefront (the workgroup is one wavefront): LDS operations of a
+// wavefront complete in order, so the writes only have to be issued before the reads - no barrier. __syncthreads() here
+// would also wait for every copy in flight, i.e. drain the three chunks the ring keeps ahead of the chain.
+__device__ __forceinline__ void chain_publish() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 template <int KIND, bool NORM = false>
 __device__ __forceinline__ void chain_widen(ChainSlot& slot, float factor = 1.0F, bool scaled = false) {
     if constexpr (KIND == 0 && NORM) {
@@ -326,7 +330,7 @@ __device__ __forceinline__ void chain_widen(ChainSlot& slot, float factor = 1.0F
             if (scaled) { v.x = v.x * w.x; v.y = v.y * w.y; v.z = v.z * w.z; v.w = v.w * w.w; }
             *reinterpret_cast<f32x4*>(&slot.x[256U * j + 4U * lane]) = v;
         }
-        __syncthreads();
+        chain_publish();
     }
     if constexpr (KIND != 0) {
         const uint32_t lane = threadIdx.x & 63U;
@@ -347,28 +351,45 @@ __device__ __forceinline__ void chain_widen(ChainSlot& slot, float factor = 1.0F
         }
         *reinterpret_cast<f32x4*>(&slot.x[8U * lane]) = f32x4{f[0], f[1], f[2], f[3]};
         *reinterpret_cast<f32x4*>(&slot.x[8U * lane + 4U]) = f32x4{f[4], f[5], f[6], f[7]};
-        __syncthreads();
+        chain_publish();
     }
 }
 
-// Operands of 16 features: eight 128-bit LDS reads (the activation reads are broadcasts). Measured on MI355X a wave
-// pays ~5 cycles per dependent fma and ~9 per ds_read_b128, with no overlap between them, so a chain step costs about
-// 10 cycles; the operands of the next 16 features are requested before the current 16 are chained (8 reads in flight,
-// within the 15 the LDS counter can express).
-struct ChainStep { f32x4 w[4]; f32x4 x[4]; };
+// Operands of 16 features: four 128-bit LDS reads of the lane's weight row and one 32-bit read that leaves feature k + t
+// in lane t of every row of 16 lanes; the fma takes its activation operand from there by a row broadcast (a DPP operand,
+// no instruction of its own). Measured on MI355X a wave pays ~5 cycles per dependent fma and ~9 per ds_read_b128, with no
+// overlap between them; the operands of the next 16 features are requested before the current 16 are chained.
+struct ChainStep { f32x4 w[4]; float x; };
 __device__ __forceinline__ void chain_load(ChainStep& s, const ChainSlot& slot, uint32_t el, uint32_t k) {
     const float* wrow = slot.w[el] + k;
 #pragma unroll
     for (uint32_t i = 0; i < 4U; ++i) s.w[i] = *reinterpret_cast<const f32x4*>(wrow + 4U * i);
-#pragma unroll
-    for (uint32_t i = 0; i < 4U; ++i) s.x[i] = *reinterpret_cast<const f32x4*>(slot.x + k + 4U * i);
+    s.x = slot.x[k + (threadIdx.x & 15U)];
 }
+// acc = fma(x[k + t], w[t], acc) for t = 0..15 in order. Written out as instructions because the compiler keeps the three-address
+// fma, which has no DPP form, and then spends a v_mov_b32_dpp per feature. The leading s_nop covers the two wait states a DPP
+// read needs after a vector-ALU write of its source register, whatever the compiler placed in front.
 __device__ __forceinline__ float chain_run(const ChainStep& s, float acc) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        acc = __builtin_fmaf(s.x[i].x, s.w[i].x, acc); acc = __builtin_fmaf(s.x[i].y, s.w[i].y, acc);
-        acc = __builtin_fmaf(s.x[i].z, s.w[i].z, acc); acc = __builtin_fmaf(s.x[i].w, s.w[i].w, acc);
-    }
+    asm("s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %1, %2 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %3 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %4 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %5 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %6 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %7 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %8 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %9 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %10 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %11 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %12 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %13 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %14 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %15 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %16 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+        "v_fmac_f32_dpp %0, %1, %17 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(s.x), "v"(s.w[0].x), "v"(s.w[0].y), "v"(s.w[0].z), "v"(s.w[0].w), "v"(s.w[1].x), "v"(s.w[1].y), "v"(s.w[1].z), "v"(s.w[1].w),
+          "v"(s.w[2].x), "v"(s.w[2].y), "v"(s.w[2].z), "v"(s.w[2].w), "v"(s.w[3].x), "v"(s.w[3].y), "v"(s.w[3].z), "v"(s.w[3].w));
     return acc;
 }
 

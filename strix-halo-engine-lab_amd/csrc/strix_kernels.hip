@@ -875,7 +875,10 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, RowsK r
 // Reference: src/cpu/core/routed_expert.cpp:429-447, src/moe_a8_down_contract.cpp:146, include/strix/moe/combine.hpp:36-59.
 constexpr uint32_t kDownMergeSlots = 8;        // top_k bound: 8 waves x 2 ring slots fill the LDS of a compute unit
 __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
-    __shared__ __attribute__((aligned(16))) uint8_t rings[kDownMergeSlots][2][slot_bytes(1)];
+    // the two ring slots are separate LDS objects: the compiler then knows that a copy into one never touches the other and lets
+    // the reads of the landed slot go ahead while the next stage's copy is in flight (as slots of one array it waited for both)
+    __shared__ __attribute__((aligned(16))) uint8_t ring_even[kDownMergeSlots][slot_bytes(1)];
+    __shared__ __attribute__((aligned(16))) uint8_t ring_odd[kDownMergeSlots][slot_bytes(1)];
     __shared__ float slot_value[kDownMergeSlots][64];
     __shared__ uint32_t slot_order[kDownMergeSlots];
     __shared__ float slot_weight[kDownMergeSlots];
@@ -891,7 +894,7 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
         const size_t stride = w.down_row_stride;
         StageSource source;
         source.init([&](uint32_t q) { return rows + q * stride; });
-        lds_u8* const slots[2] = {(lds_u8*)rings[wave][0], (lds_u8*)rings[wave][1]};
+        lds_u8* const slots[2] = {(lds_u8*)ring_even[wave], (lds_u8*)ring_odd[wave]};
         const uint32_t src[1] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(first))}, lane_rows[1] = {first};
         const ActRows<1> act(r.h, src, lane_rows);
         float swept[1];
