@@ -259,7 +259,9 @@ def prefill_config4(strix, torch, gen, keep=False, reps=10):
 
     def whole(i):
         r_ids, r_wts, _ = strix.route(xp, wr, K, bias=bias)
-        return layer.run_prefill_f16(xp, r_ids, r_wts, base=dense.run_prefill_f16(xp, zero_ids, ones))
+        # the shared expert without its one-slot combine: its unweighted outputs are the routed combine's base
+        shared = dense.run_prefill_f16(xp, zero_ids, ones, combine=strix.COMBINE_NONE).reshape(T, H)
+        return layer.run_prefill_f16(xp, r_ids, r_wts, base=shared)
     sec_whole = time_steps(torch, whole, reps, 3)
     if int(layer.status.sum()) or int(dense.status.sum()):
         raise RuntimeError("config 4: the prefill run set row status bits (non-finite or out-of-range values): the timing is void")

@@ -48,7 +48,11 @@ enum {
 enum { MI355_TYPE_Q5_1 = 7, MI355_TYPE_Q8_0 = 8, MI355_TYPE_Q4_K = 12, MI355_TYPE_Q5_K = 13, MI355_TYPE_Q6_K = 14 };              /* ggml tensor type ids */
 enum { MI355_INPUT_F32 = 0, MI355_INPUT_F16 = 1, MI355_INPUT_BF16 = 2 };
 enum { MI355_LOGITS_FMA_ASCENDING = 0, MI355_LOGITS_LANE32_BUTTERFLY = 1 };
-enum { MI355_COMBINE_FMA_SLOT_ORDER = 0, MI355_COMBINE_MULADD_ASCENDING_EXPERT = 1 };
+enum { MI355_COMBINE_FMA_SLOT_ORDER = 0, MI355_COMBINE_MULADD_ASCENDING_EXPERT = 1,
+       MI355_COMBINE_NONE = 2 };   /* mi355_moe_enqueue_prefill_f16 only: stop after the down rows. rawdots then holds the unweighted
+                                      per-slot outputs; for a top-1 layer of weight 1 (an always-on shared expert) rawdots[row] is
+                                      the layer's output - fma(1, x, 0) = x - and can be the `base` of the routed call, which saves
+                                      the copy a combine of one slot would be. The caller reads status / job_status itself. */
 enum { MI355_EXP_GFX1151 = 0, MI355_EXP_DECLARED = 1,
        MI355_EXP_LIBM = 2 };   /* router softmax only: the C library's expf as the reference's router test oracle uses it
                                   (tests/hip_moe_route_launcher_tests.hip:329), restated in double precision on the device */

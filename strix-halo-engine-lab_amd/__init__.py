@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(HERE, "libmi355_strix.so")
 TYPE_Q5_1, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K = 7, 8, 12, 13, 14
 INPUT_F32, INPUT_F16, INPUT_BF16 = 0, 1, 2
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
-COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
+COMBINE_FMA_SLOT, COMBINE_MULADD_ASC, COMBINE_NONE = 0, 1, 2
 EXP_GFX1151, EXP_DECLARED, EXP_LIBM = 0, 1, 2
 STATUS_INVALID_ROUTE, STATUS_NONFINITE_ACTIVATION, STATUS_INVALID_DELTA, STATUS_NONFINITE_PROJECTION, STATUS_AGGREGATE = 1, 2, 4, 8, 16
 E_INVALID_ARGUMENT, E_UNSUPPORTED, E_HIP = -1, -2, -3
@@ -486,6 +486,8 @@ class MoeLayer:
         """The routed experts on the matrix cores (fp16 weights x fp16 rows, fp32 accumulation): mi355_moe_enqueue_prefill_f16."""
         rows, rv = self.rows_view(x, ids, weights, base)
         check(lib().mi355_moe_enqueue_prefill_f16(C.byref(self.w), C.byref(rv), rows, combine, _stream()))
+        if combine == COMBINE_NONE:      # no combine: the unweighted per-slot outputs [rows][top_k][hidden]
+            return self.rawdots[:rows]
         return self.output[:rows]
 
     def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,

@@ -1614,7 +1614,7 @@ int32_t mi355_moe_enqueue_layer_normed(const mi355_route_policy* p, const float*
 int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv, kPrefillClass)) return rc;
-    STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe prefill: unknown combine form");
+    STRIX_REQUIRE(form <= MI355_COMBINE_NONE, "moe prefill: unknown combine form");
     STRIX_REQUIRE(r->input && r->input_kind == MI355_INPUT_F16, "moe prefill: the fp16 form takes fp16 input rows");
     STRIX_REQUIRE(r->input_stride % 16U == 0 && aligned(r->input, 16), "moe prefill: input rows must be 16-byte aligned");
     STRIX_REQUIRE(r->h_f16 && aligned(r->h_f16, 16), "moe prefill: h_f16 workspace is null or misaligned");
@@ -1669,6 +1669,7 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
         }
     }
     STRIX_LAUNCHED("moe prefill f16");
+    if (form == MI355_COMBINE_NONE) return MI355_OK;
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
 

@@ -859,6 +859,9 @@ def test_prefill_f16_mfma_q8_0_tensors(strix, H, I, E, K, T, gate_type, down_typ
         big = np.abs(ref64) > 1e-2 * rms
         assert np.max(np.abs(got[big] - ref64[big]) / np.abs(ref64[big])) < TOL_F16
     assert np.all(layer.status[:T].cpu().numpy() == 0)
+    if E == 1:      # a top-1 layer of weight 1 without the combine: its rawdots are the combined output, bit for bit
+        raw = layer.run_prefill_f16(dev(x), dev(ids_ref.astype(np.int32)), dev(w_ref), combine=strix.COMBINE_NONE)
+        assert np.array_equal(bits(raw.cpu().numpy().reshape(T, H)), bits(y))
     # the integer-class entries keep refusing Q8_0 gate / up tensors
     if gate_type == orc.Q8_0:
         with pytest.raises(strix.StrixError):
