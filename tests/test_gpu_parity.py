@@ -320,10 +320,11 @@ def test_moe_layer_declared_exp_is_bit_exact_end_to_end(strix):
     assert np.array_equal(bits(y), bits(want))
 
 
-@pytest.mark.parametrize("H,I,E,K,T,gate_q5k", [(1024, 512, 8, 4, 9, False), (1024, 512, 8, 4, 2, False), (512, 256, 6, 2, 5, True)])
+@pytest.mark.parametrize("H,I,E,K,T,gate_q5k", [(1024, 512, 8, 4, 9, False), (1024, 512, 8, 4, 2, False), (512, 256, 6, 2, 5, True),
+                                                  (512, 256, 4, 2, 70, False), (768, 256, 1, 1, 21, False)])
 def test_swiglu_clamp_trait_in_every_projection_kernel(strix, H, I, E, K, T, gate_q5k):
-    """The SwiGLU clamp (include/strix/moe/activation_policy.hpp:22-24) in the 64-row sweep (9 rows), the 16-row sweep (2 rows)
-    and the Q5_K projection: with the declared exp every bit of h, of its A8 image and of the layer output equals the oracle's,
+    """The SwiGLU clamp (include/strix/moe/activation_policy.hpp:22-24) in the 64-row sweep (9 rows), the 16-row sweep (2 rows),
+    the Q5_K projection and the matrix-core sweep's epilogue (70 rows over 4 experts; a dense FFN of 21 rows): with the declared exp every bit of h, of its A8 image and of the layer output equals the oracle's,
     the limit actually binds, and gate_out / up_out keep the RAW projections."""
     rng = np.random.default_rng(H + T)
     limit = 0.02
@@ -502,6 +503,15 @@ def test_layer_entry_one_workspace_varying_batch_sizes(strix):
         y2 = staged.run(x[:rows], ids2, wts2)
         assert torch.equal(y, y2) and torch.equal(layer.rawdots[:rows], staged.rawdots[:rows])
         assert np.all(layer.status[:rows].cpu().numpy() == 0) and bool((layer.plan[16:272] == 0).all())
+
+
+def test_tp_rank_shard_on_the_matrix_core_sweep(strix):
+    """The rank's share read in place through strides (as in config 5) at a batch that runs the matrix-core sweep: 90 rows
+    over 5 experts, items of up to 128 rows; gate / up rows and down K blocks of rank 1 of 2, declared exp."""
+    H, I, E, K, T = 768, 1024, 5, 2, 90
+    out = run_layer_both(strix, H, I, E, K, T, seed=56, combine=1, tp=(1, 2), exp_kind=1)
+    assert int(out[0].plan[4]) < T * K // 4          # grouped items, not one per assignment
+    check_layer_stages(strix, *out[:7], out[7], H, K, T, 1, 1, TOL_F16)
 
 
 def test_config5_tp_rank_partial_sums(strix):

@@ -70,7 +70,8 @@ def weights_of(strix, H, I, E, K, gate, up, down, gate_type, down_type):
     (orc.Q5_K, orc.Q8_0, 1024, 512, 16, 4, 40, torch.float16, torch.bfloat16),        # the reference twin's own formats, shared sweeps
     (orc.Q4_K, orc.Q5_1, 2560, 640, 64, 10, 16, torch.bfloat16, torch.bfloat16),      # the twin's fixed geometry but for the expert count
     (orc.Q4_K, orc.Q6_K, 512, 768, 6, 3, 5, torch.float32, torch.float32),
-    (orc.Q4_K, orc.Q4_K, 1024, 1024, 1, 1, 6, torch.bfloat16, torch.bfloat16)])       # a dense matrix through strided views
+    (orc.Q4_K, orc.Q4_K, 1024, 1024, 1, 1, 6, torch.bfloat16, torch.bfloat16),        # a dense matrix through strided views (matrix-core sweep)
+    (orc.Q4_K, orc.Q4_K, 512, 512, 4, 2, 40, torch.bfloat16, torch.float32)])         # 20 rows per expert: items of up to 128 rows on the matrix-core sweep
 def test_strided_rows_every_stage(strix, gate_type, down_type, H, I, E, K, T, in_kind, out_kind):
     rng = np.random.default_rng(H + I + 3 * T + down_type)
     if I % 256 == 0:
