@@ -241,7 +241,7 @@ int32_t mi355_a8_enqueue_probe(const mi355_a8_request* q, const mi355_a8_binding
     r.gate_out = reinterpret_cast<float*>(b->output.address); r.up_out = r.gate_out + s.rows; r.slot_stride = 2ULL * s.rows;
     r.inter_rs = 4ULL * s.top_k * r.slot_stride;
     const uint32_t items = R * s.top_k;
-    if (q->gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
+    if (q->gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else if (items <= 16U) project_quad_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else if (items <= kQuadMaxItems) project_quad_kernel<2><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else launch_project_nb<4>(w, r, R, dim3(s.rows / 32U, items), st);

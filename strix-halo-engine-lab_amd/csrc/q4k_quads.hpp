@@ -20,7 +20,10 @@ constexpr uint32_t kQuadRows = 16;
 constexpr uint32_t kQuadSlotBytes = 4096;          // [0, 3072): weights (144 pieces + padding), [3072, 4096): codes (256 bytes + padding)
 constexpr uint32_t kQuadCopies = 4;                // copy instructions per stage
 
-struct QuadSource {
+// PIECES = 16-byte pieces of one row's block: 9 (Q4_K, 144 bytes) or 11 (Q5_K, 176 bytes); 16 rows are 144 / 176 pieces, three
+// copy instructions either way (the third partly padding).
+template <uint32_t PIECES>
+struct QuadSourceT {
     const uint8_t* piece[3];
     const uint8_t* act_piece;
     // row_ptr(r) = first byte of weight row r (0..15); codes = the activation row's codes
@@ -30,8 +33,8 @@ struct QuadSource {
 #pragma unroll
         for (uint32_t i = 0; i < 3U; ++i) {
             uint32_t j = i * 64U + lane;
-            j = j < kQuadRows * 9U ? j : kQuadRows * 9U - 1U;              // padding lanes repeat the last piece into unused LDS
-            const uint32_t r = __umulhi(j, 0x1C71C71DU), c = j - 9U * r;   // j / 9 exact for j < 576
+            j = j < kQuadRows * PIECES ? j : kQuadRows * PIECES - 1U;      // padding lanes repeat the last piece into unused LDS
+            const uint32_t r = j / PIECES, c = j - PIECES * r;
             piece[i] = row_ptr(r) + 16U * c;
         }
         act_piece = reinterpret_cast<const uint8_t*>(codes) + 16U * (lane & 15U);
@@ -41,13 +44,14 @@ struct QuadSource {
         for (uint32_t i = 0; i < 3U; ++i) {
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)piece[i],
                                              (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
-            piece[i] += 144;
+            piece[i] += 16U * PIECES;
         }
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)act_piece,
                                          (__attribute__((address_space(3))) void*)(slot + 3072U), 16, 0, 0);
         act_piece += 256;
     }
 };
+typedef QuadSourceT<9> QuadSource;
 
 // The pair term of a super-block from its header words and the two integer dots (sub-blocks 2p, 2p + 1):
 // x_j = delta_j * (d * sc_j * float(dot_j) - dmin * m_j * float(sum_j)), returned as x_2p + x_(2p+1). e0 / e1: the group
@@ -93,9 +97,35 @@ __device__ __forceinline__ void quad_block_compute(const lds_u8* slot, uint32_t 
     acc = acc + quad_pair_term(hd, p, dot0, dot1, e0, e1, f0, f1);
 }
 
+// The same for a Q5_K super-block (176 bytes: header, 32 fifth-bit bytes - bit j of byte k belongs to element k of sub-block j -,
+// 128 nibble bytes; q = nibble | fifth bit << 4; src/cpu/core/routed_expert.cpp:73-108 with Q5K).
+__device__ __forceinline__ void quad_block_compute_q5k(const lds_u8* slot, uint32_t kb, float vd, float vf, float& acc) {
+    typedef const __attribute__((address_space(3))) u32x4 lds_u32x4;
+    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, r = lane >> 2;
+    lds_u32x4* blk = (lds_u32x4*)(slot + r * 176U);
+    const u32x4 hd = blk[0], h0 = blk[1], h1 = blk[2], q0 = blk[3U + 2U * p], q1 = blk[4U + 2U * p];
+    lds_u32x4* c = (lds_u32x4*)(slot + 3072U + 64U * p);
+    const u32x4 c0 = c[0], c1 = c[1], c2 = c[2], c3 = c[3];
+    const uint32_t qs[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const uint32_t qh[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+    const uint32_t cw[16] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w, c2.x, c2.y, c2.z, c2.w, c3.x, c3.y, c3.z, c3.w};
+    int dot0 = 0, dot1 = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t fifth = qh[k] >> (2U * p);                        // bit 0 of every byte: sub-block 2p, bit 1: 2p + 1
+        const uint32_t lo = (qs[k] & 0x0f0f0f0fU) | ((fifth & 0x01010101U) << 4);
+        const uint32_t hi = ((qs[k] >> 4) & 0x0f0f0f0fU) | ((fifth & 0x02020202U) << 3);
+        dot0 = __builtin_amdgcn_sdot4(static_cast<int>(lo), static_cast<int>(cw[k]), dot0, false);
+        dot1 = __builtin_amdgcn_sdot4(static_cast<int>(hi), static_cast<int>(cw[8 + k]), dot1, false);
+    }
+    const int from = static_cast<int>((kb & 7U) * 8U + 2U * p);
+    const float e0 = __shfl(vd, from), e1 = __shfl(vd, from + 1), f0 = __shfl(vf, from), f1 = __shfl(vf, from + 1);
+    acc = acc + quad_pair_term(hd, p, dot0, dot1, e0, e1, f0, f1);
+}
+
 // Whole sweep of the wave's 16 rows against activation row `row` of `img`; every lane of a quad returns the row's value.
-template <int DEPTH>
-__device__ __forceinline__ float sweep_quads(lds_u8* const (&slots)[DEPTH], QuadSource source, uint32_t blocks, const A8Image& img, uint32_t row) {
+template <int DEPTH, bool Q5K = false>
+__device__ __forceinline__ float sweep_quads(lds_u8* const (&slots)[DEPTH], QuadSourceT<Q5K ? 11U : 9U> source, uint32_t blocks, const A8Image& img, uint32_t row) {
     const uint32_t lane = threadIdx.x & 63U, groups = img.width / 32U;
     const float* deltas = img.deltas_of(row);
     const int32_t* sums = img.sums_of(row);
@@ -116,7 +146,8 @@ __device__ __forceinline__ float sweep_quads(lds_u8* const (&slots)[DEPTH], Quad
                 const uint32_t last = b + DEPTH - 1U < blocks ? b + DEPTH - 1U : blocks;
                 wait_stages_ahead<kQuadCopies>(last - 1U - b);
                 if (b + DEPTH - 1U < blocks) source.start(slots[(s + DEPTH - 1) % DEPTH]);
-                quad_block_compute(slots[s], b, vd, vf, acc);
+                if (Q5K) quad_block_compute_q5k(slots[s], b, vd, vf, acc);
+                else quad_block_compute(slots[s], b, vd, vf, acc);
             }
         }
     }

@@ -310,7 +310,7 @@ int32_t mi355_executor_run(void* executor, const mi355_expert_job* job, mi355_st
     hipStream_t st = hs(stream);
     clear_word_kernel<<<1, 1, 0, st>>>(x->job_status);
     const uint32_t items = job->count;
-    if (w.gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, k, items);
+    if (w.gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<4><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, k, items);
     else if (items <= 16U) project_quad_kernel<4><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, k, items);
     else if (items <= kQuadMaxItems) project_quad_kernel<2><<<dim3(w.ffn / 32U, items), 256, 0, st>>>(w, k, items);
     else launch_project_nb<4>(w, k, items, dim3(w.ffn / 32U, items), st);

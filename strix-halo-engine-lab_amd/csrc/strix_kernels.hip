@@ -762,20 +762,27 @@ __global__ __launch_bounds__(256) void project_quad_kernel(mi355_moe_weights w, 
     }
 }
 
-// The same for Q5_K gate / up tensors (q5k_quads.hpp), for every assignment of the item in turn.
+// The same for Q5_K gate / up tensors (176-byte blocks through the same ring), for every assignment of the item in turn.
+template <int DEPTH>
 __global__ __launch_bounds__(256) void project_q5k_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments) {
+    STRIX_QUAD_SLOTS(DEPTH)
     __shared__ float wg_amax[4];
     __shared__ int wg_sum[4], wg_bad[4];
     const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), blockIdx.y);
     const uint32_t e = item.e, begin = item.begin, end = item.end;
-    const uint32_t lane = threadIdx.x & 63U, wave = threadIdx.x >> 6, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x;
+    const uint32_t lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2, grp = blockIdx.x;
     const uint32_t f0 = grp * 32U + 8U * wave;
-    const uint8_t* wrow = (lane < 32U ? w.gate : w.up) + static_cast<size_t>(e) * w.gate_expert_stride +
-                          static_cast<size_t>(f0 + (rr & 7U)) * w.gate_row_stride;
+    const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(f0) * w.gate_row_stride;
+    const uint8_t* gate = w.gate + base;
+    const uint8_t* up = w.up + base;
+    const size_t stride = w.gate_row_stride;
+    lds_u8* const (&sl)[DEPTH] = slots;
     const bool mine = lane < 32U && p == 0;                   // the lane that publishes feature f0 + rr
     for (uint32_t a = begin; a < end; ++a) {
         const uint32_t sidx = __builtin_amdgcn_readfirstlane(ordered(r, plan_order_at(w.experts), a)), row = r.row_of(sidx);
-        const float value = sweep_q5k_row(wrow, w.hidden / 256U, r.in, row, p);
+        QuadSourceT<11> source;
+        source.init([&](uint32_t q) { return q < 8U ? gate + q * stride : up + (q - 8U) * stride; }, r.in.codes_of(row));
+        const float value = sweep_quads<DEPTH, true>(sl, source, w.hidden / 256U, r.in, row);
         const float other = __shfl_xor(value, 32);
         const float g = lane < 32U ? value : other, u = lane < 32U ? other : value;
         float gc = g, uc = u;
@@ -1148,7 +1155,10 @@ inline bool quad_sweep(const mi355_moe_weights& w, uint32_t rows) {
 // grouped: the plan's items hold several assignments (the one-assignment sweeps do not apply)
 inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st, bool grouped = false) {
     if (w.gate_type == MI355_TYPE_Q5_K) {
-        project_q5k_kernel<<<dim3(w.ffn / 32U, umax), 256, 0, st>>>(w, r, rows * w.top_k);
+        // the deepest ring at which every workgroup of the launch is resident (4 waves x DEPTH x 4 KB each)
+        const uint64_t groups = static_cast<uint64_t>(w.ffn / 32U) * umax;
+        if (groups * 4U <= resident_waves(4U * kQuadSlotBytes)) project_q5k_kernel<4><<<dim3(w.ffn / 32U, umax), 256, 0, st>>>(w, r, rows * w.top_k);
+        else project_q5k_kernel<2><<<dim3(w.ffn / 32U, umax), 256, 0, st>>>(w, r, rows * w.top_k);
         return;
     }
     if (!grouped && quad_sweep(w, rows)) {
