@@ -274,6 +274,10 @@ def prefill_config4(strix, torch, gen, keep=False, reps=10):
         "experts_ms": sec_f16 * 1e3, "experts_TFLOPs": flops_experts / sec_f16 / 1e12, "experts_frac": flops_experts / sec_f16 / MFMA_F16_PEAK_FLOPS,
         "router_ms": sec_route * 1e3, "shared_expert_ms": sec_shared * 1e3, "shared_expert_TFLOPs": flops_shared / sec_shared / 1e12,
         "note": "FAST class (fp16 MFMA on exact integer operands sc*q, fp32 block scales and accumulation), tolerance 2e-3 against the exact-weight product; router exact-order"}
+    # the routed experts of the same workload in the bit-exact integer-dot class (int8 matrix-core group dots, the reference's fp32
+    # chain on the vector ALU), router included: what exactness costs beside the FAST class
+    sec_int = time_steps(torch, lambda i: layer.run_layer(xp, wr, bias=bias), 3, 1)
+    out["routed_experts_integer_class_ms"] = sec_int * 1e3
     if keep:
         # the same expert in the integer-dot class (A8 image, gate / up, SwiGLU + A8, down), for the comparison in --extra
         def shared(i):
