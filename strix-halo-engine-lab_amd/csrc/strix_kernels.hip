@@ -1181,7 +1181,12 @@ inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t row
     if (w.down_type != MI355_TYPE_Q4_K) {      // Q8_0 / Q5_1 (blocks of 32, four chains per row) and Q6_K (pairs per super-block)
         const uint32_t assignments = rows * w.top_k, items_at = plan_items_at(w.experts, assignments), order_at = plan_order_at(w.experts);
         const dim3 grid(w.hidden / kDownGroupsRows, umax);
-        if (w.down_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+        // Q5_1 rows of whole super-blocks at 16-byte aligned addresses stream through a copy ring (its depth by residency)
+        if (w.down_type == MI355_TYPE_Q5_1 && w.ffn % 256U == 0 && w.down_row_stride % 16U == 0 && w.down_expert_stride % 16U == 0) {
+            if (static_cast<uint64_t>(grid.x) * grid.y * 4U <= resident_waves(4U * group_slot_bytes())) down_q51_ring_kernel<4><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+            else down_q51_ring_kernel<2><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+        }
+        else if (w.down_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         else if (w.down_type == MI355_TYPE_Q5_1) down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         else down_q6k_kernel<<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         return;
