@@ -264,19 +264,21 @@ __device__ __forceinline__ void route_batch_block(BatchTiles& lds, const RouteAr
 constexpr uint32_t kChainChunk = 512;                 // features per ring slot
 constexpr uint32_t kChainPitch = kChainChunk + 4;     // floats; +16 bytes keeps the 8 weight rows on different banks
 constexpr uint32_t kChainExperts = 8;
-struct __attribute__((aligned(16))) ChainSlot {
+template <bool NORM>
+struct __attribute__((aligned(16))) ChainSlotT {
     float w[kChainExperts][kChainPitch];
     float x[kChainChunk];                             // the row's features as fp32
     uint32_t raw[kChainChunk / 2];                    // fp16 / bf16 input as copied (unused for fp32 input)
-    float nw[kChainChunk];                            // the norm weights of the chunk (fused RMSNorm only)
+    float nw[NORM ? kChainChunk : 4];                 // the norm weights of the chunk (fused RMSNorm only)
 };
+// Four slots of the plain form are 78,336 bytes: two one-wave workgroups fit a compute unit's 160 KB (with the norm weights: one).
 template <int KIND, bool NORM = false> constexpr uint32_t chain_copies() { return 2U * kChainExperts + (KIND == 0 ? 2U : 1U) + (NORM ? 2U : 0U); }
 
 // Start the copy of features [k0, k0 + 512) of 8 router-weight rows and of the activation row. Every chunk issues the
 // same number of copy instructions (the waits count them): lanes past the end of the row re-fetch its last piece into
 // slot positions that are never read.
 template <int KIND, bool NORM = false>
-__device__ __forceinline__ void chain_start(ChainSlot& slot, const RouteArgs& a, uint32_t row, uint32_t e0, uint32_t k0) {
+__device__ __forceinline__ void chain_start(ChainSlotT<NORM>& slot, const RouteArgs& a, uint32_t row, uint32_t e0, uint32_t k0) {
     const uint32_t lane = threadIdx.x & 63U;
     if constexpr (NORM) {       // (a null norm weight is a unit scale: the router weights stand in and are not used)
         const float* nsrc = a.norm_w ? a.norm_w : a.wr;
@@ -318,7 +320,7 @@ __device__ __forceinline__ void chain_start(ChainSlot& slot, const RouteArgs& a,
 // would also wait for every copy in flight, i.e. drain the three chunks the ring keeps ahead of the chain.
 __device__ __forceinline__ void chain_publish() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 template <int KIND, bool NORM = false>
-__device__ __forceinline__ void chain_widen(ChainSlot& slot, float factor = 1.0F, bool scaled = false) {
+__device__ __forceinline__ void chain_widen(ChainSlotT<NORM>& slot, float factor = 1.0F, bool scaled = false) {
     if constexpr (KIND == 0 && NORM) {
         // fp32 rows arrive as they are: scale them in place, y = (x * r) * w
         const uint32_t lane = threadIdx.x & 63U;
@@ -360,7 +362,8 @@ __device__ __forceinline__ void chain_widen(ChainSlot& slot, float factor = 1.0F
 // no instruction of its own). Measured on MI355X a wave pays ~5 cycles per dependent fma and ~9 per ds_read_b128, with no
 // overlap between them; the operands of the next 16 features are requested before the current 16 are chained.
 struct ChainStep { f32x4 w[4]; float x; };
-__device__ __forceinline__ void chain_load(ChainStep& s, const ChainSlot& slot, uint32_t el, uint32_t k) {
+template <bool NORM>
+__device__ __forceinline__ void chain_load(ChainStep& s, const ChainSlotT<NORM>& slot, uint32_t el, uint32_t k) {
     const float* wrow = slot.w[el] + k;
 #pragma unroll
     for (uint32_t i = 0; i < 4U; ++i) s.w[i] = *reinterpret_cast<const f32x4*>(wrow + 4U * i);
@@ -399,13 +402,14 @@ __device__ __forceinline__ void chain_wait() { __builtin_amdgcn_s_waitcnt((N & 1
 // Logits of experts [e0, e0 + 8) for one row -> scores[row][expert] (+ bias), stored for readers in other workgroups of
 // the same launch. hidden % 32 == 0. slots: 4 separate LDS objects.
 template <int KIND, bool NORM = false>
-__device__ __forceinline__ void route_chain_block(ChainSlot* const (&slots)[4], const RouteArgs& a, uint32_t row, uint32_t e0, float r = 1.0F) {
+__device__ __forceinline__ void route_chain_block(ChainSlotT<NORM>* const (&slots)[4], const RouteArgs& a, uint32_t row, uint32_t e0, float r = 1.0F) {
     constexpr uint32_t NI = chain_copies<KIND, NORM>();
     const uint32_t lane = threadIdx.x & 63U, chunks = (a.hidden + kChainChunk - 1U) / kChainChunk;
     const bool butterfly = a.p.logits_order == MI355_LOGITS_LANE32_BUTTERFLY;
     const uint32_t el = lane & 7U;                      // chain form: the lane's expert
     const uint32_t bh = lane >> 5, bl = lane & 31U;     // butterfly form: experts bh, bh + 2, bh + 4, bh + 6; partial sum bl
     float acc = 0.0F, part[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+    chain_publish();      // a caller may have used slot memory as scratch (the norm factor): those LDS operations are complete before any copy
 #pragma unroll
     for (uint32_t s = 0; s < 3U; ++s)
         if (s < chunks) chain_start<KIND, NORM>(*slots[s], a, row, e0, s * kChainChunk);
@@ -420,7 +424,7 @@ __device__ __forceinline__ void route_chain_block(ChainSlot* const (&slots)[4], 
                 else if (ahead == 1) chain_wait<NI>();
                 else chain_wait<2 * NI>();
                 if (c + 3U < chunks) chain_start<KIND, NORM>(*slots[(s + 3U) % 4U], a, row, e0, (c + 3U) * kChainChunk);
-                ChainSlot& slot = *slots[s];
+                ChainSlotT<NORM>& slot = *slots[s];
                 chain_widen<KIND, NORM>(slot, r, a.norm_w != nullptr);
                 const uint32_t kc = a.hidden - c * kChainChunk < kChainChunk ? a.hidden - c * kChainChunk : kChainChunk;
                 if (!butterfly) {

@@ -290,13 +290,17 @@ __global__ __launch_bounds__(256, 2) void route_batch_kernel(RouteArgs a) {
 // fields of the plan are not written), so nothing waits for the other rows. Every ticket word is left zero.
 template <int KIND, bool NORM = false>
 __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
-    __shared__ ChainSlot slot0;
-    __shared__ ChainSlot slot1;
-    __shared__ ChainSlot slot2;
-    __shared__ ChainSlot slot3;
-    __shared__ __attribute__((aligned(16))) float sel_p[kRouteMaxExperts];
+    __shared__ ChainSlotT<NORM> slot0;
+    __shared__ ChainSlotT<NORM> slot1;
+    __shared__ ChainSlotT<NORM> slot2;
+    __shared__ ChainSlotT<NORM> slot3;
     __shared__ uint32_t flag;
-    ChainSlot* const slots[4] = {&slot0, &slot1, &slot2, &slot3};
+    ChainSlotT<NORM>* const slots[4] = {&slot0, &slot1, &slot2, &slot3};
+    // the scratch of the row's norm factor and of the select lives in the fourth slot, which the ring first fills after the norm
+    // factor is known and which is free again once the chain has run: LDS per workgroup stays under half a compute unit's, so a
+    // launch of more one-wave workgroups than compute units (16 rows x 160 experts: 320) still runs in one round (61 -> 32 us)
+    static_assert(sizeof(ChainSlotT<NORM>) >= kRouteMaxExperts * sizeof(float), "select scratch");
+    float* const sel_p = reinterpret_cast<float*>(&slot3);
     const uint32_t bid = blockIdx.x, lane = threadIdx.x, neb = (a.p.experts + 7U) / 8U;
     uint32_t* tickets = a.plan ? a.plan + kPlanTicketsAt : nullptr;
     if (bid < a.route_blocks) {
