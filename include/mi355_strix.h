@@ -345,6 +345,33 @@ typedef struct mi355_slot_merge_tail {
 } mi355_slot_merge_tail;
 int32_t mi355_a8_enqueue_down_rawdots_merge(const mi355_a8_down_request*, const mi355_a8_down_bindings*, const mi355_slot_merge_tail*, mi355_stream);
 
+/* Union rows form: a verify window of R <= 8 rows, each with its top_k <= 16 routes, reads every distinct expert ONCE
+ * (include/strix/moe/expert_union.hpp:1-57). `plan` is the expert-union plan, MI355_UNION_PLAN_BYTES in the caller's memory:
+ * header {count, rows, top_k, 0} (4 x uint32), then 128 entries {uint32 expert, uint8 slot[8]}: the distinct experts in
+ * first-occurrence order of (row, slot) ascending and, per row, the slot that row holds the expert in (0xff: not chosen).
+ * mi355_a8_enqueue_probe_union builds it on the device (byte for byte expert_union::build for the `count` entries; the
+ * others hold expert 0 and 0xff slots), the down entry points read it. Per (row, slot, output) the arithmetic is the
+ * single-row form's: every output is bitwise that of R single-row calls.
+ *   mi355_a8_validate_union / _down_union = validate_union / validate_down_union   src/moe_q4k_a8_contract.cpp:373-405,
+ *                                                                                  src/moe_a8_down_contract.cpp:83-113
+ *   mi355_a8_enqueue_probe_union / _down_activation_quantize_union / _down_rawdots_union
+ *                                         = the entry points of the same names     src/hip_moe_q4k_a8_probe.hip:1172-1221
+ * Admission as in the reference: R <= 8, K <= 16, Q4_K gate / up (down: Q4_K or Q6_K), every row slice of the per-row views
+ * a single-row bundle of its own (16-byte aligned: top_k % 4 == 0 when R > 1), the plan view 16-byte aligned, exactly
+ * MI355_UNION_PLAN_BYTES and disjoint from every other view. (The reference's hidden <= 1536 bound is its kernel's register
+ * staging; hidden is bounded here as in mi355_a8_validate.) An expert id >= experts, or one named twice by the same row,
+ * sets MI355_STATUS_INVALID_ROUTE in the status word, leaves count = 0 and nothing is projected. */
+#define MI355_UNION_MAX_ROWS 8u
+#define MI355_UNION_MAX_TOP_K 16u
+#define MI355_UNION_PLAN_BYTES 1552u
+int32_t mi355_a8_validate_union(const mi355_a8_request*, const mi355_a8_bindings*, mi355_device_bytes plan);
+int32_t mi355_a8_enqueue_probe_union(const mi355_a8_request*, const mi355_a8_bindings*, mi355_device_bytes plan, mi355_stream);
+int32_t mi355_a8_validate_down_union(const mi355_a8_down_request*, const mi355_a8_down_bindings*, uint32_t rows, mi355_device_bytes plan);
+int32_t mi355_a8_enqueue_down_activation_quantize_union(const mi355_a8_down_request*, const mi355_a8_down_bindings*, uint32_t rows,
+                                                        mi355_device_bytes plan, uint32_t exp_kind, mi355_stream);
+int32_t mi355_a8_enqueue_down_rawdots_union(const mi355_a8_down_request*, const mi355_a8_down_bindings*, uint32_t rows, mi355_device_bytes plan,
+                                            mi355_stream);
+
 /* ------------------------------------------------------------------------------------------------------
  * The strided form of the per-row views: the reference's multi-row entry binds every view as Strided<T>{base, stride in
  * bytes}, row r at base + r * stride (Rows, include/strix/cuda/qwen_moe.hpp:34-37,55-76 = the views of the HIP

@@ -9,6 +9,7 @@
 #include "strix/ggml_dequant.hpp"
 #include "strix/moe/activation_policy.hpp"
 #include "strix/moe/combine.hpp"
+#include "strix/moe/expert_union.hpp"
 #include "strix/moe/route_policy.hpp"
 #include "strix/moe_a8_down_contract.hpp"
 #include "strix/moe_q4k_a8_contract.hpp"
@@ -272,6 +273,42 @@ int ref_a8_validate_down(int enabled, const char* identity, std::uint32_t hidden
     for (int i = 0; i < 9; ++i) v[i] = a8::DeviceBytes{static_cast<std::uintptr_t>(views[2 * i]), views[2 * i + 1]};
     const a8::DownBindings b{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
     return guarded([&] { a8::validate_down(q, b); });
+}
+// The union rows form: validate_union / validate_down_union (src/moe_q4k_a8_contract.cpp:373-405, src/moe_a8_down_contract.cpp:83-113)
+// with the plan view as a tenth {address, bytes} pair, and expert_union::build (include/strix/moe/expert_union.hpp:34-57), whose
+// entries land in `entries` as 12 bytes each (at most 128); returns their number, -1 when build() refuses the ids.
+int ref_a8_validate_union(int enabled, const char* identity, int input_fp32, std::uint32_t hidden, std::uint32_t rows, std::uint32_t experts,
+                          std::uint32_t top_k, std::uint32_t logical_rows, std::uint32_t gate_type, std::uint32_t up_type, int fused, float limit,
+                          const std::uint64_t* views) {
+    a8::Request q;
+    q.enabled = enabled != 0; q.approved_numerical_identity = identity ? std::string_view(identity) : std::string_view();
+    q.input = input_fp32 ? a8::InputKind::fp32 : a8::InputKind::bf16;
+    q.shape = a8::Shape{hidden, rows, experts, top_k, logical_rows};
+    q.gate_type = gate_type; q.up_type = up_type; q.fused_gate_up = fused != 0; q.swiglu_limit = limit;
+    a8::DeviceBytes v[10];
+    for (int i = 0; i < 10; ++i) v[i] = a8::DeviceBytes{static_cast<std::uintptr_t>(views[2 * i]), views[2 * i + 1]};
+    const a8::Bindings b{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
+    return guarded([&] { a8::validate_union(q, b, v[9]); });
+}
+int ref_a8_validate_down_union(int enabled, const char* identity, std::uint32_t hidden, std::uint32_t intermediate, std::uint32_t experts,
+                               std::uint32_t top_k, std::uint32_t weight_type, float limit, std::uint32_t rows, const std::uint64_t* views) {
+    a8::DownRequest q;
+    q.enabled = enabled != 0; q.approved_numerical_identity = identity ? std::string_view(identity) : std::string_view();
+    q.shape = a8::DownShape{hidden, intermediate, experts, top_k};
+    q.weight_type = weight_type; q.swiglu_limit = limit;
+    a8::DeviceBytes v[10];
+    for (int i = 0; i < 10; ++i) v[i] = a8::DeviceBytes{static_cast<std::uintptr_t>(views[2 * i]), views[2 * i + 1]};
+    const a8::DownBindings b{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
+    return guarded([&] { a8::validate_down_union(q, b, rows, v[9]); });
+}
+int ref_expert_union_build(const std::uint32_t* ids, std::uint32_t rows, std::uint32_t top_k, std::uint32_t experts, unsigned char* entries) {
+    int count = -1;
+    guarded([&] {
+        const auto plan = strix::moe::expert_union::build(std::span<const std::uint32_t>(ids, std::size_t{rows} * top_k), rows, top_k, experts);
+        std::memcpy(entries, plan.data(), plan.size() * sizeof(strix::moe::expert_union::Entry));
+        count = static_cast<int>(plan.size());
+    });
+    return count;
 }
 const char* ref_a8_identity(std::uint32_t type, int down) {
     static std::string held;

@@ -18,6 +18,7 @@ EXP_GFX1151, EXP_DECLARED, EXP_LIBM = 0, 1, 2
 STATUS_INVALID_ROUTE, STATUS_NONFINITE_ACTIVATION, STATUS_INVALID_DELTA, STATUS_NONFINITE_PROJECTION, STATUS_AGGREGATE = 1, 2, 4, 8, 16
 E_INVALID_ARGUMENT, E_UNSUPPORTED, E_HIP = -1, -2, -3
 Q8_0_BLOCK, Q4_K_BLOCK = 34, 144
+UNION_MAX_ROWS, UNION_MAX_TOP_K, UNION_PLAN_BYTES = 8, 16, 1552      # expert-union plan of a verify window (mi355_a8_*_union)
 
 
 class StrixError(RuntimeError):
@@ -221,6 +222,11 @@ def lib():
         L.mi355_a8_enqueue_down_activation_quantize.argtypes = [P, P, U, U, P]
         L.mi355_a8_enqueue_down_rawdots.argtypes = [P, P, U, P]
         L.mi355_a8_enqueue_down_rawdots_merge.argtypes = [P, P, P, P]
+        L.mi355_a8_validate_union.argtypes = [P, P, DeviceBytes]
+        L.mi355_a8_enqueue_probe_union.argtypes = [P, P, DeviceBytes, P]
+        L.mi355_a8_validate_down_union.argtypes = [P, P, U, DeviceBytes]
+        L.mi355_a8_enqueue_down_activation_quantize_union.argtypes = [P, P, U, DeviceBytes, U, P]
+        L.mi355_a8_enqueue_down_rawdots_union.argtypes = [P, P, U, DeviceBytes, P]
         L.mi355_gguf_open.argtypes, L.mi355_gguf_open.restype = [C.c_char_p], P
         L.mi355_gguf_close.argtypes, L.mi355_gguf_close.restype = [P], None
         for name in ("tensor_count", "metadata_count", "alignment", "data_offset"):
@@ -251,6 +257,8 @@ EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi3
            "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
+           "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
+           "mi355_a8_enqueue_down_activation_quantize_union", "mi355_a8_enqueue_down_rawdots_union",
            "mi355_moe_strided_enqueue_prologue", "mi355_moe_strided_enqueue_csr", "mi355_moe_strided_enqueue_project", "mi355_moe_strided_enqueue_down",
            "mi355_moe_strided_enqueue_merge", "mi355_moe_strided_enqueue_commit", "mi355_moe_strided_enqueue", "mi355_executor_create",
            "mi355_executor_run", "mi355_executor_destroy", "mi355_gguf_open", "mi355_gguf_close", "mi355_gguf_tensor_count",
@@ -410,6 +418,25 @@ class A8Decode:
     def enqueue_down_rawdots(self, rows=None):
         q, b = self.down_request(), self.down_bindings(rows)
         check(lib().mi355_a8_enqueue_down_rawdots(C.byref(q), C.byref(b), rows or self.R, _stream()))
+
+    # ---- union rows form (include/strix/moe/expert_union.hpp): R <= 8 rows, every distinct expert read once
+    def union_plan(self):
+        """The caller's plan view: UNION_PLAN_BYTES of device memory, written by enqueue_probe_union."""
+        if getattr(self, "plan", None) is None:
+            self.plan = torch.zeros(UNION_PLAN_BYTES, dtype=torch.uint8, device=self.gate.device)
+        return self.plan
+
+    def enqueue_probe_union(self, rows=None):
+        q, b = self.request(rows), self.bindings(rows)
+        check(lib().mi355_a8_enqueue_probe_union(C.byref(q), C.byref(b), device_bytes(self.union_plan()), _stream()))
+
+    def enqueue_down_activation_quantize_union(self, rows=None, exp_kind=EXP_GFX1151):
+        q, b = self.down_request(), self.down_bindings(rows)
+        check(lib().mi355_a8_enqueue_down_activation_quantize_union(C.byref(q), C.byref(b), rows or self.R, device_bytes(self.union_plan()), exp_kind, _stream()))
+
+    def enqueue_down_rawdots_union(self, rows=None):
+        q, b = self.down_request(), self.down_bindings(rows)
+        check(lib().mi355_a8_enqueue_down_rawdots_union(C.byref(q), C.byref(b), rows or self.R, device_bytes(self.union_plan()), _stream()))
 
     def enqueue_down_rawdots_merge(self, route_weights, accumulation, output, record, domain=1, bf16_commit=False):
         """One row: rawdots, then the ordered slot merge, commit test and first-error record (SlotMergeTail)."""

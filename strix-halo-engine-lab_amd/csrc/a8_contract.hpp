@@ -9,6 +9,10 @@
 // shape.logical_rows may be 1..16 with the per-row views holding that many contiguous single-row extents (the reference's
 // union form without its plan view: an expert chosen by two rows is simply read twice).
 // Status words are the caller's and sticky: nothing here clears them, bits are OR-ed in.
+//   union rows form (a verify window of R <= 8 rows reads each distinct expert once): the plan of
+//   include/strix/moe/expert_union.hpp:17-57 built on the device, validate_union (src/moe_q4k_a8_contract.cpp:373-405),
+//   validate_down_union (src/moe_a8_down_contract.cpp:83-113), enqueue_probe_union / enqueue_down_*_union
+//   (src/hip_moe_q4k_a8_probe.hip:1172-1221). The items of the expert sweeps are then the plan's entries (q4k_rows.hpp).
 #pragma once
 
 namespace strix950 {
@@ -196,6 +200,86 @@ __global__ __launch_bounds__(1024) void a8_slot_merge_kernel(SlotMergeArgs t) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------- union rows
+inline bool a8_union_admits(uint32_t rows, uint32_t top_k) { return rows >= 1U && rows <= kUnionRows && top_k >= 1U && top_k <= kUnionTopK; }
+inline int32_t a8_union_plan_view(const mi355_device_bytes& plan) {
+    STRIX_REQUIRE(plan.address != 0 && plan.address % 16U == 0 && plan.bytes == kUnionPlanBytes && plan.bytes <= UINTPTR_MAX - plan.address,
+                  "A8 union plan view invalid: 16-byte aligned, exactly 1552 bytes");
+    return MI355_OK;
+}
+
+int32_t a8_validate_union(const mi355_a8_request* q, const mi355_a8_bindings* b, const mi355_device_bytes& plan) {
+    STRIX_REQUIRE(q && b, "A8 union probe: null request or bindings");
+    const mi355_a8_shape& s = q->shape;
+    STRIX_REQUIRE(a8_union_admits(s.logical_rows, s.top_k) && q->gate_type == MI355_TYPE_Q4_K, "A8 union rows admit R <= 8, K <= 16 and Q4_K gate / up only");
+    // every row slice is a single-row bundle of its own: with R > 1 the per-row extents keep the slices on 16 bytes
+    STRIX_REQUIRE(s.logical_rows == 1U || (s.top_k * 4U) % 16U == 0, "A8 union per-row views: every row slice must start on 16 bytes (top_k % 4 == 0 for R > 1)");
+    if (const int32_t rc = a8_validate(q, b)) return rc;
+    if (const int32_t rc = a8_union_plan_view(plan)) return rc;
+    const mi355_device_bytes views[9] = {b->input, b->gate, b->up, b->routes, b->codes, b->deltas, b->sums, b->status, b->output};
+    for (const mi355_device_bytes& v : views) STRIX_REQUIRE(!a8_overlap(plan, v), "A8 union plan must not overlap any other view");
+    return MI355_OK;
+}
+
+int32_t a8_validate_down_union(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t rows, const mi355_device_bytes& plan) {
+    STRIX_REQUIRE(q && b, "A8 down union: null request or bindings");
+    STRIX_REQUIRE(a8_union_admits(rows, q->shape.top_k) && (q->weight_type == MI355_TYPE_Q4_K || q->weight_type == MI355_TYPE_Q6_K),
+                  "A8 down union rows admit R <= 8, K <= 16 and the K-quant class (Q4_K / Q6_K) only");
+    if (const int32_t rc = a8_validate_down(q, b, rows)) return rc;
+    if (const int32_t rc = a8_union_plan_view(plan)) return rc;
+    const mi355_device_bytes views[9] = {b->intermediates, b->weights, b->routes, b->codes, b->deltas, b->sums, b->rawdots, b->status, b->aggregate_status};
+    for (size_t i = 0; i < 9; ++i) {
+        if (i == 8 && views[i].address == 0 && views[i].bytes == 0) continue;
+        STRIX_REQUIRE(!a8_overlap(plan, views[i]), "A8 down union views and the plan must be disjoint");
+    }
+    return MI355_OK;
+}
+
+// The union plan of R x top_k routes, one workgroup of two wavefronts, thread t = assignment t = (row t / top_k, slot t % top_k).
+// An assignment is a "first" when no earlier assignment names its expert; the firsts, in assignment order, are the entries.
+// An expert id >= experts or an expert named twice by one row sets MI355_STATUS_INVALID_ROUTE and leaves count = 0 (no sweep
+// runs). All 128 entries are written: the unused ones hold expert 0 and 0xff slots.
+__global__ __launch_bounds__(kUnionEntries) void a8_union_plan_kernel(const uint32_t* routes, uint32_t rows, uint32_t top_k, uint32_t experts,
+                                                                     uint32_t* plan, uint32_t* status) {
+    __shared__ uint32_t expert_of[kUnionEntries], entry_of_first[kUnionEntries], entry_expert[kUnionEntries];
+    __shared__ uint8_t entry_slots[kUnionEntries][kUnionRows];
+    __shared__ uint32_t firsts_in_wave0, invalid;
+    const uint32_t t = threadIdx.x, n = rows * top_k, lane = t & 63U;
+    if (t == 0) invalid = 0;
+    entry_expert[t] = 0;
+    reinterpret_cast<uint32_t*>(entry_slots[t])[0] = 0xffffffffU;
+    reinterpret_cast<uint32_t*>(entry_slots[t])[1] = 0xffffffffU;
+    const uint32_t e = t < n ? routes[t] : 0xffffffffU;
+    expert_of[t] = e;
+    __syncthreads();
+    uint32_t first = t;
+    bool bad = false;
+    if (t < n) {
+        for (uint32_t a = 0; a < t; ++a)
+            if (expert_of[a] == e) { first = a; break; }
+        bad = e >= experts || (first != t && first >= t - t % top_k);
+    }
+    const bool is_first = t < n && first == t;
+    const uint64_t firsts = __ballot(is_first);
+    if (t == 0) firsts_in_wave0 = static_cast<uint32_t>(__popcll(firsts));
+    if (__ballot(bad) != 0 && lane == 0) invalid = 1;
+    __syncthreads();
+    const uint32_t before = static_cast<uint32_t>(__popcll(firsts & ((1ULL << lane) - 1ULL))) + (t >= 64U ? firsts_in_wave0 : 0U);
+    if (is_first) { entry_of_first[t] = before; entry_expert[before] = e; }
+    __syncthreads();
+    if (t < n) entry_slots[entry_of_first[first]][t / top_k] = static_cast<uint8_t>(t % top_k);
+    __syncthreads();
+    if (t == kUnionEntries - 1U) {         // (the last thread of the second wave knows the number of entries)
+        const uint32_t count = before + (is_first ? 1U : 0U);
+        plan[0] = invalid ? 0U : count; plan[1] = rows; plan[2] = top_k; plan[3] = 0U;
+        if (invalid) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+    }
+    uint32_t* entry = plan + 4U + 3U * t;
+    entry[0] = entry_expert[t];
+    entry[1] = reinterpret_cast<const uint32_t*>(entry_slots[t])[0];
+    entry[2] = reinterpret_cast<const uint32_t*>(entry_slots[t])[1];
+}
+
 // the bundle of the single-row entry points: no plan, no job word of its own, R contiguous single-row extents per view
 inline RowsK a8_rows(const mi355_moe_weights& w) {
     return rows_k(mi355_moe_rows{}, w);
@@ -212,16 +296,20 @@ int32_t mi355_a8_validate_down(const mi355_a8_down_request* q, const mi355_a8_do
     return a8_validate_down(q, b, logical_rows);
 }
 
-int32_t mi355_a8_enqueue_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, mi355_stream stream) {
-    if (const int32_t rc = a8_validate(q, b)) return rc;          // the whole bundle is validated before the first enqueue
+namespace {
+// Probe of R logical rows. union_plan == nullptr: item i = assignment i (an expert chosen by two rows is read twice);
+// otherwise the plan is built first and the items are its entries (each distinct expert read once).
+int32_t a8_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, uint32_t* union_plan, hipStream_t st) {
     const mi355_a8_shape& s = q->shape;
-    hipStream_t st = hs(stream);
     const uint32_t R = s.logical_rows, groups = s.hidden / 32U;
     const uint8_t* x = reinterpret_cast<const uint8_t*>(b->input.address);
+    const uint32_t* routes = reinterpret_cast<const uint32_t*>(b->routes.address);
     uint32_t* status = reinterpret_cast<uint32_t*>(b->status.address);
+    if (union_plan) a8_union_plan_kernel<<<1, kUnionEntries, 0, st>>>(routes, R, s.top_k, s.experts, union_plan, status);
     const dim3 pgrid((groups + 7U) / 8U, R);
+    const uint32_t checked = union_plan ? 0U : s.top_k;       // (the union builder has checked the routes)
     const auto prologue = [&](auto kind) {
-        a8_probe_prologue_kernel<decltype(kind)::value><<<pgrid, 256, 0, st>>>(x, s.hidden, reinterpret_cast<const uint32_t*>(b->routes.address), s.experts, s.top_k,
+        a8_probe_prologue_kernel<decltype(kind)::value><<<pgrid, 256, 0, st>>>(x, s.hidden, routes, s.experts, checked,
             reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), status);
     };
     if (q->input == MI355_INPUT_F32) prologue(std::integral_constant<int, 0>{});
@@ -232,20 +320,41 @@ int32_t mi355_a8_enqueue_probe(const mi355_a8_request* q, const mi355_a8_binding
     w.gate = reinterpret_cast<const uint8_t*>(b->gate.address); w.up = reinterpret_cast<const uint8_t*>(b->up.address);
     w.gate_row_stride = moe_row_bytes(q->gate_type, s.hidden); w.gate_expert_stride = w.gate_row_stride * s.rows;
     w.exp_kind = MI355_EXP_GFX1151; w.swiglu_limit = INFINITY;
-    // projection only: output[(assignment * 2 + which) * rows + row], no plan (item i = assignment i), no image of h
+    // projection only: output[(assignment * 2 + which) * rows + row], no image of h
     RowsK r = a8_rows(w);
-    r.routes = reinterpret_cast<const uint32_t*>(b->routes.address);
+    r.routes = routes;
     r.in = dense_image(reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), s.hidden);
     r.status = status; r.job_status = status;
     r.status_rs = 0;                // one shared status word
     r.gate_out = reinterpret_cast<float*>(b->output.address); r.up_out = r.gate_out + s.rows; r.slot_stride = 2ULL * s.rows;
     r.inter_rs = 4ULL * s.top_k * r.slot_stride;
+    r.union_plan = union_plan;
     const uint32_t items = R * s.top_k;
-    if (q->gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
+    if (union_plan) launch_project_nb<8>(w, r, R, dim3(s.rows / 32U, items), st);       // up to 8 holders share one sweep of an entry's expert
+    else if (q->gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else if (items <= 16U) project_quad_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else if (items <= kQuadMaxItems) project_quad_kernel<2><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else launch_project_nb<4>(w, r, R, dim3(s.rows / 32U, items), st);
+    return MI355_OK;
+}
+}  // namespace
+
+int32_t mi355_a8_enqueue_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, mi355_stream stream) {
+    if (const int32_t rc = a8_validate(q, b)) return rc;          // the whole bundle is validated before the first enqueue
+    a8_probe(q, b, nullptr, hs(stream));
     STRIX_LAUNCHED("A8 probe");
+    return MI355_OK;
+}
+
+int32_t mi355_a8_validate_union(const mi355_a8_request* q, const mi355_a8_bindings* b, mi355_device_bytes plan) { return a8_validate_union(q, b, plan); }
+int32_t mi355_a8_validate_down_union(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t rows, mi355_device_bytes plan) {
+    return a8_validate_down_union(q, b, rows, plan);
+}
+
+int32_t mi355_a8_enqueue_probe_union(const mi355_a8_request* q, const mi355_a8_bindings* b, mi355_device_bytes plan, mi355_stream stream) {
+    if (const int32_t rc = a8_validate_union(q, b, plan)) return rc;
+    a8_probe(q, b, reinterpret_cast<uint32_t*>(plan.address), hs(stream));
+    STRIX_LAUNCHED("A8 union probe");
     return MI355_OK;
 }
 
@@ -264,7 +373,8 @@ int32_t mi355_a8_enqueue_down_activation_quantize(const mi355_a8_down_request* q
 }
 
 namespace {
-int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t logical_rows, hipStream_t st) {
+int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t logical_rows, hipStream_t st,
+                        const uint32_t* union_plan = nullptr) {
     const mi355_a8_down_shape& s = q->shape;
     mi355_moe_weights w{};
     w.hidden = s.hidden; w.ffn = s.intermediate; w.experts = s.experts; w.top_k = s.top_k; w.gate_type = MI355_TYPE_Q4_K; w.down_type = q->weight_type;
@@ -279,7 +389,11 @@ int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bind
     r.status_rs = 0;
     r.job_status = r.status;        // a non-finite projection recorded by the producer (bit 8) skips the rows, as in the layer entries
     const uint32_t items = logical_rows * s.top_k;
-    if (q->weight_type != MI355_TYPE_Q4_K) {
+    r.union_plan = union_plan;
+    if (union_plan) {               // K-quant only: the items are the plan's entries
+        if (q->weight_type == MI355_TYPE_Q6_K) down_q6k_kernel<<<dim3(s.hidden / kDownGroupsRows, items), 256, 0, st>>>(w, r, items, 0U, 0U);
+        else launch_down_nb<8>(w, r, logical_rows, dim3(s.hidden / 64U, items), st);
+    } else if (q->weight_type != MI355_TYPE_Q4_K) {
         const dim3 grid(s.hidden / kDownGroupsRows, items);
         if (q->weight_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
         else if (q->weight_type == MI355_TYPE_Q5_1) down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
@@ -295,6 +409,21 @@ int32_t mi355_a8_enqueue_down_rawdots(const mi355_a8_down_request* q, const mi35
     if (const int32_t rc = a8_validate_down(q, b, logical_rows)) return rc;
     a8_down_rawdots(q, b, logical_rows, hs(stream));
     STRIX_LAUNCHED("A8 down rawdots");
+    return MI355_OK;
+}
+
+int32_t mi355_a8_enqueue_down_activation_quantize_union(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t rows,
+                                                        mi355_device_bytes plan, uint32_t exp_kind, mi355_stream stream) {
+    if (const int32_t rc = a8_validate_down_union(q, b, rows, plan)) return rc;
+    // elementwise per (row, slot): the plan is admitted with the bundle and not read
+    return mi355_a8_enqueue_down_activation_quantize(q, b, rows, exp_kind, stream);
+}
+
+int32_t mi355_a8_enqueue_down_rawdots_union(const mi355_a8_down_request* q, const mi355_a8_down_bindings* b, uint32_t rows, mi355_device_bytes plan,
+                                            mi355_stream stream) {
+    if (const int32_t rc = a8_validate_down_union(q, b, rows, plan)) return rc;
+    a8_down_rawdots(q, b, rows, hs(stream), reinterpret_cast<const uint32_t*>(plan.address));
+    STRIX_LAUNCHED("A8 union down rawdots");
     return MI355_OK;
 }
 

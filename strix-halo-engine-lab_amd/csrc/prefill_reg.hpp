@@ -222,6 +222,9 @@ __global__ __launch_bounds__(kRgThreads) void prefill_reg_kernel(PrefillArgs a, 
                         part[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(frag[m % W], bcur, part[i], 0, 0, 0);
                     }
                     if (m + W < N) request(m + W);
+                    // the scheduler otherwise sinks the request down to its use (registers are scarce) and the MFMA then waits
+                    // for the whole LDS round trip: nothing moves across this point (1874 -> 1828 us gate / up, 1642 -> 1565 us down)
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 if (p == 1U) {
                     // this lane's M operand: the eight sub-blocks of super-block 2 g + half of the group

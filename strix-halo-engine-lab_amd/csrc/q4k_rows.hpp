@@ -89,6 +89,7 @@ struct RowsK : mi355_moe_rows {
     const mi355_expert_assignment* assignments;      // job form (src/cpu/core/routed_expert.hpp:47-49): item i = assignments[i]
     uint32_t top_k;
     uint32_t nonfinite_bit;   // what a non-finite gate / up / h value ORs into its row's status (8; the host executor's job: 1)
+    const uint32_t* union_plan;     // verify-window form: the expert-union plan (below) names the items instead of `plan`
 
     __device__ __forceinline__ void place(uint32_t i, uint32_t& row, uint32_t& slot) const {
         if (assignments) { row = assignments[i].row; slot = assignments[i].slot; }
@@ -130,7 +131,36 @@ struct RowsK : mi355_moe_rows {
 // forms of the reference entry points (include/strix/hip_moe_q4k_a8_probe.hpp:12, include/strix/hip_moe_a8_down.hpp:11-30) and
 // the host executor's Job bring no plan view.
 struct WorkItem { uint32_t e, begin, end; };
+
+// Expert-union plan of a verify window (include/strix/moe/expert_union.hpp:17-27): words {count, rows, top_k, 0}, then 128
+// entries of three words {expert, slot bytes of rows 0-3, of rows 4-7}; a slot byte 0xff = that row did not choose the
+// expert. Item u = entry u: its expert's weights are swept once for the rows that hold it, in ascending row order. The
+// positions of such an item are (u << 8) + i, i counting the holders.
+constexpr uint32_t kUnionRows = 8, kUnionTopK = 16, kUnionEntries = kUnionRows * kUnionTopK, kUnionPlanBytes = 16U + 12U * kUnionEntries;
+__device__ __forceinline__ uint32_t union_held(uint32_t four_slots) {      // one bit per byte that is not 0xff, at the byte's bit 7
+    const uint32_t y = ~four_slots;                                        // a byte of y is zero exactly where the slot byte is 0xff
+    return (((y & 0x7f7f7f7fU) + 0x7f7f7f7fU) | y) & 0x80808080U;
+}
+__device__ __forceinline__ WorkItem union_item(const uint32_t* plan, uint32_t u) {
+    if (u >= plan[0]) return {0U, 0U, 0U};
+    const uint32_t* entry = plan + 4U + 3U * u;
+    const uint32_t holders = static_cast<uint32_t>(__popc(union_held(entry[1])) + __popc(union_held(entry[2])));
+    return {entry[0], u << 8, (u << 8) + holders};
+}
+__device__ __forceinline__ uint32_t union_assignment(const uint32_t* plan, uint32_t position) {
+    const uint32_t* entry = plan + 4U + 3U * (position >> 8);
+    uint32_t left = position & 255U;
+    for (uint32_t row = 0; row < kUnionRows; ++row) {
+        const uint32_t slot = (entry[1U + (row >> 2)] >> (8U * (row & 3U))) & 255U;
+        if (slot == 255U) continue;
+        if (left == 0U) return row * plan[2] + slot;
+        --left;
+    }
+    return 0U;
+}
+
 __device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const RowsK& r, uint32_t items_at, uint32_t index) {
+    if (r.union_plan) return union_item(r.union_plan, index);
     if (r.plan) {
         const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * index);
         return {item.x, item.y, item.z};
@@ -144,7 +174,10 @@ __device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const 
     }
     return {e, index, e < w.experts ? index + 1U : index};      // an invalid route has no item (its row is flagged)
 }
-__device__ __forceinline__ uint32_t ordered(const RowsK& r, uint32_t order_at, uint32_t i) { return r.plan ? r.plan[order_at + i] : i; }
+__device__ __forceinline__ uint32_t ordered(const RowsK& r, uint32_t order_at, uint32_t i) {
+    if (r.union_plan) return union_assignment(r.union_plan, i);
+    return r.plan ? r.plan[order_at + i] : i;
+}
 
 // Per-lane source pointers of the nine pieces the lane copies in every stage. row_ptr(r) = first byte of row r (0..63).
 struct StageSource {

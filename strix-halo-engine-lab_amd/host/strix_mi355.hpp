@@ -27,6 +27,7 @@
 #include <string>
 #include <string_view>
 #include <type_traits>
+#include <vector>
 
 #include "mi355_strix.h"
 
@@ -147,6 +148,43 @@ inline Status enqueue_dense(const WeightView& weight, const DenseArguments& args
 }
 }  // namespace weight
 
+// ---------------------------------------------------------------------------------------------- expert union of a verify window
+// include/strix/moe/expert_union.hpp: the plan layout the union entry points of the A8 contract share, and its host builder
+// (the reference of the device builder inside enqueue_probe_union).
+namespace moe::expert_union {
+inline constexpr std::uint32_t max_rows = MI355_UNION_MAX_ROWS, max_top_k = MI355_UNION_MAX_TOP_K, max_assignments = max_rows * max_top_k;
+inline constexpr std::uint8_t no_slot = 0xFFU;
+struct Header { std::uint32_t count = 0, rows = 0, top_k = 0, reserved = 0; };
+struct Entry { std::uint32_t expert; std::uint8_t slot[max_rows]; };
+static_assert(sizeof(Header) == 16U && sizeof(Entry) == 12U);
+inline constexpr std::uint64_t plan_bytes = sizeof(Header) + std::uint64_t{max_assignments} * sizeof(Entry);
+static_assert(plan_bytes == MI355_UNION_PLAN_BYTES);
+[[nodiscard]] constexpr bool admits(std::uint32_t rows, std::uint32_t top_k) noexcept { return rows >= 1U && rows <= max_rows && top_k >= 1U && top_k <= max_top_k; }
+// ids: rows x top_k expert ids, row-major. std::invalid_argument on a shape outside admits(), an id >= experts or an id named
+// twice by one row.
+[[nodiscard]] inline std::vector<Entry> build(const std::uint32_t* ids, std::size_t count, std::uint32_t rows, std::uint32_t top_k, std::uint32_t experts) {
+    if (!admits(rows, top_k) || count != std::size_t{rows} * top_k) throw std::invalid_argument("expert union: rows <= 8, top_k <= 16 and rows x top_k ids required");
+    std::vector<Entry> plan;
+    for (std::size_t a = 0; a < count; ++a) {
+        const std::uint32_t e = ids[a], row = static_cast<std::uint32_t>(a / top_k);
+        if (e >= experts) throw std::invalid_argument("expert union: expert id out of range");
+        Entry* held = nullptr;
+        for (Entry& entry : plan)
+            if (entry.expert == e) { held = &entry; break; }
+        if (!held) {
+            Entry fresh;
+            fresh.expert = e;
+            for (std::uint8_t& slot : fresh.slot) slot = no_slot;
+            plan.push_back(fresh);
+            held = &plan.back();
+        }
+        if (held->slot[row] != no_slot) throw std::invalid_argument("expert union: expert repeated within one row");
+        held->slot[row] = static_cast<std::uint8_t>(a % top_k);
+    }
+    return plan;
+}
+}  // namespace moe::expert_union
+
 // ---------------------------------------------------------------------------------------------- A8 request / bindings
 namespace moe_q4k_a8 {
 inline constexpr float kSwigluNoClamp = std::numeric_limits<float>::infinity();
@@ -205,6 +243,19 @@ inline void enqueue_probe(const Request& request, const Bindings& bindings, mi35
     check(mi355_a8_enqueue_probe(&q.q, &b, stream));
 }
 
+// Union rows form (include/strix/moe_q4k_a8_contract.hpp:123-132, src/hip_moe_q4k_a8_probe.hip:1172-1191): shape.logical_rows = R
+// (1..8); the per-row views are R contiguous single-row extents; plan = moe::expert_union::plan_bytes, written by the probe.
+inline void validate_union(const Request& request, const Bindings& bindings, DeviceBytes plan) {
+    detail::CRequest q; detail::fill(request, q);
+    const mi355_a8_bindings b = detail::c(bindings);
+    check(mi355_a8_validate_union(&q.q, &b, detail::c(plan)));
+}
+inline void enqueue_probe_union(const Request& request, const Bindings& bindings, DeviceBytes plan, mi355_stream stream) {
+    detail::CRequest q; detail::fill(request, q);
+    const mi355_a8_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_probe_union(&q.q, &b, detail::c(plan), stream));
+}
+
 struct DownShape { std::uint32_t hidden = 0, intermediate = 0, experts = 0, top_k = 0; };
 struct DownRequest {
     bool enabled = false;
@@ -257,6 +308,22 @@ inline void enqueue_down_rawdots(const DownRequest& request, const DownBindings&
     const mi355_slot_merge_tail t{tail.tickets, tail.route_weights, tail.accumulation, tail.output, tail.output_bf16 ? 1U : 0U, tail.bf16_commit ? 1U : 0U,
                                   tail.record, tail.domain};
     check(mi355_a8_enqueue_down_rawdots_merge(&q.q, &b, &t, stream));
+}
+// Union rows form of the K-quant down class (include/strix/moe_a8_down_contract.hpp:57-60, src/hip_moe_q4k_a8_probe.hip:1192-1221).
+inline void validate_down_union(const DownRequest& request, const DownBindings& bindings, std::uint32_t rows, DeviceBytes plan) {
+    detail::CDownRequest q; detail::fill(request, q);
+    const mi355_a8_down_bindings b = detail::c(bindings);
+    check(mi355_a8_validate_down_union(&q.q, &b, rows, detail::c(plan)));
+}
+inline void enqueue_down_activation_quantize_union(const DownRequest& request, const DownBindings& bindings, std::uint32_t rows, DeviceBytes plan, mi355_stream stream) {
+    detail::CDownRequest q; detail::fill(request, q);
+    const mi355_a8_down_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_down_activation_quantize_union(&q.q, &b, rows, detail::c(plan), MI355_EXP_GFX1151, stream));
+}
+inline void enqueue_down_rawdots_union(const DownRequest& request, const DownBindings& bindings, std::uint32_t rows, DeviceBytes plan, mi355_stream stream) {
+    detail::CDownRequest q; detail::fill(request, q);
+    const mi355_a8_down_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_down_rawdots_union(&q.q, &b, rows, detail::c(plan), stream));
 }
 }  // namespace moe_q4k_a8
 

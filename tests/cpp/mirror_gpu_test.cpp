@@ -196,6 +196,58 @@ static void a8_single_row(const Layer& L) {
     expect(threw, "moe_q4k_a8::enqueue_probe throws std::invalid_argument without the identity approval");
 }
 
+// The union rows form: three rows, each naming all four experts in its own order, so every entry is held by every row.
+static void a8_union_rows(const Layer& L) {
+    namespace a8 = m::moe_q4k_a8;
+    namespace eu = m::moe::expert_union;
+    constexpr std::uint32_t R = T, K4 = 4;
+    const std::vector<std::uint32_t> routes{2, 0, 3, 1, 0, 1, 2, 3, 3, 2, 1, 0};
+    // the oracle's job over the same routes
+    std::vector<float> g(R * K4 * I), u(g.size()), h(g.size()), raw(R * K4 * H), hd(R * K4 * I / 32);
+    std::vector<std::int8_t> hc(R * K4 * I);
+    std::vector<std::int32_t> hs(R * K4 * I / 32);
+    std::vector<std::uint32_t> ostatus(R);
+    const std::uint64_t grb = H / 256 * 144, drb = I / 256 * 144;
+    const orc_expert_weights w{H, I, E, K4, 12, 12, L.gate.data(), L.up.data(), L.down.data(), grb * I, grb, drb * H, drb, 0, INFINITY};
+    const orc_expert_job job{L.c.data(), L.d.data(), L.s.data(), routes.data(), R, g.data(), u.data(), h.data(), hc.data(), hd.data(), hs.data(), raw.data(), ostatus.data()};
+    orc_routed_experts(&w, &job, 1);
+    Dev<std::uint8_t> gate(L.gate), up(L.up), down(L.down), plan(eu::plan_bytes);
+    Dev<std::uint16_t> input(L.x);
+    Dev<std::uint32_t> droutes(routes), status(1);
+    Dev<std::int8_t> codes(R * H), hcodes(R * K4 * I);
+    Dev<float> deltas(R * H / 32), output(R * K4 * 2 * I), hdeltas(R * K4 * I / 32), rawdots(R * K4 * H);
+    Dev<std::int32_t> sums(R * H / 32), hsums(R * K4 * I / 32);
+    a8::Request q;
+    q.enabled = true; q.approved_numerical_identity = a8::numerical_identity_for_gate_type(12); q.input = a8::InputKind::bf16;
+    q.shape = a8::Shape{H, I, E, K4, R};
+    const a8::Bindings b{input.bytes(), gate.bytes(), up.bytes(), droutes.bytes(), codes.bytes(), deltas.bytes(), sums.bytes(), status.bytes(), output.bytes()};
+    a8::validate_union(q, b, plan.bytes());
+    a8::enqueue_probe_union(q, b, plan.bytes(), nullptr);
+    const std::vector<std::uint8_t> got_plan = plan.get();
+    const std::vector<eu::Entry> want_plan = eu::build(routes.data(), routes.size(), R, K4, E);
+    eu::Header header;
+    std::memcpy(&header, got_plan.data(), sizeof header);
+    expect(header.count == want_plan.size() && header.count == E && header.rows == R && header.top_k == K4 &&
+           std::memcmp(got_plan.data() + sizeof header, want_plan.data(), want_plan.size() * sizeof(eu::Entry)) == 0,
+           "moe_q4k_a8::enqueue_probe_union: device plan == moe::expert_union::build");
+    const std::vector<float> out = output.get();
+    bool ok = true;
+    for (std::uint32_t a = 0; a < R * K4; ++a)
+        ok = ok && std::memcmp(out.data() + (a * 2) * I, g.data() + a * I, I * 4) == 0 && std::memcmp(out.data() + (a * 2 + 1) * I, u.data() + a * I, I * 4) == 0;
+    expect(ok, "moe_q4k_a8::enqueue_probe_union: gate / up rows of every (row, slot) == oracle");
+    a8::DownRequest dq;
+    dq.enabled = true; dq.approved_numerical_identity = a8::down_numerical_identity(12); dq.shape = a8::DownShape{H, I, E, K4}; dq.weight_type = 12;
+    const a8::DownBindings db{output.bytes(), down.bytes(), droutes.bytes(), hcodes.bytes(), hdeltas.bytes(), hsums.bytes(), rawdots.bytes(), status.bytes(), {0, 0}};
+    a8::validate_down_union(dq, db, R, plan.bytes());
+    a8::enqueue_down_activation_quantize_union(dq, db, R, plan.bytes(), nullptr);
+    a8::enqueue_down_rawdots_union(dq, db, R, plan.bytes(), nullptr);
+    expect(same_bits(hcodes.get(), hc) && same_bits(hdeltas.get(), hd) && same_bits(rawdots.get(), raw) && status.get()[0] == 0,
+           "moe_q4k_a8::enqueue_down_*_union: h image and raw dots == oracle, clean status");
+    bool threw = false;
+    try { a8::validate_union(q, b, a8::DeviceBytes{plan.bytes().address, eu::plan_bytes - 4}); } catch (const std::invalid_argument&) { threw = true; }
+    expect(threw, "moe_q4k_a8::validate_union throws std::invalid_argument for a plan view of another extent");
+}
+
 static void strided_rows(const Layer& L) {
     namespace qm = m::qwen_moe;
     const Layer::Result ref = L.oracle(L.down8, 8);
@@ -290,6 +342,7 @@ int main() {
         kernel_table();
         const Layer L;
         a8_single_row(L);
+        a8_union_rows(L);
         strided_rows(L);
         executor_job(L);
     } catch (const std::exception& e) {

@@ -432,3 +432,43 @@ def base_linear(qtype, weight, row_stride, outputs, n_in, x, threads=0):
     lib().orc_base_linear(qtype, _ptr(weight, u8p), C.c_uint64(row_stride), outputs, n_in, _ptr(x, f32p), rows,
                           x.shape[1], _ptr(y, f32p), outputs, threads or lib().orc_max_threads())
     return y
+
+
+# ---------------------------------------------------------------- expert union of a verify window
+UNION_MAX_ROWS, UNION_MAX_TOP_K, UNION_NO_SLOT, UNION_PLAN_BYTES = 8, 16, 0xFF, 16 + 128 * 12
+
+
+def expert_union_build(ids, rows, top_k, experts):
+    """The host reference of the union plan (include/strix/moe/expert_union.hpp:34-57): the distinct experts of rows x top_k
+    ids in first-occurrence order of (row, slot) ascending, each with the slot every row holds it in (0xff: not chosen).
+    Returns [(expert, [slot of row 0..7])]. ValueError on a shape outside R <= 8, K <= 16, an id >= experts, or an id
+    repeated within one row."""
+    ids = [int(v) for v in np.asarray(ids).reshape(-1)]
+    if not (1 <= rows <= UNION_MAX_ROWS and 1 <= top_k <= UNION_MAX_TOP_K) or len(ids) != rows * top_k:
+        raise ValueError("expert union: rows <= 8, top_k <= 16 and rows x top_k ids required")
+    out = []
+    for r in range(rows):
+        for s in range(top_k):
+            e = ids[r * top_k + s]
+            if e >= experts:
+                raise ValueError("expert union: expert id out of range")
+            u = next((i for i, entry in enumerate(out) if entry[0] == e), len(out))
+            if u == len(out):
+                out.append((e, [UNION_NO_SLOT] * UNION_MAX_ROWS))
+            if out[u][1][r] != UNION_NO_SLOT:
+                raise ValueError("expert union: expert repeated within one row")
+            out[u][1][r] = s
+    return out
+
+
+def expert_union_plan_bytes(entries, rows, top_k):
+    """The device layout of a plan (expert_union.hpp:17-27): Header {count, rows, top_k, 0}, then 128 Entry {u32 expert,
+    u8 slot[8]}; the entries past count as the device builder leaves them (expert 0, 0xff slots)."""
+    plan = np.zeros(UNION_PLAN_BYTES, np.uint8)
+    plan[:16] = np.array([len(entries), rows, top_k, 0], np.uint32).view(np.uint8)
+    body = plan[16:].reshape(128, 12)
+    body[:, 4:] = UNION_NO_SLOT
+    for u, (e, slots) in enumerate(entries):
+        body[u, :4] = np.array([e], np.uint32).view(np.uint8)
+        body[u, 4:] = np.array(slots, np.uint8)
+    return plan

@@ -235,3 +235,132 @@ def test_down_admission_agrees_with_the_reference(lib, ref, pkg):
         q = down_request(lib)
         mine, _ = call_down(lib, ref, pkg, q, lay_out(down_required(2048, 768, 128, 8, max(R, 1), 12)), R=R)
         assert mine == ok, R
+
+
+# ------------------------------------------------------------------------------------------------ union rows form
+def test_union_plan_oracle_on_the_reference_vectors():
+    """The known answers of the reference's own host test (tests/moe_expert_union_tests.cpp:33-66)."""
+    NO = orc.UNION_NO_SLOT
+    p1 = orc.expert_union_build([7, 3, 9], 1, 3, 16)
+    assert [e for e, _ in p1] == [7, 3, 9] and p1[1][1][0] == 1 and p1[1][1][1] == NO
+    ids = [5, 1, 2, 2, 6, 5, 7, 1, 6]
+    p = orc.expert_union_build(ids, 3, 3, 8)
+    assert [e for e, _ in p] == [5, 1, 2, 6, 7]
+    assert p[0][1][:3] == [0, 2, NO] and p[1][1][:3] == [1, NO, 1] and p[3][1][:3] == [NO, 1, 2]
+    assert sum(s != NO for _, slots in p for s in slots) == 9
+    for bad in (([0] * 18, 9, 2, 8), ([0] * 17, 1, 17, 32), ([1, 8], 1, 2, 8), ([3, 3], 1, 2, 8)):
+        with pytest.raises(ValueError):
+            orc.expert_union_build(*bad)
+    assert len(orc.expert_union_build([3, 4, 3, 4], 2, 2, 8)) == 2
+    assert orc.UNION_PLAN_BYTES == 16 + 128 * 12
+
+
+def test_union_plan_oracle_equals_the_compiled_reference(ref):
+    """orc.expert_union_build against expert_union::build of the reference (include/strix/moe/expert_union.hpp:34-57), entry bytes and refusals."""
+    import numpy as np
+    rng = np.random.default_rng(31)
+    refused = 0
+    for case in range(300):
+        rows, top_k = int(rng.integers(1, 9)), int(rng.integers(1, 17))
+        experts = int(rng.choice([top_k, top_k + 3, 64, 512]))
+        ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(rows)]).astype(np.uint32)
+        if case % 7 == 3:
+            ids[rng.integers(rows), rng.integers(top_k)] = experts + int(rng.integers(0, 3))        # out of range
+        if case % 7 == 5 and top_k > 1:
+            r = int(rng.integers(rows))
+            ids[r, 1] = ids[r, 0]                                                                 # repeated within a row
+        entries = np.zeros(128 * 12, np.uint8)
+        n = ref.ref_expert_union_build(ids.ctypes.data_as(C.c_void_p), rows, top_k, experts, entries.ctypes.data_as(C.c_void_p))
+        try:
+            mine = orc.expert_union_build(ids, rows, top_k, experts)
+        except ValueError:
+            assert n == -1, (case, ids)
+            refused += 1
+            continue
+        assert n == len(mine), (case, ids)
+        want = orc.expert_union_plan_bytes(mine, rows, top_k)[16:16 + 12 * n]
+        assert np.array_equal(entries[:12 * n], want), (case, ids)
+    assert refused > 40
+
+
+def call_probe_union(lib, ref, pkg, q, views, plan):
+    req = pkg.A8Request(q["enabled"], q["identity"], pkg.INPUT_F32 if q["fp32"] else pkg.INPUT_BF16,
+                        pkg.A8Shape(q["hidden"], q["rows"], q["experts"], q["top_k"], q["R"]), q["gate"], q["up"], q["fused"], q["limit"])
+    b = pkg.A8Bindings(*[pkg.DeviceBytes(a, n) for a, n in views])
+    lib.mi355_a8_validate_union.argtypes = [C.c_void_p, C.c_void_p, pkg.DeviceBytes]
+    mine = lib.mi355_a8_validate_union(C.byref(req), C.byref(b), pkg.DeviceBytes(*plan)) == 0
+    flat = (C.c_uint64 * 20)(*[v for pair in list(views) + [plan] for v in pair])
+    theirs = ref.ref_a8_validate_union(q["enabled"], q["identity"], int(q["fp32"]), q["hidden"], q["rows"], q["experts"], q["top_k"], q["R"], q["gate"],
+                                       q["up"], q["fused"], C.c_float(q["limit"]), flat) == 0
+    return mine, theirs
+
+
+def call_down_union(lib, ref, pkg, q, views, plan, R):
+    req = pkg.A8DownRequest(q["enabled"], q["identity"], pkg.A8DownShape(q["hidden"], q["inter"], q["experts"], q["top_k"]), q["type"], q["limit"])
+    b = pkg.A8DownBindings(*[pkg.DeviceBytes(a, n) for a, n in views])
+    lib.mi355_a8_validate_down_union.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, pkg.DeviceBytes]
+    mine = lib.mi355_a8_validate_down_union(C.byref(req), C.byref(b), R, pkg.DeviceBytes(*plan)) == 0
+    flat = (C.c_uint64 * 20)(*[v for pair in list(views) + [plan] for v in pair])
+    theirs = ref.ref_a8_validate_down_union(q["enabled"], q["identity"], q["hidden"], q["inter"], q["experts"], q["top_k"], q["type"], C.c_float(q["limit"]),
+                                            R, flat) == 0
+    return mine, theirs
+
+
+def test_union_admission_agrees_with_the_reference(lib, ref, pkg):
+    """validate_union / validate_down_union (src/moe_q4k_a8_contract.cpp:373-405, src/moe_a8_down_contract.cpp:83-113) in the Hy4
+    preset geometry of the reference's host test (tests/moe_expert_union_tests.cpp:69-143) and around it."""
+    L, I, E, K = 1536, 1536, 512, 16
+    PLAN = orc.UNION_PLAN_BYTES
+
+    def probe(R, **over):
+        q = probe_request(lib, **{**dict(fp32=True, hidden=L, rows=I, experts=E, top_k=K, R=R), **over})
+        v = lay_out(probe_required(L, I, E, q["top_k"], R, q["gate"], True))
+        return q, v, [v[-1][0] + (v[-1][1] + 511) // 256 * 256, PLAN]
+    for R in (1, 2, 4, 8):
+        q, v, plan = probe(R)
+        assert call_probe_union(lib, ref, pkg, q, v, plan) == (True, True), R
+    q, v, plan = probe(9)
+    assert call_probe_union(lib, ref, pkg, q, v, plan) == (False, False)
+    q, v, plan = probe(2)
+    _, v3, _ = probe(3)
+    assert call_probe_union(lib, ref, pkg, q, v3, plan) == (False, False)                                  # per-row extents are R x the single-row one
+    assert call_probe_union(lib, ref, pkg, q, v, [plan[0], PLAN - 4]) == (False, False)                    # plan extent exact
+    assert call_probe_union(lib, ref, pkg, q, v, [plan[0] + 8, PLAN]) == (False, False)                    # plan on 16 bytes
+    assert call_probe_union(lib, ref, pkg, q, v, [0, PLAN]) == (False, False)
+    for i in (3, 4, 5, 6, 7, 8):                                                                           # plan disjoint from the routes and every mutable view
+        assert call_probe_union(lib, ref, pkg, q, v, [v[i][0], PLAN]) == (False, False), i
+    q5, v5, plan5 = probe(2, gate=13, up=13, identity=lib.mi355_numerical_identity(13, 0))
+    assert call_probe_union(lib, ref, pkg, q5, v5, plan5) == (False, False)                                # Q4_K gate / up only
+    for top_k, R, ok in ((6, 2, False), (6, 1, True), (12, 2, True), (3, 3, False)):                       # every row slice on 16 bytes
+        q, v, plan = probe(R, top_k=top_k)
+        assert call_probe_union(lib, ref, pkg, q, v, plan) == (ok, ok), (top_k, R)
+
+    def down(R, type_, **over):
+        q = down_request(lib, hidden=L, inter=I, experts=E, top_k=K, type=type_, limit=10.0, **over)
+        v = lay_out(down_required(L, I, E, K, R, type_))
+        return q, v, [v[-1][0] + 512, PLAN]
+    for R in (1, 4, 8):
+        for type_ in (14, 12):
+            q, v, plan = down(R, type_)
+            assert call_down_union(lib, ref, pkg, q, v, plan, R) == (True, True), (R, type_)
+            assert call_down_union(lib, ref, pkg, q, v, plan, R + 1) == (False, False)                      # rows must match the extents
+            for i in range(8):
+                assert call_down_union(lib, ref, pkg, q, v, [v[i][0], PLAN], R) == (False, False), i
+        for type_ in (7, 8):                                                                               # K-quant class only
+            q = down_request(lib, hidden=L, inter=I, experts=E, top_k=K, type=type_)
+            v = lay_out(down_required(L, I, E, K, R, type_))
+            assert call_down_union(lib, ref, pkg, q, v, [v[-1][0] + 512, PLAN], R) == (False, False)
+    q, v, plan = down(9, 14)
+    assert call_down_union(lib, ref, pkg, q, v, plan, 9) == (False, False)
+    # the aggregate word stays optional
+    q, v, plan = down(2, 14)
+    v[8] = [0, 0]
+    assert call_down_union(lib, ref, pkg, q, v, plan, 2) == (True, True)
+
+
+def test_union_admission_beyond_the_reference_caps(lib, ref, pkg):
+    """hidden past 1536 is this library's widening of the union form (the reference's bound is its kernel's register staging)."""
+    q = probe_request(lib, fp32=False, hidden=2048, rows=768, experts=128, top_k=8, R=4)
+    v = lay_out(probe_required(2048, 768, 128, 8, 4, 12, False))
+    plan = [v[-1][0] + (v[-1][1] + 511) // 256 * 256, orc.UNION_PLAN_BYTES]
+    assert call_probe_union(lib, ref, pkg, q, v, plan) == (True, False)
