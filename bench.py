@@ -305,6 +305,14 @@ def extra_configs(strix, torch, steps, warmup):
     sec = time_steps(torch, lambda i: torch.matmul(ga, gb), 10, 3)
     out["probe_fp16_gemm_8192_vendor_library"] = {"TFLOPs": 2.0 * 8192 ** 3 / sec / 1e12, "frac_of_fp16_mfma_peak": 2.0 * 8192 ** 3 / sec / 2.5e15}
     del ga, gb
+    # the matrix cores on their own: a register-operand MFMA loop of this library on every compute unit, with constant and with
+    # pseudo-random operands (the second is the ceiling a product on real data has under the chip's power limit)
+    sink = torch.empty(512 * 1024, dtype=torch.float32, device="cuda")
+    for name, rnd in (("constant_operands", False), ("random_operands", True)):
+        flops = strix.probe_mfma_f16(20000, rnd, sink)
+        sec = time_steps(torch, lambda i: strix.probe_mfma_f16(20000, rnd, sink), 3, 1)
+        out["probe_mfma_f16_register_loop_" + name] = {"TFLOPs": flops / sec / 1e12, "frac_of_fp16_mfma_peak": flops / sec / 2.5e15}
+    del sink
     # config 1: Q8_0 4096 x 4096 GEMV, one fp32 row
     n = 4096
     sets = []

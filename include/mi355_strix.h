@@ -59,6 +59,11 @@ enum { MI355_EXP_GFX1151 = 0, MI355_EXP_DECLARED = 1,
 
 const char* mi355_last_error(void);
 const char* mi355_version(void);
+/* Measurement aid of the benchmark (no counterpart in the reference, not a product path): one launch in which every wave of
+ * every compute unit runs iterations x 4 independent v_mfma_f32_32x32x16_f16 on register operands - constant ones, or
+ * (random_operands != 0) pseudo-random halves, whose switching power is what a real product meets. sink: at least 512
+ * floats per compute unit; *flops = the launch's matrix-core FLOPs. */
+int32_t mi355_probe_mfma_f16(uint32_t iterations, uint32_t random_operands, float* sink, uint64_t sink_floats, uint64_t* flops, mi355_stream stream);
 /* Numerical identity strings this library implements (the caller opts in by passing them back, as with
  * Request::approved_numerical_identity, include/strix/moe_q4k_a8_contract.hpp:24-26,104-116). */
 const char* mi355_numerical_identity(uint32_t weight_type, int down);

@@ -222,6 +222,7 @@ def lib():
         L.mi355_a8_enqueue_down_activation_quantize.argtypes = [P, P, U, U, P]
         L.mi355_a8_enqueue_down_rawdots.argtypes = [P, P, U, P]
         L.mi355_a8_enqueue_down_rawdots_merge.argtypes = [P, P, P, P]
+        L.mi355_probe_mfma_f16.argtypes = [U, U, P, C.c_uint64, P, P]
         L.mi355_a8_validate_union.argtypes = [P, P, DeviceBytes]
         L.mi355_a8_enqueue_probe_union.argtypes = [P, P, DeviceBytes, P]
         L.mi355_a8_validate_down_union.argtypes = [P, P, U, DeviceBytes]
@@ -257,7 +258,7 @@ EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi3
            "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
-           "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
+           "mi355_probe_mfma_f16", "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
            "mi355_a8_enqueue_down_activation_quantize_union", "mi355_a8_enqueue_down_rawdots_union",
            "mi355_moe_strided_enqueue_prologue", "mi355_moe_strided_enqueue_csr", "mi355_moe_strided_enqueue_project", "mi355_moe_strided_enqueue_down",
            "mi355_moe_strided_enqueue_merge", "mi355_moe_strided_enqueue_commit", "mi355_moe_strided_enqueue", "mi355_executor_create",
@@ -308,6 +309,13 @@ def quantize_weight_rows(qtype, x):
     out = torch.empty(x.shape[:-1] + (row_bytes(qtype, x.shape[-1]),), dtype=torch.uint8, device=x.device)
     check(lib().mi355_quantize_weight_rows(qtype, _p(x), rows, x.shape[-1], _p(out), _stream()))
     return out
+
+
+def probe_mfma_f16(iterations, random_operands, sink):
+    """One launch of the matrix-core probe (mi355_probe_mfma_f16); returns its FLOPs. sink: fp32 device tensor, 512 floats per compute unit."""
+    flops = C.c_uint64(0)
+    check(lib().mi355_probe_mfma_f16(iterations, int(random_operands), _p(sink), sink.numel(), C.byref(flops), _stream()))
+    return flops.value
 
 
 def quantize_a8(x, want_sums=True):

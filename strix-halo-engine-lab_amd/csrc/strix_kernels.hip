@@ -1310,7 +1310,50 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
 // ============================================================================================================ C ABI
 using namespace strix950;
 
+// What the matrix cores of this machine sustain on their own: every wave of a 512-thread workgroup (two waves per SIMD)
+// runs `iterations` x 4 independent v_mfma_f32_32x32x16_f16 on operands that stay in registers. random_operands != 0 fills
+// the operands with pseudo-random halves (weights in the range of the prefill's sc * q operands): the sustained rate then
+// falls with the switching power, which is the ceiling a real product has. A measurement aid for the benchmark, not a product path.
+__global__ __launch_bounds__(512) void probe_mfma_f16_kernel(uint32_t iterations, uint32_t random_operands, float* sink) {
+    floatx16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.0F;
+    half8 a, b;
+    uint32_t state = (threadIdx.x + blockIdx.x * 977U) * 2654435761U;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        state = state * 1664525U + 1013904223U;
+        const float u = static_cast<float>(state >> 8) * (1.0F / 16777216.0F) - 0.5F;
+        state = state * 1664525U + 1013904223U;
+        const float v = static_cast<float>(state >> 8) * (1.0F / 16777216.0F) - 0.5F;
+        a[i] = static_cast<_Float16>(random_operands ? u : 0.001F * static_cast<float>(threadIdx.x));
+        b[i] = static_cast<_Float16>(random_operands ? 945.0F * v : 0.5F);
+    }
+    for (uint32_t it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+        asm volatile("" : "+v"(a), "+v"(b));                  // the operands stay what they are; the loop is not folded
+    }
+    float total = 0.0F;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) total += acc[i][j];
+    sink[blockIdx.x * 512U + threadIdx.x] = total;
+}
+
 extern "C" {
+
+int32_t mi355_probe_mfma_f16(uint32_t iterations, uint32_t random_operands, float* sink, uint64_t sink_floats, uint64_t* flops, mi355_stream stream) {
+    const uint32_t blocks = compute_units();
+    STRIX_REQUIRE(sink && flops && sink_floats >= 512ULL * blocks && iterations > 0, "mfma probe: sink of 512 floats per compute unit, iterations > 0");
+    probe_mfma_f16_kernel<<<blocks, 512, 0, hs(stream)>>>(iterations, random_operands, sink);
+    STRIX_LAUNCHED("mfma probe");
+    *flops = 2ULL * 32U * 32U * 16U * 4U * iterations * 8ULL * blocks;
+    return MI355_OK;
+}
 
 const char* mi355_last_error(void) { return g_error.c_str(); }
 const char* mi355_version(void) { return "mi355-strix 0.1 (gfx950)"; }
