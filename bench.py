@@ -487,7 +487,7 @@ def cpu_baseline_config3(cfg, budget_s=12.0):
     med = statistics.median(times)
     return {"value": med * 1e6, "unit": "us/layer", "cores": threads, "kind": "port",
             "sample": f"layer 0 of the same config-3 workload (T={T}), median of {len(times)} passes after one warm-up; "
-                      "C restatement of the reference CPU path (group dots vectorised by the compiler for the host ISA, the fp32 chain scalar), "
+                      "C restatement of the reference CPU path (Q4_K rows: byte dot-product instruction and the sub-block chain in vector lanes where the host has AVX-VNNI, same bits as the plain loop), "
                       "OpenMP over (assignment, 32-output group) and (assignment, output)"}
 
 

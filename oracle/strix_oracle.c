@@ -278,8 +278,87 @@ static void q4k_block_dots(const uint8_t* qs, const int8_t* codes, int dot[8]) {
     }
 }
 
+#if defined(__x86_64__)
+#include <immintrin.h>
+/* The same eight dots with the byte dot-product instruction where the host has it (unsigned nibbles x signed codes, four
+ * products per 32-bit lane, no saturation: 4 x 15 x 127 fits): the form the reference's own AVX2 + VNNI rows take
+ * (src/cpu/arch/avx2/routed_expert_avx2.cpp). Integer sums are exact in any order, so the bits do not change. */
+__attribute__((target("avx2,avxvnni")))
+static void q4k_block_dots_vnni(const uint8_t* qs, const int8_t* codes, int dot[8]) {
+    const __m256i nibble = _mm256_set1_epi8(0x0f), zero = _mm256_setzero_si256();
+    __m256i part[8];
+    for (int p = 0; p < 4; ++p) {
+        const __m256i q = _mm256_loadu_si256((const __m256i*)(qs + 32 * p));
+        const __m256i lo = _mm256_and_si256(q, nibble), hi = _mm256_and_si256(_mm256_srli_epi16(q, 4), nibble);
+        part[2 * p] = _mm256_dpbusd_avx_epi32(zero, lo, _mm256_loadu_si256((const __m256i*)(codes + 64 * p)));
+        part[2 * p + 1] = _mm256_dpbusd_avx_epi32(zero, hi, _mm256_loadu_si256((const __m256i*)(codes + 64 * p + 32)));
+    }
+    /* eight vectors of eight partial sums -> one vector of the eight dots */
+    const __m256i a = _mm256_hadd_epi32(_mm256_hadd_epi32(part[0], part[1]), _mm256_hadd_epi32(part[2], part[3]));
+    const __m256i b = _mm256_hadd_epi32(_mm256_hadd_epi32(part[4], part[5]), _mm256_hadd_epi32(part[6], part[7]));
+    const __m128i first = _mm_add_epi32(_mm256_castsi256_si128(a), _mm256_extracti128_si256(a, 1));
+    const __m128i second = _mm_add_epi32(_mm256_castsi256_si128(b), _mm256_extracti128_si256(b, 1));
+    _mm_storeu_si128((__m128i*)dot, first);
+    _mm_storeu_si128((__m128i*)(dot + 4), second);
+}
+/* The whole row with the chain of the eight sub-blocks of a super-block in the eight lanes of a vector: every lane does the
+ * scalar function's operations in the scalar function's order (products, one subtraction, the delta product; then x[2p] + x[2p+1]
+ * and the pair accumulators), with separate multiplies and adds, so the bits are those of orc_q4k_row_a8's plain loop. */
+__attribute__((target("avx2,avxvnni")))
+static float q4k_row_a8_vnni(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas, const int32_t* sums) {
+    __m128 acc = _mm_setzero_ps();
+    for (uint32_t b = 0; b < blocks; ++b) {
+        const uint8_t* blk = wrow + (size_t)b * ORC_Q4_K_BLOCK;
+        const float d = orc_half_to_float(le16(blk)), dm = orc_half_to_float(le16(blk + 2));
+        int dots[8], sc[8], mn[8];
+        q4k_block_dots_vnni(blk + 16, codes + 256 * b, dots);
+        const uint32_t y = le32(blk + 4), z = le32(blk + 8), w = le32(blk + 12);
+        for (unsigned j = 0; j < 4; ++j) {                      /* src/cpu/core/routed_expert.cpp:65-71 */
+            const unsigned a8 = (y >> (8 * j)) & 255U, b8 = (z >> (8 * j)) & 255U, c8 = (w >> (8 * j)) & 255U;
+            sc[j] = (int)(a8 & 63U); mn[j] = (int)(b8 & 63U);
+            sc[4 + j] = (int)((c8 & 15U) | ((a8 >> 6U) << 4U)); mn[4 + j] = (int)((c8 >> 4U) | ((b8 >> 6U) << 4U));
+        }
+        const __m256 D = _mm256_mul_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(_mm256_loadu_si256((const __m256i*)sc)));
+        const __m256 DM = _mm256_mul_ps(_mm256_set1_ps(dm), _mm256_cvtepi32_ps(_mm256_loadu_si256((const __m256i*)mn)));
+        const __m256 u = _mm256_mul_ps(D, _mm256_cvtepi32_ps(_mm256_loadu_si256((const __m256i*)dots)));
+        const __m256 v = _mm256_mul_ps(DM, _mm256_cvtepi32_ps(_mm256_loadu_si256((const __m256i*)(sums + 8 * b))));
+        const __m256 x = _mm256_mul_ps(_mm256_loadu_ps(deltas + 8 * b), _mm256_sub_ps(u, v));
+        const __m256 pairs = _mm256_hadd_ps(x, x);              /* x0+x1, x2+x3, (again) | x4+x5, x6+x7, (again) */
+        const __m128 four = _mm_shuffle_ps(_mm256_castps256_ps128(pairs), _mm256_extractf128_ps(pairs, 1), _MM_SHUFFLE(1, 0, 1, 0));
+        acc = _mm_add_ps(acc, four);
+    }
+    float a[4];
+    _mm_storeu_ps(a, acc);
+    const float s01 = a[0] + a[1], s23 = a[2] + a[3];
+    return s01 + s23;
+}
+static int vector_rows_allowed = 1;
+static int host_has_vnni(void) {
+    static int known = -1;
+    if (known < 0) known = __builtin_cpu_supports("avx2") && __builtin_cpu_supports("avxvnni") ? 1 : 0;
+    return known && vector_rows_allowed;
+}
+#else
+static float q4k_row_a8_vnni(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas, const int32_t* sums) {
+    (void)wrow; (void)blocks; (void)codes; (void)deltas; (void)sums;
+    return 0.0F;
+}
+static int vector_rows_allowed = 1;
+static int host_has_vnni(void) { return 0; }
+#endif
+/* Tests switch the vector form of the Q4_K row off to compare it with the plain loop; returns whether the host has it. */
+int orc_vector_rows(int allowed) {
+    vector_rows_allowed = allowed != 0;
+    const int had = vector_rows_allowed;
+    vector_rows_allowed = 1;
+    const int has = host_has_vnni();
+    vector_rows_allowed = had;
+    return has;
+}
+
 float orc_q4k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,
                      const int32_t* sums) {
+    if (host_has_vnni()) return q4k_row_a8_vnni(wrow, blocks, codes, deltas, sums);
     float acc[4] = {0.0F, 0.0F, 0.0F, 0.0F};
     for (uint32_t b = 0; b < blocks; ++b) {
         const uint8_t* blk = wrow + (size_t)b * ORC_Q4_K_BLOCK;

@@ -79,6 +79,10 @@ int orc_gemv_q8_0_a8(const orc_q8a8_view* view, int threads);   /* -1: in % 32 !
 
 /* ---- Q4_K x A8 row (src/cpu/core/routed_expert.cpp:73-108 == src/moe_q4k_a8_contract.cpp:126-140) */
 void orc_rmsnorm_f32(const float* x, const float* w, uint32_t n, float eps, float* y, uint32_t rows);
+/* The Q4_K row has a vector form (byte dot-product instruction, the chain of a super-block's eight sub-blocks in eight
+ * lanes) on hosts with AVX2 + AVX-VNNI; same operations in the same order, same bits. orc_vector_rows(0) makes every later
+ * call take the plain loop, orc_vector_rows(1) allows the vector form again; returns 1 when the host has the vector form. */
+int orc_vector_rows(int allowed);
 float orc_q4k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,
                      const int32_t* sums);
 float orc_q5k_row_a8(const uint8_t* wrow, uint32_t blocks, const int8_t* codes, const float* deltas,

@@ -1017,3 +1017,34 @@ def test_committed_reference_vectors():
         x = (rng.standard_normal((rows, n)) * 2.0).astype(np.float32)
         w = rng.standard_normal(n).astype(np.float32)
         assert np.array_equal(bits(orc.rmsnorm_f32(x, w, 1e-6)), gold[f"rmsnorm_{seed}_bits"])
+
+
+def test_vector_form_of_the_q4k_row_equals_the_plain_loop():
+    """orc_q4k_row_a8 takes a vector form on hosts with AVX2 + AVX-VNNI (the reference's own fast rows are of that kind,
+    src/cpu/arch/avx2/routed_expert_avx2.cpp); the plain loop is the statement of src/cpu/core/routed_expert.cpp:73-108. Same
+    bits on random blocks, on extreme codes and on non-finite block scales."""
+    L = orc.lib()
+    if not L.orc_vector_rows(1):
+        pytest.skip("this host has no AVX-VNNI: only the plain loop runs")
+    rng = np.random.default_rng(2024)
+    try:
+        for case in range(200):
+            blocks = int(rng.integers(1, 9))
+            row = rng.integers(0, 256, blocks * 144, dtype=np.uint8)
+            if case % 3:
+                row.reshape(blocks, 144)[:, 1] = (row.reshape(blocks, 144)[:, 1] & 0x83) | 0x18        # moderate |d|
+                row.reshape(blocks, 144)[:, 3] = (row.reshape(blocks, 144)[:, 3] & 0x83) | 0x18
+            codes = rng.integers(-127, 128, blocks * 256, dtype=np.int8)
+            if case % 5 == 0:
+                codes[:] = 127 if case % 10 == 0 else -127
+                row.reshape(blocks, 144)[:, 16:] = 0xFF
+            deltas = (rng.standard_normal(blocks * 8) * 0.05).astype(np.float32)
+            sums = codes.reshape(-1, 32).astype(np.int32).sum(axis=1).astype(np.int32)
+            L.orc_vector_rows(1)
+            fast = orc.q4k_row_a8(row, codes, deltas, sums)
+            L.orc_vector_rows(0)
+            plain = orc.q4k_row_a8(row, codes, deltas, sums)
+            # (a NaN's payload depends on which operand an instruction takes it from: every NaN counts as the same value)
+            assert (np.isnan(fast) and np.isnan(plain)) or np.float32(fast).view(np.uint32) == np.float32(plain).view(np.uint32), case
+    finally:
+        L.orc_vector_rows(1)
