@@ -74,6 +74,28 @@ def test_union_rows_equal_single_row_calls_bit_for_bit(strix, H, I, E, K, R, dow
                                   bits(rows[r][name][0]) if got.dtype == np.float32 else rows[r][name][0]), (name, r)
 
 
+@pytest.mark.parametrize("H,I,E,K,R,same", [
+    (512, 256, 16, 3, 1, False),       # one row, top-3: the routes view is 12 bytes (a single row slice needs no 16-byte pitch)
+    (1024, 512, 16, 8, 8, True),       # every row names the same eight experts in its own order: eight holders per entry
+    (1024, 512, 16, 4, 7, True)])      # seven holders: the last sweep of an entry serves three rows
+def test_union_rows_small_shapes_and_full_entries(strix, H, I, E, K, R, same):
+    rng = np.random.default_rng(3 * H + R)
+    gate, up, down = make_layer(rng, H, I, E)
+    pool = rng.permutation(E)[:K]
+    ids = np.stack([rng.permutation(pool) if same else rng.permutation(E)[:K] for _ in range(R)]).astype(np.uint32)
+    rows, un, _ = run_paths(strix, rng, H, I, E, K, R, orc.Q4_K, ids, gate, up, down)
+    assert int(un.status.item()) == 0
+    entries = orc.expert_union_build(ids, R, K, E)
+    assert np.array_equal(un.plan.cpu().numpy(), orc.expert_union_plan_bytes(entries, R, K))
+    if same:
+        assert len(entries) == K and all(sum(s != orc.UNION_NO_SLOT for s in slots) == R for _, slots in entries)
+    for name in FIELDS:
+        got = getattr(un, name).cpu().numpy()
+        for r in range(R):
+            a, b = got[r], rows[r][name][0]
+            assert np.array_equal(bits(a) if a.dtype == np.float32 else a, bits(b) if b.dtype == np.float32 else b), (name, r)
+
+
 def test_union_rows_against_the_oracle(strix):
     H, I, E, K, R = 1024, 512, 16, 4, 6
     rng = np.random.default_rng(77)
