@@ -391,13 +391,13 @@ int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bind
     const uint32_t items = logical_rows * s.top_k;
     r.union_plan = union_plan;
     if (union_plan) {               // K-quant only: the items are the plan's entries
-        if (q->weight_type == MI355_TYPE_Q6_K) down_q6k_kernel<<<dim3(s.hidden / kDownGroupsRows, items), 256, 0, st>>>(w, r, items, 0U, 0U);
+        if (q->weight_type == MI355_TYPE_Q6_K) launch_down_q6k(w, r, dim3(s.hidden / kDownGroupsRows, items), items, 0U, 0U, st);
         else launch_down_nb<8>(w, r, logical_rows, dim3(s.hidden / 64U, items), st);
     } else if (q->weight_type != MI355_TYPE_Q4_K) {
         const dim3 grid(s.hidden / kDownGroupsRows, items);
         if (q->weight_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
         else if (q->weight_type == MI355_TYPE_Q5_1) down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
-        else down_q6k_kernel<<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
+        else launch_down_q6k(w, r, grid, items, 0U, 0U, st);
     } else if (items <= 16U) down_quad_kernel<4><<<dim3(s.hidden / 64U, items), 256, 0, st>>>(w, r, items);
     else if (items <= kQuadMaxItems) down_quad_kernel<2><<<dim3(s.hidden / 64U, items), 256, 0, st>>>(w, r, items);
     else launch_down_nb<4>(w, r, logical_rows, dim3(s.hidden / 64U, items), st);

@@ -1209,7 +1209,7 @@ inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t row
         }
         else if (w.down_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         else if (w.down_type == MI355_TYPE_Q5_1) down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
-        else down_q6k_kernel<<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
+        else launch_down_q6k(w, r, grid, assignments, items_at, order_at, st);
         return;
     }
     if (!grouped && quad_sweep(w, rows)) {
