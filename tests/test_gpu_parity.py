@@ -662,7 +662,9 @@ def test_expert_plan_words(strix, E, K, T):
     (orc.Q5_K, orc.Q8_0, 768, 512, 1, 1, 6, "staged"),          # a dense layer: the plan is still built
     (orc.Q4_K, orc.Q6_K, 512, 768, 6, 3, 5, "staged"),          # Q6_K down (src/moe_a8_down_contract.cpp:147): odd block count, 2-byte aligned rows
     (orc.Q5_K, orc.Q6_K, 2048, 768, 128, 8, 8, "layer"),
-    (orc.Q4_K, orc.Q6_K, 1024, 1280, 16, 4, 40, "staged"),
+    (orc.Q4_K, orc.Q6_K, 1024, 1280, 16, 4, 40, "staged"),      # five super-blocks per row: the direct-load kernel
+    (orc.Q4_K, orc.Q6_K, 512, 256, 6, 3, 7, "staged"),          # one and four super-blocks per row through LDS
+    (orc.Q4_K, orc.Q6_K, 512, 1024, 6, 3, 9, "layer"),
     (orc.Q4_K, orc.Q8_0, 768, 512, 5, 2, 23, "layer")])
 def test_down_rows_in_the_host_executor_formats(strix, gate_type, down_type, H, I, E, K, T, entry):
     """The formats of the reference's host executor (src/cpu/core/routed_expert.hpp:27-28): gate/up Q4_K or Q5_K, down Q8_0 or Q5_1.
