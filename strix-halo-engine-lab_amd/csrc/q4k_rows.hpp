@@ -130,7 +130,9 @@ struct RowsK : mi355_moe_rows {
 // (plan == nullptr) item i is assignment i alone, its expert read from the routes (or from the job's list): the single-row
 // forms of the reference entry points (include/strix/hip_moe_q4k_a8_probe.hpp:12, include/strix/hip_moe_a8_down.hpp:11-30) and
 // the host executor's Job bring no plan view.
-struct WorkItem { uint32_t e, begin, end; };
+// first: the assignment at position `begin` of the plan order, plus one, when the plan's writer left it in the item's fourth
+// word (the fused decode router does); 0 = look it up in the order. It spares the down + combine launch a dependent load.
+struct WorkItem { uint32_t e, begin, end, first; };
 
 // Expert-union plan of a verify window (include/strix/moe/expert_union.hpp:17-27): words {count, rows, top_k, 0}, then 128
 // entries of three words {expert, slot bytes of rows 0-3, of rows 4-7}; a slot byte 0xff = that row did not choose the
@@ -142,10 +144,10 @@ __device__ __forceinline__ uint32_t union_held(uint32_t four_slots) {      // on
     return (((y & 0x7f7f7f7fU) + 0x7f7f7f7fU) | y) & 0x80808080U;
 }
 __device__ __forceinline__ WorkItem union_item(const uint32_t* plan, uint32_t u) {
-    if (u >= plan[0]) return {0U, 0U, 0U};
+    if (u >= plan[0]) return {0U, 0U, 0U, 0U};
     const uint32_t* entry = plan + 4U + 3U * u;
     const uint32_t holders = static_cast<uint32_t>(__popc(union_held(entry[1])) + __popc(union_held(entry[2])));
-    return {entry[0], u << 8, (u << 8) + holders};
+    return {entry[0], u << 8, (u << 8) + holders, 0U};
 }
 __device__ __forceinline__ uint32_t union_assignment(const uint32_t* plan, uint32_t position) {
     const uint32_t* entry = plan + 4U + 3U * (position >> 8);
@@ -163,7 +165,7 @@ __device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const 
     if (r.union_plan) return union_item(r.union_plan, index);
     if (r.plan) {
         const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * index);
-        return {item.x, item.y, item.z};
+        return {item.x, item.y, item.z, item.w};
     }
     uint32_t e;
     if (r.assignments) e = r.assignments[index].expert;
@@ -172,7 +174,7 @@ __device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const 
         r.place(index, row, slot);
         e = r.routes_of(row)[slot];
     }
-    return {e, index, e < w.experts ? index + 1U : index};      // an invalid route has no item (its row is flagged)
+    return {e, index, e < w.experts ? index + 1U : index, index + 1U};      // an invalid route has no item (its row is flagged)
 }
 __device__ __forceinline__ uint32_t ordered(const RowsK& r, uint32_t order_at, uint32_t i) {
     if (r.union_plan) return union_assignment(r.union_plan, i);

@@ -326,7 +326,7 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
             uint32_t* order = a.plan + plan_order_at(all);
             if (lane < K) {
                 const uint32_t at = row * K + lane;
-                *reinterpret_cast<uint4*>(items + 4U * at) = make_uint4(expert, at, at + 1U, 0U);
+                *reinterpret_cast<uint4*>(items + 4U * at) = make_uint4(expert, at, at + 1U, row * P + lane + 1U);     // (the item names its assignment)
                 order[at] = row * P + lane;
             } else if (lane < P) order[a.rows * K + (lane - K) * a.rows + row] = row * P + lane;
         }
@@ -911,13 +911,14 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
     __shared__ uint32_t slot_order[kDownMergeSlots];
     __shared__ float slot_weight[kDownMergeSlots];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, row = blockIdx.y, o = blockIdx.x * 64U + lane;
-    if (*r.job_status & MI355_STATUS_NONFINITE_PROJECTION) return;            // the whole job: no down rows, nothing published
+    const uint32_t job = *r.job_status;                                        // (requested together with the item: one round trip, not two)
     const uint32_t a = row * w.top_k + wave;
     const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), a);
     const uint32_t e = __builtin_amdgcn_readfirstlane(item.e), begin = __builtin_amdgcn_readfirstlane(item.begin), end = __builtin_amdgcn_readfirstlane(item.end);
+    if (job & MI355_STATUS_NONFINITE_PROJECTION) return;                       // the whole job: no down rows, nothing published
     float value = 0.0F;
     if (begin != end) {                                                        // (an invalid route has no item: its row is flagged)
-        const uint32_t first = ordered(r, plan_order_at(w.experts), begin);
+        const uint32_t first = item.first ? item.first - 1U : ordered(r, plan_order_at(w.experts), begin);
         const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
         const size_t stride = w.down_row_stride;
         StageSource source;
