@@ -955,6 +955,63 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
+// The same for the smallest decode batches, in the 16-rows-per-wavefront layout of down_quad_kernel: a workgroup owns (row, 16
+// output columns), wave k sweeps the 16 down rows of the expert in slot k (lane = (row, pair)), the slots' values meet in LDS
+// and the first sixteen lanes of wave 0 fold them as merge_kernel does. One launch instead of two for one to six rows.
+template <int DEPTH>
+__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_quad_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
+    __shared__ __attribute__((aligned(16))) uint8_t mq0[kDownMergeSlots][kQuadSlotBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t mq1[kDownMergeSlots][kQuadSlotBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t mq2[DEPTH > 2 ? kDownMergeSlots : 1][DEPTH > 2 ? kQuadSlotBytes : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t mq3[DEPTH > 3 ? kDownMergeSlots : 1][DEPTH > 3 ? kQuadSlotBytes : 16];
+    __shared__ float slot_value[kDownMergeSlots][kQuadRows];
+    __shared__ uint32_t slot_order[kDownMergeSlots];
+    __shared__ float slot_weight[kDownMergeSlots];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, p = lane & 3U, rr = lane >> 2, row = blockIdx.y, o0 = blockIdx.x * kQuadRows;
+    lds_u8* const ring[4] = {(lds_u8*)mq0[wave], (lds_u8*)mq1[wave], (lds_u8*)mq2[DEPTH > 2 ? wave : 0], (lds_u8*)mq3[DEPTH > 3 ? wave : 0]};
+    lds_u8* slots[DEPTH];
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i) slots[i] = ring[i];
+    const uint32_t job = *r.job_status;                                        // (requested together with the item)
+    const uint32_t a = row * w.top_k + wave;
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), a);
+    if (job & MI355_STATUS_NONFINITE_PROJECTION) return;                       // the whole job: no down rows, nothing published
+    float value = 0.0F;
+    if (item.begin != item.end) {                                              // (an invalid route has no item: its row is flagged)
+        const uint32_t src = __builtin_amdgcn_readfirstlane(item.first ? item.first - 1U : ordered(r, plan_order_at(w.experts), item.begin));
+        const uint8_t* rows = w.down + static_cast<size_t>(item.e) * w.down_expert_stride + static_cast<size_t>(o0) * w.down_row_stride;
+        const size_t stride = w.down_row_stride;
+        QuadSource source;
+        source.init([&](uint32_t q) { return rows + q * stride; }, r.h.codes_of(src));
+        lds_u8* const (&sl)[DEPTH] = slots;
+        value = sweep_quads<DEPTH>(sl, source, w.ffn / 256U, r.h, src);
+        if (p == 0) r.rawdots_of(src, w.hidden)[o0 + rr] = value;
+    }
+    if (p == 0) slot_value[wave][rr] = value;
+    if (threadIdx.x == 0) {
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
+        if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
+            for (uint32_t i = 1; i < w.top_k; ++i)
+                for (uint32_t j = i; j > 0 && r.routes_of(row)[slot_order[j]] < r.routes_of(row)[slot_order[j - 1]]; --j) {
+                    const uint32_t t = slot_order[j]; slot_order[j] = slot_order[j - 1]; slot_order[j - 1] = t;
+                }
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights_of(row)[slot_order[k]];
+    }
+    __syncthreads();
+    // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is the combine's own)
+    if (threadIdx.x >= kQuadRows || (*r.status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
+    float acc = 0.0F;
+    for (uint32_t k = 0; k < w.top_k; ++k) {
+        const float ev = slot_value[slot_order[k]][lane];
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], ev, acc);
+        else acc = acc + slot_weight[k] * ev;
+    }
+    const uint32_t o = o0 + lane;
+    const float y = r.base ? acc + r.base_of(row)[o] : acc;
+    if (!finite_f(y)) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
+}
+
 // SwiGLU + A8 re-quantisation of dense gate/up rows. Reference: src/cpu/core/routed_expert.cpp:147-170.
 __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate, const float* up, uint32_t ffn, uint32_t exp_kind, float limit,
                                                               int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
@@ -1675,6 +1732,13 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     if (!quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
         (wv.hidden / 64U) * rows <= compute_units()) {
         down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        STRIX_LAUNCHED("moe layer experts + combine");
+        return MI355_OK;
+    }
+    if (quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.top_k <= kDownMergeSlots && wv.hidden % kQuadRows == 0 && rows <= 65535U) {
+        const dim3 grid(wv.hidden / kQuadRows, rows);
+        if (rows <= 2U) down_merge_quad_kernel<4><<<grid, 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        else down_merge_quad_kernel<2><<<grid, 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }

@@ -547,12 +547,14 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
 
 
 @pytest.mark.parametrize("combine", [0, 1])
-def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine):
+@pytest.mark.parametrize("T", [8, 1, 2, 5])
+def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine, T):
     """A decode batch whose (row, 64 columns) workgroups are all resident takes the down rows and the ordered combine in one
     launch (a wave per slot): output, rawdots and status words must equal the staged entry points' bit for bit, for both
-    combine forms and with a base term."""
-    E, H, I, K, T = 32, 1024, 512, 8, 8
-    rng = np.random.default_rng(91 + combine)
+    combine forms and with a base term. One to six rows take the same in the 16-rows-per-wavefront layout (T = 1, 2: the
+    four-slot ring, T = 5: the two-slot ring)."""
+    E, H, I, K = 32, 1024, 512, 8
+    rng = np.random.default_rng(91 + combine + 7 * T)
     gate, up, down = make_layer(rng, H, I, E)
     x = dev(rng.standard_normal((T, H)).astype(np.float16))
     wr = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
