@@ -1012,6 +1012,71 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_quad_kernel(m
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
+// Down rows + combine in one launch for Q8_0 down tensors (the host executor's format, src/cpu/core/routed_expert.cpp:110-126): the
+// workgroup of (row, 16 columns) again, wave k = the expert in slot k, lane = (row, chain) with the direct block loads and the
+// chain order of down_groups_kernel<0>; one item per assignment (the fused decode router's plan).
+__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_q8_0_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
+    typedef uint32_t u32x4_g __attribute__((ext_vector_type(4)));
+    __shared__ float slot_value[kDownMergeSlots][16];
+    __shared__ uint32_t slot_order[kDownMergeSlots];
+    __shared__ float slot_weight[kDownMergeSlots];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, j = lane & 3U, odd = j & 1U, rr = lane >> 2, row = blockIdx.y;
+    const uint32_t o = blockIdx.x * 16U + rr;
+    const uint32_t job = *r.job_status;                                        // (requested together with the item)
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), row * w.top_k + wave);
+    if (job & MI355_STATUS_NONFINITE_PROJECTION) return;                       // the whole job: no down rows, nothing published
+    float value = 0.0F;
+    if (item.begin != item.end) {                                              // (an invalid route has no item: its row is flagged)
+        const uint32_t src = item.first ? item.first - 1U : ordered(r, plan_order_at(w.experts), item.begin);
+        const uint32_t per_chain = w.ffn / 128U;
+        const uint8_t* wrow = w.down + static_cast<size_t>(item.e) * w.down_expert_stride + static_cast<size_t>(o) * w.down_row_stride + 34U * j;
+        const int8_t* h_codes = r.h.codes_of(src);
+        const float* h_deltas = r.h.deltas_of(src);
+        float chain = 0.0F;
+#pragma unroll 2
+        for (uint32_t c = 0; c < per_chain; ++c) {
+            const uint32_t g = 4U * c + j;
+            float d, m;
+            uint32_t q[8];
+            load_group_block<0>(wrow + static_cast<size_t>(c) * (4U * 34U), odd, d, m, q);
+            const u32x4_g* codes = reinterpret_cast<const u32x4_g*>(h_codes + 32U * g);
+            const u32x4_g c_lo = codes[0], c_hi = codes[1];
+            const uint32_t cw[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+            int dot = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot = __builtin_amdgcn_sdot4(static_cast<int>(q[i]), static_cast<int>(cw[i]), dot, false);
+            chain = chain + (h_deltas[g] * (d * static_cast<float>(dot)));
+        }
+        value = chain;
+        value = value + xor1_f(value);          // chain0 + chain1 | chain2 + chain3
+        value = value + xor2_f(value);          // (chain0 + chain1) + (chain2 + chain3)
+        if (j == 0) r.rawdots_of(src, w.hidden)[o] = value;
+    }
+    if (j == 0) slot_value[wave][rr] = value;
+    if (threadIdx.x == 0) {
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
+        if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
+            for (uint32_t i = 1; i < w.top_k; ++i)
+                for (uint32_t jj = i; jj > 0 && r.routes_of(row)[slot_order[jj]] < r.routes_of(row)[slot_order[jj - 1]]; --jj) {
+                    const uint32_t t = slot_order[jj]; slot_order[jj] = slot_order[jj - 1]; slot_order[jj - 1] = t;
+                }
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights_of(row)[slot_order[k]];
+    }
+    __syncthreads();
+    // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is the combine's own)
+    if (threadIdx.x >= 16U || (*r.status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
+    float acc = 0.0F;
+    for (uint32_t k = 0; k < w.top_k; ++k) {
+        const float ev = slot_value[slot_order[k]][lane];
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], ev, acc);
+        else acc = acc + slot_weight[k] * ev;
+    }
+    const uint32_t oc = blockIdx.x * 16U + lane;
+    const float y = r.base ? acc + r.base_of(row)[oc] : acc;
+    if (!finite_f(y)) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    r.output[static_cast<size_t>(row) * r.output_stride + oc] = y;
+}
+
 // SwiGLU + A8 re-quantisation of dense gate/up rows. Reference: src/cpu/core/routed_expert.cpp:147-170.
 __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float* gate, const float* up, uint32_t ffn, uint32_t exp_kind, float limit,
                                                               int8_t* codes, float* deltas, int32_t* sums, float* h_out, uint32_t* status,
@@ -1739,6 +1804,11 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
         const dim3 grid(wv.hidden / kQuadRows, rows);
         if (rows <= 2U) down_merge_quad_kernel<4><<<grid, 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
         else down_merge_quad_kernel<2><<<grid, 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        STRIX_LAUNCHED("moe layer experts + combine");
+        return MI355_OK;
+    }
+    if (wv.down_type == MI355_TYPE_Q8_0 && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && wv.ffn % 128U == 0 && rows <= 65535U) {
+        down_merge_q8_0_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }

@@ -547,23 +547,25 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
 
 
 @pytest.mark.parametrize("combine", [0, 1])
-@pytest.mark.parametrize("T", [8, 1, 2, 5])
-def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine, T):
+@pytest.mark.parametrize("T,down_type", [(8, orc.Q4_K), (1, orc.Q4_K), (2, orc.Q4_K), (5, orc.Q4_K), (8, orc.Q8_0), (3, orc.Q8_0)])
+def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine, T, down_type):
     """A decode batch whose (row, 64 columns) workgroups are all resident takes the down rows and the ordered combine in one
     launch (a wave per slot): output, rawdots and status words must equal the staged entry points' bit for bit, for both
     combine forms and with a base term. One to six rows take the same in the 16-rows-per-wavefront layout (T = 1, 2: the
-    four-slot ring, T = 5: the two-slot ring)."""
+    four-slot ring, T = 5: the two-slot ring); Q8_0 down rows (the host executor's format) in their four-chains-per-row layout."""
     E, H, I, K = 32, 1024, 512, 8
-    rng = np.random.default_rng(91 + combine + 7 * T)
+    rng = np.random.default_rng(91 + combine + 7 * T + down_type)
     gate, up, down = make_layer(rng, H, I, E)
+    if down_type == orc.Q8_0:
+        down = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32))
     x = dev(rng.standard_normal((T, H)).astype(np.float16))
     wr = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
     base = dev(rng.standard_normal((T, H)).astype(np.float32))
-    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, down_type=down_type)
     y, ids, wts, _ = layer.run_layer(x, wr, base=base, combine=combine)
     y, raw = y.clone(), layer.rawdots[:T].clone()
     assert int(layer.status.sum()) == 0
-    staged = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, T)
+    staged = strix.MoeLayer(H, I, E, K, layer.gate, layer.up, layer.down, T, down_type=down_type)
     want = staged.run(x, ids.clone(), wts.clone(), base=base, combine=combine)
     assert torch.equal(raw, staged.rawdots[:T]) and torch.equal(y, want)
     ids_n, w_n = ids.cpu().numpy().astype(np.uint32), wts.cpu().numpy()
