@@ -238,14 +238,19 @@ __global__ __launch_bounds__(256) void down_q6k_tile_kernel(mi355_moe_weights w,
     }
 }
 
+// Rows the LDS forms can copy: dense (back to back) from a 16-byte aligned start, and the A8 image of h in whole 16-byte
+// pieces (the activation rows are copied to LDS as well).
+inline bool q6k_tile_rows(const mi355_moe_weights& w, const RowsK& r) {
+    return w.down_row_stride == static_cast<uint64_t>(kQ6kBlock) * (w.ffn / 256U) && reinterpret_cast<uintptr_t>(w.down) % 16U == 0 &&
+           w.down_expert_stride % 16U == 0 && !r.h.table && reinterpret_cast<uintptr_t>(r.h.codes) % 16U == 0 &&
+           reinterpret_cast<uintptr_t>(r.h.deltas) % 16U == 0 && r.h.codes_rs % 16U == 0 && r.h.deltas_rs % 16U == 0;
+}
+
 // Q6_K down rows of a launch: through LDS when the rows are dense (back to back) and at most four super-blocks long.
 inline void launch_down_q6k(const mi355_moe_weights& w, const RowsK& r, dim3 grid, uint32_t assignments, uint32_t items_at, uint32_t order_at,
                             hipStream_t st) {
     const uint32_t blocks = w.ffn / 256U;
-    // (and the A8 image of h in whole 16-byte pieces: the workgroup copies its activation rows to LDS as well)
-    const bool dense = w.down_row_stride == static_cast<uint64_t>(kQ6kBlock) * blocks && reinterpret_cast<uintptr_t>(w.down) % 16U == 0 &&
-                       w.down_expert_stride % 16U == 0 && !r.h.table && reinterpret_cast<uintptr_t>(r.h.codes) % 16U == 0 &&
-                       reinterpret_cast<uintptr_t>(r.h.deltas) % 16U == 0 && r.h.codes_rs % 16U == 0 && r.h.deltas_rs % 16U == 0;
+    const bool dense = q6k_tile_rows(w, r);
     if (dense && blocks == 1U) down_q6k_tile_kernel<1><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
     else if (dense && blocks == 2U) down_q6k_tile_kernel<2><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
     else if (dense && blocks == 3U) down_q6k_tile_kernel<3><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);

@@ -1012,6 +1012,93 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_quad_kernel(m
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
+// Down rows + combine in one launch for Q6_K down rows (src/moe_a8_down_contract.cpp:147-158): the workgroup of (row, 16 columns),
+// wave k = the expert in slot k, lane = (row, pair) with the direct loads and the order of down_q6k_kernel.
+__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_q6k_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
+    typedef uint32_t u32x4_g __attribute__((ext_vector_type(4)));
+    __shared__ float slot_value[kDownMergeSlots][16];
+    __shared__ uint32_t slot_order[kDownMergeSlots];
+    __shared__ float slot_weight[kDownMergeSlots];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, p = lane & 3U, half = p >> 1, odd = p & 1U, rr = lane >> 2, row = blockIdx.y;
+    const uint32_t o = blockIdx.x * 16U + rr;
+    const uint32_t job = *r.job_status;                                        // (requested together with the item)
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), row * w.top_k + wave);
+    if (job & MI355_STATUS_NONFINITE_PROJECTION) return;                       // the whole job: no down rows, nothing published
+    float value = 0.0F;
+    if (item.begin != item.end) {                                              // (an invalid route has no item: its row is flagged)
+        const uint32_t src = item.first ? item.first - 1U : ordered(r, plan_order_at(w.experts), item.begin);
+        const uint32_t blocks = w.ffn / 256U;
+        const uint8_t* wrow = w.down + static_cast<size_t>(item.e) * w.down_expert_stride + static_cast<size_t>(o) * w.down_row_stride;
+        const int8_t* h_codes = r.h.codes_of(src);
+        const float* h_deltas = r.h.deltas_of(src);
+        float acc = 0.0F;
+#pragma unroll 2
+        for (uint32_t b = 0; b < blocks; ++b) {
+            const uint8_t* blk = wrow + static_cast<size_t>(b) * kQ6kBlock;
+            uint32_t ql[16], qh[8];
+            load_words_2aligned<16>(blk + 64U * half, ql);
+            load_words_2aligned<8>(blk + 128U + 32U * half, qh);
+            const uint16_t* tail = reinterpret_cast<const uint16_t*>(blk + 192U);
+            const uint32_t sc01 = tail[2U * p], sc23 = tail[2U * p + 1U];          // scales 4p, 4p + 1 | 4p + 2, 4p + 3
+            const float d = half_bits_to_float(tail[8]);
+            const int s[2][2] = {{static_cast<int8_t>(sc01 & 255U), static_cast<int8_t>(sc01 >> 8)},
+                                 {static_cast<int8_t>(sc23 & 255U), static_cast<int8_t>(sc23 >> 8)}};
+            const u32x4_g* codes = reinterpret_cast<const u32x4_g*>(h_codes + 256U * b + 64U * p);
+            const float2 delta = *reinterpret_cast<const float2*>(h_deltas + 8U * b + 2U * p);
+            float term[2];
+#pragma unroll
+            for (uint32_t k = 0; k < 2U; ++k) {
+                uint32_t q[8];
+#pragma unroll
+                for (uint32_t i = 0; i < 8U; ++i) {
+                    const uint32_t nibbles = (ql[8U * k + i] >> (4U * odd)) & 0x0f0f0f0fU;
+                    const uint32_t pairs = (qh[i] >> (4U * odd + 2U * k)) & 0x03030303U;
+                    const uint32_t six = nibbles | (pairs << 4);                   // 0 .. 63 per byte
+                    q[i] = ((six | 0x80808080U) - 0x20202020U) ^ 0x80808080U;      // minus 32 per byte, no borrow between bytes
+                }
+                const u32x4_g c_lo = codes[2U * k], c_hi = codes[2U * k + 1U];
+                const uint32_t cw[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+                int first = 0, last = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    first = __builtin_amdgcn_sdot4(static_cast<int>(q[i]), static_cast<int>(cw[i]), first, false);
+                    last = __builtin_amdgcn_sdot4(static_cast<int>(q[4 + i]), static_cast<int>(cw[4 + i]), last, false);
+                }
+                const int integer = s[k][0] * first + s[k][1] * last;
+                term[k] = (k == 0 ? delta.x : delta.y) * (d * static_cast<float>(integer));
+            }
+            acc = acc + (term[0] + term[1]);
+        }
+        value = acc;
+        value = value + xor1_f(value);          // acc0 + acc1 | acc2 + acc3
+        value = value + xor2_f(value);          // (acc0 + acc1) + (acc2 + acc3)
+        if (p == 0) r.rawdots_of(src, w.hidden)[o] = value;
+    }
+    if (p == 0) slot_value[wave][rr] = value;
+    if (threadIdx.x == 0) {
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
+        if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
+            for (uint32_t i = 1; i < w.top_k; ++i)
+                for (uint32_t jj = i; jj > 0 && r.routes_of(row)[slot_order[jj]] < r.routes_of(row)[slot_order[jj - 1]]; --jj) {
+                    const uint32_t t = slot_order[jj]; slot_order[jj] = slot_order[jj - 1]; slot_order[jj - 1] = t;
+                }
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights_of(row)[slot_order[k]];
+    }
+    __syncthreads();
+    // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is the combine's own)
+    if (threadIdx.x >= 16U || (*r.status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
+    float sum = 0.0F;
+    for (uint32_t k = 0; k < w.top_k; ++k) {
+        const float ev = slot_value[slot_order[k]][lane];
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER) sum = __builtin_fmaf(slot_weight[k], ev, sum);
+        else sum = sum + slot_weight[k] * ev;
+    }
+    const uint32_t oc = blockIdx.x * 16U + lane;
+    const float y = r.base ? sum + r.base_of(row)[oc] : sum;
+    if (!finite_f(y)) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    r.output[static_cast<size_t>(row) * r.output_stride + oc] = y;
+}
+
 // Down rows + combine in one launch for Q8_0 down tensors (the host executor's format, src/cpu/core/routed_expert.cpp:110-126): the
 // workgroup of (row, 16 columns) again, wave k = the expert in slot k, lane = (row, chain) with the direct block loads and the
 // chain order of down_groups_kernel<0>; one item per assignment (the fused decode router's plan).
@@ -1809,6 +1896,11 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     }
     if (wv.down_type == MI355_TYPE_Q8_0 && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && wv.ffn % 128U == 0 && rows <= 65535U) {
         down_merge_q8_0_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        STRIX_LAUNCHED("moe layer experts + combine");
+        return MI355_OK;
+    }
+    if (wv.down_type == MI355_TYPE_Q6_K && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && rows <= 65535U) {
+        down_merge_q6k_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }

@@ -547,17 +547,21 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
 
 
 @pytest.mark.parametrize("combine", [0, 1])
-@pytest.mark.parametrize("T,down_type", [(8, orc.Q4_K), (1, orc.Q4_K), (2, orc.Q4_K), (5, orc.Q4_K), (8, orc.Q8_0), (3, orc.Q8_0)])
+@pytest.mark.parametrize("T,down_type", [(8, orc.Q4_K), (1, orc.Q4_K), (2, orc.Q4_K), (5, orc.Q4_K), (8, orc.Q8_0), (3, orc.Q8_0),
+                                         (8, orc.Q6_K), (3, orc.Q6_K)])
 def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine, T, down_type):
     """A decode batch whose (row, 64 columns) workgroups are all resident takes the down rows and the ordered combine in one
     launch (a wave per slot): output, rawdots and status words must equal the staged entry points' bit for bit, for both
     combine forms and with a base term. One to six rows take the same in the 16-rows-per-wavefront layout (T = 1, 2: the
-    four-slot ring, T = 5: the two-slot ring); Q8_0 down rows (the host executor's format) in their four-chains-per-row layout."""
+    four-slot ring, T = 5: the two-slot ring); Q8_0 down rows (the host executor's format) in their four-chains-per-row layout,
+    dense Q6_K down rows through LDS."""
     E, H, I, K = 32, 1024, 512, 8
     rng = np.random.default_rng(91 + combine + 7 * T + down_type)
     gate, up, down = make_layer(rng, H, I, E)
     if down_type == orc.Q8_0:
         down = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32))
+    elif down_type == orc.Q6_K:
+        down = orc.random_q6_k(rng, (E, H), I)
     x = dev(rng.standard_normal((T, H)).astype(np.float16))
     wr = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
     base = dev(rng.standard_normal((T, H)).astype(np.float32))
@@ -669,7 +673,8 @@ def test_expert_plan_words(strix, E, K, T):
     (orc.Q4_K, orc.Q6_K, 1024, 1280, 16, 4, 40, "staged"),      # five super-blocks per row: the direct-load kernel
     (orc.Q4_K, orc.Q6_K, 512, 256, 6, 3, 7, "staged"),          # one and four super-blocks per row through LDS
     (orc.Q4_K, orc.Q6_K, 512, 1024, 6, 3, 9, "layer"),
-    (orc.Q4_K, orc.Q8_0, 768, 512, 5, 2, 23, "layer")])
+    (orc.Q4_K, orc.Q8_0, 768, 512, 5, 2, 23, "layer"),
+    (orc.Q4_K, orc.Q6_K, 512, 256, 6, 2, 4, "layer")])          # one super-block per down row
 def test_down_rows_in_the_host_executor_formats(strix, gate_type, down_type, H, I, E, K, T, entry):
     """The formats of the reference's host executor (src/cpu/core/routed_expert.hpp:27-28): gate/up Q4_K or Q5_K, down Q8_0 or Q5_1.
     Device rawdots == the oracle's down rows on the device's own h image, bit for bit; the combine likewise; and, when the
