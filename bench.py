@@ -229,6 +229,66 @@ def extra_config3_executor_formats(strix, torch, cfg, steps, warmup, with_cpu):
     return out
 
 
+def extra_union_rows(strix, torch, steps, warmup):
+    """The union rows form of the A8 entry points (R = 8 rows of a verify window; geometry and routes of the reference's device
+    test, tests/hip_moe_a8_union_tests.hip:117-119: hidden = intermediate = 1536, 64 experts top-16, Q4_K gate / up, Q6_K down):
+    probe + down quantise + down rows in three calls that read every distinct expert once, beside the same rows as eight
+    single-row call triples. Weight sets rotate so that no pass finds its experts in the cache."""
+    H, I, E, K, R = 1536, 1536, 64, 16, 8
+    gen = torch.Generator(device="cuda").manual_seed(23)
+    ids = torch.tensor([[(k * 5 + r * 3) % E for k in range(K)] for r in range(R)], dtype=torch.int32, device="cuda")
+    x = torch.randn((R, H), device="cuda", generator=gen).to(torch.bfloat16)
+    sets = []
+    for _ in range(6):                                           # 6 x 0.36 GB of experts
+        gate, up = device_q4k(torch, gen, (E, I), H), device_q4k(torch, gen, (E, I), H)
+        down = device_blocks(torch, gen, E * H, I // 256, 210, (209,), 0x08).reshape(E, H, -1)
+        un = strix.A8Decode(H, I, E, K, gate, up, down, rows=R, down_type=strix.TYPE_Q6_K)
+        one = strix.A8Decode(H, I, E, K, gate, up, down, rows=1, down_type=strix.TYPE_Q6_K)
+        un.input.copy_(x)
+        un.routes.copy_(ids)
+        sets.append((un, one))
+    n = len(sets)
+
+    def union_step(i):
+        un = sets[i % n][0]
+        un.enqueue_probe_union()
+        un.enqueue_down_activation_quantize_union()
+        un.enqueue_down_rawdots_union()
+
+    def single_step(i):
+        one = sets[i % n][1]
+        for r in range(R):                                       # (the row's input and routes are in place: only the calls are timed)
+            one.enqueue_probe()
+            one.enqueue_down_activation_quantize()
+            one.enqueue_down_rawdots()
+    for _, one in sets:
+        one.input.copy_(x[:1])
+        one.routes.copy_(ids[:1])
+    # the calls are shorter than their Python wrappers: one pass over the weight sets of each form is captured in a HIP graph
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graphs = []
+    with torch.cuda.stream(side):
+        for step in (union_step, single_step):
+            for i in range(n):
+                step(i)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(n):
+                    step(i)
+            graphs.append(graph)
+    torch.cuda.synchronize()
+    sec = time_steps(torch, lambda i: graphs[0].replay(), max(steps // 4, 10), 3) / n
+    sec_single = time_steps(torch, lambda i: graphs[1].replay(), max(steps // 4, 10), 3) / n
+    if any(int(un.status.item()) or int(one.status.item()) for un, one in sets):
+        raise RuntimeError("union rows: a run set status bits: the timing is void")
+    u = int(torch.unique(ids).numel())
+    nbytes = u * (2 * I * Q4K_ROW(H) + H * (I // 256) * 210) + R * H * 2 + R * K * (3 * I * 4 + I * 1.25 + H * 4)
+    return {"a8_union_rows_R8_q6_k_down": {"us": sec * 1e6, "us_as_8_single_row_calls": sec_single * 1e6, "distinct_experts": u, "assignments": R * K,
+                                           "GBps": nbytes / sec / 1e9, "hbm_frac": nbytes / sec / 1e9 / HBM_PEAK_GBPS, "algorithmic_bytes": nbytes}}
+
+
 def prefill_config4(strix, torch, gen, keep=False, reps=10):
     """BASELINE config 4: 4096 fp16 rows, hidden 4096, 256 routed Q4_K experts top-8 (router logits + N(0, 1.5) per-expert bias:
     Zipf-like load) of intermediate 2048, plus the always-on shared Q8_0 expert; router + shared expert + routed experts +
@@ -550,6 +610,7 @@ def main():
         small = extra_config3_small(strix, torch, cfg, args.steps, args.warmup) if args.tokens >= 4 else {}
         small.update(extra_config3_executor_formats(strix, torch, cfg, args.steps, args.warmup, not args.no_cpu))
         del cfg.layers[1:]
+        small.update(extra_union_rows(strix, torch, args.steps, args.warmup))
         out["extra"] = {**small, **extra_configs(strix, torch, args.steps, args.warmup)}
     if args.extra:
         out["prefill"] = out["extra"]["config4_prefill_T4096_f16_mfma"]

@@ -99,12 +99,81 @@ int32_t a8_validate_down(const mi355_a8_down_request* q, const mi355_a8_down_bin
 }
 
 // ---------------------------------------------------------------------------------------------------------- kernels
+// The union plan of R x top_k routes, built by the first two wavefronts of one 256-thread workgroup, thread t = assignment t = (row t / top_k, slot t % top_k).
+// An assignment is a "first" when no earlier assignment names its expert; the firsts, in assignment order, are the entries.
+// An expert id >= experts or an expert named twice by one row sets MI355_STATUS_INVALID_ROUTE and leaves count = 0 (no sweep
+// runs). All 128 entries are written: the unused ones hold expert 0 and 0xff slots.
+__device__ __forceinline__ void a8_union_plan_block(const uint32_t* routes, uint32_t rows, uint32_t top_k, uint32_t experts, uint32_t* plan, uint32_t* status) {
+    __shared__ __attribute__((aligned(16))) uint32_t expert_of[kUnionEntries];
+    __shared__ uint32_t entry_of_first[kUnionEntries], entry_expert[kUnionEntries];
+    __shared__ uint8_t entry_slots[kUnionEntries][kUnionRows];
+    __shared__ uint32_t firsts_in_wave0, invalid;
+    const uint32_t t = threadIdx.x, n = rows * top_k, lane = t & 63U;
+    const bool mine = t < kUnionEntries;                   // thread t of the first two wavefronts = assignment t = entry t
+    uint32_t e = 0xffffffffU;
+    if (mine) {
+        if (t == 0) invalid = 0;
+        entry_expert[t] = 0;
+        reinterpret_cast<uint32_t*>(entry_slots[t])[0] = 0xffffffffU;
+        reinterpret_cast<uint32_t*>(entry_slots[t])[1] = 0xffffffffU;
+        if (t < n) e = routes[t];
+        expert_of[t] = e;
+    }
+    __syncthreads();
+    uint32_t first = t, before = 0;
+    bool is_first = false;
+    if (mine) {
+        bool bad = false;
+        if (t < n) {
+            // the earliest assignment with this expert: every lane reads every word (broadcast reads, no early exit to wait for)
+            typedef const uint32_t u32x4_s __attribute__((ext_vector_type(4)));
+            const u32x4_s* four = reinterpret_cast<const u32x4_s*>(expert_of);
+#pragma unroll 8
+            for (uint32_t a = 0; a < (n + 3U) / 4U; ++a) {
+                const auto q = four[a];
+                const uint32_t hit = q.x == e ? 4U * a : q.y == e ? 4U * a + 1U : q.z == e ? 4U * a + 2U : q.w == e ? 4U * a + 3U : 0xffffffffU;
+                first = hit < first ? hit : first;
+            }
+            bad = e >= experts || (first != t && first >= t - t % top_k);
+        }
+        is_first = t < n && first == t;
+        const uint64_t firsts = __ballot(is_first);
+        if (t == 0) firsts_in_wave0 = static_cast<uint32_t>(__popcll(firsts));
+        if (__ballot(bad) != 0 && lane == 0) invalid = 1;
+        before = static_cast<uint32_t>(__popcll(firsts & ((1ULL << lane) - 1ULL)));
+    }
+    __syncthreads();
+    if (mine) {
+        before += t >= 64U ? firsts_in_wave0 : 0U;
+        if (is_first) { entry_of_first[t] = before; entry_expert[before] = e; }
+    }
+    __syncthreads();
+    if (mine && t < n) entry_slots[entry_of_first[first]][t / top_k] = static_cast<uint8_t>(t % top_k);
+    __syncthreads();
+    if (!mine) return;
+    if (t == kUnionEntries - 1U) {         // (the last thread of the second wave knows the number of entries)
+        const uint32_t count = before + (is_first ? 1U : 0U);
+        plan[0] = invalid ? 0U : count; plan[1] = rows; plan[2] = top_k; plan[3] = 0U;
+        if (invalid) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+    }
+    uint32_t* entry = plan + 4U + 3U * t;
+    entry[0] = entry_expert[t];
+    entry[1] = reinterpret_cast<const uint32_t*>(entry_slots[t])[0];
+    entry[2] = reinterpret_cast<const uint32_t*>(entry_slots[t])[1];
+}
+
 // Route check + A8 image of the input rows of the probe (src/hip_moe_q4k_a8_probe.hip:41-90: validation and quantizer of one
 // row; here blockIdx.y = logical row). Block x quantises 8 groups of 32; block (0, row) also checks the row's routes.
 template <int KIND>
 __global__ __launch_bounds__(256) void a8_probe_prologue_kernel(const uint8_t* x, uint32_t hidden, const uint32_t* routes, uint32_t experts,
-                                                                uint32_t top_k, int8_t* codes, float* deltas, int32_t* sums, uint32_t* status) {
+                                                                uint32_t top_k, int8_t* codes, float* deltas, int32_t* sums, uint32_t* status,
+                                                                uint32_t* union_plan, uint32_t union_top_k) {
     const uint32_t r = blockIdx.y, groups = hidden / 32U, g = blockIdx.x * 8U + (threadIdx.x >> 5), j = threadIdx.x & 31U;
+    // the union rows form: one more block per launch builds the plan beside the quantiser's blocks
+    if (union_plan && blockIdx.x == gridDim.x - 1U) {
+        if (r == 0) a8_union_plan_block(routes, gridDim.y, union_top_k, experts, union_plan, status);
+        return;
+    }
     if (blockIdx.x == 0 && threadIdx.x < top_k && routes[r * top_k + threadIdx.x] >= experts) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
     if (g >= groups) return;
     // the probe contract's quantiser ("g32-sym127-zero1-finite-noflush", src/moe_q4k_a8_contract.cpp:67-91): delta = amax / 127
@@ -235,51 +304,6 @@ int32_t a8_validate_down_union(const mi355_a8_down_request* q, const mi355_a8_do
     return MI355_OK;
 }
 
-// The union plan of R x top_k routes, one workgroup of two wavefronts, thread t = assignment t = (row t / top_k, slot t % top_k).
-// An assignment is a "first" when no earlier assignment names its expert; the firsts, in assignment order, are the entries.
-// An expert id >= experts or an expert named twice by one row sets MI355_STATUS_INVALID_ROUTE and leaves count = 0 (no sweep
-// runs). All 128 entries are written: the unused ones hold expert 0 and 0xff slots.
-__global__ __launch_bounds__(kUnionEntries) void a8_union_plan_kernel(const uint32_t* routes, uint32_t rows, uint32_t top_k, uint32_t experts,
-                                                                     uint32_t* plan, uint32_t* status) {
-    __shared__ uint32_t expert_of[kUnionEntries], entry_of_first[kUnionEntries], entry_expert[kUnionEntries];
-    __shared__ uint8_t entry_slots[kUnionEntries][kUnionRows];
-    __shared__ uint32_t firsts_in_wave0, invalid;
-    const uint32_t t = threadIdx.x, n = rows * top_k, lane = t & 63U;
-    if (t == 0) invalid = 0;
-    entry_expert[t] = 0;
-    reinterpret_cast<uint32_t*>(entry_slots[t])[0] = 0xffffffffU;
-    reinterpret_cast<uint32_t*>(entry_slots[t])[1] = 0xffffffffU;
-    const uint32_t e = t < n ? routes[t] : 0xffffffffU;
-    expert_of[t] = e;
-    __syncthreads();
-    uint32_t first = t;
-    bool bad = false;
-    if (t < n) {
-        for (uint32_t a = 0; a < t; ++a)
-            if (expert_of[a] == e) { first = a; break; }
-        bad = e >= experts || (first != t && first >= t - t % top_k);
-    }
-    const bool is_first = t < n && first == t;
-    const uint64_t firsts = __ballot(is_first);
-    if (t == 0) firsts_in_wave0 = static_cast<uint32_t>(__popcll(firsts));
-    if (__ballot(bad) != 0 && lane == 0) invalid = 1;
-    __syncthreads();
-    const uint32_t before = static_cast<uint32_t>(__popcll(firsts & ((1ULL << lane) - 1ULL))) + (t >= 64U ? firsts_in_wave0 : 0U);
-    if (is_first) { entry_of_first[t] = before; entry_expert[before] = e; }
-    __syncthreads();
-    if (t < n) entry_slots[entry_of_first[first]][t / top_k] = static_cast<uint8_t>(t % top_k);
-    __syncthreads();
-    if (t == kUnionEntries - 1U) {         // (the last thread of the second wave knows the number of entries)
-        const uint32_t count = before + (is_first ? 1U : 0U);
-        plan[0] = invalid ? 0U : count; plan[1] = rows; plan[2] = top_k; plan[3] = 0U;
-        if (invalid) atomicOr(status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
-    }
-    uint32_t* entry = plan + 4U + 3U * t;
-    entry[0] = entry_expert[t];
-    entry[1] = reinterpret_cast<const uint32_t*>(entry_slots[t])[0];
-    entry[2] = reinterpret_cast<const uint32_t*>(entry_slots[t])[1];
-}
-
 // the bundle of the single-row entry points: no plan, no job word of its own, R contiguous single-row extents per view
 inline RowsK a8_rows(const mi355_moe_weights& w) {
     return rows_k(mi355_moe_rows{}, w);
@@ -305,12 +329,12 @@ int32_t a8_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, uint32_t
     const uint8_t* x = reinterpret_cast<const uint8_t*>(b->input.address);
     const uint32_t* routes = reinterpret_cast<const uint32_t*>(b->routes.address);
     uint32_t* status = reinterpret_cast<uint32_t*>(b->status.address);
-    if (union_plan) a8_union_plan_kernel<<<1, kUnionEntries, 0, st>>>(routes, R, s.top_k, s.experts, union_plan, status);
-    const dim3 pgrid((groups + 7U) / 8U, R);
+    const dim3 pgrid((groups + 7U) / 8U + (union_plan ? 1U : 0U), R);
     const uint32_t checked = union_plan ? 0U : s.top_k;       // (the union builder has checked the routes)
     const auto prologue = [&](auto kind) {
         a8_probe_prologue_kernel<decltype(kind)::value><<<pgrid, 256, 0, st>>>(x, s.hidden, routes, s.experts, checked,
-            reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), status);
+            reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), status,
+            union_plan, s.top_k);
     };
     if (q->input == MI355_INPUT_F32) prologue(std::integral_constant<int, 0>{});
     else if (q->input == MI355_INPUT_F16) prologue(std::integral_constant<int, 1>{});
@@ -330,7 +354,9 @@ int32_t a8_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, uint32_t
     r.inter_rs = 4ULL * s.top_k * r.slot_stride;
     r.union_plan = union_plan;
     const uint32_t items = R * s.top_k;
-    if (union_plan) launch_project_nb<8>(w, r, R, dim3(s.rows / 32U, items), st);       // up to 8 holders share one sweep of an entry's expert
+    // up to 8 holders share one sweep of an entry's expert (an entry has at most R holders)
+    if (union_plan && R > 4U) launch_project_nb<8>(w, r, R, dim3(s.rows / 32U, items), st);
+    else if (union_plan) launch_project_nb<4>(w, r, R, dim3(s.rows / 32U, items), st);
     else if (q->gate_type == MI355_TYPE_Q5_K) project_q5k_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else if (items <= 16U) project_quad_kernel<4><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
     else if (items <= kQuadMaxItems) project_quad_kernel<2><<<dim3(s.rows / 32U, items), 256, 0, st>>>(w, r, items);
@@ -392,7 +418,8 @@ int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bind
     r.union_plan = union_plan;
     if (union_plan) {               // K-quant only: the items are the plan's entries
         if (q->weight_type == MI355_TYPE_Q6_K) launch_down_q6k(w, r, dim3(s.hidden / kDownGroupsRows, items), items, 0U, 0U, st);
-        else launch_down_nb<8>(w, r, logical_rows, dim3(s.hidden / 64U, items), st);
+        else if (logical_rows > 4U) launch_down_nb<8>(w, r, logical_rows, dim3(s.hidden / 64U, items), st);
+        else launch_down_nb<4>(w, r, logical_rows, dim3(s.hidden / 64U, items), st);
     } else if (q->weight_type != MI355_TYPE_Q4_K) {
         const dim3 grid(s.hidden / kDownGroupsRows, items);
         if (q->weight_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, items, 0U, 0U);
