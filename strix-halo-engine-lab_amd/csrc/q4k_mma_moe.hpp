@@ -113,7 +113,10 @@ __global__ __launch_bounds__(256 * TEAMS) void q4k_mma_down_kernel(mi355_moe_wei
             const uint32_t a = 2U * v + (lane >> 5);
             if (a >= n) return;
             if (GATE_UP) r.inter_of(inter, slot_of(a))[row0 + (lane & 31U)] = value[0];
-            else r.rawdots_of(slot_of(a), w.hidden)[row0 + (lane & 31U)] = value[0];
+            else {
+                r.rawdots_of(slot_of(a), w.hidden)[row0 + (lane & 31U)] = value[0];
+                if (r.top1_form) r.publish_top1(slot_of(a), row0 + (lane & 31U), value[0]);      // (top-1: assignment = row)
+            }
         });
     }
 }

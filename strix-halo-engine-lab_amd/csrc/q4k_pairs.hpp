@@ -33,6 +33,7 @@ struct PairArgs {
     uint32_t nacts;
     const uint32_t* skip_flag;   // optional: the launch does nothing when *skip_flag & skip_mask
     uint32_t skip_mask;
+    RowsK publish;               // publish.top1_form != 0: matrix 0 holds a top-1 job's down rows, and each value's row output is published with it
 };
 
 constexpr uint32_t kPairBlocks = 4;                              // super-blocks per stage
@@ -221,7 +222,10 @@ __global__ __launch_bounds__(64, 2) void q4k_pairs_kernel(PairArgs args) {
             v = v + xor2_f(v);      // (acc0 + acc1) + (acc2 + acc3)
         }
         const uint32_t a = al + AL * i;
-        if (p == 0 && kl == 0 && a < args.nacts) m.out[static_cast<size_t>(a) * m.out_stride + row0 + r] = v;
+        if (p == 0 && kl == 0 && a < args.nacts) {
+            m.out[static_cast<size_t>(a) * m.out_stride + row0 + r] = v;
+            if (args.publish.top1_form) args.publish.publish_top1(a, row0 + r, v);
+        }
     }
 }
 

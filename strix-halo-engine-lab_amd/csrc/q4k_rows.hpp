@@ -90,6 +90,7 @@ struct RowsK : mi355_moe_rows {
     uint32_t top_k;
     uint32_t nonfinite_bit;   // what a non-finite gate / up / h value ORs into its row's status (8; the host executor's job: 1)
     const uint32_t* union_plan;     // verify-window form: the expert-union plan (below) names the items instead of `plan`
+    uint32_t top1_form;       // a dense top-1 job whose down launch also publishes the output: combine form + 1 (0: the merge launch does)
 
     __device__ __forceinline__ void place(uint32_t i, uint32_t& row, uint32_t& slot) const {
         if (assignments) { row = assignments[i].row; slot = assignments[i].slot; }
@@ -107,6 +108,17 @@ struct RowsK : mi355_moe_rows {
     }
     __device__ __forceinline__ const float* base_of(uint32_t row) const {
         return reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(base) + row * base_rs);
+    }
+    // The ordered combine of a top-1 row at the place that produced its one unweighted value (include/strix/moe/combine.hpp:36-59 with
+    // one slot; product-then-add of src/ds41_expert_tp.cpp:189-199 likewise): fail closed on a flagged row, the aggregate bit for
+    // a non-finite output. The caller has checked the job word.
+    __device__ __forceinline__ void publish_top1(uint32_t row, uint32_t o, float raw) const {
+        if (*status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE)) return;
+        const float wt = route_weights_of(row)[0];
+        const float acc = top1_form == MI355_COMBINE_FMA_SLOT_ORDER + 1U ? __builtin_fmaf(wt, raw, 0.0F) : 0.0F + wt * raw;
+        const float y = base ? acc + base_of(row)[o] : acc;
+        if (!finite_f(y)) atomicOr(status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+        output[static_cast<size_t>(row) * output_stride + o] = y;
     }
     // the `hidden` unweighted outputs of assignment i
     __device__ __forceinline__ float* rawdots_of(uint32_t i, uint32_t hidden) const {

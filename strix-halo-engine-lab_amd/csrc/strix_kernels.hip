@@ -1309,6 +1309,7 @@ inline void launch_down_dense(const mi355_moe_weights& w, const RowsK& r, uint32
     a.m[0] = PairMatrix{w.down, w.down_row_stride, r.rawdots, w.hidden};
     a.rows = w.hidden; a.blocks = w.ffn / 256U; a.img = r.h; a.nacts = rows;
     a.skip_flag = r.job_status; a.skip_mask = MI355_STATUS_NONFINITE_PROJECTION;
+    a.publish = r;                 // (r.top1_form != 0: the launch publishes the rows' outputs as well)
     launch_pairs(a, 1, st);
 }
 
@@ -1408,7 +1409,8 @@ inline void launch_project(const mi355_moe_weights& w, const RowsK& r, uint32_t 
     if (w.experts == 1U && rows > 4U) launch_project_nb<8>(w, r, rows, grid, st);
     else launch_project_nb<4>(w, r, rows, grid, st);
 }
-inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st, bool grouped = false) {
+// Returns true when the launch also published the output rows (a dense top-1 job with r.top1_form set: the two dense sweeps).
+inline bool launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t rows, uint32_t umax, hipStream_t st, bool grouped = false) {
     if (w.down_type != MI355_TYPE_Q4_K) {      // Q8_0 / Q5_1 (blocks of 32, four chains per row) and Q6_K (pairs per super-block)
         const uint32_t assignments = rows * w.top_k, items_at = plan_items_at(w.experts, assignments), order_at = plan_order_at(w.experts);
         const dim3 grid(w.hidden / kDownGroupsRows, umax);
@@ -1420,20 +1422,23 @@ inline void launch_down(const mi355_moe_weights& w, const RowsK& r, uint32_t row
         else if (w.down_type == MI355_TYPE_Q8_0) down_groups_kernel<0><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         else if (w.down_type == MI355_TYPE_Q5_1) down_groups_kernel<1><<<grid, 256, 0, st>>>(w, r, assignments, items_at, order_at);
         else launch_down_q6k(w, r, grid, assignments, items_at, order_at, st);
-        return;
+        return false;
     }
     if (!grouped && quad_sweep(w, rows)) {
         const uint32_t items = rows * w.top_k;
         if (items <= 16U) down_quad_kernel<4><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
         else down_quad_kernel<2><<<dim3(w.hidden / 64U, items), 256, 0, st>>>(w, r, items);
-        return;
+        return false;
     }
-    if (mma_dense(w, r, rows)) return launch_mma_down(w, r, rows, rows, 0, rows, st);
-    if (const uint32_t split = mma_grouped_split(w, rows); split && r.plan) return launch_mma_down(w, r, rows, 0, umax, split, st);
-    if (dense_pairs_ok(w, rows) && dense_rows(r, w)) return launch_down_dense(w, r, rows, st);
+    if (mma_dense(w, r, rows)) { launch_mma_down(w, r, rows, rows, 0, rows, st); return r.top1_form != 0; }
+    RowsK plain = r;
+    plain.top1_form = 0;
+    if (const uint32_t split = mma_grouped_split(w, rows); split && r.plan) { launch_mma_down(w, plain, rows, 0, umax, split, st); return false; }
+    if (dense_pairs_ok(w, rows) && dense_rows(r, w)) { launch_down_dense(w, r, rows, st); return r.top1_form != 0; }
     const dim3 grid(w.hidden / 64U, umax);
     if (w.experts == 1U && rows > 4U) launch_down_nb<8>(w, r, rows, grid, st);
     else launch_down_nb<4>(w, r, rows, grid, st);
+    return false;
 }
 // An expert's assignments are cut into work items of at most `split` rows: a wave's instruction stream grows with every
 // activation row it serves while its weight stream does not, so wide items finish last; the second read of a split
@@ -1811,7 +1816,12 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, u
     if (!(dense_pairs_ok(wv, rows) && r->gate_out && r->up_out))
         if (const int32_t rc = mi355_moe_enqueue_csr(w, r, rows, stream)) return rc;
     if (const int32_t rc = mi355_moe_enqueue_project(w, r, rows, stream)) return rc;
-    if (const int32_t rc = mi355_moe_enqueue_down(w, r, rows, stream)) return rc;
+    // a dense top-1 job: the down launch publishes each row's output with its one unweighted value (no merge launch)
+    RowsK k = rows_k(*r, wv);
+    if (wv.experts == 1U && wv.top_k == 1U && rows <= 65535U) k.top1_form = form + 1U;
+    const bool published = launch_down(wv, k, rows, item_bound(wv, rows), hs(stream));
+    STRIX_LAUNCHED("moe down");
+    if (published) return MI355_OK;
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }
 

@@ -547,6 +547,45 @@ def test_dense_q4k_ffn_is_the_single_expert_case(strix, H, I, batches):
 
 
 @pytest.mark.parametrize("combine", [0, 1])
+@pytest.mark.parametrize("H,I,T", [(1024, 2048, 1), (1024, 2048, 2), (1024, 2048, 4), (1280, 1792, 7), (1024, 2048, 12)])
+def test_dense_top1_job_publishes_its_rows_from_the_down_launch(strix, combine, H, I, T):
+    """A dense top-1 job through mi355_moe_enqueue has no merge launch: the dense sweeps (pair-per-lane for 1 - 2 rows, matrix
+    cores from 3) publish weight x value (+ base) with the value they computed. Output, rawdots and status words must equal the
+    staged entry points' (down, then merge) bit for bit, for both combine forms, weights other than 1, a base term, and a row
+    with an invalid route, which is flagged and publishes nothing."""
+    import ctypes as C
+    rng = np.random.default_rng(40 + T + combine)
+    gate, up, down = make_layer(rng, H, I, 1)
+    x = dev(rng.standard_normal((T, H)).astype(np.float16))
+    ids = torch.zeros((T, 1), dtype=torch.int32, device="cuda")
+    if T >= 2:
+        ids[1, 0] = 3                                            # no such expert: the row is flagged, the job goes on
+    w = dev((rng.standard_normal((T, 1)) * 0.7).astype(np.float32))
+    base = dev(rng.standard_normal((T, H)).astype(np.float32))
+    outs = []
+    for staged in (False, True):
+        layer = strix.MoeLayer(H, I, 1, 1, dev(gate), dev(up), dev(down), T, intermediates=True)
+        layer.output.fill_(-7.0)
+        if staged:
+            rows, rv = layer.rows_view(x, ids, w, base)
+            L, st = strix.lib(), torch.cuda.current_stream().cuda_stream
+            for call in (L.mi355_moe_enqueue_prologue, L.mi355_moe_enqueue_csr, L.mi355_moe_enqueue_project, L.mi355_moe_enqueue_down):
+                assert call(C.byref(layer.w), C.byref(rv), rows, C.c_void_p(st)) == 0, L.mi355_last_error()
+            assert L.mi355_moe_enqueue_merge(C.byref(layer.w), C.byref(rv), rows, combine, C.c_void_p(st)) == 0, L.mi355_last_error()
+        else:
+            layer.run(x, ids, w, base=base, combine=combine)
+        torch.cuda.synchronize()
+        outs.append((layer.output[:T].clone(), layer.rawdots[:T].clone(), layer.status[:T].clone()))
+    (y, raw, status), (y_s, raw_s, status_s) = outs
+    assert torch.equal(status, status_s) and torch.equal(raw, raw_s)
+    assert torch.equal(y.view(torch.int32), y_s.view(torch.int32))
+    good = [t for t in range(T) if t != 1]
+    assert all(int(status[t]) == 0 for t in good) and (T < 2 or (int(status[1]) != 0 and bool((y[1] == -7.0).all())))
+    want = orc.combine(combine, w.cpu().numpy(), np.zeros((T, 1), np.uint32), raw.cpu().numpy(), base=base.cpu().numpy())
+    assert np.array_equal(bits(y.cpu().numpy()[good]), bits(want[good]))
+
+
+@pytest.mark.parametrize("combine", [0, 1])
 @pytest.mark.parametrize("T,down_type", [(8, orc.Q4_K), (1, orc.Q4_K), (2, orc.Q4_K), (5, orc.Q4_K), (8, orc.Q8_0), (3, orc.Q8_0),
                                          (8, orc.Q6_K), (3, orc.Q6_K)])
 def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine, T, down_type):
