@@ -1012,6 +1012,126 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_quad_kernel(m
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
+// Down rows + combine in one launch for Q5_1 down rows of whole, 16-byte aligned super-blocks (the host executor's format,
+// src/cpu/core/routed_expert.cpp:110-126): the workgroup of (row, 16 columns), wave k = the expert in slot k, each wave with
+// the copy ring, the lane layout and the chain order of down_q51_ring_kernel for its one assignment.
+template <int DEPTH>
+__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_q51_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
+    typedef const __attribute__((address_space(3))) u32x4 lds_u32x4;
+    typedef const __attribute__((address_space(3))) float lds_f32c;
+    typedef const __attribute__((address_space(3))) int32_t lds_i32c;
+    constexpr uint32_t kBlock = kQ51Block, RP = group_row_pieces(), WC = group_weight_copies(), PER = WC + 2U;
+    // a slot: the 16 rows' 8 groups (3 KB), the one assignment's 256 codes and its [8 deltas][8 sums]
+    constexpr uint32_t ROWB = kGroupStage * kBlock, CODES_AT = 1024U * WC, TABLE_AT = CODES_AT + 256U, SLOT = TABLE_AT + 64U;
+    static_assert(16U * ROWB == 1024U * WC, "the rows of a stage fill the weight copies");
+    __shared__ __attribute__((aligned(16))) uint8_t ring_mem[DEPTH][kDownMergeSlots][SLOT];
+    __shared__ float slot_value[kDownMergeSlots][16];
+    __shared__ uint32_t slot_order[kDownMergeSlots];
+    __shared__ float slot_weight[kDownMergeSlots];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, j = lane & 3U, rr = lane >> 2, row = blockIdx.y;
+    const uint32_t o0 = blockIdx.x * 16U, o = o0 + rr;
+    const uint32_t job = *r.job_status;                                        // (requested together with the item)
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), row * w.top_k + wave);
+    if (job & MI355_STATUS_NONFINITE_PROJECTION) return;                       // the whole job: no down rows, nothing published
+    float value = 0.0F;
+    if (item.begin != item.end) {                                              // (an invalid route has no item: its row is flagged)
+        const uint32_t src = item.first ? item.first - 1U : ordered(r, plan_order_at(w.experts), item.begin);
+        const uint32_t stages = w.ffn / 256U;
+        const uint8_t* rows = w.down + static_cast<size_t>(item.e) * w.down_expert_stride + static_cast<size_t>(o0) * w.down_row_stride;
+        // the lane's pieces of a stage: piece index i * 64 + lane = row * RP + piece of the row's 8-group segment
+        const uint8_t* wsrc[WC];
+#pragma unroll
+        for (uint32_t i = 0; i < WC; ++i) {
+            uint32_t k = i * 64U + lane;
+            k = k < 16U * RP ? k : 16U * RP - 1U;                  // padding lanes repeat the last piece into unused LDS
+            const uint32_t wr = k / RP, piece = k - RP * wr;
+            wsrc[i] = rows + static_cast<size_t>(wr) * w.down_row_stride + 16U * piece;
+        }
+        // the stage's 256 codes (lanes 0..15) and its [8 deltas][8 sums] (lanes 0..3)
+        const uint8_t* csrc = reinterpret_cast<const uint8_t*>(r.h.codes_of(src)) + 16U * (lane & 15U);
+        const uint32_t tq = lane & 3U;
+        const uint8_t* tsrc = tq < 2U ? reinterpret_cast<const uint8_t*>(r.h.deltas_of(src)) + 16U * tq : reinterpret_cast<const uint8_t*>(r.h.sums_of(src)) + 16U * (tq - 2U);
+        const auto start = [&](lds_u8* slot) {
+#pragma unroll
+            for (uint32_t i = 0; i < WC; ++i) {
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)wsrc[i],
+                                                 (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
+                wsrc[i] += ROWB;
+            }
+            if (lane < 16U)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)csrc,
+                                                 (__attribute__((address_space(3))) void*)(slot + CODES_AT), 16, 0, 0);
+            csrc += 256;
+            if (lane < 4U)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)tsrc,
+                                                 (__attribute__((address_space(3))) void*)(slot + TABLE_AT), 16, 0, 0);
+            tsrc += 32;
+        };
+        lds_u8* ring[DEPTH];
+#pragma unroll
+        for (int s = 0; s < DEPTH; ++s) ring[s] = (lds_u8*)ring_mem[s][wave];
+        float chain = 0.0F;
+#pragma unroll
+        for (int s = 0; s < DEPTH - 1; ++s)
+            if (static_cast<uint32_t>(s) < stages) start(ring[s]);
+        for (uint32_t b0 = 0; b0 < stages; b0 += DEPTH) {
+#pragma unroll
+            for (int s = 0; s < DEPTH; ++s) {
+                const uint32_t b = b0 + s;
+                if (b < stages) {
+                    const uint32_t last = b + DEPTH - 1U < stages ? b + DEPTH - 1U : stages;
+                    wait_stages_ahead<PER>(last - 1U - b);
+                    if (b + DEPTH - 1U < stages) start(ring[(s + DEPTH - 1) % DEPTH]);
+                    const lds_u8* slot = ring[s];
+#pragma unroll
+                    for (uint32_t c = 0; c < kGroupStage / 4U; ++c) {
+                        const uint32_t gl = 4U * c + j;                                 // the lane's group inside the stage
+                        float d, m;
+                        uint32_t q[8];
+                        load_q51_block_lds(slot + rr * ROWB + gl * kBlock, d, m, q);
+                        lds_u32x4* codes = (lds_u32x4*)(slot + CODES_AT + 32U * gl);
+                        const u32x4 c_lo = codes[0], c_hi = codes[1];
+                        const uint32_t cw[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+                        int dot = 0;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) dot = __builtin_amdgcn_sdot4(static_cast<int>(q[i]), static_cast<int>(cw[i]), dot, false);
+                        const float first = d * static_cast<float>(dot);
+                        const float combined = first + (m * static_cast<float>(*(lds_i32c*)(slot + TABLE_AT + 32U + 4U * gl)));
+                        chain = chain + (*(lds_f32c*)(slot + TABLE_AT + 4U * gl) * combined);
+                    }
+                }
+            }
+        }
+        value = chain;
+        value = value + xor1_f(value);          // chain0 + chain1 | chain2 + chain3
+        value = value + xor2_f(value);          // (chain0 + chain1) + (chain2 + chain3)
+        if (j == 0) r.rawdots_of(src, w.hidden)[o] = value;
+    }
+    if (j == 0) slot_value[wave][rr] = value;
+    if (threadIdx.x == 0) {
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
+        if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
+            for (uint32_t i = 1; i < w.top_k; ++i)
+                for (uint32_t jj = i; jj > 0 && r.routes_of(row)[slot_order[jj]] < r.routes_of(row)[slot_order[jj - 1]]; --jj) {
+                    const uint32_t t = slot_order[jj]; slot_order[jj] = slot_order[jj - 1]; slot_order[jj - 1] = t;
+                }
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights_of(row)[slot_order[k]];
+    }
+    __syncthreads();
+    // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is the combine's own)
+    if (threadIdx.x >= 16U || (*r.status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
+    float sum = 0.0F;
+    for (uint32_t k = 0; k < w.top_k; ++k) {
+        const float ev = slot_value[slot_order[k]][lane];
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER) sum = __builtin_fmaf(slot_weight[k], ev, sum);
+        else sum = sum + slot_weight[k] * ev;
+    }
+    const uint32_t oc = blockIdx.x * 16U + lane;
+    const float y = r.base ? sum + r.base_of(row)[oc] : sum;
+    if (!finite_f(y)) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    r.output[static_cast<size_t>(row) * r.output_stride + oc] = y;
+}
+
 // Down rows + combine in one launch for Q6_K down rows (src/moe_a8_down_contract.cpp:147-158): the workgroup of (row, 16 columns),
 // wave k = the expert in slot k, lane = (row, pair) with the direct loads and the order of down_q6k_kernel.
 __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_q6k_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
@@ -1906,6 +2026,12 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     }
     if (wv.down_type == MI355_TYPE_Q8_0 && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && wv.ffn % 128U == 0 && rows <= 65535U) {
         down_merge_q8_0_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        STRIX_LAUNCHED("moe layer experts + combine");
+        return MI355_OK;
+    }
+    if (wv.down_type == MI355_TYPE_Q5_1 && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && rows <= 65535U && wv.ffn % 256U == 0 &&
+        wv.down_row_stride % 16U == 0 && wv.down_expert_stride % 16U == 0) {       // (what down_q51_ring_kernel's copies need)
+        down_merge_q51_kernel<2><<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }

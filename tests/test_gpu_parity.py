@@ -587,13 +587,13 @@ def test_dense_top1_job_publishes_its_rows_from_the_down_launch(strix, combine, 
 
 @pytest.mark.parametrize("combine", [0, 1])
 @pytest.mark.parametrize("T,down_type", [(8, orc.Q4_K), (1, orc.Q4_K), (2, orc.Q4_K), (5, orc.Q4_K), (8, orc.Q8_0), (3, orc.Q8_0),
-                                         (8, orc.Q6_K), (3, orc.Q6_K)])
+                                         (8, orc.Q6_K), (3, orc.Q6_K), (8, orc.Q5_1), (3, orc.Q5_1)])
 def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine, T, down_type):
     """A decode batch whose (row, 64 columns) workgroups are all resident takes the down rows and the ordered combine in one
     launch (a wave per slot): output, rawdots and status words must equal the staged entry points' bit for bit, for both
     combine forms and with a base term. One to six rows take the same in the 16-rows-per-wavefront layout (T = 1, 2: the
     four-slot ring, T = 5: the two-slot ring); Q8_0 down rows (the host executor's format) in their four-chains-per-row layout,
-    dense Q6_K down rows through LDS."""
+    Q6_K down rows with direct loads, Q5_1 down rows through a copy ring per wave."""
     E, H, I, K = 32, 1024, 512, 8
     rng = np.random.default_rng(91 + combine + 7 * T + down_type)
     gate, up, down = make_layer(rng, H, I, E)
@@ -601,6 +601,8 @@ def test_layer_entry_down_rows_and_combine_in_one_launch(strix, combine, T, down
         down = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32))
     elif down_type == orc.Q6_K:
         down = orc.random_q6_k(rng, (E, H), I)
+    elif down_type == orc.Q5_1:
+        down = orc.random_q5_1(rng, (E, H), I)
     x = dev(rng.standard_normal((T, H)).astype(np.float16))
     wr = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
     base = dev(rng.standard_normal((T, H)).astype(np.float32))
