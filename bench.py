@@ -330,7 +330,7 @@ def prefill_config4(strix, torch, gen, keep=False, reps=10):
         "workload": "BASELINE config 4: 4096 fp16 rows, hidden 4096, 256 routed Q4_K experts top-8 (biased router) + 1 shared Q8_0 expert, intermediate 2048",
         "ms": sec_whole * 1e3, "TFLOPs": total / sec_whole / 1e12, "frac": total / sec_whole / MFMA_F16_PEAK_FLOPS, "peak": MFMA_F16_PEAK_FLOPS / 1e12,
         "unit": "TFLOP/s", "bound": "mfma", "dtype": "f16 operands, f32 accumulation", "algorithmic_flops": total,
-        "kernel": "prefill_f16_kernel (gate/up + SwiGLU, then down) of the routed experts",
+        "kernel": "prefill_reg_kernel<0> (gate/up + SwiGLU) and <1> (down) of the routed Q4_K experts; prefill_f16_kernel for the shared Q8_0 expert",
         "experts_ms": sec_f16 * 1e3, "experts_TFLOPs": flops_experts / sec_f16 / 1e12, "experts_frac": flops_experts / sec_f16 / MFMA_F16_PEAK_FLOPS,
         "router_ms": sec_route * 1e3, "shared_expert_ms": sec_shared * 1e3, "shared_expert_TFLOPs": flops_shared / sec_shared / 1e12,
         "note": "FAST class (fp16 MFMA on exact integer operands sc*q, fp32 block scales and accumulation), tolerance 2e-3 against the exact-weight product; router exact-order"}
