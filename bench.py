@@ -7,12 +7,13 @@ SwiGLU/re-quantise + down + ordered combine. Inputs are resident in HBM before t
 of the 256 MB last-level cache between steps, the steps rotate over several independent layers (distinct weights and
 tokens), as consecutive layers of a model do.
 
-Prints ONE JSON line. `value` = microseconds per layer (lower is better). `roofline` prices the dominant kernel (gate/up
-projection) by its algorithmic bytes against the 8 TB/s HBM peak, from HIP events recorded around that kernel on its own
-stream inside this run. `prefill` is the metric's second figure: BASELINE config 4 (4096 rows) on the matrix cores, TFLOP/s against
+Prints ONE JSON line. `value` = microseconds per layer (lower is better). `roofline` prices the dominant kernel (the layer's
+front launch: early routes, A8 prologue, the exact router and the gate/up projection) by its algorithmic bytes against the
+8 TB/s HBM peak, from HIP events recorded around that launch on its own stream inside this run. `prefill` is the metric's second figure: BASELINE config 4 (4096 rows) on the matrix cores, TFLOP/s against
 the fp16 MFMA peak. `cpu_baseline` times the CPU oracle (a port of the reference's CPU path) on the same layer, with the
 compiled reference's own Executor beside it where that library was built, the host CPU model and its read-bandwidth ceiling."""
 import argparse
+import ctypes as C
 import json
 import os
 import statistics
@@ -27,9 +28,10 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0     # MI355X published HBM3E peak
 MFMA_F16_PEAK_FLOPS = 2.5e15     # MI355X published dense fp16 MFMA peak
-# HBM bytes per launch of the gate/up kernel on the default workload, from two rocprofv3 --pmc passes (FETCH_SIZE scaled
-# x2.000, WRITE_SIZE x1.000 by a 256 MiB device copy in the same runs): profiles/project_wave_kernel_config3_moe_decode_T8.txt
-PROJECT_TRAFFIC_BYTES_DEFAULT = 99_723_264 + 147_466
+# HBM bytes per launch of the layer's front kernel on the default workload, from two rocprofv3 --pmc passes (FETCH_SIZE scaled
+# x2.000, WRITE_SIZE x1.000 by a 256 MiB device copy in the same runs): profiles/layer_front_kernel_config3_moe_decode_T8.txt
+FRONT_TRAFFIC_BYTES_DEFAULT = None
+FRONT_TRAFFIC_SOURCE = "profiles/layer_front_kernel_config3_moe_decode_T8.txt (a constant from that profile, not measured in this run)"
 Q4K_ROW = lambda k: k // 256 * 144
 
 
@@ -108,6 +110,31 @@ class Config3:
                 layer.stage("down", x, ids, wts)
                 layer.stage("merge", x, ids, wts)
         return total / reps
+
+    def halves_launch_us(self, reps):
+        """Mean durations of the layer's two launches on the timed path (mi355_moe_enqueue_layer_front / _back: the kernels the
+        whole call enqueues): the front launches of all rotating layers back to back between ONE pair of events on the launch
+        stream, then the back launches likewise (the pairs also span the gaps between the launches, about 1.5 us each)."""
+        torch = self.torch
+        front = back = 0.0
+        for _ in range(reps):
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+            e[0].record()
+            for layer, wr, x in self.layers:
+                layer.run_layer(x, wr, half="front")
+            e[1].record()
+            e[2].record()
+            for layer, wr, x in self.layers:
+                layer.run_layer(x, wr, half="back")
+            e[3].record()
+            torch.cuda.synchronize()
+            front += e[0].elapsed_time(e[1]) * 1e3 / len(self.layers)
+            back += e[2].elapsed_time(e[3]) * 1e3 / len(self.layers)
+        return front / reps, back / reps
+
+    def front_bytes(self, u):
+        # the front launch: router weight and the rows, gate + up rows of the touched experts, the A8 image written and read, the h image written
+        return self.E * self.H * 4 + self.T * self.H * 2 + self.project_bytes(u)
 
     def distinct_experts(self):
         out = []
@@ -365,14 +392,42 @@ def extra_configs(strix, torch, steps, warmup):
     sec = time_steps(torch, lambda i: torch.matmul(ga, gb), 10, 3)
     out["probe_fp16_gemm_8192_vendor_library"] = {"TFLOPs": 2.0 * 8192 ** 3 / sec / 1e12, "frac_of_fp16_mfma_peak": 2.0 * 8192 ** 3 / sec / 2.5e15}
     del ga, gb
-    # the matrix cores on their own: a register-operand MFMA loop of this library on every compute unit, with constant and with
-    # pseudo-random operands (the second is the ceiling a product on real data has under the chip's power limit)
+    # hand-written measurement kernels of the benchmark's own library (libmi355_bench_probes.so; not part of the product):
+    probes = load_probes()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # (a) the matrix cores on their own: a register-operand MFMA loop on every compute unit, with constant and with pseudo-random
+    #     operands (the second is the ceiling a product on real data has under the chip's power limit)
     sink = torch.empty(512 * 1024, dtype=torch.float32, device="cuda")
+    def mfma(rnd):
+        flops = C.c_uint64(0)
+        rc = probes.bench_probe_mfma_f16(20000, int(rnd), C.c_void_p(sink.data_ptr()), sink.numel(), C.byref(flops), stream)
+        assert rc == 0, rc
+        return flops.value
     for name, rnd in (("constant_operands", False), ("random_operands", True)):
-        flops = strix.probe_mfma_f16(20000, rnd, sink)
-        sec = time_steps(torch, lambda i: strix.probe_mfma_f16(20000, rnd, sink), 3, 1)
+        flops = mfma(rnd)
+        sec = time_steps(torch, lambda i: mfma(rnd), 3, 1)
         out["probe_mfma_f16_register_loop_" + name] = {"TFLOPs": flops / sec / 1e12, "frac_of_fp16_mfma_peak": flops / sec / 2.5e15}
     del sink
+    # (b) a read-only stream in the decode sweeps' own shape: one-wave workgroups, stages of 9,216 bytes, register loads or
+    #     global -> LDS copies through a ring, contiguous or as 144-byte blocks of 64 rows; launches of the decode layer's sizes
+    #     (1536 waves x 8 stages = the gate / up launch, 2048 x 3 = the down launch) and a 1 GiB stream. Every step reads a
+    #     different part of a 4 GiB buffer, so nothing is cache resident.
+    pool = torch.randint(0, 256, (4 << 30,), dtype=torch.uint8, device="cuda", generator=gen)
+    words = torch.empty(1 << 16, dtype=torch.int32, device="cuda")
+    reads = {}
+    for label, waves, stages in (("gate_up_launch_1536x8", 1536, 8), ("down_launch_2048x3", 2048, 3), ("stream_1GiB_14563x8", 14563, 8), ("stream_1GiB_1536x76", 1536, 76)):
+        nbytes = waves * stages * 9216
+        slots = pool.numel() // nbytes
+        for mode, mname in ((0, "registers"), (1, "lds_ring_contiguous"), (2, "lds_ring_144B_of_64_rows")):
+            for depth in (2, 4):
+                def run(i):
+                    at = (i % slots) * nbytes
+                    rc = probes.bench_probe_read_stream(C.c_void_p(pool.data_ptr() + at), waves, stages, mode, depth, C.c_void_p(words.data_ptr()), stream)
+                    assert rc == 0, rc
+                sec = time_steps(torch, run, 12 if nbytes < (1 << 29) else 4, 3)
+                reads[f"{label}_{mname}_depth{depth}"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+    out["probe_read_only_stream"] = reads
+    del pool, words
     # config 1: Q8_0 4096 x 4096 GEMV, one fp32 row
     n = 4096
     sets = []
@@ -443,6 +498,14 @@ def extra_configs(strix, torch, steps, warmup):
         "ms": sec * 1e3, "TFLOPs": (flops_experts + flops_router) / sec / 1e12, "algorithmic_flops": flops_experts + flops_router,
         "note": "same work in the bit-exact integer-dot class: int8 matrix-core group dots, the fp32 chain on the vector ALU (router included)"}
     return out
+
+
+def load_probes():
+    """The benchmark's own measurement kernels (strix-halo-engine-lab_amd/bench_probes/probes.hip), built by __graft_entry__.build()."""
+    lib = C.CDLL(os.path.join(ROOT, "strix-halo-engine-lab_amd", "libmi355_bench_probes.so"))
+    lib.bench_probe_read_stream.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+    lib.bench_probe_mfma_f16.argtypes = [C.c_uint32, C.c_uint32, C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
+    return lib
 
 
 def time_steps(torch, fn, steps, warmup):
@@ -587,8 +650,8 @@ def main():
     names = ("route", "prologue", "csr", "project", "down", "merge")
     staged_call_us = {n: statistics.mean(m[k].elapsed_time(m[k + 1]) for m in events) * 1e3 for k, n in enumerate(names)}
     project_us = cfg.project_launch_us(max(args.steps // len(cfg.layers), 4))
-    proj_s = project_us * 1e-6
-    achieved = cfg.project_bytes(u_mean) / proj_s / 1e9
+    front_us, back_us = cfg.halves_launch_us(max(args.steps // len(cfg.layers), 4))
+    achieved = cfg.front_bytes(u_mean) / (front_us * 1e-6) / 1e9
     layer_gbps = cfg.layer_bytes(u_mean) / sec / 1e9
 
     out = {
@@ -600,11 +663,14 @@ def main():
                    "tokens": args.tokens, "distinct_experts_mean": u_mean},
         "hbm_GBps_layer": layer_gbps, "hbm_frac_layer": layer_gbps / HBM_PEAK_GBPS,
         "layer_algorithmic_bytes": cfg.layer_bytes(u_mean), "staged_call_us": staged_call_us,
-        "roofline": {"bound": "hbm", "kernel": "project_wave_kernel (gate/up + SwiGLU + A8 re-quantise)", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": PROJECT_TRAFFIC_BYTES_DEFAULT if (args.tokens, args.layers) == (8, 6) else None,
-                     "algorithmic_bytes_per_launch": cfg.project_bytes(u_mean), "avg_launch_us": project_us,
-                     "timing": "HIP events on the launch stream around one back-to-back projection launch per rotating layer"},
+        "launch_us": {"front (layer_front_kernel)": front_us, "back (down_merge_kernel)": back_us,
+                      "staged gate/up alone (project_wave_kernel)": project_us},
+        "roofline": {"bound": "hbm", "kernel": "layer_front_kernel (early routes + A8 prologue + exact router + gate/up + SwiGLU + A8 re-quantise)",
+                     "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": FRONT_TRAFFIC_BYTES_DEFAULT if (args.tokens, args.layers) == (8, 6) else None,
+                     "traffic_source": FRONT_TRAFFIC_SOURCE,
+                     "algorithmic_bytes_per_launch": cfg.front_bytes(u_mean), "avg_launch_us": front_us,
+                     "timing": "HIP events on the launch stream around the front launches (mi355_moe_enqueue_layer_front) of all rotating layers enqueued back to back"},
     }
     if args.extra:
         small = extra_config3_small(strix, torch, cfg, args.steps, args.warmup) if args.tokens >= 4 else {}

@@ -59,11 +59,6 @@ enum { MI355_EXP_GFX1151 = 0, MI355_EXP_DECLARED = 1,
 
 const char* mi355_last_error(void);
 const char* mi355_version(void);
-/* Measurement aid of the benchmark (no counterpart in the reference, not a product path): one launch in which every wave of
- * every compute unit runs iterations x 4 independent v_mfma_f32_32x32x16_f16 on register operands - constant ones, or
- * (random_operands != 0) pseudo-random halves, whose switching power is what a real product meets. sink: at least 512
- * floats per compute unit; *flops = the launch's matrix-core FLOPs. */
-int32_t mi355_probe_mfma_f16(uint32_t iterations, uint32_t random_operands, float* sink, uint64_t sink_floats, uint64_t* flops, mi355_stream stream);
 /* Numerical identity strings this library implements (the caller opts in by passing them back, as with
  * Request::approved_numerical_identity, include/strix/moe_q4k_a8_contract.hpp:24-26,104-116). */
 const char* mi355_numerical_identity(uint32_t weight_type, int down);
@@ -221,7 +216,11 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights*, const mi355_moe_rows*, uint3
  * and weights), scores is a [rows][experts] workspace and output. For rows <= 16 the router, the A8 prologue and the expert
  * plan run in ONE launch (the workgroup that completes a row's logits also selects its experts and writes the row's work
  * items: one item per assignment, in assignment order; the CSR fields of the plan are not written), followed by project,
- * down and merge (down and merge share a launch when the batch is small enough for every workgroup to be resident). Where an
+ * down and merge (down and merge share a launch when the batch is small enough for every workgroup to be resident). Batches of
+ * 7 .. 16 rows over Q4_K experts of hidden <= 2048 run as two launches: the gate / up sweeps start on experts picked from
+ * lane-parallel logits while the reference's logit chains, softmax and selection run beside them in the same launch; an
+ * assignment whose early pick differs from the exact one is recomputed on the exact expert before the down rows, so the results
+ * are the exact router's in every case (the unweighted-output view serves as the early logits' scratch until then). Where an
  * expert's gate + up rows exceed 4 MB (and the batch is too large for the 16-rows-per-wavefront sweep) such a batch goes the
  * staged way instead - router, prologue, plan with up to two rows per work item - so that two rows that chose one expert
  * share one sweep of its weights; the results are the same bits. rows->plan must be zero-filled once when it is allocated; every launch leaves its ticket words zero, and
@@ -229,6 +228,23 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights*, const mi355_moe_rows*, uint3
 int32_t mi355_moe_enqueue_layer(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
                                 float* scores, const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows,
                                 uint32_t combine_form, mi355_stream);
+/* mi355_moe_enqueue_layer as its two halves, for a caller that places other work between them (the reference's walk enqueues
+ * moe_route / moe_experts and moe_combine as separate steps, include/strix/execution_plan.hpp:22-25) or times them apart:
+ * front = router, A8 prologue, expert plan, gate / up + SwiGLU + A8 of h; back = down rows + ordered combine on what the front
+ * call left in the row views. Both take the arguments of the whole call; front followed by back on one stream is that call. */
+int32_t mi355_moe_enqueue_layer_front(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
+                                      float* scores, const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows,
+                                      uint32_t combine_form, mi355_stream);
+int32_t mi355_moe_enqueue_layer_back(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
+                                     float* scores, const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows,
+                                     uint32_t combine_form, mi355_stream);
+
+/* Test aid of the decode layer (no counterpart in the reference). A decode batch on the 64-row sweeps picks its experts from
+ * lane-parallel logits in a short first launch and runs the reference's logit chain, softmax and selection beside the
+ * projection; where the two choices differ the assignment is recomputed on the exact expert before the down rows. The results
+ * are the exact router's either way. amount != 0 displaces the early logits (by amount * 1e-3 * a per-expert integer in
+ * -8..7) so that a test can make the choices differ; 0 (the default) restores them. Process-wide; not for production use. */
+void mi355_debug_early_route_perturb(uint32_t amount);
 
 /* The layer with the RMSNorm of its input inside the first launch (the reference normalises the residual stream in front of
  * the MoE, src/ops/norm/norm.hpp:40-58, and runs the shared expert beside the routed ones, src/hip_shared_expert_launcher.hip):

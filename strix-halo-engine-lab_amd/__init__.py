@@ -222,7 +222,6 @@ def lib():
         L.mi355_a8_enqueue_down_activation_quantize.argtypes = [P, P, U, U, P]
         L.mi355_a8_enqueue_down_rawdots.argtypes = [P, P, U, P]
         L.mi355_a8_enqueue_down_rawdots_merge.argtypes = [P, P, P, P]
-        L.mi355_probe_mfma_f16.argtypes = [U, U, P, C.c_uint64, P, P]
         L.mi355_a8_validate_union.argtypes = [P, P, DeviceBytes]
         L.mi355_a8_enqueue_probe_union.argtypes = [P, P, DeviceBytes, P]
         L.mi355_a8_validate_down_union.argtypes = [P, P, U, DeviceBytes]
@@ -255,10 +254,10 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
-           "mi355_probe_mfma_f16", "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
+           "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
            "mi355_a8_enqueue_down_activation_quantize_union", "mi355_a8_enqueue_down_rawdots_union",
            "mi355_moe_strided_enqueue_prologue", "mi355_moe_strided_enqueue_csr", "mi355_moe_strided_enqueue_project", "mi355_moe_strided_enqueue_down",
            "mi355_moe_strided_enqueue_merge", "mi355_moe_strided_enqueue_commit", "mi355_moe_strided_enqueue", "mi355_executor_create",
@@ -309,13 +308,6 @@ def quantize_weight_rows(qtype, x):
     out = torch.empty(x.shape[:-1] + (row_bytes(qtype, x.shape[-1]),), dtype=torch.uint8, device=x.device)
     check(lib().mi355_quantize_weight_rows(qtype, _p(x), rows, x.shape[-1], _p(out), _stream()))
     return out
-
-
-def probe_mfma_f16(iterations, random_operands, sink):
-    """One launch of the matrix-core probe (mi355_probe_mfma_f16); returns its FLOPs. sink: fp32 device tensor, 512 floats per compute unit."""
-    flops = C.c_uint64(0)
-    check(lib().mi355_probe_mfma_f16(iterations, int(random_operands), _p(sink), sink.numel(), C.byref(flops), _stream()))
-    return flops.value
 
 
 def quantize_a8(x, want_sums=True):
@@ -526,7 +518,7 @@ class MoeLayer:
         return self.output[:rows]
 
     def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,
-                  scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED, shared_experts=0, norm=None):
+                  scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED, shared_experts=0, norm=None, half=None):
         """Router + experts + combine through mi355_moe_enqueue_layer. Returns (output, ids, weights, scores).
         shared_experts: the last `shared_experts` experts of the tensors are always on (the router picks among the others).
         norm: (weight or None, eps) - the RMSNorm of x runs inside the first launch (mi355_moe_enqueue_layer_normed); the
@@ -542,8 +534,9 @@ class MoeLayer:
         p = RoutePolicy(self.experts - shared_experts, self.top_k - shared_experts, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single),
                         exp_kind, shared_experts)
         if norm is None:
-            check(lib().mi355_moe_enqueue_layer(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), C.byref(self.w), C.byref(rv), rows,
-                                                combine, _stream()))
+            # half: "front" / "back" = the layer's two halves as calls of their own (mi355_moe_enqueue_layer_front / _back)
+            entry = lib().mi355_moe_enqueue_layer if half is None else getattr(lib(), "mi355_moe_enqueue_layer_" + half)
+            check(entry(C.byref(p), _p(router_weight), _p(bias), _p(self.scores), C.byref(self.w), C.byref(rv), rows, combine, _stream()))
         else:
             if not hasattr(self, "normed"):
                 self.normed = torch.zeros((self.max_rows, self.hidden), dtype=torch.float32, device=x.device)

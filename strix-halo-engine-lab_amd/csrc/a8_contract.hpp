@@ -239,9 +239,12 @@ __global__ __launch_bounds__(1024) void a8_slot_merge_kernel(SlotMergeArgs t) {
     __shared__ uint32_t flagged, invalid;
     if (threadIdx.x == 0) { flagged = 0; invalid = 0; }
     __syncthreads();
-    const uint32_t initial = *t.status;
+    // an invalid route fails the step whatever ran before: the rawdots launch in front of this one flags it as well, but a status
+    // word cleared in between must not let a stale accumulation through (src/hip_moe_q4k_a8_probe.hip:743)
     if (threadIdx.x < t.top_k && t.routes[threadIdx.x] >= t.experts) invalid = 1;
     __syncthreads();
+    if (threadIdx.x == 0 && invalid) atomicOr(t.status, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+    const uint32_t initial = *t.status | (invalid ? static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE) : 0U);
     if (initial == 0U) {
         const bool written = invalid == 0;
         for (uint32_t o = threadIdx.x; o < t.hidden; o += 1024U) {
@@ -414,6 +417,7 @@ int32_t a8_down_rawdots(const mi355_a8_down_request* q, const mi355_a8_down_bind
     r.status = reinterpret_cast<uint32_t*>(b->status.address);
     r.status_rs = 0;
     r.job_status = r.status;        // a non-finite projection recorded by the producer (bit 8) skips the rows, as in the layer entries
+    r.aggregate = reinterpret_cast<uint32_t*>(b->aggregate_status.address);      // (optional: 0 = not bound)
     const uint32_t items = logical_rows * s.top_k;
     r.union_plan = union_plan;
     if (union_plan) {               // K-quant only: the items are the plan's entries

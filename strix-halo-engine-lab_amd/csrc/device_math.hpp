@@ -130,6 +130,14 @@ __device__ __forceinline__ void swiglu_clamp(float& g, float& u, float limit) {
     u = u < -limit ? -limit : (u > limit ? limit : u);
 }
 
+// A store that another workgroup of the same launch reads (device scope: performed at the memory side, past the per-XCD
+// caches), or a plain one.
+template <class T>
+__device__ __forceinline__ void store_shared_or_plain(bool device_scope, T* p, T v) {
+    if (device_scope) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
 // ---- cross-lane moves inside a 64-wide wavefront ----------------------------------------------------------------
 // lane ^ 1 and lane ^ 2 are DPP quad permutes (no LDS traffic); wider distances go through the swizzle crossbar.
 __device__ __forceinline__ int xor1_i(int v) { return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true); }

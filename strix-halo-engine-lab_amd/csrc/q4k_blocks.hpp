@@ -1,0 +1,148 @@
+// Q4_K x A8 rows with one super-block per lane: the sweep whose stages are contiguous runs of memory.
+//
+// Rows in dense GGUF order lie back to back: R rows of B super-blocks are R * B * 144 consecutive bytes. A stage is such a
+// run - R * B <= 64 blocks, R the largest power of two that fits - copied global -> LDS as whole 1 KB pieces (a read-only
+// stream of this shape was measured at 20.6 us for 113 MB in 1536 waves against 22.6 us when a stage is one 144-byte block of
+// each of 64 rows 1152 bytes apart; 11.8 against 14.4 us for the 57 MB of 2048 waves x 3 stages). Lane l of the first R * B
+// evaluates block l % B of row l / B of the stage: the lane's block index never changes, so its share of the activation row
+// - 256 codes, 8 deltas, 8 sums - is loaded once into registers and no activation operand goes through LDS. A row's value is
+// the reference's chain over its blocks in ascending order,
+//   acc[p] = (((0 + t_0[p]) + t_1[p]) + ...) + t_(B-1)[p],  t_b[p] = x_2p + x_2p+1 of block b,  value = (acc0 + acc1) + (acc2 + acc3),
+// run across the row's B neighbouring lanes as B - 1 shift-and-add steps (a whole-wave DPP shift by one lane), so the bits are
+// those of q4k_rows.hpp's lane-per-row sweep. One activation row per sweep.
+// Reference arithmetic: src/cpu/core/routed_expert.cpp:73-108 == src/moe_q4k_a8_contract.cpp:126-140.
+#pragma once
+#include "q4k_rows.hpp"
+
+namespace strix950 {
+
+struct BlockLanes { uint32_t B, R, used, stage_bytes; };
+constexpr uint32_t kBlockLaneCopies = 9;        // copy instructions per stage (a stage is at most 9,216 bytes)
+// max_rows: the rows of one contiguous run (a power of two)
+__host__ __device__ inline bool block_lanes_ok(uint32_t B, uint32_t max_rows) { return B >= 1U && B <= 64U && max_rows >= 1U; }
+__host__ __device__ inline BlockLanes block_lanes(uint32_t B, uint32_t max_rows) {
+    uint32_t R = 1;
+    while (2U * R * B <= 64U && 2U * R <= max_rows) R *= 2U;
+    return BlockLanes{B, R, R * B, R * B * 144U};
+}
+
+template <int N> __device__ __forceinline__ void block_lane_wait() { __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8)); }
+
+__device__ __forceinline__ float wave_shr1(float v) {       // lane l receives lane l - 1's value (lane 0: 0)
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138, 0xF, 0xF, true));
+}
+
+// stage_base(s): first byte of stage s (16-byte aligned). Returns, in lane i < stages * R, the value of row i (rows in stage
+// order) against image row `image_row` of img; other lanes: 0. slots: DEPTH separate LDS objects of >= 9,216 bytes with
+// nothing in flight; on exit every copy has landed and been consumed.
+template <int DEPTH, class StageBase>
+__device__ __forceinline__ float sweep_block_lanes(lds_u8* const (&slots)[DEPTH], StageBase stage_base, uint32_t stages, const BlockLanes g,
+                                                   const A8Image& img, uint32_t image_row) {
+    typedef const __attribute__((address_space(3))) u32x4 lds_u32x4;
+    const uint32_t lane = threadIdx.x & 63U;
+    const bool active = lane < g.used;
+    const uint32_t b = active ? lane % g.B : 0U, r_in_stage = lane / g.B;
+    // every copy instruction moves 64 pieces of 16 bytes; the pieces past the stage's end re-read its first piece into the slot's
+    // unused tail, so that each stage is the same number of operations and the waits can count them
+    uint32_t piece_offset[kBlockLaneCopies];
+#pragma unroll
+    for (uint32_t i = 0; i < kBlockLaneCopies; ++i) {
+        const uint32_t at = (i * 64U + lane) * 16U;
+        piece_offset[i] = at < g.stage_bytes ? at : 0U;
+    }
+    const auto start = [&](uint32_t s, lds_u8* slot) {
+        const uint8_t* base = stage_base(s);
+#pragma unroll
+        for (uint32_t i = 0; i < kBlockLaneCopies; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + piece_offset[i]),
+                                             (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
+    };
+#pragma unroll
+    for (int s = 0; s < DEPTH - 1; ++s)
+        if (static_cast<uint32_t>(s) < stages) start(static_cast<uint32_t>(s), slots[s]);
+    // the lane's share of the activation row: block b's 256 codes, 8 deltas, 8 sums
+    u32x4 code[16];
+    float delta[8], fsum[8];
+    {
+        const u32x4* cs = reinterpret_cast<const u32x4*>(img.codes_of(image_row) + 256U * b);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) code[i] = cs[i];
+        const f32x4* ds = reinterpret_cast<const f32x4*>(img.deltas_of(image_row) + 8U * b);
+        const f32x4 d0 = ds[0], d1 = ds[1];
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+        const i32x4* ss = reinterpret_cast<const i32x4*>(img.sums_of(image_row) + 8U * b);
+        const i32x4 s0 = ss[0], s1 = ss[1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            delta[j] = d0[j]; delta[4 + j] = d1[j];
+            fsum[j] = static_cast<float>(s0[j]); fsum[4 + j] = static_cast<float>(s1[j]);
+        }
+    }
+    float value = 0.0F;
+    for (uint32_t s0 = 0; s0 < stages; s0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const uint32_t s = s0 + d;
+            if (s < stages) {
+                // started so far: stages 0 .. min(stages, s + DEPTH - 1) - 1; stage s must have landed (the activation loads, issued
+                // after the first DEPTH - 1 stages, are older than every later stage)
+                const uint32_t last = s + DEPTH - 1U < stages ? s + DEPTH - 1U : stages, ahead = last - 1U - s;
+                if (ahead == 0) block_lane_wait<0>();
+                else if (ahead == 1) block_lane_wait<kBlockLaneCopies>();
+                else if (ahead == 2) block_lane_wait<2 * kBlockLaneCopies>();
+                else block_lane_wait<3 * kBlockLaneCopies>();
+                if (s + DEPTH - 1U < stages) start(s + DEPTH - 1U, slots[(d + DEPTH - 1) % DEPTH]);
+                lds_u32x4* blk = (lds_u32x4*)(slots[d] + (active ? lane : 0U) * 144U);
+                const u32x4 hd = blk[0];
+                u32x4 q[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = blk[1 + i];
+                const float dd = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
+                uint32_t sc[8], mn[8];
+                q4k_factors<0>(hd, sc[0], mn[0]); q4k_factors<1>(hd, sc[1], mn[1]); q4k_factors<2>(hd, sc[2], mn[2]); q4k_factors<3>(hd, sc[3], mn[3]);
+                q4k_factors<4>(hd, sc[4], mn[4]); q4k_factors<5>(hd, sc[5], mn[5]); q4k_factors<6>(hd, sc[6], mn[6]); q4k_factors<7>(hd, sc[7], mn[7]);
+                float t[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const uint32_t wq[8] = {q[2 * p].x, q[2 * p].y, q[2 * p].z, q[2 * p].w, q[2 * p + 1].x, q[2 * p + 1].y, q[2 * p + 1].z, q[2 * p + 1].w};
+                    const uint32_t c[16] = {code[4 * p].x, code[4 * p].y, code[4 * p].z, code[4 * p].w, code[4 * p + 1].x, code[4 * p + 1].y, code[4 * p + 1].z, code[4 * p + 1].w,
+                                            code[4 * p + 2].x, code[4 * p + 2].y, code[4 * p + 2].z, code[4 * p + 2].w, code[4 * p + 3].x, code[4 * p + 3].y, code[4 * p + 3].z, code[4 * p + 3].w};
+                    int dot0 = 0, dot1 = 0;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        dot0 = __builtin_amdgcn_sdot4(static_cast<int>(wq[k] & 0x0f0f0f0fU), static_cast<int>(c[k]), dot0, false);
+                        dot1 = __builtin_amdgcn_sdot4(static_cast<int>((wq[k] >> 4) & 0x0f0f0f0fU), static_cast<int>(c[8 + k]), dot1, false);
+                    }
+                    const float D0 = dd * static_cast<float>(sc[2 * p]), D1 = dd * static_cast<float>(sc[2 * p + 1]);
+                    const float M0 = dm * static_cast<float>(mn[2 * p]), M1 = dm * static_cast<float>(mn[2 * p + 1]);
+                    const float u0 = D0 * static_cast<float>(dot0), v0 = M0 * fsum[2 * p];
+                    const float u1 = D1 * static_cast<float>(dot1), v1 = M1 * fsum[2 * p + 1];
+                    const float t0 = u0 - v0, t1 = u1 - v1;
+                    const float x0 = delta[2 * p] * t0, x1 = delta[2 * p + 1] * t1;
+                    t[p] = x0 + x1;
+                }
+                // the row's chain over its blocks: after step i the lanes of blocks 0..i hold their prefix
+                float acc[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) acc[p] = 0.0F + t[p];
+                for (uint32_t step = 1; step < g.B; ++step) {
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const float chained = wave_shr1(acc[p]) + t[p];
+                        acc[p] = b == 0 ? acc[p] : chained;
+                    }
+                }
+                const float row_value = (acc[0] + acc[1]) + (acc[2] + acc[3]);      // valid in the lane of the row's last block
+                // row i of the stage sits in lane i * B + B - 1; the sweep's row s * R + i belongs in lane s * R + i
+                for (uint32_t i = 0; i < g.R; ++i) {
+                    const int got = __builtin_amdgcn_readlane(__builtin_bit_cast(int, row_value), static_cast<int>(i * g.B + g.B - 1U));
+                    value = lane == s * g.R + i ? __builtin_bit_cast(float, got) : value;
+                }
+                (void)r_in_stage;
+            }
+        }
+    }
+    return value;
+}
+
+}  // namespace strix950

@@ -91,6 +91,9 @@ struct RowsK : mi355_moe_rows {
     uint32_t nonfinite_bit;   // what a non-finite gate / up / h value ORs into its row's status (8; the host executor's job: 1)
     const uint32_t* union_plan;     // verify-window form: the expert-union plan (below) names the items instead of `plan`
     uint32_t top1_form;       // a dense top-1 job whose down launch also publishes the output: combine form + 1 (0: the merge launch does)
+    uint32_t* aggregate;      // optional summary word of the A8 down bindings (include/strix/moe_a8_down_contract.hpp:50-52): bit 16 beside a row's flag
+    uint32_t* awords;         // a decode batch planned from early routes: one word per assignment (finished projection waves in the low
+                              // half, bit 31 = non-finite projection), in place of direct updates of the status words
 
     __device__ __forceinline__ void place(uint32_t i, uint32_t& row, uint32_t& slot) const {
         if (assignments) { row = assignments[i].row; slot = assignments[i].slot; }
@@ -185,6 +188,12 @@ __device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const 
         uint32_t row, slot;
         r.place(index, row, slot);
         e = r.routes_of(row)[slot];
+        // a route out of range: no item, and the row is flagged here as well - a caller may reach a down stage without the producer
+        // that checks the routes (down_rawdots_rows flags it itself, src/hip_moe_q4k_a8_probe.hip:743)
+        if (e >= w.experts) {
+            atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+            if (r.aggregate) atomicOr(r.aggregate, static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+        }
     }
     return {e, index, e < w.experts ? index + 1U : index, index + 1U};      // an invalid route has no item (its row is flagged)
 }

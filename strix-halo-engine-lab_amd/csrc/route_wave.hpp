@@ -32,6 +32,10 @@ struct RouteArgs {
     // RMSNorm of the input rows inside the launch (norm_on): the router and the A8 image see y = (x * r) * norm_w, r = 1 / sqrt(mean(x^2) + eps)
     // in the declared order of src/cpu/core/reference.cpp:86-103; normed (optional) receives y as fp32 [rows][hidden]
     uint32_t norm_on; const float* norm_w; float norm_eps; float* normed;
+    // early-routes form (route_early.hpp): one word per assignment - the count of finished projection waves in the low half, a
+    // non-finite projection in bit 31 -, and a test knob that displaces the early logits so that the repair path runs
+    uint32_t* awords; uint32_t early_perturb;
+    float* early_logits; uint32_t early_stride;      // where the early logits of row i go: early_logits + i * early_stride (floats)
 };
 
 // r of one row by a 64-thread workgroup, bit for bit rmsnorm_f32_kernel: lane l of L = 256 (n >= 512) or 128 chains
@@ -507,8 +511,9 @@ __device__ __forceinline__ uint64_t key_max_wave(uint64_t key) {        // the w
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 // Returns, in lane k < top_k + shared_experts, the expert of slot k.
+// shared_out: ids and weights are also read by other workgroups of the same launch (device-scope stores).
 template <uint32_t PER>
-__device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const RouteArgs& a, uint32_t row) {
+__device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const RouteArgs& a, uint32_t row, bool shared_out) {
     const uint32_t lane = threadIdx.x & 63U, E = a.p.experts, K = a.p.top_k, P = K + a.p.shared_experts;
     float* z = a.scores + static_cast<size_t>(row) * E;
     float v[PER];
@@ -575,9 +580,9 @@ __device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const Rou
     }
     const float den = sum + a.p.renorm_eps;
     if (lane < K) {
-        a.ids[static_cast<size_t>(row) * P + lane] = my_id;
+        store_shared_or_plain(shared_out, a.ids + static_cast<size_t>(row) * P + lane, my_id);
         const bool renorm = a.p.renormalize && (K > 1U || a.p.renorm_single);      // include/strix/moe/route_policy.hpp:146
-        a.weights[static_cast<size_t>(row) * P + lane] = (renorm ? my_v / den : my_v) * a.p.scale;
+        store_shared_or_plain(shared_out, a.weights + static_cast<size_t>(row) * P + lane, (renorm ? my_v / den : my_v) * a.p.scale);
     } else if (lane < P) {      // the always-on experts behind the routed ones: ids experts .. experts + shared - 1, weight 1
         my_id = E + (lane - K);
         a.ids[static_cast<size_t>(row) * P + lane] = my_id;
@@ -586,12 +591,12 @@ __device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const Rou
     __syncthreads();
     return my_id;
 }
-__device__ __forceinline__ uint32_t route_select_row(float* p_lds, const RouteArgs& a, uint32_t row) {
+__device__ __forceinline__ uint32_t route_select_row(float* p_lds, const RouteArgs& a, uint32_t row, bool shared_out = false) {
     const uint32_t E = a.p.experts;
-    if (E <= 128U) return route_select_row_per<2>(p_lds, a, row);
-    if (E <= 256U) return route_select_row_per<4>(p_lds, a, row);
-    if (E <= 512U) return route_select_row_per<8>(p_lds, a, row);
-    return route_select_row_per<16>(p_lds, a, row);
+    if (E <= 128U) return route_select_row_per<2>(p_lds, a, row, shared_out);
+    if (E <= 256U) return route_select_row_per<4>(p_lds, a, row, shared_out);
+    if (E <= 512U) return route_select_row_per<8>(p_lds, a, row, shared_out);
+    return route_select_row_per<16>(p_lds, a, row, shared_out);
 }
 
 }  // namespace strix950

@@ -13,6 +13,7 @@
 
 #include "device_math.hpp"
 #include "q4k_rows.hpp"
+#include "q4k_blocks.hpp"
 #include "q4k_pairs.hpp"
 #include "q4k_mma.hpp"
 #include "q4k_quads.hpp"
@@ -22,6 +23,7 @@
 #include "prefill_f16.hpp"
 #include "prefill_reg.hpp"
 #include "route_wave.hpp"
+#include "route_early.hpp"
 
 namespace strix950 {
 
@@ -253,7 +255,22 @@ __host__ __device__ constexpr uint32_t pad4(uint32_t v) { return (v + 3U) & ~3U;
 // ticket / scratch words right after the header, at the same place for every batch size (every launch leaves them zero, and a
 // workspace is reused with varying row counts): [0, 16) row tickets of the fused router, [16, 32) its quantiser tickets,
 // [128, 144) per-row A8 flags of the fused prologue
-constexpr uint32_t kPlanTicketsAt = 16, kPlanTicketWords = 256, kPlanOffsetsAt = kPlanTicketsAt + kPlanTicketWords;
+constexpr uint32_t kPlanTicketsAt = 16, kPlanTicketWords = 256;
+// Behind the ticket words, also at a fixed place, the words of a decode batch planned from early routes (route_early.hpp):
+//   one word per assignment (finished projection waves in the low half, bit 31 = non-finite projection);
+//   one 64-bit tag per assignment {epoch, early expert};
+//   three 128-byte lines per row (arrival counts of the early blocks, of the A8 prologue blocks - with the row's flag word beside
+//     it - and of the exact router's side blocks) and a line with one tag per row (epoch of the call whose A8 image of that row is
+//     complete) and the epoch word.
+// Counts are zero when the plan is allocated and every launch leaves them zero. The epoch of a call is the epoch word + 1; the
+// call's down launch stores it back, so tags of earlier calls never look current and nothing has to be reset.
+constexpr uint32_t kLineWords = 32, kEarlyMaxAssignments = 128, kEarlyMaxRows = 16;
+constexpr uint32_t kPlanAwordsAt = kPlanTicketsAt + kPlanTicketWords, kPlanEtagsAt = kPlanAwordsAt + kEarlyMaxAssignments;
+constexpr uint32_t kPlanLinesAt = (kPlanEtagsAt + 2U * kEarlyMaxAssignments + kLineWords - 1U) / kLineWords * kLineWords;      // (lines of a 128-byte aligned plan)
+constexpr uint32_t kLinesEarly = 0, kLinesPrologue = kEarlyMaxRows * kLineWords, kLinesSide = 2U * kEarlyMaxRows * kLineWords;
+constexpr uint32_t kLinesRowTags = 3U * kEarlyMaxRows * kLineWords, kLinesEpoch = kLinesRowTags + kEarlyMaxRows;
+constexpr uint32_t kPlanOffsetsAt = kPlanLinesAt + kLinesRowTags + kLineWords;
+static_assert(kPlanEtagsAt % 2U == 0 && kPlanOffsetsAt % 4U == 0, "tags on 8 bytes, the plan arrays on 16");
 __host__ __device__ constexpr uint32_t plan_touched_at(uint32_t experts) { return kPlanOffsetsAt + pad4(experts + 1U); }
 __host__ __device__ constexpr uint32_t plan_order_at(uint32_t experts) { return plan_touched_at(experts) + pad4(experts); }
 // most work items a plan can hold (layout) and most a launch with pieces of `split` assignments can produce (grid size)
@@ -280,6 +297,66 @@ template <int KIND>
 __global__ __launch_bounds__(256, 2) void route_batch_kernel(RouteArgs a) {
     __shared__ __attribute__((aligned(16))) BatchTiles lds;
     route_batch_block<KIND>(lds, a, blockIdx.y * kBatchTile, blockIdx.x * kBatchTile);
+}
+
+// A8 prologue block qb of a fused decode launch (src/cpu/core/reference.cpp:35-55): two groups of 32 at a time, 8 groups per
+// block; the last of a row's blocks publishes the row's status word. scratch: 256 floats of LDS (fused RMSNorm only).
+// Row r counts its finished blocks in ticket[r * stride] and collects its flags in flags[r * stride]. LINES: the words are reached
+// by device-scope atomics only and the count is a plain arrival (route_early.hpp); otherwise the count is an acquire-release ticket.
+template <int KIND, bool NORM, bool LINES = false>
+__device__ __forceinline__ void a8_prologue_block(const RouteArgs& a, uint32_t qb, uint32_t* ticket, uint32_t* flags, uint32_t stride, float* scratch,
+                                                  uint32_t* row_tag = nullptr, uint32_t epoch = 0) {
+    const uint32_t lane = threadIdx.x;
+    {
+        const uint32_t groups = a.hidden / 32U, total = a.rows * groups, g0 = qb * 8U;
+        float factor = 1.0F;         // (a block's eight groups belong to one row: hidden % 256 == 0)
+        if constexpr (NORM) factor = row_norm_factor<KIND>(scratch, a.x + (g0 / groups) * a.x_stride, a.hidden, a.norm_eps);
+        for (uint32_t i = 0; i < 8U; i += 2U) {
+            const uint32_t g = g0 + i + (lane >> 5), j = lane & 31U;
+            if (g < total) {
+                const uint32_t r = g / groups, gi = g % groups;
+                float v = load_activation<KIND>(a.x + r * a.x_stride, gi * 32U + j);
+                if constexpr (NORM) {
+                    v = v * factor;
+                    if (a.norm_w) v = v * a.norm_w[gi * 32U + j];
+                    if (a.normed) a.normed[static_cast<size_t>(r) * a.hidden + gi * 32U + j] = v;
+                }
+                const float amax = max32(__builtin_fabsf(v));
+                const bool tiny = amax > 0.0F && amax < 0x1p-119F;
+                const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+                const int code = a8_code(v, delta, tiny);
+                const int sum = sum32_i(code);
+                const int bad = or32_i(finite_f(v) ? 0 : 1);
+                store_shared_or_plain(LINES, a.codes + static_cast<size_t>(r) * a.hidden + gi * 32U + j, static_cast<int8_t>(code));
+                if (j == 0) {
+                    store_shared_or_plain(LINES, a.deltas + static_cast<size_t>(r) * groups + gi, delta);
+                    store_shared_or_plain(LINES, a.sums + static_cast<size_t>(r) * groups + gi, static_cast<int32_t>(sum));
+                    if (bad) atomicOr(&flags[r * stride], static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
+                }
+            }
+        }
+        // the row's last quantiser block publishes the row's status word (a row's 32-groups fill whole blocks: hidden % 256 == 0)
+        // (the flag words are read-modify-written by device-scope atomics only; the ticket orders them as above)
+        const uint32_t r = g0 / groups;
+        if constexpr (LINES) {
+            // (the A8 image is written by device-scope stores: waves of the same launch, on other XCDs, read it once the row's tag says so)
+            if (arrive_last(&ticket[r * stride], groups / 8U)) {
+                if (lane == 0) {
+                    __hip_atomic_store(&a.status[r], __hip_atomic_load(&flags[r * stride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&flags[r * stride], 0U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                stores_acknowledged();
+                if (lane == 0) __hip_atomic_store(row_tag + r, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        } else {
+            __syncthreads();
+            if (lane == 0 && __hip_atomic_fetch_add(&ticket[r * stride], 1U, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == groups / 8U - 1U) {
+                a.status[r] = __hip_atomic_load(&flags[r * stride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                flags[r * stride] = 0;
+                ticket[r * stride] = 0;
+            }
+        }
+    }
 }
 
 // Decode router launch (rows <= 16). Blocks [0, route_blocks) run the logit chains of (row, 8 experts). In the plain form
@@ -346,44 +423,7 @@ __global__ __launch_bounds__(64) void route_decode_kernel(RouteArgs a) {
             }
         }
     } else {
-        // A8 prologue (src/cpu/core/reference.cpp:35-55): two groups of 32 at a time, 8 groups per block
-        const uint32_t groups = a.hidden / 32U, total = a.rows * groups, g0 = (bid - a.route_blocks) * 8U;
-        uint32_t* flags = tickets + 128U;
-        float factor = 1.0F;         // (a block's eight groups belong to one row: hidden % 256 == 0)
-        if constexpr (NORM) factor = row_norm_factor<KIND>(sel_p, a.x + (g0 / groups) * a.x_stride, a.hidden, a.norm_eps);
-        for (uint32_t i = 0; i < 8U; i += 2U) {
-            const uint32_t g = g0 + i + (lane >> 5), j = lane & 31U;
-            if (g < total) {
-                const uint32_t r = g / groups, gi = g % groups;
-                float v = load_activation<KIND>(a.x + r * a.x_stride, gi * 32U + j);
-                if constexpr (NORM) {
-                    v = v * factor;
-                    if (a.norm_w) v = v * a.norm_w[gi * 32U + j];
-                    if (a.normed) a.normed[static_cast<size_t>(r) * a.hidden + gi * 32U + j] = v;
-                }
-                const float amax = max32(__builtin_fabsf(v));
-                const bool tiny = amax > 0.0F && amax < 0x1p-119F;
-                const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
-                const int code = a8_code(v, delta, tiny);
-                const int sum = sum32_i(code);
-                const int bad = or32_i(finite_f(v) ? 0 : 1);
-                a.codes[static_cast<size_t>(r) * a.hidden + gi * 32U + j] = static_cast<int8_t>(code);
-                if (j == 0) {
-                    a.deltas[static_cast<size_t>(r) * groups + gi] = delta;
-                    a.sums[static_cast<size_t>(r) * groups + gi] = sum;
-                    if (bad) atomicOr(&flags[r], static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
-                }
-            }
-        }
-        // the row's last quantiser block publishes the row's status word (a row's 32-groups fill whole blocks: hidden % 256 == 0)
-        // (the flag words are read-modify-written by device-scope atomics only; the ticket orders them as above)
-        const uint32_t r = g0 / groups;
-        __syncthreads();
-        if (lane == 0 && __hip_atomic_fetch_add(&tickets[16U + r], 1U, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == groups / 8U - 1U) {
-            a.status[r] = __hip_atomic_load(flags + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            flags[r] = 0;
-            tickets[16U + r] = 0;
-        }
+        a8_prologue_block<KIND, NORM>(a, bid - a.route_blocks, tickets + 16U, tickets + 128U, 1U, sel_p);
     }
 }
 
@@ -536,24 +576,43 @@ __global__ __launch_bounds__(64) void clear_validate_kernel(const uint32_t* rout
 // gate rows of the group, lanes 32..63 the up rows; one cross-half exchange pairs them, then both halves evaluate the
 // same 32-value h group.
 // Reference: src/cpu/core/routed_expert.cpp:403-427 (gate item), :147-170 (swiglu_quantize).
-template <int NA, int DEPTH>
-__device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
-                                              const RowsK& r, uint32_t grp, uint32_t order_at, uint32_t c0) {
+template <int NA, class IndexOf>
+__device__ __forceinline__ void project_epilogue(const float (&value)[NA], const mi355_moe_weights& w, const RowsK& r, uint32_t grp, IndexOf index_of);
+
+// index_of(a): the assignment index of the sweep's activation row a < NA (a may differ between lanes).
+template <int NA, int DEPTH, bool NARROW = false, class IndexOf>
+__device__ __forceinline__ void project_chunk_of(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
+                                                 const RowsK& r, uint32_t grp, IndexOf index_of) {
     const uint32_t lane = threadIdx.x & 63U, o = lane & 31U;
     uint32_t sidx[NA], src[NA], lane_rows[(NA + 3) / 4];
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
-        sidx[a] = __builtin_amdgcn_readfirstlane(ordered(r, order_at, c0 + a));
+        sidx[a] = __builtin_amdgcn_readfirstlane(index_of(static_cast<uint32_t>(a)));
         src[a] = r.row_of(sidx[a]);
     }
 #pragma unroll
     for (int h = 0; h < (NA + 3) / 4; ++h) {
         const uint32_t a = 4U * h + (lane >> 4);
-        lane_rows[h] = r.row_of(ordered(r, order_at, c0 + (a < static_cast<uint32_t>(NA) ? a : 0U)));
+        lane_rows[h] = r.row_of(index_of(a < static_cast<uint32_t>(NA) ? a : 0U));
     }
     const ActRows<NA> act(r.in, src, lane_rows);
     float value[NA];
-    sweep_rows<NA, DEPTH>(slots, source, w.hidden / 256U, act, value);
+    sweep_rows<NA, DEPTH, NARROW>(slots, source, w.hidden / 256U, act, value);
+    project_epilogue<NA>(value, w, r, grp, index_of);
+}
+
+// SwiGLU + A8 re-quantisation of one 32-output group: lanes 0..31 hold the gate values, lanes 32..63 the up values of outputs
+// 32 grp .. 32 grp + 31 for each of the NA assignments index_of(0 .. NA - 1). Reference: src/cpu/core/routed_expert.cpp:147-170.
+template <int NA, class IndexOf>
+__device__ __forceinline__ void project_epilogue(const float (&value)[NA], const mi355_moe_weights& w, const RowsK& r, uint32_t grp, IndexOf index_of) {
+    const uint32_t lane = threadIdx.x & 63U, o = lane & 31U;
+    uint32_t sidx[NA], src[NA];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+        sidx[a] = __builtin_amdgcn_readfirstlane(index_of(static_cast<uint32_t>(a)));
+        src[a] = r.row_of(sidx[a]);
+    }
+    const bool ds = r.awords != nullptr;      // early routes: device-scope stores (an assignment may be written again by a repair)
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
         const float other = __shfl_xor(value[a], 32);
@@ -563,15 +622,18 @@ __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], con
         const float h = (gc / (1.0F + exp_of(w.exp_kind, -gc))) * uc;
         const uint32_t at_out = grp * 32U + o;
         if (lane < 32U) {
-            if (r.gate_out) r.inter_of(r.gate_out, sidx[a])[at_out] = g;
-            if (r.up_out) r.inter_of(r.up_out, sidx[a])[at_out] = u;
-            if (r.h_out) r.inter_of(r.h_out, sidx[a])[at_out] = h;
+            if (r.gate_out) store_shared_or_plain(ds, r.inter_of(r.gate_out, sidx[a]) + at_out, g);
+            if (r.up_out) store_shared_or_plain(ds, r.inter_of(r.up_out, sidx[a]) + at_out, u);
+            if (r.h_out) store_shared_or_plain(ds, r.inter_of(r.h_out, sidx[a]) + at_out, h);
         }
         if (!r.h.codes) continue;                         // projection only (the probe form): no A8 image of h
         if (or32_i((finite_f(g) && finite_f(u) && finite_f(h)) ? 0 : 1)) {
             if (lane == 0) {
-                atomicOr(r.status_of(src[a]), r.nonfinite_bit);
-                atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                if (r.awords) atomicOr(&r.awords[sidx[a]], 0x80000000U);        // early routes: per assignment, folded by the down launch
+                else {
+                    atomicOr(r.status_of(src[a]), r.nonfinite_bit);
+                    atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                }
             }
         } else {
             const float amax = max32(__builtin_fabsf(h));
@@ -579,13 +641,19 @@ __device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], con
             const float dl = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
             const int code = a8_code(h, dl, tiny);
             const int sum = sum32_i(code);
-            if (lane < 32U) r.h_codes_of(sidx[a])[at_out] = static_cast<int8_t>(code);
+            if (lane < 32U) store_shared_or_plain(ds, r.h_codes_of(sidx[a]) + at_out, static_cast<int8_t>(code));
             if (lane == 0) {
-                r.h_deltas_of(sidx[a])[grp] = dl;
-                r.h_sums_of(sidx[a])[grp] = sum;
+                store_shared_or_plain(ds, r.h_deltas_of(sidx[a]) + grp, dl);
+                store_shared_or_plain(ds, r.h_sums_of(sidx[a]) + grp, static_cast<int32_t>(sum));
             }
         }
     }
+}
+
+template <int NA, int DEPTH, bool NARROW = false>
+__device__ __forceinline__ void project_chunk(lds_u8* const (&slots)[DEPTH], const StageSource& source, const mi355_moe_weights& w,
+                                              const RowsK& r, uint32_t grp, uint32_t order_at, uint32_t c0) {
+    project_chunk_of<NA, DEPTH, NARROW>(slots, source, w, r, grp, [&](uint32_t a) { return ordered(r, order_at, c0 + a); });
 }
 
 #define STRIX_RING_SLOTS(DEPTH, NBMAX)                                                           \
@@ -635,6 +703,167 @@ __global__ __launch_bounds__(64, DEPTH > 3 ? 1 : 2) void project_wave_kernel(mi3
         }
         c0 += na;
     }
+}
+
+// ---- the front launch of a decode batch planned from early routes (route_early.hpp) ----------------------------------
+// One-wave workgroups, in dispatch order:
+//   early blocks (row, 4 experts): lane-parallel logits; the block that completes a row picks the row's experts, clears the
+//     row's assignment words and publishes one tag {epoch, expert} per assignment;
+//   A8 prologue blocks: the A8 image of the input rows; the block that completes a row publishes the row's status word and tag;
+//   side blocks (row, 2 experts): the exact logit chains; the block that completes a row runs the exact softmax / top-k / weights
+//     (the caller's ids, weights and scores), writes the row's work items (the exact experts: what the down launch reads) and
+//     compares its ids with the early ones: where they differ it waits until the assignment's speculative waves have all
+//     finished (their count in the assignment's word), clears the word's non-finite flag and recomputes the assignment's h image
+//     on the exact expert;
+//   projection blocks (assignment, 32-output group): wait for the assignment's tag and the row's tag, then one sweep of the
+//     tagged expert's gate / up rows; each counts itself into its assignment's word when its part of the h image is acknowledged.
+// Blocks are dispatched in index order, so what a waiting block waits for has been dispatched before it (the repair waits for
+// projection blocks, which themselves wait only for blocks in front of them); every wait is bounded, and a wait that runs out (it
+// cannot, short of a lost launch) flags the row as an invalid route: nothing of it is published. Everything that crosses
+// workgroups inside the launch - logits, tags, counts, the A8 images of x and of h, the optional fp32 intermediates - moves by
+// device-scope stores and loads (an assignment that is repaired is written twice, by waves of different XCDs, and the later
+// write has to win at the memory side).
+// A waiting wave polls rarely at first and sleeps between polls: a thousand waves polling one line at full rate saturate the
+// L2 channel that holds it, and every weight stream crossing that channel with it.
+// Two ring slots of 10,240 bytes: eight workgroups share a compute unit.
+constexpr uint32_t kFrontSpinLimit = 1U << 22;
+struct FrontBlocks { uint32_t early, prologue, side; };
+
+// gate + up + SwiGLU + A8 of assignment `at` on expert e, outputs 32 grp .. 32 grp + 31: rows in dense GGUF order stream as
+// contiguous stages (q4k_blocks.hpp), others as one super-block of each row per stage.
+__device__ __forceinline__ void front_project(lds_u8* const (&slots)[2], const mi355_moe_weights& w, const RowsK& r, uint32_t e, uint32_t grp, uint32_t at) {
+    const size_t base = static_cast<size_t>(e) * w.gate_expert_stride + static_cast<size_t>(grp * 32U) * w.gate_row_stride;
+    const uint8_t* gate = w.gate + base;
+    const uint8_t* up = w.up + base;
+    const uint32_t B = w.hidden / 256U;
+    if (w.gate_row_stride == static_cast<uint64_t>(B) * kQ4kBlock && block_lanes_ok(B, 32U)) {
+        const BlockLanes g = block_lanes(B, 32U);
+        const uint32_t half = 32U / g.R;                  // stages of the gate rows, then as many of the up rows
+        float value[1];
+        value[0] = sweep_block_lanes<2>(slots, [&](uint32_t s) { return s < half ? gate + static_cast<size_t>(s) * g.stage_bytes : up + static_cast<size_t>(s - half) * g.stage_bytes; },
+                                        2U * half, g, r.in, r.row_of(at));
+        project_epilogue<1>(value, w, r, grp, [&](uint32_t) { return at; });
+        return;
+    }
+    const size_t stride = w.gate_row_stride;
+    StageSource source;
+    source.init([&](uint32_t q) { return q < 32U ? gate + q * stride : up + (q - 32U) * stride; });
+    project_chunk<1, 2>(slots, source, w, r, grp, 0U, at);
+}
+
+template <int KIND>
+__device__ __forceinline__ void side_router_block(lds_u8* const (&slots)[2], const mi355_moe_weights& w, const RowsK& r,
+                                                  const RouteArgs& a, uint32_t sb, uint32_t assignments, uint32_t epoch) {
+    const uint32_t lane = threadIdx.x & 63U, neb = (a.p.experts + kSideExperts - 1U) / kSideExperts, row = sb / neb;
+    side_chain_block<KIND>(slots[0], slots[1], a, row, (sb % neb) * kSideExperts);
+    uint32_t* lines = a.plan + kPlanLinesAt;
+    if (!arrive_last(&lines[kLinesSide + row * kLineWords], neb)) return;
+    const uint32_t expert = route_select_row(reinterpret_cast<float*>((uint8_t*)slots[0]), a, row);
+    const uint32_t K = a.p.top_k, groups = w.ffn / 32U;
+    if (lane < K) {
+        const uint32_t at = row * K + lane;
+        *reinterpret_cast<uint4*>(a.plan + plan_items_at(w.experts, assignments) + 4U * at) = make_uint4(expert, at, at + 1U, at + 1U);
+        a.plan[plan_order_at(w.experts) + at] = at;
+    }
+    // the early choice of this row and the A8 image of its input (the repair reads it)
+    const unsigned long long* etags = reinterpret_cast<const unsigned long long*>(a.plan + kPlanEtagsAt);
+    unsigned long long tag = 0;
+    uint32_t image = 0;
+    bool there = false;
+    for (uint32_t spins = 0; spins < kFrontSpinLimit && !there; ++spins) {
+        if (lane < K) tag = __hip_atomic_load(&etags[row * K + lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        image = __hip_atomic_load(&lines[kLinesRowTags + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        there = __ballot(lane < K && static_cast<uint32_t>(tag >> 32) != epoch) == 0 && image == epoch;
+        if (!there) __builtin_amdgcn_s_sleep(16);
+    }
+    asm volatile("" ::: "memory");
+    if (!there) {
+        if (lane == 0) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+        return;
+    }
+    uint64_t differ = __ballot(lane < K && static_cast<uint32_t>(tag) != expert);
+    while (differ) {
+        const uint32_t k = static_cast<uint32_t>(__ffsll(static_cast<long long>(differ))) - 1U;
+        differ &= differ - 1ULL;
+        const uint32_t at = row * K + k, e = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(expert), static_cast<int>(k)));
+        uint32_t seen = 0;
+        for (uint32_t spins = 0; spins < kFrontSpinLimit; ++spins) {
+            seen = __hip_atomic_load(&r.awords[at], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffffU;
+            if (seen >= groups) break;
+            __builtin_amdgcn_s_sleep(32);
+        }
+        asm volatile("" ::: "memory");
+        if (seen < groups) {
+            if (lane == 0) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+            continue;
+        }
+        if (lane == 0) __hip_atomic_store(&r.awords[at], groups, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (uint32_t grp = 0; grp < groups; ++grp) front_project(slots, w, r, e, grp, at);
+    }
+}
+
+template <int KIND>
+__global__ __launch_bounds__(64, 2) void layer_front_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, RouteArgs a, FrontBlocks nb) {
+    // exactly 20,480 bytes of LDS: eight workgroups fill a compute unit's 160 KB (one more byte and only seven fit)
+    __shared__ __attribute__((aligned(16))) uint8_t ring0[kSideSlotBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t ring1[kSideSlotBytes];
+    static_assert(kSideSlotBytes == slot_bytes(4), "the projection sweep's slot");
+    lds_u8* const slots[2] = {(lds_u8*)ring0, (lds_u8*)ring1};
+    lds_u8* const (&sl)[2] = slots;
+    uint32_t bid = blockIdx.x;
+    const uint32_t lane = threadIdx.x, K = a.p.top_k;
+    uint32_t* lines = a.plan + kPlanLinesAt;
+    const uint32_t epoch = lines[kLinesEpoch] + 1U;                 // (stored back by the down launch of this call)
+    unsigned long long* etags = reinterpret_cast<unsigned long long*>(a.plan + kPlanEtagsAt);
+    if (bid < nb.early) {
+        const uint32_t neb = (a.p.experts + kEarlyExperts - 1U) / kEarlyExperts, row = bid / neb;
+        early_logits_block<KIND>(a, row, (bid % neb) * kEarlyExperts);
+        if (bid == 0 && lane == 0) {
+            *a.job_status = 0;
+            a.plan[0] = assignments; a.plan[1] = 0; a.plan[2] = 1U; a.plan[4] = assignments;
+        }
+        const bool last = arrive_last(&lines[kLinesEarly + row * kLineWords], neb);
+        if (!last) return;
+        const uint32_t expert = early_select_row(a, row);
+        if (lane < K) __hip_atomic_store(&r.awords[row * K + lane], 0U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        stores_acknowledged();
+        if (lane < K) __hip_atomic_store(&etags[row * K + lane], (static_cast<unsigned long long>(epoch) << 32) | expert, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    bid -= nb.early;
+    if (bid < nb.prologue) {
+        a8_prologue_block<KIND, false, true>(a, bid, lines + kLinesPrologue, lines + kLinesPrologue + 1U, kLineWords, nullptr, lines + kLinesRowTags, epoch);
+        return;
+    }
+    bid -= nb.prologue;
+    if (bid < nb.side) {
+        side_router_block<KIND>(sl, w, r, a, bid, assignments, epoch);
+        return;
+    }
+    bid -= nb.side;
+    // Projection block: assignment `at`, 32-output group `grp`. (Sharing one sweep among the rows that chose an expert was
+    // measured slower: the sweeps that serve several rows finish last, and the others do not speed up.)
+    const uint32_t groups = w.ffn / 32U, at = bid / groups, grp = bid - at * groups, row = at / K;
+    unsigned long long tag = 0;
+    uint32_t image = 0;
+    bool there = false;
+    for (uint32_t spins = 0; spins < kFrontSpinLimit && !there; ++spins) {
+        tag = __hip_atomic_load(&etags[at], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        image = __hip_atomic_load(&lines[kLinesRowTags + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        there = static_cast<uint32_t>(tag >> 32) == epoch && image == epoch;
+        // a block that finds nothing at its first look started with the launch: the tags are microseconds away (one long sleep,
+        // about 3 us); a block dispatched later, into a freed slot, finds them at once
+        if (!there) { if (spins == 0) __builtin_amdgcn_s_sleep(127); else __builtin_amdgcn_s_sleep(8); }
+    }
+    asm volatile("" ::: "memory");
+    if (!there) {
+        if (lane == 0) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+        return;
+    }
+    const uint32_t e = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(tag))));
+    front_project(sl, w, r, e, grp, at);
+    stores_acknowledged();
+    if (lane == 0) __hip_atomic_fetch_add(&r.awords[at], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // down rows: one wavefront per (touched expert, 64 hidden outputs), lane = output row.
@@ -896,12 +1125,12 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, RowsK r
     *reinterpret_cast<vec_t*>(r.output + static_cast<size_t>(row) * r.output_stride + o) = y;
 }
 
+constexpr uint32_t kDownMergeSlots = 8;        // top_k bound: 8 waves x 2 ring slots fill the LDS of a compute unit
 // Down rows and the ordered combine of a decode batch in one launch: a workgroup owns (row, 64 output columns) and has one
 // wave per slot of the row, wave k sweeping the down rows of the expert in slot k (the plan holds one item per assignment,
 // in assignment order); the waves leave their 64 values in LDS and wave 0 folds them exactly as merge_kernel does. Only
 // waves of one workgroup exchange data, so nothing depends on the visibility of another workgroup's stores.
 // Reference: src/cpu/core/routed_expert.cpp:429-447, src/moe_a8_down_contract.cpp:146, include/strix/moe/combine.hpp:36-59.
-constexpr uint32_t kDownMergeSlots = 8;        // top_k bound: 8 waves x 2 ring slots fill the LDS of a compute unit
 __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
     // the two ring slots are separate LDS objects: the compiler then knows that a copy into one never touches the other and lets
     // the reads of the landed slot go ahead while the next stage's copy is in flight (as slots of one array it waited for both)
@@ -911,20 +1140,42 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
     __shared__ uint32_t slot_order[kDownMergeSlots];
     __shared__ float slot_weight[kDownMergeSlots];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, row = blockIdx.y, o = blockIdx.x * 64U + lane;
-    const uint32_t job = *r.job_status;                                        // (requested together with the item: one round trip, not two)
+    uint32_t job;                                                              // (requested together with the item: one round trip, not two)
+    uint32_t word[2] = {0U, 0U};
+    if (r.awords) {
+        if (lane < assignments) word[0] = r.awords[lane];
+        if (lane + 64U < assignments) word[1] = r.awords[lane + 64U];
+    } else job = *r.job_status;
     const uint32_t a = row * w.top_k + wave;
     const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), a);
     const uint32_t e = __builtin_amdgcn_readfirstlane(item.e), begin = __builtin_amdgcn_readfirstlane(item.begin), end = __builtin_amdgcn_readfirstlane(item.end);
+    if (r.awords) {
+        // a batch planned from early routes: the front launch left its non-finite flags per assignment; every workgroup folds them
+        // to the same job word, the first workgroup of a row publishes its row's
+        job = (__ballot(word[0] >> 31) | __ballot(word[1] >> 31)) ? static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION) : 0U;
+        if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) r.plan[kPlanLinesAt + kLinesEpoch] += 1U;      // this call's epoch is spent
+        if (job && blockIdx.x == 0 && wave == 0) {
+            const uint32_t lo = row * w.top_k, hi = lo + w.top_k;
+            const bool mine = (lane >= lo && lane < hi && (word[0] >> 31)) || (lane + 64U >= lo && lane + 64U < hi && (word[1] >> 31));
+            const bool any = __ballot(mine) != 0;
+            if (lane == 0) {
+                if (any) atomicOr(r.status_of(row), r.nonfinite_bit);
+                atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            }
+        }
+    }
     if (job & MI355_STATUS_NONFINITE_PROJECTION) return;                       // the whole job: no down rows, nothing published
     float value = 0.0F;
     if (begin != end) {                                                        // (an invalid route has no item: its row is flagged)
         const uint32_t first = item.first ? item.first - 1U : ordered(r, plan_order_at(w.experts), begin);
         const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
         const size_t stride = w.down_row_stride;
-        StageSource source;
-        source.init([&](uint32_t q) { return rows + q * stride; });
         lds_u8* const slots[2] = {(lds_u8*)ring_even[wave], (lds_u8*)ring_odd[wave]};
         const uint32_t src[1] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(first))}, lane_rows[1] = {first};
+        // (contiguous stages - q4k_blocks.hpp - would be four of 16 rows here instead of three of 64: a wave's time is its number of
+        // stage waits, and that form measured 16.9 us against 15.5)
+        StageSource source;
+        source.init([&](uint32_t q) { return rows + q * stride; });
         const ActRows<1> act(r.h, src, lane_rows);
         float swept[1];
         sweep_rows<1, 2, true>(slots, source, w.ffn / 256U, act, swept);      // narrow codes copies: the slots are slot_bytes(1)
@@ -1645,50 +1896,7 @@ int32_t check_moe(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t 
 // ============================================================================================================ C ABI
 using namespace strix950;
 
-// What the matrix cores of this machine sustain on their own: every wave of a 512-thread workgroup (two waves per SIMD)
-// runs `iterations` x 4 independent v_mfma_f32_32x32x16_f16 on operands that stay in registers. random_operands != 0 fills
-// the operands with pseudo-random halves (weights in the range of the prefill's sc * q operands): the sustained rate then
-// falls with the switching power, which is the ceiling a real product has. A measurement aid for the benchmark, not a product path.
-__global__ __launch_bounds__(512) void probe_mfma_f16_kernel(uint32_t iterations, uint32_t random_operands, float* sink) {
-    floatx16 acc[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[i][j] = 0.0F;
-    half8 a, b;
-    uint32_t state = (threadIdx.x + blockIdx.x * 977U) * 2654435761U;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        state = state * 1664525U + 1013904223U;
-        const float u = static_cast<float>(state >> 8) * (1.0F / 16777216.0F) - 0.5F;
-        state = state * 1664525U + 1013904223U;
-        const float v = static_cast<float>(state >> 8) * (1.0F / 16777216.0F) - 0.5F;
-        a[i] = static_cast<_Float16>(random_operands ? u : 0.001F * static_cast<float>(threadIdx.x));
-        b[i] = static_cast<_Float16>(random_operands ? 945.0F * v : 0.5F);
-    }
-    for (uint32_t it = 0; it < iterations; ++it) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
-        asm volatile("" : "+v"(a), "+v"(b));                  // the operands stay what they are; the loop is not folded
-    }
-    float total = 0.0F;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) total += acc[i][j];
-    sink[blockIdx.x * 512U + threadIdx.x] = total;
-}
-
 extern "C" {
-
-int32_t mi355_probe_mfma_f16(uint32_t iterations, uint32_t random_operands, float* sink, uint64_t sink_floats, uint64_t* flops, mi355_stream stream) {
-    const uint32_t blocks = compute_units();
-    STRIX_REQUIRE(sink && flops && sink_floats >= 512ULL * blocks && iterations > 0, "mfma probe: sink of 512 floats per compute unit, iterations > 0");
-    probe_mfma_f16_kernel<<<blocks, 512, 0, hs(stream)>>>(iterations, random_operands, sink);
-    STRIX_LAUNCHED("mfma probe");
-    *flops = 2ULL * 32U * 32U * 16U * 4U * iterations * 8ULL * blocks;
-    return MI355_OK;
-}
 
 const char* mi355_last_error(void) { return g_error.c_str(); }
 const char* mi355_version(void) { return "mi355-strix 0.1 (gfx950)"; }
@@ -1948,6 +2156,27 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, u
 }  // extern "C"
 
 namespace {
+// mi355_moe_enqueue by halves: front = prologue, plan, gate / up; back = down rows, combine.
+int32_t enqueue_staged(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream, bool do_front, bool do_back) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
+    if (do_front) {
+        STRIX_REQUIRE(r->input && r->input_kind <= MI355_INPUT_BF16, "moe: input view invalid");
+        if (const int32_t rc = mi355_moe_enqueue_prologue(w, r, rows, stream)) return rc;
+        if (!(dense_pairs_ok(wv, rows) && r->gate_out && r->up_out))
+            if (const int32_t rc = mi355_moe_enqueue_csr(w, r, rows, stream)) return rc;
+        if (const int32_t rc = mi355_moe_enqueue_project(w, r, rows, stream)) return rc;
+    }
+    if (!do_back) return MI355_OK;
+    RowsK k = rows_k(*r, wv);
+    if (wv.experts == 1U && wv.top_k == 1U && rows <= 65535U) k.top1_form = form + 1U;
+    const bool published = launch_down(wv, k, rows, item_bound(wv, rows), hs(stream));
+    STRIX_LAUNCHED("moe down");
+    if (published) return MI355_OK;
+    return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+}
+
 // RMSNorm of rows of any input kind into fp32 rows (the staged form of the fused norm): rmsnorm_f32_kernel's order.
 template <int KIND>
 __global__ __launch_bounds__(64) void rmsnorm_rows_kernel(const uint8_t* x, uint64_t x_stride, const float* w, uint32_t n, float eps, float* y) {
@@ -1962,9 +2191,14 @@ __global__ __launch_bounds__(64) void rmsnorm_rows_kernel(const uint8_t* x, uint
 }
 
 struct LayerNorm { bool on; const float* weight; float eps; float* normed; };
+std::atomic<uint32_t> g_early_perturb{0};
 
+// phase: 0 = the whole layer; 1 = its front half (router, A8 prologue, plan, gate / up); 2 = its back half (down rows, combine) on
+// what a front call with the same arguments left in the row views.
+enum { kLayerWhole = 0, kLayerFront = 1, kLayerBack = 2 };
 int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores, const LayerNorm& norm,
-                      const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+                      const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream, uint32_t phase = kLayerWhole) {
+    const bool do_front = phase != kLayerBack, do_back = phase != kLayerFront;
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
@@ -1979,16 +2213,18 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     hipStream_t st = hs(stream);
     if (rows > kFusedMaxRows || plan_split(wv, rows) != 1U) {      // large batches, and decode batches over large experts (shared sweeps): router, then the staged prologue / plan
         mi355_moe_rows staged = *r;
-        if (norm.on) {
+        if (norm.on && do_front) {
             const uint8_t* x = static_cast<const uint8_t*>(r->input);
             if (r->input_kind == MI355_INPUT_F32) rmsnorm_rows_kernel<0><<<rows, 64, 0, st>>>(x, r->input_stride, norm.weight, wv.hidden, norm.eps, norm.normed);
             else if (r->input_kind == MI355_INPUT_F16) rmsnorm_rows_kernel<1><<<rows, 64, 0, st>>>(x, r->input_stride, norm.weight, wv.hidden, norm.eps, norm.normed);
             else rmsnorm_rows_kernel<2><<<rows, 64, 0, st>>>(x, r->input_stride, norm.weight, wv.hidden, norm.eps, norm.normed);
             STRIX_LAUNCHED("moe layer norm");
-            staged.input = norm.normed; staged.input_kind = MI355_INPUT_F32; staged.input_stride = 4ULL * wv.hidden;
         }
-        if (const int32_t rc = mi355_moe_route(p, staged.input, staged.input_kind, rows, wv.hidden, staged.input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
-        return mi355_moe_enqueue(w, &staged, rows, form, stream);
+        if (norm.on) { staged.input = norm.normed; staged.input_kind = MI355_INPUT_F32; staged.input_stride = 4ULL * wv.hidden; }
+        if (do_front)
+            if (const int32_t rc = mi355_moe_route(p, staged.input, staged.input_kind, rows, wv.hidden, staged.input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
+        if (phase == kLayerWhole) return mi355_moe_enqueue(w, &staged, rows, form, stream);
+        return enqueue_staged(w, &staged, rows, form, stream, do_front, do_back);
     }
     RouteArgs a{};
     a.p = *p; a.x = static_cast<const uint8_t*>(r->input); a.kind = r->input_kind; a.x_stride = r->input_stride; a.rows = rows; a.hidden = wv.hidden;
@@ -1996,18 +2232,52 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     a.codes = r->codes; a.deltas = r->deltas; a.sums = r->sums; a.status = r->status; a.job_status = r->job_status; a.plan = r->plan;
     a.quant_blocks = (rows * (wv.hidden / 32U) + 7U) / 8U;
     a.norm_on = norm.on ? 1U : 0U; a.norm_w = norm.weight; a.norm_eps = norm.eps; a.normed = norm.normed;
-    launch_route_logits(a, st);
-    STRIX_LAUNCHED("moe layer router");
-    // the fused router planned one item per routed assignment (and one per four rows of an always-on expert)
     const uint32_t items = rows * wv.top_k;
+    // Early routes (route_early.hpp): the expert choice from lane-parallel logits in a short first launch, the exact router beside
+    // the projection, down rows + combine on the verified work items. Taken where the 64-row projection sweep and the down +
+    // combine launch serve the batch.
+    if (!norm.on && p->shared_experts == 0 && p->logits_order == MI355_LOGITS_FMA_ASCENDING && wv.gate_type == MI355_TYPE_Q4_K &&
+        wv.down_type == MI355_TYPE_Q4_K && !quad_sweep(wv, rows) && wv.experts > 1U && wv.top_k <= kDownMergeSlots && items <= kEarlyMaxAssignments &&
+        wv.hidden <= kSideMaxHidden && wv.hidden % 64U == 0 && (wv.hidden / 64U) * rows <= compute_units() && wv.experts <= wv.top_k * wv.hidden) {
+        a.awords = r->plan + kPlanAwordsAt;
+        a.early_perturb = g_early_perturb.load(std::memory_order_relaxed);
+        // the early logits of row i live in the row's (still unused) unweighted-output block: the exact logits own `scores`
+        a.early_logits = r->rawdots; a.early_stride = wv.top_k * wv.hidden;
+        RowsK k = rows_k(*r, wv);
+        k.awords = a.awords;
+        RowsK front = k;
+        front.plan = nullptr;              // (the front launch names its assignments itself: the work items are written inside it)
+        const FrontBlocks nb{rows * ((p->experts + kEarlyExperts - 1U) / kEarlyExperts), a.quant_blocks, rows * ((p->experts + kSideExperts - 1U) / kSideExperts)};
+        const uint32_t blocks = nb.early + nb.prologue + nb.side + items * (wv.ffn / 32U);
+        if (do_front) {
+            if (a.kind == MI355_INPUT_F32) layer_front_kernel<0><<<blocks, 64, 0, st>>>(wv, front, items, a, nb);
+            else if (a.kind == MI355_INPUT_F16) layer_front_kernel<1><<<blocks, 64, 0, st>>>(wv, front, items, a, nb);
+            else layer_front_kernel<2><<<blocks, 64, 0, st>>>(wv, front, items, a, nb);
+            STRIX_LAUNCHED("moe layer early routes + gate / up");
+        }
+        if (do_back) {
+            down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, st>>>(wv, k, items, form);
+            STRIX_LAUNCHED("moe layer experts + combine");
+        }
+        return MI355_OK;
+    }
+    if (do_front) {
+        launch_route_logits(a, st);
+        STRIX_LAUNCHED("moe layer router");
+    }
+    // the fused router planned one item per routed assignment (and one per four rows of an always-on expert)
     if (p->shared_experts) {       // items of several rows: the 64-row sweeps
-        launch_project(wv, rows_k(*r, wv), rows, items, st, true);
-        STRIX_LAUNCHED("moe layer gate / up");
+        if (do_front) {
+            launch_project(wv, rows_k(*r, wv), rows, items, st, true);
+            STRIX_LAUNCHED("moe layer gate / up");
+        }
+        if (!do_back) return MI355_OK;
         launch_down(wv, rows_k(*r, wv), rows, items, st, true);
         STRIX_LAUNCHED("moe layer experts");
         return mi355_moe_enqueue_merge(w, r, rows, form, stream);
     }
-    launch_project(wv, rows_k(*r, wv), rows, items, st);
+    if (do_front) launch_project(wv, rows_k(*r, wv), rows, items, st);
+    if (!do_back) return MI355_OK;
     // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
     // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
     // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
@@ -2048,9 +2318,21 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
 
 extern "C" {
 
+void mi355_debug_early_route_perturb(uint32_t amount) { g_early_perturb.store(amount, std::memory_order_relaxed); }
+
 int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
                                 const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
     return enqueue_layer(p, router_weight, logit_bias, scores, LayerNorm{false, nullptr, 0.0F, nullptr}, w, r, rows, form, stream);
+}
+
+int32_t mi355_moe_enqueue_layer_front(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
+                                      const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    return enqueue_layer(p, router_weight, logit_bias, scores, LayerNorm{false, nullptr, 0.0F, nullptr}, w, r, rows, form, stream, kLayerFront);
+}
+
+int32_t mi355_moe_enqueue_layer_back(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
+                                     const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    return enqueue_layer(p, router_weight, logit_bias, scores, LayerNorm{false, nullptr, 0.0F, nullptr}, w, r, rows, form, stream, kLayerBack);
 }
 
 int32_t mi355_moe_enqueue_layer_normed(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,

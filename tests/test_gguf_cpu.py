@@ -1,6 +1,7 @@
-"""The GGUF v3 reader and the MoE layer map on files written by tests/golden/make_tiny_gguf.py (an independent writer following
-the published container layout), and the reader's refusals: the rules of the reference reader (src/gguf_reader.cpp:22-90,
-130-260, 296-360). Host code only."""
+"""The GGUF v3 reader and the MoE layer map: the byte fixtures the reference's own reader tests build (tests/core_tests.cpp:56-126
+with the outcomes of :289-370, tests/gguf_pack_writer_test.cpp:19-31), files written by tests/golden/make_tiny_gguf.py (an
+independent writer following the published container layout), and the reader's refusals: the rules of the reference reader
+(src/gguf_reader.cpp:22-90, 130-260, 296-360). Host code only."""
 import os
 import struct
 import sys
@@ -130,3 +131,99 @@ def test_layer_map_refusals(pkg, tmp_path):
     layer_refused(wrong_router, "router must be an F32")
     down_f32 = [(n, d, (0 if "down_exps" in n else t), (bytes(256 * 256 * 2 * 4) if "down_exps" in n else b)) for n, d, t, b in tensors]
     layer_refused(down_f32, "down experts must be")
+
+
+# ---- the reference's own byte fixtures -------------------------------------------------------------------------------
+def _le(fmt, v):
+    return struct.pack("<" + fmt, v)
+
+
+def _s(text):
+    return _le("Q", len(text)) + text.encode()
+
+
+def ref_valid_gguf(tensor_offset=0, tensor_type=1):
+    """valid_gguf of tests/core_tests.cpp:56-82: two metadata values, one tensor [16, 32] of `tensor_type`, 1024 data bytes."""
+    b = b"GGUF" + _le("I", 3) + _le("Q", 1) + _le("Q", 2)
+    b += _s("general.architecture") + _le("I", 8) + _s("qwen4exp")
+    b += _s("general.alignment") + _le("I", 4) + _le("I", 32)
+    b += _s("blk.0.weight") + _le("I", 2) + _le("Q", 16) + _le("Q", 32) + _le("I", tensor_type) + _le("Q", tensor_offset)
+    b += bytes(-len(b) % 32)
+    return b + bytes(1024)
+
+
+def ref_array_gguf():
+    """array_gguf of tests/core_tests.cpp:84-99: one metadata array of three uint32."""
+    b = b"GGUF" + _le("I", 3) + _le("Q", 0) + _le("Q", 1)
+    b += _s("test.values") + _le("I", 9) + _le("I", 4) + _le("Q", 3) + _le("I", 10) + _le("I", 20) + _le("I", 30)
+    return b + bytes(-len(b) % 32)
+
+
+def ref_two_tensor_gguf(second_offset):
+    """two_tensor_gguf of tests/core_tests.cpp:101-121: two F16 tensors [16, 32] (1024 bytes each), 2048 data bytes."""
+    b = b"GGUF" + _le("I", 3) + _le("Q", 2) + _le("Q", 0)
+    for name, offset in (("first.weight", 0), ("second.weight", second_offset)):
+        b += _s(name) + _le("I", 2) + _le("Q", 16) + _le("Q", 32) + _le("I", 1) + _le("Q", offset)
+    b += bytes(-len(b) % 32)
+    return b + bytes(2048)
+
+
+def ref_pack_writer_source():
+    """The source file of tests/gguf_pack_writer_test.cpp:19-31: a string and a uint32, an F32 [4] and a BF16 [128, 16] tensor."""
+    b = b"GGUF" + _le("I", 3) + _le("Q", 2) + _le("Q", 2)
+    b += _s("general.architecture") + _le("I", 8) + _s("qwen35")
+    b += _s("qwen35.block_count") + _le("I", 4) + _le("I", 7)
+    b += _s("norm.weight") + _le("I", 1) + _le("Q", 4) + _le("I", 0) + _le("Q", 0)
+    b += _s("w.weight") + _le("I", 2) + _le("Q", 128) + _le("Q", 16) + _le("I", 30) + _le("Q", 32)
+    b += bytes(-len(b) % 32)
+    return b + b"n" * 16 + bytes(16) + b"w" * 4096
+
+
+def test_reference_reader_fixtures(pkg, tmp_path):
+    """The reference's parse results and refusals on its own fixtures (tests/core_tests.cpp:289-370). Not replayed: the two cases
+    that pass a Limits object (max_string_bytes = 4, max_total_array_elements = 2) - this reader's limits are fixed."""
+    path = str(tmp_path / "ref.gguf")
+
+    def opened(raw):
+        open(path, "wb").write(raw)
+        return pkg.GgufFile(path)
+
+    def refuses(raw, reason):
+        open(path, "wb").write(raw)
+        refused(pkg, path, reason)
+
+    raw = ref_valid_gguf()
+    g = opened(raw)
+    assert g.alignment == 32 and len(g.tensors()) == 1                                    # "GGUF alignment metadata is applied", "tensor directory parses"
+    assert int(pkg.lib().mi355_gguf_metadata_count(g.handle)) == 2                        # "metadata count is preserved"
+    t = g.tensors()[0]
+    assert t["offset"] == g.data_offset and g.data_offset % 32 == 0                       # "relative tensor offset resolves from data section"
+    assert t["bytes"] == 1024 and t["offset"] + t["bytes"] == len(raw)                    # "F16 tensor range is computed exactly"
+    assert t["name"] == "blk.0.weight" and t["dims"] == [16, 32] and t["type"] == 1
+    assert g.metadata("general.architecture") == "qwen4exp"                               # "architecture metadata is available"
+    g.close()
+    refuses(b"B" + raw[1:], "invalid GGUF magic")                                         # "rejects invalid magic"
+    refuses(ref_valid_gguf(1), "offset is not aligned")                                   # "rejects unaligned tensor offsets"
+    refuses(ref_valid_gguf(0, 31), "unsupported or removed GGML tensor type")             # "rejects removed tensor types"
+    refuses(ref_valid_gguf(0, 2), "not divisible by its quantization block")              # "rows not divisible by quantization block size"
+    refuses(raw[:-1], "exceeds file size")                                                # "tensor ranges extending beyond the file"
+    g = opened(ref_two_tensor_gguf(1024))
+    first, second = g.tensors()
+    assert second["offset"] == first["offset"] + first["bytes"]                           # "permits adjacent non-overlapping tensor ranges"
+    g.close()
+    refuses(ref_two_tensor_gguf(0), "overlap")                                            # "rejects overlapping tensor data ranges"
+    flag = b"GGUF" + _le("I", 3) + _le("Q", 0) + _le("Q", 1) + _s("test.flag") + _le("I", 7) + _le("B", 2)
+    refuses(flag + bytes(-len(flag) % 32), "boolean must be zero or one")                 # "rejects non-canonical booleans"
+    g = opened(ref_array_gguf())
+    assert g.metadata("test.values") == 3 and len(g.tensors()) == 0                       # "array summary parses without retaining its payload"
+    g.close()
+    # the pack writer's source file: 32-byte default alignment, an F32 and a BF16 tensor with a gap between them
+    raw = ref_pack_writer_source()
+    g = opened(raw)
+    norm, wt = g.tensors()
+    assert g.alignment == 32 and g.metadata("qwen35.block_count") == 7 and g.metadata("general.architecture") == "qwen35"
+    assert (norm["name"], norm["dims"], norm["type"], norm["bytes"], norm["offset"]) == ("norm.weight", [4], 0, 16, g.data_offset)
+    assert (wt["name"], wt["dims"], wt["type"], wt["bytes"], wt["offset"]) == ("w.weight", [128, 16], 30, 4096, g.data_offset + 32)
+    assert wt["offset"] + wt["bytes"] == len(raw)
+    assert bytes(g.read(pkg.GgufTensor(b"norm.weight", 1, (pkg.C.c_uint64 * 4)(4), 0, norm["offset"], 16)).numpy()) == b"n" * 16
+    g.close()

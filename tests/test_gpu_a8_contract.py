@@ -268,6 +268,47 @@ def test_rawdots_with_slot_merge_tail(strix, down_type, out_dtype, bf16_commit):
     assert np.array_equal(bits(p.rawdots.cpu().numpy()[0]), bits(raw))
 
 
+@pytest.mark.parametrize("down_type", [orc.Q4_K, orc.Q8_0, orc.Q6_K])
+def test_rawdots_and_slot_merge_flag_an_invalid_route_on_their_own(strix, down_type):
+    """A route out of range reaches the down rows without the producer that checks the routes (the routes are overwritten after
+    a valid producer run and the status word is clear): mi355_a8_enqueue_down_rawdots sets the invalid-route bit and the summary
+    word itself, as the reference's down_rawdots_rows does (src/hip_moe_q4k_a8_probe.hip:743); with the slot-merge tail nothing
+    is accumulated or committed and the first-error record is set - also when the status word is cleared between the two."""
+    H, I, E, K = 1024, 256 if down_type != orc.Q8_0 else 384, 8, 4
+    rng = np.random.default_rng(90 + down_type)
+    gate = orc.quantize_rows(orc.Q4_K, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32))
+    down = make_down(rng, down_type, E, H, I)
+    p = strix.A8Decode(H, I, E, K, dev(gate), dev(gate), dev(down), down_type=down_type)
+    p.intermediates.copy_(torch.from_numpy(rng.standard_normal((1, K, 2, I)).astype(np.float32)))
+    p.routes.copy_(torch.tensor([[1, 2, 5, 7]], dtype=torch.int32))
+    p.enqueue_down_activation_quantize()
+    p.enqueue_down_rawdots()
+    torch.cuda.synchronize()
+    assert int(p.status.item()) == 0 and int(p.aggregate.item()) == 0
+    good = p.rawdots.clone()
+    p.routes.copy_(torch.tensor([[1, E + 3, 5, 7]], dtype=torch.int32))
+    p.rawdots.fill_(-7.0)
+    p.enqueue_down_rawdots()
+    torch.cuda.synchronize()
+    assert int(p.status.item()) == 1 and int(p.aggregate.item()) == 16
+    raw = p.rawdots.cpu()
+    assert torch.all(raw[0, 1] == -7.0) and torch.equal(raw[0, 0], good[0, 0].cpu()) and torch.equal(raw[0, 3], good[0, 3].cpu())
+    # the merge tail: a cleared status word, the invalid route still there
+    for clear_between in (False, True):
+        p.status.zero_()
+        p.aggregate.zero_()
+        acc, out = torch.full((H,), 5.0, device="cuda"), torch.full((H,), -3.0, device="cuda")
+        record = torch.zeros(2, dtype=torch.int32, device="cuda")
+        w = dev(np.full(K, 0.25, np.float32))
+        if clear_between:
+            p.enqueue_down_rawdots()
+            p.status.zero_()
+        p.enqueue_down_rawdots_merge(w, acc, out, record, domain=6, bf16_commit=False)
+        torch.cuda.synchronize()
+        assert int(p.status.item()) & 1 and record.tolist() == [6, int(p.status.item())]
+        assert torch.all(out == -3.0) and torch.all(acc == 5.0)                  # nothing accumulated, nothing committed
+
+
 def test_slot_merge_commit_threshold_and_first_error_record(strix):
     """A merged value that is finite in fp32 but rounds to bf16 infinity (bits >= 0x7f7f8000) fails a bf16 commit and passes an
     fp32 one; a failed step stores no output and the record keeps the FIRST failure of the stream

@@ -133,16 +133,3 @@ def test_union_refuses_a_repeated_expert_and_an_id_out_of_range(strix):
     p.enqueue_probe_union()
     torch.cuda.synchronize()
     assert int(p.status.item()) == 0 and p.plan.cpu().numpy()[:4].view(np.uint32)[0] == 4
-
-
-def test_matrix_core_probe_runs_and_reports_its_flops(strix):
-    """The benchmark's measurement aid (mi355_probe_mfma_f16): 256 compute units x 8 waves x iterations x 4 MFMAs of 32 x 32 x 16."""
-    sink = torch.zeros(512 * 1024, dtype=torch.float32, device="cuda")
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    for rnd in (False, True):
-        flops = strix.probe_mfma_f16(3, rnd, sink)
-        torch.cuda.synchronize()
-        assert flops == 2 * 32 * 32 * 16 * 4 * 3 * 8 * cus
-        assert bool(torch.isfinite(sink[: 512 * cus]).all())
-    with pytest.raises(strix.StrixError):
-        strix.probe_mfma_f16(3, False, sink[:100])

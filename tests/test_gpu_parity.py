@@ -14,6 +14,10 @@ pytestmark = pytest.mark.gpu
 TOL_F32, TOL_F16 = 1e-3, 2e-3
 
 
+# plan words: header [0, 16), ticket words [16, 272), the words of the early-routes decode layer [272, 2240), then offsets / touched /
+# order / items
+PLAN_OFFSETS_AT = 2240
+
 def bits(a):
     return np.ascontiguousarray(a, np.float32).view(np.uint32)
 
@@ -663,7 +667,7 @@ def test_expert_plan_words(strix, E, K, T):
     x = dev(rng.standard_normal((T, H)).astype(np.float16))
     w = dev(np.ones((T, K), np.float32))
     layer.plan.fill_(-1)
-    layer.plan[16:272] = 0
+    layer.plan[16:PLAN_OFFSETS_AT] = 0               # (the words that launches expect zero)
     layer.stage("csr", x, dev(ids), w)
     plan = layer.plan.cpu().numpy().view(np.uint32)
     flat = ids.reshape(-1).astype(np.int64)
@@ -675,7 +679,7 @@ def test_expert_plan_words(strix, E, K, T):
     counts = np.bincount(flat[valid], minlength=E)
     offsets = np.concatenate([[0], np.cumsum(counts)])
     pad4 = lambda v: (v + 3) & ~3
-    offsets_at = 272
+    offsets_at = PLAN_OFFSETS_AT
     touched_at = offsets_at + pad4(E + 1)
     order_at = touched_at + pad4(E)
     items_at = order_at + pad4(A)
@@ -797,6 +801,115 @@ def test_invalid_route_and_nonfinite_projection_fail_closed(strix):
     st = layer.status[:T].cpu().numpy()
     assert st[1] & strix.STATUS_NONFINITE_PROJECTION and st[0] == 0
     assert bool((layer.rawdots == -3.0).all())
+
+
+@pytest.mark.parametrize("E,H,I,K,T", [(128, 2048, 768, 8, 8), (128, 2048, 768, 8, 2), (12, 2048, 2048, 4, 16), (160, 1536, 512, 8, 16), (6, 768, 512, 2, 40)])
+def test_layer_entry_halves_equal_the_whole_call(strix, E, H, I, K, T):
+    """mi355_moe_enqueue_layer_front followed by mi355_moe_enqueue_layer_back is mi355_moe_enqueue_layer, bit for bit, on every
+    path of the layer entry: early routes, the fused router with either sweep, shared sweeps over large experts, large batches."""
+    rng = np.random.default_rng(E * T)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
+    wr = dev((rng.standard_normal((E, H)) * 0.02).astype(np.float32))
+    x = dev(rng.standard_normal((T, H)).astype(np.float16))
+    whole = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T)
+    halves = strix.MoeLayer(H, I, E, K, whole.gate, whole.up, whole.down, T)
+    y, ids, wts, scores = whole.run_layer(x, wr)
+    halves.output.fill_(-3.0)
+    halves.run_layer(x, wr, half="front")
+    torch.cuda.synchronize()
+    assert bool((halves.output == -3.0).all())                                  # nothing is published by the front half
+    y2, ids2, wts2, scores2 = halves.run_layer(x, wr, half="back")
+    assert torch.equal(y2, y) and torch.equal(ids2, ids) and torch.equal(wts2, wts) and torch.equal(scores2, scores)
+    assert torch.equal(halves.rawdots[:T], whole.rawdots[:T]) and torch.equal(halves.status[:T], whole.status[:T])
+
+
+def early_choice(x, wr, K, amount):
+    """What the early launch of the layer entry picks: plain dot products, displaced by the test knob (route_early.hpp)."""
+    z = x.astype(np.float64) @ wr.astype(np.float64).T
+    e = np.arange(wr.shape[0], dtype=np.uint64)
+    z = z + amount * 1e-3 * ((((e * 2654435761) & 0xffffffff) >> 28).astype(np.float64) - 8.0)
+    return np.argsort(-z, axis=1, kind="stable")[:, :K].astype(np.uint32)
+
+
+@pytest.mark.parametrize("E,H,I,K,T,amount", [(128, 2048, 768, 8, 8, 0), (128, 2048, 768, 8, 8, 40), (128, 2048, 768, 8, 7, 400),
+                                               (32, 1024, 512, 4, 16, 25), (24, 512, 256, 8, 16, 300)])
+def test_layer_entry_early_routes_are_verified_and_repaired(strix, E, H, I, K, T, amount):
+    """Decode batches on the 64-row sweeps pick their experts from lane-parallel logits first and run the exact router beside
+    the projection. With the early logits displaced by the test knob the two choices differ in many slots: ids, weights, the
+    A8 image of h, rawdots and the output must still be the exact router's, bit for bit, the work items must name the exact
+    experts, and a second call on the same workspace without the displacement must give the same bits."""
+    rng = np.random.default_rng(E + T + amount)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, intermediates=True)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    differ = int((early_choice(x, wr, K, amount) != ids_ref).sum())
+    assert (differ == 0) if amount == 0 else (differ >= 3)
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    ref = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref)
+    want = orc.combine(0, w_ref, ids_ref, ref.rawdots)
+    strix.lib().mi355_debug_early_route_perturb(amount)
+    try:
+        y, ids, wts, _ = layer.run_layer(dev(x), dev(wr))
+        y = y.clone()
+        torch.cuda.synchronize()
+    finally:
+        strix.lib().mi355_debug_early_route_perturb(0)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    pad4 = lambda v: (v + 3) & ~3
+    items_at = PLAN_OFFSETS_AT + pad4(E + 1) + pad4(E) + pad4(T * K)          # offsets, touched, order
+    items = layer.plan[items_at: items_at + 4 * T * K].cpu().numpy().astype(np.uint32).reshape(-1, 4)
+    assert np.array_equal(items[:, 0], ids_ref.reshape(-1))                      # the work items name the exact experts
+    assert bool((layer.plan[16:272] == 0).all()) and int(layer.job_status[0]) == 0
+    check_layer_stages(strix, layer, y.cpu().numpy(), ref, want, (c, d, s), ids_ref, w_ref, (gate, up, down, I, {}), H, K, T, 0, 0, TOL_F16)
+    again, ids2, wts2, _ = layer.run_layer(dev(x), dev(wr))
+    assert torch.equal(again, y) and torch.equal(ids2, ids) and torch.equal(wts2, wts)
+
+
+@pytest.mark.parametrize("amount", [0, 500])
+def test_layer_entry_early_routes_nonfinite_flags_follow_the_exact_choice(strix, amount):
+    """One expert carries a non-finite block scale. The displaced early choice sends rows to it that the exact router does not
+    (and the other way round): only the rows whose EXACT experts include it may be flagged, the job word carries the
+    non-finite-projection bit exactly when there is such a row, and then nothing is published."""
+    E, H, I, K, T = 32, 1024, 512, 4, 16
+    rng = np.random.default_rng(5 + amount)
+    gate, up, down = make_layer(rng, H, I, E)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    shift = ((((np.arange(E, dtype=np.uint64) * 2654435761) & 0xffffffff) >> 28).astype(np.int64) - 8)
+    counts = np.bincount(ids_ref.reshape(-1), minlength=E)
+    # an expert that the displacement favours and that some, not all, rows choose exactly; and one that no row chooses exactly
+    some = [e for e in range(E) if shift[e] >= 5 and 0 < np.any(ids_ref == e, axis=1).sum() < T]
+    none = [e for e in range(E) if shift[e] >= 5 and counts[e] == 0]
+    for bad, expect_rows in ((some[0], True), (none[0] if none else None, False)):
+        if bad is None:
+            continue
+        g2 = gate.copy()
+        g2.reshape(E, I, -1)[bad, 3, 0:2] = np.frombuffer(np.float16(np.inf).tobytes(), np.uint8)
+        layer = strix.MoeLayer(H, I, E, K, dev(g2), dev(up), dev(down), T)
+        layer.output.fill_(-7.0)
+        if amount:
+            assert np.any(early_choice(x, wr, K, amount) == bad)                  # the early launch does send rows to it
+        strix.lib().mi355_debug_early_route_perturb(amount)
+        try:
+            y, ids, wts, _ = layer.run_layer(dev(x), dev(wr))
+            torch.cuda.synchronize()
+        finally:
+            strix.lib().mi355_debug_early_route_perturb(0)
+        assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref)
+        hit = np.any(ids_ref == bad, axis=1)
+        st = layer.status[:T].cpu().numpy()
+        assert hit.any() == expect_rows
+        assert np.all((st[hit] & strix.STATUS_NONFINITE_PROJECTION) != 0) and np.all(st[~hit] == 0)
+        assert bool(int(layer.job_status[0]) & strix.STATUS_NONFINITE_PROJECTION) == expect_rows
+        if expect_rows:
+            assert bool((y[:T] == -7.0).all())
+        else:
+            c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+            ref = orc.routed_experts(H, I, K, g2, up, down, orc.Q4_K, c, d, s, ids_ref)
+            assert np.array_equal(bits(layer.rawdots[:T].cpu().numpy()), bits(ref.rawdots)) or rel_err(y.cpu().numpy(), orc.combine(0, w_ref, ids_ref, ref.rawdots))[0] < TOL_F16
 
 
 @pytest.mark.parametrize("T", [1, 2, 8, 16])
