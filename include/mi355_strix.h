@@ -49,6 +49,7 @@ enum { MI355_TYPE_Q5_1 = 7, MI355_TYPE_Q8_0 = 8, MI355_TYPE_Q4_K = 12, MI355_TYP
 enum { MI355_INPUT_F32 = 0, MI355_INPUT_F16 = 1, MI355_INPUT_BF16 = 2 };
 enum { MI355_LOGITS_FMA_ASCENDING = 0, MI355_LOGITS_LANE32_BUTTERFLY = 1 };
 enum { MI355_COMBINE_FMA_SLOT_ORDER = 0, MI355_COMBINE_MULADD_ASCENDING_EXPERT = 1,
+       MI355_COMBINE_BF16_STEPS = 3,   /* mi355_moe_enqueue_combine only: every step of the reduction rounded to bfloat16 */
        MI355_COMBINE_NONE = 2 };   /* mi355_moe_enqueue_prefill_f16 only: stop after the down rows. rawdots then holds the unweighted
                                       per-slot outputs; for a top-1 layer of weight 1 (an always-on shared expert) rawdots[row] is
                                       the layer's output - fma(1, x, 0) = x - and can be the `base` of the routed call, which saves
@@ -211,6 +212,18 @@ int32_t mi355_moe_enqueue_merge(const mi355_moe_weights*, const mi355_moe_rows*,
 int32_t mi355_moe_enqueue(const mi355_moe_weights*, const mi355_moe_rows*, uint32_t rows, uint32_t combine_form,
                           mi355_stream);
 
+/* The combine as an operator of its own (strix::moe_core::enqueue_combine / enqueue_combine_rounded_eo,
+ * src/moe_core/route_wave_kernel.hpp:98-160; host restatement strix::moe::combine_ref, include/strix/moe/combine.hpp:36-59).
+ * eo [rows][top_k][width], w [rows][top_k], base [rows][width], y [rows][width], all dense fp32 on the device.
+ *   MI355_COMBINE_FMA_SLOT_ORDER: acc = fma(w_k, e_k, acc) in slot order, y = acc + base; w and base are required.
+ *   MI355_COMBINE_BF16_STEPS:     acc = bf16(acc + term_k), term_k = w ? bf16(e_k * w_k) : e_k (w NULL: unit weights);
+ *                                 y = base ? bf16(acc + base) : acc. round_eo != 0 reads every e_k as bf16(e_k), the value a
+ *                                 separate rounding launch over eo would have stored (bf16-steps form only).
+ * bf16() rounds to nearest even into the upper 16 bits and passes a NaN through unchanged. No status words: like the
+ * reference operator this one only computes. rows == 0 is a no-op. */
+int32_t mi355_moe_enqueue_combine(uint32_t form, uint32_t rows, uint32_t top_k, uint32_t width, const float* w, const float* eo,
+                                  const float* base, float* y, uint32_t round_eo, mi355_stream);
+
 /* The same layer with its router in front (the reference's per-layer walk moe_route -> moe_experts -> moe_combine,
  * include/strix/execution_plan.hpp:22-25): rows->routes and rows->route_weights are OUTPUTS of this call (the selected ids
  * and weights), scores is a [rows][experts] workspace and output. For rows <= 16 the router, the A8 prologue and the expert
@@ -240,7 +253,7 @@ int32_t mi355_moe_enqueue_layer_back(const mi355_route_policy* policy, const flo
                                      uint32_t combine_form, mi355_stream);
 
 /* Test aid of the decode layer (no counterpart in the reference). A decode batch on the 64-row sweeps picks its experts from
- * lane-parallel logits in a short first launch and runs the reference's logit chain, softmax and selection beside the
+ * lane-parallel logits and runs the reference's logit chain, softmax and selection beside the
  * projection; where the two choices differ the assignment is recomputed on the exact expert before the down rows. The results
  * are the exact router's either way. amount != 0 displaces the early logits (by amount * 1e-3 * a per-expert integer in
  * -8..7) so that a test can make the choices differ; 0 (the default) restores them. Process-wide; not for production use. */
@@ -331,8 +344,22 @@ typedef struct mi355_a8_bindings { mi355_device_bytes input, gate, up, routes, c
 int32_t mi355_a8_validate(const mi355_a8_request*, const mi355_a8_bindings*);
 /* enqueue_probe (include/strix/hip_moe_q4k_a8_probe.hpp:12): route check, A8 image of the input row(s), gate and up rows of
  * the chosen experts: output[((row * top_k + slot) * 2 + which) * shape.rows + i] fp32 (which 0 = gate, 1 = up), bitwise
- * the reference row contract (src/moe_q4k_a8_contract.cpp:126-140). */
+ * the reference row contract (src/moe_q4k_a8_contract.cpp:126-140). On a flagged step (status != 0 after the prologue) the
+ * projection stores nothing: `output` keeps its previous contents, as in the reference (src/hip_moe_q4k_a8_probe.hip:224-225).
+ * With one logical row the image is stored only when the whole row is clean (src/hip_moe_q4k_a8_probe.hip:47-90); with several
+ * rows (this library's extension) the image views are unspecified after a flagged step. */
 int32_t mi355_a8_enqueue_probe(const mi355_a8_request*, const mi355_a8_bindings*, mi355_stream);
+/* enqueue_serial_prologue_probe (include/strix/hip_moe_q4k_a8_probe.hpp:20-23; src/hip_moe_q4k_a8_probe.hip:187-199,503-519): the
+ * serial row's step with its glue folded in - one workgroup zeroes clear[0 .. clear_words), checks the routes AND the route
+ * weights (an index out of range or a non-finite weight: bit 1, and the quantiser is skipped), quantises, stores the image only
+ * when the row is clean, and OVERWRITES the status word with route bits | quantiser bits; then the projection as above.
+ * shape.logical_rows must be 1. clear and route_weights ([top_k]) are device pointers, 4-byte aligned. */
+int32_t mi355_a8_enqueue_serial_prologue_probe(const mi355_a8_request*, const mi355_a8_bindings*, float* clear, uint32_t clear_words,
+                                               const float* route_weights, mi355_stream);
+/* enqueue_quantize_only (include/strix/hip_moe_q4k_a8_probe.hpp:24; src/hip_moe_q4k_a8_probe.hip:540-554): route check and
+ * quantiser without the projection. The status word is ORed into; a step whose status is already set (or whose route check sets it)
+ * is not quantised and stores nothing. shape.logical_rows must be 1; every binding is validated as for the probe. */
+int32_t mi355_a8_enqueue_quantize_only(const mi355_a8_request*, const mi355_a8_bindings*, mi355_stream);
 
 typedef struct mi355_a8_down_shape { uint32_t hidden, intermediate, experts, top_k; } mi355_a8_down_shape;
 typedef struct mi355_a8_down_request {

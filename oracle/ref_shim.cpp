@@ -328,5 +328,17 @@ int ref_combine_fma(std::uint32_t rows, std::uint32_t top_k, std::uint32_t width
                                 std::span<const float>(eo, n * top_k), std::span<const float>(base, n), std::span<float>(y, n));
     });
 }
+// w and / or base may be null (unit weights, no base): the bf16-steps form of the same function
+int ref_combine_bf16_steps(std::uint32_t rows, std::uint32_t top_k, std::uint32_t width, const float* w, const float* eo,
+                           const float* base, float* y) {
+    return guarded([&] {
+        const std::size_t n = std::size_t{rows} * width;
+        strix::moe::combine_ref(strix::moe::CombineForm::bf16_steps, rows, top_k, width,
+                                w ? std::span<const float>(w, std::size_t{rows} * top_k) : std::span<const float>(),
+                                std::span<const float>(eo, n * top_k), base ? std::span<const float>(base, n) : std::span<const float>(),
+                                std::span<float>(y, n));
+    });
+}
+float ref_combine_round_bf16(float x) { return strix::moe::combine_round_bf16(x); }
 
 }  // extern "C"

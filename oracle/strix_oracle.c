@@ -647,8 +647,33 @@ void orc_route(const orc_route_policy* p, const float* x, uint32_t rows, uint32_
 }
 
 /* ------------------------------------------------------------------ combine */
+/* include/strix/moe/combine.hpp:24-33: nearest-even into the upper 16 bits; a NaN is returned as it came */
+static float combine_round_bf16(float x) {
+    uint32_t bits;
+    memcpy(&bits, &x, 4);
+    if ((bits & 0x7f800000U) == 0x7f800000U && (bits & 0x7fffffU)) return x;
+    bits = (bits + 0x7fffU + ((bits >> 16) & 1U)) & 0xffff0000U;
+    memcpy(&x, &bits, 4);
+    return x;
+}
+
 void orc_combine(int form, uint32_t rows, uint32_t top_k, uint32_t width, const float* w, const uint32_t* ids,
                  const float* raw, const float* base, float* y) {
+    if (form == ORC_COMBINE_BF16_STEPS || form == ORC_COMBINE_BF16_STEPS_ROUNDED_EO) {
+        for (uint32_t r = 0; r < rows; ++r)
+            for (uint32_t d = 0; d < width; ++d) {
+                float acc = 0.0F;
+                for (uint32_t k = 0; k < top_k; ++k) {
+                    float e = raw[((size_t)r * top_k + k) * width + d];
+                    if (form == ORC_COMBINE_BF16_STEPS_ROUNDED_EO) e = combine_round_bf16(e);   /* route_wave_kernel.hpp:113-114 */
+                    const float term = w ? combine_round_bf16(e * w[(size_t)r * top_k + k]) : e;  /* combine.hpp:52 */
+                    acc = combine_round_bf16(acc + term);                                         /* combine.hpp:53 */
+                }
+                const size_t at = (size_t)r * width + d;
+                y[at] = base ? combine_round_bf16(acc + base[at]) : acc;                          /* combine.hpp:57 */
+            }
+        return;
+    }
     for (uint32_t r = 0; r < rows; ++r) {
         uint32_t order[64];
         for (uint32_t k = 0; k < top_k; ++k) order[k] = k;

@@ -42,7 +42,8 @@ enum { ORC_STATUS_INVALID_ROUTE = 1, ORC_STATUS_NONFINITE_ACTIVATION = 2, ORC_ST
 enum { ORC_EXP_GFX1151_NOTABLE = 0, ORC_EXP_DECLARED = 1,
        ORC_EXP_LIBM = 2 };   /* expf of the C library: the Math::exp of the reference's router test oracle (tests/hip_moe_route_launcher_tests.hip:329) */
 enum { ORC_LOGITS_FMA_ASCENDING = 0, ORC_LOGITS_LANE32_BUTTERFLY = 1 };
-enum { ORC_COMBINE_FMA_SLOT_ORDER = 0, ORC_COMBINE_MULADD_ASCENDING_EXPERT = 1 };
+enum { ORC_COMBINE_FMA_SLOT_ORDER = 0, ORC_COMBINE_MULADD_ASCENDING_EXPERT = 1, ORC_COMBINE_BF16_STEPS = 3,
+       ORC_COMBINE_BF16_STEPS_ROUNDED_EO = 4 };
 
 /* ---- scalar conversions --------------------------------------------------------------------- */
 float orc_half_to_float(uint16_t bits);        /* src/cpu/core/reference.cpp:15-24 */
@@ -128,7 +129,8 @@ void orc_route_select(const orc_route_policy* p, const float* scores, uint32_t* 
 
 /* ---- combine (include/strix/moe/combine.hpp:36-59; src/ds41_expert_tp.cpp:189-199) ------------- */
 /* raw [rows][top_k][width], w [rows][top_k], ids [rows][top_k] (needed for the ascending-expert form),
- * base [rows][width] or NULL, y [rows][width]. */
+ * base [rows][width] or NULL, y [rows][width]. The bf16-steps forms (combine.hpp:52-57; operands rounded on read:
+ * src/moe_core/route_wave_kernel.hpp:112-120) take w == NULL as unit weights and round every step to bfloat16. */
 void orc_combine(int form, uint32_t rows, uint32_t top_k, uint32_t width, const float* w, const uint32_t* ids,
                  const float* raw, const float* base, float* y);
 

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(HERE, "libmi355_strix.so")
 TYPE_Q5_1, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K = 7, 8, 12, 13, 14
 INPUT_F32, INPUT_F16, INPUT_BF16 = 0, 1, 2
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
-COMBINE_FMA_SLOT, COMBINE_MULADD_ASC, COMBINE_NONE = 0, 1, 2
+COMBINE_FMA_SLOT, COMBINE_MULADD_ASC, COMBINE_NONE, COMBINE_BF16_STEPS = 0, 1, 2, 3
 EXP_GFX1151, EXP_DECLARED, EXP_LIBM = 0, 1, 2
 STATUS_INVALID_ROUTE, STATUS_NONFINITE_ACTIVATION, STATUS_INVALID_DELTA, STATUS_NONFINITE_PROJECTION, STATUS_AGGREGATE = 1, 2, 4, 8, 16
 E_INVALID_ARGUMENT, E_UNSUPPORTED, E_HIP = -1, -2, -3
@@ -254,8 +254,8 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
-           "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue_combine", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
+           "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe", "mi355_a8_enqueue_serial_prologue_probe", "mi355_a8_enqueue_quantize_only",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
            "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
            "mi355_a8_enqueue_down_activation_quantize_union", "mi355_a8_enqueue_down_rawdots_union",
@@ -364,6 +364,15 @@ def swiglu_quantize(gate, up, exp_kind=EXP_GFX1151, swiglu_limit=float("inf")):
     return codes, deltas, sums, h, status
 
 
+def combine(form, eo, w=None, base=None, round_eo=False):
+    """The combine operator on its own (strix::moe_core::enqueue_combine, src/moe_core/route_wave_kernel.hpp:138-160):
+    eo [rows][top_k][width] fp32, w [rows][top_k] or None (bf16-steps: unit weights), base [rows][width] or None."""
+    rows, top_k, width = eo.shape
+    y = torch.zeros((rows, width), dtype=torch.float32, device=eo.device)
+    check(lib().mi355_moe_enqueue_combine(form, rows, top_k, width, _p(w), _p(eo), _p(base), _p(y), 1 if round_eo else 0, _stream()))
+    return y
+
+
 class A8Decode:
     """The reference's single-row A8 pipeline over the request / bindings entry points (include/strix/hip_moe_q4k_a8_probe.hpp:12,
     include/strix/hip_moe_a8_down.hpp:18-30): probe -> down_activation_quantize -> down_rawdots (+ slot merge). Owns the views the
@@ -410,6 +419,14 @@ class A8Decode:
     def enqueue_probe(self, rows=None):
         q, b = self.request(rows), self.bindings(rows)
         check(lib().mi355_a8_enqueue_probe(C.byref(q), C.byref(b), _stream()))
+
+    def enqueue_serial_prologue_probe(self, clear, clear_words, route_weights):
+        req, b = self.request(1), self.bindings(1)
+        check(lib().mi355_a8_enqueue_serial_prologue_probe(C.byref(req), C.byref(b), _p(clear), clear_words, _p(route_weights), _stream()))
+
+    def enqueue_quantize_only(self):
+        req, b = self.request(1), self.bindings(1)
+        check(lib().mi355_a8_enqueue_quantize_only(C.byref(req), C.byref(b), _stream()))
 
     def enqueue_down_activation_quantize(self, rows=None, exp_kind=EXP_GFX1151):
         q, b = self.down_request(), self.down_bindings(rows)

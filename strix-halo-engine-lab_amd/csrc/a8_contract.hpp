@@ -196,6 +196,63 @@ __global__ __launch_bounds__(256) void a8_probe_prologue_kernel(const uint8_t* x
     }
 }
 
+// One serial row's prologue in one workgroup, with the reference's store rules (src/hip_moe_q4k_a8_probe.hip:47-90,187-199):
+//   SERIAL: zero clear[0 .. clear_words), check the routes (an index out of range or a non-finite route weight: bit 1), quantise
+//           unless a route failed, and OVERWRITE the status word with route bits | quantiser bits;
+//   else:   the pair validate_routes + quantize: OR bit 1 for an index out of range (route weights are not looked at), quantise only
+//           when the status word is still zero after that, OR the quantiser's bits in.
+// The quantiser stages codes / deltas / sums in LDS and stores them only when the whole row is clean: a flagged step leaves the
+// image of the previous step in place.
+template <int KIND, bool SERIAL>
+__global__ __launch_bounds__(1024) void a8_serial_prologue_kernel(const uint8_t* x, const uint32_t* routes, const float* route_weights, float* clear,
+                                                                  uint32_t clear_words, uint32_t hidden, uint32_t top_k, uint32_t experts,
+                                                                  int8_t* codes, float* deltas, int32_t* sums, uint32_t* status) {
+    __shared__ __attribute__((aligned(16))) int8_t local_codes[kA8MaxHidden];
+    __shared__ __attribute__((aligned(16))) float local_deltas[kA8MaxHidden / 32U];
+    __shared__ __attribute__((aligned(16))) int32_t local_sums[kA8MaxHidden / 32U];
+    __shared__ uint32_t route_bits, bad_bits, initial;
+    const uint32_t t = threadIdx.x, groups = hidden / 32U;
+    if (t == 0) { route_bits = 0; bad_bits = 0; initial = SERIAL ? 0U : *status; }
+    if (SERIAL) for (uint32_t i = t; i < clear_words; i += 1024U) clear[i] = 0.0F;
+    __syncthreads();
+    if (t < top_k && (routes[t] >= experts || (SERIAL && !finite_f(route_weights[t])))) atomicOr(&route_bits, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+    __syncthreads();
+    const uint32_t before = initial | route_bits;
+    if (!SERIAL && t == 0 && route_bits) atomicOr(status, route_bits);
+    if (before != 0U) {                                      // the quantiser is skipped: nothing stored
+        if (SERIAL && t == 0) *status = route_bits;
+        return;
+    }
+    for (uint32_t g = t >> 5; g < groups; g += 32U) {
+        const uint32_t i = g * 32U + (t & 31U);
+        float v = load_activation<KIND>(x, i);
+        const int bad = or32_i(finite_f(v) ? 0 : 1);
+        if (!finite_f(v)) v = 0.0F;
+        const float amax = max32(__builtin_fabsf(v));
+        float delta = amax == 0.0F ? 1.0F : amax / 127.0F;
+        const bool underflow = !(delta > 0.0F) || !finite_f(delta);
+        if (underflow) delta = 1.0F;
+        const int code = a8_code(v, delta, false);
+        const int sum = sum32_i(code);
+        local_codes[i] = static_cast<int8_t>(code);
+        if ((t & 31U) == 0) {
+            local_deltas[g] = delta; local_sums[g] = sum;
+            if (bad) atomicOr(&bad_bits, static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
+            if (underflow) atomicOr(&bad_bits, static_cast<uint32_t>(MI355_STATUS_INVALID_DELTA));
+        }
+    }
+    __syncthreads();
+    const uint32_t bad = bad_bits;
+    if (bad == 0U) {
+        for (uint32_t i = t; i < hidden / 16U; i += 1024U) reinterpret_cast<u32x4*>(codes)[i] = reinterpret_cast<const u32x4*>(local_codes)[i];
+        for (uint32_t i = t; i < groups; i += 1024U) { deltas[i] = local_deltas[i]; sums[i] = local_sums[i]; }
+    }
+    if (t == 0) {
+        if (SERIAL) *status = bad;
+        else if (bad) atomicOr(status, bad);
+    }
+}
+
 // The down producer (src/hip_moe_q4k_a8_probe.hip:594-621): intermediates hold, per assignment, [gate I | up I]; h replaces the
 // gate half, its A8 image goes to codes / deltas / sums [assignment][I]. One half-wave per group of 32.
 __global__ __launch_bounds__(256) void a8_down_activation_kernel(float* intermediates, const uint32_t* routes, uint32_t experts, uint32_t width,
@@ -326,22 +383,39 @@ int32_t mi355_a8_validate_down(const mi355_a8_down_request* q, const mi355_a8_do
 namespace {
 // Probe of R logical rows. union_plan == nullptr: item i = assignment i (an expert chosen by two rows is read twice);
 // otherwise the plan is built first and the items are its entries (each distinct expert read once).
-int32_t a8_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, uint32_t* union_plan, hipStream_t st) {
+enum { kA8PrologueProbe = 0, kA8PrologueSerial = 1, kA8PrologueQuantize = 2, kA8PrologueQuantizeOnly = 3 };
+int32_t a8_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, uint32_t* union_plan, hipStream_t st, int prologue_form = kA8PrologueProbe,
+                 float* clear = nullptr, uint32_t clear_words = 0, const float* route_weights = nullptr) {
     const mi355_a8_shape& s = q->shape;
     const uint32_t R = s.logical_rows, groups = s.hidden / 32U;
     const uint8_t* x = reinterpret_cast<const uint8_t*>(b->input.address);
     const uint32_t* routes = reinterpret_cast<const uint32_t*>(b->routes.address);
     uint32_t* status = reinterpret_cast<uint32_t*>(b->status.address);
-    const dim3 pgrid((groups + 7U) / 8U + (union_plan ? 1U : 0U), R);
-    const uint32_t checked = union_plan ? 0U : s.top_k;       // (the union builder has checked the routes)
-    const auto prologue = [&](auto kind) {
-        a8_probe_prologue_kernel<decltype(kind)::value><<<pgrid, 256, 0, st>>>(x, s.hidden, routes, s.experts, checked,
-            reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), status,
-            union_plan, s.top_k);
-    };
-    if (q->input == MI355_INPUT_F32) prologue(std::integral_constant<int, 0>{});
-    else if (q->input == MI355_INPUT_F16) prologue(std::integral_constant<int, 1>{});
-    else prologue(std::integral_constant<int, 2>{});
+    if (prologue_form == kA8PrologueProbe) {
+        const dim3 pgrid((groups + 7U) / 8U + (union_plan ? 1U : 0U), R);
+        const uint32_t checked = union_plan ? 0U : s.top_k;       // (the union builder has checked the routes)
+        const auto prologue = [&](auto kind) {
+            a8_probe_prologue_kernel<decltype(kind)::value><<<pgrid, 256, 0, st>>>(x, s.hidden, routes, s.experts, checked,
+                reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), status,
+                union_plan, s.top_k);
+        };
+        if (q->input == MI355_INPUT_F32) prologue(std::integral_constant<int, 0>{});
+        else if (q->input == MI355_INPUT_F16) prologue(std::integral_constant<int, 1>{});
+        else prologue(std::integral_constant<int, 2>{});
+    } else {
+        const auto prologue = [&](auto kind, auto serial) {
+            a8_serial_prologue_kernel<decltype(kind)::value, decltype(serial)::value><<<1, 1024, 0, st>>>(x, routes, route_weights, clear, clear_words,
+                s.hidden, s.top_k, s.experts, reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address),
+                reinterpret_cast<int32_t*>(b->sums.address), status);
+        };
+        const auto by_kind = [&](auto serial) {
+            if (q->input == MI355_INPUT_F32) prologue(std::integral_constant<int, 0>{}, serial);
+            else if (q->input == MI355_INPUT_F16) prologue(std::integral_constant<int, 1>{}, serial);
+            else prologue(std::integral_constant<int, 2>{}, serial);
+        };
+        if (prologue_form == kA8PrologueSerial) by_kind(std::true_type{}); else by_kind(std::false_type{});
+        if (prologue_form == kA8PrologueQuantizeOnly) return MI355_OK;
+    }
     mi355_moe_weights w{};
     w.hidden = s.hidden; w.ffn = s.rows; w.experts = s.experts; w.top_k = s.top_k; w.gate_type = q->gate_type; w.down_type = MI355_TYPE_Q4_K;
     w.gate = reinterpret_cast<const uint8_t*>(b->gate.address); w.up = reinterpret_cast<const uint8_t*>(b->up.address);
@@ -353,6 +427,7 @@ int32_t a8_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, uint32_t
     r.in = dense_image(reinterpret_cast<int8_t*>(b->codes.address), reinterpret_cast<float*>(b->deltas.address), reinterpret_cast<int32_t*>(b->sums.address), s.hidden);
     r.status = status; r.job_status = status;
     r.status_rs = 0;                // one shared status word
+    r.clean_only = 1U;              // a step flagged by the prologue leaves `output` as it was
     r.gate_out = reinterpret_cast<float*>(b->output.address); r.up_out = r.gate_out + s.rows; r.slot_stride = 2ULL * s.rows;
     r.inter_rs = 4ULL * s.top_k * r.slot_stride;
     r.union_plan = union_plan;
@@ -370,8 +445,33 @@ int32_t a8_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, uint32_t
 
 int32_t mi355_a8_enqueue_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, mi355_stream stream) {
     if (const int32_t rc = a8_validate(q, b)) return rc;          // the whole bundle is validated before the first enqueue
-    a8_probe(q, b, nullptr, hs(stream));
+    // one logical row is the reference's own form (src/hip_moe_q4k_a8_probe.hip:487-502): its one-workgroup quantiser, which leaves
+    // the previous image in place when the step is flagged; several rows share the status word and take the many-workgroup prologue
+    a8_probe(q, b, nullptr, hs(stream), q->shape.logical_rows == 1U ? kA8PrologueQuantize : kA8PrologueProbe);
     STRIX_LAUNCHED("A8 probe");
+    return MI355_OK;
+}
+
+// The serial row's step with its glue folded into the prologue (enqueue_serial_prologue_probe, include/strix/hip_moe_q4k_a8_probe.hpp:20-23,
+// src/hip_moe_q4k_a8_probe.hip:503-519): clear + route and route-weight check + quantiser in one workgroup, status overwritten, then the
+// projection. One logical row.
+int32_t mi355_a8_enqueue_serial_prologue_probe(const mi355_a8_request* q, const mi355_a8_bindings* b, float* clear, uint32_t clear_words,
+                                               const float* route_weights, mi355_stream stream) {
+    if (const int32_t rc = a8_validate(q, b)) return rc;
+    STRIX_REQUIRE(clear && route_weights && aligned(clear, 4) && aligned(route_weights, 4), "A8 serial prologue bindings are invalid");   // :507
+    STRIX_REQUIRE(q->shape.logical_rows == 1U, "A8 serial prologue: one logical row");
+    a8_probe(q, b, nullptr, hs(stream), kA8PrologueSerial, clear, clear_words, route_weights);
+    STRIX_LAUNCHED("A8 serial prologue probe");
+    return MI355_OK;
+}
+
+// Route check + quantiser without the projection (enqueue_quantize_only, include/strix/hip_moe_q4k_a8_probe.hpp:24,
+// src/hip_moe_q4k_a8_probe.hip:540-554): status is ORed into, and a row whose status is already set is not quantised. One logical row.
+int32_t mi355_a8_enqueue_quantize_only(const mi355_a8_request* q, const mi355_a8_bindings* b, mi355_stream stream) {
+    if (const int32_t rc = a8_validate(q, b)) return rc;
+    STRIX_REQUIRE(q->shape.logical_rows == 1U, "A8 quantize only: one logical row");
+    a8_probe(q, b, nullptr, hs(stream), kA8PrologueQuantizeOnly);
+    STRIX_LAUNCHED("A8 quantize only");
     return MI355_OK;
 }
 

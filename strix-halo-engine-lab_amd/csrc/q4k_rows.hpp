@@ -92,6 +92,8 @@ struct RowsK : mi355_moe_rows {
     const uint32_t* union_plan;     // verify-window form: the expert-union plan (below) names the items instead of `plan`
     uint32_t top1_form;       // a dense top-1 job whose down launch also publishes the output: combine form + 1 (0: the merge launch does)
     uint32_t* aggregate;      // optional summary word of the A8 down bindings (include/strix/moe_a8_down_contract.hpp:50-52): bit 16 beside a row's flag
+    uint32_t clean_only;      // probe form: nothing is computed or stored once the shared status word is set ("this kernel never changes
+                              // status" and returns on a set one, src/hip_moe_q4k_a8_probe.hip:224-225,257-258)
     uint32_t* awords;         // a decode batch planned from early routes: one word per assignment (finished projection waves in the low
                               // half, bit 31 = non-finite projection), in place of direct updates of the status words
 
@@ -177,6 +179,7 @@ __device__ __forceinline__ uint32_t union_assignment(const uint32_t* plan, uint3
 }
 
 __device__ __forceinline__ WorkItem work_item(const mi355_moe_weights& w, const RowsK& r, uint32_t items_at, uint32_t index) {
+    if (r.clean_only && *r.status != 0U) return {0U, index, index, index + 1U};
     if (r.union_plan) return union_item(r.union_plan, index);
     if (r.plan) {
         const uint4 item = *reinterpret_cast<const uint4*>(r.plan + items_at + 4U * index);

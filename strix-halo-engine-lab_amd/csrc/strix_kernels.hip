@@ -2489,4 +2489,5 @@ int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float*
 
 #include "a8_contract.hpp"
 #include "rows_forms.hpp"
+#include "combine_forms.hpp"
 #include "gguf_reader.hpp"

@@ -53,6 +53,24 @@ Q6K_WIDTHS = [256, 768, 1280, 1536]
 RMSNORM_CASES = [(401, 64, 3), (402, 511, 2), (403, 2048, 4), (404, 6144, 2)]
 ROW_WIDTHS = [2048, 768, 4096, 5120, 6144, 1280, 27648]
 GEMV_CASES = [(201, 4096, 64, 2), (202, 1024, 33, 3)]
+# (seed, rows, top_k, width, weights bound, base bound, operands already bfloat16 values): the reference's own two shapes
+# (tests/hip_hy4_routed_tests.hip:205-206) and a ragged one with full fp32 operands
+COMBINE_CASES = [(501, 5, 16, 1536, True, False, True), (502, 5, 1, 3072, False, True, True), (503, 3, 7, 100, True, True, False),
+                 (504, 2, 3, 33, False, False, False)]
+
+
+def combine_case(seed, rows, top_k, width, has_w, has_base, bf16_operands):
+    rng = np.random.default_rng(seed)
+    eo = rng.standard_normal((rows, top_k, width)).astype(np.float32)
+    base = rng.standard_normal((rows, width)).astype(np.float32)
+    if bf16_operands:
+        eo = ((eo.view(np.uint32) + 0x8000) & 0xffff0000).astype(np.uint32).view(np.float32)
+        base = ((base.view(np.uint32) + 0x8000) & 0xffff0000).astype(np.uint32).view(np.float32)
+    w = rng.random((rows, top_k)).astype(np.float32)
+    eo[0, 0, 0] = np.float32(np.nan); eo[rows - 1, top_k - 1, width - 1] = np.float32(np.inf)
+    eo[0, 0, 1] = np.float32(1.00390625)          # an exact tie of the rounding (1 + 2^-8): to even = 1.0
+    eo[0, 0, 2] = np.float32(1.01171875)          # 1 + 3 * 2^-8: to even = 1 + 2^-6
+    return eo, (w if has_w else None), (base if has_base else None)
 
 
 def main():
@@ -121,6 +139,18 @@ def main():
         y = np.empty_like(x)
         assert R.ref_rmsnorm_f32(x.ctypes.data_as(orc.f32p), w.ctypes.data_as(orc.f32p), n, C.c_float(1e-6), y.ctypes.data_as(orc.f32p), rows) == 0
         out[f"rmsnorm_{seed}_bits"] = y.view(np.uint32)
+    for case in COMBINE_CASES:
+        eo, w, base = combine_case(*case)
+        rows, top_k, width = eo.shape
+        y = np.zeros((rows, width), np.float32)
+        ptr = lambda a: None if a is None else a.ctypes.data_as(orc.f32p)
+        assert R.ref_combine_bf16_steps(rows, top_k, width, ptr(w), ptr(eo), ptr(base), ptr(y)) == 0
+        out[f"combine_{case[0]}_bits"] = y.view(np.uint32).copy()
+        # operands rounded on read == the same combine over operands rounded beforehand (src/moe_core/route_wave_kernel.hpp:96-97)
+        R.ref_combine_round_bf16.restype = C.c_float
+        rounded = np.array([R.ref_combine_round_bf16(C.c_float(float(v))) if np.isfinite(v) else v for v in eo.ravel()], np.float32).reshape(eo.shape)
+        assert R.ref_combine_bf16_steps(rows, top_k, width, ptr(w), ptr(rounded), ptr(base), ptr(y)) == 0
+        out[f"combine_{case[0]}_rounded_bits"] = y.view(np.uint32).copy()
     np.savez_compressed(os.path.join(HERE, "ref_vectors.npz"), **out)
     print("wrote", {k: v.shape for k, v in out.items()})
 

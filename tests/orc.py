@@ -13,7 +13,7 @@ Q5_1, Q8_0, Q4_K, Q5_K, Q6_K = 7, 8, 12, 13, 14
 Q5_1_BLOCK, Q8_0_BLOCK, Q4_K_BLOCK, Q5_K_BLOCK, Q6_K_BLOCK = 24, 34, 144, 176, 210
 EXP_GFX1151, EXP_DECLARED, EXP_LIBM = 0, 1, 2
 LOGITS_FMA, LOGITS_LANE32 = 0, 1
-COMBINE_FMA_SLOT, COMBINE_MULADD_ASC = 0, 1
+COMBINE_FMA_SLOT, COMBINE_MULADD_ASC, COMBINE_BF16_STEPS, COMBINE_BF16_STEPS_ROUNDED_EO = 0, 1, 3, 4
 
 u8p, i8p, f32p, i32p, u32p = (C.POINTER(t) for t in (C.c_uint8, C.c_int8, C.c_float, C.c_int32, C.c_uint32))
 
@@ -369,8 +369,8 @@ def route_select(scores, top_k, renorm_eps=0.0, scale=1.0, renormalize=True, ren
 def combine(form, w, ids, raw, base=None):
     rows, top_k, width = raw.shape
     raw = np.ascontiguousarray(raw, np.float32)
-    w = np.ascontiguousarray(w, np.float32)
-    ids = np.ascontiguousarray(ids, np.uint32)
+    w = None if w is None else np.ascontiguousarray(w, np.float32)
+    ids = np.zeros((rows, top_k), np.uint32) if ids is None else np.ascontiguousarray(ids, np.uint32)
     y = np.zeros((rows, width), np.float32)
     b = None if base is None else np.ascontiguousarray(base, np.float32)
     lib().orc_combine(form, rows, top_k, width, _ptr(w, f32p), _ptr(ids, u32p), _ptr(raw, f32p), _ptr(b, f32p), _ptr(y, f32p))

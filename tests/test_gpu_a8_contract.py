@@ -98,6 +98,8 @@ def test_probe_rows_in_multiples_of_32_only(strix):
 
 
 def test_probe_invalid_route_and_nonfinite_input_are_sticky_status_bits(strix):
+    """Status bits are ORed in and stay; a step whose status word is set when the projection starts stores no gate / up row at all
+    (src/hip_moe_q4k_a8_probe.hip:224-225: the projection returns on a set status)."""
     H, I, E, K = 1024, 256, 8, 2
     rng = np.random.default_rng(1)
     gate, up, _ = make_layer(rng, H, I, E)
@@ -109,14 +111,112 @@ def test_probe_invalid_route_and_nonfinite_input_are_sticky_status_bits(strix):
     p.status.fill_(32)                                                          # a bit the caller already holds stays
     p.enqueue_probe()
     assert int(p.status.item()) == 32 | 1
-    out = p.intermediates.cpu().numpy()
-    assert np.all(out[0, 1] == -7.0) and not np.any(out[1] == -7.0) and not np.any(out[0, 0] == -7.0)    # only the bad slot is left alone
+    assert np.all(p.intermediates.cpu().numpy() == -7.0)
+    p.status.zero_()
+    p.enqueue_probe()
+    assert int(p.status.item()) == 1 and np.all(p.intermediates.cpu().numpy() == -7.0)
     x[1, 5] = np.inf
     p.input.copy_(torch.from_numpy(x))
     p.routes.copy_(torch.tensor([[1, 0], [3, 2]], dtype=torch.int32))
     p.status.zero_()
     p.enqueue_probe()
-    assert int(p.status.item()) == 2
+    assert int(p.status.item()) == 2 and np.all(p.intermediates.cpu().numpy() == -7.0)
+    x[1, 5] = 0.25
+    p.input.copy_(torch.from_numpy(x))
+    p.status.zero_()
+    p.enqueue_probe()
+    assert int(p.status.item()) == 0 and not np.any(p.intermediates.cpu().numpy() == -7.0)
+
+
+def _poisoned_decode(strix, rng, H, I, E, K, kind):
+    gate, up, _ = make_layer(rng, H, I, E)
+    p = strix.A8Decode(H, I, E, K, dev(gate), dev(up), None, rows=1, input_dtype=DT[kind])
+    p.codes.fill_(77); p.deltas.fill_(-3.0); p.sums.fill_(-99); p.intermediates.fill_(-7.0)
+    return p, gate, up
+
+
+def _image_untouched(p):
+    return bool((p.codes == 77).all() and (p.deltas == -3.0).all() and (p.sums == -99).all())
+
+
+@pytest.mark.parametrize("H,I,K,kind", [(2560, 640, 10, "bf16"), (2560, 640, 10, "f32"), (256, 32, 1, "bf16"), (2048, 768, 8, "f16")])
+@pytest.mark.parametrize("error", ["none", "route_index", "route_weight", "input"])
+def test_serial_prologue_probe(strix, H, I, K, kind, error):
+    """mi355_a8_enqueue_serial_prologue_probe on the reference's own cases (tests/hip_moe_q4k_a8_probe_tests.hip:303-376: hidden 2560 x
+    640 x top-10 and 256 x 32 x top-1, both input kinds, each error): the cleared words, the OVERWRITTEN status word, the image
+    (stored only for a clean row) and the gate / up rows (stored only for a clean step)."""
+    E = 16
+    rng = np.random.default_rng(H + K + len(error))
+    p, gate, up = _poisoned_decode(strix, rng, H, I, E, K, kind)
+    x = rng.standard_normal((1, H)).astype(np.float32)
+    ids = rng.permutation(E)[:K].astype(np.uint32)[None, :]
+    weights = rng.random(K).astype(np.float32)
+    if error == "route_index":
+        ids[0, K - 1] = E
+    if error == "route_weight":
+        weights[0] = np.inf
+    if error == "input":
+        x[0, H - 3] = np.nan
+    x_t, x32 = to_input(x, kind)
+    p.input.copy_(x_t)
+    p.routes.copy_(torch.from_numpy(ids.astype(np.int32)))
+    clear = torch.full((H + 5,), 9.0, dtype=torch.float32, device="cuda")
+    p.status.fill_(0x5a5a)                                                       # stale: the prologue overwrites it
+    p.enqueue_serial_prologue_probe(clear, H, dev(weights))
+    torch.cuda.synchronize()
+    assert bool((clear[:H] == 0).all()) and bool((clear[H:] == 9.0).all())
+    want_status = {"none": 0, "route_index": 1, "route_weight": 1, "input": 2}[error]
+    assert int(p.status.item()) == want_status
+    if error != "none":
+        assert _image_untouched(p) and np.all(p.intermediates.cpu().numpy() == -7.0)
+        return
+    c, d, s, _ = orc.quantize_a8(x32)
+    assert np.array_equal(p.codes.cpu().numpy(), c) and np.array_equal(bits(p.deltas.cpu().numpy()), bits(d)) and np.array_equal(p.sums.cpu().numpy(), s)
+    dummy_down = np.zeros((E, H, orc.row_bytes(orc.Q8_0, I)), np.uint8)
+    ref = orc.routed_experts(H, I, K, gate, up, dummy_down, orc.Q8_0, c, d, s, ids)
+    out = p.intermediates.cpu().numpy()
+    assert np.array_equal(bits(out[0, :, 0]), bits(ref.gate.reshape(K, I))) and np.array_equal(bits(out[0, :, 1]), bits(ref.up.reshape(K, I)))
+
+
+def test_quantize_only_and_the_single_row_probe_store_rules(strix):
+    """mi355_a8_enqueue_quantize_only (src/hip_moe_q4k_a8_probe.hip:540-554): the image of a clean row, status ORed into, no gate / up
+    row; a row whose status is already set, whose route names no expert or that holds a non-finite value stores nothing. The
+    one-row probe keeps the same rules for the image and stores no row on a flagged step."""
+    H, I, E, K = 2048, 768, 32, 8
+    rng = np.random.default_rng(540)
+    x = rng.standard_normal((1, H)).astype(np.float32)
+    ids = rng.permutation(E)[:K].astype(np.uint32)[None, :]
+    for entry in ("quantize_only", "probe"):
+        for case, preset, want in (("clean", 0, 0), ("held", 32, 32), ("route", 0, 1), ("route_held", 64, 65), ("input", 0, 2)):
+            p, gate, up = _poisoned_decode(strix, rng, H, I, E, K, "bf16")
+            xs, routes = x.copy(), ids.copy()
+            if case.startswith("route"):
+                routes[0, 0] = E + 7
+            if case == "input":
+                xs[0, 1] = -np.inf
+            x_t, x32 = to_input(xs, "bf16")
+            p.input.copy_(x_t)
+            p.routes.copy_(torch.from_numpy(routes.astype(np.int32)))
+            p.status.fill_(preset)
+            getattr(p, "enqueue_" + entry)()
+            torch.cuda.synchronize()
+            assert int(p.status.item()) == want, (entry, case)
+            out = p.intermediates.cpu().numpy()
+            if case != "clean":
+                assert _image_untouched(p) and np.all(out == -7.0), (entry, case)
+                continue
+            c, d, s, _ = orc.quantize_a8(x32)
+            assert np.array_equal(p.codes.cpu().numpy(), c) and np.array_equal(bits(p.deltas.cpu().numpy()), bits(d)) and np.array_equal(p.sums.cpu().numpy(), s)
+            if entry == "quantize_only":
+                assert np.all(out == -7.0)
+            else:
+                assert not np.any(out == -7.0)
+    p, _, _ = _poisoned_decode(strix, rng, H, I, E, K, "bf16")
+    with pytest.raises(strix.StrixError, match="serial prologue bindings"):
+        p.enqueue_serial_prologue_probe(None, 0, dev(np.ones(K, np.float32)))
+    two = strix.A8Decode(H, I, E, K, p.gate, p.up, None, rows=2)
+    with pytest.raises(strix.StrixError, match="one logical row"):
+        strix.check(strix.lib().mi355_a8_enqueue_quantize_only(__import__("ctypes").byref(two.request(2)), __import__("ctypes").byref(two.bindings(2)), None))
 
 
 def test_probe_and_down_refuse_a_bad_bundle_before_any_launch(strix):

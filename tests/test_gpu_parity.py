@@ -1096,3 +1096,62 @@ def test_prefill_f16_mfma_matches_exact_weight_product(strix, H, I, E, K, T):
     g_oracle = orc.base_linear(orc.Q4_K, gate[e0], H // 256 * 144, I, H, x[:4].astype(np.float32))
     g64 = x[:4].astype(np.float64) @ orc.dequant_rows(orc.Q4_K, gate[e0], H).astype(np.float64).T
     assert rel_err(g_oracle, g64.astype(np.float32))[0] < 1e-5
+
+
+# ------------------------------------------------------------------------------------------- the combine operator
+def _combine_operands(seed, rows, top_k, width, bf16_values):
+    rng = np.random.default_rng(seed)
+    eo = rng.standard_normal((rows, top_k, width)).astype(np.float32)
+    base = rng.standard_normal((rows, width)).astype(np.float32)
+    if bf16_values:                                    # the reference's own cases feed bfloat16 values (tests/hip_hy4_routed_tests.hip:173-174)
+        eo = ((eo.view(np.uint32) + 0x8000) & 0xffff0000).astype(np.uint32).view(np.float32)
+        base = ((base.view(np.uint32) + 0x8000) & 0xffff0000).astype(np.uint32).view(np.float32)
+    w = rng.random((rows, top_k)).astype(np.float32)
+    eo[0, 0, 0] = np.nan
+    eo[rows - 1, top_k - 1, width - 1] = np.inf
+    eo[0, 0, 1], eo[0, 0, 2] = 1.00390625, 1.01171875   # exact ties of the rounding
+    return eo, w, base
+
+
+@pytest.mark.parametrize("rows,top_k,width,bf16_values", [(5, 16, 1536, True), (5, 1, 3072, True), (3, 7, 100, False), (2, 3, 33, False),
+                                                          (1, 20, 257, False), (1100, 8, 4096, False)])
+def test_combine_operator_bit_exact(strix, rows, top_k, width, bf16_values):
+    """mi355_moe_enqueue_combine in the bf16-steps form (weights and base bound or not, operands rounded on read or not) and
+    the fma form, against the oracle (itself equal to the compiled reference's combine_ref on these forms and to the vectors
+    it left in tests/golden). The last shape takes the four-columns-per-thread launch."""
+    eo, w, base = _combine_operands(rows * 31 + top_k, rows, top_k, width, bf16_values)
+    for has_w in (True, False):
+        for has_base in (True, False):
+            for rounded in (False, True):
+                got = strix.combine(strix.COMBINE_BF16_STEPS, dev(eo), dev(w) if has_w else None, dev(base) if has_base else None, round_eo=rounded).cpu().numpy()
+                want = orc.combine(orc.COMBINE_BF16_STEPS_ROUNDED_EO if rounded else orc.COMBINE_BF16_STEPS, w if has_w else None, None, eo, base if has_base else None)
+                assert np.array_equal(bits(got), bits(want)), (has_w, has_base, rounded)
+    got = strix.combine(strix.COMBINE_FMA_SLOT, dev(eo), dev(w), dev(base)).cpu().numpy()
+    want = orc.combine(orc.COMBINE_FMA_SLOT, w, None, eo, base)
+    nan = np.isnan(want)
+    assert np.array_equal(nan, np.isnan(got)) and np.array_equal(bits(got)[~nan], bits(want)[~nan])
+
+
+def test_combine_operator_golden_and_refusals(strix):
+    """The vectors the compiled reference wrote, straight through the device operator; and the argument rules of the
+    reference's host entry (src/moe_core/route_wave_kernel.hpp:146-147, include/strix/moe/combine.hpp:41-44)."""
+    import importlib.util, os
+    here = os.path.dirname(os.path.abspath(__file__))
+    spec = importlib.util.spec_from_file_location("make_ref_vectors", os.path.join(here, "golden", "make_ref_vectors.py"))
+    mk = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mk)
+    gold = np.load(os.path.join(here, "golden", "ref_vectors.npz"))
+    for case in mk.COMBINE_CASES:
+        eo, w, base = mk.combine_case(*case)
+        d = lambda a: None if a is None else dev(a)
+        assert np.array_equal(bits(strix.combine(strix.COMBINE_BF16_STEPS, dev(eo), d(w), d(base)).cpu().numpy()), gold[f"combine_{case[0]}_bits"])
+        assert np.array_equal(bits(strix.combine(strix.COMBINE_BF16_STEPS, dev(eo), d(w), d(base), round_eo=True).cpu().numpy()), gold[f"combine_{case[0]}_rounded_bits"])
+    eo = dev(np.ones((2, 2, 8), np.float32))
+    w = dev(np.ones((2, 2), np.float32))
+    with pytest.raises(strix.StrixError, match="fma_f32 needs weights and base"):
+        strix.combine(strix.COMBINE_FMA_SLOT, eo, w, None)
+    with pytest.raises(strix.StrixError, match="bf16-steps form only"):
+        strix.combine(strix.COMBINE_FMA_SLOT, eo, w, dev(np.ones((2, 8), np.float32)), round_eo=True)
+    with pytest.raises(strix.StrixError, match="form must be"):
+        strix.combine(strix.COMBINE_MULADD_ASC, eo, w, None)
+    assert strix.combine(strix.COMBINE_BF16_STEPS, dev(np.ones((0, 2, 8), np.float32)), None, None).shape == (0, 8)

@@ -856,6 +856,11 @@ def test_ref_router_policy_and_combine_bits():
                              y_ref.ctypes.data_as(orc.f32p)) == 0
     y = orc.combine(orc.COMBINE_FMA_SLOT, w, np.zeros((3, 8), np.uint32), raw, base)
     assert np.array_equal(bits(y), bits(y_ref))
+    for has_w, has_base in ((True, True), (True, False), (False, True), (False, False)):         # CombineForm::bf16_steps
+        p = lambda a, on: a.ctypes.data_as(orc.f32p) if on else None
+        assert R.ref_combine_bf16_steps(3, 8, 64, p(w, has_w), p(raw, True), p(base, has_base), p(y_ref, True)) == 0
+        y = orc.combine(orc.COMBINE_BF16_STEPS, w if has_w else None, None, raw, base if has_base else None)
+        assert np.array_equal(bits(y), bits(y_ref)), (has_w, has_base)
 
 
 @needs_ref
@@ -1017,6 +1022,36 @@ def test_committed_reference_vectors():
         x = (rng.standard_normal((rows, n)) * 2.0).astype(np.float32)
         w = rng.standard_normal(n).astype(np.float32)
         assert np.array_equal(bits(orc.rmsnorm_f32(x, w, 1e-6)), gold[f"rmsnorm_{seed}_bits"])
+    for case in mk.COMBINE_CASES:                                           # the bf16-steps combine, weights / base bound or not
+        eo, w, base = mk.combine_case(*case)
+        assert np.array_equal(bits(orc.combine(orc.COMBINE_BF16_STEPS, w, None, eo, base)), gold[f"combine_{case[0]}_bits"]), case
+        assert np.array_equal(bits(orc.combine(orc.COMBINE_BF16_STEPS_ROUNDED_EO, w, None, eo, base)), gold[f"combine_{case[0]}_rounded_bits"]), case
+
+
+def test_bf16_steps_combine_against_what_the_rounding_fixes():
+    """Independent of the reference build: numpy's own arithmetic restates the chain for one slot and unit weights, where
+    it reduces to a single rounding (acc = bf16(0 + e)); exact ties go to even; a NaN comes back with its payload; with
+    weights of one and operands that are bfloat16 values whose sums stay within 8 bits the chain is exact integer addition."""
+    def bf16(a):
+        b = np.asarray(a, np.float32).view(np.uint32).astype(np.uint64)
+        return (((b + 0x7fff + ((b >> 16) & 1)) & 0xffff0000).astype(np.uint32)).view(np.float32)
+    rng = np.random.default_rng(77)
+    e = rng.standard_normal((4, 1, 50)).astype(np.float32)
+    assert np.array_equal(bits(orc.combine(orc.COMBINE_BF16_STEPS, None, None, e)), bits(bf16(e[:, 0])))
+    ties = np.array([[[1.00390625, 1.01171875, -1.00390625, 3.0e38]]], np.float32)
+    assert orc.combine(orc.COMBINE_BF16_STEPS, None, None, ties).tolist() == [[1.0, 1.015625, -1.0, float(bf16(np.float32(3.0e38)))]]
+    nan = np.array([[[0]]], np.uint32); nan[0, 0, 0] = 0x7fc12345
+    assert bits(orc.combine(orc.COMBINE_BF16_STEPS, None, None, nan.view(np.float32)))[0, 0] == 0x7fc12345
+    small = rng.integers(-7, 8, (3, 16, 40)).astype(np.float32)               # every partial sum is an integer of <= 8 bits
+    ones = np.ones((3, 16), np.float32)
+    base = rng.integers(-7, 8, (3, 40)).astype(np.float32)
+    assert np.array_equal(orc.combine(orc.COMBINE_BF16_STEPS, ones, None, small, base), small.sum(axis=1) + base)
+    # a weight enters as bf16(e * w), not as an fma: 3 * (1 + 2^-7) = 3.0234375 is a tie and rounds to 3.03125 before it is added
+    # to 256 (259.03125 -> 260 in bfloat16, whose steps are 2 there); the fma form keeps 259.0234375
+    e2 = np.array([[[256.0], [3.0]]], np.float32)
+    w2 = np.array([[1.0, 1.0078125]], np.float32)
+    assert orc.combine(orc.COMBINE_BF16_STEPS, w2, None, e2)[0, 0] == 260.0
+    assert orc.combine(orc.COMBINE_FMA_SLOT, w2, None, e2, np.zeros((1, 1), np.float32))[0, 0] == 259.0234375
 
 
 def test_vector_form_of_the_q4k_row_equals_the_plain_loop():
