@@ -16,6 +16,9 @@
 //                                                                                     include/strix/hip_moe_a8_down.hpp:11-30
 //   qwen_moe::Strided / Rows / Weights, enqueue_prologue .. enqueue_commit, enqueue   include/strix/cuda/qwen_moe.hpp:34-110
 //   expert::LayerWeights / RowA8 / Assignment / Job / Executor                        src/cpu/core/routed_expert.hpp:28-95
+//   moe_q4k_a8::enqueue_serial_prologue_probe, enqueue_quantize_only                  include/strix/hip_moe_q4k_a8_probe.hpp:20-24
+//   moe::CombineForm, moe_core::enqueue_combine, enqueue_combine_rounded_eo           include/strix/moe/combine.hpp:13,
+//                                                                                     src/moe_core/route_wave_kernel.hpp:138-160
 //   moe_route::enqueue                                                                the policy of include/strix/moe_core/route_policy.hpp
 // Admission failures throw std::invalid_argument before anything is enqueued, HIP failures throw std::runtime_error, as the
 // reference's check / hip_check do. Nothing here allocates (Executor's constructor aside) or synchronises.
@@ -243,6 +246,21 @@ inline void enqueue_probe(const Request& request, const Bindings& bindings, mi35
     check(mi355_a8_enqueue_probe(&q.q, &b, stream));
 }
 
+// include/strix/hip_moe_q4k_a8_probe.hpp:20-23: the serial row's clear + route / route-weight check + quantiser in one workgroup,
+// status overwritten, then the projection
+inline void enqueue_serial_prologue_probe(const Request& request, const Bindings& bindings, float* clear, unsigned clear_words,
+                                          const float* route_weights, mi355_stream stream) {
+    detail::CRequest q; detail::fill(request, q);
+    const mi355_a8_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_serial_prologue_probe(&q.q, &b, clear, clear_words, route_weights, stream));
+}
+// include/strix/hip_moe_q4k_a8_probe.hpp:24: route check + quantiser, no projection
+inline void enqueue_quantize_only(const Request& request, const Bindings& bindings, mi355_stream stream) {
+    detail::CRequest q; detail::fill(request, q);
+    const mi355_a8_bindings b = detail::c(bindings);
+    check(mi355_a8_enqueue_quantize_only(&q.q, &b, stream));
+}
+
 // Union rows form (include/strix/moe_q4k_a8_contract.hpp:123-132, src/hip_moe_q4k_a8_probe.hip:1172-1191): shape.logical_rows = R
 // (1..8); the per-row views are R contiguous single-row extents; plan = moe::expert_union::plan_bytes, written by the probe.
 inline void validate_union(const Request& request, const Bindings& bindings, DeviceBytes plan) {
@@ -458,6 +476,26 @@ private:
     void* handle_;
 };
 }  // namespace expert
+
+// ---------------------------------------------------------------------------------------------- combine
+// include/strix/moe/combine.hpp:13 (CombineForm) and src/moe_core/route_wave_kernel.hpp:138-160 (enqueue_combine,
+// enqueue_combine_rounded_eo); TopK and Width are template arguments there and stay so here.
+namespace moe {
+enum class CombineForm : std::uint8_t { fma_f32, bf16_steps };
+}
+namespace moe_core {
+template <moe::CombineForm Form, unsigned TopK, unsigned Width>
+void enqueue_combine(const float* w, const float* eo, const float* shared, float* y, unsigned rows, mi355_stream stream) {
+    if (Form == moe::CombineForm::fma_f32 && (w == nullptr || shared == nullptr)) throw std::invalid_argument("moe combine: fma_f32 needs w and shared");
+    check(mi355_moe_enqueue_combine(Form == moe::CombineForm::fma_f32 ? MI355_COMBINE_FMA_SLOT_ORDER : MI355_COMBINE_BF16_STEPS, rows, TopK, Width, w, eo,
+                                    shared, y, 0U, stream));
+}
+template <moe::CombineForm Form, unsigned TopK, unsigned Width>
+void enqueue_combine_rounded_eo(const float* w, const float* eo, const float* shared, float* y, unsigned rows, mi355_stream stream) {
+    static_assert(Form == moe::CombineForm::bf16_steps, "moe combine: RoundEo is bound for bf16_steps only");
+    check(mi355_moe_enqueue_combine(MI355_COMBINE_BF16_STEPS, rows, TopK, Width, w, eo, shared, y, 1U, stream));
+}
+}  // namespace moe_core
 
 // ---------------------------------------------------------------------------------------------- router
 namespace moe_route {

@@ -196,6 +196,100 @@ static void a8_single_row(const Layer& L) {
     expect(threw, "moe_q4k_a8::enqueue_probe throws std::invalid_argument without the identity approval");
 }
 
+// The serial row's fused prologue, the quantiser alone, and the alignment rule of the down weights.
+static void a8_serial_forms(const Layer& L) {
+    namespace a8 = m::moe_q4k_a8;
+    const Layer::Result ref = L.oracle(L.down, 12);
+    Dev<std::uint8_t> gate(L.gate), up(L.up);
+    Dev<std::uint16_t> input(std::vector<std::uint16_t>(L.x.begin(), L.x.begin() + H));
+    Dev<std::uint32_t> routes(std::vector<std::uint32_t>(L.routes.begin(), L.routes.begin() + K)), status(std::vector<std::uint32_t>{0xabcdU});
+    Dev<std::int8_t> codes(H);
+    Dev<float> deltas(H / 32), output(K * 2 * I), clear(std::vector<float>(H + 3, 5.0F)), route_w(std::vector<float>(L.weights.begin(), L.weights.begin() + K));
+    Dev<std::int32_t> sums(H / 32);
+    a8::Request q;
+    q.enabled = true; q.approved_numerical_identity = a8::numerical_identity_for_gate_type(12); q.input = a8::InputKind::bf16;
+    q.shape = a8::Shape{H, I, E, K, 1};
+    const a8::Bindings b{input.bytes(), gate.bytes(), up.bytes(), routes.bytes(), codes.bytes(), deltas.bytes(), sums.bytes(), status.bytes(), output.bytes()};
+    a8::enqueue_serial_prologue_probe(q, b, clear.p, H, route_w.p, nullptr);
+    const std::vector<float> out = output.get(), cleared = clear.get();
+    bool ok = status.get()[0] == 0;                                       // the stale word is overwritten
+    for (std::uint32_t i = 0; i < H + 3; ++i) ok = ok && cleared[i] == (i < H ? 0.0F : 5.0F);
+    ok = ok && same_bits(codes.get(), std::vector<std::int8_t>(L.c.begin(), L.c.begin() + H)) && same_bits(deltas.get(), std::vector<float>(L.d.begin(), L.d.begin() + H / 32));
+    for (std::uint32_t k = 0; k < K; ++k)
+        ok = ok && std::memcmp(out.data() + (k * 2) * I, ref.gate.data() + k * I, I * 4) == 0 && std::memcmp(out.data() + (k * 2 + 1) * I, ref.up.data() + k * I, I * 4) == 0;
+    expect(ok, "moe_q4k_a8::enqueue_serial_prologue_probe: cleared words, overwritten status, image and gate / up rows == oracle");
+    // a non-finite route weight: bit 1, nothing stored
+    Dev<float> bad_w(std::vector<float>{0.5F, INFINITY});
+    Dev<std::int8_t> codes2(std::vector<std::int8_t>(H, 77));
+    Dev<float> output2(std::vector<float>(K * 2 * I, -7.0F));
+    const a8::Bindings b2{input.bytes(), gate.bytes(), up.bytes(), routes.bytes(), codes2.bytes(), deltas.bytes(), sums.bytes(), status.bytes(), output2.bytes()};
+    a8::enqueue_serial_prologue_probe(q, b2, clear.p, H, bad_w.p, nullptr);
+    expect(status.get()[0] == a8::invalid_route && codes2.get() == std::vector<std::int8_t>(H, 77) && output2.get() == std::vector<float>(K * 2 * I, -7.0F),
+           "moe_q4k_a8::enqueue_serial_prologue_probe: a non-finite route weight sets bit 1 and stores neither image nor rows");
+    Dev<std::uint32_t> status3(1);
+    const a8::Bindings b3{input.bytes(), gate.bytes(), up.bytes(), routes.bytes(), codes2.bytes(), deltas.bytes(), sums.bytes(), status3.bytes(), output2.bytes()};
+    a8::enqueue_quantize_only(q, b3, nullptr);
+    expect(status3.get()[0] == 0 && same_bits(codes2.get(), std::vector<std::int8_t>(L.c.begin(), L.c.begin() + H)) && output2.get() == std::vector<float>(K * 2 * I, -7.0F),
+           "moe_q4k_a8::enqueue_quantize_only: the image == oracle, no projection");
+    // the down weights: this library asks 16 bytes of every class; a Q8_0 tensor on 2 bytes, which the reference admits
+    // (src/moe_a8_down_contract.cpp:72-73), is refused by name
+    Dev<std::uint8_t> down8(std::vector<std::uint8_t>(L.down8.size() + 16));
+    Dev<std::int8_t> hcodes(K * I);
+    Dev<float> hdeltas(K * I / 32), rawdots(K * H);
+    Dev<std::int32_t> hsums(K * I / 32);
+    Dev<std::uint32_t> dstatus(1), aggregate(1);
+    a8::DownRequest dq;
+    dq.enabled = true; dq.approved_numerical_identity = a8::down_numerical_identity(8); dq.shape = a8::DownShape{H, I, E, K}; dq.weight_type = 8;
+    a8::DownBindings db{output.bytes(), a8::DeviceBytes{reinterpret_cast<std::uintptr_t>(down8.p), L.down8.size()}, routes.bytes(), hcodes.bytes(), hdeltas.bytes(),
+                        hsums.bytes(), rawdots.bytes(), dstatus.bytes(), aggregate.bytes()};
+    bool admitted = true, refused = false;
+    try { a8::validate_down(dq, db); } catch (const std::invalid_argument&) { admitted = false; }
+    db.weights.address += 2;
+    try { a8::validate_down(dq, db); } catch (const std::invalid_argument& e) { refused = std::strstr(e.what(), "alignment") != nullptr; }
+    expect(admitted && refused, "moe_q4k_a8::validate_down: a Q8_0 weight tensor on 16 bytes is admitted, on 2 bytes refused with the alignment rule");
+}
+
+// moe_core::enqueue_combine in both forms (the reference's two bf16-steps shapes, tests/hip_hy4_routed_tests.hip:205-206).
+static void combine_forms() {
+    namespace mc = m::moe_core;
+    using m::moe::CombineForm;
+    constexpr unsigned R = 5;
+    const auto bf16_values = [](std::vector<float> v) { for (float& x : v) x = bf16_value(bf16_rne(x)); return v; };
+    {
+        const std::vector<float> eo = bf16_values(normal(size_t(R) * 16 * 1536, 1.0F)), w = normal(R * 16, 0.3F);
+        Dev<float> deo(eo), dw(w), y(R * 1536), y2(R * 1536);
+        std::vector<float> want(R * 1536), want2(R * 1536);
+        mc::enqueue_combine<CombineForm::bf16_steps, 16, 1536>(dw.p, deo.p, nullptr, y.p, R, nullptr);
+        orc_combine(ORC_COMBINE_BF16_STEPS, R, 16, 1536, w.data(), nullptr, eo.data(), nullptr, want.data());
+        expect(same_bits(y.get(), want), "moe_core::enqueue_combine<bf16_steps, 16, 1536> (latent merge, no base) == oracle");
+        const std::vector<float> raw = normal(size_t(R) * 16 * 1536, 1.0F);
+        Dev<float> draw(raw);
+        mc::enqueue_combine_rounded_eo<CombineForm::bf16_steps, 16, 1536>(dw.p, draw.p, nullptr, y2.p, R, nullptr);
+        orc_combine(ORC_COMBINE_BF16_STEPS_ROUNDED_EO, R, 16, 1536, w.data(), nullptr, raw.data(), nullptr, want2.data());
+        expect(same_bits(y2.get(), want2), "moe_core::enqueue_combine_rounded_eo<bf16_steps, 16, 1536> == oracle");
+    }
+    {
+        const std::vector<float> eo = bf16_values(normal(size_t(R) * 3072, 1.0F)), sh = bf16_values(normal(size_t(R) * 3072, 1.0F));
+        Dev<float> deo(eo), dsh(sh), y(R * 3072);
+        std::vector<float> want(R * 3072);
+        mc::enqueue_combine<CombineForm::bf16_steps, 1, 3072>(nullptr, deo.p, dsh.p, y.p, R, nullptr);
+        orc_combine(ORC_COMBINE_BF16_STEPS, R, 1, 3072, nullptr, nullptr, eo.data(), sh.data(), want.data());
+        expect(same_bits(y.get(), want), "moe_core::enqueue_combine<bf16_steps, 1, 3072> (unit weights, shared add) == oracle");
+    }
+    {
+        const std::vector<float> eo = normal(size_t(R) * 8 * 4096, 1.0F), w = normal(R * 8, 0.3F), sh = normal(size_t(R) * 4096, 1.0F);
+        Dev<float> deo(eo), dw(w), dsh(sh), y(R * 4096);
+        std::vector<float> want(R * 4096);
+        const std::vector<std::uint32_t> ids(R * 8, 0U);
+        mc::enqueue_combine<CombineForm::fma_f32, 8, 4096>(dw.p, deo.p, dsh.p, y.p, R, nullptr);
+        orc_combine(ORC_COMBINE_FMA_SLOT_ORDER, R, 8, 4096, w.data(), ids.data(), eo.data(), sh.data(), want.data());
+        expect(same_bits(y.get(), want), "moe_core::enqueue_combine<fma_f32, 8, 4096> (with the shared base) == oracle");
+        bool threw = false;
+        try { mc::enqueue_combine<CombineForm::fma_f32, 8, 4096>(dw.p, deo.p, nullptr, y.p, R, nullptr); } catch (const std::invalid_argument&) { threw = true; }
+        expect(threw, "moe_core::enqueue_combine<fma_f32> throws std::invalid_argument without the shared base");
+    }
+}
+
 // The union rows form: three rows, each naming all four experts in its own order, so every entry is held by every row.
 static void a8_union_rows(const Layer& L) {
     namespace a8 = m::moe_q4k_a8;
@@ -342,6 +436,8 @@ int main() {
         kernel_table();
         const Layer L;
         a8_single_row(L);
+        a8_serial_forms(L);
+        combine_forms();
         a8_union_rows(L);
         strided_rows(L);
         executor_job(L);
