@@ -135,6 +135,12 @@ typedef struct mi355_route_policy {
     uint32_t shared_experts;          /* 0..4 always-on experts behind the routed ones: ids / weights rows are then
                                          [top_k + shared_experts] wide, slot top_k + s holds expert id experts + s with weight 1
                                          (the shared expert of a layer stored as one more expert of the same tensors) */
+    const float* shared_slot_weights; /* NULL, or device fp32 [rows][shared_experts]: the weight of each always-on slot in the place of 1 -
+                                         the shared expert's sigmoid gate (mi355_shared_gate). An always-on slot enters the ordered
+                                         combine as acc + (weight * value), product and sum rounded separately: the reference scales
+                                         the shared expert's output by its gate (one multiply, src/hip_shared_expert_launcher.hip:727,
+                                         :779) and adds that row to the routed sum (include/strix/moe/combine.hpp:56); with weight 1
+                                         this is acc + value */
 } mi355_route_policy;
 /* x: [rows] activations (input_kind), row r at x + r * x_stride_bytes. router_weight: fp32 [experts][hidden].
  * logit_bias: fp32 [experts] or NULL. ids / weights: [rows][top_k + shared_experts]. scores: [rows][experts] workspace AND output. */
@@ -258,6 +264,15 @@ int32_t mi355_moe_enqueue_layer_back(const mi355_route_policy* policy, const flo
  * are the exact router's either way. amount != 0 displaces the early logits (by amount * 1e-3 * a per-expert integer in
  * -8..7) so that a test can make the choices differ; 0 (the default) restores them. Process-wide; not for production use. */
 void mi355_debug_early_route_perturb(uint32_t amount);
+
+/* The scalar gate of an always-on shared expert (tensor ffn_gate_inp_shexp, fp32 [hidden]): gate[row * gate_stride] =
+ * 1 / (1 + exp(-dot(x[row], scalar_weight))), the reference's shared_gate_dot (src/hip_shared_expert_launcher.hip:624-645): 256
+ * thread-strided fma chains (thread t takes features t, t + 256, ... in ascending order), the 256-leaf halving tree
+ * s[l] + s[l + h], h = 128 .. 1 (src/core/ordered_reduce.hpp:8-16), the device expf (exp_kind MI355_EXP_GFX1151 is the
+ * reference's) and a correctly rounded division. x: rows of input_kind, row r at x + r * x_stride_bytes. gate_stride in floats:
+ * [rows][shared_experts] for the policy's shared_slot_weights, or 1 for the route weights of a top-1 shared-expert layer call. */
+int32_t mi355_shared_gate(const void* x, uint32_t input_kind, uint32_t rows, uint32_t hidden, uint64_t x_stride_bytes,
+                          const float* scalar_weight, uint32_t exp_kind, float* gate, uint64_t gate_stride, mi355_stream);
 
 /* The layer with the RMSNorm of its input inside the first launch (the reference normalises the residual stream in front of
  * the MoE, src/ops/norm/norm.hpp:40-58, and runs the shared expert beside the routed ones, src/hip_shared_expert_launcher.hip):

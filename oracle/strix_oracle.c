@@ -697,6 +697,38 @@ void orc_combine(int form, uint32_t rows, uint32_t top_k, uint32_t width, const 
     }
 }
 
+void orc_combine_shared(int form, uint32_t rows, uint32_t top_k, uint32_t shared_slots, uint32_t width, const float* w, const uint32_t* ids,
+                        const float* raw, const float* base, float* y) {
+    const uint32_t routed = top_k - shared_slots;
+    for (uint32_t r = 0; r < rows; ++r) {
+        /* the routed slots in the form's order (the always-on ids are the largest, so they are last in both orders) */
+        orc_combine(form, 1, routed, width, w + (size_t)r * top_k, ids + (size_t)r * top_k, raw + (size_t)r * top_k * width, NULL, y + (size_t)r * width);
+        for (uint32_t d = 0; d < width; ++d) {
+            float acc = y[(size_t)r * width + d];
+            for (uint32_t k = routed; k < top_k; ++k) {
+                const float product = w[(size_t)r * top_k + k] * raw[((size_t)r * top_k + k) * width + d];
+                acc = acc + product;
+            }
+            y[(size_t)r * width + d] = base ? acc + base[(size_t)r * width + d] : acc;
+        }
+    }
+}
+
+void orc_shared_gate(const float* x, const float* w, uint32_t rows, uint32_t hidden, int exp_kind, float* gate, float* dots) {
+    for (uint32_t r = 0; r < rows; ++r) {
+        float s[256];
+        for (uint32_t t = 0; t < 256; ++t) {                  /* src/hip_shared_expert_launcher.hip:629-632 */
+            float sum = 0.0F;
+            for (uint32_t f = t; f < hidden; f += 256) sum = fmaf(x[(size_t)r * hidden + f], w[f], sum);
+            s[t] = sum;
+        }
+        for (uint32_t h = 128; h >= 1; h >>= 1)                /* src/core/ordered_reduce.hpp:8-9 */
+            for (uint32_t l = 0; l < h; ++l) s[l] = s[l] + s[l + h];
+        if (dots) dots[r] = s[0];
+        gate[r] = 1.0F / (1.0F + exp_of(exp_kind, -s[0]));      /* :635 */
+    }
+}
+
 /* ------------------------------------------------------------------ routed experts */
 static const uint8_t* gate_row_ptr(const orc_expert_weights* w, const uint8_t* base, uint32_t expert, uint32_t o) {
     return base + (size_t)expert * w->gate_expert_stride + (size_t)o * w->gate_row_stride;

@@ -134,6 +134,20 @@ void orc_route_select(const orc_route_policy* p, const float* scores, uint32_t* 
 void orc_combine(int form, uint32_t rows, uint32_t top_k, uint32_t width, const float* w, const uint32_t* ids,
                  const float* raw, const float* base, float* y);
 
+/* The ordered combine of a layer whose last `shared_slots` slots are always-on experts: those enter as acc + (w * value), product
+ * and sum rounded separately, in both forms (the gate scales the shared expert's output with one multiply,
+ * src/hip_shared_expert_launcher.hip:727,779; the sum with the routed row is one add, include/strix/moe/combine.hpp:56). */
+void orc_combine_shared(int form, uint32_t rows, uint32_t top_k, uint32_t shared_slots, uint32_t width, const float* w, const uint32_t* ids,
+                        const float* raw, const float* base, float* y);
+
+/* ---- the shared expert's scalar gate (src/hip_shared_expert_launcher.hip:624-645 shared_gate_dot; tree src/core/ordered_reduce.hpp:8-16)
+ * x [rows][hidden] fp32 values of the stored activations, w [hidden]; gate [rows] = 1 / (1 + exp(-dot)):
+ * 256 thread-strided fma chains (thread t: features t, t + 256, ... ascending; the reference's build fuses `sum += x * w`, its
+ * target sets no contraction flag), halving tree s[l] = s[l] + s[l + h] for h = 128 .. 1, exp of the given kind, one division.
+ * Parity: the device header cannot be compiled into oracle/_ref; pinned by order fixtures (tests/test_oracle_golden.py) that a
+ * sequential or adjacent-pair reduction, or an unfused multiply-add, changes. dots: optional [rows], the value before the sigmoid. */
+void orc_shared_gate(const float* x, const float* w, uint32_t rows, uint32_t hidden, int exp_kind, float* gate, float* dots);
+
 /* ---- routed expert layer (src/cpu/core/routed_expert.cpp:264-300 generalised to Q4_K / Q8_0 down) - */
 typedef struct {
     uint32_t hidden, ffn, experts, top_k;   /* ffn = intermediate rows computed here (rank-local for a TP shard) */

@@ -36,7 +36,8 @@ class Q8a8View(C.Structure):
 class RoutePolicy(C.Structure):
     _fields_ = [("experts", C.c_uint32), ("top_k", C.c_uint32), ("logits_order", C.c_uint32),
                 ("renorm_eps", C.c_float), ("scale", C.c_float), ("renormalize", C.c_uint32),
-                ("renorm_single", C.c_uint32), ("exp_kind", C.c_uint32), ("shared_experts", C.c_uint32)]
+                ("renorm_single", C.c_uint32), ("exp_kind", C.c_uint32), ("shared_experts", C.c_uint32),
+                ("shared_slot_weights", C.c_void_p)]
 
 
 class MoeWeights(C.Structure):
@@ -255,7 +256,7 @@ EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi3
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
            "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue_combine", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
-           "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe", "mi355_a8_enqueue_serial_prologue_probe", "mi355_a8_enqueue_quantize_only",
+           "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_shared_gate", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe", "mi355_a8_enqueue_serial_prologue_probe", "mi355_a8_enqueue_quantize_only",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
            "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
            "mi355_a8_enqueue_down_activation_quantize_union", "mi355_a8_enqueue_down_rawdots_union",
@@ -330,6 +331,16 @@ def rmsnorm_f32(x, weight=None, eps=1e-6):
     return y
 
 
+def shared_gate(x, scalar_weight, exp_kind=EXP_GFX1151, out=None):
+    """gate[row] = sigmoid(dot(x[row], scalar_weight)) as the reference's shared-expert launcher computes it (mi355_shared_gate)."""
+    rows, hidden = x.shape
+    if out is None:
+        out = torch.zeros((rows, 1), dtype=torch.float32, device=x.device)
+    check(lib().mi355_shared_gate(_p(x), input_kind(x), rows, hidden, C.c_uint64(x.stride(0) * x.element_size()), _p(scalar_weight), exp_kind,
+                                  _p(out), C.c_uint64(out.stride(0)), _stream()))
+    return out
+
+
 def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False, row_bytes_=None, out_stride=None):
     rows = codes.shape[0]
     if out is None:
@@ -341,10 +352,11 @@ def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False,
 
 
 def route(x, router_weight, top_k, bias=None, logits_order=LOGITS_FMA, renorm_eps=0.0, scale=1.0, renormalize=True, renorm_single=True,
-          exp_kind=EXP_DECLARED, shared_experts=0):
+          exp_kind=EXP_DECLARED, shared_experts=0, shared_slot_weights=None):
     rows, hidden = x.shape
     experts = router_weight.shape[0]
-    p = RoutePolicy(experts, top_k, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single), exp_kind, shared_experts)
+    p = RoutePolicy(experts, top_k, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single), exp_kind, shared_experts,
+                    None if shared_slot_weights is None else shared_slot_weights.data_ptr())
     ids = torch.empty((rows, top_k + shared_experts), dtype=torch.int32, device=x.device)
     weights = torch.empty((rows, top_k + shared_experts), dtype=torch.float32, device=x.device)
     scores = torch.empty((rows, experts), dtype=torch.float32, device=x.device)
@@ -535,9 +547,10 @@ class MoeLayer:
         return self.output[:rows]
 
     def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,
-                  scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED, shared_experts=0, norm=None, half=None):
+                  scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED, shared_experts=0, norm=None, half=None, shared_slot_weights=None):
         """Router + experts + combine through mi355_moe_enqueue_layer. Returns (output, ids, weights, scores).
-        shared_experts: the last `shared_experts` experts of the tensors are always on (the router picks among the others).
+        shared_experts: the last `shared_experts` experts of the tensors are always on (the router picks among the others);
+        shared_slot_weights [rows][shared_experts]: their weights in the place of 1 (the sigmoid gate of shared_gate()).
         norm: (weight or None, eps) - the RMSNorm of x runs inside the first launch (mi355_moe_enqueue_layer_normed); the
         normalised rows are left in self.normed."""
         rows = x.shape[0]
@@ -549,7 +562,7 @@ class MoeLayer:
             self.scores = torch.zeros((self.max_rows, self.experts), dtype=torch.float32, device=x.device)
         _, rv = self.rows_view(x, self.ids, self.route_w, base)
         p = RoutePolicy(self.experts - shared_experts, self.top_k - shared_experts, logits_order, renorm_eps, scale, int(renormalize), int(renorm_single),
-                        exp_kind, shared_experts)
+                        exp_kind, shared_experts, None if shared_slot_weights is None else shared_slot_weights.data_ptr())
         if norm is None:
             # half: "front" / "back" = the layer's two halves as calls of their own (mi355_moe_enqueue_layer_front / _back)
             entry = lib().mi355_moe_enqueue_layer if half is None else getattr(lib(), "mi355_moe_enqueue_layer_" + half)

@@ -92,6 +92,9 @@ struct RowsK : mi355_moe_rows {
     const uint32_t* union_plan;     // verify-window form: the expert-union plan (below) names the items instead of `plan`
     uint32_t top1_form;       // a dense top-1 job whose down launch also publishes the output: combine form + 1 (0: the merge launch does)
     uint32_t* aggregate;      // optional summary word of the A8 down bindings (include/strix/moe_a8_down_contract.hpp:50-52): bit 16 beside a row's flag
+    uint32_t shared_slots;    // the last shared_slots slots of a row are always-on experts: they enter the ordered combine as
+                              // acc + (weight * value) in both forms (the gate scales the shared expert's output with one multiply,
+                              // src/hip_shared_expert_launcher.hip:727; the sum with the routed row is one add, include/strix/moe/combine.hpp:56)
     uint32_t clean_only;      // probe form: nothing is computed or stored once the shared status word is set ("this kernel never changes
                               // status" and returns on a set one, src/hip_moe_q4k_a8_probe.hip:224-225,257-258)
     uint32_t* awords;         // a decode batch planned from early routes: one word per assignment (finished projection waves in the low

@@ -583,10 +583,10 @@ __device__ __forceinline__ uint32_t route_select_row_per(float* p_lds, const Rou
         store_shared_or_plain(shared_out, a.ids + static_cast<size_t>(row) * P + lane, my_id);
         const bool renorm = a.p.renormalize && (K > 1U || a.p.renorm_single);      // include/strix/moe/route_policy.hpp:146
         store_shared_or_plain(shared_out, a.weights + static_cast<size_t>(row) * P + lane, (renorm ? my_v / den : my_v) * a.p.scale);
-    } else if (lane < P) {      // the always-on experts behind the routed ones: ids experts .. experts + shared - 1, weight 1
+    } else if (lane < P) {      // the always-on experts behind the routed ones: ids experts .. experts + shared - 1, weight 1 or the given gate
         my_id = E + (lane - K);
         a.ids[static_cast<size_t>(row) * P + lane] = my_id;
-        a.weights[static_cast<size_t>(row) * P + lane] = 1.0F;
+        a.weights[static_cast<size_t>(row) * P + lane] = a.p.shared_slot_weights ? a.p.shared_slot_weights[static_cast<size_t>(row) * a.p.shared_experts + (lane - K)] : 1.0F;
     }
     __syncthreads();
     return my_id;

@@ -1114,7 +1114,7 @@ __global__ __launch_bounds__(256) void merge_kernel(mi355_moe_weights w, RowsK r
         for (uint32_t k = 0; k < 16U; ++k) {
             if (k >= w.top_k) continue;
             const float v = e[k][c];
-            if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], v, acc);
+            if (form == MI355_COMBINE_FMA_SLOT_ORDER && k + r.shared_slots < w.top_k) acc = __builtin_fmaf(slot_weight[k], v, acc);
             else acc = acc + slot_weight[k] * v;
         }
         const float out = r.base ? acc + r.base_of(row)[o + c] : acc;
@@ -1198,7 +1198,7 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
     float acc = 0.0F;
     for (uint32_t k = 0; k < w.top_k; ++k) {
         const float ev = slot_value[slot_order[k]][lane];
-        if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], ev, acc);
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER && k + r.shared_slots < w.top_k) acc = __builtin_fmaf(slot_weight[k], ev, acc);
         else acc = acc + slot_weight[k] * ev;
     }
     const float y = r.base ? acc + r.base_of(row)[o] : acc;
@@ -1254,7 +1254,7 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_quad_kernel(m
     float acc = 0.0F;
     for (uint32_t k = 0; k < w.top_k; ++k) {
         const float ev = slot_value[slot_order[k]][lane];
-        if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], ev, acc);
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER && k + r.shared_slots < w.top_k) acc = __builtin_fmaf(slot_weight[k], ev, acc);
         else acc = acc + slot_weight[k] * ev;
     }
     const uint32_t o = o0 + lane;
@@ -1374,7 +1374,7 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_q51_kernel(mi
     float sum = 0.0F;
     for (uint32_t k = 0; k < w.top_k; ++k) {
         const float ev = slot_value[slot_order[k]][lane];
-        if (form == MI355_COMBINE_FMA_SLOT_ORDER) sum = __builtin_fmaf(slot_weight[k], ev, sum);
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER && k + r.shared_slots < w.top_k) sum = __builtin_fmaf(slot_weight[k], ev, sum);
         else sum = sum + slot_weight[k] * ev;
     }
     const uint32_t oc = blockIdx.x * 16U + lane;
@@ -1461,7 +1461,7 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_q6k_kernel(mi
     float sum = 0.0F;
     for (uint32_t k = 0; k < w.top_k; ++k) {
         const float ev = slot_value[slot_order[k]][lane];
-        if (form == MI355_COMBINE_FMA_SLOT_ORDER) sum = __builtin_fmaf(slot_weight[k], ev, sum);
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER && k + r.shared_slots < w.top_k) sum = __builtin_fmaf(slot_weight[k], ev, sum);
         else sum = sum + slot_weight[k] * ev;
     }
     const uint32_t oc = blockIdx.x * 16U + lane;
@@ -1526,7 +1526,7 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_q8_0_kernel(m
     float acc = 0.0F;
     for (uint32_t k = 0; k < w.top_k; ++k) {
         const float ev = slot_value[slot_order[k]][lane];
-        if (form == MI355_COMBINE_FMA_SLOT_ORDER) acc = __builtin_fmaf(slot_weight[k], ev, acc);
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER && k + r.shared_slots < w.top_k) acc = __builtin_fmaf(slot_weight[k], ev, acc);
         else acc = acc + slot_weight[k] * ev;
     }
     const uint32_t oc = blockIdx.x * 16U + lane;
@@ -2118,12 +2118,16 @@ int32_t mi355_moe_enqueue_down(const mi355_moe_weights* w, const mi355_moe_rows*
     return MI355_OK;
 }
 
-int32_t mi355_moe_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+}  // extern "C"
+namespace {
+// shared_slots: the last slots of every row are always-on experts (a layer call with policy->shared_experts)
+int32_t enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream, uint32_t shared_slots) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv, kAnyClass)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe merge: unknown combine form");
     STRIX_REQUIRE(rows <= 65535U, "moe merge: at most 65535 rows per call");
-    const RowsK k = rows_k(*r, wv);
+    RowsK k = rows_k(*r, wv);
+    k.shared_slots = shared_slots;
     // four columns per thread once that still leaves every compute unit several workgroups (4096 rows x 4096: 194 -> 113 us;
     // a decode batch is faster with one column per thread: 16 rows x 6144: 8.5 against 10.9 us)
     const bool quads = static_cast<uint64_t>(rows) * ((wv.hidden + 1023U) / 1024U) >= 4ULL * compute_units() && wv.hidden % 4U == 0 && aligned(k.rawdots, 16) && k.rawdots_rs % 16U == 0 && aligned(k.output, 16) && k.output_stride % 4U == 0 &&
@@ -2132,6 +2136,12 @@ int32_t mi355_moe_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows
     else merge_kernel<1><<<dim3((wv.hidden + 255U) / 256U, rows), 256, 0, hs(stream)>>>(wv, k, form);
     STRIX_LAUNCHED("moe merge");
     return MI355_OK;
+}
+}  // namespace
+extern "C" {
+
+int32_t mi355_moe_enqueue_merge(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    return enqueue_merge(w, r, rows, form, stream, 0U);
 }
 
 int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
@@ -2157,7 +2167,8 @@ int32_t mi355_moe_enqueue(const mi355_moe_weights* w, const mi355_moe_rows* r, u
 
 namespace {
 // mi355_moe_enqueue by halves: front = prologue, plan, gate / up; back = down rows, combine.
-int32_t enqueue_staged(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream, bool do_front, bool do_back) {
+int32_t enqueue_staged(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream, bool do_front, bool do_back,
+                       uint32_t shared_slots = 0) {
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
@@ -2174,7 +2185,7 @@ int32_t enqueue_staged(const mi355_moe_weights* w, const mi355_moe_rows* r, uint
     const bool published = launch_down(wv, k, rows, item_bound(wv, rows), hs(stream));
     STRIX_LAUNCHED("moe down");
     if (published) return MI355_OK;
-    return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+    return enqueue_merge(w, r, rows, form, stream, shared_slots);
 }
 
 // RMSNorm of rows of any input kind into fp32 rows (the staged form of the fused norm): rmsnorm_f32_kernel's order.
@@ -2201,6 +2212,7 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     const bool do_front = phase != kLayerBack, do_back = phase != kLayerFront;
     mi355_moe_weights wv;
     if (const int32_t rc = check_moe(w, r, rows, wv)) return rc;
+    const auto layer_rows = [&] { RowsK k = rows_k(*r, wv); k.shared_slots = p->shared_experts; return k; };
     STRIX_REQUIRE(form <= MI355_COMBINE_MULADD_ASCENDING_EXPERT, "moe: unknown combine form");
     STRIX_REQUIRE(r->input && r->input_kind <= MI355_INPUT_BF16, "moe: input view invalid");
     uint32_t* ids = const_cast<uint32_t*>(r->routes);
@@ -2223,8 +2235,7 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
         if (norm.on) { staged.input = norm.normed; staged.input_kind = MI355_INPUT_F32; staged.input_stride = 4ULL * wv.hidden; }
         if (do_front)
             if (const int32_t rc = mi355_moe_route(p, staged.input, staged.input_kind, rows, wv.hidden, staged.input_stride, router_weight, logit_bias, ids, weights, scores, stream)) return rc;
-        if (phase == kLayerWhole) return mi355_moe_enqueue(w, &staged, rows, form, stream);
-        return enqueue_staged(w, &staged, rows, form, stream, do_front, do_back);
+        return enqueue_staged(w, &staged, rows, form, stream, do_front, do_back, p->shared_experts);
     }
     RouteArgs a{};
     a.p = *p; a.x = static_cast<const uint8_t*>(r->input); a.kind = r->input_kind; a.x_stride = r->input_stride; a.rows = rows; a.hidden = wv.hidden;
@@ -2243,7 +2254,7 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
         a.early_perturb = g_early_perturb.load(std::memory_order_relaxed);
         // the early logits of row i live in the row's (still unused) unweighted-output block: the exact logits own `scores`
         a.early_logits = r->rawdots; a.early_stride = wv.top_k * wv.hidden;
-        RowsK k = rows_k(*r, wv);
+        RowsK k = layer_rows();
         k.awords = a.awords;
         RowsK front = k;
         front.plan = nullptr;              // (the front launch names its assignments itself: the work items are written inside it)
@@ -2268,51 +2279,51 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     // the fused router planned one item per routed assignment (and one per four rows of an always-on expert)
     if (p->shared_experts) {       // items of several rows: the 64-row sweeps
         if (do_front) {
-            launch_project(wv, rows_k(*r, wv), rows, items, st, true);
+            launch_project(wv, layer_rows(), rows, items, st, true);
             STRIX_LAUNCHED("moe layer gate / up");
         }
         if (!do_back) return MI355_OK;
-        launch_down(wv, rows_k(*r, wv), rows, items, st, true);
+        launch_down(wv, layer_rows(), rows, items, st, true);
         STRIX_LAUNCHED("moe layer experts");
-        return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+        return enqueue_merge(w, r, rows, form, stream, p->shared_experts);
     }
-    if (do_front) launch_project(wv, rows_k(*r, wv), rows, items, st);
+    if (do_front) launch_project(wv, layer_rows(), rows, items, st);
     if (!do_back) return MI355_OK;
     // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
     // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
     // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
     if (!quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
         (wv.hidden / 64U) * rows <= compute_units()) {
-        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, st>>>(wv, layer_rows(), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
     if (quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.top_k <= kDownMergeSlots && wv.hidden % kQuadRows == 0 && rows <= 65535U) {
         const dim3 grid(wv.hidden / kQuadRows, rows);
-        if (rows <= 2U) down_merge_quad_kernel<4><<<grid, 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
-        else down_merge_quad_kernel<2><<<grid, 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        if (rows <= 2U) down_merge_quad_kernel<4><<<grid, 64U * wv.top_k, 0, st>>>(wv, layer_rows(), items, form);
+        else down_merge_quad_kernel<2><<<grid, 64U * wv.top_k, 0, st>>>(wv, layer_rows(), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
     if (wv.down_type == MI355_TYPE_Q8_0 && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && wv.ffn % 128U == 0 && rows <= 65535U) {
-        down_merge_q8_0_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        down_merge_q8_0_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, layer_rows(), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
     if (wv.down_type == MI355_TYPE_Q5_1 && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && rows <= 65535U && wv.ffn % 256U == 0 &&
         wv.down_row_stride % 16U == 0 && wv.down_expert_stride % 16U == 0) {       // (what down_q51_ring_kernel's copies need)
-        down_merge_q51_kernel<2><<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        down_merge_q51_kernel<2><<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, layer_rows(), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
     if (wv.down_type == MI355_TYPE_Q6_K && wv.top_k <= kDownMergeSlots && wv.hidden % 16U == 0 && rows <= 65535U) {
-        down_merge_q6k_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, rows_k(*r, wv), items, form);
+        down_merge_q6k_kernel<<<dim3(wv.hidden / 16U, rows), 64U * wv.top_k, 0, st>>>(wv, layer_rows(), items, form);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
-    launch_down(wv, rows_k(*r, wv), rows, items, st);
+    launch_down(wv, layer_rows(), rows, items, st);
     STRIX_LAUNCHED("moe layer experts");
-    return mi355_moe_enqueue_merge(w, r, rows, form, stream);
+    return enqueue_merge(w, r, rows, form, stream, p->shared_experts);
 }
 }  // namespace
 
@@ -2490,4 +2501,5 @@ int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float*
 #include "a8_contract.hpp"
 #include "rows_forms.hpp"
 #include "combine_forms.hpp"
+#include "shared_gate.hpp"
 #include "gguf_reader.hpp"

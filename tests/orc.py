@@ -377,6 +377,23 @@ def combine(form, w, ids, raw, base=None):
     return y
 
 
+def combine_shared(form, w, ids, raw, shared_slots, base=None):
+    rows, top_k, width = raw.shape
+    raw, w, ids = np.ascontiguousarray(raw, np.float32), np.ascontiguousarray(w, np.float32), np.ascontiguousarray(ids, np.uint32)
+    y = np.zeros((rows, width), np.float32)
+    b = None if base is None else np.ascontiguousarray(base, np.float32)
+    lib().orc_combine_shared(form, rows, top_k, shared_slots, width, _ptr(w, f32p), _ptr(ids, u32p), _ptr(raw, f32p), _ptr(b, f32p), _ptr(y, f32p))
+    return y
+
+
+def shared_gate(x, w, exp_kind=EXP_GFX1151):
+    x, w = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(w, np.float32)
+    rows, hidden = x.shape
+    gate, dots = np.zeros(rows, np.float32), np.zeros(rows, np.float32)
+    lib().orc_shared_gate(_ptr(x, f32p), _ptr(w, f32p), rows, hidden, exp_kind, _ptr(gate, f32p), _ptr(dots, f32p))
+    return gate, dots
+
+
 class ExpertResult:
     pass
 

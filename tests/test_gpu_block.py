@@ -113,3 +113,65 @@ def test_block_norm_and_shared_expert_together_and_admission(strix):
         layer.run_layer(dev(x), dev(wr), shared_experts=0)
     with pytest.raises(strix.StrixError):
         strix.route(dev(x), dev(wr), K, shared_experts=5)
+
+
+@pytest.mark.parametrize("kind,H,T", [("bf16", 2048, 8), ("f16", 2560, 3), ("f32", 300, 5), ("bf16", 4096, 40), ("f32", 256, 1)])
+def test_shared_gate_bit_exact(strix, kind, H, T):
+    """mi355_shared_gate against the oracle (src/hip_shared_expert_launcher.hip:624-645: thread-strided fma chains, 256-leaf halving
+    tree, device expf, one division), and on the order fixtures that a wrong pairing or an unfused multiply-add changes."""
+    rng = np.random.default_rng(H + T)
+    x_t = torch.from_numpy((rng.standard_normal((T, H)) * 2.0).astype(np.float32)).to(DT[kind])
+    w = (rng.standard_normal(H) * 0.05).astype(np.float32)
+    want, _ = orc.shared_gate(x_t.to(torch.float32).numpy(), w)
+    got = strix.shared_gate(x_t.cuda(), dev(w)).cpu().numpy()[:, 0]
+    assert np.array_equal(bits(got), bits(want))
+    # written with a stride, into a wider buffer
+    wide = torch.full((T, 3), -1.0, dtype=torch.float32, device="cuda")
+    strix.shared_gate(x_t.cuda(), dev(w), out=wide[:, 1:2])
+    assert np.array_equal(bits(wide[:, 1].cpu().numpy()), bits(want)) and bool((wide[:, 0] == -1).all()) and bool((wide[:, 2] == -1).all())
+    if kind != "f32":
+        return
+    sig1 = orc.shared_gate(np.ones((1, 1), np.float32), np.ones(1, np.float32))[0][0]            # sigmoid(1) as the oracle rounds it
+    x1, w1 = np.ones((1, 256), np.float32), np.zeros(256, np.float32)
+    w1[0], w1[1], w1[128], w1[129] = 2.0 ** 24, -(2.0 ** 24), 1.0, 1.0                            # the tree gives 1, index order 2
+    x2, w2 = np.zeros((1, 512), np.float32), np.zeros(512, np.float32)
+    x2[0, 0], w2[0], x2[0, 256], w2[256] = -1.0, 2.0 ** 24 + 2.0 ** 13, 2.0 ** 12 + 1.0, 2.0 ** 12 + 1.0   # fused: 1, unfused: 0
+    for xs, ws in ((x1, w1), (x2, w2)):
+        assert orc.shared_gate(xs, ws)[1][0] == 1.0
+        assert bits(strix.shared_gate(dev(xs), dev(ws)).cpu().numpy())[0, 0] == bits(np.array([sig1], np.float32))[0]
+
+
+@pytest.mark.parametrize("down_type,H,I,E,K,S,T,form", [
+    (orc.Q4_K, 2048, 768, 128, 8, 1, 8, 0),        # config 3 plus a gated shared expert
+    (orc.Q4_K, 1024, 512, 16, 4, 1, 3, 0),         # the one-launch down + combine of a small batch
+    (orc.Q8_0, 1024, 512, 16, 4, 1, 16, 0),
+    (orc.Q6_K, 512, 768, 6, 3, 2, 5, 0),           # two always-on experts, each with its own gate column
+    (orc.Q5_1, 1024, 384, 8, 2, 1, 9, 1),          # the product-then-sum form
+    (orc.Q4_K, 1024, 512, 16, 4, 1, 24, 0)])       # the staged path: merge launch
+def test_shared_expert_with_its_sigmoid_gate(strix, down_type, H, I, E, K, S, T, form):
+    """The shared expert as the reference computes it: gate = sigmoid(x . ffn_gate_inp_shexp) from mi355_shared_gate is the always-on
+    slot's weight (policy.shared_slot_weights) and the slot enters the sum as acc + (gate * value)
+    (src/hip_shared_expert_launcher.hip:727,779; include/strix/moe/combine.hpp:56)."""
+    rng = np.random.default_rng(H + 7 * T + S + down_type)
+    gate, up, down = layer_tensors(rng, H, I, E + S, orc.Q4_K, down_type)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    scalar = (rng.standard_normal((S, H)) * 0.05).astype(np.float32)
+    residual = rng.standard_normal((T, H)).astype(np.float32)
+    gates = torch.zeros((T, S), dtype=torch.float32, device="cuda")
+    for s_ in range(S):
+        strix.shared_gate(dev(x), dev(scalar[s_]), out=gates[:, s_:s_ + 1])
+    want_g = np.stack([orc.shared_gate(x.astype(np.float32), scalar[s_])[0] for s_ in range(S)], axis=1)
+    assert np.array_equal(bits(gates.cpu().numpy()), bits(want_g))
+    layer = strix.MoeLayer(H, I, E + S, K + S, dev(gate), dev(up), dev(down), T, intermediates=True, down_type=down_type)
+    y, ids, wts, _ = layer.run_layer(dev(x), dev(wr), shared_experts=S, shared_slot_weights=gates, base=dev(residual), combine=form)
+    torch.cuda.synchronize()
+    ids_r, w_r, _, _ = orc.route(x.astype(np.float32), wr, K)
+    ids_ref = np.concatenate([ids_r, np.tile(np.arange(E, E + S, dtype=np.uint32), (T, 1))], axis=1)
+    w_ref = np.concatenate([w_r, want_g], axis=1)
+    assert np.array_equal(ids.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(wts.cpu().numpy()), bits(w_ref))
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    ref = orc.routed_experts(H, I, K + S, gate, up, down, down_type, c, d, s, ids_ref)
+    assert np.array_equal(bits(layer.rawdots[:T].cpu().numpy()), bits(ref.rawdots))
+    assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine_shared(form, w_ref, ids_ref, ref.rawdots, S, base=residual)))
+    assert np.all(layer.status[:T].cpu().numpy() == 0)

@@ -1083,3 +1083,66 @@ def test_vector_form_of_the_q4k_row_equals_the_plain_loop():
             assert (np.isnan(fast) and np.isnan(plain)) or np.float32(fast).view(np.uint32) == np.float32(plain).view(np.uint32), case
     finally:
         L.orc_vector_rows(1)
+
+
+def test_shared_gate_order_fixtures():
+    """orc_shared_gate (src/hip_shared_expert_launcher.hip:624-645): what the arithmetic fixes, on inputs where a plausible mistake
+    shows. (1) the halving tree pairs lane l with l + 128, then l + 64, ...: with 2^24, 1, -2^24 + ... placed on lanes 0, 128, 64, 192
+    the tree gives 1, a sequential sum 2, adjacent pairs 2. (2) each step is one fma: (2^12 + 1)^2 = 2^24 + 2^13 + 1 keeps its last
+    bit only inside an fma. (3) thread t owns features t, t + 256, ... in ascending order. (4) against float64 on random rows."""
+    E = orc.EXP_GFX1151
+    sig = lambda d: np.float32(1.0) / (np.float32(1.0) + np.float32(orc.lib().orc_expf_gfx1151(float(-d))))
+    # (1) pairing
+    x = np.ones((1, 256), np.float32)
+    w = np.zeros(256, np.float32)
+    w[0], w[128], w[64], w[192] = 2.0 ** 24, 1.0, -(2.0 ** 24), 1.0
+    gate, dots = orc.shared_gate(x, w, E)
+    assert dots[0] == 1.0 and bits(gate)[0] == bits(np.array([sig(1.0)], np.float32))[0]
+    # (a sum of the lanes in index order gives 2 here, and so does the adjacent pairing; a second placement of the same kind:)
+    w2 = np.zeros(256, np.float32)
+    w2[0], w2[1], w2[128], w2[129] = 2.0 ** 24, -(2.0 ** 24), 1.0, 1.0     # tree: (2^24 + 1) + (-2^24 + 1) = 2^24 + (-2^24 + 1) = 1; lanes in index order: 0 + 1 + 1 = 2
+    _, dots2 = orc.shared_gate(x, w2, E)
+    assert dots2[0] == 1.0
+    # (2) fma: thread 0 takes features 0 and 256
+    x3 = np.zeros((1, 512), np.float32); w3 = np.zeros(512, np.float32)
+    x3[0, 0], w3[0] = -1.0, 2.0 ** 24 + 2.0 ** 13
+    x3[0, 256], w3[256] = 2.0 ** 12 + 1.0, 2.0 ** 12 + 1.0
+    gate3, dots3 = orc.shared_gate(x3, w3, E)
+    assert dots3[0] == 1.0                                                  # product then sum would give 0
+    assert bits(gate3)[0] == bits(np.array([sig(1.0)], np.float32))[0] and gate3[0] != 0.5
+    # (3) ascending features within a thread: 2^24 first, then 1 twice -> 2^24 (each 1 is lost); descending would give 2^24 + 2
+    x4 = np.ones((1, 768), np.float32); w4 = np.zeros(768, np.float32)
+    w4[5], w4[261], w4[517] = 2.0 ** 24, 1.0, 1.0
+    _, dots4 = orc.shared_gate(x4, w4, E)
+    assert dots4[0] == 2.0 ** 24
+    # (4) random rows against float64, and the sigmoid's fixed points
+    rng = np.random.default_rng(635)
+    xr = rng.standard_normal((6, 2048)).astype(np.float32)
+    wr = (rng.standard_normal(2048) * 0.05).astype(np.float32)
+    gate5, dots5 = orc.shared_gate(xr, wr, E)
+    d64 = xr.astype(np.float64) @ wr.astype(np.float64)
+    assert np.allclose(dots5, d64, rtol=0, atol=2e-5) and np.allclose(gate5, 1.0 / (1.0 + np.exp(-d64)), rtol=0, atol=1e-6)
+    g0, _ = orc.shared_gate(np.zeros((1, 300), np.float32), np.ones(300, np.float32), E)
+    assert g0[0] == 0.5
+
+
+def test_shared_slot_enters_the_combine_as_product_then_sum():
+    """orc_combine_shared: the routed slots by fma, an always-on slot as acc + (w * value). With weight 1 it is the plain combine
+    (fma(1, v, acc) = acc + v); with a gate the product is rounded on its own, which a cancellation makes visible."""
+    rng = np.random.default_rng(56)
+    raw = rng.standard_normal((4, 5, 40)).astype(np.float32)
+    w = rng.random((4, 5)).astype(np.float32)
+    ids = np.tile(np.arange(5, dtype=np.uint32), (4, 1))
+    base = rng.standard_normal((4, 40)).astype(np.float32)
+    w1 = w.copy(); w1[:, 4] = 1.0
+    assert np.array_equal(bits(orc.combine_shared(0, w1, ids, raw, 1, base)), bits(orc.combine(0, w1, ids, raw, base)))
+    got = orc.combine_shared(0, w, ids, raw, 1, base)
+    routed = orc.combine(0, w[:, :4].copy(), ids[:, :4].copy(), raw[:, :4].copy())
+    want = (routed + (w[:, 4:5] * raw[:, 4]).astype(np.float32)).astype(np.float32) + base
+    assert np.array_equal(bits(got), bits(want))
+    # (1 + 2^-12)^2 = 1 + 2^-11 + 2^-24: rounded on its own the last term is lost, inside an fma it survives the cancellation
+    one = np.array([[[-(1.0 + 2.0 ** -11)], [1.0 + 2.0 ** -12]]], np.float32)
+    ww = np.array([[1.0, 1.0 + 2.0 ** -12]], np.float32)
+    i2 = np.array([[0, 1]], np.uint32)
+    assert orc.combine_shared(0, ww, i2, one, 1)[0, 0] == 0.0
+    assert orc.combine(0, ww, i2, one, np.zeros((1, 1), np.float32))[0, 0] == 2.0 ** -24
