@@ -295,7 +295,15 @@ int32_t mi355_moe_enqueue_layer_normed(const mi355_route_policy* policy, const f
  * of about 5.1 MB that is part of the library image (each device the library runs on holds its own copy until the process
  * ends). Limits: rows <= 16, top_k <= 8, hidden <= 8192, ffn <= 4096, experts <= 1024; beyond them the call returns
  * MI355_E_INVALID_ARGUMENT. The call allocates nothing and computes the same bits as mi355_moe_enqueue_layer. Every call on
- * a device shares that device's array: two calls that overlap on one device (different streams or threads) race. */
+ * a device shares that device's array: two calls that overlap on one device (different streams or threads) race. The counters
+ * inside the array are left zero by every call; when a launch of the sequence fails (MI355_E_HIP) the entry point enqueues their
+ * reset itself. The first call on a device (or mi355_static_workspace_prepare) must happen outside a stream capture. */
+/* (belongs to mi355_moe_enqueue_layer_static; no counterpart in the reference) Looks up the built-in workspace of the current device
+ * and enqueues a kernel that zeroes the counters in it which every call expects to find zero. Call it once per device at set-up -
+ * the address look-up is a runtime call that does not belong inside a stream capture; mi355_moe_enqueue_layer_static does the
+ * look-up itself on its first call on a device otherwise, so that first call must then happen outside capture - and again
+ * after any call of the static entry point was interrupted (a device reset handled by the caller). Allocates nothing. */
+int32_t mi355_static_workspace_prepare(mi355_stream);
 int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* policy, const float* router_weight, const float* logit_bias,
                                        const mi355_moe_weights*, const void* input, uint32_t input_kind, uint64_t input_stride,
                                        uint32_t rows, uint32_t* routes, float* route_weights, uint32_t* status, const float* base,

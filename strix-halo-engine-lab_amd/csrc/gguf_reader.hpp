@@ -143,6 +143,52 @@ private:
         at_ += n;
         return true;
     }
+    bool skip(uint64_t n) {                        // pass over n bytes unread: one bounds check, one seek
+        if (n > size_ - at_) return fail("unexpected end of GGUF file");
+        if (n != 0 && fseeko(f_, static_cast<off_t>(n), SEEK_CUR) != 0) return fail("failed to read GGUF bytes");
+        at_ += n;
+        return true;
+    }
+    static uint32_t scalar_bytes(uint32_t type) {  // 0 for the types that are no fixed-size scalars (string, array)
+        switch (type) {
+        case 0: case 1: case 7: return 1U;
+        case 2: case 3: return 2U;
+        case 4: case 5: case 6: return 4U;
+        case 10: case 11: case 12: return 8U;
+        default: return 0U;
+        }
+    }
+    // the elements of an array whose values nobody asked for: scalars in one step (booleans are still checked, in blocks),
+    // strings by their length fields
+    bool skip_elements(uint32_t element, uint64_t length, uint32_t depth) {
+        if (element == 7U) {
+            uint8_t block[4096];
+            for (uint64_t done = 0; done < length;) {
+                const size_t n = static_cast<size_t>(length - done < sizeof block ? length - done : sizeof block);
+                if (!bytes(block, n)) return false;
+                for (size_t i = 0; i < n; ++i)
+                    if (block[i] > 1) return fail("GGUF boolean must be zero or one");
+                done += n;
+            }
+            return true;
+        }
+        if (const uint32_t unit = scalar_bytes(element)) {
+            uint64_t total = length;
+            return mul(total, unit) && skip(total);
+        }
+        if (element == 8U) {
+            for (uint64_t n = 0; n < length; ++n) {
+                uint64_t len;
+                if (!get(len)) return false;
+                if (len > 64ULL * 1024ULL * 1024ULL) return fail("GGUF string exceeds configured limit");
+                if (!skip(len)) return false;
+            }
+            return true;
+        }
+        for (uint64_t n = 0; n < length; ++n)
+            if (!value(element, nullptr, depth + 1U)) return false;
+        return true;
+    }
     template <class T> bool get(T& v) {            // little-endian scalar (the hosts this library runs on are little-endian)
         return bytes(&v, sizeof(T));
     }
@@ -183,9 +229,7 @@ private:
             if (length > 100000000ULL - array_elements_) return fail("GGUF arrays exceed configured element limit");
             array_elements_ += length;
             if (o) { o->array_type = element; o->array_length = length; }
-            for (uint64_t n = 0; n < length; ++n)
-                if (!value(element, nullptr, depth + 1U)) return false;
-            return true;
+            return skip_elements(element, length, depth);
         }
         case 10: return scalar_u<uint64_t>(o);
         case 11: return scalar_i<int64_t>(o);

@@ -2467,7 +2467,25 @@ unsigned char* scratch_on_current_device() {
     g_scratch_of_device[device].store(static_cast<unsigned char*>(found), std::memory_order_release);   // (a racing first call stores the same address)
     return static_cast<unsigned char*>(found);
 }
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* words, uint32_t count) {
+    const uint32_t i = blockIdx.x * 256U + threadIdx.x;
+    if (i < count) words[i] = 0U;
+}
+// The plan words every launch expects to find zero and leaves zero (tickets, arrival counts, tags, the epoch): all zero is the
+// state of a freshly loaded library. A kernel store, so that the call may sit inside a captured graph.
+int32_t static_plan_reset(unsigned char* ws, hipStream_t st) {
+    zero_words_kernel<<<(kPlanOffsetsAt - kPlanTicketsAt + 255U) / 256U, 256, 0, st>>>(reinterpret_cast<uint32_t*>(ws + kStaticPlanAt) + kPlanTicketsAt,
+                                                                                  kPlanOffsetsAt - kPlanTicketsAt);
+    STRIX_LAUNCHED("static workspace reset");
+    return MI355_OK;
+}
 }  // namespace
+
+int32_t mi355_static_workspace_prepare(mi355_stream stream) {
+    unsigned char* ws = scratch_on_current_device();
+    if (!ws) return g_error.rfind("static workspace: device", 0) == 0 ? MI355_E_UNSUPPORTED : MI355_E_HIP;
+    return static_plan_reset(ws, hs(stream));
+}
 
 int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float* router_weight, const float* logit_bias,
                                        const mi355_moe_weights* w, const void* input, uint32_t input_kind, uint64_t input_stride,
@@ -2493,7 +2511,15 @@ int32_t mi355_moe_enqueue_layer_static(const mi355_route_policy* p, const float*
     r.down_deltas = reinterpret_cast<float*>(ws + kStaticDownDeltasAt);
     r.down_sums = reinterpret_cast<int32_t*>(ws + kStaticDownSumsAt);
     r.rawdots = reinterpret_cast<float*>(ws + kStaticRawdotsAt);
-    return mi355_moe_enqueue_layer(p, router_weight, logit_bias, reinterpret_cast<float*>(ws + kStaticScoresAt), w, &r, rows, form, stream);
+    const int32_t rc = mi355_moe_enqueue_layer(p, router_weight, logit_bias, reinterpret_cast<float*>(ws + kStaticScoresAt), w, &r, rows, form, stream);
+    // a launch that failed part-way (MI355_E_HIP) may have left counters of the shared plan half-way: put them back to zero for the
+    // next call (an admission failure enqueued nothing)
+    if (rc == MI355_E_HIP) {
+        const std::string first = g_error;
+        (void)static_plan_reset(ws, hs(stream));
+        g_error = first;
+    }
+    return rc;
 }
 
 }  // extern "C"

@@ -47,3 +47,35 @@ def test_static_workspace_layer_refuses_sizes_beyond_its_limits(strix):
     assert err.value.code == strix.E_INVALID_ARGUMENT and "1..16" in str(err.value)
     torch.cuda.synchronize()
     assert bool((out == -7.0).all())
+
+
+def test_static_workspace_layer_inside_a_captured_graph(strix):
+    """The entry point is for callers under stream capture: after mi355_static_workspace_prepare (the symbol look-up, outside
+    capture) the call is captured into a HIP graph and replayed with eager calls of the library in between; every replay
+    gives the eager result's bits. Nothing in the sequence allocates or records a memset node."""
+    H, I, E, K, T = 2048, 768, 128, 8, 8
+    layer, wr, x = _layer(strix, H, I, E, K, T, seed=91)
+    strix.check(strix.lib().mi355_static_workspace_prepare(None))
+    want, ids, wts, _ = layer.run_layer(x, wr)
+    want, ids = want.clone(), ids.clone()
+    ids2 = torch.zeros((T, K), dtype=torch.int32, device="cuda")
+    wts2 = torch.zeros((T, K), dtype=torch.float32, device="cuda")
+    status2 = torch.zeros((T,), dtype=torch.int32, device="cuda")
+    out2 = torch.zeros((T, H), dtype=torch.float32, device="cuda")
+    layer.run_layer_static(x, wr, ids2, wts2, status2, out2)          # warm call outside capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer.run_layer_static(x, wr, ids2, wts2, status2, out2)
+    for replay in range(4):
+        out2.fill_(-3.0); ids2.fill_(-1); status2.fill_(55)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ids2, ids) and int(status2.sum()) == 0, replay
+        assert np.array_equal(out2.cpu().numpy().view(np.uint32), want.cpu().numpy().view(np.uint32)), replay
+        # eager work of the same library between the replays: another shape through the same built-in workspace
+        other, _, _, _ = layer.run_layer(x[:3].contiguous(), wr)
+        o3 = torch.zeros((3, H), dtype=torch.float32, device="cuda")
+        layer.run_layer_static(x[:3].contiguous(), wr, ids2[:3].clone(), wts2[:3].clone(), status2[:3].clone(), o3)
+        torch.cuda.synchronize()
+        assert np.array_equal(o3.cpu().numpy().view(np.uint32), other.cpu().numpy().view(np.uint32)), replay
