@@ -484,6 +484,26 @@ int32_t mi355_moe_strided_enqueue_commit(const mi355_moe_weights*, const mi355_m
 int32_t mi355_moe_strided_enqueue(const mi355_moe_weights*, const mi355_moe_rows_strided*, uint32_t rows, uint32_t clear_words, uint32_t* record,
                                   uint32_t domain, mi355_stream);
 
+/* Known-prompt prefill over strided rows, FAST class (known_rows::PrefillRows / enqueue_prefill with the separate FP16 prefill
+ * contract, include/strix/hip_moe_q4k_a8_known_rows.hpp:75-111): every per-row view is row 0 plus r times its own byte stride.
+ * Runs the prologue (zeroes clear[row][0 .. clear_words), checks routes and route weights, OVERWRITES status[row], clears the
+ * job word), the expert plan over the rows * top_k assignments (stable: rows then slots), gate / up + SwiGLU and the down rows;
+ * rawdots[row][slot][hidden] receives the unweighted outputs and THE CALLER MERGES AND COMMITS (mi355_moe_strided_enqueue_merge /
+ * _commit take the same views). rawdots_bf16: every unweighted output is stored once rounded to bfloat16 (as an fp32 value), the
+ * stored output of a bfloat16 Linear - the same bits as the fp32 store followed by a rounding pass over rawdots. A non-finite
+ * gate / up / h value of a (row, slot) sets bit 8 in the row's status and in the job word; the down rows are then skipped.
+ * The views of the integer forms (codes, deltas, sums, down_*) are not part of this bundle: the fp16 form has no A8 image;
+ * the integer-class stages over strided rows are mi355_moe_strided_enqueue*. input: fp16 rows; plan: mi355_moe_plan_words words;
+ * h_f16: mi355_moe_prefill_f16_workspace_bytes bytes. Arithmetic and tolerance: mi355_moe_enqueue_prefill_f16. */
+typedef struct mi355_prefill_rows {
+    mi355_strided input, routes, route_weights, status, clear, rawdots;
+    uint32_t* plan;
+    uint32_t* job_status;
+    void* h_f16;
+    uint32_t rawdots_bf16;
+} mi355_prefill_rows;
+int32_t mi355_moe_enqueue_prefill_rows_f16(const mi355_moe_weights*, const mi355_prefill_rows*, uint32_t rows, uint32_t clear_words, mi355_stream);
+
 /* ------------------------------------------------------------------------------------------------------
  * The job form of the host executor (strix::cpu::expert::Job / LayerWeights / Executor, src/cpu/core/routed_expert.hpp:28-61,
  * 79-95): a list of (row, slot, expert) assignments over per-row A8 images, every pointer device memory.

@@ -104,6 +104,12 @@ class MoeRowsStrided(C.Structure):
                [("plan", C.c_void_p), ("job_status", C.c_void_p), ("input_kind", C.c_uint32), ("output_kind", C.c_uint32)]
 
 
+class PrefillRows(C.Structure):
+    """mi355_prefill_rows: the strided views of the fp16 prefill (known_rows::PrefillRows, include/strix/hip_moe_q4k_a8_known_rows.hpp:75-95)."""
+    _fields_ = [(n, Strided) for n in ("input", "routes", "route_weights", "status", "clear", "rawdots")] + \
+               [("plan", C.c_void_p), ("job_status", C.c_void_p), ("h_f16", C.c_void_p), ("rawdots_bf16", C.c_uint32)]
+
+
 class RowA8(C.Structure):
     _fields_ = [("codes", C.c_void_p), ("deltas", C.c_void_p), ("sums", C.c_void_p)]
 
@@ -255,7 +261,7 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue_combine", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_static_workspace_prepare", "mi355_moe_enqueue_prefill_f16", "mi355_moe_prefill_f16_workspace_bytes",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue_combine", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_static_workspace_prepare", "mi355_moe_enqueue_prefill_f16", "mi355_moe_enqueue_prefill_rows_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_shared_gate", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe", "mi355_a8_enqueue_serial_prologue_probe", "mi355_a8_enqueue_quantize_only",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
            "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",
@@ -545,6 +551,13 @@ class MoeLayer:
         if combine == COMBINE_NONE:      # no combine: the unweighted per-slot outputs [rows][top_k][hidden]
             return self.rawdots[:rows]
         return self.output[:rows]
+
+    def run_prefill_rows_f16(self, views, rows, clear_words=0):
+        """mi355_moe_enqueue_prefill_rows_f16 over caller-built strided views (PrefillRows); plan / job word / h_f16 default to this
+        layer's own buffers."""
+        if not views.plan:
+            views.plan, views.job_status, views.h_f16 = self.plan.data_ptr(), self.job_status.data_ptr(), self.h_f16.data_ptr()
+        check(lib().mi355_moe_enqueue_prefill_rows_f16(C.byref(self.w), C.byref(views), rows, clear_words, _stream()))
 
     def run_layer(self, x, router_weight, bias=None, base=None, combine=COMBINE_FMA_SLOT, logits_order=LOGITS_FMA, renorm_eps=0.0,
                   scale=1.0, renormalize=True, renorm_single=True, exp_kind=EXP_DECLARED, shared_experts=0, norm=None, half=None, shared_slot_weights=None):

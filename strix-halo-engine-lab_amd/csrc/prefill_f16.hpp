@@ -84,7 +84,25 @@ struct PrefillArgs {
     const uint32_t* plan; uint32_t experts, assignments;
     uint32_t* status; uint32_t* job_status;
     uint32_t tiles, items, units;                 // feature tiles per item, item bound of the launch, tiles * items rounded up to 8 items
+    uint64_t status_rs, rawdots_rs;               // bytes between the rows of status / rawdots; rawdots_rs == 0: dense [assignment][features]
+    uint32_t rawdots_bf16;                        // MODE 1: every unweighted output is stored once rounded to bfloat16 (as an fp32 value)
 };
+
+// the status word of an assignment's row, and the first of its `features` unweighted outputs
+__device__ __forceinline__ uint32_t* pf_status_of(const PrefillArgs& a, uint32_t assignment) {
+    return reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(a.status) + static_cast<size_t>(assignment / a.top_k) * a.status_rs);
+}
+__device__ __forceinline__ float* pf_rawdots_of(const PrefillArgs& a, uint32_t assignment) {
+    if (a.rawdots_rs == 0) return a.rawdots + static_cast<size_t>(assignment) * a.features;
+    const uint32_t row = assignment / a.top_k, slot = assignment - row * a.top_k;
+    return reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.rawdots) + static_cast<size_t>(row) * a.rawdots_rs) + static_cast<size_t>(slot) * a.features;
+}
+// include/strix/moe/combine.hpp:24-33 (the stored output of a bfloat16 Linear: nearest even, a NaN as it is)
+__device__ __forceinline__ float pf_round_bf16(float x) {
+    const uint32_t bits = __builtin_bit_cast(uint32_t, x);
+    if ((bits & 0x7f800000U) == 0x7f800000U && (bits & 0x7fffffU)) return x;
+    return __builtin_bit_cast(float, (bits + 0x7fffU + ((bits >> 16U) & 1U)) & 0xffff0000U);
+}
 
 __device__ __forceinline__ uint32_t pack_half2(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{a, b}, half2v));      // v_cvt_pk_f16_f32: round to nearest even
@@ -581,14 +599,16 @@ __global__ __launch_bounds__(kPfThreads) void prefill_f16_kernel(PrefillArgs a, 
                         split_half(sum, sums[sub_block], sums[pf_sum_slots(a.features) + sub_block]);
                     }
                     if (!(finite_f(g) && finite_f(u) && finite_f(static_cast<float>(h16)))) {     // h beyond fp16 counts as non-finite
-                        atomicOr(&a.status[order[begin + n] / a.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                        atomicOr(pf_status_of(a, order[begin + n]), static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
                         atomicOr(a.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
                     }
                 }
             } else if (live) {
-                float* out = a.rawdots + static_cast<size_t>(dest[i][j]) * a.features + m0 + 64U * wr + l31;
-                if (a.lo_pass) { out[0] += acc[i][0][j]; out[32] += acc[i][1][j]; }
-                else { out[0] = acc[i][0][j]; out[32] = acc[i][1][j]; }
+                float* out = pf_rawdots_of(a, dest[i][j]) + m0 + 64U * wr + l31;
+                if (a.lo_pass) {            // the second pass completes the value: the one rounding to bfloat16, if asked for, happens here
+                    const float v0 = out[0] + acc[i][0][j], v1 = out[32] + acc[i][1][j];
+                    out[0] = a.rawdots_bf16 ? pf_round_bf16(v0) : v0; out[32] = a.rawdots_bf16 ? pf_round_bf16(v1) : v1;
+                } else { out[0] = acc[i][0][j]; out[32] = acc[i][1][j]; }
             }
         }
     }

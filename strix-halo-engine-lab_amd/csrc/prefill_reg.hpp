@@ -322,7 +322,7 @@ __global__ __launch_bounds__(kRgThreads) void prefill_reg_kernel(PrefillArgs a, 
                     a.h[at] = h_hi;
                     a.h_lo[at] = h_lo;
                     if (!(finite_f(g) && finite_f(u) && finite_f(static_cast<float>(h_hi)))) {     // h beyond fp16 counts as non-finite
-                        atomicOr(&a.status[order[begin + t] / a.top_k], static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+                        atomicOr(pf_status_of(a, order[begin + t]), static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
                         atomicOr(a.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
                     }
                 }
@@ -344,7 +344,7 @@ __global__ __launch_bounds__(kRgThreads) void prefill_reg_kernel(PrefillArgs a, 
 #pragma unroll
             for (uint32_t r = 0; r < 16U; ++r) {
                 const uint32_t t = 32U * i + 8U * (r / 4U) + 4U * half + (r & 3U);
-                if (t < count) a.rawdots[static_cast<size_t>(order[begin + t]) * a.features + f_out] = acc[i][r];
+                if (t < count) pf_rawdots_of(a, order[begin + t])[f_out] = a.rawdots_bf16 ? pf_round_bf16(acc[i][r]) : acc[i][r];
             }
     }
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(hd_cur), "+v"(hd_next), "+v"(qs[0]), "+v"(qs[1]), "+v"(qs[2]), "+v"(qs[3]) : : "memory");

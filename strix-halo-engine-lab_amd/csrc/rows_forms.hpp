@@ -163,6 +163,29 @@ int32_t check_strided(const mi355_moe_weights* w, const mi355_moe_rows_strided* 
     return MI355_OK;
 }
 
+// The prologue of the fp16 prefill over strided rows (enqueue_prefill_prologue, include/strix/hip_moe_q4k_a8_known_rows.hpp:86-87,
+// without the A8 quantiser, which the fp16 form does not use): zero the row's `clear` words, check its routes and route weights,
+// OVERWRITE its status word; row 0 clears the job word.
+__global__ __launch_bounds__(256) void prefill_rows_prologue_kernel(mi355_prefill_rows v, uint32_t experts, uint32_t top_k, uint32_t clear_words) {
+    __shared__ uint32_t route_bits;
+    const uint32_t row = blockIdx.x, t = threadIdx.x;
+    if (t == 0) route_bits = 0;
+    if (v.clear.base) {
+        float* clear = row_at<float>(v.clear, row);
+        for (uint32_t i = t; i < clear_words; i += 256U) clear[i] = 0.0F;
+    }
+    __syncthreads();
+    const uint32_t* routes = row_at<const uint32_t>(v.routes, row);
+    const float* weights = row_at<const float>(v.route_weights, row);
+    for (uint32_t k = t; k < top_k; k += 256U)
+        if (routes[k] >= experts || !finite_f(weights[k])) atomicOr(&route_bits, static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+    __syncthreads();
+    if (t == 0) {
+        *row_at<uint32_t>(v.status, row) = route_bits;
+        if (row == 0) *v.job_status = 0U;
+    }
+}
+
 // --------------------------------------------------------------------------------------------------------- job form
 // The executor object of the job form: the A8 image of h for up to max_assignments assignments and the job word, allocated
 // once (as Executor owns its scratch vectors, src/cpu/core/routed_expert.cpp:356-363).
@@ -182,6 +205,38 @@ __global__ void clear_word_kernel(uint32_t* word) { *word = 0U; }
 using namespace strix950;
 
 extern "C" {
+
+// Known-prompt prefill over strided rows in the FAST class (known_rows::enqueue_prefill with the fp16 form,
+// include/strix/hip_moe_q4k_a8_known_rows.hpp:75-111): prologue, expert plan, gate / up + SwiGLU, down rows into rawdots; the caller
+// merges and commits.
+int32_t mi355_moe_enqueue_prefill_rows_f16(const mi355_moe_weights* w, const mi355_prefill_rows* v, uint32_t rows, uint32_t clear_words, mi355_stream stream) {
+    STRIX_REQUIRE(w && v, "moe prefill rows: null weights or rows");
+    mi355_moe_rows shell{};                     // check_moe looks at the dense bundle's pointers: stand-ins that pass its null / alignment tests
+    shell.routes = static_cast<const uint32_t*>(v->routes.base); shell.route_weights = static_cast<const float*>(v->route_weights.base);
+    shell.status = static_cast<uint32_t*>(v->status.base); shell.rawdots = static_cast<float*>(v->rawdots.base);
+    shell.plan = v->plan; shell.job_status = v->job_status; shell.h_f16 = v->h_f16;
+    shell.output = static_cast<float*>(v->rawdots.base); shell.output_stride = w->hidden;
+    shell.codes = reinterpret_cast<int8_t*>(v->h_f16); shell.deltas = reinterpret_cast<float*>(v->h_f16); shell.sums = reinterpret_cast<int32_t*>(v->h_f16);
+    shell.down_codes = shell.codes; shell.down_deltas = shell.deltas; shell.down_sums = shell.sums;     // (the fp16 form has no A8 images)
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, &shell, rows, wv, kPrefillClass)) return rc;
+    STRIX_REQUIRE(rows <= 65535U, "moe prefill rows: at most 65535 rows per call");
+    STRIX_REQUIRE(wv.hidden % 128U == 0 && wv.ffn % 64U == 0, "moe prefill rows: hidden must be a multiple of 128, ffn of 64");
+    STRIX_REQUIRE(v->h_f16 && aligned(v->h_f16, 16), "moe prefill rows: h_f16 workspace is null or misaligned");
+    STRIX_REQUIRE(strided_ok(v->input, 16) && strided_ok(v->rawdots, 16) && strided_ok(v->routes, 4) && strided_ok(v->route_weights, 4) &&
+                  strided_ok(v->status, 4) && (v->clear.base == nullptr || strided_ok(v->clear, 4)),
+                  "moe prefill rows: input and rawdots need a 16-byte aligned base and stride (routes, route weights, status, clear: 4)");
+    const uint64_t K = wv.top_k;
+    STRIX_REQUIRE(v->input.stride >= 2ULL * wv.hidden && v->routes.stride >= 4U * K && v->route_weights.stride >= 4U * K && v->status.stride >= 4U &&
+                  v->rawdots.stride >= 4U * K * wv.hidden, "moe prefill rows: a view's stride is shorter than one row's extent");
+    STRIX_REQUIRE(clear_words == 0 || (v->clear.base && (rows == 1U || 4ULL * clear_words <= v->clear.stride)),
+                  "moe prefill rows: clear_words needs the clear view and must stay inside a row's stride");
+    hipStream_t st = hs(stream);
+    prefill_rows_prologue_kernel<<<rows, 256, 0, st>>>(*v, wv.experts, wv.top_k, clear_words);
+    const PrefillViews views{v->input.base, v->input.stride, RoutesView{shell.routes, v->routes.stride, wv.top_k}, shell.status, v->status.stride,
+                             v->job_status, shell.rawdots, v->rawdots.stride, v->rawdots_bf16 ? 1U : 0U, v->plan, v->h_f16};
+    return enqueue_prefill_core(wv, views, rows, st);
+}
 
 int32_t mi355_moe_strided_enqueue_prologue(const mi355_moe_weights* w, const mi355_moe_rows_strided* v, uint32_t rows, uint32_t clear_words, mi355_stream stream) {
     mi355_moe_weights wv; RowsK k;

@@ -2352,28 +2352,32 @@ int32_t mi355_moe_enqueue_layer_normed(const mi355_route_policy* p, const float*
     return enqueue_layer(p, router_weight, logit_bias, scores, LayerNorm{true, norm_weight, norm_eps, normed}, w, r, rows, form, stream);
 }
 
-int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
-    mi355_moe_weights wv;
-    if (const int32_t rc = check_moe(w, r, rows, wv, kPrefillClass)) return rc;
-    STRIX_REQUIRE(form <= MI355_COMBINE_NONE, "moe prefill: unknown combine form");
-    STRIX_REQUIRE(r->input && r->input_kind == MI355_INPUT_F16, "moe prefill: the fp16 form takes fp16 input rows");
-    STRIX_REQUIRE(r->input_stride % 16U == 0 && aligned(r->input, 16), "moe prefill: input rows must be 16-byte aligned");
-    STRIX_REQUIRE(r->h_f16 && aligned(r->h_f16, 16), "moe prefill: h_f16 workspace is null or misaligned");
-    STRIX_REQUIRE(rows <= 65535U, "moe prefill: at most 65535 rows per call");
-    STRIX_REQUIRE(wv.hidden % 128U == 0 && wv.ffn % 64U == 0, "moe prefill: hidden must be a multiple of 128, ffn of 64");
+}  // extern "C"
+namespace {
+// What the prefill kernels see of the caller's rows: dense bundles and the strided PrefillRows views fill it alike.
+struct PrefillViews {
+    const void* input; uint64_t input_stride;
+    RoutesView routes;
+    uint32_t* status; uint64_t status_rs;
+    uint32_t* job_status;
+    float* rawdots; uint64_t rawdots_rs;          // rawdots_rs == 0: dense [assignment][hidden]
+    uint32_t rawdots_bf16;
+    uint32_t* plan;
+    void* h_f16;
+};
+// expert plan, sub-block sums of the input rows, gate / up + SwiGLU, down rows (the status words are already written)
+int32_t enqueue_prefill_core(const mi355_moe_weights& wv, const PrefillViews& v, uint32_t rows, hipStream_t st) {
     const uint32_t assignments = rows * wv.top_k, bound = plan_item_bound(wv.experts, assignments, kPfTile);
-    hipStream_t st = hs(stream);
-    clear_validate_kernel<<<rows, 64, 0, st>>>(r->routes, r->route_weights, wv.experts, wv.top_k, r->status, r->job_status);
-    launch_plan(dense_routes(r->routes, wv.top_k), wv.experts, assignments, kPfTile, bound, r->plan, st);
+    launch_plan(v.routes, wv.experts, assignments, kPfTile, bound, v.plan, st);
     PrefillArgs a{};
-    a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.swiglu_limit = wv.swiglu_limit; a.x = static_cast<const uint8_t*>(r->input); a.x_stride = r->input_stride;
-    uint8_t* ws = static_cast<uint8_t*>(r->h_f16);
+    a.top_k = wv.top_k; a.exp_kind = wv.exp_kind; a.swiglu_limit = wv.swiglu_limit; a.x = static_cast<const uint8_t*>(v.input); a.x_stride = v.input_stride;
+    uint8_t* ws = static_cast<uint8_t*>(v.h_f16);
     a.h = reinterpret_cast<_Float16*>(ws); a.h_lo = reinterpret_cast<_Float16*>(ws + pf_h_plane_bytes(assignments, wv.ffn));
     a.h_sums = ws + pf_h_bytes(assignments, wv.ffn);
     uint8_t* x_sums = a.h_sums + static_cast<size_t>(assignments) * pf_sum_row_bytes(wv.ffn);
     a.x_sums = x_sums;
-    a.rawdots = r->rawdots; a.plan = r->plan; a.experts = wv.experts; a.assignments = assignments;
-    a.status = r->status; a.job_status = r->job_status; a.items = bound;
+    a.rawdots = v.rawdots; a.rawdots_rs = v.rawdots_rs; a.rawdots_bf16 = v.rawdots_bf16; a.plan = v.plan; a.experts = wv.experts; a.assignments = assignments;
+    a.status = v.status; a.status_rs = v.status_rs; a.job_status = v.job_status; a.items = bound;
     token_sums_kernel<<<rows, 256, 0, st>>>(a.x, a.x_stride, wv.hidden, x_sums);
     if (pf_sum_slots(wv.ffn) != wv.ffn / 32U) clear_sum_padding_kernel<<<assignments, 64, 0, st>>>(a.h_sums, wv.ffn);
     const uint32_t items_at = plan_items_at(wv.experts, assignments), order_at = plan_order_at(wv.experts), item_slots = (bound + 7U) / 8U * 8U;
@@ -2410,6 +2414,24 @@ int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_mo
         }
     }
     STRIX_LAUNCHED("moe prefill f16");
+    return MI355_OK;
+}
+}  // namespace
+extern "C" {
+
+int32_t mi355_moe_enqueue_prefill_f16(const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
+    mi355_moe_weights wv;
+    if (const int32_t rc = check_moe(w, r, rows, wv, kPrefillClass)) return rc;
+    STRIX_REQUIRE(form <= MI355_COMBINE_NONE, "moe prefill: unknown combine form");
+    STRIX_REQUIRE(r->input && r->input_kind == MI355_INPUT_F16, "moe prefill: the fp16 form takes fp16 input rows");
+    STRIX_REQUIRE(r->input_stride % 16U == 0 && aligned(r->input, 16), "moe prefill: input rows must be 16-byte aligned");
+    STRIX_REQUIRE(r->h_f16 && aligned(r->h_f16, 16), "moe prefill: h_f16 workspace is null or misaligned");
+    STRIX_REQUIRE(rows <= 65535U, "moe prefill: at most 65535 rows per call");
+    STRIX_REQUIRE(wv.hidden % 128U == 0 && wv.ffn % 64U == 0, "moe prefill: hidden must be a multiple of 128, ffn of 64");
+    hipStream_t st = hs(stream);
+    clear_validate_kernel<<<rows, 64, 0, st>>>(r->routes, r->route_weights, wv.experts, wv.top_k, r->status, r->job_status);
+    const PrefillViews v{r->input, r->input_stride, dense_routes(r->routes, wv.top_k), r->status, 4, r->job_status, r->rawdots, 0, 0U, r->plan, r->h_f16};
+    if (const int32_t rc = enqueue_prefill_core(wv, v, rows, st)) return rc;
     if (form == MI355_COMBINE_NONE) return MI355_OK;
     return mi355_moe_enqueue_merge(w, r, rows, form, stream);
 }

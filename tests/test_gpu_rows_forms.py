@@ -304,3 +304,80 @@ def test_executor_job_nonfinite_fails_closed_and_limits(strix):
     assert L.mi355_executor_run(ex.handle, C.byref(job), None) == 0          # an empty job is nothing
     assert not L.mi355_executor_create(0, 256, 0) and not L.mi355_executor_create(16, 100, 0)
     ex.close()
+
+
+# ---------------------------------------------------------------------------------- the fp16 prefill over strided rows
+def _bf16_round(a):
+    b = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return (((b + 0x7fff + ((b >> 16) & 1)) & 0xffff0000).astype(np.uint32)).view(np.float32)
+
+
+@pytest.mark.parametrize("gate_type,down_type,H,I,E,K,T", [
+    (orc.Q4_K, orc.Q4_K, 1024, 512, 8, 2, 70),          # the register-operand kernels (one down pass)
+    (orc.Q8_0, orc.Q8_0, 512, 256, 4, 2, 33),           # the loader / multiplier kernels (two down passes: the rounding belongs to the second)
+    (orc.Q4_K, orc.Q4_K, 2048, 768, 16, 4, 9)])
+def test_prefill_rows_f16_strided_views(strix, gate_type, down_type, H, I, E, K, T):
+    """mi355_moe_enqueue_prefill_rows_f16 (known_rows::PrefillRows / enqueue_prefill with the fp16 form,
+    include/strix/hip_moe_q4k_a8_known_rows.hpp:75-111): every view strided inside one record per row. The unweighted outputs are
+    bit for bit those of the dense entry point (the same kernels behind another view), with rawdots_bf16 their bfloat16 rounding;
+    the prologue zeroes the clear words, overwrites the status words and flags a bad route or route weight; the caller's merge
+    over the same strided views gives the dense entry's combined rows."""
+    rng = np.random.default_rng(H + T)
+    if gate_type == orc.Q8_0:
+        gate, up = (orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, I, H)) * 0.05).astype(np.float32)) for _ in range(2))
+        down = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((E, H, I)) * 0.05).astype(np.float32))
+    else:
+        gate, up, down = make_layer(rng, H, I, E)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.int32)
+    wts = rng.random((T, K)).astype(np.float32)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T, prefill_f16=True, gate_type=gate_type, down_type=down_type)
+    dense_raw = layer.run_prefill_f16(dev(x), dev(ids), dev(wts), combine=strix.COMBINE_NONE).cpu().numpy().copy()
+    assert int(layer.status.sum()) == 0
+    dense_out = layer.run_prefill_f16(dev(x), dev(ids), dev(wts)).cpu().numpy().copy()
+
+    sizes = dict(input=2 * H, routes=4 * K, route_weights=4 * K, status=4, clear=4 * H, rawdots=4 * K * H)
+    at, off = {}, 0
+    for f, n in sizes.items():
+        at[f] = off
+        off += pad16(n) + 32
+    stride = pad16(off + 16)
+    for bf16 in (False, True):
+        buf = torch.full((T, stride), 0x5A, dtype=torch.uint8, device="cuda")
+        put = lambda f, a: buf.__setitem__((slice(None), slice(at[f], at[f] + sizes[f])), torch.from_numpy(np.ascontiguousarray(a)).view(torch.uint8).reshape(T, -1).cuda())
+        get = lambda f, dt, shape: buf[:, at[f]: at[f] + sizes[f]].contiguous().cpu().numpy().view(dt).reshape((T,) + shape)
+        put("input", x); put("routes", ids); put("route_weights", wts)
+        v = strix.PrefillRows()
+        for f in sizes:
+            setattr(v, f, strix.Strided(buf.data_ptr() + at[f], stride))
+        v.rawdots_bf16 = 1 if bf16 else 0
+        layer.run_prefill_rows_f16(v, T, clear_words=H - 7)
+        torch.cuda.synchronize()
+        raw = get("rawdots", np.float32, (K, H))
+        assert np.array_equal(bits(raw), bits(_bf16_round(dense_raw) if bf16 else dense_raw)), bf16
+        clear = get("clear", np.uint32, (H,))
+        assert np.all(clear[:, :H - 7] == 0) and np.all(clear[:, H - 7:] == 0x5A5A5A5A)
+        assert np.all(get("status", np.uint32, (1,)) == 0) and int(layer.job_status[0]) == 0
+        assert np.all(buf[:, at["status"] + 4: at["clear"]].cpu().numpy() == 0x5A)          # nothing past a field's extent
+    # the caller's merge over the same views (fp32 rawdots): the dense entry's combined rows
+    buf = torch.full((T, stride), 0x5A, dtype=torch.uint8, device="cuda")
+    put = lambda f, a: buf.__setitem__((slice(None), slice(at[f], at[f] + sizes[f])), torch.from_numpy(np.ascontiguousarray(a)).view(torch.uint8).reshape(T, -1).cuda())
+    put("input", x); put("routes", ids); put("route_weights", wts)
+    v = strix.PrefillRows()
+    for f in sizes:
+        setattr(v, f, strix.Strided(buf.data_ptr() + at[f], stride))
+    layer.run_prefill_rows_f16(v, T)
+    merged = strix.combine(strix.COMBINE_FMA_SLOT, torch.from_numpy(dense_raw).cuda(), dev(wts), torch.zeros((T, H), dtype=torch.float32, device="cuda"))
+    assert np.array_equal(bits(merged.cpu().numpy()), bits(dense_out))
+    # a route that names no expert and a non-finite route weight: bit 1 in those rows, overwritten stale words elsewhere
+    bad_ids, bad_w = ids.copy(), wts.copy()
+    bad_ids[1, 0] = E
+    bad_w[T - 1, K - 1] = np.inf
+    put("routes", bad_ids); put("route_weights", bad_w)
+    layer.run_prefill_rows_f16(v, T)
+    torch.cuda.synchronize()
+    status = buf[:, at["status"]: at["status"] + 4].contiguous().cpu().numpy().view(np.uint32)[:, 0]
+    want = np.zeros(T, np.uint32); want[1] = 1; want[T - 1] = 1
+    assert np.array_equal(status, want)
+    with pytest.raises(strix.StrixError, match="clear_words"):
+        layer.run_prefill_rows_f16(v, T, clear_words=stride)
