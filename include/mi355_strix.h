@@ -264,6 +264,10 @@ int32_t mi355_moe_enqueue_layer_back(const mi355_route_policy* policy, const flo
  * are the exact router's either way. amount != 0 displaces the early logits (by amount * 1e-3 * a per-expert integer in
  * -8..7) so that a test can make the choices differ; 0 (the default) restores them. Process-wide; not for production use. */
 void mi355_debug_early_route_perturb(uint32_t amount);
+/* Test and measurement aid (no counterpart in the reference): the down rows + combine launch of a decode batch streams dense rows of at
+ * most four super-blocks as contiguous stages; on = 0 sends them through the 144-byte-block stages that every other shape uses, so that
+ * the two forms can be compared (same bits). Process-wide; the default is on. */
+void mi355_debug_down_merge_flat(uint32_t on);
 
 /* The scalar gate of an always-on shared expert (tensor ffn_gate_inp_shexp, fp32 [hidden]): gate[row * gate_stride] =
  * 1 / (1 + exp(-dot(x[row], scalar_weight))), the reference's shared_gate_dot (src/hip_shared_expert_launcher.hip:624-645): 256

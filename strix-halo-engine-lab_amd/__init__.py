@@ -261,7 +261,7 @@ def lib():
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
            "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
-           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue_combine", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_static_workspace_prepare", "mi355_moe_enqueue_prefill_f16", "mi355_moe_enqueue_prefill_rows_f16", "mi355_moe_prefill_f16_workspace_bytes",
+           "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue_combine", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_debug_down_merge_flat", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_static_workspace_prepare", "mi355_moe_enqueue_prefill_f16", "mi355_moe_enqueue_prefill_rows_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_shared_gate", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe", "mi355_a8_enqueue_serial_prologue_probe", "mi355_a8_enqueue_quantize_only",
            "mi355_a8_enqueue_down_activation_quantize", "mi355_a8_enqueue_down_rawdots", "mi355_a8_enqueue_down_rawdots_merge",
            "mi355_a8_validate_union", "mi355_a8_enqueue_probe_union", "mi355_a8_validate_down_union",

@@ -145,4 +145,119 @@ __device__ __forceinline__ float sweep_block_lanes(lds_u8* const (&slots)[DEPTH]
     return value;
 }
 
+// ---------------------------------------------------------------------------------------------------------------- flat rows
+// 64 dense rows of B super-blocks against ONE activation row, as the byte stream they are: 64 * B blocks = B stages of 64 blocks,
+// each stage 9,216 contiguous bytes (nine 1 KB pieces). Lane l of stage s evaluates block g = 64 s + l, which is block g % B of
+// row g / B, so the lane's activation share changes from stage to stage: the row's A8 image (codes, deltas, sums: 320 B bytes)
+// is copied to LDS once and every lane reads its block's 320 bytes from there. The four pair terms of every block are kept in
+// registers; at the end they are laid out in LDS in block order, where lane r finds the terms of its row's B blocks side by
+// side and adds them in ascending order: acc[p] = ((0 + t_0[p]) + t_1[p]) + ..., value = (acc0 + acc1) + (acc2 + acc3) - the
+// reference's chain (src/cpu/core/routed_expert.cpp:73-108), the bits of the lane-per-row sweep.
+// slots: DEPTH separate LDS objects of >= 9,216 bytes (slot 0 also serves the final exchange: B * 1 KB), act: >= 320 * B bytes of LDS;
+// nothing in flight on entry, everything landed and consumed on exit.
+constexpr uint32_t kFlatStageBytes = 9216;
+__host__ __device__ constexpr uint32_t flat_act_bytes(uint32_t B) { return 320U * B; }
+
+template <int B, int DEPTH>
+__device__ __forceinline__ float sweep_flat_rows(lds_u8* const (&slots)[DEPTH], lds_u8* act, const uint8_t* rows, const A8Image& img, uint32_t image_row) {
+    static_assert(B >= 1 && B <= 9 && DEPTH >= 2 && DEPTH <= 4, "flat rows: 1..9 super-blocks per row (the exchange fits slot 0), ring of 2..4 slots");
+    typedef const __attribute__((address_space(3))) u32x4 lds_u32x4;
+    typedef const __attribute__((address_space(3))) f32x4 lds_f32x4;
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    typedef const __attribute__((address_space(3))) i32x4 lds_i32x4;
+    const uint32_t lane = threadIdx.x & 63U;
+    // the activation row: codes 256 B | deltas 32 B | sums 32 B bytes, in pieces of 16 (20 B pieces, at most three copy instructions)
+    constexpr uint32_t kActPieces = 20U * B, kActCopies = (kActPieces + 63U) / 64U;
+    {
+        const uint8_t* codes = reinterpret_cast<const uint8_t*>(img.codes_of(image_row));
+        const uint8_t* deltas = reinterpret_cast<const uint8_t*>(img.deltas_of(image_row));
+        const uint8_t* sums = reinterpret_cast<const uint8_t*>(img.sums_of(image_row));
+#pragma unroll
+        for (uint32_t i = 0; i < kActCopies; ++i) {
+            const uint32_t piece = i * 64U + lane;
+            const uint8_t* src = piece < 16U * B ? codes + 16U * piece : piece < 18U * B ? deltas + 16U * (piece - 16U * B) : sums + 16U * (piece - 18U * B);
+            if (piece < kActPieces)                                // (the lanes past the image copy nothing)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src, (__attribute__((address_space(3))) void*)(act + 1024U * i), 16, 0, 0);
+        }
+    }
+    const auto start = [&](uint32_t s, lds_u8* slot) {
+        const uint8_t* base = rows + static_cast<size_t>(s) * kFlatStageBytes + 16U * lane;
+#pragma unroll
+        for (uint32_t i = 0; i < kBlockLaneCopies; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + 1024U * i),
+                                             (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
+    };
+#pragma unroll
+    for (int s = 0; s < DEPTH - 1; ++s)
+        if (s < B) start(static_cast<uint32_t>(s), slots[s]);
+    float t[B][4];
+#pragma unroll
+    for (int s = 0; s < B; ++s) {
+        // started so far: the activation image and stages 0 .. min(B, s + DEPTH - 1) - 1; stage s (and everything older) must have landed
+        const int last = s + DEPTH - 1 < B ? s + DEPTH - 1 : B, ahead = last - 1 - s;
+        asm volatile("" ::: "memory");          // a stage's LDS reads stay inside the stage (hoisted, the three activation shares alone fill the register file)
+        if (ahead == 0) block_lane_wait<0>();
+        else if (ahead == 1) block_lane_wait<kBlockLaneCopies>();
+        else if (ahead == 2) block_lane_wait<2 * kBlockLaneCopies>();
+        else block_lane_wait<3 * kBlockLaneCopies>();
+        if (s + DEPTH - 1 < B) start(static_cast<uint32_t>(s + DEPTH - 1), slots[(s + DEPTH - 1) % DEPTH]);
+        const uint32_t b = (64U * static_cast<uint32_t>(s) + lane) % static_cast<uint32_t>(B);
+        u32x4 code[16];
+        float delta[8], fsum[8];
+        lds_u32x4* cs = (lds_u32x4*)(act + 256U * b);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) code[i] = cs[i];
+        lds_f32x4* ds = (lds_f32x4*)(act + 256U * B + 32U * b);
+        const f32x4 d0 = ds[0], d1 = ds[1];
+        lds_i32x4* ss = (lds_i32x4*)(act + 288U * B + 32U * b);
+        const i32x4 s0 = ss[0], s1 = ss[1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            delta[j] = d0[j]; delta[4 + j] = d1[j];
+            fsum[j] = static_cast<float>(s0[j]); fsum[4 + j] = static_cast<float>(s1[j]);
+        }
+        lds_u32x4* blk = (lds_u32x4*)(slots[s % DEPTH] + lane * 144U);
+        const u32x4 hd = blk[0];
+        u32x4 q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = blk[1 + i];
+        const float dd = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
+        uint32_t sc[8], mn[8];
+        q4k_factors<0>(hd, sc[0], mn[0]); q4k_factors<1>(hd, sc[1], mn[1]); q4k_factors<2>(hd, sc[2], mn[2]); q4k_factors<3>(hd, sc[3], mn[3]);
+        q4k_factors<4>(hd, sc[4], mn[4]); q4k_factors<5>(hd, sc[5], mn[5]); q4k_factors<6>(hd, sc[6], mn[6]); q4k_factors<7>(hd, sc[7], mn[7]);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t wq[8] = {q[2 * p].x, q[2 * p].y, q[2 * p].z, q[2 * p].w, q[2 * p + 1].x, q[2 * p + 1].y, q[2 * p + 1].z, q[2 * p + 1].w};
+            const uint32_t c[16] = {code[4 * p].x, code[4 * p].y, code[4 * p].z, code[4 * p].w, code[4 * p + 1].x, code[4 * p + 1].y, code[4 * p + 1].z, code[4 * p + 1].w,
+                                    code[4 * p + 2].x, code[4 * p + 2].y, code[4 * p + 2].z, code[4 * p + 2].w, code[4 * p + 3].x, code[4 * p + 3].y, code[4 * p + 3].z, code[4 * p + 3].w};
+            int dot0 = 0, dot1 = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                dot0 = __builtin_amdgcn_sdot4(static_cast<int>(wq[k] & 0x0f0f0f0fU), static_cast<int>(c[k]), dot0, false);
+                dot1 = __builtin_amdgcn_sdot4(static_cast<int>((wq[k] >> 4) & 0x0f0f0f0fU), static_cast<int>(c[8 + k]), dot1, false);
+            }
+            const float D0 = dd * static_cast<float>(sc[2 * p]), D1 = dd * static_cast<float>(sc[2 * p + 1]);
+            const float M0 = dm * static_cast<float>(mn[2 * p]), M1 = dm * static_cast<float>(mn[2 * p + 1]);
+            const float u0 = D0 * static_cast<float>(dot0), v0 = M0 * fsum[2 * p];
+            const float u1 = D1 * static_cast<float>(dot1), v1 = M1 * fsum[2 * p + 1];
+            const float t0 = u0 - v0, t1 = u1 - v1;
+            const float x0 = delta[2 * p] * t0, x1 = delta[2 * p + 1] * t1;
+            t[s][p] = x0 + x1;
+        }
+    }
+    // the terms in block order: block g at 16 g bytes of slot 0 (every read of the slots has returned: the terms depend on them)
+    typedef __attribute__((address_space(3))) f32x4 lds_f32x4_w;
+#pragma unroll
+    for (int s = 0; s < B; ++s) *((lds_f32x4_w*)(slots[0] + 16U * (64U * static_cast<uint32_t>(s) + lane))) = f32x4{t[s][0], t[s][1], t[s][2], t[s][3]};
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // one wave: its own stores are visible to its own later reads once issued in order
+    float acc[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+        const f32x4 term = *((lds_f32x4*)(slots[0] + 16U * (static_cast<uint32_t>(B) * lane + static_cast<uint32_t>(b))));
+#pragma unroll
+        for (int p = 0; p < 4; ++p) acc[p] = acc[p] + term[p];
+    }
+    return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+}
+
 }  // namespace strix950

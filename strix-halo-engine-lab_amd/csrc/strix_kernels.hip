@@ -1206,6 +1206,79 @@ __global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_kernel(mi355_
     r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
 }
 
+// down_merge_kernel for dense rows of at most four super-blocks (down_row_stride = B * 144): the 64 rows of a column block stream as B
+// contiguous stages of 1 KB pieces instead of B stages of 64 separate 144-byte blocks (a read-only launch of this shape moves the
+// same bytes in 11.8 us against 14.4 us), the block terms meet in LDS in block order and lane = row adds them in ascending order.
+template <int B>
+__global__ __launch_bounds__(64 * kDownMergeSlots) void down_merge_flat_kernel(mi355_moe_weights w, RowsK r, uint32_t assignments, uint32_t form) {
+    // (the two ring slots are separate LDS objects, as in down_merge_kernel)
+    __shared__ __attribute__((aligned(16))) uint8_t ring_even[kDownMergeSlots][kFlatStageBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t ring_odd[kDownMergeSlots][kFlatStageBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t act_rows[kDownMergeSlots][flat_act_bytes(B)];
+    __shared__ float slot_value[kDownMergeSlots][64];
+    __shared__ uint32_t slot_order[kDownMergeSlots];
+    __shared__ float slot_weight[kDownMergeSlots];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63U, row = blockIdx.y, o = blockIdx.x * 64U + lane;
+    uint32_t job;                                                              // (requested together with the item: one round trip, not two)
+    uint32_t word[2] = {0U, 0U};
+    if (r.awords) {
+        if (lane < assignments) word[0] = r.awords[lane];
+        if (lane + 64U < assignments) word[1] = r.awords[lane + 64U];
+    } else job = *r.job_status;
+    const uint32_t a = row * w.top_k + wave;
+    const WorkItem item = work_item(w, r, plan_items_at(w.experts, assignments), a);
+    const uint32_t e = __builtin_amdgcn_readfirstlane(item.e), begin = __builtin_amdgcn_readfirstlane(item.begin), end = __builtin_amdgcn_readfirstlane(item.end);
+    if (r.awords) {
+        // a batch planned from early routes: the front launch left its non-finite flags per assignment; every workgroup folds them
+        // to the same job word, the first workgroup of a row publishes its row's
+        job = (__ballot(word[0] >> 31) | __ballot(word[1] >> 31)) ? static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION) : 0U;
+        if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) r.plan[kPlanLinesAt + kLinesEpoch] += 1U;      // this call's epoch is spent
+        if (job && blockIdx.x == 0 && wave == 0) {
+            const uint32_t lo = row * w.top_k, hi = lo + w.top_k;
+            const bool mine = (lane >= lo && lane < hi && (word[0] >> 31)) || (lane + 64U >= lo && lane + 64U < hi && (word[1] >> 31));
+            const bool any = __ballot(mine) != 0;
+            if (lane == 0) {
+                if (any) atomicOr(r.status_of(row), r.nonfinite_bit);
+                atomicOr(r.job_status, static_cast<uint32_t>(MI355_STATUS_NONFINITE_PROJECTION));
+            }
+        }
+    }
+    if (job & MI355_STATUS_NONFINITE_PROJECTION) return;                       // the whole job: no down rows, nothing published
+    float value = 0.0F;
+    if (begin != end) {                                                        // (an invalid route has no item: its row is flagged)
+        const uint32_t first = item.first ? item.first - 1U : ordered(r, plan_order_at(w.experts), begin);
+        // the 64 rows of the column block are one run of 64 * B super-blocks: B contiguous stages (q4k_blocks.hpp)
+        const uint8_t* rows = w.down + static_cast<size_t>(e) * w.down_expert_stride + static_cast<size_t>(blockIdx.x * 64U) * w.down_row_stride;
+        lds_u8* const slots[2] = {(lds_u8*)ring_even[wave], (lds_u8*)ring_odd[wave]};
+        const uint32_t src[1] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(first))};
+        value = sweep_flat_rows<B, 2>(slots, (lds_u8*)act_rows[wave], rows, r.h, src[0]);
+        r.rawdots_of(src[0], w.hidden)[o] = value;
+    }
+    slot_value[wave][lane] = value;
+    if (threadIdx.x == 0) {
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_order[k] = k;
+        if (form == MI355_COMBINE_MULADD_ASCENDING_EXPERT)
+            for (uint32_t i = 1; i < w.top_k; ++i)
+                for (uint32_t j = i; j > 0 && r.routes_of(row)[slot_order[j]] < r.routes_of(row)[slot_order[j - 1]]; --j) {
+                    const uint32_t t = slot_order[j]; slot_order[j] = slot_order[j - 1]; slot_order[j - 1] = t;
+                }
+        for (uint32_t k = 0; k < w.top_k; ++k) slot_weight[k] = r.route_weights_of(row)[slot_order[k]];
+    }
+    __syncthreads();
+    // fail closed: a row flagged by an earlier stage publishes nothing (the aggregate bit is the combine's own)
+    if (wave != 0 || (*r.status_of(row) & ~static_cast<uint32_t>(MI355_STATUS_AGGREGATE))) return;
+    float acc = 0.0F;
+    for (uint32_t k = 0; k < w.top_k; ++k) {
+        const float ev = slot_value[slot_order[k]][lane];
+        if (form == MI355_COMBINE_FMA_SLOT_ORDER && k + r.shared_slots < w.top_k) acc = __builtin_fmaf(slot_weight[k], ev, acc);
+        else acc = acc + slot_weight[k] * ev;
+    }
+    const float y = r.base ? acc + r.base_of(row)[o] : acc;
+    if (!finite_f(y)) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_AGGREGATE));
+    r.output[static_cast<size_t>(row) * r.output_stride + o] = y;
+}
+
+
 // The same for the smallest decode batches, in the 16-rows-per-wavefront layout of down_quad_kernel: a workgroup owns (row, 16
 // output columns), wave k sweeps the 16 down rows of the expert in slot k (lane = (row, pair)), the slots' values meet in LDS
 // and the first sixteen lanes of wave 0 fold them as merge_kernel does. One launch instead of two for one to six rows.
@@ -2203,10 +2276,25 @@ __global__ __launch_bounds__(64) void rmsnorm_rows_kernel(const uint8_t* x, uint
 
 struct LayerNorm { bool on; const float* weight; float eps; float* normed; };
 std::atomic<uint32_t> g_early_perturb{0};
+std::atomic<bool> g_down_merge_flat{true};
 
 // phase: 0 = the whole layer; 1 = its front half (router, A8 prologue, plan, gate / up); 2 = its back half (down rows, combine) on
 // what a front call with the same arguments left in the row views.
 enum { kLayerWhole = 0, kLayerFront = 1, kLayerBack = 2 };
+// down rows + combine of a decode batch whose every workgroup is resident: dense rows of at most four super-blocks stream as
+// contiguous stages (down_merge_flat_kernel), other shapes as 144-byte blocks of 64 rows (down_merge_kernel)
+void launch_down_merge(const mi355_moe_weights& wv, const RowsK& k, uint32_t rows, uint32_t items, uint32_t form, hipStream_t st) {
+    const dim3 grid(wv.hidden / 64U, rows);
+    const uint32_t threads = 64U * wv.top_k, B = wv.ffn / 256U;
+    const bool flat = wv.down_row_stride == static_cast<uint64_t>(B) * kQ4kBlock && wv.down_expert_stride % 16U == 0 && !k.h.table && k.h.codes &&
+                      aligned(k.h.codes, 16) && aligned(k.h.deltas, 16) && aligned(k.h.sums, 16) && wv.ffn % 256U == 0 && g_down_merge_flat.load(std::memory_order_relaxed);
+    if (flat && B == 1U) down_merge_flat_kernel<1><<<grid, threads, 0, st>>>(wv, k, items, form);
+    else if (flat && B == 2U) down_merge_flat_kernel<2><<<grid, threads, 0, st>>>(wv, k, items, form);
+    else if (flat && B == 3U) down_merge_flat_kernel<3><<<grid, threads, 0, st>>>(wv, k, items, form);
+    else if (flat && B == 4U) down_merge_flat_kernel<4><<<grid, threads, 0, st>>>(wv, k, items, form);
+    else down_merge_kernel<<<grid, threads, 0, st>>>(wv, k, items, form);
+}
+
 int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores, const LayerNorm& norm,
                       const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream, uint32_t phase = kLayerWhole) {
     const bool do_front = phase != kLayerBack, do_back = phase != kLayerFront;
@@ -2267,7 +2355,7 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
             STRIX_LAUNCHED("moe layer early routes + gate / up");
         }
         if (do_back) {
-            down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, st>>>(wv, k, items, form);
+            launch_down_merge(wv, k, rows, items, form, st);
             STRIX_LAUNCHED("moe layer experts + combine");
         }
         return MI355_OK;
@@ -2294,7 +2382,7 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
     if (!quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
         (wv.hidden / 64U) * rows <= compute_units()) {
-        down_merge_kernel<<<dim3(wv.hidden / 64U, rows), 64U * wv.top_k, 0, st>>>(wv, layer_rows(), items, form);
+        launch_down_merge(wv, layer_rows(), rows, items, form, st);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
     }
@@ -2330,6 +2418,7 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
 extern "C" {
 
 void mi355_debug_early_route_perturb(uint32_t amount) { g_early_perturb.store(amount, std::memory_order_relaxed); }
+void mi355_debug_down_merge_flat(uint32_t on) { g_down_merge_flat.store(on != 0, std::memory_order_relaxed); }
 
 int32_t mi355_moe_enqueue_layer(const mi355_route_policy* p, const float* router_weight, const float* logit_bias, float* scores,
                                 const mi355_moe_weights* w, const mi355_moe_rows* r, uint32_t rows, uint32_t form, mi355_stream stream) {
