@@ -663,7 +663,7 @@ def main():
                    "tokens": args.tokens, "distinct_experts_mean": u_mean},
         "hbm_GBps_layer": layer_gbps, "hbm_frac_layer": layer_gbps / HBM_PEAK_GBPS,
         "layer_algorithmic_bytes": cfg.layer_bytes(u_mean), "staged_call_us": staged_call_us,
-        "launch_us": {"front (layer_front_kernel)": front_us, "back (down_merge_kernel)": back_us,
+        "launch_us": {"front (layer_front_kernel)": front_us, "back (down rows + combine: down_merge_flat_kernel)": back_us,
                       "staged gate/up alone (project_wave_kernel)": project_us},
         "roofline": {"bound": "hbm", "kernel": "layer_front_kernel (early routes + A8 prologue + exact router + gate/up + SwiGLU + A8 re-quantise)",
                      "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
