@@ -115,6 +115,20 @@ typedef struct mi355_q8a8_view {
 } mi355_q8a8_view;
 int32_t mi355_gemv_q8_0_a8(const mi355_q8a8_view* view, mi355_stream stream);
 
+/* The reference's DENSE A8 profile of its Q8_0 projections (numerical profile dense-a8-q80-v1: the shared expert and the other dense
+ * sites of the decode step, src/hip_shared_expert_launcher.hip:1084-1142, row contract src/hip_q8_rows_gemv.hpp:1155-1170, stated on
+ * the host in tests/dense_a8_small_reference_tests.cpp:93-104):
+ *   quantiser, per block of 32: any non-finite x -> delta = NaN (0x7fc00000), codes 0; amax = max |x|; tiny = 0 < amax < 2^-119;
+ *     delta = (amax == 0 || tiny) ? 1 : amax / 127; code = tiny ? 0 : clamp(rint(x / delta), -127, 127)  (no status word, no sums);
+ *   product: acc = +0, then acc = fma(float(d_w[n][b]) * delta[r][b], float(sum_k q_w[n][b][k] * code[r][b][k]), acc) over the blocks b
+ *     in ascending order; y = isnan(acc) ? 0x7fc00000 : acc.
+ * The view is mi355_q8a8_view (accumulate must be 0; in % 64 == 0, in <= 8192, weight rows 4-byte aligned). With the shared gate
+ * (mi355_shared_gate), the SiLU of mi355_swiglu_quantize's h_out and one multiply by the gate these are the steps of the reference's
+ * shared expert in that profile. */
+int32_t mi355_dense_a8_quantize(const void* x, uint32_t input_kind, uint32_t rows, uint32_t width, uint64_t x_stride_bytes, int8_t* codes,
+                                float* deltas, mi355_stream stream);
+int32_t mi355_gemv_q8_0_a8_chain(const mi355_q8a8_view* view, mi355_stream stream);
+
 /* ------------------------------------------------------------------------------------------------------
  * Router. Replaces the Qwen route launcher (include/strix/hip_moe_route_launcher.hpp:16-30,
  * src/hip_moe_route_launcher.hip:322-365) with the host policy's bits (include/strix/moe/route_policy.hpp:99-156):

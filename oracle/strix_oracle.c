@@ -714,6 +714,45 @@ void orc_combine_shared(int form, uint32_t rows, uint32_t top_k, uint32_t shared
     }
 }
 
+void orc_dense_a8_quantize(const float* x, uint32_t width, int8_t* codes, float* deltas) {
+    for (uint32_t g = 0; g < width / 32; ++g) {                 /* src/hip_q8_rows_gemv.hpp:1232-1250 */
+        int bad = 0;
+        float amax = 0.0F;
+        for (uint32_t k = 0; k < 32; ++k) {
+            const float v = x[g * 32 + k];
+            bad |= !isfinite(v);
+            amax = fmaxf(amax, fabsf(v));
+        }
+        const int tiny = amax > 0.0F && amax < 0x1p-119F;
+        uint32_t nan_bits = 0x7fc00000U;
+        float nan_value;
+        memcpy(&nan_value, &nan_bits, 4);
+        const float delta = bad ? nan_value : (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
+        deltas[g] = delta;
+        for (uint32_t k = 0; k < 32; ++k) {
+            const float rounded = (bad || tiny) ? 0.0F : rintf(x[g * 32 + k] / delta);
+            codes[g * 32 + k] = (int8_t)(int)fminf(127.0F, fmaxf(-127.0F, rounded));
+        }
+    }
+}
+
+void orc_gemv_q8_0_a8_chain(const uint8_t* weight, uint32_t row_bytes, const int8_t* codes, const float* deltas, uint32_t in, uint32_t count,
+                            uint32_t rows, uint32_t x_stride, float* out, uint32_t out_stride) {
+    for (uint32_t r = 0; r < rows; ++r)
+        for (uint32_t o = 0; o < count; ++o) {
+            float acc = 0.0F;
+            for (uint32_t b = 0; b < in / 32; ++b) {            /* src/hip_q8_rows_gemv.hpp:1162-1165 */
+                const uint8_t* p = weight + (size_t)o * row_bytes + (size_t)b * 34;
+                int32_t dot = 0;
+                for (uint32_t k = 0; k < 32; ++k) dot += (int32_t)(int8_t)p[2 + k] * (int32_t)codes[(size_t)r * x_stride + b * 32 + k];
+                const float scale = orc_half_to_float((uint16_t)(p[0] | (p[1] << 8))) * deltas[(size_t)r * (x_stride / 32) + b];
+                acc = fmaf(scale, (float)dot, acc);
+            }
+            if (isnan(acc)) { const uint32_t bits = 0x7fc00000U; memcpy(&acc, &bits, 4); }
+            out[(size_t)r * out_stride + o] = acc;
+        }
+}
+
 void orc_shared_gate(const float* x, const float* w, uint32_t rows, uint32_t hidden, int exp_kind, float* gate, float* dots) {
     for (uint32_t r = 0; r < rows; ++r) {
         float s[256];

@@ -140,6 +140,17 @@ void orc_combine(int form, uint32_t rows, uint32_t top_k, uint32_t width, const 
 void orc_combine_shared(int form, uint32_t rows, uint32_t top_k, uint32_t shared_slots, uint32_t width, const float* w, const uint32_t* ids,
                         const float* raw, const float* base, float* y);
 
+/* ---- the dense A8 profile of the reference's Q8_0 projections (src/hip_q8_rows_gemv.hpp:1155-1170,1232-1250; host statement of the
+ * row contract: tests/dense_a8_small_reference_tests.cpp:93-104)
+ * quantiser, per block of 32: any non-finite x -> delta = NaN (0x7fc00000), codes 0; tiny = 0 < amax < 2^-119; delta = (amax == 0 ||
+ * tiny) ? 1 : amax / 127; code = tiny ? 0 : clamp(rint(x / delta), -127, 127).
+ * product: acc = +0; acc = fma(float(d_w) * delta, float(dot), acc) over the blocks in ascending order; a NaN result is 0x7fc00000.
+ * Parity: device code only in the reference (no compiled form here); pinned by order fixtures that the tree32 order of
+ * orc_gemv_q8_0_a8, an unfused multiply-add or the other association of the three-factor product changes. */
+void orc_dense_a8_quantize(const float* x, uint32_t width, int8_t* codes, float* deltas);
+void orc_gemv_q8_0_a8_chain(const uint8_t* weight, uint32_t row_bytes, const int8_t* codes, const float* deltas, uint32_t in, uint32_t count,
+                            uint32_t rows, uint32_t x_stride, float* out, uint32_t out_stride);
+
 /* ---- the shared expert's scalar gate (src/hip_shared_expert_launcher.hip:624-645 shared_gate_dot; tree src/core/ordered_reduce.hpp:8-16)
  * x [rows][hidden] fp32 values of the stored activations, w [hidden]; gate [rows] = 1 / (1 + exp(-dot)):
  * 256 thread-strided fma chains (thread t: features t, t + 256, ... ascending; the reference's build fuses `sum += x * w`, its

@@ -259,7 +259,7 @@ def lib():
 
 
 EXPORTS = ["mi355_last_error", "mi355_version", "mi355_numerical_identity", "mi355_dequantize_rows",
-           "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_moe_route",
+           "mi355_quantize_weight_rows", "mi355_quantize_a8", "mi355_gemv_q8_0_a8", "mi355_dense_a8_quantize", "mi355_gemv_q8_0_a8_chain", "mi355_moe_route",
            "mi355_moe_plan_words", "mi355_moe_enqueue_prologue", "mi355_moe_enqueue_csr", "mi355_moe_enqueue_project",
            "mi355_moe_enqueue_down", "mi355_moe_enqueue_merge", "mi355_moe_enqueue_combine", "mi355_moe_enqueue", "mi355_moe_enqueue_layer", "mi355_moe_enqueue_layer_front", "mi355_moe_enqueue_layer_back", "mi355_debug_early_route_perturb", "mi355_debug_down_merge_flat", "mi355_moe_enqueue_layer_normed", "mi355_moe_enqueue_layer_static", "mi355_static_workspace_prepare", "mi355_moe_enqueue_prefill_f16", "mi355_moe_enqueue_prefill_rows_f16", "mi355_moe_prefill_f16_workspace_bytes",
            "mi355_swiglu_quantize", "mi355_rmsnorm_f32", "mi355_shared_gate", "mi355_a8_validate", "mi355_a8_validate_down", "mi355_a8_enqueue_probe", "mi355_a8_enqueue_serial_prologue_probe", "mi355_a8_enqueue_quantize_only",
@@ -354,6 +354,25 @@ def gemv_q8_0_a8(weight, codes, deltas, n_in, count, out=None, accumulate=False,
     v = Q8a8View(weight.data_ptr(), codes.data_ptr(), deltas.data_ptr(), out.data_ptr(),
                  row_bytes_ or n_in // 32 * Q8_0_BLOCK, n_in, count, rows, codes.shape[1], out_stride or out.shape[1], int(accumulate))
     check(lib().mi355_gemv_q8_0_a8(C.byref(v), _stream()))
+    return out
+
+
+def dense_a8_quantize(x):
+    """The dense A8 profile's quantiser (mi355_dense_a8_quantize): a non-finite group gets delta = NaN and codes 0."""
+    rows, width = x.shape
+    codes = torch.zeros((rows, width), dtype=torch.int8, device=x.device)
+    deltas = torch.zeros((rows, width // 32), dtype=torch.float32, device=x.device)
+    check(lib().mi355_dense_a8_quantize(_p(x), input_kind(x), rows, width, C.c_uint64(x.stride(0) * x.element_size()), _p(codes), _p(deltas), _stream()))
+    return codes, deltas
+
+
+def gemv_q8_0_a8_chain(weight, codes, deltas, n_in, count):
+    """Q8_0 x A8 with the dense A8 profile's row contract: one ascending fma chain per output (mi355_gemv_q8_0_a8_chain)."""
+    rows = codes.shape[0]
+    out = torch.zeros((rows, count), dtype=torch.float32, device=codes.device)
+    v = Q8a8View(weight.data_ptr(), codes.data_ptr(), deltas.data_ptr(), out.data_ptr(), n_in // 32 * Q8_0_BLOCK, n_in, count, rows, codes.shape[1],
+                 out.shape[1], 0)
+    check(lib().mi355_gemv_q8_0_a8_chain(C.byref(v), _stream()))
     return out
 
 

@@ -162,9 +162,11 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* x, const 
 
 // One aligned group of 32 lanes per 32-value group; 8 groups per 256-thread block.
 // Reference: src/cpu/core/reference.cpp:35-55.
+// nan_delta: the dense A8 profile's rule for a group that holds a non-finite value (src/hip_q8_rows_gemv.hpp:1157-1161,1232-1250): its
+// delta is the canonical NaN 0x7fc00000 and its codes are 0, so that every product over the group is NaN.
 template <int KIND>
 __global__ __launch_bounds__(256) void quantize_a8_kernel(const uint8_t* x, uint64_t x_stride, uint32_t width, int8_t* codes,
-                                                          float* deltas, int32_t* sums, uint32_t* status) {
+                                                          float* deltas, int32_t* sums, uint32_t* status, uint32_t nan_delta = 0) {
     const uint32_t r = blockIdx.y, groups = width / 32U;
     const uint32_t g = blockIdx.x * 8U + (threadIdx.x >> 5), j = threadIdx.x & 31U;
     if (g >= groups) return;
@@ -172,12 +174,12 @@ __global__ __launch_bounds__(256) void quantize_a8_kernel(const uint8_t* x, uint
     const float amax = max32(__builtin_fabsf(v));
     const bool tiny = amax > 0.0F && amax < 0x1p-119F;
     const float delta = (amax == 0.0F || tiny) ? 1.0F : amax / 127.0F;
-    const int code = a8_code(v, delta, tiny);
-    const int sum = sum32_i(code);
     const int bad = or32_i(finite_f(v) ? 0 : 1);
+    const int code = (bad && nan_delta) ? 0 : a8_code(v, delta, tiny);
+    const int sum = sum32_i(code);
     codes[static_cast<size_t>(r) * width + g * 32U + j] = static_cast<int8_t>(code);
     if (j == 0) {
-        deltas[static_cast<size_t>(r) * groups + g] = delta;
+        deltas[static_cast<size_t>(r) * groups + g] = (bad && nan_delta) ? __builtin_bit_cast(float, 0x7fc00000U) : delta;
         if (sums) sums[static_cast<size_t>(r) * groups + g] = sum;
         if (bad && status) atomicOr(&status[r], static_cast<uint32_t>(MI355_STATUS_NONFINITE_ACTIVATION));
     }
@@ -189,9 +191,15 @@ __global__ __launch_bounds__(256) void quantize_a8_kernel(const uint8_t* x, uint
 // Reference: src/cpu/core/reference.cpp:57-84, src/core/integer_math.hpp:11-13,43-47.
 // DW: the weight rows are 4-byte aligned. A block (34 bytes: fp16 scale, 32 codes) is then fetched as nine aligned dwords
 // (two 128-bit loads and one 32-bit load) around its codes and shifted into place, instead of seventeen 16-bit loads.
+// CHAIN (RB = 1): the row contract of the reference's dense A8 profile (src/hip_q8_rows_gemv.hpp:1155-1170; host statement
+// tests/dense_a8_small_reference_tests.cpp:93-104): acc = +0, then for the blocks in ascending order acc = fma(float(d_w) * delta,
+// float(dot), acc), and a NaN result is stored as 0x7fc00000. The lanes evaluate their blocks as before and leave every block's
+// (scale, dot) pair in LDS; lane 0 of the output's 32 lanes then walks them in order.
+constexpr uint32_t kGemvChainMaxGroups = 256;          // in <= 8192 (kDenseA8MaxWidth, src/hip_q8_rows_gemv.hpp:1176)
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
-template <int RB, bool DW>
+template <int RB, bool DW, bool CHAIN = false>
 __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v) {
+    __shared__ float2 chain_pairs[CHAIN ? 8 : 1][CHAIN ? kGemvChainMaxGroups : 1];
     const uint32_t o = blockIdx.x * 8U + (threadIdx.x >> 5), l = threadIdx.x & 31U, row0 = blockIdx.y * RB;
     if (o >= v.count) return;
     const uint32_t groups = v.in / 32U;
@@ -229,9 +237,25 @@ __global__ __launch_bounds__(256) void gemv_q8_0_a8_kernel(mi355_q8a8_view v) {
                 dot = __builtin_amdgcn_sdot4(w[4], c.x, dot, false); dot = __builtin_amdgcn_sdot4(w[5], c.y, dot, false);
                 dot = __builtin_amdgcn_sdot4(w[6], c.z, dot, false); dot = __builtin_amdgcn_sdot4(w[7], c.w, dot, false);
                 const float xd = v.deltas[static_cast<size_t>(row0 + r) * (v.x_stride / 32U) + g];
-                lane[r] = lane[r] + static_cast<float>(dot) * (scale * xd);
+                if constexpr (CHAIN) chain_pairs[threadIdx.x >> 5][g] = make_float2(scale * xd, static_cast<float>(dot));
+                else lane[r] = lane[r] + static_cast<float>(dot) * (scale * xd);
             }
         }
+    }
+    if constexpr (CHAIN) {
+        // the pairs were written by lanes of this wave: program order of one wave's LDS accesses
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (l == 0) {
+            float acc = 0.0F;
+            for (uint32_t g = 0; g < groups; ++g) {
+                const float2 c = chain_pairs[threadIdx.x >> 5][g];
+                acc = __builtin_fmaf(c.x, c.y, acc);
+            }
+            v.out[static_cast<size_t>(row0) * v.out_stride + o] = acc != acc ? __builtin_bit_cast(float, 0x7fc00000U) : acc;
+        }
+        return;
     }
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
@@ -2055,6 +2079,36 @@ int32_t mi355_quantize_a8(const void* x, uint32_t kind, uint32_t rows, uint32_t 
     else if (kind == MI355_INPUT_F16) quantize_a8_kernel<1><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, sums, status);
     else quantize_a8_kernel<2><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, sums, status);
     STRIX_LAUNCHED("quantize_a8");
+    return MI355_OK;
+}
+
+int32_t mi355_dense_a8_quantize(const void* x, uint32_t kind, uint32_t rows, uint32_t width, uint64_t x_stride, int8_t* codes, float* deltas,
+                                mi355_stream stream) {
+    STRIX_REQUIRE(width % 32U == 0, "dense A8 activation width must be a multiple of 32");
+    STRIX_REQUIRE(kind <= MI355_INPUT_BF16, "dense A8: unknown input kind");
+    if (rows == 0 || width == 0) return MI355_OK;
+    STRIX_REQUIRE(x && codes && deltas, "dense A8: null pointer");
+    STRIX_REQUIRE(rows <= 65535U, "dense A8: at most 65535 rows per call");
+    const dim3 grid((width / 32U + 7U) / 8U, rows);
+    const uint8_t* xb = static_cast<const uint8_t*>(x);
+    if (kind == MI355_INPUT_F32) quantize_a8_kernel<0><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, nullptr, nullptr, 1U);
+    else if (kind == MI355_INPUT_F16) quantize_a8_kernel<1><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, nullptr, nullptr, 1U);
+    else quantize_a8_kernel<2><<<grid, 256, 0, hs(stream)>>>(xb, x_stride, width, codes, deltas, nullptr, nullptr, 1U);
+    STRIX_LAUNCHED("dense A8 quantize");
+    return MI355_OK;
+}
+
+int32_t mi355_gemv_q8_0_a8_chain(const mi355_q8a8_view* v, mi355_stream stream) {
+    STRIX_REQUIRE(v, "Q8_0 chain product: null view");
+    STRIX_REQUIRE(v->in % 64U == 0 && v->in <= 32U * kGemvChainMaxGroups, "Q8_0 chain product: width must be a multiple of 64, at most 8192");   // dense_a8_width, src/hip_q8_rows_gemv.hpp:1184
+    STRIX_REQUIRE(!v->accumulate, "Q8_0 chain product: the chain starts at +0 (no accumulate)");
+    if (v->rows == 0 || v->count == 0) return MI355_OK;
+    STRIX_REQUIRE(v->weight && v->codes && v->deltas && v->out, "Q8_0 chain product: null pointer");
+    STRIX_REQUIRE(aligned(v->weight, 4) && v->row_bytes % 4U == 0, "Q8_0 chain product: weight rows must be 4-byte aligned");
+    STRIX_REQUIRE(aligned(v->codes, 16) && v->x_stride % 32U == 0 && v->x_stride >= v->in, "Q8_0 chain product: codes must be 16-byte aligned with x_stride a multiple of 32");
+    STRIX_REQUIRE(v->row_bytes >= v->in / 32U * kQ80Block && v->out_stride >= v->count && v->rows <= 65535U, "Q8_0 chain product: stride shorter than the row, or too many rows");
+    gemv_q8_0_a8_kernel<1, true, true><<<dim3((v->count + 7U) / 8U, v->rows), 256, 0, hs(stream)>>>(*v);
+    STRIX_LAUNCHED("gemv_q8_0_a8 chain");
     return MI355_OK;
 }
 

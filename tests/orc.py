@@ -386,6 +386,23 @@ def combine_shared(form, w, ids, raw, shared_slots, base=None):
     return y
 
 
+def dense_a8_quantize(x):
+    x = np.ascontiguousarray(x, np.float32)
+    rows, width = x.shape
+    codes, deltas = np.zeros((rows, width), np.int8), np.zeros((rows, width // 32), np.float32)
+    for r in range(rows):
+        lib().orc_dense_a8_quantize(_ptr(x[r], f32p), width, _ptr(codes[r], i8p), _ptr(deltas[r], f32p))
+    return codes, deltas
+
+
+def gemv_q8_0_a8_chain(weight, codes, deltas, n_in, count):
+    weight, codes, deltas = np.ascontiguousarray(weight, np.uint8), np.ascontiguousarray(codes, np.int8), np.ascontiguousarray(deltas, np.float32)
+    rows = codes.shape[0]
+    out = np.zeros((rows, count), np.float32)
+    lib().orc_gemv_q8_0_a8_chain(_ptr(weight, u8p), n_in // 32 * 34, _ptr(codes, i8p), _ptr(deltas, f32p), n_in, count, rows, codes.shape[1], _ptr(out, f32p), count)
+    return out
+
+
 def shared_gate(x, w, exp_kind=EXP_GFX1151):
     x, w = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(w, np.float32)
     rows, hidden = x.shape

@@ -175,3 +175,78 @@ def test_shared_expert_with_its_sigmoid_gate(strix, down_type, H, I, E, K, S, T,
     assert np.array_equal(bits(layer.rawdots[:T].cpu().numpy()), bits(ref.rawdots))
     assert np.array_equal(bits(y.cpu().numpy()), bits(orc.combine_shared(form, w_ref, ids_ref, ref.rawdots, S, base=residual)))
     assert np.all(layer.status[:T].cpu().numpy() == 0)
+
+
+# ---------------------------------------------------------------------------------- the dense A8 profile of the shared expert
+@pytest.mark.parametrize("n_in,count,rows", [(4096, 2048, 1), (2048, 4096, 3), (64, 9, 2), (8192, 40, 1), (1024, 33, 5)])
+def test_dense_a8_quantiser_and_chain_product_bit_exact(strix, n_in, count, rows):
+    """mi355_dense_a8_quantize and mi355_gemv_q8_0_a8_chain against the oracle (the reference's dense A8 row contract,
+    src/hip_q8_rows_gemv.hpp:1155-1170; tests/dense_a8_small_reference_tests.cpp:93-104), with the reference test's scale patterns
+    (zero, denormal, infinity, NaN) in some blocks and a non-finite and a tiny group in the activations."""
+    rng = np.random.default_rng(n_in + count)
+    w = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((count, n_in)) * 0.05).astype(np.float32)).reshape(count, n_in // 32, 34)
+    special = [0x0000, 0x8000, 0x0001, 0x03ff, 0x0400, 0x7bff, 0x7c00, 0xfc00, 0x7e01]      # tests/dense_a8_small_reference_tests.cpp:43-44
+    for i, bits_ in enumerate(special):
+        o, b = (7 * i + 1) % count, (3 * i) % (n_in // 32)
+        w[o, b, 0], w[o, b, 1] = bits_ & 0xff, bits_ >> 8
+    w = w.reshape(count, -1)
+    x = (rng.standard_normal((rows, n_in)) * 2.0).astype(np.float32)
+    x[0, 33] = np.nan                                   # block 1 of row 0: delta NaN, codes 0
+    x[rows - 1, 0:32] = 2.0 ** -121                     # a tiny group: delta 1, codes 0
+    c, d = strix.dense_a8_quantize(dev(x))
+    c_ref, d_ref = orc.dense_a8_quantize(x)
+    assert np.array_equal(c.cpu().numpy(), c_ref) and np.array_equal(bits(d.cpu().numpy()), bits(d_ref))
+    assert bits(d_ref)[0, 1] == 0x7fc00000 and d_ref[rows - 1, 0] == 1.0
+    y = strix.gemv_q8_0_a8_chain(dev(w), c, d, n_in, count).cpu().numpy()
+    y_ref = orc.gemv_q8_0_a8_chain(w, c_ref, d_ref, n_in, count)
+    assert np.array_equal(bits(y), bits(y_ref))
+    assert np.all(bits(y_ref)[0] == 0x7fc00000)          # row 0: every output runs through the NaN block
+    # the order fixture on the device: 64 blocks, ascending chain 0, the kernel table's lane tree 61
+    blocks = 64
+    cx = np.zeros((1, blocks * 32), np.int8); cx[0, ::32] = 1
+    dl = np.ones((1, blocks), np.float32); dl[0, 0], dl[0, -1] = 2.0 ** 24, -(2.0 ** 24)
+    wf = np.zeros((1, blocks, 34), np.uint8); wf[0, :, 1] = 0x3c; wf[0, :, 2] = 1
+    wf = wf.reshape(1, -1)
+    assert strix.gemv_q8_0_a8_chain(dev(wf), dev(cx), dev(dl), blocks * 32, 1).item() == 0.0
+    assert strix.gemv_q8_0_a8(dev(wf), dev(cx), dev(dl), blocks * 32, 1).item() == 61.0
+    with pytest.raises(strix.StrixError, match="multiple of 64"):
+        strix.gemv_q8_0_a8_chain(dev(wf[:, :34]), dev(cx[:, :32]), dev(dl[:, :1]), 32, 1)
+
+
+def test_shared_expert_in_the_dense_a8_profile_end_to_end(strix):
+    """The reference's shared expert in its dense A8 profile, step by step (src/hip_shared_expert_launcher.hip:1084-1142): A8 image
+    of the bf16 row, gate and up by the ascending chain, h = silu(gate) * up with the device expf, A8 image of h, down by the chain,
+    one multiply by the sigmoid gate, stored as bfloat16 - every intermediate and the result bit for bit the oracle composition."""
+    H, I, T = 2048, 1024, 3
+    rng = np.random.default_rng(1142)
+    q8 = lambda shape: orc.quantize_rows(orc.Q8_0, (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    wg, wu, wd = q8((I, H)), q8((I, H)), q8((H, I))
+    scalar = (rng.standard_normal(H) * 0.05).astype(np.float32)
+    x_t = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(torch.bfloat16)
+    x32 = x_t.to(torch.float32).numpy()
+    # device
+    c, d = strix.dense_a8_quantize(x_t.cuda())
+    g = strix.gemv_q8_0_a8_chain(dev(wg), c, d, H, I)
+    u = strix.gemv_q8_0_a8_chain(dev(wu), c, d, H, I)
+    _, _, _, h, status = strix.swiglu_quantize(g, u, exp_kind=strix.EXP_GFX1151)          # h_out: (gate / (1 + expf(-gate))) * up
+    hc, hd = strix.dense_a8_quantize(h)
+    down = strix.gemv_q8_0_a8_chain(dev(wd), hc, hd, I, H)
+    gate = strix.shared_gate(x_t.cuda(), dev(scalar))
+    out = (gate * down).to(torch.bfloat16)                                                # one multiply, then the bfloat16 store
+    # oracle
+    c_r, d_r = orc.dense_a8_quantize(x32)
+    g_r, u_r = orc.gemv_q8_0_a8_chain(wg, c_r, d_r, H, I), orc.gemv_q8_0_a8_chain(wu, c_r, d_r, H, I)
+    assert np.array_equal(bits(g.cpu().numpy()), bits(g_r)) and np.array_equal(bits(u.cpu().numpy()), bits(u_r))
+    h_r = np.zeros((T, I), np.float32)
+    for t in range(T):
+        for grp in range(I // 32):
+            sl = slice(32 * grp, 32 * grp + 32)
+            ok, _, _, _, h_r[t, sl] = orc.swiglu_quantize(g_r[t, sl], u_r[t, sl], orc.EXP_GFX1151, float("inf"))
+            assert ok
+    assert np.array_equal(bits(h.cpu().numpy()), bits(h_r)) and int(status.sum()) == 0
+    hc_r, hd_r = orc.dense_a8_quantize(h_r)
+    down_r = orc.gemv_q8_0_a8_chain(wd, hc_r, hd_r, I, H)
+    assert np.array_equal(bits(down.cpu().numpy()), bits(down_r))
+    gate_r, _ = orc.shared_gate(x32, scalar)
+    want = torch.from_numpy((gate_r[:, None] * down_r).astype(np.float32)).to(torch.bfloat16)
+    assert torch.equal(out.cpu().view(torch.int16), want.view(torch.int16))

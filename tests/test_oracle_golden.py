@@ -1146,3 +1146,80 @@ def test_shared_slot_enters_the_combine_as_product_then_sum():
     i2 = np.array([[0, 1]], np.uint32)
     assert orc.combine_shared(0, ww, i2, one, 1)[0, 0] == 0.0
     assert orc.combine(0, ww, i2, one, np.zeros((1, 1), np.float32))[0, 0] == 2.0 ** -24
+
+
+def _q8_rows(scales_bits, codes):
+    """Q8_0 rows from fp16 scale bit patterns [rows][blocks] and codes [rows][blocks][32]."""
+    rows, blocks = scales_bits.shape
+    w = np.zeros((rows, blocks, 34), np.uint8)
+    w[:, :, 0], w[:, :, 1] = scales_bits & 0xff, scales_bits >> 8
+    w[:, :, 2:] = codes.astype(np.int8).view(np.uint8)
+    return w.reshape(rows, blocks * 34)
+
+
+def test_dense_a8_profile_order_fixtures():
+    """The row contract of the reference's dense A8 profile (src/hip_q8_rows_gemv.hpp:1155-1170; host statement
+    tests/dense_a8_small_reference_tests.cpp:93-104) as what the arithmetic fixes: (1) one ascending chain, not the 32-lane tree of
+    the CPU kernel table; (2) each step one fma; (3) the scale is float(d_w) * delta, formed first; (4) NaN scales and NaN deltas
+    give the canonical NaN, an infinite scale times a zero dot as well; (5) the quantiser's rules; (6) against float64."""
+    one, zero = 0x3c00, 0x0000
+    # (1) blocks 0..63 with dots 2^24, 1, 1, ..., -2^24 at the end: ascending fma chain keeps 2^24 through the ones (each lost), ends at 0;
+    #     lane-strided partial sums + tree (orc.gemv_q8_0_a8) give 61
+    blocks = 64
+    codes_x = np.zeros((1, blocks * 32), np.int8); codes_x[0, ::32] = 1                # one live code per block
+    deltas = np.ones((1, blocks), np.float32)
+    wcodes = np.zeros((1, blocks, 32), np.int32); wcodes[0, :, 0] = 1
+    sb = np.full((1, blocks), one, np.uint16)
+    deltas[0, 0], deltas[0, blocks - 1] = 2.0 ** 24, -(2.0 ** 24)
+    w = _q8_rows(sb, wcodes)
+    assert orc.gemv_q8_0_a8_chain(w, codes_x, deltas, blocks * 32, 1)[0, 0] == 0.0
+    assert orc.gemv_q8_0_a8(w, codes_x, deltas, blocks * 32, 1)[0][0, 0] == 61.0
+    # (2) fma: acc = -(2^24 + 2^13) from block 0, block 1 scale 2^12 + 1 (as delta), dot 2^12 + 1 -> exact product 2^24 + 2^13 + 1
+    cx = np.zeros((1, 64), np.int8); cx[0, 0] = 1
+    wc = np.zeros((1, 2, 32), np.int32); wc[0, 0, 0] = -1                              # block 0: dot -1
+    wc[0, 1, 0] = wc[0, 1, 1] = 127; cx[0, 32] = cx[0, 33] = 16                        # block 1: 2 * 127 * 16 = 4064
+    wc[0, 1, 2] = 33; cx[0, 34] = 1                                                    # + 33 = 4097 = 2^12 + 1
+    d2 = np.array([[2.0 ** 24 + 2.0 ** 13, 2.0 ** 12 + 1.0]], np.float32)
+    w2 = _q8_rows(np.full((1, 2), one, np.uint16), wc)
+    assert orc.gemv_q8_0_a8_chain(w2, cx, d2, 64, 1)[0, 0] == 1.0                      # product then sum would give 0
+    # (3) the three-factor product: float(d_w) * delta is rounded first, then multiplies the dot inside the fma. d_w = 1 + 2^-10,
+    #     delta = 1 + 342 * 2^-23, dot = 3: the other two associations (one rounding of the whole product; d * (delta * dot)) differ
+    sb3 = np.array([[0x3c01]], np.uint16)
+    wc3 = np.zeros((1, 1, 32), np.int32); wc3[0, 0, 0] = 3
+    cx3 = np.zeros((1, 32), np.int8); cx3[0, 0] = 1
+    d3 = np.array([[1.0 + 342 * 2.0 ** -23]], np.float32)
+    got = orc.gemv_q8_0_a8_chain(_q8_rows(sb3, wc3), cx3, d3, 32, 1)[0, 0]
+    dw, dl = np.float32(1.0 + 2.0 ** -10), d3[0, 0]
+    assert got == np.float32(np.float64(np.float32(dw * dl)) * 3.0)
+    assert got != np.float32(np.float64(dw) * np.float64(dl) * 3.0) and got != np.float32(np.float64(dw) * np.float64(np.float32(dl * np.float32(3.0))))
+    # (4) NaN and infinity: the reference's own scale patterns (tests/dense_a8_small_reference_tests.cpp:43-44)
+    for bits_, want_nan in ((0x7e01, True), (0x7c00, True), (0xfc00, True), (0x7bff, False)):
+        sbn = np.array([[bits_, one]], np.uint16)
+        wcn = np.zeros((1, 2, 32), np.int32); wcn[0, 1, 0] = 5                          # block 0: dot 0 (inf * 0 = NaN), block 1: 5
+        cxn = np.zeros((1, 64), np.int8); cxn[0, 32] = 1
+        y = orc.gemv_q8_0_a8_chain(_q8_rows(sbn, wcn), cxn, np.ones((1, 2), np.float32), 64, 1)
+        assert (bits(y)[0, 0] == 0x7fc00000) == want_nan and (want_nan or y[0, 0] == 5.0)
+    nan_delta = np.array([[np.nan, 1.0]], np.float32); nan_delta.view(np.uint32)[0, 0] = 0xffc12345
+    y = orc.gemv_q8_0_a8_chain(_q8_rows(np.full((1, 2), one, np.uint16), wcn), cxn, nan_delta, 64, 1)
+    assert bits(y)[0, 0] == 0x7fc00000
+    # (5) the quantiser
+    x = np.zeros((1, 128), np.float32)
+    x[0, :32] = np.linspace(-3.0, 3.0, 32)
+    x[0, 40] = np.inf                                                                   # block 1: non-finite
+    x[0, 64:96] = 2.0 ** -120                                                           # block 2: tiny
+    c, d = orc.dense_a8_quantize(x)
+    c_ref, d_ref, _, _ = orc.quantize_a8(x[:, :32].copy(), tiny_rule=True)
+    assert np.array_equal(c[0, :32], c_ref[0]) and d[0, 0] == d_ref[0, 0] == np.float32(3.0) / np.float32(127.0)
+    assert bits(d)[0, 1] == 0x7fc00000 and not c[0, 32:64].any()
+    assert d[0, 2] == 1.0 and not c[0, 64:96].any() and d[0, 3] == 1.0 and not c[0, 96:].any()
+    # (6) random rows against float64
+    rng = np.random.default_rng(1155)
+    wq = orc.quantize_rows(orc.Q8_0, (rng.standard_normal((24, 1024)) * 0.05).astype(np.float32))
+    xr = rng.standard_normal((3, 1024)).astype(np.float32)
+    cq, dq = orc.dense_a8_quantize(xr)
+    cq2, dq2, _, _ = orc.quantize_a8(xr, tiny_rule=True)
+    assert np.array_equal(cq, cq2) and np.array_equal(bits(dq), bits(dq2))              # finite rows: the kernel table's quantiser
+    y = orc.gemv_q8_0_a8_chain(wq, cq, dq, 1024, 24)
+    wd = orc.dequant_rows(orc.Q8_0, wq, 1024).astype(np.float64)
+    xd = (cq.astype(np.float64).reshape(3, 32, 32) * dq.astype(np.float64)[:, :, None]).reshape(3, 1024)
+    assert np.allclose(y, xd @ wd.T, rtol=0, atol=2e-5 * np.abs(xd @ wd.T).max())
