@@ -26,7 +26,11 @@ __host__ __device__ inline BlockLanes block_lanes(uint32_t B, uint32_t max_rows)
     return BlockLanes{B, R, R * B, R * B * 144U};
 }
 
-template <int N> __device__ __forceinline__ void block_lane_wait() { __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8)); }
+// At most N copies outstanding, and every LDS read of this wave returned. The second half matters: a copy writes LDS when its
+// data arrives, not in the order of the wave's LDS instructions - a read of a slot that is still queued in the LDS when the next
+// copy into that slot lands returns the new bytes (seen with eight waves per workgroup reading 29 KB each while a stage that hit in
+// the caches came back in under a microsecond). So a slot is overwritten only after the reads of it have returned.
+template <int N> __device__ __forceinline__ void block_lane_wait() { __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8)); }
 
 __device__ __forceinline__ float wave_shr1(float v) {       // lane l receives lane l - 1's value (lane 0: 0)
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138, 0xF, 0xF, true));

@@ -252,10 +252,12 @@ struct StageSource {
     }
 };
 
-// s_waitcnt vmcnt(N): at most N vector memory operations (here: stage copies, PER per stage) still outstanding.
+// s_waitcnt vmcnt(N) lgkmcnt(0): at most N vector memory operations (here: stage copies, PER per stage) still outstanding, and
+// every LDS read of this wave returned - the copy that follows overwrites a slot this wave has read, and a copy's data is
+// written to LDS when it arrives, whatever reads of the slot are still queued there.
 template <int N>
 __device__ __forceinline__ void wait_copies() {
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));
 }
 template <int PER>
 __device__ __forceinline__ void wait_stages_ahead(uint32_t ahead) {   // ahead = stages started after the one needed

@@ -3,13 +3,14 @@
 // The reference's logits are one ascending fma chain per (row, expert) - `hidden` dependent operations, microseconds of
 // latency during which nothing else of the layer can start. The expert *ids* do not need those bits: a dot product in any
 // summation order picks the same top-k except where two logits lie within rounding of each other. So the layer runs as
-//   1. early launch: logits as lane-parallel sums (one wave per row and four experts, operands straight into registers),
-//      top-k of the logits, one work item per assignment; the A8 prologue rides in the same launch;
-//   2. projection launch on the early ids, with the exact router beside it in the same launch (side blocks: the chain, the
-//      softmax, the selection, the weights - the reference's bits, written to the caller's ids / weights / scores); the block
-//      that finishes a row compares its exact ids with the early ones and, where they differ, waits for that assignment's
-//      speculative waves, recomputes the assignment on the exact expert and corrects the work item;
-//   3. down rows + combine on work items that are exact by then.
+//   1. front launch (layer_front_kernel): early blocks compute the logits as lane-parallel sums (one wave per row and four
+//      experts, operands straight into registers) and pick the top-k, the A8 prologue rides beside them, projection blocks
+//      sweep gate / up on the early ids as soon as those are tagged, and side blocks run the exact router (the chain, the
+//      softmax, the selection, the weights - the reference's bits, written to the caller's ids / weights / scores); the side
+//      block that finishes a row compares its exact ids with the early ones and, where they differ, waits for that
+//      assignment's speculative waves and repairs the assignment (a copy of the h image the row already holds under another
+//      slot, or a sweep on the exact expert) and writes the work items with the exact experts;
+//   2. down rows + combine on work items that are exact by then.
 // Every output is the exact router's; the early choice only decides which weights stream first.
 // Reference (the bits kept): tests/hip_moe_route_launcher_tests.hip:281-330, include/strix/moe/route_policy.hpp:99-156.
 #pragma once

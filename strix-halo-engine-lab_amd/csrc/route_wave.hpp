@@ -401,7 +401,7 @@ __device__ __forceinline__ float chain_run(const ChainStep& s, float acc) {
 }
 
 template <int N>
-__device__ __forceinline__ void chain_wait() { __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8)); }
+__device__ __forceinline__ void chain_wait() { __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8)); }      // (and every LDS read returned: the next copy reuses a slot this wave has read)
 
 // Logits of experts [e0, e0 + 8) for one row -> scores[row][expert] (+ bias), stored for readers in other workgroups of
 // the same launch. hidden % 32 == 0. slots: 4 separate LDS objects.

@@ -806,6 +806,58 @@ __device__ __forceinline__ void side_router_block(lds_u8* const (&slots)[2], con
         return;
     }
     uint64_t differ = __ballot(lane < K && static_cast<uint32_t>(tag) != expert);
+    // Most differences are the same experts in another order (two scores closer than the early logits resolve): the h image
+    // such a slot needs exists already, under the slot that held its expert, and is copied. Only an expert the early choice did not
+    // hold at all is swept again. (With the optional fp32 intermediates bound every differing slot is swept again.)
+    const uint32_t image_words = w.ffn / 4U + 2U * groups;         // codes, deltas, sums of one assignment, in 32-bit words
+    if (differ && !r.gate_out && !r.up_out && !r.h_out && K * image_words * 4U <= kSideSlotBytes) {
+        uint32_t src = 0xffU;
+        for (uint32_t j = 0; j < K; ++j) {
+            const uint32_t held = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(tag)), static_cast<int>(j)));
+            if (lane < K && expert == held) src = j;
+        }
+        uint64_t copy = __ballot(lane < K && ((differ >> lane) & 1ULL) && src != 0xffU);
+        if (copy) {
+            // every speculative wave of the row has to be through: a slot is read as a source or overwritten as a destination
+            bool through = false;
+            for (uint32_t spins = 0; spins < kFrontSpinLimit && !through; ++spins) {
+                const uint32_t seen = lane < K ? __hip_atomic_load(&r.awords[row * K + lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffffU : groups;
+                through = __ballot(seen < groups) == 0;
+                if (!through) __builtin_amdgcn_s_sleep(32);
+            }
+            asm volatile("" ::: "memory");
+            if (!through) {
+                if (lane == 0) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+                return;
+            }
+            const auto image_word = [&](uint32_t at, uint32_t i) -> uint32_t* {
+                if (i < w.ffn / 4U) return reinterpret_cast<uint32_t*>(r.h_codes_of(at)) + i;
+                if (i < w.ffn / 4U + groups) return reinterpret_cast<uint32_t*>(r.h_deltas_of(at)) + (i - w.ffn / 4U);
+                return reinterpret_cast<uint32_t*>(r.h_sums_of(at)) + (i - w.ffn / 4U - groups);
+            };
+            uint32_t* stage = reinterpret_cast<uint32_t*>((uint8_t*)slots[0]);
+            uint32_t flags = 0;                                   // bit k: the source of slot k carried the non-finite flag
+            for (uint64_t left = copy; left;) {                   // all sources first: a source may itself be a destination
+                const uint32_t k = static_cast<uint32_t>(__ffsll(static_cast<long long>(left))) - 1U;
+                left &= left - 1ULL;
+                const uint32_t from = row * K + static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(src), static_cast<int>(k)));
+                for (uint32_t i = lane; i < image_words; i += 64U) stage[k * image_words + i] = __hip_atomic_load(image_word(from, i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                flags |= (__hip_atomic_load(&r.awords[from], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 31) << k;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            for (uint64_t left = copy; left;) {
+                const uint32_t k = static_cast<uint32_t>(__ffsll(static_cast<long long>(left))) - 1U;
+                left &= left - 1ULL;
+                const uint32_t to = row * K + k;
+                for (uint32_t i = lane; i < image_words; i += 64U) __hip_atomic_store(image_word(to, i), stage[k * image_words + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (lane == 0) __hip_atomic_store(&r.awords[to], groups | (((flags >> k) & 1U) << 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");      // the staged images are out of LDS before a sweep reuses the slot
+            differ &= ~copy;
+        }
+    }
     while (differ) {
         const uint32_t k = static_cast<uint32_t>(__ffsll(static_cast<long long>(differ))) - 1U;
         differ &= differ - 1ULL;

@@ -867,6 +867,70 @@ def test_layer_entry_early_routes_are_verified_and_repaired(strix, E, H, I, K, T
     assert torch.equal(again, y) and torch.equal(ids2, ids) and torch.equal(wts2, wts)
 
 
+@pytest.mark.parametrize("E,H,I,K,T,amount", [(128, 2048, 768, 8, 8, 10), (32, 1024, 512, 4, 16, 40)])
+def test_layer_entry_repairs_reordered_slots_by_copying_their_h_image(strix, E, H, I, K, T, amount):
+    """Without the optional fp32 intermediates a slot whose exact expert the early choice held under ANOTHER slot of the row is
+    repaired by copying that slot's A8 image of h; only experts the early choice did not hold are swept again. Rows of both
+    kinds (and rows with both at once) must leave the bits of an undisturbed call: ids, weights, the A8 image of h, rawdots
+    (== the oracle's down rows on that image), the output (== the oracle's combine of them)."""
+    rng = np.random.default_rng(E + T + amount + 1000)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
+    ids_ref, w_ref, _, _ = orc.route(x.astype(np.float32), wr, K)
+    early = early_choice(x, wr, K, amount)
+    reordered = [r for r in range(T) if set(early[r]) == set(ids_ref[r]) and (early[r] != ids_ref[r]).any()]
+    replaced = [r for r in range(T) if set(early[r]) != set(ids_ref[r])]
+    assert len(reordered) >= 3 and len(replaced) >= 3
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T)
+    n = T * K
+    snapshot = lambda: [t[:n].clone() for t in (layer.down_codes, layer.down_deltas, layer.down_sums)] + [layer.rawdots[:T].clone()]
+    y0, ids0, w0, _ = layer.run_layer(dev(x), dev(wr))
+    y0, ids0, w0, plain = y0.clone(), ids0.clone(), w0.clone(), snapshot()
+    assert np.array_equal(ids0.cpu().numpy().astype(np.uint32), ids_ref) and np.array_equal(bits(w0.cpu().numpy()), bits(w_ref))
+    c, d, s, _ = orc.quantize_a8(x.astype(np.float32))
+    dc, dd_, ds = (t.cpu().numpy() for t in plain[:3])
+    ref_down = orc.routed_experts(H, I, K, gate, up, down, orc.Q4_K, c, d, s, ids_ref, down_only_from=(dc, dd_, ds))
+    assert np.array_equal(bits(plain[3].cpu().numpy()), bits(ref_down.rawdots))
+    assert np.array_equal(bits(y0.cpu().numpy()), bits(orc.combine(0, w_ref, ids_ref, ref_down.rawdots)))
+    for _ in range(3):
+        strix.lib().mi355_debug_early_route_perturb(amount)
+        try:
+            y, ids, wts, _ = layer.run_layer(dev(x), dev(wr))
+            y, ids, wts, repaired = y.clone(), ids.clone(), wts.clone(), snapshot()
+            torch.cuda.synchronize()
+        finally:
+            strix.lib().mi355_debug_early_route_perturb(0)
+        assert torch.equal(ids, ids0) and torch.equal(wts, w0)
+        for got, want in zip(repaired, plain):
+            assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+        assert torch.equal(y.view(torch.int32), y0.view(torch.int32))
+        assert np.all(layer.status[:T].cpu().numpy() == 0) and int(layer.job_status[0]) == 0
+
+
+def test_down_rows_of_a_decode_batch_give_the_same_bits_launch_after_launch(strix):
+    """The down rows of a decode batch stream through two LDS slots per wave, eight waves per workgroup. A copy into a slot lands
+    when its data arrives, not in the order of the wave's LDS instructions, so the slot's earlier reads have to be complete
+    before the copy is issued; with only 'issued' a read now and then returned the NEXT stage's bytes (a few launches in a
+    hundred, a few rows of one wave). The back half of the layer, launched 3000 times on one front half: every launch leaves the
+    first one's rawdots and output."""
+    E, H, I, K, T = 128, 2048, 768, 8, 7
+    rng = np.random.default_rng(535)
+    gate, up, down = make_layer(rng, H, I, E, full_entropy=True)
+    wr = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float16)
+    layer = strix.MoeLayer(H, I, E, K, dev(gate), dev(up), dev(down), T)
+    xd, wd = dev(x), dev(wr)
+    y, _, _, _ = layer.run_layer(xd, wd)
+    y, raw = y.clone(), layer.rawdots[:T].clone()
+    layer.run_layer(xd, wd, half="front")
+    bad = torch.zeros((), dtype=torch.int64, device=xd.device)
+    for _ in range(3000):
+        again, _, _, _ = layer.run_layer(xd, wd, half="back")
+        bad += (layer.rawdots[:T].view(torch.int32) != raw.view(torch.int32)).sum() + (again.view(torch.int32) != y.view(torch.int32)).sum()
+    assert int(bad) == 0
+
+
 @pytest.mark.parametrize("amount", [0, 500])
 def test_layer_entry_early_routes_nonfinite_flags_follow_the_exact_choice(strix, amount):
     """One expert carries a non-finite block scale. The displaced early choice sends rows to it that the exact router does not
