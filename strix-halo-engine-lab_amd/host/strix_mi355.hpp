@@ -10,6 +10,10 @@
 //   cpu::Q8a8View / Stream / Kernels            src/cpu/core/backend.hpp:52-73
 //   weight::Candidate / Plan / WeightView / KernelArguments / enqueue / enqueue_dense   include/strix/weight/resolve.hpp:67-84,
 //                                                                                     src/cpu/weight/registry.cpp:11-63
+//   weight::RuntimeCallbacks / ExecutionContext / Retirement / Hardware / RuntimeAdapter, bind_runtime, enqueue(.., context)
+//                                                                                     include/strix/weight/cache.hpp:6-33, runtime.hpp:5-13,
+//                                                                                     src/weight/cache.cpp:192-200 (the HIP binding:
+//                                                                                     strix_mi355_runtime.hpp, bind_native_runtime)
 //   moe_q4k_a8::Request .. Bindings, validate, enqueue_probe                          include/strix/moe_q4k_a8_contract.hpp:101-122,
 //                                                                                     include/strix/hip_moe_q4k_a8_probe.hpp:12
 //   moe_q4k_a8::DownRequest .. DownBindings, validate_down, enqueue_down_*, SlotMergeTail   include/strix/moe_a8_down_contract.hpp:39-54,
@@ -25,6 +29,8 @@
 #pragma once
 #include <cstddef>
 #include <cstdint>
+#include <functional>
+#include <memory>
 #include <limits>
 #include <stdexcept>
 #include <string>
@@ -90,8 +96,67 @@ struct Status { Error code; std::string detail; explicit operator bool() const {
 struct Shape { std::uint64_t dims[4]; std::uint8_t rank; };
 struct WeightView { TensorId tensor; FormatId storage; Shape shape; const std::uint8_t* payload; std::uint64_t payload_bytes; };   // payload: device memory
 struct Candidate { KernelId kernel; FormatId storage; ArithmeticId arithmetic; ImageId image; Backend backend; Strategy strategy; Exactness exactness; };
-struct Plan { Candidate selected; };
+struct Plan { Candidate selected; std::uint64_t workspace_bytes = 0; };
 struct KernelArguments { KernelId schema; std::uint32_t abi_revision; const void* data; std::size_t bytes; };
+// What a backend installs under the registry (include/strix/weight/cache.hpp:6-33, include/strix/weight/runtime.hpp:5-13,
+// include/strix/weight/resolve.hpp:7-15): allocation, events, the upload of a weight image, deferred reclamation and the typed
+// launch. strix_mi355_runtime.hpp binds them to HIP and to this library (bind_native_runtime).
+struct Retirement {
+    std::vector<void*> events;                 // last-use events: the allocation is reclaimed after all of them
+    std::vector<void*> unresolved_streams;     // streams whose last use could not be recorded: drained before reclamation
+    std::shared_ptr<void> reservation;         // released only after the allocation is actually freed
+};
+struct ExecutionContext;
+struct RuntimeCallbacks {
+    std::function<Status(std::uint64_t, void*&)> allocate;
+    std::function<void(void*)> free;
+    std::function<Status(ExecutionContext&, void*&)> record_event;
+    std::function<Status(ExecutionContext&, void*)> wait_event;
+    std::function<bool(void*)> event_complete;
+    std::function<void(void*)> destroy_event;
+    std::function<Status(const WeightView&, const Plan&, void*, ExecutionContext&)> convert;
+    std::function<void(void*, Retirement, ExecutionContext)> retire;       // takes the allocation, its fences and its budget; must not throw
+    std::function<Status(const Plan&, const WeightView&, const KernelArguments&, void*, void*, std::size_t, ExecutionContext&)> enqueue;
+};
+struct ExecutionContext {
+    Backend backend = Backend::cpu;
+    void* stream = nullptr;
+    std::uint32_t device_index = 0;
+    std::shared_ptr<const RuntimeCallbacks> callbacks;
+};
+struct Hardware {
+    Backend backend; std::string arch, compiler_id, device_class;
+    std::uint64_t isa_mask, free_bytes, cache_budget_bytes;
+    std::uint32_t registers_per_sm, registers_per_thread_limit;
+    std::uint32_t shared_bytes_per_sm, warp_or_wave;
+    double memory_bytes_per_second, lookup_per_second, dot4_per_second;
+    double valu_ops_per_second, matrix_ops_per_second;
+    bool valu_matrix_serialize;
+};
+struct RuntimeAdapter {
+    std::shared_ptr<const RuntimeCallbacks> callbacks;
+    std::function<Status(std::uint32_t, Hardware&)> query_hardware;
+};
+inline std::string current_compiler_id() {       // src/weight/runtime.cpp:3-13
+#if defined(__clang__)
+    return "clang/" __clang_version__;
+#elif defined(__GNUC__)
+    return "gcc/" __VERSION__;
+#else
+    return "unknown-compiler";
+#endif
+}
+// src/weight/runtime.cpp:15-24: the same refusals in the same order
+inline Status bind_runtime(Backend backend, const RuntimeAdapter& adapter, void* stream, std::uint32_t device, ExecutionContext& context, Hardware& hardware) {
+    if (!adapter.callbacks || !adapter.query_hardware) return {Error::unsupported_backend, "backend runtime not registered"};
+    Hardware h{};
+    Status status = adapter.query_hardware(device, h);
+    if (!status) return status;
+    if (h.backend != backend) return {Error::unsupported_backend, "capability query returned another backend"};
+    context = {backend, stream, device, adapter.callbacks};
+    hardware = std::move(h);
+    return {Error::ok, {}};
+}
 template <class Args> struct ArgumentTraits;
 template <class Args> KernelArguments arguments(Args& args) {
     using Type = std::remove_cv_t<Args>;
@@ -126,6 +191,18 @@ inline Status validate_q8_shape(const WeightView& weight, std::uint64_t count, s
     if (!weight.payload || weight.payload_bytes < count * (in / 32U) * 34U) return {Error::malformed, "Q8 weight payload shorter than its shape"};
     return {Error::ok, {}};
 }
+// The launch through a bound context (src/weight/cache.cpp:192-200): backend, storage, workspace, envelope, launcher - refused
+// in that order - then the backend's own enqueue callback.
+inline Status enqueue(const Plan& plan, const WeightView& view, const KernelArguments& args, void* output, void* workspace, std::size_t workspace_bytes,
+                      ExecutionContext& context) {
+    if (context.backend != plan.selected.backend) return {Error::unsupported_backend, "enqueue context backend differs"};
+    if (!(view.storage == plan.selected.storage)) return {Error::unknown_format, "enqueue storage differs"};
+    if (workspace_bytes < plan.workspace_bytes || (plan.workspace_bytes && !workspace)) return {Error::memory_budget, "workspace missing or too short"};
+    if (!args.data || !args.bytes || !args.schema || !args.abi_revision || !output) return {Error::malformed, "invalid typed argument envelope"};
+    if (!context.callbacks || !context.callbacks->enqueue) return {Error::unsupported_arithmetic, "backend has no registered launcher"};
+    return context.callbacks->enqueue(plan, view, args, output, workspace, workspace_bytes, context);
+}
+// The registration's own dispatch (src/cpu/weight/registry.cpp:11-32): what the enqueue callback of a bound context calls.
 inline Status enqueue(const Plan& plan, const WeightView& weight, const KernelArguments& envelope, void* output, void* /*workspace*/, std::size_t /*workspace_bytes*/) {
     if (plan.selected.kernel != q8_tree32_kernel || !(plan.selected.arithmetic == ArithmeticId{"cpu-q8a8-tree32", 1}) || plan.selected.strategy != Strategy::native)
         return {Error::unsupported_arithmetic, "the registry only provides the raw Q8_0 tree32 incumbent"};
@@ -143,11 +220,24 @@ inline Status enqueue(const Plan& plan, const WeightView& weight, const KernelAr
     if (rc != MI355_OK) return {rc == MI355_E_HIP ? Error::device_failure : Error::unsupported_shape, mi355_last_error()};
     return {Error::ok, {}};
 }
+// A context that carries only the launcher (src/cpu/weight/registry.cpp:49-59); strix_mi355_runtime.hpp's bind_native_runtime
+// gives one with allocation, events, upload and retirement as well.
+inline ExecutionContext execution_context() {
+    static const std::shared_ptr<const RuntimeCallbacks> callbacks = [] {
+        auto result = std::make_shared<RuntimeCallbacks>();
+        result->enqueue = [](const Plan& plan, const WeightView& weight, const KernelArguments& args, void* output, void* workspace, std::size_t bytes, ExecutionContext&) {
+            return enqueue(plan, weight, args, output, workspace, bytes);
+        };
+        return result;
+    }();
+    return {Backend::hip, nullptr, 0, callbacks};
+}
 inline Status enqueue_dense(const WeightView& weight, const DenseArguments& args) {
     std::size_t n;
     Plan plan{candidates(n)[0]};
+    ExecutionContext context = execution_context();
     DenseArguments launch = args;
-    return enqueue(plan, weight, arguments(launch), args.view.out, nullptr, 0);
+    return enqueue(plan, weight, arguments(launch), args.view.out, nullptr, 0, context);
 }
 }  // namespace weight
 

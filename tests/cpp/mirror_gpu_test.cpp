@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "strix_mi355.hpp"
+#include "strix_mi355_runtime.hpp"
 extern "C" {
 #include "strix_oracle.h"
 }
@@ -121,6 +122,88 @@ static void kernel_table() {
     other.shape.dims[1] = count + 1;
     envelope = wt::arguments(args);
     expect(wt::enqueue(plan, other, envelope, dout2.p, nullptr, 0).code == wt::Error::unsupported_shape, "weight::enqueue refuses a weight whose shape differs from the launch");
+}
+
+// ----------------------------------------------------------------------------------------------- the registry's runtime callbacks
+// include/strix/weight/cache.hpp:14-33 bound to HIP and to this library: a weight image allocated, uploaded from host memory
+// and launched through the context, on a stream of its own, with its last use recorded and the allocation retired.
+static void weight_runtime() {
+    namespace wt = m::weight;
+    hipStream_t stream{};
+    hip(hipStreamCreate(&stream), "hipStreamCreate");
+    wt::ExecutionContext context;
+    wt::Hardware hardware{};
+    expect(static_cast<bool>(wt::bind_native_runtime(stream, 0, context, hardware)) && context.backend == wt::Backend::hip && context.stream == stream &&
+               context.callbacks && hardware.backend == wt::Backend::hip && hardware.arch.rfind("gfx950", 0) == 0 && hardware.warp_or_wave == 64 &&
+               hardware.free_bytes > 0 && !hardware.compiler_id.empty(),
+           "weight::bind_native_runtime: HIP context on the caller's stream, hardware gfx950 / wave 64");
+    wt::RuntimeAdapter none;
+    wt::ExecutionContext unbound;
+    expect(wt::bind_runtime(wt::Backend::hip, none, stream, 0, unbound, hardware).code == wt::Error::unsupported_backend, "weight::bind_runtime refuses an adapter without callbacks");
+    wt::RuntimeAdapter adapter{context.callbacks, [](std::uint32_t, wt::Hardware& h) { h.backend = wt::Backend::cpu; return wt::Status{wt::Error::ok, {}}; }};
+    expect(wt::bind_runtime(wt::Backend::hip, adapter, stream, 0, unbound, hardware).code == wt::Error::unsupported_backend, "weight::bind_runtime refuses a capability query of another backend");
+    adapter.query_hardware = [](std::uint32_t, wt::Hardware& h) { h.backend = wt::Backend::hip; h.arch = "gfx950"; return wt::Status{wt::Error::ok, {}}; };
+    expect(static_cast<bool>(wt::bind_runtime(wt::Backend::hip, adapter, stream, 0, unbound, hardware)) && unbound.callbacks == context.callbacks, "weight::bind_runtime installs the adapter's callbacks");
+
+    const std::uint32_t width = 2048, count = 160;
+    const std::vector<float> x = normal(width, 1.0F);
+    std::vector<std::int8_t> c(width); std::vector<float> d(width / 32); std::vector<std::int32_t> sums(width / 32);
+    orc_quantize_a8(x.data(), width, c.data(), d.data(), sums.data(), 1);
+    const std::vector<std::uint8_t> w = q8_0_tensor(count, width, 0.05F);
+    std::vector<float> want(count);
+    const orc_q8a8_view ov{w.data(), c.data(), d.data(), want.data(), width / 32 * 34, width, count, 1, width, count, 0};
+    orc_gemv_q8_0_a8(&ov, 1);
+    Dev<std::int8_t> dc(c);
+    Dev<float> dd(d), dout(count);
+
+    // the image: allocate, upload from HOST memory, then the typed launch on the context's stream
+    void* image = nullptr;
+    const wt::WeightView host_view{11, {"gguf.q8_0", 1}, wt::Shape{{width, count, 0, 0}, 2}, w.data(), w.size()};
+    std::size_t n = 0;
+    wt::Plan plan{wt::candidates(n)[0]};
+    bool ok = static_cast<bool>(context.callbacks->allocate(w.size(), image)) && image != nullptr;
+    ok = ok && static_cast<bool>(context.callbacks->convert(host_view, plan, image, context));
+    wt::WeightView device_view = host_view;
+    device_view.payload = static_cast<const std::uint8_t*>(image);
+    wt::DenseArguments args{m::cpu::Q8a8View{device_view.payload, dc.p, dd.p, dout.p, width / 32 * 34, width, count, 1, width, count, 0}, m::cpu::Stream{}};
+    ok = ok && static_cast<bool>(wt::enqueue(plan, device_view, wt::arguments(args), dout.p, nullptr, 0, context));
+    void* last_use = nullptr;
+    ok = ok && static_cast<bool>(context.callbacks->record_event(context, last_use)) && last_use != nullptr;
+    wt::ExecutionContext other = context;
+    other.stream = nullptr;                                             // a consumer on another stream waits for the producer's event
+    ok = ok && static_cast<bool>(context.callbacks->wait_event(other, last_use));
+    hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+    expect(ok && context.callbacks->event_complete(last_use) && same_bits(dout.get(), want), "weight runtime: allocate + convert + enqueue on the context's stream == oracle");
+
+    // the refusals of the launch through a context, in the reference's order
+    wt::ExecutionContext cpu_context = context;
+    cpu_context.backend = wt::Backend::cpu;
+    wt::KernelArguments envelope = wt::arguments(args);
+    expect(wt::enqueue(plan, device_view, envelope, dout.p, nullptr, 0, cpu_context).code == wt::Error::unsupported_backend, "weight::enqueue(context) refuses another backend");
+    wt::WeightView q4 = device_view;
+    q4.storage = wt::FormatId{"gguf.q4_k", 1};
+    expect(wt::enqueue(plan, q4, envelope, dout.p, nullptr, 0, context).code == wt::Error::unknown_format, "weight::enqueue(context) refuses another storage");
+    wt::Plan hungry = plan;
+    hungry.workspace_bytes = 64;
+    expect(wt::enqueue(hungry, device_view, envelope, dout.p, nullptr, 0, context).code == wt::Error::memory_budget, "weight::enqueue(context) refuses a missing workspace");
+    expect(wt::enqueue(plan, device_view, envelope, nullptr, nullptr, 0, context).code == wt::Error::malformed, "weight::enqueue(context) refuses a null output");
+    wt::ExecutionContext bare{wt::Backend::hip, stream, 0, nullptr};
+    expect(wt::enqueue(plan, device_view, envelope, dout.p, nullptr, 0, bare).code == wt::Error::unsupported_arithmetic, "weight::enqueue(context) refuses a context without a launcher");
+    wt::Plan staged = plan;
+    staged.selected.strategy = wt::Strategy::converted;
+    expect(context.callbacks->convert(host_view, staged, image, context).code == wt::Error::unsupported_arithmetic, "weight runtime: convert refuses a strategy without a registered source");
+
+    // retirement: the allocation, its last-use event and its budget token go together; reclaimed once the event has completed
+    auto token = std::make_shared<int>(1);
+    std::weak_ptr<int> watch = token;
+    const std::size_t before = wt::retirements_reclaimed();
+    wt::Retirement retirement;
+    retirement.events.push_back(last_use);
+    retirement.reservation = std::move(token);
+    context.callbacks->retire(image, std::move(retirement), context);
+    wt::shutdown_native_runtime();
+    expect(wt::retirements_pending() == 0 && wt::retirements_reclaimed() == before + 1 && watch.expired(), "weight runtime: a retired image is reclaimed after its last use, its reservation released");
+    hip(hipStreamDestroy(stream), "hipStreamDestroy");
 }
 
 // ----------------------------------------------------------------------------------------------- one expert layer, three ways
@@ -434,6 +517,7 @@ int main() {
     hip(hipSetDevice(0), "hipSetDevice");
     try {
         kernel_table();
+        weight_runtime();
         const Layer L;
         a8_single_row(L);
         a8_serial_forms(L);

@@ -18,4 +18,4 @@ def test_cpp_mirror_program_on_the_gpu():
     print(run.stderr)
     assert run.returncode == 0, run.stdout + run.stderr
     lines = [l for l in run.stdout.splitlines() if l.startswith(("PASS", "FAIL"))]
-    assert len(lines) >= 26 and all(l.startswith("PASS") for l in lines)
+    assert len(lines) >= 38 and all(l.startswith("PASS") for l in lines)
