@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0     # MI355X published HBM3E peak
 MFMA_F16_PEAK_FLOPS = 2.5e15     # MI355X published dense fp16 MFMA peak
 # HBM bytes per launch of the layer's front kernel on the default workload, from two rocprofv3 --pmc passes (FETCH_SIZE scaled
 # x2.000, WRITE_SIZE x1.000 by a 256 MiB device copy in the same runs): profiles/layer_front_kernel_config3_moe_decode_T8.txt
-FRONT_TRAFFIC_BYTES_DEFAULT = 93_889_468
+FRONT_TRAFFIC_BYTES_DEFAULT = 93_935_206
 FRONT_TRAFFIC_SOURCE = "profiles/layer_front_kernel_config3_moe_decode_T8.txt (a constant from that profile, not measured in this run)"
 Q4K_ROW = lambda k: k // 256 * 144
 
@@ -41,7 +41,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--tokens", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=6, help="independent layers rotated through (cold-cache working set)")
+    ap.add_argument("--layers", type=int, default=5, help="independent layers rotated through (cold-cache working set); at most --warmup of them, so that none is first run inside the timed steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the config-4 prefill leg")
     ap.add_argument("--extra", action="store_true",
@@ -625,7 +625,10 @@ def main():
     strix.require_gpu()
     torch.cuda.set_device(0)
 
-    cfg = Config3(strix, torch, args.layers, args.tokens)
+    # every rotating layer is run in the warm-up: a layer's first call pays for things that are not decode throughput (first touch
+    # of its workspace, page-table walks over its 340 MB of weights: 30 - 80 us once, 1.5 - 4 us per step over 20 steps)
+    n_layers = max(2, min(args.layers, args.warmup)) if args.warmup > 0 else args.layers
+    cfg = Config3(strix, torch, n_layers, args.tokens)
     u_list = cfg.distinct_experts()
     u_mean = sum(u_list) / len(u_list)
 
@@ -659,7 +662,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "i8", "data": "synthetic",
         "config": {"workload": f"BASELINE config 3: MoE decode layer, Q4_K experts, hidden 2048, 128 experts, softmax router top-8, "
-                               f"intermediate 768, {args.tokens} fp16 tokens, router + experts + combine, {args.layers} rotating layers (cold cache)",
+                               f"intermediate 768, {args.tokens} fp16 tokens, router + experts + combine, {n_layers} rotating layers (cold cache)",
                    "tokens": args.tokens, "distinct_experts_mean": u_mean},
         "hbm_GBps_layer": layer_gbps, "hbm_frac_layer": layer_gbps / HBM_PEAK_GBPS,
         "layer_algorithmic_bytes": cfg.layer_bytes(u_mean), "staged_call_us": staged_call_us,
@@ -667,7 +670,7 @@ def main():
                       "staged gate/up alone (project_wave_kernel)": project_us},
         "roofline": {"bound": "hbm", "kernel": "layer_front_kernel (early routes + A8 prologue + exact router + gate/up + SwiGLU + A8 re-quantise)",
                      "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": FRONT_TRAFFIC_BYTES_DEFAULT if (args.tokens, args.layers) == (8, 6) else None,
+                     "traffic": FRONT_TRAFFIC_BYTES_DEFAULT if args.tokens == 8 else None,
                      "traffic_source": FRONT_TRAFFIC_SOURCE,
                      "algorithmic_bytes_per_launch": cfg.front_bytes(u_mean), "avg_launch_us": front_us,
                      "timing": "HIP events on the launch stream around the front launches (mi355_moe_enqueue_layer_front) of all rotating layers enqueued back to back"},

@@ -170,6 +170,18 @@ __device__ __forceinline__ float sweep_flat_rows(lds_u8* const (&slots)[DEPTH], 
     typedef int i32x4 __attribute__((ext_vector_type(4)));
     typedef const __attribute__((address_space(3))) i32x4 lds_i32x4;
     const uint32_t lane = threadIdx.x & 63U;
+    const auto start = [&](uint32_t s, lds_u8* slot) {
+        const uint8_t* base = rows + static_cast<size_t>(s) * kFlatStageBytes + 16U * lane;
+#pragma unroll
+        for (uint32_t i = 0; i < kBlockLaneCopies; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + 1024U * i),
+                                             (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
+    };
+#pragma unroll
+    for (int s = 0; s < DEPTH - 1; ++s)
+        if (s < B) start(static_cast<uint32_t>(s), slots[s]);
+    // (behind the first stage, not in front of it: the stage's address waits for the work item, the image's for nothing - issued
+    // first, the image's copy would be waited for together with the work item and the stage would start a round trip late)
     // the activation row: codes 256 B | deltas 32 B | sums 32 B bytes, in pieces of 16 (20 B pieces, at most three copy instructions)
     constexpr uint32_t kActPieces = 20U * B, kActCopies = (kActPieces + 63U) / 64U;
     {
@@ -184,23 +196,13 @@ __device__ __forceinline__ float sweep_flat_rows(lds_u8* const (&slots)[DEPTH], 
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src, (__attribute__((address_space(3))) void*)(act + 1024U * i), 16, 0, 0);
         }
     }
-    const auto start = [&](uint32_t s, lds_u8* slot) {
-        const uint8_t* base = rows + static_cast<size_t>(s) * kFlatStageBytes + 16U * lane;
-#pragma unroll
-        for (uint32_t i = 0; i < kBlockLaneCopies; ++i)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + 1024U * i),
-                                             (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
-    };
-#pragma unroll
-    for (int s = 0; s < DEPTH - 1; ++s)
-        if (s < B) start(static_cast<uint32_t>(s), slots[s]);
     float t[B][4];
 #pragma unroll
     for (int s = 0; s < B; ++s) {
         // started so far: the activation image and stages 0 .. min(B, s + DEPTH - 1) - 1; stage s (and everything older) must have landed
         const int last = s + DEPTH - 1 < B ? s + DEPTH - 1 : B, ahead = last - 1 - s;
         asm volatile("" ::: "memory");          // a stage's LDS reads stay inside the stage (hoisted, the three activation shares alone fill the register file)
-        if (ahead == 0) block_lane_wait<0>();
+        if (ahead == 0 || s == 0) block_lane_wait<0>();      // (stage 0 also waits for the image, the youngest copy so far)
         else if (ahead == 1) block_lane_wait<kBlockLaneCopies>();
         else if (ahead == 2) block_lane_wait<2 * kBlockLaneCopies>();
         else block_lane_wait<3 * kBlockLaneCopies>();

@@ -20,11 +20,12 @@
 namespace strix950 {
 
 constexpr uint32_t kEarlyExperts = 4;         // experts per early block
+constexpr uint32_t kEarlySpinLimit = 1U << 20;      // polls of the selecting block (cannot run out, short of a lost launch)
 
 // ---------------------------------------------------------------------------------------------------- early logits
 // Lane l owns features 8 l .. 8 l + 7 of every run of 512; four runs are requested together (36 loads in flight).
 template <int KIND>
-__device__ __forceinline__ void early_logits_block(const RouteArgs& a, uint32_t row, uint32_t e0) {
+__device__ __forceinline__ void early_logits_block(const RouteArgs& a, uint32_t row, uint32_t e0, uint32_t epoch) {
     const uint32_t lane = threadIdx.x & 63U;
     float acc[kEarlyExperts];
     const float* wrow[kEarlyExperts];
@@ -84,7 +85,9 @@ __device__ __forceinline__ void early_logits_block(const RouteArgs& a, uint32_t 
             }
         }
     }
-    float* out = a.early_logits + static_cast<size_t>(row) * a.early_stride;
+    // a logit travels as one 64-bit word {this call's epoch, its bits}: the row's selecting block reads the words until all carry the
+    // epoch - no count, no wait for an acknowledgement in between
+    unsigned long long* out = reinterpret_cast<unsigned long long*>(a.early_logits) + static_cast<size_t>(row) * (a.early_stride / 2U);
 #pragma unroll
     for (uint32_t i = 0; i < kEarlyExperts; ++i) {
         float v = acc[i];
@@ -95,7 +98,7 @@ __device__ __forceinline__ void early_logits_block(const RouteArgs& a, uint32_t 
             if (a.bias) v = v + a.bias[e];
             // test knob: displaces the early logits (never the exact ones), so that early and exact ids differ
             if (a.early_perturb) v = v + static_cast<float>(a.early_perturb) * 1e-3F * (static_cast<float>((e * 2654435761U) >> 28) - 8.0F);
-            __hip_atomic_store(out + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(out + e, (static_cast<unsigned long long>(epoch) << 32) | b_of(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
@@ -133,21 +136,31 @@ __device__ __forceinline__ uint32_t max_wave_u32(uint32_t v) {
     v = max_step_u32<0x142, 0xA>(v); v = max_step_u32<0x143, 0xC>(v);
     return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63));
 }
+// ok (all lanes): every logit of the row arrived within the bounded wait.
 template <uint32_t PER>
-__device__ __forceinline__ uint32_t early_select_row_per(const RouteArgs& a, uint32_t row) {
+__device__ __forceinline__ uint32_t early_select_row_per(const RouteArgs& a, uint32_t row, uint32_t epoch, bool& ok) {
     const uint32_t lane = threadIdx.x & 63U, E = a.p.experts, K = a.p.top_k;
-    const float* z = a.early_logits + static_cast<size_t>(row) * a.early_stride;
+    const unsigned long long* z = reinterpret_cast<const unsigned long long*>(a.early_logits) + static_cast<size_t>(row) * (a.early_stride / 2U);
     uint32_t key[PER];
+    uint64_t missing = ~0ULL;
+    for (uint32_t spins = 0; spins < kEarlySpinLimit && missing; ++spins) {
+        bool mine = false;
 #pragma unroll
-    for (uint32_t i = 0; i < PER; ++i) {
-        const uint32_t e = lane + 64U * i;
-        key[i] = 0;                                                              // 0 = absent or taken
-        if (e < E) {
-            const uint32_t b = b_of(__hip_atomic_load(z + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));       // written by other workgroups of this launch
-            const uint32_t sortable = (b & 0x80000000U) ? ~b : (b | 0x80000000U);
-            key[i] = sortable ? sortable : 1U;
+        for (uint32_t i = 0; i < PER; ++i) {
+            const uint32_t e = lane + 64U * i;
+            key[i] = 0;                                                          // 0 = absent or taken
+            if (e < E) {
+                const unsigned long long word = __hip_atomic_load(z + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);       // written by other workgroups of this launch
+                mine = mine || static_cast<uint32_t>(word >> 32) != epoch;
+                const uint32_t b = static_cast<uint32_t>(word);
+                const uint32_t sortable = (b & 0x80000000U) ? ~b : (b | 0x80000000U);
+                key[i] = sortable ? sortable : 1U;
+            }
         }
+        missing = __ballot(mine);
+        if (missing) __builtin_amdgcn_s_sleep(4);
     }
+    ok = missing == 0;
     uint32_t my_id = 0;
 #pragma unroll 1
     for (uint32_t k = 0; k < K; ++k) {
@@ -171,12 +184,12 @@ __device__ __forceinline__ uint32_t early_select_row_per(const RouteArgs& a, uin
     }
     return my_id;
 }
-__device__ __forceinline__ uint32_t early_select_row(const RouteArgs& a, uint32_t row) {
+__device__ __forceinline__ uint32_t early_select_row(const RouteArgs& a, uint32_t row, uint32_t epoch, bool& ok) {
     const uint32_t E = a.p.experts;
-    if (E <= 128U) return early_select_row_per<2>(a, row);
-    if (E <= 256U) return early_select_row_per<4>(a, row);
-    if (E <= 512U) return early_select_row_per<8>(a, row);
-    return early_select_row_per<16>(a, row);
+    if (E <= 128U) return early_select_row_per<2>(a, row, epoch, ok);
+    if (E <= 256U) return early_select_row_per<4>(a, row, epoch, ok);
+    if (E <= 512U) return early_select_row_per<8>(a, row, epoch, ok);
+    return early_select_row_per<16>(a, row, epoch, ok);
 }
 
 // ---------------------------------------------------------------------------------------------------- the exact chain as a side block

@@ -893,15 +893,22 @@ __global__ __launch_bounds__(64, 2) void layer_front_kernel(mi355_moe_weights w,
     unsigned long long* etags = reinterpret_cast<unsigned long long*>(a.plan + kPlanEtagsAt);
     if (bid < nb.early) {
         const uint32_t neb = (a.p.experts + kEarlyExperts - 1U) / kEarlyExperts, row = bid / neb;
-        early_logits_block<KIND>(a, row, (bid % neb) * kEarlyExperts);
+        // the row's first early block also selects: it clears the row's assignment words before anything else (acknowledged long before
+        // its tags go out), brings its own four logits, then reads the row's logits until every one carries this call's epoch
+        const bool selects = bid % neb == 0;
+        if (selects && lane < K) __hip_atomic_store(&r.awords[row * K + lane], 0U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        early_logits_block<KIND>(a, row, (bid % neb) * kEarlyExperts, epoch);
         if (bid == 0 && lane == 0) {
             *a.job_status = 0;
             a.plan[0] = assignments; a.plan[1] = 0; a.plan[2] = 1U; a.plan[4] = assignments;
         }
-        const bool last = arrive_last(&lines[kLinesEarly + row * kLineWords], neb);
-        if (!last) return;
-        const uint32_t expert = early_select_row(a, row);
-        if (lane < K) __hip_atomic_store(&r.awords[row * K + lane], 0U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!selects) return;
+        bool ok;
+        const uint32_t expert = early_select_row(a, row, epoch, ok);
+        if (!ok) {
+            if (lane == 0) atomicOr(r.status_of(row), static_cast<uint32_t>(MI355_STATUS_INVALID_ROUTE));
+            return;
+        }
         stores_acknowledged();
         if (lane < K) __hip_atomic_store(&etags[row * K + lane], (static_cast<unsigned long long>(epoch) << 32) | expert, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
@@ -937,6 +944,15 @@ __global__ __launch_bounds__(64, 2) void layer_front_kernel(mi355_moe_weights w,
         return;
     }
     const uint32_t e = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(tag))));
+    // The compute unit issues its oldest waves first, so the blocks dispatched last fall behind the others stage by stage and the
+    // launch ends with a few hundred of them alone on the memory system: the later a block's place in the dispatch, the higher
+    // its issue priority (the launch at 8 rows: 0.3 - 0.5 us).
+    {
+        const uint32_t quarter = bid * 4U / (assignments * groups);
+        if (quarter == 1U) __builtin_amdgcn_s_setprio(1);
+        else if (quarter == 2U) __builtin_amdgcn_s_setprio(2);
+        else if (quarter == 3U) __builtin_amdgcn_s_setprio(3);
+    }
     front_project(sl, w, r, e, grp, at);
     stores_acknowledged();
     if (lane == 0) __hip_atomic_fetch_add(&r.awords[at], 1U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -2443,10 +2459,10 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     // combine launch serve the batch.
     if (!norm.on && p->shared_experts == 0 && p->logits_order == MI355_LOGITS_FMA_ASCENDING && wv.gate_type == MI355_TYPE_Q4_K &&
         wv.down_type == MI355_TYPE_Q4_K && !quad_sweep(wv, rows) && wv.experts > 1U && wv.top_k <= kDownMergeSlots && items <= kEarlyMaxAssignments &&
-        wv.hidden <= kSideMaxHidden && wv.hidden % 64U == 0 && (wv.hidden / 64U) * rows <= compute_units() && wv.experts <= wv.top_k * wv.hidden) {
+        wv.hidden <= kSideMaxHidden && wv.hidden % 64U == 0 && (wv.hidden / 64U) * rows <= compute_units() && 2U * wv.experts <= wv.top_k * wv.hidden) {
         a.awords = r->plan + kPlanAwordsAt;
         a.early_perturb = g_early_perturb.load(std::memory_order_relaxed);
-        // the early logits of row i live in the row's (still unused) unweighted-output block: the exact logits own `scores`
+        // the early logits of row i (64-bit words) live in the row's (still unused) unweighted-output block: the exact logits own `scores`
         a.early_logits = r->rawdots; a.early_stride = wv.top_k * wv.hidden;
         RowsK k = layer_rows();
         k.awords = a.awords;
