@@ -288,7 +288,7 @@ constexpr uint32_t kPlanTicketsAt = 16, kPlanTicketWords = 256;
 //     complete) and the epoch word.
 // Counts are zero when the plan is allocated and every launch leaves them zero. The epoch of a call is the epoch word + 1; the
 // call's down launch stores it back, so tags of earlier calls never look current and nothing has to be reset.
-constexpr uint32_t kLineWords = 32, kEarlyMaxAssignments = 128, kEarlyMaxRows = 16;
+constexpr uint32_t kLineWords = 32, kEarlyMaxAssignments = 128, kEarlyMinAssignments = 24, kEarlyMaxRows = 16;
 constexpr uint32_t kPlanAwordsAt = kPlanTicketsAt + kPlanTicketWords, kPlanEtagsAt = kPlanAwordsAt + kEarlyMaxAssignments;
 constexpr uint32_t kPlanLinesAt = (kPlanEtagsAt + 2U * kEarlyMaxAssignments + kLineWords - 1U) / kLineWords * kLineWords;      // (lines of a 128-byte aligned plan)
 constexpr uint32_t kLinesEarly = 0, kLinesPrologue = kEarlyMaxRows * kLineWords, kLinesSide = 2U * kEarlyMaxRows * kLineWords;
@@ -2457,8 +2457,11 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     // Early routes (route_early.hpp): the expert choice from lane-parallel logits in a short first launch, the exact router beside
     // the projection, down rows + combine on the verified work items. Taken where the 64-row projection sweep and the down +
     // combine launch serve the batch.
+    // From 24 assignments on (three rows of top-8): measured at hidden 2048 / ffn 768 against the three launches of the smallest
+    // batches (router, 16-row projection, 16-row down + combine): 1 row 32.2 / 30.9 us, 2 rows 35.8 / 34.8, 3 rows 37.7 / 38.5,
+    // 4 rows 38.5 / 41.1, 5 rows 41.2 / 49.4, 6 rows 44.2 / 57.6.
     if (!norm.on && p->shared_experts == 0 && p->logits_order == MI355_LOGITS_FMA_ASCENDING && wv.gate_type == MI355_TYPE_Q4_K &&
-        wv.down_type == MI355_TYPE_Q4_K && !quad_sweep(wv, rows) && wv.experts > 1U && wv.top_k <= kDownMergeSlots && items <= kEarlyMaxAssignments &&
+        wv.down_type == MI355_TYPE_Q4_K && items >= kEarlyMinAssignments && wv.experts > 1U && wv.top_k <= kDownMergeSlots && items <= kEarlyMaxAssignments &&
         wv.hidden <= kSideMaxHidden && wv.hidden % 64U == 0 && (wv.hidden / 64U) * rows <= compute_units() && 2U * wv.experts <= wv.top_k * wv.hidden) {
         a.awords = r->plan + kPlanAwordsAt;
         a.early_perturb = g_early_perturb.load(std::memory_order_relaxed);
