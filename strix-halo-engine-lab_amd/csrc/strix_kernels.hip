@@ -2457,12 +2457,15 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     // Early routes (route_early.hpp): the expert choice from lane-parallel logits in a short first launch, the exact router beside
     // the projection, down rows + combine on the verified work items. Taken where the 64-row projection sweep and the down +
     // combine launch serve the batch.
+    // Up to two rounds of the down + combine launch's workgroups (each fills a compute unit's LDS): at hidden 2048 / ffn 768, 9..16
+    // rows take 61.5 / 63.2 / 71.4 / 78.0 us (9, 10, 12, 16 rows) against 66.8 / 75.4 / 88.4 / 100 us on the router launch, the
+    // 64-row projection and the staged down rows + combine.
     // From 24 assignments on (three rows of top-8): measured at hidden 2048 / ffn 768 against the three launches of the smallest
     // batches (router, 16-row projection, 16-row down + combine): 1 row 32.2 / 30.9 us, 2 rows 35.8 / 34.8, 3 rows 37.7 / 38.5,
     // 4 rows 38.5 / 41.1, 5 rows 41.2 / 49.4, 6 rows 44.2 / 57.6.
     if (!norm.on && p->shared_experts == 0 && p->logits_order == MI355_LOGITS_FMA_ASCENDING && wv.gate_type == MI355_TYPE_Q4_K &&
         wv.down_type == MI355_TYPE_Q4_K && items >= kEarlyMinAssignments && wv.experts > 1U && wv.top_k <= kDownMergeSlots && items <= kEarlyMaxAssignments &&
-        wv.hidden <= kSideMaxHidden && wv.hidden % 64U == 0 && (wv.hidden / 64U) * rows <= compute_units() && 2U * wv.experts <= wv.top_k * wv.hidden) {
+        wv.hidden <= kSideMaxHidden && wv.hidden % 64U == 0 && (wv.hidden / 64U) * rows <= 2U * compute_units() && 2U * wv.experts <= wv.top_k * wv.hidden) {
         a.awords = r->plan + kPlanAwordsAt;
         a.early_perturb = g_early_perturb.load(std::memory_order_relaxed);
         // the early logits of row i (64-bit words) live in the row's (still unused) unweighted-output block: the exact logits own `scores`
