@@ -2506,10 +2506,10 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     if (do_front) launch_project(wv, layer_rows(), rows, items, st);
     if (!do_back) return MI355_OK;
     // down rows and the combine in one launch (the fused router's plan: one item per assignment, in assignment order).
-    // A workgroup of that kernel fills a compute unit's LDS, so it only pays while every workgroup is resident at once
-    // (measured: 16.7 us against 14.1 + 4.2 us at hidden 2048, 8 rows; 5 % slower than two launches at hidden 6144, 16 rows)
+    // A workgroup of that kernel fills a compute unit's LDS; up to four rounds of them it still beats the staged pair of launches
+    // (hidden 3072 / ffn 768, 64 experts top-8: 8 rows 76.3 against 82.4 us, 16 rows 115.8 against 121.6 us)
     if (!quad_sweep(wv, rows) && wv.down_type == MI355_TYPE_Q4_K && wv.experts > 1U && wv.top_k <= kDownMergeSlots && wv.hidden % 64U == 0 &&
-        (wv.hidden / 64U) * rows <= compute_units()) {
+        (wv.hidden / 64U) * rows <= 4U * compute_units()) {
         launch_down_merge(wv, layer_rows(), rows, items, form, st);
         STRIX_LAUNCHED("moe layer experts + combine");
         return MI355_OK;
