@@ -149,6 +149,98 @@ __device__ __forceinline__ float sweep_block_lanes(lds_u8* const (&slots)[DEPTH]
     return value;
 }
 
+// The same sweep for stages that fill the wave (R * B = 64) and a stage count known at compile time, with the rows' chains taken
+// out of the stages: every stage leaves its block's four pair terms in registers; after the last stage the terms are laid out in
+// LDS in block order (stage s, lane l at 16 (64 s + l) bytes of slot 0, which nothing copies into any more) and lane i = sweep row
+// i = stage i / R, row i % R of it, adds the B terms of its row in ascending order - the additions of the shift-and-add chain,
+// in its order, once per sweep instead of B - 1 whole-wave steps and R lane broadcasts per stage (at B = 8: 43 vector
+// instructions and 16 LDS accesses per sweep in the place of 114 per stage). STAGES * 1 KB must fit a slot.
+template <int STAGES, class StageBase>
+__device__ __forceinline__ float sweep_block_lanes_terms(lds_u8* const (&slots)[2], StageBase stage_base, const BlockLanes g, const A8Image& img, uint32_t image_row) {
+    static_assert(STAGES >= 2 && STAGES <= 9, "terms of every stage side by side in one slot");
+    typedef const __attribute__((address_space(3))) u32x4 lds_u32x4;
+    typedef const __attribute__((address_space(3))) f32x4 lds_f32x4;
+    typedef __attribute__((address_space(3))) f32x4 lds_f32x4_w;
+    const uint32_t lane = threadIdx.x & 63U;
+    const uint32_t b = lane % g.B;
+    const auto start = [&](uint32_t s, lds_u8* slot) {
+        const uint8_t* base = stage_base(s) + 16U * lane;
+#pragma unroll
+        for (uint32_t i = 0; i < kBlockLaneCopies; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + 1024U * i),
+                                             (__attribute__((address_space(3))) void*)(slot + 1024U * i), 16, 0, 0);
+    };
+    start(0U, slots[0]);
+    // the lane's share of the activation row: block b's 256 codes, 8 deltas, 8 sums
+    u32x4 code[16];
+    float delta[8], fsum[8];
+    {
+        const u32x4* cs = reinterpret_cast<const u32x4*>(img.codes_of(image_row) + 256U * b);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) code[i] = cs[i];
+        const f32x4* ds = reinterpret_cast<const f32x4*>(img.deltas_of(image_row) + 8U * b);
+        const f32x4 d0 = ds[0], d1 = ds[1];
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+        const i32x4* ss = reinterpret_cast<const i32x4*>(img.sums_of(image_row) + 8U * b);
+        const i32x4 s0 = ss[0], s1 = ss[1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            delta[j] = d0[j]; delta[4 + j] = d1[j];
+            fsum[j] = static_cast<float>(s0[j]); fsum[4 + j] = static_cast<float>(s1[j]);
+        }
+    }
+    float t[STAGES][4];
+#pragma unroll
+    for (int S = 0; S < STAGES; ++S) {
+        // stage S has landed (the activation loads are older than every stage after the first), the reads of the slot the next copy
+        // goes into have returned
+        block_lane_wait<0>();
+        if (S + 1 < STAGES) start(static_cast<uint32_t>(S + 1), slots[(S + 1) % 2]);
+        lds_u32x4* blk = (lds_u32x4*)(slots[S % 2] + lane * 144U);
+        const u32x4 hd = blk[0];
+        u32x4 q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = blk[1 + i];
+        const float dd = half_bits_to_float(hd.x & 0xffffU), dm = half_bits_to_float(hd.x >> 16);
+        uint32_t sc[8], mn[8];
+        q4k_factors<0>(hd, sc[0], mn[0]); q4k_factors<1>(hd, sc[1], mn[1]); q4k_factors<2>(hd, sc[2], mn[2]); q4k_factors<3>(hd, sc[3], mn[3]);
+        q4k_factors<4>(hd, sc[4], mn[4]); q4k_factors<5>(hd, sc[5], mn[5]); q4k_factors<6>(hd, sc[6], mn[6]); q4k_factors<7>(hd, sc[7], mn[7]);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t wq[8] = {q[2 * p].x, q[2 * p].y, q[2 * p].z, q[2 * p].w, q[2 * p + 1].x, q[2 * p + 1].y, q[2 * p + 1].z, q[2 * p + 1].w};
+            const uint32_t c[16] = {code[4 * p].x, code[4 * p].y, code[4 * p].z, code[4 * p].w, code[4 * p + 1].x, code[4 * p + 1].y, code[4 * p + 1].z, code[4 * p + 1].w,
+                                    code[4 * p + 2].x, code[4 * p + 2].y, code[4 * p + 2].z, code[4 * p + 2].w, code[4 * p + 3].x, code[4 * p + 3].y, code[4 * p + 3].z, code[4 * p + 3].w};
+            int dot0 = 0, dot1 = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                dot0 = __builtin_amdgcn_sdot4(static_cast<int>(wq[k] & 0x0f0f0f0fU), static_cast<int>(c[k]), dot0, false);
+                dot1 = __builtin_amdgcn_sdot4(static_cast<int>((wq[k] >> 4) & 0x0f0f0f0fU), static_cast<int>(c[8 + k]), dot1, false);
+            }
+            const float D0 = dd * static_cast<float>(sc[2 * p]), D1 = dd * static_cast<float>(sc[2 * p + 1]);
+            const float M0 = dm * static_cast<float>(mn[2 * p]), M1 = dm * static_cast<float>(mn[2 * p + 1]);
+            const float u0 = D0 * static_cast<float>(dot0), v0 = M0 * fsum[2 * p];
+            const float u1 = D1 * static_cast<float>(dot1), v1 = M1 * fsum[2 * p + 1];
+            const float t0 = u0 - v0, t1 = u1 - v1;
+            const float x0 = delta[2 * p] * t0, x1 = delta[2 * p + 1] * t1;
+            t[S][p] = x0 + x1;
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // the last stage's reads have returned: slot 0 is free for the terms
+#pragma unroll
+    for (int S = 0; S < STAGES; ++S) *((lds_f32x4_w*)(slots[0] + 16U * (64U * static_cast<uint32_t>(S) + lane))) = f32x4{t[S][0], t[S][1], t[S][2], t[S][3]};
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // sweep row `lane`: stage lane / R, blocks (lane % R) * B .. + B - 1 of it
+    const uint32_t first = 64U * (lane / g.R) + (lane % g.R) * g.B;
+    float acc[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+    for (uint32_t k = 0; k < g.B; ++k) {
+        const f32x4 term = *((lds_f32x4*)(slots[0] + 16U * (first + k)));
+#pragma unroll
+        for (int p = 0; p < 4; ++p) acc[p] = acc[p] + term[p];
+    }
+    const float value = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    return lane < static_cast<uint32_t>(STAGES) * g.R ? value : 0.0F;
+}
+
 // ---------------------------------------------------------------------------------------------------------------- flat rows
 // 64 dense rows of B super-blocks against ONE activation row, as the byte stream they are: 64 * B blocks = B stages of 64 blocks,
 // each stage 9,216 contiguous bytes (nine 1 KB pieces). Lane l of stage s evaluates block g = 64 s + l, which is block g % B of

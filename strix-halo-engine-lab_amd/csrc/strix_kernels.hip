@@ -764,8 +764,10 @@ __device__ __forceinline__ void front_project(lds_u8* const (&slots)[2], const m
         const BlockLanes g = block_lanes(B, 32U);
         const uint32_t half = 32U / g.R;                  // stages of the gate rows, then as many of the up rows
         float value[1];
-        value[0] = sweep_block_lanes<2>(slots, [&](uint32_t s) { return s < half ? gate + static_cast<size_t>(s) * g.stage_bytes : up + static_cast<size_t>(s - half) * g.stage_bytes; },
-                                        2U * half, g, r.in, r.row_of(at));
+        const auto stage_base = [&](uint32_t s) { return s < half ? gate + static_cast<size_t>(s) * g.stage_bytes : up + static_cast<size_t>(s - half) * g.stage_bytes; };
+        if (g.used == 64U && half == 4U) value[0] = sweep_block_lanes_terms<8>(slots, stage_base, g, r.in, r.row_of(at));      // (hidden 2048)
+        else if (g.used == 64U && half == 2U) value[0] = sweep_block_lanes_terms<4>(slots, stage_base, g, r.in, r.row_of(at)); // (hidden 1024)
+        else value[0] = sweep_block_lanes<2>(slots, stage_base, 2U * half, g, r.in, r.row_of(at));
         project_epilogue<1>(value, w, r, grp, [&](uint32_t) { return at; });
         return;
     }
