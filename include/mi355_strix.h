@@ -249,10 +249,11 @@ int32_t mi355_moe_enqueue_combine(uint32_t form, uint32_t rows, uint32_t top_k, 
  * and weights), scores is a [rows][experts] workspace and output. For rows <= 16 the router, the A8 prologue and the expert
  * plan run in ONE launch (the workgroup that completes a row's logits also selects its experts and writes the row's work
  * items: one item per assignment, in assignment order; the CSR fields of the plan are not written), followed by project,
- * down and merge (down and merge share a launch when the batch is small enough for every workgroup to be resident). Batches of
- * 7 .. 16 rows over Q4_K experts of hidden <= 2048 run as two launches: the gate / up sweeps start on experts picked from
+ * down and merge (down and merge share a launch up to a few rounds of that launch's workgroups on the chip). Batches of
+ * 24 .. 128 assignments (3 .. 16 rows of top-8) over Q4_K experts of hidden <= 2048 run as two launches: the gate / up sweeps start on experts picked from
  * lane-parallel logits while the reference's logit chains, softmax and selection run beside them in the same launch; an
- * assignment whose early pick differs from the exact one is recomputed on the exact expert before the down rows, so the results
+ * assignment whose early pick differs from the exact one is repaired before the down rows (copied from the slot that held its
+ * expert, or swept again on the exact expert), so the results
  * are the exact router's in every case (the unweighted-output view serves as the early logits' scratch until then). Where an
  * expert's gate + up rows exceed 4 MB (and the batch is too large for the 16-rows-per-wavefront sweep) such a batch goes the
  * staged way instead - router, prologue, plan with up to two rows per work item - so that two rows that chose one expert
