@@ -250,7 +250,7 @@ int32_t mi355_moe_enqueue_combine(uint32_t form, uint32_t rows, uint32_t top_k, 
  * plan run in ONE launch (the workgroup that completes a row's logits also selects its experts and writes the row's work
  * items: one item per assignment, in assignment order; the CSR fields of the plan are not written), followed by project,
  * down and merge (down and merge share a launch up to a few rounds of that launch's workgroups on the chip). Batches of
- * 24 .. 128 assignments (3 .. 16 rows of top-8) over Q4_K experts of hidden <= 2048 run as two launches: the gate / up sweeps start on experts picked from
+ * 8 .. 128 assignments (1 .. 16 rows of top-8) over Q4_K experts of hidden <= 2048 run as two launches: the gate / up sweeps start on experts picked from
  * lane-parallel logits while the reference's logit chains, softmax and selection run beside them in the same launch; an
  * assignment whose early pick differs from the exact one is repaired before the down rows (copied from the slot that held its
  * expert, or swept again on the exact expert), so the results

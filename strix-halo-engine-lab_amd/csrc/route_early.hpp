@@ -202,7 +202,7 @@ __device__ __forceinline__ uint32_t early_select_row(const RouteArgs& a, uint32_
 //     lanes, widened once, and the fma takes it by a DPP row broadcast (chain_run of route_wave.hpp).
 //   fp32 rows do not fit beside the weights: they sit in registers (lane L holds features 32 L .. 32 L + 31) and reach the fma
 //     as a scalar operand through v_readlane (about four times the latency per step; still off the layer's critical path).
-// Needs hidden <= 2048, hidden % 32 == 0.
+// Needs hidden <= 2048, hidden % 64 == 0.
 constexpr uint32_t kSideExperts = 2, kSideMaxHidden = 2048, kSideSlotBytes = 10240, kSideRowBytes = 8192;
 
 __device__ __forceinline__ void side_copy16(const void* src, uint32_t lds_at) {
@@ -275,24 +275,37 @@ __device__ __forceinline__ void side_chain_block(lds_u8* ring0, lds_u8* ring1, c
             if constexpr (KIND == 1) return half_bits_to_float(h);
             else return f_of(h << 16);
         };
-        ChainStep A, B;
-        uint32_t ra, rb;
+        // Operands are fetched 48 features ahead of the chain (four buffers): with one step of 16 ahead every step waited for its
+        // LDS reads (128 waits of ~200 cycles: the loop took 12.6 us inside the layer launch against ~5 us for the 2048 fmas).
+        ChainStep S0, S1, S2, S3;
+        uint32_t r0, r1, r2, r3;
         auto load = [&](ChainStep& s, uint32_t& raw, uint32_t k) {
+            const uint32_t kk = k < a.hidden ? k : a.hidden - 16U;      // (past the end: a valid place, never used)
 #pragma unroll
-            for (uint32_t i = 0; i < 4U; ++i) s.w[i] = *reinterpret_cast<const f32x4*>(wrow + k + 4U * i);
-            raw = raw_of(k);
+            for (uint32_t i = 0; i < 4U; ++i) s.w[i] = *reinterpret_cast<const f32x4*>(wrow + kk + 4U * i);
+            raw = raw_of(kk);
         };
-        load(A, ra, 0);
-        for (uint32_t k = 0; k < a.hidden; k += 32U) {      // hidden % 32 == 0
-            load(B, rb, k + 16U);
+        load(S0, r0, 0U); load(S1, r1, 16U); load(S2, r2, 32U);
+        for (uint32_t k = 0; k < a.hidden; k += 64U) {      // hidden % 64 == 0 on this path
+            load(S3, r3, k + 48U);
             __builtin_amdgcn_sched_barrier(0);
-            A.x = widen(ra);
-            acc = chain_run(A, acc);
+            S0.x = widen(r0);
+            acc = chain_run(S0, acc);
             __builtin_amdgcn_sched_barrier(0);
-            load(A, ra, k + 32U < a.hidden ? k + 32U : k);
+            load(S0, r0, k + 64U);
             __builtin_amdgcn_sched_barrier(0);
-            B.x = widen(rb);
-            acc = chain_run(B, acc);
+            S1.x = widen(r1);
+            acc = chain_run(S1, acc);
+            __builtin_amdgcn_sched_barrier(0);
+            load(S1, r1, k + 80U);
+            __builtin_amdgcn_sched_barrier(0);
+            S2.x = widen(r2);
+            acc = chain_run(S2, acc);
+            __builtin_amdgcn_sched_barrier(0);
+            load(S2, r2, k + 96U);
+            __builtin_amdgcn_sched_barrier(0);
+            S3.x = widen(r3);
+            acc = chain_run(S3, acc);
             __builtin_amdgcn_sched_barrier(0);
         }
     }

@@ -288,7 +288,7 @@ constexpr uint32_t kPlanTicketsAt = 16, kPlanTicketWords = 256;
 //     complete) and the epoch word.
 // Counts are zero when the plan is allocated and every launch leaves them zero. The epoch of a call is the epoch word + 1; the
 // call's down launch stores it back, so tags of earlier calls never look current and nothing has to be reset.
-constexpr uint32_t kLineWords = 32, kEarlyMaxAssignments = 128, kEarlyMinAssignments = 24, kEarlyMaxRows = 16;
+constexpr uint32_t kLineWords = 32, kEarlyMaxAssignments = 128, kEarlyMinAssignments = 8, kEarlyMaxRows = 16;
 constexpr uint32_t kPlanAwordsAt = kPlanTicketsAt + kPlanTicketWords, kPlanEtagsAt = kPlanAwordsAt + kEarlyMaxAssignments;
 constexpr uint32_t kPlanLinesAt = (kPlanEtagsAt + 2U * kEarlyMaxAssignments + kLineWords - 1U) / kLineWords * kLineWords;      // (lines of a 128-byte aligned plan)
 constexpr uint32_t kLinesEarly = 0, kLinesPrologue = kEarlyMaxRows * kLineWords, kLinesSide = 2U * kEarlyMaxRows * kLineWords;
@@ -2462,9 +2462,9 @@ int32_t enqueue_layer(const mi355_route_policy* p, const float* router_weight, c
     // Up to two rounds of the down + combine launch's workgroups (each fills a compute unit's LDS): at hidden 2048 / ffn 768, 9..16
     // rows take 61.5 / 63.2 / 71.4 / 78.0 us (9, 10, 12, 16 rows) against 66.8 / 75.4 / 88.4 / 100 us on the router launch, the
     // 64-row projection and the staged down rows + combine.
-    // From 24 assignments on (three rows of top-8): measured at hidden 2048 / ffn 768 against the three launches of the smallest
-    // batches (router, 16-row projection, 16-row down + combine): 1 row 32.2 / 30.9 us, 2 rows 35.8 / 34.8, 3 rows 37.7 / 38.5,
-    // 4 rows 38.5 / 41.1, 5 rows 41.2 / 49.4, 6 rows 44.2 / 57.6.
+    // From 8 assignments on (one row of top-8): measured at hidden 2048 / ffn 768 against the three launches of the smallest batches
+    // (router, 16-row projection, 16-row down + combine): 1 row 28.7 / 31.3 us, 2 rows 31.6 / 35.4, 3 rows 33.4 / 37.8, 4 rows
+    // 35.7 / 40.3, 5 rows 38.4 / 48.6, 6 rows 41.2 / 57.8.
     if (!norm.on && p->shared_experts == 0 && p->logits_order == MI355_LOGITS_FMA_ASCENDING && wv.gate_type == MI355_TYPE_Q4_K &&
         wv.down_type == MI355_TYPE_Q4_K && items >= kEarlyMinAssignments && wv.experts > 1U && wv.top_k <= kDownMergeSlots && items <= kEarlyMaxAssignments &&
         wv.hidden <= kSideMaxHidden && wv.hidden % 64U == 0 && (wv.hidden / 64U) * rows <= 2U * compute_units() && 2U * wv.experts <= wv.top_k * wv.hidden) {
