@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0     # MI355X published HBM3E peak
 MFMA_F16_PEAK_FLOPS = 2.5e15     # MI355X published dense fp16 MFMA peak
 # HBM bytes per launch of the layer's front kernel on the default workload, from two rocprofv3 --pmc passes (FETCH_SIZE scaled
 # x2.000, WRITE_SIZE x1.000 by a 256 MiB device copy in the same runs): profiles/layer_front_kernel_config3_moe_decode_T8.txt
-FRONT_TRAFFIC_BYTES_DEFAULT = 94_622_515
+FRONT_TRAFFIC_BYTES_DEFAULT = 94_804_992
 FRONT_TRAFFIC_SOURCE = "profiles/layer_front_kernel_config3_moe_decode_T8.txt (a constant from that profile, not measured in this run)"
 Q4K_ROW = lambda k: k // 256 * 144
 
